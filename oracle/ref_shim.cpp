@@ -1,0 +1,455 @@
+/*
+ * ref_shim.cpp — C entry points over the UNMODIFIED tiny-dnn headers.
+ *
+ * TEST INFRASTRUCTURE ONLY. Built by oracle/Makefile against the reference
+ * tree where it lies (-I$(REF)); nothing of the reference is copied. The
+ * resulting libraries (oracle/_ref/) validate oracle/td_oracle.c and serve as
+ * the "reference" CPU baseline of the benchmark. They are never loaded by the
+ * product library.
+ *
+ * Each entry point drives real tiny-dnn objects through their public API:
+ * layer::forward / layer::backward (tiny_dnn/layers/layer.h:464-507),
+ * edge::merge_grads (tiny_dnn/node.h:89-103), optimizer::update
+ * (tiny_dnn/optimizers/optimizer.h) and network<sequential>::fit
+ * (tiny_dnn/network.h:368-386).
+ *
+ * Include order works around tiny_dnn/tiny_dnn.h:122 naming linear_layer
+ * without including its header.
+ */
+#include <iostream>
+#ifdef CNN_USE_OMP
+#include <omp.h>
+#endif
+
+#include "tiny_dnn/util/util.h"
+#include "tiny_dnn/layers/layer.h"
+#include "tiny_dnn/layers/linear_layer.h"
+#include "tiny_dnn/tiny_dnn.h"
+
+#include <chrono>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <vector>
+
+using namespace tiny_dnn;
+
+namespace {
+
+struct conv_desc {
+  int32_t in_w, in_h, in_c, k_w, k_h, out_c, w_stride, h_stride, w_dilation, h_dilation, pad_same,
+    has_bias;
+  const uint8_t *tbl;
+};
+struct pool_desc {
+  int32_t in_w, in_h, in_c, pool_w, pool_h, stride_w, stride_h, pad_same, ceil_mode;
+};
+struct opt_desc {
+  int32_t kind;
+  float alpha, lambda, mu, b1, b2, eps, b1_t, b2_t;
+};
+struct layer_desc {
+  int32_t kind, act;
+  conv_desc conv;
+  pool_desc pool;
+  int32_t fc_in, fc_out, fc_bias;
+};
+
+core::backend_t engine_of(int engine) {
+  return engine == 0 ? core::backend_t::internal : core::default_engine();
+}
+
+tensor_t to_tensor(const float *p, int batch, size_t len) {
+  tensor_t t(batch);
+  for (int s = 0; s < batch; s++) t[s].assign(p + len * s, p + len * (s + 1));
+  return t;
+}
+
+void from_tensor(const tensor_t &t, int batch, size_t len, float *p) {
+  for (int s = 0; s < batch; s++) std::memcpy(p + len * s, t[s].data(), sizeof(float) * len);
+}
+
+std::unique_ptr<convolutional_layer> make_conv(const conv_desc &d, int engine) {
+  core::connection_table tbl;
+  if (d.tbl) {
+    std::vector<char> flags(size_t(d.in_c) * d.out_c);
+    for (size_t i = 0; i < flags.size(); i++) flags[i] = d.tbl[i] != 0;
+    tbl = core::connection_table(reinterpret_cast<const bool *>(flags.data()), d.in_c, d.out_c);
+  }
+  return std::unique_ptr<convolutional_layer>(new convolutional_layer(
+    d.in_w, d.in_h, d.k_w, d.k_h, d.in_c, d.out_c, tbl,
+    d.pad_same ? padding::same : padding::valid, d.has_bias != 0, d.w_stride, d.h_stride,
+    d.w_dilation, d.h_dilation, engine_of(engine)));
+}
+
+std::unique_ptr<max_pooling_layer> make_maxpool(const pool_desc &d, int engine) {
+  return std::unique_ptr<max_pooling_layer>(new max_pooling_layer(
+    d.in_w, d.in_h, d.in_c, d.pool_w, d.pool_h, d.stride_w, d.stride_h, d.ceil_mode != 0,
+    d.pad_same ? padding::same : padding::valid, engine_of(engine)));
+}
+
+std::unique_ptr<average_pooling_layer> make_avepool(const pool_desc &d) {
+  return std::unique_ptr<average_pooling_layer>(new average_pooling_layer(
+    d.in_w, d.in_h, d.in_c, d.pool_w, d.pool_h, d.stride_w, d.stride_h, d.ceil_mode != 0,
+    d.pad_same ? padding::same : padding::valid));
+}
+
+/* Loads the first wn/bn entries of the layer's weight/bias vectors and zero-fills the rest
+ * (average_pooling_layer declares a weight vector of pool_w*pool_h*channels entries,
+ * tiny_dnn/layers/average_pooling_layer.h:222-226, of which only the first `channels`
+ * are ever read). */
+void load_weights(layer &l, const float *w, size_t wn, const float *b, size_t bn) {
+  l.setup(false);
+  auto wv = l.weights();
+  std::vector<float_t> flat;
+  if (wv.size() > 0) {
+    std::vector<float_t> part(wv[0]->size(), 0.0f);
+    if (w) std::copy(w, w + std::min(wn, part.size()), part.begin());
+    flat.insert(flat.end(), part.begin(), part.end());
+  }
+  if (wv.size() > 1) {
+    std::vector<float_t> part(wv[1]->size(), 0.0f);
+    if (b) std::copy(b, b + std::min(bn, part.size()), part.begin());
+    flat.insert(flat.end(), part.begin(), part.end());
+  }
+  int idx = 0;
+  l.load(flat, idx);
+}
+
+/* merged gradient of in-edge i: exactly what update_weight feeds to the optimizer
+ * before the 1/batch scaling */
+void merged_grad(layer &l, size_t edge_index, float *dst, size_t n = 0) {
+  vec_t merged;
+  l.inputs()[edge_index]->merge_grads(&merged);
+  std::memcpy(dst, merged.data(), sizeof(float) * (n ? std::min(n, merged.size()) : merged.size()));
+}
+
+/* run forward then backward on one layer with `batch` samples */
+void layer_fwd(layer &l, int batch, const float *x, size_t in_len, float *y, size_t out_len) {
+  std::vector<const tensor_t *> out;
+  l.forward({to_tensor(x, batch, in_len)}, out);
+  if (y) from_tensor(*out[0], batch, out_len, y);
+}
+
+double layer_bwd(layer &l, int batch, const float *dy, size_t out_len, float *dx, size_t in_len) {
+  std::vector<tensor_t> g{to_tensor(dy, batch, out_len)};
+  /* layer::forward cleared the out-edge gradient only; start weight grads from zero as
+   * update_weight/clear_grads leaves them */
+  l.clear_grads();
+  auto t0 = std::chrono::steady_clock::now();
+  std::vector<tensor_t> in_grads = l.backward(g);
+  auto t1 = std::chrono::steady_clock::now();
+  if (dx) from_tensor(in_grads[0], batch, in_len, dx);
+  return std::chrono::duration<double>(t1 - t0).count();
+}
+
+template <typename Act>
+int act_run(int batch, int len, const float *x, float *y, const float *dy, float *dx) {
+  Act a((size_t)len);
+  layer_fwd(a, batch, x, len, y, len);
+  if (dy) layer_bwd(a, batch, dy, len, dx, len);
+  return 0;
+}
+
+template <typename Opt>
+void run_updates(Opt &o, size_t n, const float *g, float *w, int steps) {
+  vec_t W(w, w + n), G(g, g + n);
+  for (int s = 0; s < steps; s++) o.update(G, W, false);
+  std::memcpy(w, W.data(), sizeof(float) * n);
+}
+
+}  // namespace
+
+extern "C" {
+
+int tdr_num_threads() {
+#ifdef CNN_USE_OMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* 1 when the build's default engine is the AVX one */
+int tdr_default_engine_is_avx() { return core::default_engine() == core::backend_t::avx; }
+
+int tdr_conv2d_fwd(const conv_desc *d, int engine, int batch, const float *x, const float *w,
+                   const float *b, float *y) {
+  try {
+    auto l = make_conv(*d, engine);
+    load_weights(*l, w, l->weights()[0]->size(), d->has_bias ? b : nullptr, d->out_c);
+    layer_fwd(*l, batch, x, l->in_shape()[0].size(), y, l->out_shape()[0].size());
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* returns seconds spent inside layer::backward (negative on error) */
+double tdr_conv2d_bwd(const conv_desc *d, int engine, int batch, const float *x, const float *w,
+                      const float *dy, float *dx, float *dw, float *db, int repeat) {
+  try {
+    auto l = make_conv(*d, engine);
+    std::vector<float> zb(d->out_c, 0.0f);
+    load_weights(*l, w, l->weights()[0]->size(), d->has_bias ? zb.data() : nullptr, d->out_c);
+    const size_t in_len = l->in_shape()[0].size(), out_len = l->out_shape()[0].size();
+    layer_fwd(*l, batch, x, in_len, nullptr, out_len);
+    double best = 1e30;
+    for (int r = 0; r < (repeat < 1 ? 1 : repeat); r++) {
+      const double t = layer_bwd(*l, batch, dy, out_len, dx, in_len);
+      if (t < best) best = t;
+    }
+    if (dw) merged_grad(*l, 1, dw);
+    if (db && d->has_bias) merged_grad(*l, 2, db);
+    return best;
+  } catch (const std::exception &) { return -1.0; }
+}
+
+int tdr_fc_fwd(int in, int out, int has_bias, int engine, int batch, const float *x,
+               const float *w, const float *b, float *y) {
+  try {
+    fully_connected_layer l(in, out, has_bias != 0, engine_of(engine));
+    load_weights(l, w, size_t(in) * out, has_bias ? b : nullptr, out);
+    layer_fwd(l, batch, x, in, y, out);
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+double tdr_fc_bwd(int in, int out, int has_bias, int engine, int batch, const float *x,
+                  const float *w, const float *dy, float *dx, float *dw, float *db, int repeat) {
+  try {
+    fully_connected_layer l(in, out, has_bias != 0, engine_of(engine));
+    std::vector<float> zb(out, 0.0f);
+    load_weights(l, w, size_t(in) * out, has_bias ? zb.data() : nullptr, out);
+    layer_fwd(l, batch, x, in, nullptr, out);
+    double best = 1e30;
+    for (int r = 0; r < (repeat < 1 ? 1 : repeat); r++) {
+      const double t = layer_bwd(l, batch, dy, out, dx, in);
+      if (t < best) best = t;
+    }
+    if (dw) merged_grad(l, 1, dw);
+    if (db && has_bias) merged_grad(l, 2, db);
+    return best;
+  } catch (const std::exception &) { return -1.0; }
+}
+
+int tdr_maxpool_fwd(const pool_desc *d, int engine, int batch, const float *x, float *y) {
+  try {
+    auto l = make_maxpool(*d, engine);
+    layer_fwd(*l, batch, x, l->in_shape()[0].size(), y, l->out_shape()[0].size());
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* forward on x (records the argmax inside the layer) then backward with dy */
+int tdr_maxpool_fwd_bwd(const pool_desc *d, int engine, int batch, const float *x, float *y,
+                        const float *dy, float *dx) {
+  try {
+    auto l = make_maxpool(*d, engine);
+    const size_t in_len = l->in_shape()[0].size(), out_len = l->out_shape()[0].size();
+    layer_fwd(*l, batch, x, in_len, y, out_len);
+    layer_bwd(*l, batch, dy, out_len, dx, in_len);
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+int tdr_avepool_fwd(const pool_desc *d, int batch, const float *x, const float *w,
+                    const float *b, float *y) {
+  try {
+    auto l = make_avepool(*d);
+    load_weights(*l, w, d->in_c, b, d->in_c);
+    layer_fwd(*l, batch, x, l->in_shape()[0].size(), y, l->out_shape()[0].size());
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+int tdr_avepool_bwd(const pool_desc *d, int batch, const float *x, const float *w,
+                    const float *dy, float *dx, float *dw, float *db) {
+  try {
+    auto l = make_avepool(*d);
+    std::vector<float> zb(d->in_c, 0.0f);
+    load_weights(*l, w, d->in_c, zb.data(), d->in_c);
+    const size_t in_len = l->in_shape()[0].size(), out_len = l->out_shape()[0].size();
+    layer_fwd(*l, batch, x, in_len, nullptr, out_len);
+    layer_bwd(*l, batch, dy, out_len, dx, in_len);
+    if (dw) merged_grad(*l, 1, dw, d->in_c);
+    if (db) merged_grad(*l, 2, db, d->in_c);
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* kind: 0 tanh, 1 relu, 2 softmax, 3 sigmoid; dy/dx may be NULL (forward only) */
+int tdr_act(int kind, int batch, int len, const float *x, float *y, const float *dy, float *dx) {
+  try {
+    switch (kind) {
+      case 0: return act_run<tanh_layer>(batch, len, x, y, dy, dx);
+      case 1: return act_run<relu_layer>(batch, len, x, y, dy, dx);
+      case 2: return act_run<softmax_layer>(batch, len, x, y, dy, dx);
+      case 3: return act_run<sigmoid_layer>(batch, len, x, y, dy, dx);
+    }
+    return -2;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* kind: 0 mse, 1 cross_entropy_multiclass, 2 cross_entropy */
+int tdr_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy) {
+  std::vector<tensor_t> yy(batch), tt(batch), cost;
+  for (int s = 0; s < batch; s++) {
+    yy[s] = {vec_t(y + size_t(len) * s, y + size_t(len) * (s + 1))};
+    tt[s] = {vec_t(t + size_t(len) * s, t + size_t(len) * (s + 1))};
+  }
+  std::vector<tensor_t> g;
+  switch (kind) {
+    case 0: g = gradient<mse>(yy, tt, cost); break;
+    case 1: g = gradient<cross_entropy_multiclass>(yy, tt, cost); break;
+    case 2: g = gradient<cross_entropy>(yy, tt, cost); break;
+    default: return -2;
+  }
+  for (int s = 0; s < batch; s++) std::memcpy(dy + size_t(len) * s, g[s][0].data(), sizeof(float) * len);
+  return 0;
+}
+
+/* `steps` consecutive optimizer::update(g, w) calls on one fresh optimizer object with
+ * the hyper-parameters of *o (kinds as in td_oracle.h) */
+int tdr_opt_updates(const opt_desc *o, size_t n, const float *g, float *w, int steps) {
+  switch (o->kind) {
+    case 0: { gradient_descent p; p.alpha = o->alpha; p.lambda = o->lambda; run_updates(p, n, g, w, steps); } break;
+    case 1: { momentum p; p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; run_updates(p, n, g, w, steps); } break;
+    case 2: { adam p; p.alpha = o->alpha; p.b1 = o->b1; p.b2 = o->b2; p.b1_t = o->b1_t; p.b2_t = o->b2_t; run_updates(p, n, g, w, steps); } break;
+    case 3: { adagrad p; p.alpha = o->alpha; run_updates(p, n, g, w, steps); } break;
+    case 4: { RMSprop p; p.alpha = o->alpha; p.mu = o->mu; run_updates(p, n, g, w, steps); } break;
+    case 5: { adamax p; p.alpha = o->alpha; p.b1 = o->b1; p.b2 = o->b2; p.b1_t = o->b1_t; run_updates(p, n, g, w, steps); } break;
+    case 6: { nesterov_momentum p; p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; run_updates(p, n, g, w, steps); } break;
+    default: return -2;
+  }
+  return 0;
+}
+
+/* ---- whole network: network<sequential>::fit on caller-provided arrays ---- */
+
+struct tdr_net {
+  network<sequential> net;
+  std::vector<layer_desc> spec;
+};
+
+tdr_net *tdr_net_create(const layer_desc *layers, int n_layers, int engine) {
+  try {
+    std::unique_ptr<tdr_net> h(new tdr_net());
+    h->spec.assign(layers, layers + n_layers);
+    for (int i = 0; i < n_layers; i++) {
+      const layer_desc &s = layers[i];
+      switch (s.kind) {
+        case 0: {
+          core::connection_table tbl;
+          if (s.conv.tbl) {
+            std::vector<char> flags(size_t(s.conv.in_c) * s.conv.out_c);
+            for (size_t k = 0; k < flags.size(); k++) flags[k] = s.conv.tbl[k] != 0;
+            tbl = core::connection_table(reinterpret_cast<const bool *>(flags.data()), s.conv.in_c,
+                                         s.conv.out_c);
+          }
+          h->net << convolutional_layer(
+            s.conv.in_w, s.conv.in_h, s.conv.k_w, s.conv.k_h, s.conv.in_c, s.conv.out_c, tbl,
+            s.conv.pad_same ? padding::same : padding::valid, s.conv.has_bias != 0,
+            s.conv.w_stride, s.conv.h_stride, s.conv.w_dilation, s.conv.h_dilation,
+            engine_of(engine));
+        } break;
+        case 1:
+          h->net << fully_connected_layer(s.fc_in, s.fc_out, s.fc_bias != 0, engine_of(engine));
+          break;
+        case 2:
+          h->net << max_pooling_layer(s.pool.in_w, s.pool.in_h, s.pool.in_c, s.pool.pool_w,
+                                      s.pool.pool_h, s.pool.stride_w, s.pool.stride_h,
+                                      s.pool.ceil_mode != 0,
+                                      s.pool.pad_same ? padding::same : padding::valid,
+                                      engine_of(engine));
+          break;
+        case 3:
+          h->net << average_pooling_layer(s.pool.in_w, s.pool.in_h, s.pool.in_c, s.pool.pool_w,
+                                          s.pool.pool_h, s.pool.stride_w, s.pool.stride_h,
+                                          s.pool.ceil_mode != 0,
+                                          s.pool.pad_same ? padding::same : padding::valid);
+          break;
+        case 4:
+          switch (s.act) {
+            case 0: h->net << tanh_layer(); break;
+            case 1: h->net << relu_layer(); break;
+            case 2: h->net << softmax_layer(); break;
+            case 3: h->net << sigmoid_layer(); break;
+            default: return nullptr;
+          }
+          break;
+        default: return nullptr;
+      }
+    }
+    h->net.init_weight();
+    return h.release();
+  } catch (const std::exception &) { return nullptr; }
+}
+
+void tdr_net_destroy(tdr_net *h) { delete h; }
+
+size_t tdr_net_param_size(tdr_net *h, int layer, int which) {
+  auto w = h->net[layer]->weights();
+  return size_t(which) < w.size() ? w[which]->size() : 0;
+}
+
+int tdr_net_set_param(tdr_net *h, int layer, int which, const float *src) {
+  auto w = h->net[layer]->weights();
+  if (size_t(which) >= w.size()) return -2;
+  std::copy(src, src + w[which]->size(), w[which]->begin());
+  return 0;
+}
+
+int tdr_net_get_param(tdr_net *h, int layer, int which, float *dst) {
+  auto w = h->net[layer]->weights();
+  if (size_t(which) >= w.size()) return -2;
+  std::copy(w[which]->begin(), w[which]->end(), dst);
+  return 0;
+}
+
+/* `steps` mini-batch steps on the same batch (fit over `steps` epochs of one batch) with one
+ * optimizer object; returns seconds per step (negative on error). loss: 0 mse,
+ * 1 cross_entropy_multiclass, 2 cross_entropy. */
+double tdr_net_fit(tdr_net *h, const opt_desc *o, int loss, int batch, const float *x,
+                   size_t in_len, const float *t, size_t out_len, int steps) {
+  try {
+    std::vector<vec_t> X(batch), T(batch);
+    for (int s = 0; s < batch; s++) {
+      X[s].assign(x + in_len * s, x + in_len * (s + 1));
+      T[s].assign(t + out_len * s, t + out_len * (s + 1));
+    }
+    auto nop = []() {};
+    auto t0  = std::chrono::steady_clock::now();
+    bool ok  = false;
+#define TDR_FIT(OPT)                                                                   \
+  switch (loss) {                                                                      \
+    case 0: ok = h->net.fit<mse>(OPT, X, T, batch, steps, nop, nop); break;            \
+    case 1: ok = h->net.fit<cross_entropy_multiclass>(OPT, X, T, batch, steps, nop, nop); break; \
+    case 2: ok = h->net.fit<cross_entropy>(OPT, X, T, batch, steps, nop, nop); break;  \
+    default: return -2.0;                                                              \
+  }
+    switch (o->kind) {
+      case 0: { gradient_descent p; p.alpha = o->alpha; p.lambda = o->lambda; TDR_FIT(p) } break;
+      case 1: { momentum p; p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; TDR_FIT(p) } break;
+      case 2: { adam p; p.alpha = o->alpha; p.b1 = o->b1; p.b2 = o->b2; p.b1_t = o->b1_t; p.b2_t = o->b2_t; TDR_FIT(p) } break;
+      default: return -2.0;
+    }
+#undef TDR_FIT
+    auto t1 = std::chrono::steady_clock::now();
+    if (!ok) return -1.0;
+    return std::chrono::duration<double>(t1 - t0).count() / steps;
+  } catch (const std::exception &) { return -1.0; }
+}
+
+/* forward only, returns the network output for the batch */
+int tdr_net_predict(tdr_net *h, int batch, const float *x, size_t in_len, float *y,
+                    size_t out_len) {
+  try {
+    for (int s = 0; s < batch; s++) {
+      vec_t in(x + in_len * s, x + in_len * (s + 1));
+      vec_t out = h->net.predict(in);
+      std::memcpy(y + out_len * s, out.data(), sizeof(float) * out_len);
+    }
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+}  // extern "C"

@@ -1,0 +1,151 @@
+/*
+ * td_oracle.h — CPU restatement of tiny-dnn's training hot path (TEST INFRASTRUCTURE ONLY).
+ *
+ * This is the checker the HIP path is compared against. It is never linked
+ * into, imported by or called from the product library. Only the test-suite,
+ * the smoke check and the cpu_baseline leg of the benchmark may load it.
+ *
+ * All tensors are dense fp32, [batch][flat] with the reference's per-sample
+ * CHW layout: index = (H*c + y)*W + x   (tiny_dnn/util/util.h:168-173).
+ * Conv weights are OIHW, FC weights are [in][out] row-major.
+ *
+ * Weight/bias gradients are returned MERGED: the in-order sum over samples of
+ * the per-sample gradients, i.e. what edge::merge_grads (tiny_dnn/node.h:89-103)
+ * produces. layer::update_weight (tiny_dnn/layers/layer.h:663-682) multiplies it
+ * by 1/size-of-the-weight-edge's-data-tensor, which is 1: the optimizer sees the
+ * SUM over the batch, not the mean.
+ *
+ * Pinning status of each function (what fixes its behaviour independently of
+ * this file) is listed in td_oracle.c above each definition and checked by
+ * tests/test_oracle_*.py.
+ */
+#ifndef TD_ORACLE_H
+#define TD_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tdo_conv_desc {
+  int32_t in_w, in_h, in_c;
+  int32_t k_w, k_h, out_c;
+  int32_t w_stride, h_stride;
+  int32_t w_dilation, h_dilation;
+  int32_t pad_same; /* 0 = padding::valid, 1 = padding::same */
+  int32_t has_bias;
+  const uint8_t *tbl; /* NULL or [in_c][out_c] connection table (1 = connected) */
+} tdo_conv_desc;
+
+typedef struct tdo_pool_desc {
+  int32_t in_w, in_h, in_c;
+  int32_t pool_w, pool_h;
+  int32_t stride_w, stride_h;
+  int32_t pad_same;
+  int32_t ceil_mode;
+} tdo_pool_desc;
+
+enum { TDO_ACT_TANH = 0, TDO_ACT_RELU = 1, TDO_ACT_SOFTMAX = 2, TDO_ACT_SIGMOID = 3 };
+enum { TDO_LOSS_MSE = 0, TDO_LOSS_CE_MULTICLASS = 1, TDO_LOSS_CE = 2 };
+enum { TDO_OPT_SGD = 0, TDO_OPT_MOMENTUM = 1, TDO_OPT_ADAM = 2, TDO_OPT_ADAGRAD = 3,
+       TDO_OPT_RMSPROP = 4, TDO_OPT_ADAMAX = 5, TDO_OPT_NESTEROV = 6 };
+
+/* optimizer hyper-parameters + the scalar state the reference keeps in the
+ * optimizer object (b1_t/b2_t advance once per update() call). */
+typedef struct tdo_opt {
+  int32_t kind;
+  float alpha, lambda, mu, b1, b2, eps;
+  float b1_t, b2_t;
+} tdo_opt;
+
+void tdo_opt_default(tdo_opt *o, int kind);
+
+/* shape helpers */
+int tdo_conv_out_w(const tdo_conv_desc *d);
+int tdo_conv_out_h(const tdo_conv_desc *d);
+int tdo_conv_padded_w(const tdo_conv_desc *d);
+int tdo_conv_padded_h(const tdo_conv_desc *d);
+int tdo_pool_out_w(const tdo_pool_desc *d);
+int tdo_pool_out_h(const tdo_pool_desc *d);
+
+/* convolution; x is UNPADDED [batch][in_c*in_h*in_w]; dx likewise */
+int tdo_conv2d_fwd(const tdo_conv_desc *d, int batch, const float *x, const float *w,
+                   const float *b, float *y);
+int tdo_conv2d_bwd(const tdo_conv_desc *d, int batch, const float *x, const float *w,
+                   const float *dy, float *dx, float *dw, float *db);
+
+/* fully connected */
+int tdo_fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+               const float *b, float *y);
+int tdo_fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+               const float *dy, float *dx, float *dw, float *db);
+
+/* max pooling; argmax holds the flat per-sample CHW input index */
+int tdo_maxpool_fwd(const tdo_pool_desc *d, int batch, const float *x, float *y,
+                    int64_t *argmax);
+int tdo_maxpool_bwd(const tdo_pool_desc *d, int batch, const float *dy,
+                    const int64_t *argmax, float *dx);
+
+/* average pooling with trainable per-channel scale w[c] and bias b[c] */
+int tdo_avepool_fwd(const tdo_pool_desc *d, int batch, const float *x, const float *w,
+                    const float *b, float *y);
+int tdo_avepool_bwd(const tdo_pool_desc *d, int batch, const float *x, const float *w,
+                    const float *dy, float *dx, float *dw, float *db);
+
+/* activations: len = per-sample vector length */
+int tdo_act_fwd(int kind, int batch, int len, const float *x, float *y);
+int tdo_act_bwd(int kind, int batch, int len, const float *x, const float *y,
+                const float *dy, float *dx);
+
+/* loss gradient for a mini-batch (no 1/batch factor, as in the reference) */
+int tdo_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
+float tdo_loss_value(int kind, int batch, int len, const float *y, const float *t);
+
+/* optimizer::update on an already merged+scaled gradient g (s0/s1: state vectors) */
+int tdo_opt_update(tdo_opt *o, size_t n, const float *g, float *w, float *s0, float *s1);
+/* layer::update_weight for one tensor: g = merged * (1/weight_edge_samples), then update.
+ * In the reference weight_edge_samples is always 1 (see td_oracle.c). */
+int tdo_update_weight(tdo_opt *o, size_t n, int weight_edge_samples, const float *merged,
+                      float *w, float *s0, float *s1);
+
+/* ---- sequential network (one train step = fprop, loss grad, bprop, update) ---- */
+enum { TDO_L_CONV = 0, TDO_L_FC = 1, TDO_L_MAXPOOL = 2, TDO_L_AVEPOOL = 3, TDO_L_ACT = 4 };
+
+typedef struct tdo_layer {
+  int32_t kind;
+  int32_t act; /* TDO_L_ACT: activation kind */
+  tdo_conv_desc conv;
+  tdo_pool_desc pool;
+  int32_t fc_in, fc_out, fc_bias;
+} tdo_layer;
+
+typedef struct tdo_net tdo_net;
+
+tdo_net *tdo_net_create(const tdo_layer *layers, int n_layers, int max_batch);
+void tdo_net_destroy(tdo_net *net);
+int tdo_net_num_layers(const tdo_net *net);
+size_t tdo_net_in_size(const tdo_net *net);
+size_t tdo_net_out_size(const tdo_net *net);
+/* per layer: weight count, bias count, out size */
+size_t tdo_net_weight_size(const tdo_net *net, int layer);
+size_t tdo_net_bias_size(const tdo_net *net, int layer);
+size_t tdo_net_layer_out_size(const tdo_net *net, int layer);
+float *tdo_net_weight(tdo_net *net, int layer);
+float *tdo_net_bias(tdo_net *net, int layer);
+/* after a step: layer outputs [batch][out], merged dW/db, dX (grad wrt layer input) */
+const float *tdo_net_layer_out(const tdo_net *net, int layer);
+const float *tdo_net_layer_dx(const tdo_net *net, int layer);
+const float *tdo_net_layer_dw(const tdo_net *net, int layer);
+const float *tdo_net_layer_db(const tdo_net *net, int layer);
+const int64_t *tdo_net_layer_argmax(const tdo_net *net, int layer);
+int tdo_net_forward(tdo_net *net, int batch, const float *x);
+/* full step; returns 0 on success. do_update = 0 leaves weights untouched */
+int tdo_net_train_step(tdo_net *net, tdo_opt *opt, int loss_kind, int batch, const float *x,
+                       const float *t, int do_update);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
