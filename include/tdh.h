@@ -1,0 +1,226 @@
+/*
+ * tdh.h — C ABI of libtdh.so: tiny-dnn's training hot path on one AMD Instinct
+ * MI355X (gfx950), hand-written HIP.
+ *
+ * The entry points are what tiny-dnn's operator layer binds for this path: each
+ * one replaces the body of an OpKernel::compute (or of the free function the
+ * reference calls in its place) and is cited next to its declaration (paths
+ * relative to the tiny-dnn tree).
+ *
+ * Conventions
+ *  - Every tensor argument is a DEVICE pointer obtained from tdh_malloc, dense
+ *    fp32, [batch][flat] with tiny-dnn's per-sample CHW layout
+ *    index = (H*c + y)*W + x  (tiny_dnn/util/util.h:168-173). Conv weights are
+ *    OIHW, fully-connected weights [in][out] row-major.
+ *  - Convolution inputs/gradients are UNPADDED; padding::same is applied
+ *    implicitly by the kernels (the reference copies into padded buffers,
+ *    tiny_dnn/core/params/conv_params.h:106-166).
+ *  - Weight/bias gradients are produced already reduced over the batch (the sum
+ *    over samples that edge::merge_grads computes, tiny_dnn/node.h:89-103) in a
+ *    fixed order: the same inputs always give the same bits.
+ *  - All work is queued on one library-owned stream; calls return without
+ *    waiting for the GPU except tdh_sync, tdh_memcpy_d2h and tdh_event_elapsed_ms.
+ *  - Every function returns TDH_OK (0) or a negative tdh_status; the message for
+ *    the last failure on the calling thread is tdh_last_error(). The C++ host
+ *    layer turns failures into tiny_dnn::nn_error, the reference's convention
+ *    (tiny_dnn/util/nn_error.h:19-26).
+ *  - Single caller thread (the reference's training thread); not re-entrant.
+ */
+#ifndef TDH_H
+#define TDH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tdh_status {
+  TDH_OK                = 0,
+  TDH_ERR_INVALID       = -1, /* bad argument / unsupported shape */
+  TDH_ERR_HIP           = -2, /* a HIP runtime call failed */
+  TDH_ERR_NOT_INIT      = -3, /* tdh_init has not been called */
+  TDH_ERR_UNSUPPORTED   = -4, /* valid in the reference but not built here */
+  TDH_ERR_OOM           = -5
+} tdh_status;
+
+/* activation_layer subclasses (tiny_dnn/activations/) */
+enum { TDH_ACT_TANH = 0, TDH_ACT_RELU = 1, TDH_ACT_SOFTMAX = 2, TDH_ACT_SIGMOID = 3, TDH_ACT_NONE = -1 };
+/* loss functions (tiny_dnn/lossfunctions/loss_function.h) */
+enum { TDH_LOSS_MSE = 0, TDH_LOSS_CE_MULTICLASS = 1, TDH_LOSS_CE = 2 };
+/* optimizers (tiny_dnn/optimizers/optimizer.h) */
+enum { TDH_OPT_SGD = 0, TDH_OPT_MOMENTUM = 1, TDH_OPT_ADAM = 2, TDH_OPT_ADAGRAD = 3,
+       TDH_OPT_RMSPROP = 4, TDH_OPT_ADAMAX = 5, TDH_OPT_NESTEROV = 6 };
+/* layer kinds of a sequential network */
+enum { TDH_L_CONV = 0, TDH_L_FC = 1, TDH_L_MAXPOOL = 2, TDH_L_AVEPOOL = 3, TDH_L_ACT = 4 };
+
+/* core::conv_params (tiny_dnn/core/params/conv_params.h:63-90) */
+typedef struct tdh_conv_desc {
+  int32_t in_w, in_h, in_c;
+  int32_t k_w, k_h, out_c;
+  int32_t w_stride, h_stride;
+  int32_t w_dilation, h_dilation; /* forward only, as in the reference; backward needs 1 */
+  int32_t pad_same;               /* 0 = padding::valid, 1 = padding::same */
+  int32_t has_bias;
+  const uint8_t *tbl;             /* HOST pointer: NULL or connection_table [in_c][out_c] */
+} tdh_conv_desc;
+
+/* core::maxpool_params (tiny_dnn/core/params/maxpool_params.h:17-34) and the
+ * constructor arguments of average_pooling_layer */
+typedef struct tdh_pool_desc {
+  int32_t in_w, in_h, in_c;
+  int32_t pool_w, pool_h;
+  int32_t stride_w, stride_h;
+  int32_t pad_same;
+  int32_t ceil_mode;
+} tdh_pool_desc;
+
+/* Hyper-parameters plus the scalar state tiny-dnn keeps inside the optimizer
+ * object: adam/adamax advance b1_t (and b2_t) once per update() call, i.e. once
+ * per weight TENSOR (tiny_dnn/optimizers/optimizer.h:112-127,153-165). */
+typedef struct tdh_opt {
+  int32_t kind;
+  float alpha, lambda, mu, b1, b2, eps;
+  float b1_t, b2_t;
+} tdh_opt;
+
+typedef struct tdh_layer {
+  int32_t kind;
+  int32_t act; /* TDH_L_ACT: activation kind */
+  tdh_conv_desc conv;
+  tdh_pool_desc pool;
+  int32_t fc_in, fc_out, fc_bias;
+} tdh_layer;
+
+/* ------------------------------------------------------------ library state */
+int tdh_init(int device);
+int tdh_shutdown(void);
+const char *tdh_last_error(void);
+const char *tdh_version(void);
+/* name, compute units and memory of the device selected by tdh_init */
+int tdh_device_info(char *name, size_t name_len, int32_t *compute_units, size_t *global_mem_bytes);
+
+/* ----------------------------------------------------------- device memory */
+int tdh_malloc(void **dptr, size_t bytes);
+int tdh_free(void *dptr);
+int tdh_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int tdh_memcpy_d2h(void *dst, const void *src, size_t bytes); /* waits for queued work */
+int tdh_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int tdh_fill_zero(void *dptr, size_t bytes);                  /* fill kernel, graph-safe */
+int tdh_sync(void);
+
+/* timing on the library stream */
+int tdh_event_create(void **event);
+int tdh_event_destroy(void *event);
+int tdh_event_record(void *event);
+int tdh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
+
+/* shape helpers: conv_out_length / pool_out_length (tiny_dnn/util/util.h:329-363) */
+int tdh_conv_out_w(const tdh_conv_desc *d);
+int tdh_conv_out_h(const tdh_conv_desc *d);
+int tdh_pool_out_w(const tdh_pool_desc *d);
+int tdh_pool_out_h(const tdh_pool_desc *d);
+
+/* ------------------------------------------------------------- convolution */
+/* Conv2dOp::compute (tiny_dnn/core/kernels/conv2d_op.h:23-51,
+ * conv2d_op_internal.h:13-74): y = conv(x, w) + b */
+int tdh_conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w,
+                   const float *b, float *y);
+/* Conv2dGradOp::compute (tiny_dnn/core/kernels/conv2d_grad_op.h:22-50,
+ * conv2d_op_internal.h:78-181). dx is overwritten; dw/db are overwritten
+ * (accumulate = 0) or added to (accumulate = 1, the reference's += into gradients
+ * that update_weight later clears). Any of dx, dw, db may be NULL to skip it. */
+int tdh_conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w,
+                   const float *dy, float *dx, float *dw, float *db, int accumulate);
+
+/* --------------------------------------------------------- fully connected */
+/* FullyConnectedOp::compute (tiny_dnn/core/kernels/fully_connected_op.h:25-63,
+ * fully_connected_op_internal.h:15-36) */
+int tdh_fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+               const float *b, float *y);
+/* FullyConnectedGradOp::compute (tiny_dnn/core/kernels/fully_connected_grad_op.h:22-52,
+ * fully_connected_op_internal.h:38-71) */
+int tdh_fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+               const float *dy, float *dx, float *dw, float *db, int accumulate);
+
+/* ----------------------------------------------------------------- pooling */
+/* MaxPoolOp::compute (tiny_dnn/core/kernels/maxpool_op.h:23-61,
+ * maxpool_op_internal.h:16-40). argmax[batch][out] = flat per-sample CHW index of
+ * the first maximum in (dy,dx) scan order (the reference's out2inmax, held as
+ * int32 here). */
+int tdh_maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y,
+                    int32_t *argmax);
+/* MaxPoolGradOp::compute (tiny_dnn/core/kernels/maxpool_grad_op.h:22-46,
+ * maxpool_op_internal.h:42-57) */
+int tdh_maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
+                    float *dx);
+/* AvePoolOp: tiny_average_pooling_kernel (tiny_dnn/layers/average_pooling_layer.h:25-55);
+ * w and b hold one trainable scale / bias per channel */
+int tdh_avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w,
+                    const float *b, float *y);
+/* AvePoolGradOp: tiny_average_pooling_back_kernel
+ * (tiny_dnn/layers/average_pooling_layer.h:58-106) */
+int tdh_avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w,
+                    const float *dy, float *dx, float *dw, float *db, int accumulate);
+
+/* ------------------------------------------------- activations and losses */
+/* activation_layer::forward_propagation / back_propagation
+ * (tiny_dnn/activations/activation_layer.h:74-91; tanh_layer.h:24-38,
+ * relu_layer.h:25-39, softmax_layer.h:24-55, sigmoid_layer.h:24-38).
+ * len = per-sample vector length; the backward uses the layer OUTPUT y. */
+int tdh_act_fwd(int kind, int batch, int len, const float *x, float *y);
+int tdh_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx);
+/* gradient<E> for a mini-batch (tiny_dnn/lossfunctions/loss_function.h:191-218) */
+int tdh_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
+/* softmax_layer backward applied to cross_entropy_multiclass::df in one kernel:
+ * dz = y * sum(t) - t  (= y - t for one-hot targets) */
+int tdh_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz);
+
+/* -------------------------------------------------------------- optimizers */
+/* layer::update_weight for one tensor (tiny_dnn/layers/layer.h:663-682) followed by
+ * optimizer::update (tiny_dnn/optimizers/optimizer.h): g = merged_grad * grad_scale,
+ * then the update of `kind`. tiny-dnn's own grad_scale is 1 (its rcp_batch_size is
+ * taken from the weight edge, whose data tensor has one entry). s0/s1 are the
+ * optimizer's per-weight state vectors (may be NULL where unused). *o is updated on
+ * the host exactly as the reference updates b1_t/b2_t. */
+int tdh_opt_update(tdh_opt *o, size_t n, const float *merged_grad, float grad_scale, float *w,
+                   float *s0, float *s1);
+void tdh_opt_default(tdh_opt *o, int kind);
+
+/* ------------------------------------------------------ sequential network */
+/* network<sequential>::fit / train_onebatch (tiny_dnn/network.h:840-926) with
+ * every tensor resident on the device. */
+typedef struct tdh_net tdh_net;
+
+enum {
+  TDH_NET_FUSE_ACT_GRAD = 1, /* fold activation gradients into the next layer's dX epilogue */
+  TDH_NET_GRAPH         = 2  /* replay the step as a captured HIP graph */
+};
+
+int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int flags,
+                   tdh_net **net);
+int tdh_net_destroy(tdh_net *net);
+size_t tdh_net_in_size(const tdh_net *net);
+size_t tdh_net_out_size(const tdh_net *net);
+size_t tdh_net_layer_out_size(const tdh_net *net, int layer);
+/* which: 0 = weight, 1 = bias; sizes in floats */
+size_t tdh_net_param_size(const tdh_net *net, int layer, int which);
+int tdh_net_set_param(tdh_net *net, int layer, int which, const float *host_src);
+int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst);
+/* device views valid until the net is destroyed */
+float *tdh_net_param(tdh_net *net, int layer, int which);
+const float *tdh_net_layer_out(const tdh_net *net, int layer);
+const float *tdh_net_layer_dx(const tdh_net *net, int layer);
+const float *tdh_net_layer_grad(const tdh_net *net, int layer, int which);
+const int32_t *tdh_net_layer_argmax(const tdh_net *net, int layer);
+/* x: [batch][in_size], t: [batch][out_size], device pointers */
+int tdh_net_forward(tdh_net *net, int batch, const float *x);
+/* fprop, loss gradient, bprop and (do_update != 0) update_weights + clear_grads */
+int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
+                       const float *t, int do_update);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TDH_H */

@@ -1,0 +1,410 @@
+"""tiny-cnn_amd — tiny-dnn's training hot path on one MI355X.
+
+This module is the Python face of ``libtdh.so`` (hand-written HIP for gfx950, C ABI in
+``include/tdh.h``). It only marshals numpy arrays to device buffers and calls the library;
+there is no CPU fallback: importing works without a GPU (so the ABI can be inspected),
+but every compute entry point needs the built library and a device, and raises otherwise.
+
+The directory name carries a hyphen, so load it with ``importlib`` (see ``load()`` in
+``__graft_entry__.py``) or put this directory's parent on ``sys.path`` and use
+``importlib.import_module("tiny-cnn_amd")``.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libtdh.so")
+CSRC = os.path.join(HERE, "csrc")
+HEADER = os.path.join(os.path.dirname(HERE), "include", "tdh.h")
+
+ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3}
+LOSS = {"mse": 0, "ce_multiclass": 1, "ce": 2}
+OPT = {"sgd": 0, "momentum": 1, "adam": 2, "adagrad": 3, "rmsprop": 4, "adamax": 5, "nesterov": 6}
+L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT = range(5)
+NET_FUSE_ACT_GRAD, NET_GRAPH = 1, 2
+
+f32p = C.POINTER(C.c_float)
+
+
+class TdhError(RuntimeError):
+    """A libtdh call failed (the reference raises nn_error in the same places)."""
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "in_w", "in_h", "in_c", "k_w", "k_h", "out_c", "w_stride", "h_stride",
+        "w_dilation", "h_dilation", "pad_same", "has_bias")] + [("tbl", C.c_void_p)]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "in_w", "in_h", "in_c", "pool_w", "pool_h", "stride_w", "stride_h", "pad_same",
+        "ceil_mode")]
+
+
+class OptDesc(C.Structure):
+    _fields_ = [("kind", C.c_int32)] + [(n, C.c_float) for n in (
+        "alpha", "lam", "mu", "b1", "b2", "eps", "b1_t", "b2_t")]
+
+
+class LayerDesc(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("act", C.c_int32), ("conv", ConvDesc), ("pool", PoolDesc),
+                ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32)]
+
+
+def build(verbose=False):
+    """Compile libtdh.so for gfx950 (hipcc cross-compiles; no GPU needed)."""
+    r = subprocess.run(["make", "-C", CSRC, "-j8"], capture_output=True, text=True)
+    if verbose or r.returncode != 0:
+        print(r.stdout[-4000:])
+        print(r.stderr[-4000:])
+    if r.returncode != 0:
+        raise TdhError("building libtdh.so failed")
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library. Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TdhError(f"{LIB_PATH} is missing: run build() (make -C tiny-cnn_amd/csrc) first")
+        l = C.CDLL(LIB_PATH)
+        l.tdh_last_error.restype = C.c_char_p
+        l.tdh_version.restype = C.c_char_p
+        for n in ("tdh_net_in_size", "tdh_net_out_size", "tdh_net_layer_out_size",
+                  "tdh_net_param_size"):
+            getattr(l, n).restype = C.c_size_t
+        for n in ("tdh_net_param", "tdh_net_layer_out", "tdh_net_layer_dx", "tdh_net_layer_grad",
+                  "tdh_net_layer_argmax"):
+            getattr(l, n).restype = C.c_void_p
+        l.tdh_opt_default.restype = None
+        _lib = l
+    return _lib
+
+
+def check(rc, what=""):
+    if rc != 0:
+        raise TdhError(f"{what}: [{rc}] {lib().tdh_last_error().decode()}")
+
+
+_inited = False
+
+
+def init(device=0):
+    global _inited
+    check(lib().tdh_init(device), "tdh_init")
+    _inited = True
+
+
+def device_info():
+    name = C.create_string_buffer(256)
+    cus = C.c_int32()
+    mem = C.c_size_t()
+    check(lib().tdh_device_info(name, 256, C.byref(cus), C.byref(mem)), "tdh_device_info")
+    return name.value.decode(), cus.value, mem.value
+
+
+def sync():
+    check(lib().tdh_sync(), "tdh_sync")
+
+
+class DevBuf:
+    """A device allocation with the shape/dtype of the numpy array it mirrors."""
+
+    def __init__(self, shape, dtype=np.float32, zero=False):
+        self.shape = tuple(shape) if not np.isscalar(shape) else (int(shape),)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = C.c_void_p()
+        check(lib().tdh_malloc(C.byref(p), C.c_size_t(self.nbytes)), "tdh_malloc")
+        self.ptr = p
+        self.owned = True
+        if zero and self.nbytes:
+            check(lib().tdh_fill_zero(self.ptr, C.c_size_t(self.nbytes)), "tdh_fill_zero")
+
+    @classmethod
+    def view(cls, ptr, shape, dtype=np.float32):
+        self = cls.__new__(cls)
+        self.shape = tuple(shape)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        self.ptr = C.c_void_p(ptr)
+        self.owned = False
+        return self
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a, dtype=self.dtype)
+        assert a.nbytes == self.nbytes, (a.shape, self.shape)
+        check(lib().tdh_memcpy_h2d(self.ptr, a.ctypes.data_as(C.c_void_p), C.c_size_t(self.nbytes)),
+              "tdh_memcpy_h2d")
+        return self
+
+    def numpy(self):
+        out = np.empty(self.shape, self.dtype)
+        check(lib().tdh_memcpy_d2h(out.ctypes.data_as(C.c_void_p), self.ptr,
+                                   C.c_size_t(self.nbytes)), "tdh_memcpy_d2h")
+        return out
+
+    def free(self):
+        if getattr(self, "owned", False) and self.ptr:
+            lib().tdh_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def to_device(a, dtype=np.float32):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return DevBuf(a.shape, dtype).upload(a)
+
+
+class Event:
+    def __init__(self):
+        p = C.c_void_p()
+        check(lib().tdh_event_create(C.byref(p)), "tdh_event_create")
+        self.ptr = p
+
+    def record(self):
+        check(lib().tdh_event_record(self.ptr), "tdh_event_record")
+
+    def elapsed_ms_since(self, start):
+        ms = C.c_float()
+        check(lib().tdh_event_elapsed_ms(start.ptr, self.ptr, C.byref(ms)), "tdh_event_elapsed_ms")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().tdh_event_destroy(self.ptr)
+        except Exception:
+            pass
+
+
+# ------------------------------------------------------------------ descriptors
+
+def conv_desc(in_w, in_h, in_c, k_w, k_h, out_c, pad_same=False, has_bias=True, w_stride=1,
+              h_stride=1, w_dilation=1, h_dilation=1, tbl=None):
+    d = ConvDesc(in_w, in_h, in_c, k_w, k_h, out_c, w_stride, h_stride, w_dilation, h_dilation,
+                 int(pad_same), int(has_bias), None)
+    if tbl is not None:
+        keep = np.ascontiguousarray(np.asarray(tbl, dtype=np.uint8).reshape(in_c, out_c))
+        d._keep = keep
+        d.tbl = keep.ctypes.data
+    return d
+
+
+def pool_desc(in_w, in_h, in_c, pool_w, pool_h=None, stride_w=None, stride_h=None,
+              pad_same=False, ceil_mode=False):
+    pool_h = pool_w if pool_h is None else pool_h
+    stride_w = pool_w if stride_w is None else stride_w
+    stride_h = pool_h if stride_h is None else stride_h
+    return PoolDesc(in_w, in_h, in_c, pool_w, pool_h, stride_w, stride_h, int(pad_same),
+                    int(ceil_mode))
+
+
+def opt_desc(kind, **kw):
+    o = OptDesc()
+    lib().tdh_opt_default(C.byref(o), OPT[kind] if isinstance(kind, str) else kind)
+    for k, v in kw.items():
+        setattr(o, "lam" if k == "lambda_" else k, v)
+    return o
+
+
+def conv_out_shape(d):
+    return lib().tdh_conv_out_w(C.byref(d)), lib().tdh_conv_out_h(C.byref(d))
+
+
+def pool_out_shape(d):
+    return lib().tdh_pool_out_w(C.byref(d)), lib().tdh_pool_out_h(C.byref(d))
+
+
+# ------------------------------------------------- operators on device buffers
+
+def _p(buf):
+    return buf.ptr if buf is not None else None
+
+
+def conv2d_fwd(d, batch, x, w, b, y):
+    check(lib().tdh_conv2d_fwd(C.byref(d), batch, _p(x), _p(w), _p(b), _p(y)), "tdh_conv2d_fwd")
+
+
+def conv2d_bwd(d, batch, x, w, dy, dx, dw, db, accumulate=False):
+    check(lib().tdh_conv2d_bwd(C.byref(d), batch, _p(x), _p(w), _p(dy), _p(dx), _p(dw), _p(db),
+                               int(accumulate)), "tdh_conv2d_bwd")
+
+
+def fc_fwd(n_in, n_out, has_bias, batch, x, w, b, y):
+    check(lib().tdh_fc_fwd(n_in, n_out, int(has_bias), batch, _p(x), _p(w), _p(b), _p(y)),
+          "tdh_fc_fwd")
+
+
+def fc_bwd(n_in, n_out, has_bias, batch, x, w, dy, dx, dw, db, accumulate=False):
+    check(lib().tdh_fc_bwd(n_in, n_out, int(has_bias), batch, _p(x), _p(w), _p(dy), _p(dx), _p(dw),
+                           _p(db), int(accumulate)), "tdh_fc_bwd")
+
+
+def maxpool_fwd(d, batch, x, y, argmax):
+    check(lib().tdh_maxpool_fwd(C.byref(d), batch, _p(x), _p(y), _p(argmax)), "tdh_maxpool_fwd")
+
+
+def maxpool_bwd(d, batch, dy, argmax, dx):
+    check(lib().tdh_maxpool_bwd(C.byref(d), batch, _p(dy), _p(argmax), _p(dx)), "tdh_maxpool_bwd")
+
+
+def avepool_fwd(d, batch, x, w, b, y):
+    check(lib().tdh_avepool_fwd(C.byref(d), batch, _p(x), _p(w), _p(b), _p(y)), "tdh_avepool_fwd")
+
+
+def avepool_bwd(d, batch, x, w, dy, dx, dw, db, accumulate=False):
+    check(lib().tdh_avepool_bwd(C.byref(d), batch, _p(x), _p(w), _p(dy), _p(dx), _p(dw), _p(db),
+                                int(accumulate)), "tdh_avepool_bwd")
+
+
+def act_fwd(kind, batch, length, x, y):
+    check(lib().tdh_act_fwd(ACT[kind], batch, length, _p(x), _p(y)), "tdh_act_fwd")
+
+
+def act_bwd(kind, batch, length, y, dy, dx):
+    check(lib().tdh_act_bwd(ACT[kind], batch, length, _p(y), _p(dy), _p(dx)), "tdh_act_bwd")
+
+
+def loss_grad(kind, batch, length, y, t, dy):
+    check(lib().tdh_loss_grad(LOSS[kind], batch, length, _p(y), _p(t), _p(dy)), "tdh_loss_grad")
+
+
+def softmax_xent_grad(batch, length, y, t, dz):
+    check(lib().tdh_softmax_xent_grad(batch, length, _p(y), _p(t), _p(dz)),
+          "tdh_softmax_xent_grad")
+
+
+def opt_update(o, n, merged_grad, w, s0=None, s1=None, grad_scale=1.0):
+    check(lib().tdh_opt_update(C.byref(o), C.c_size_t(n), _p(merged_grad), C.c_float(grad_scale),
+                               _p(w), _p(s0), _p(s1)), "tdh_opt_update")
+
+
+# ------------------------------------------------------------ sequential net
+
+def L_conv(in_w, in_h, in_c, k, out_c, pad_same=False, has_bias=True, stride=1, tbl=None):
+    l = LayerDesc()
+    l.kind = L_CONV
+    l.conv = conv_desc(in_w, in_h, in_c, k, k, out_c, pad_same, has_bias, stride, stride, tbl=tbl)
+    l._keep = getattr(l.conv, "_keep", None)
+    return l
+
+
+def L_fc(n_in, n_out, has_bias=True):
+    l = LayerDesc()
+    l.kind, l.fc_in, l.fc_out, l.fc_bias = L_FC, n_in, n_out, int(has_bias)
+    return l
+
+
+def L_maxpool(in_w, in_h, in_c, pool, stride=None):
+    l = LayerDesc()
+    l.kind = L_MAXPOOL
+    l.pool = pool_desc(in_w, in_h, in_c, pool, stride_w=stride)
+    return l
+
+
+def L_avepool(in_w, in_h, in_c, pool, stride=None):
+    l = LayerDesc()
+    l.kind = L_AVEPOOL
+    l.pool = pool_desc(in_w, in_h, in_c, pool, stride_w=stride)
+    return l
+
+
+def L_act(kind):
+    l = LayerDesc()
+    l.kind, l.act = L_ACT, ACT[kind]
+    return l
+
+
+class Net:
+    """network<sequential> with device-resident tensors (tdh_net_*)."""
+
+    def __init__(self, layers, max_batch, flags=0):
+        self.layers = list(layers)
+        arr = (LayerDesc * len(layers))()
+        for i, l in enumerate(layers):
+            arr[i] = l
+        self._arr = arr
+        h = C.c_void_p()
+        check(lib().tdh_net_create(arr, len(layers), max_batch, flags, C.byref(h)),
+              "tdh_net_create")
+        self.h = h
+        self.n = len(layers)
+        self.max_batch = max_batch
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().tdh_net_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def in_size(self):
+        return lib().tdh_net_in_size(self.h)
+
+    def out_size(self):
+        return lib().tdh_net_out_size(self.h)
+
+    def layer_out_size(self, i):
+        return lib().tdh_net_layer_out_size(self.h, i)
+
+    def param_size(self, i, which):
+        return lib().tdh_net_param_size(self.h, i, which)
+
+    def params(self):
+        """[(layer, which, size)] in update order (weight before bias, front to back)."""
+        return [(i, k, self.param_size(i, k)) for i in range(self.n) for k in (0, 1)
+                if self.param_size(i, k)]
+
+    def set_param(self, i, which, a):
+        a = np.ascontiguousarray(a, dtype=np.float32).ravel()
+        assert a.size == self.param_size(i, which)
+        check(lib().tdh_net_set_param(self.h, i, which, a.ctypes.data_as(f32p)),
+              "tdh_net_set_param")
+
+    def get_param(self, i, which):
+        a = np.empty(self.param_size(i, which), np.float32)
+        check(lib().tdh_net_get_param(self.h, i, which, a.ctypes.data_as(f32p)),
+              "tdh_net_get_param")
+        return a
+
+    def layer_out(self, i, batch):
+        n = self.layer_out_size(i)
+        return DevBuf.view(lib().tdh_net_layer_out(self.h, i), (batch, n)).numpy()
+
+    def layer_dx(self, i, batch):
+        n = self.in_size() if i == 0 else self.layer_out_size(i - 1)
+        return DevBuf.view(lib().tdh_net_layer_dx(self.h, i), (batch, n)).numpy()
+
+    def layer_grad(self, i, which):
+        n = self.param_size(i, which)
+        return DevBuf.view(lib().tdh_net_layer_grad(self.h, i, which), (n,)).numpy()
+
+    def layer_argmax(self, i, batch):
+        n = self.layer_out_size(i)
+        return DevBuf.view(lib().tdh_net_layer_argmax(self.h, i), (batch, n), np.int32).numpy()
+
+    def forward(self, batch, x):
+        check(lib().tdh_net_forward(self.h, batch, _p(x)), "tdh_net_forward")
+
+    def train_step(self, opt, loss, batch, x, t, do_update=True):
+        check(lib().tdh_net_train_step(self.h, C.byref(opt) if opt is not None else None,
+                                       LOSS[loss], batch, _p(x), _p(t), int(do_update)),
+              "tdh_net_train_step")

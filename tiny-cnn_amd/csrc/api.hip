@@ -1,0 +1,412 @@
+// api.hip — library state, device memory, events and the thin extern "C" layer that
+// validates arguments before anything is launched.
+#include <cmath>
+#include <cstring>
+
+#include "common.h"
+
+namespace tdh {
+
+Context &ctx() {
+  static Context c;
+  return c;
+}
+
+static thread_local char g_error[512] = "";
+
+int set_error(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int ws_begin(size_t total) {
+  Context &c = ctx();
+  c.workspace_off = 0;
+  if (total <= c.workspace_size) return TDH_OK;
+  if (c.ws_locked)
+    return set_error(TDH_ERR_INVALID, "scratch reservation of %zu bytes exceeds the locked %zu",
+                     total, c.workspace_size);
+  if (c.workspace) TDH_HIP(hipFree(c.workspace));
+  c.workspace      = nullptr;
+  c.workspace_size = 0;
+  const size_t want = ws_align(total + (total >> 2));
+  void *p           = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    return set_error(TDH_ERR_OOM, "cannot allocate %zu bytes of scratch", want);
+  }
+  c.workspace      = static_cast<char *>(p);
+  c.workspace_size = want;
+  return TDH_OK;
+}
+
+int ws_take(size_t bytes, void **out) {
+  Context &c = ctx();
+  const size_t need = ws_align(bytes);
+  if (c.workspace_off + need > c.workspace_size)
+    return set_error(TDH_ERR_INVALID, "scratch overrun: %zu + %zu > %zu (reservation too small)",
+                     c.workspace_off, need, c.workspace_size);
+  *out = c.workspace + c.workspace_off;
+  c.workspace_off += need;
+  return TDH_OK;
+}
+
+// tiny_dnn/util/util.h:329-344
+int conv_out_length(int in_length, int window, int stride, int dilation, int pad_same) {
+  const int output_length = pad_same ? in_length : in_length - dilation * window + dilation;
+  return (output_length + stride - 1) / stride;
+}
+
+// tiny_dnn/util/util.h:346-363: the quotient is formed in float, then floor/ceil
+int pool_out_length(int in_length, int window, int stride, int ceil_mode, int pad_same) {
+  const int output_length = pad_same ? in_length : in_length - window + 1;
+  const float tmp = static_cast<float>(output_length + stride - 1) / static_cast<float>(stride);
+  return static_cast<int>(ceil_mode ? std::ceil(tmp) : std::floor(tmp));
+}
+
+static int check_conv_desc(const tdh_conv_desc *d, int batch, bool backward) {
+  TDH_CHECK_ARG(d != nullptr, "conv: null descriptor");
+  TDH_CHECK_ARG(batch >= 0, "conv: negative batch %d", batch);
+  TDH_CHECK_ARG(d->in_w > 0 && d->in_h > 0 && d->in_c > 0 && d->out_c > 0 && d->k_w > 0 &&
+                  d->k_h > 0,
+                "conv: non-positive dimension");
+  TDH_CHECK_ARG(d->w_stride > 0 && d->h_stride > 0 && d->w_dilation > 0 && d->h_dilation > 0,
+                "conv: stride and dilation must be positive");
+  if (backward && (d->w_dilation != 1 || d->h_dilation != 1))
+    return set_error(TDH_ERR_UNSUPPORTED,
+                     "conv backward with dilation %dx%d: the reference's backward kernel ignores "
+                     "dilation, so no defined result exists to match",
+                     d->w_dilation, d->h_dilation);
+  if (!d->pad_same)
+    TDH_CHECK_ARG(d->in_w >= d->w_dilation * (d->k_w - 1) + 1 &&
+                    d->in_h >= d->h_dilation * (d->k_h - 1) + 1,
+                  "conv: window larger than the input");
+  const long ow = conv_out_length(d->in_w, d->k_w, d->w_stride, d->w_dilation, d->pad_same);
+  const long oh = conv_out_length(d->in_h, d->k_h, d->h_stride, d->h_dilation, d->pad_same);
+  const long lim = 1L << 31;
+  TDH_CHECK_ARG(static_cast<long>(batch) * d->in_c * d->in_h * d->in_w < lim &&
+                  static_cast<long>(batch) * d->out_c * oh * ow < lim &&
+                  static_cast<long>(d->out_c) * d->in_c * d->k_h * d->k_w < lim,
+                "conv: tensor exceeds 2^31 elements");
+  return TDH_OK;
+}
+
+static int check_pool_desc(const tdh_pool_desc *d, int batch) {
+  TDH_CHECK_ARG(d != nullptr, "pool: null descriptor");
+  TDH_CHECK_ARG(batch >= 0, "pool: negative batch %d", batch);
+  TDH_CHECK_ARG(d->in_w > 0 && d->in_h > 0 && d->in_c > 0 && d->pool_w > 0 && d->pool_h > 0 &&
+                  d->stride_w > 0 && d->stride_h > 0,
+                "pool: non-positive dimension");
+  if (!d->pad_same)
+    TDH_CHECK_ARG(d->in_w >= d->pool_w && d->in_h >= d->pool_h, "pool: window larger than input");
+  TDH_CHECK_ARG(static_cast<long>(batch) * d->in_c * d->in_h * d->in_w < (1L << 31),
+                "pool: tensor exceeds 2^31 elements");
+  return TDH_OK;
+}
+
+}  // namespace tdh
+
+using namespace tdh;
+
+extern "C" {
+
+const char *tdh_version(void) { return "tdh 0.1 (gfx950)"; }
+
+const char *tdh_last_error(void) { return g_error; }
+
+int tdh_init(int device) {
+  Context &c = ctx();
+  if (c.ready && c.device == device) return TDH_OK;
+  if (c.ready) TDH_TRY(tdh_shutdown());
+  int count = 0;
+  TDH_HIP(hipGetDeviceCount(&count));
+  TDH_CHECK_ARG(device >= 0 && device < count, "tdh_init: device %d of %d", device, count);
+  TDH_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  TDH_HIP(hipGetDeviceProperties(&prop, device));
+  std::snprintf(c.name, sizeof(c.name), "%s (%s)", prop.name, prop.gcnArchName);
+  c.compute_units = prop.multiProcessorCount;
+  c.global_mem    = prop.totalGlobalMem;
+  TDH_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+  c.device = device;
+  c.ready  = true;
+  return TDH_OK;
+}
+
+int tdh_shutdown(void) {
+  Context &c = ctx();
+  if (!c.ready) return TDH_OK;
+  TDH_HIP(hipStreamSynchronize(c.stream));
+  if (c.workspace) TDH_HIP(hipFree(c.workspace));
+  TDH_HIP(hipStreamDestroy(c.stream));
+  c = Context();
+  return TDH_OK;
+}
+
+int tdh_device_info(char *name, size_t name_len, int32_t *compute_units, size_t *global_mem_bytes) {
+  TDH_REQUIRE_INIT();
+  if (name && name_len) std::snprintf(name, name_len, "%s", ctx().name);
+  if (compute_units) *compute_units = ctx().compute_units;
+  if (global_mem_bytes) *global_mem_bytes = ctx().global_mem;
+  return TDH_OK;
+}
+
+int tdh_malloc(void **dptr, size_t bytes) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(dptr != nullptr, "tdh_malloc: null result pointer");
+  *dptr = nullptr;
+  if (bytes == 0) bytes = 4;
+  if (hipMalloc(dptr, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return set_error(TDH_ERR_OOM, "tdh_malloc: cannot allocate %zu bytes", bytes);
+  }
+  return TDH_OK;
+}
+
+int tdh_free(void *dptr) {
+  TDH_REQUIRE_INIT();
+  if (dptr) TDH_HIP(hipFree(dptr));
+  return TDH_OK;
+}
+
+int tdh_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+  TDH_REQUIRE_INIT();
+  if (bytes == 0) return TDH_OK;
+  TDH_CHECK_ARG(dst && src, "tdh_memcpy_h2d: null pointer");
+  TDH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
+  TDH_HIP(hipStreamSynchronize(ctx().stream));  // the host buffer may be reused on return
+  return TDH_OK;
+}
+
+int tdh_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+  TDH_REQUIRE_INIT();
+  if (bytes == 0) return TDH_OK;
+  TDH_CHECK_ARG(dst && src, "tdh_memcpy_d2h: null pointer");
+  TDH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  return TDH_OK;
+}
+
+int tdh_memcpy_d2d(void *dst, const void *src, size_t bytes) {
+  TDH_REQUIRE_INIT();
+  if (bytes == 0) return TDH_OK;
+  TDH_CHECK_ARG(dst && src, "tdh_memcpy_d2d: null pointer");
+  TDH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));
+  return TDH_OK;
+}
+
+int tdh_fill_zero(void *dptr, size_t bytes) {
+  TDH_REQUIRE_INIT();
+  if (bytes == 0) return TDH_OK;
+  TDH_CHECK_ARG(dptr != nullptr, "tdh_fill_zero: null pointer");
+  TDH_CHECK_ARG(bytes % 4 == 0, "tdh_fill_zero: size %zu is not a multiple of 4", bytes);
+  return launch_fill_zero(dptr, bytes);
+}
+
+int tdh_sync(void) {
+  TDH_REQUIRE_INIT();
+  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  return TDH_OK;
+}
+
+int tdh_event_create(void **event) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(event != nullptr, "tdh_event_create: null result pointer");
+  hipEvent_t e;
+  TDH_HIP(hipEventCreate(&e));
+  *event = e;
+  return TDH_OK;
+}
+
+int tdh_event_destroy(void *event) {
+  TDH_REQUIRE_INIT();
+  if (event) TDH_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return TDH_OK;
+}
+
+int tdh_event_record(void *event) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(event != nullptr, "tdh_event_record: null event");
+  TDH_HIP(hipEventRecord(static_cast<hipEvent_t>(event), ctx().stream));
+  return TDH_OK;
+}
+
+int tdh_event_elapsed_ms(void *start, void *stop, float *ms) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(start && stop && ms, "tdh_event_elapsed_ms: null argument");
+  TDH_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+  TDH_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return TDH_OK;
+}
+
+int tdh_conv_out_w(const tdh_conv_desc *d) {
+  return conv_out_length(d->in_w, d->k_w, d->w_stride, d->w_dilation, d->pad_same);
+}
+int tdh_conv_out_h(const tdh_conv_desc *d) {
+  return conv_out_length(d->in_h, d->k_h, d->h_stride, d->h_dilation, d->pad_same);
+}
+int tdh_pool_out_w(const tdh_pool_desc *d) {
+  return pool_out_length(d->in_w, d->pool_w, d->stride_w, d->ceil_mode, d->pad_same);
+}
+int tdh_pool_out_h(const tdh_pool_desc *d) {
+  return pool_out_length(d->in_h, d->pool_h, d->stride_h, d->ceil_mode, d->pad_same);
+}
+
+// ------------------------------------------------------------------ operators
+
+int tdh_conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w,
+                   const float *b, float *y) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_conv_desc(d, batch, false));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && y, "tdh_conv2d_fwd: null tensor");
+  TDH_CHECK_ARG(!d->has_bias || b, "tdh_conv2d_fwd: has_bias set but b is null");
+  TDH_TRY(ws_begin(conv2d_workspace_bytes(d, batch)));
+  return conv2d_fwd(d, batch, x, w, b, y);
+}
+
+int tdh_conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w,
+                   const float *dy, float *dx, float *dw, float *db, int accumulate) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_conv_desc(d, batch, true));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && dy, "tdh_conv2d_bwd: null tensor");
+  TDH_TRY(ws_begin(conv2d_workspace_bytes(d, batch)));
+  return conv2d_bwd(d, batch, x, w, dy, dx, dw, d->has_bias ? db : nullptr, accumulate, ActGrad());
+}
+
+int tdh_fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+               const float *b, float *y) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(in > 0 && out > 0 && batch >= 0, "tdh_fc_fwd: bad shape %d->%d batch %d", in, out,
+                batch);
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && y, "tdh_fc_fwd: null tensor");
+  TDH_CHECK_ARG(!has_bias || b, "tdh_fc_fwd: has_bias set but b is null");
+  TDH_CHECK_ARG(static_cast<long>(in) * out < (1L << 31) &&
+                  static_cast<long>(batch) * in < (1L << 31) &&
+                  static_cast<long>(batch) * out < (1L << 31),
+                "tdh_fc_fwd: tensor exceeds 2^31 elements");
+  TDH_TRY(ws_begin(fc_workspace_bytes(in, out, batch)));
+  return fc_fwd(in, out, has_bias, batch, x, w, b, y);
+}
+
+int tdh_fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+               const float *dy, float *dx, float *dw, float *db, int accumulate) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(in > 0 && out > 0 && batch >= 0, "tdh_fc_bwd: bad shape %d->%d batch %d", in, out,
+                batch);
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && dy, "tdh_fc_bwd: null tensor");
+  TDH_CHECK_ARG(static_cast<long>(in) * out < (1L << 31) &&
+                  static_cast<long>(batch) * in < (1L << 31) &&
+                  static_cast<long>(batch) * out < (1L << 31),
+                "tdh_fc_bwd: tensor exceeds 2^31 elements");
+  TDH_TRY(ws_begin(fc_workspace_bytes(in, out, batch)));
+  return fc_bwd(in, out, has_bias, batch, x, w, dy, dx, dw, has_bias ? db : nullptr, accumulate,
+                ActGrad());
+}
+
+int tdh_maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_pool_desc(d, batch));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && y, "tdh_maxpool_fwd: null tensor");
+  return maxpool_fwd(d, batch, x, y, argmax);
+}
+
+int tdh_maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
+                    float *dx) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_pool_desc(d, batch));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(dy && argmax && dx, "tdh_maxpool_bwd: null tensor");
+  return maxpool_bwd(d, batch, dy, argmax, dx);
+}
+
+int tdh_avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w,
+                    const float *b, float *y) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_pool_desc(d, batch));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && b && y, "tdh_avepool_fwd: null tensor");
+  return avepool_fwd(d, batch, x, w, b, y);
+}
+
+int tdh_avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w,
+                    const float *dy, float *dx, float *dw, float *db, int accumulate) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_pool_desc(d, batch));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && dy, "tdh_avepool_bwd: null tensor");
+  TDH_TRY(ws_begin(avepool_workspace_bytes(d, batch)));
+  return avepool_bwd(d, batch, x, w, dy, dx, dw, db, accumulate);
+}
+
+int tdh_act_fwd(int kind, int batch, int len, const float *x, float *y) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_act_fwd: negative size");
+  if (batch == 0 || len == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && y, "tdh_act_fwd: null tensor");
+  TDH_CHECK_ARG(static_cast<long>(batch) * len < (1L << 31), "tdh_act_fwd: tensor too large");
+  return launch_act_fwd(kind, batch, len, x, y);
+}
+
+int tdh_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_act_bwd: negative size");
+  if (batch == 0 || len == 0) return TDH_OK;
+  TDH_CHECK_ARG(y && dy && dx, "tdh_act_bwd: null tensor");
+  TDH_CHECK_ARG(static_cast<long>(batch) * len < (1L << 31), "tdh_act_bwd: tensor too large");
+  return launch_act_bwd(kind, batch, len, y, dy, dx);
+}
+
+int tdh_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_loss_grad: negative size");
+  if (batch == 0 || len == 0) return TDH_OK;
+  TDH_CHECK_ARG(y && t && dy, "tdh_loss_grad: null tensor");
+  return launch_loss_grad(kind, batch, len, y, t, dy);
+}
+
+int tdh_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_softmax_xent_grad: negative size");
+  if (batch == 0 || len == 0) return TDH_OK;
+  TDH_CHECK_ARG(y && t && dz, "tdh_softmax_xent_grad: null tensor");
+  return launch_softmax_xent_grad(batch, len, y, t, dz);
+}
+
+// constructor defaults of tiny_dnn/optimizers/optimizer.h
+void tdh_opt_default(tdh_opt *o, int kind) {
+  std::memset(o, 0, sizeof(*o));
+  o->kind = kind;
+  switch (kind) {
+    case TDH_OPT_SGD: o->alpha = 0.01f; break;
+    case TDH_OPT_MOMENTUM:
+    case TDH_OPT_NESTEROV: o->alpha = 0.01f; o->mu = 0.9f; break;
+    case TDH_OPT_ADAM:
+      o->alpha = 0.001f; o->b1 = 0.9f; o->b2 = 0.999f; o->b1_t = 0.9f; o->b2_t = 0.999f;
+      o->eps = 1e-8f;
+      break;
+    case TDH_OPT_ADAGRAD: o->alpha = 0.01f; o->eps = 1e-8f; break;
+    case TDH_OPT_RMSPROP: o->alpha = 0.0001f; o->mu = 0.99f; o->eps = 1e-8f; break;
+    case TDH_OPT_ADAMAX:
+      o->alpha = 0.002f; o->b1 = 0.9f; o->b2 = 0.999f; o->b1_t = 0.9f; o->eps = 1e-8f;
+      break;
+  }
+}
+
+int tdh_opt_update(tdh_opt *o, size_t n, const float *merged_grad, float grad_scale, float *w,
+                   float *s0, float *s1) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(o != nullptr, "tdh_opt_update: null optimizer");
+  if (n == 0) return launch_opt_update(o, 0, nullptr, grad_scale, nullptr, nullptr, nullptr);
+  TDH_CHECK_ARG(merged_grad && w, "tdh_opt_update: null tensor");
+  return launch_opt_update(o, n, merged_grad, grad_scale, w, s0, s1);
+}
+
+}  // extern "C"

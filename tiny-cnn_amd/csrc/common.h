@@ -1,0 +1,154 @@
+// common.h — library context, error plumbing and small device helpers shared by
+// every translation unit of libtdh.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/tdh.h"
+
+namespace tdh {
+
+// ---------------------------------------------------------------- context
+struct Context {
+  bool ready            = false;
+  int device            = -1;
+  hipStream_t stream    = nullptr;
+  int compute_units     = 0;
+  size_t global_mem     = 0;
+  char name[256]        = {0};
+  // grow-only scratch for split-K partial sums and staged reductions; every public op
+  // reserves its whole need up front (ws_begin) and then carves pieces off (ws_take), so
+  // the buffer never moves while an op is queueing kernels
+  char *workspace       = nullptr;
+  size_t workspace_size = 0;
+  size_t workspace_off  = 0;
+  bool ws_locked        = false;  // a network owns the reservation: ops must fit, never grow
+};
+
+Context &ctx();
+int set_error(int code, const char *fmt, ...);
+// Makes sure the scratch buffer holds `total` bytes and rewinds it. Growing frees and
+// reallocates (hipFree waits for queued kernels), which is refused while ws_locked.
+int ws_begin(size_t total);
+// Next 256-byte aligned piece of the reserved scratch.
+int ws_take(size_t bytes, void **out);
+inline size_t ws_align(size_t bytes) { return (bytes + 255) & ~static_cast<size_t>(255); }
+
+#define TDH_REQUIRE_INIT()                                                     \
+  do {                                                                         \
+    if (!::tdh::ctx().ready)                                                   \
+      return ::tdh::set_error(TDH_ERR_NOT_INIT, "%s: tdh_init has not been called", __func__); \
+  } while (0)
+
+#define TDH_CHECK_ARG(cond, ...)                                               \
+  do {                                                                         \
+    if (!(cond)) return ::tdh::set_error(TDH_ERR_INVALID, __VA_ARGS__);         \
+  } while (0)
+
+#define TDH_HIP(call)                                                          \
+  do {                                                                         \
+    hipError_t e_ = (call);                                                    \
+    if (e_ != hipSuccess)                                                      \
+      return ::tdh::set_error(TDH_ERR_HIP, "%s:%d %s -> %s", __FILE__, __LINE__, #call, \
+                              hipGetErrorString(e_));                          \
+  } while (0)
+
+#define TDH_LAUNCH_CHECK() TDH_HIP(hipGetLastError())
+
+#define TDH_TRY(call)                                                          \
+  do {                                                                         \
+    int rc_ = (call);                                                          \
+    if (rc_ != TDH_OK) return rc_;                                             \
+  } while (0)
+
+// ---------------------------------------------------------------- helpers
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline size_t ceil_div_sz(size_t a, size_t b) { return (a + b - 1) / b; }
+
+// Division by a runtime constant as multiply-high + shift. Exact for 0 <= n < 2^31.
+struct FastDiv {
+  uint32_t d = 1, mul = 1, shift = 0;
+  FastDiv() = default;
+  explicit FastDiv(uint32_t divisor) : d(divisor) {
+    shift = 0;
+    while ((1u << shift) < d && shift < 31) ++shift;
+    const uint64_t one = 1;
+    mul = static_cast<uint32_t>(((one << 32) * ((one << shift) - d)) / d + 1);
+  }
+  __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t t = __umulhi(mul, n);
+#else
+    const uint32_t t = static_cast<uint32_t>((static_cast<uint64_t>(mul) * n) >> 32);
+#endif
+    return (t + n) >> shift;
+  }
+  __host__ __device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const {
+    q = div(n);
+    r = n - q * d;
+  }
+};
+
+// shapes (tiny_dnn/util/util.h:329-363)
+int conv_out_length(int in_length, int window, int stride, int dilation, int pad_same);
+int pool_out_length(int in_length, int window, int stride, int ceil_mode, int pad_same);
+
+// ------------------------------------------------- internal launchers (device ptrs)
+// elementwise.hip
+int launch_fill_zero(void *p, size_t bytes);
+int launch_act_fwd(int kind, int batch, int len, const float *x, float *y);
+int launch_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx);
+int launch_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
+int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz);
+int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, float *w, float *s0,
+                      float *s1);
+// deterministic reductions: out[r] (+)= sum over `cols` contiguous values of row r,
+// rows laid out as [outer][rows][cols] and summed over outer in order
+int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate);
+size_t rowsum_workspace_bytes(int outer, int rows, int cols);
+// out[c] (+)= sum_s src[s*cols + c]
+int launch_colsum(const float *src, int rows, int cols, float *out, int accumulate);
+
+// activation-gradient factor fused into GEMM epilogues
+struct ActGrad {
+  int kind = TDH_ACT_NONE;  // TDH_ACT_TANH / RELU / SIGMOID or NONE
+  const float *y = nullptr; // activation OUTPUT, same indexing as the GEMM result
+};
+
+// conv.hip / fc.hip
+int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
+               float *y);
+int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
+               float *dx, float *dw, float *db, int accumulate, ActGrad dx_act);
+int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+           const float *b, float *y);
+int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
+           const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act);
+// workspace bytes the op may ask for (so a net can reserve it before graph capture)
+size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
+size_t fc_workspace_bytes(int in, int out, int batch);
+
+// pool.hip
+int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax);
+int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
+                float *dx);
+int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *b,
+                float *y);
+int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,
+                float *dx, float *dw, float *db, int accumulate);
+size_t avepool_workspace_bytes(const tdh_pool_desc *d, int batch);
+
+__device__ __forceinline__ float act_grad_factor(int kind, float y) {
+  switch (kind) {
+    case TDH_ACT_TANH: return 1.0f - y * y;
+    case TDH_ACT_RELU: return y > 0.0f ? 1.0f : 0.0f;
+    case TDH_ACT_SIGMOID: return y * (1.0f - y);
+    default: return 1.0f;
+  }
+}
+
+}  // namespace tdh

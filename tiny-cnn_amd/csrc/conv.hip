@@ -1,0 +1,296 @@
+// conv.hip — 2-D convolution forward and backward as implicit GEMMs (no im2col / col2im
+// buffer is ever materialised and padding::same costs no copies):
+//
+//   forward  Y[img][co][p]      M = Cout        N = batch*OH*OW   K = Cin*KH*KW
+//            A = W (OIHW rows), B = input gathered at (p, tap)
+//   dW       dW[co][ci,ky,kx]   M = Cout        N = Cin*KH*KW     K = batch*OH*OW
+//            A = dY, B = input gathered at (p, tap); K spans the whole batch, so the
+//            gradient leaves the kernel already reduced over samples
+//   dX       dX[img][ci][q]     M = Cin         N = batch*H*W     K = Cout*KH*KW
+//            A = W regrouped by input channel, B = dY gathered at the output positions
+//            whose window covers q (the gather form of the reference's scatter)
+//   db       row sums of dY per output channel, fixed two-stage order
+//
+// Reference: conv2d_op_internal.h:13-74 (forward), :78-181 (backward).
+#include "gemm_mfma.h"
+
+namespace tdh {
+
+namespace {
+
+struct ConvGeom {
+  int C, H, W, Kc, R, S, OH, OW;
+  int pad_h, pad_w, sh, sw, dh, dw;
+  FastDiv div_ohw, div_ow, div_rs, div_s, div_hw, div_w, div_sh, div_sw;
+};
+
+ConvGeom make_geom(const tdh_conv_desc *d) {
+  ConvGeom g;
+  g.C = d->in_c; g.H = d->in_h; g.W = d->in_w;
+  g.Kc = d->out_c; g.R = d->k_h; g.S = d->k_w;
+  g.OW = conv_out_length(d->in_w, d->k_w, d->w_stride, d->w_dilation, d->pad_same);
+  g.OH = conv_out_length(d->in_h, d->k_h, d->h_stride, d->h_dilation, d->pad_same);
+  // padding::same puts k/2 zeros before the data (conv_params.h:119-120)
+  g.pad_h = d->pad_same ? d->k_h / 2 : 0;
+  g.pad_w = d->pad_same ? d->k_w / 2 : 0;
+  g.sh = d->h_stride; g.sw = d->w_stride; g.dh = d->h_dilation; g.dw = d->w_dilation;
+  g.div_ohw = FastDiv(g.OH * g.OW); g.div_ow = FastDiv(g.OW);
+  g.div_rs = FastDiv(g.R * g.S); g.div_s = FastDiv(g.S);
+  g.div_hw = FastDiv(g.H * g.W); g.div_w = FastDiv(g.W);
+  g.div_sh = FastDiv(g.sh); g.div_sw = FastDiv(g.sw);
+  return g;
+}
+
+// forward B operand: n = (img, oy, ox), k = (ci, ky, kx) -> x[img][ci][oy*sh + ky*dh - pad][..]
+struct FwdInputOperand {
+  const float *x;
+  ConvGeom g;
+  int n_extent;
+  struct Fix {
+    int base, iy0, ix0;
+    bool valid;
+  };
+  struct KDec {
+    int coff, dy, dx;
+  };
+  __device__ __forceinline__ Fix fix(int n) const {
+    uint32_t img, p, oy, ox;
+    g.div_ohw.divmod(n, img, p);
+    g.div_ow.divmod(p, oy, ox);
+    return {static_cast<int>(img) * g.C * g.H * g.W, static_cast<int>(oy) * g.sh - g.pad_h,
+            static_cast<int>(ox) * g.sw - g.pad_w, n < n_extent};
+  }
+  __device__ __forceinline__ KDec kdec(int k) const {
+    uint32_t ci, t, ky, kx;
+    g.div_rs.divmod(k, ci, t);
+    g.div_s.divmod(t, ky, kx);
+    return {static_cast<int>(ci) * g.H * g.W, static_cast<int>(ky) * g.dh,
+            static_cast<int>(kx) * g.dw};
+  }
+  __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
+    const int iy = f.iy0 + k.dy, ix = f.ix0 + k.dx;
+    const bool ok = f.valid && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H) &&
+                    static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+    return ok ? x[f.base + k.coff + iy * g.W + ix] : 0.0f;
+  }
+};
+
+// dW A operand: m = co, k = (img, p) -> dy[img][co][p]
+struct DwDyOperand {
+  const float *dy;
+  int Kc, ohw;
+  FastDiv div_ohw;
+  struct Fix {
+    int off;
+    bool valid;
+  };
+  struct KDec {
+    int off;
+  };
+  __device__ __forceinline__ Fix fix(int m) const { return {m * ohw, m < Kc}; }
+  __device__ __forceinline__ KDec kdec(int k) const {
+    uint32_t img, p;
+    div_ohw.divmod(k, img, p);
+    return {static_cast<int>(img) * Kc * ohw + static_cast<int>(p)};
+  }
+  __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
+    return f.valid ? dy[f.off + k.off] : 0.0f;
+  }
+};
+
+// dW B operand: n = (ci, ky, kx), k = (img, oy, ox) -> x[img][ci][oy*sh + ky - pad][..]
+struct DwInputOperand {
+  const float *x;
+  ConvGeom g;
+  int n_extent;
+  struct Fix {
+    int coff, dy, dx;
+    bool valid;
+  };
+  struct KDec {
+    int base, iy0, ix0;
+  };
+  __device__ __forceinline__ Fix fix(int n) const {
+    uint32_t ci, t, ky, kx;
+    g.div_rs.divmod(n, ci, t);
+    g.div_s.divmod(t, ky, kx);
+    return {static_cast<int>(ci) * g.H * g.W, static_cast<int>(ky) - g.pad_h,
+            static_cast<int>(kx) - g.pad_w, n < n_extent};
+  }
+  __device__ __forceinline__ KDec kdec(int k) const {
+    uint32_t img, p, oy, ox;
+    g.div_ohw.divmod(k, img, p);
+    g.div_ow.divmod(p, oy, ox);
+    return {static_cast<int>(img) * g.C * g.H * g.W, static_cast<int>(oy) * g.sh,
+            static_cast<int>(ox) * g.sw};
+  }
+  __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
+    const int iy = k.iy0 + f.dy, ix = k.ix0 + f.dx;
+    const bool ok = f.valid && static_cast<unsigned>(iy) < static_cast<unsigned>(g.H) &&
+                    static_cast<unsigned>(ix) < static_cast<unsigned>(g.W);
+    return ok ? x[k.base + f.coff + iy * g.W + ix] : 0.0f;
+  }
+};
+
+// dX A operand: m = ci, k = (co, ky, kx) -> w[co][ci][ky][kx]
+struct DxWeightOperand {
+  const float *w;
+  int C, rs;
+  FastDiv div_rs;
+  struct Fix {
+    int off;
+    bool valid;
+  };
+  struct KDec {
+    int off;
+  };
+  __device__ __forceinline__ Fix fix(int m) const { return {m * rs, m < C}; }
+  __device__ __forceinline__ KDec kdec(int k) const {
+    uint32_t co, t;
+    div_rs.divmod(k, co, t);
+    return {static_cast<int>(co) * C * rs + static_cast<int>(t)};
+  }
+  __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
+    return f.valid ? w[f.off + k.off] : 0.0f;
+  }
+};
+
+// dX B operand: n = (img, iy, ix), k = (co, ky, kx) -> dy[img][co][oy][ox] where
+// oy*sh + ky = iy + pad (and likewise in x); zero when no such output exists
+struct DxDyOperand {
+  const float *dy;
+  ConvGeom g;
+  int n_extent;
+  struct Fix {
+    int base, ty, tx;
+    bool valid;
+  };
+  struct KDec {
+    int coff, ky, kx;
+  };
+  __device__ __forceinline__ Fix fix(int n) const {
+    uint32_t img, q, iy, ix;
+    g.div_hw.divmod(n, img, q);
+    g.div_w.divmod(q, iy, ix);
+    return {static_cast<int>(img) * g.Kc * g.OH * g.OW, static_cast<int>(iy) + g.pad_h,
+            static_cast<int>(ix) + g.pad_w, n < n_extent};
+  }
+  __device__ __forceinline__ KDec kdec(int k) const {
+    uint32_t co, t, ky, kx;
+    g.div_rs.divmod(k, co, t);
+    g.div_s.divmod(t, ky, kx);
+    return {static_cast<int>(co) * g.OH * g.OW, static_cast<int>(ky), static_cast<int>(kx)};
+  }
+  __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
+    const int uy = f.ty - k.ky, ux = f.tx - k.kx;
+    if (!f.valid || uy < 0 || ux < 0) return 0.0f;
+    uint32_t oy = uy, ox = ux;
+    if (g.sh != 1 || g.sw != 1) {
+      uint32_t ry, rx;
+      g.div_sh.divmod(uy, oy, ry);
+      g.div_sw.divmod(ux, ox, rx);
+      if (ry != 0 || rx != 0) return 0.0f;
+    }
+    if (oy >= static_cast<uint32_t>(g.OH) || ox >= static_cast<uint32_t>(g.OW)) return 0.0f;
+    return dy[f.base + k.coff + static_cast<int>(oy) * g.OW + static_cast<int>(ox)];
+  }
+};
+
+// connection_table support: w_masked[i] = w[i] * tbl[ci][co]; dw (+)= tmp * tbl
+__global__ void __launch_bounds__(256)
+mask_weights_kernel(const float *__restrict__ src, const uint8_t *__restrict__ tbl,
+                    float *__restrict__ dst, const int n, const int C, const int Kc, const int rs,
+                    const int accumulate) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int pair = i / rs;  // co*C + ci
+  const int co = pair / C, ci = pair - co * C;
+  const float v = tbl[ci * Kc + co] ? src[i] : 0.0f;
+  dst[i]        = accumulate ? dst[i] + v : v;
+}
+
+}  // namespace
+
+size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
+  const ConvGeom g = make_geom(d);
+  const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
+  size_t total = 0;
+  total += gemm_workspace_bytes(g.Kc, batch * ohw, crs, true);        // forward
+  total += gemm_workspace_bytes(g.Kc, crs, batch * ohw, true);        // dW
+  total += gemm_workspace_bytes(g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true);  // dX
+  total += rowsum_workspace_bytes(batch, g.Kc, ohw);                  // db
+  if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
+  return total;
+}
+
+// Uploads the connection table (if any) and returns masked weights in scratch.
+static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float *w,
+                         const uint8_t **tbl_dev, const float **w_eff) {
+  *tbl_dev = nullptr;
+  *w_eff   = w;
+  if (!d->tbl) return TDH_OK;
+  void *t = nullptr, *wm = nullptr;
+  const int nw = g.Kc * g.C * g.R * g.S;
+  TDH_TRY(ws_take(static_cast<size_t>(g.C) * g.Kc, &t));
+  TDH_TRY(ws_take(sizeof(float) * nw, &wm));
+  // pageable source: the copy is staged before the call returns
+  TDH_HIP(hipMemcpyAsync(t, d->tbl, static_cast<size_t>(g.C) * g.Kc, hipMemcpyHostToDevice,
+                         ctx().stream));
+  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(nw, 256)), dim3(256), 0, ctx().stream, w,
+                     static_cast<const uint8_t *>(t), static_cast<float *>(wm), nw, g.C, g.Kc,
+                     g.R * g.S, 0);
+  TDH_LAUNCH_CHECK();
+  *tbl_dev = static_cast<const uint8_t *>(t);
+  *w_eff   = static_cast<const float *>(wm);
+  return TDH_OK;
+}
+
+int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
+               float *y) {
+  const ConvGeom g = make_geom(d);
+  const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
+  const uint8_t *tbl_dev;
+  const float *w_eff;
+  TDH_TRY(prepare_table(d, g, w, &tbl_dev, &w_eff));
+  StridedOperand A{w_eff, crs, 1, g.Kc};
+  FwdInputOperand B{x, g, batch * ohw};
+  EpiImageRows epi{y, g.Kc, ohw, g.div_ohw, d->has_bias ? b : nullptr, ActGrad()};
+  return launch_gemm<true, false>(A, B, epi, g.Kc, batch * ohw, crs, true);
+}
+
+int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
+               float *dx, float *dw, float *db, int accumulate, ActGrad dx_act) {
+  const ConvGeom g = make_geom(d);
+  const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
+  const uint8_t *tbl_dev;
+  const float *w_eff;
+  TDH_TRY(prepare_table(d, g, w, &tbl_dev, &w_eff));
+  if (dx) {
+    DxWeightOperand A{w_eff, g.C, g.R * g.S, g.div_rs};
+    DxDyOperand B{dy, g, batch * g.H * g.W};
+    EpiImageRows epi{dx, g.C, g.H * g.W, g.div_hw, nullptr, dx_act};
+    TDH_TRY((launch_gemm<true, false>(A, B, epi, g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true)));
+  }
+  if (dw) {
+    DwDyOperand A{dy, g.Kc, ohw, g.div_ohw};
+    DwInputOperand B{x, g, crs};
+    if (tbl_dev) {
+      void *tmp = nullptr;
+      TDH_TRY(ws_take(sizeof(float) * g.Kc * crs, &tmp));
+      EpiRowMajor epi{static_cast<float *>(tmp), crs, nullptr, ActGrad(), 0};
+      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true)));
+      hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(g.Kc * crs, 256)), dim3(256), 0,
+                         ctx().stream, static_cast<const float *>(tmp), tbl_dev, dw, g.Kc * crs,
+                         g.C, g.Kc, g.R * g.S, accumulate);
+      TDH_LAUNCH_CHECK();
+    } else {
+      EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
+      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true)));
+    }
+  }
+  if (db) TDH_TRY(launch_rowsum(dy, batch, g.Kc, ohw, db, accumulate));
+  return TDH_OK;
+}
+
+}  // namespace tdh

@@ -1,0 +1,460 @@
+// elementwise.hip — bandwidth-bound kernels: fills, activations and their gradients,
+// loss gradients, optimizer updates and the fixed-order reductions used for bias
+// gradients. One pass over each array, 16-byte accesses where alignment allows.
+// Built with -ffp-contract=off so that a*b+c rounds twice, as in the scalar reference.
+#include <cfloat>
+
+#include "common.h"
+
+namespace tdh {
+
+namespace {
+
+constexpr int EW_THREADS = 256;
+
+inline int ew_blocks(size_t work_items) {
+  const size_t want = ceil_div_sz(work_items, EW_THREADS);
+  const size_t cap  = 256 * 16;  // enough waves to cover HBM latency on 256 CUs
+  return static_cast<int>(want < 1 ? 1 : (want > cap ? cap : want));
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// out[i] = Op::apply(a[i], b[i], prm); n4 float4 groups when vec, scalar tail after
+template <class Op, bool HAS_B>
+__global__ void __launch_bounds__(EW_THREADS)
+map_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out,
+           const size_t n4, const size_t n, const typename Op::Params prm) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * EW_THREADS;
+  const size_t t0     = static_cast<size_t>(blockIdx.x) * EW_THREADS + threadIdx.x;
+  for (size_t i = t0; i < n4; i += stride) {
+    const float4 va = reinterpret_cast<const float4 *>(a)[i];
+    float4 vb       = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (HAS_B) vb = reinterpret_cast<const float4 *>(b)[i];
+    float4 r;
+    r.x = Op::apply(va.x, vb.x, prm);
+    r.y = Op::apply(va.y, vb.y, prm);
+    r.z = Op::apply(va.z, vb.z, prm);
+    r.w = Op::apply(va.w, vb.w, prm);
+    reinterpret_cast<float4 *>(out)[i] = r;
+  }
+  for (size_t j = n4 * 4 + t0; j < n; j += stride)
+    out[j] = Op::apply(a[j], HAS_B ? b[j] : 0.0f, prm);
+}
+
+template <class Op, bool HAS_B>
+int launch_map(const float *a, const float *b, float *out, size_t n,
+               const typename Op::Params &prm) {
+  const bool vec  = aligned16(a) && aligned16(out) && (!HAS_B || aligned16(b));
+  const size_t n4 = vec ? n / 4 : 0;
+  hipLaunchKernelGGL((map_kernel<Op, HAS_B>), dim3(ew_blocks(vec ? n4 + 3 : n)), dim3(EW_THREADS),
+                     0, ctx().stream, a, b, out, n4, n, prm);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+struct NoParams {};
+
+// forward activations: tanh_layer.h:24-28, relu_layer.h:25-29, sigmoid_layer.h:24-28
+struct TanhFwd {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float x, float, Params) { return tanhf(x); }
+};
+struct ReluFwd {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float x, float, Params) {
+    return x > 0.0f ? x : 0.0f;  // std::max(float_t(0), x): NaN maps to 0
+  }
+};
+struct SigmoidFwd {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float x, float, Params) {
+    return 1.0f / (1.0f + expf(-x));
+  }
+};
+// backward activations on the OUTPUT y: tanh_layer.h:30-38, relu_layer.h:31-39,
+// sigmoid_layer.h:30-38.  a = y, b = dy
+struct TanhBwd {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params) {
+    return dy * (1.0f - y * y);
+  }
+};
+struct ReluBwd {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params) {
+    return dy * (y > 0.0f ? 1.0f : 0.0f);
+  }
+};
+struct SigmoidBwd {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params) {
+    return dy * y * (1.0f - y);
+  }
+};
+// loss gradients: loss_function.h:28-36, :143-150, :120-128.  a = y, b = t
+struct MseGrad {
+  struct Params {
+    float factor;
+  };
+  static __device__ __forceinline__ float apply(float y, float t, Params p) {
+    return p.factor * (y - t);
+  }
+};
+struct CeMultiGrad {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float y, float t, Params) { return -t / y; }
+};
+struct CeGrad {
+  typedef NoParams Params;
+  static __device__ __forceinline__ float apply(float y, float t, Params) {
+    return (y - t) / (y * (1.0f - y));
+  }
+};
+
+__global__ void __launch_bounds__(EW_THREADS)
+fill_zero_kernel(uint32_t *__restrict__ p, const size_t n4, const size_t n) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * EW_THREADS;
+  const size_t t0     = static_cast<size_t>(blockIdx.x) * EW_THREADS + threadIdx.x;
+  for (size_t i = t0; i < n4; i += stride) reinterpret_cast<uint4 *>(p)[i] = make_uint4(0, 0, 0, 0);
+  for (size_t j = n4 * 4 + t0; j < n; j += stride) p[j] = 0u;
+}
+
+// ------------------------------------------------------------------ softmax
+// One wave64 per sample row; reductions by butterfly shuffles (every lane ends with the
+// same value, summed in a fixed tree).
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// softmax_layer.h:24-34: y = exp(x - max) / sum
+__global__ void __launch_bounds__(EW_THREADS)
+softmax_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, const int batch,
+                   const int len) {
+  const int row  = blockIdx.x * (EW_THREADS / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= batch) return;
+  const float *xr = x + static_cast<size_t>(row) * len;
+  float *yr       = y + static_cast<size_t>(row) * len;
+  float m         = -FLT_MAX;
+  for (int j = lane; j < len; j += 64) m = fmaxf(m, xr[j]);
+  m       = wave_max(m);
+  float s = 0.0f;
+  for (int j = lane; j < len; j += 64) {
+    const float e = expf(xr[j] - m);
+    yr[j]         = e;
+    s += e;
+  }
+  s = wave_sum(s);
+  for (int j = lane; j < len; j += 64) yr[j] = yr[j] / s;
+}
+
+// softmax_layer.h:36-55: dx_j = sum_k dy_k * (delta_jk*y_j - y_j*y_k) = y_j * (dy_j - <dy, y>)
+__global__ void __launch_bounds__(EW_THREADS)
+softmax_bwd_kernel(const float *__restrict__ y, const float *__restrict__ dy,
+                   float *__restrict__ dx, const int batch, const int len) {
+  const int row  = blockIdx.x * (EW_THREADS / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= batch) return;
+  const float *yr  = y + static_cast<size_t>(row) * len;
+  const float *dyr = dy + static_cast<size_t>(row) * len;
+  float dot        = 0.0f;
+  for (int j = lane; j < len; j += 64) dot += dyr[j] * yr[j];
+  dot = wave_sum(dot);
+  for (int j = lane; j < len; j += 64)
+    dx[static_cast<size_t>(row) * len + j] = yr[j] * (dyr[j] - dot);
+}
+
+// softmax backward of cross_entropy_multiclass::df (= -t/y) in closed form:
+// dz_j = y_j * (-t_j/y_j + sum_k t_k) = y_j * sum(t) - t_j
+__global__ void __launch_bounds__(EW_THREADS)
+softmax_xent_grad_kernel(const float *__restrict__ y, const float *__restrict__ t,
+                         float *__restrict__ dz, const int batch, const int len) {
+  const int row  = blockIdx.x * (EW_THREADS / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= batch) return;
+  const float *yr = y + static_cast<size_t>(row) * len;
+  const float *tr = t + static_cast<size_t>(row) * len;
+  float st        = 0.0f;
+  for (int j = lane; j < len; j += 64) st += tr[j];
+  st = wave_sum(st);
+  for (int j = lane; j < len; j += 64) dz[static_cast<size_t>(row) * len + j] = yr[j] * st - tr[j];
+}
+
+// --------------------------------------------------------------- optimizers
+// tiny_dnn/optimizers/optimizer.h; g = merged * grad_scale is layer::update_weight's
+// diff (tiny_dnn/layers/layer.h:668-673). Scalars that the reference derives once per
+// call from its float members (1 - b1_t, ...) arrive precomputed in float.
+struct OptScalars {
+  float alpha, lambda, mu, b1, b2, eps, omb1, omb2, omb1t, omb2t, grad_scale;
+  double adamax_lr;  // alpha / (1.0 - b1_t), evaluated in double as the reference does
+};
+
+template <int KIND>
+__device__ __forceinline__ void opt_one(float g, float &w, float &s0, float &s1,
+                                        const OptScalars &p) {
+  g *= p.grad_scale;
+  if (KIND == TDH_OPT_SGD) {  // :185-188
+    w = w - p.alpha * (g + p.lambda * w);
+  } else if (KIND == TDH_OPT_MOMENTUM) {  // :205-213
+    const float V = p.mu * s0 - p.alpha * (g + w * p.lambda);
+    w += V;
+    s0 = V;
+  } else if (KIND == TDH_OPT_NESTEROV) {  // :231-239
+    const float V = p.mu * s0 - p.alpha * (g + w * p.lambda);
+    w += (-p.mu) * s0 + (1 + p.mu) * V;
+    s0 = V;
+  } else if (KIND == TDH_OPT_ADAM) {  // :112-127, eps inside the square root
+    s0 = p.b1 * s0 + p.omb1 * g;
+    s1 = p.b2 * s1 + p.omb2 * g * g;
+    w -= p.alpha * (s0 / p.omb1t) / sqrtf((s1 / p.omb2t) + p.eps);
+  } else if (KIND == TDH_OPT_ADAGRAD) {  // :60-66
+    s0 += g * g;
+    w -= p.alpha * g / (sqrtf(s0) + p.eps);
+  } else if (KIND == TDH_OPT_RMSPROP) {  // :81-88
+    s0 = p.mu * s0 + (1 - p.mu) * g * g;
+    w -= p.alpha * g / sqrtf(s0 + p.eps);
+  } else if (KIND == TDH_OPT_ADAMAX) {  // :153-165
+    s0 = p.b1 * s0 + p.omb1 * g;
+    s1 = fmaxf(p.b2 * s1, fabsf(g));
+    w  = static_cast<float>(static_cast<double>(w) -
+                           p.adamax_lr * static_cast<double>(s0 / (s1 + p.eps)));
+  }
+}
+
+template <int KIND, int NSTATE>
+__global__ void __launch_bounds__(EW_THREADS)
+opt_kernel(const float *__restrict__ g, float *__restrict__ w, float *__restrict__ s0,
+           float *__restrict__ s1, const size_t n4, const size_t n, const OptScalars p) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * EW_THREADS;
+  const size_t t0     = static_cast<size_t>(blockIdx.x) * EW_THREADS + threadIdx.x;
+  for (size_t i = t0; i < n4; i += stride) {
+    const float4 vg = reinterpret_cast<const float4 *>(g)[i];
+    float4 vw       = reinterpret_cast<float4 *>(w)[i];
+    float4 v0       = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
+    if (NSTATE >= 1) v0 = reinterpret_cast<float4 *>(s0)[i];
+    if (NSTATE >= 2) v1 = reinterpret_cast<float4 *>(s1)[i];
+    opt_one<KIND>(vg.x, vw.x, v0.x, v1.x, p);
+    opt_one<KIND>(vg.y, vw.y, v0.y, v1.y, p);
+    opt_one<KIND>(vg.z, vw.z, v0.z, v1.z, p);
+    opt_one<KIND>(vg.w, vw.w, v0.w, v1.w, p);
+    reinterpret_cast<float4 *>(w)[i] = vw;
+    if (NSTATE >= 1) reinterpret_cast<float4 *>(s0)[i] = v0;
+    if (NSTATE >= 2) reinterpret_cast<float4 *>(s1)[i] = v1;
+  }
+  for (size_t j = n4 * 4 + t0; j < n; j += stride) {
+    float ww = w[j], a = 0.0f, b = 0.0f;
+    if (NSTATE >= 1) a = s0[j];
+    if (NSTATE >= 2) b = s1[j];
+    opt_one<KIND>(g[j], ww, a, b, p);
+    w[j] = ww;
+    if (NSTATE >= 1) s0[j] = a;
+    if (NSTATE >= 2) s1[j] = b;
+  }
+}
+
+template <int KIND, int NSTATE>
+int launch_opt(size_t n, const float *g, float *w, float *s0, float *s1, const OptScalars &p) {
+  const bool vec = aligned16(g) && aligned16(w) && (NSTATE < 1 || aligned16(s0)) &&
+                   (NSTATE < 2 || aligned16(s1));
+  const size_t n4 = vec ? n / 4 : 0;
+  hipLaunchKernelGGL((opt_kernel<KIND, NSTATE>), dim3(ew_blocks(vec ? n4 + 3 : n)),
+                     dim3(EW_THREADS), 0, ctx().stream, g, w, s0, s1, n4, n, p);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+// ---------------------------------------------------------------- reductions
+// Block-wide sum with a fixed shape: wave butterflies, then wave 0 adds the four wave
+// totals in order. Every thread of the block must call it.
+__device__ __forceinline__ float block_sum(float v, float *smem4) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) smem4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float r = (smem4[0] + smem4[1]) + (smem4[2] + smem4[3]);
+  __syncthreads();
+  return r;
+}
+
+// stage 1: partial[(o*rows + r)*chunks + c] = sum of a slice of row r in image o
+__global__ void __launch_bounds__(EW_THREADS)
+rowsum_stage1_kernel(const float *__restrict__ src, const int rows, const int cols,
+                     const int chunks, const int chunk_len, float *__restrict__ partial) {
+  __shared__ float smem4[4];
+  const int row = blockIdx.x;  // o*rows + r
+  const int c   = blockIdx.y;
+  const float *p = src + static_cast<size_t>(row) * cols;
+  const int beg = c * chunk_len;
+  const int end = min(cols, beg + chunk_len);
+  float s = 0.0f;
+  for (int i = beg + threadIdx.x; i < end; i += EW_THREADS) s += p[i];
+  s = block_sum(s, smem4);
+  if (threadIdx.x == 0) partial[static_cast<size_t>(row) * chunks + c] = s;
+}
+
+// stage 2: out[r] (+)= sum over o (outer) and chunks, in index order
+__global__ void __launch_bounds__(EW_THREADS)
+rowsum_stage2_kernel(const float *__restrict__ partial, const int outer, const int rows,
+                     const int chunks, float *__restrict__ out, const int accumulate) {
+  const int r = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (r >= rows) return;
+  float s = 0.0f;
+  for (int o = 0; o < outer; ++o)
+    for (int c = 0; c < chunks; ++c) s += partial[(static_cast<size_t>(o) * rows + r) * chunks + c];
+  out[r] = accumulate ? out[r] + s : s;
+}
+
+// out[c] (+)= sum_s src[s*cols + c], s ascending (fully_connected bias gradient)
+__global__ void __launch_bounds__(EW_THREADS)
+colsum_kernel(const float *__restrict__ src, const int rows, const int cols,
+              float *__restrict__ out, const int accumulate) {
+  const int c = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (c >= cols) return;
+  float s = 0.0f;
+  for (int r = 0; r < rows; ++r) s += src[static_cast<size_t>(r) * cols + c];
+  out[c] = accumulate ? out[c] + s : s;
+}
+
+}  // namespace
+
+int launch_fill_zero(void *p, size_t bytes) {
+  const size_t n  = bytes / 4;
+  const size_t n4 = aligned16(p) ? n / 4 : 0;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0,
+                     ctx().stream, static_cast<uint32_t *>(p), n4, n);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+int launch_act_fwd(int kind, int batch, int len, const float *x, float *y) {
+  const size_t n = static_cast<size_t>(batch) * len;
+  switch (kind) {
+    case TDH_ACT_TANH: return launch_map<TanhFwd, false>(x, nullptr, y, n, NoParams());
+    case TDH_ACT_RELU: return launch_map<ReluFwd, false>(x, nullptr, y, n, NoParams());
+    case TDH_ACT_SIGMOID: return launch_map<SigmoidFwd, false>(x, nullptr, y, n, NoParams());
+    case TDH_ACT_SOFTMAX:
+      hipLaunchKernelGGL(softmax_fwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
+                         dim3(EW_THREADS), 0, ctx().stream, x, y, batch, len);
+      TDH_LAUNCH_CHECK();
+      return TDH_OK;
+  }
+  return set_error(TDH_ERR_INVALID, "activation kind %d is not supported", kind);
+}
+
+int launch_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx) {
+  const size_t n = static_cast<size_t>(batch) * len;
+  switch (kind) {
+    case TDH_ACT_TANH: return launch_map<TanhBwd, true>(y, dy, dx, n, NoParams());
+    case TDH_ACT_RELU: return launch_map<ReluBwd, true>(y, dy, dx, n, NoParams());
+    case TDH_ACT_SIGMOID: return launch_map<SigmoidBwd, true>(y, dy, dx, n, NoParams());
+    case TDH_ACT_SOFTMAX:
+      hipLaunchKernelGGL(softmax_bwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
+                         dim3(EW_THREADS), 0, ctx().stream, y, dy, dx, batch, len);
+      TDH_LAUNCH_CHECK();
+      return TDH_OK;
+  }
+  return set_error(TDH_ERR_INVALID, "activation kind %d is not supported", kind);
+}
+
+int launch_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy) {
+  const size_t n = static_cast<size_t>(batch) * len;
+  switch (kind) {
+    case TDH_LOSS_MSE: {
+      MseGrad::Params p;
+      p.factor = 2.0f / static_cast<float>(len);
+      return launch_map<MseGrad, true>(y, t, dy, n, p);
+    }
+    case TDH_LOSS_CE_MULTICLASS: return launch_map<CeMultiGrad, true>(y, t, dy, n, NoParams());
+    case TDH_LOSS_CE: return launch_map<CeGrad, true>(y, t, dy, n, NoParams());
+  }
+  return set_error(TDH_ERR_INVALID, "loss kind %d is not supported", kind);
+}
+
+int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz) {
+  hipLaunchKernelGGL(softmax_xent_grad_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
+                     dim3(EW_THREADS), 0, ctx().stream, y, t, dz, batch, len);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, float *w, float *s0,
+                      float *s1) {
+  OptScalars p;
+  p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; p.b1 = o->b1; p.b2 = o->b2;
+  p.eps = o->eps;
+  p.omb1 = 1.0f - o->b1; p.omb2 = 1.0f - o->b2;
+  p.omb1t = 1.0f - o->b1_t; p.omb2t = 1.0f - o->b2_t;
+  p.grad_scale = grad_scale;
+  p.adamax_lr  = static_cast<double>(o->alpha) / (1.0 - static_cast<double>(o->b1_t));
+  int rc = TDH_OK;
+  const int nstate = (o->kind == TDH_OPT_SGD) ? 0
+                     : (o->kind == TDH_OPT_ADAM || o->kind == TDH_OPT_ADAMAX) ? 2 : 1;
+  if (n > 0) {
+    if (nstate >= 1 && !s0) return set_error(TDH_ERR_INVALID, "optimizer %d needs state s0", o->kind);
+    if (nstate >= 2 && !s1) return set_error(TDH_ERR_INVALID, "optimizer %d needs state s1", o->kind);
+    switch (o->kind) {
+      case TDH_OPT_SGD: rc = launch_opt<TDH_OPT_SGD, 0>(n, g, w, s0, s1, p); break;
+      case TDH_OPT_MOMENTUM: rc = launch_opt<TDH_OPT_MOMENTUM, 1>(n, g, w, s0, s1, p); break;
+      case TDH_OPT_NESTEROV: rc = launch_opt<TDH_OPT_NESTEROV, 1>(n, g, w, s0, s1, p); break;
+      case TDH_OPT_ADAM: rc = launch_opt<TDH_OPT_ADAM, 2>(n, g, w, s0, s1, p); break;
+      case TDH_OPT_ADAGRAD: rc = launch_opt<TDH_OPT_ADAGRAD, 1>(n, g, w, s0, s1, p); break;
+      case TDH_OPT_RMSPROP: rc = launch_opt<TDH_OPT_RMSPROP, 1>(n, g, w, s0, s1, p); break;
+      case TDH_OPT_ADAMAX: rc = launch_opt<TDH_OPT_ADAMAX, 2>(n, g, w, s0, s1, p); break;
+      default: return set_error(TDH_ERR_INVALID, "optimizer kind %d is not supported", o->kind);
+    }
+  }
+  if (rc != TDH_OK) return rc;
+  // the reference advances the powers once per update() call, whatever the tensor size
+  if (o->kind == TDH_OPT_ADAM) {
+    o->b1_t *= o->b1;
+    o->b2_t *= o->b2;
+  } else if (o->kind == TDH_OPT_ADAMAX) {
+    o->b1_t *= o->b1;
+  }
+  return TDH_OK;
+}
+
+// chunking depends on the shape only
+static void rowsum_chunks(int cols, int &chunks, int &chunk_len) {
+  chunks = ceil_div(cols, 4096);
+  if (chunks > 64) chunks = 64;
+  chunk_len = ceil_div(cols, chunks);
+  chunks    = ceil_div(cols, chunk_len);
+}
+
+size_t rowsum_workspace_bytes(int outer, int rows, int cols) {
+  int chunks, chunk_len;
+  rowsum_chunks(cols, chunks, chunk_len);
+  return ws_align(static_cast<size_t>(outer) * rows * chunks * sizeof(float));
+}
+
+int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate) {
+  int chunks, chunk_len;
+  rowsum_chunks(cols, chunks, chunk_len);
+  void *ws = nullptr;
+  TDH_TRY(ws_take(static_cast<size_t>(outer) * rows * chunks * sizeof(float), &ws));
+  hipLaunchKernelGGL(rowsum_stage1_kernel, dim3(outer * rows, chunks), dim3(EW_THREADS), 0,
+                     ctx().stream, src, rows, cols, chunks, chunk_len, static_cast<float *>(ws));
+  TDH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(rowsum_stage2_kernel, dim3(ceil_div(rows, EW_THREADS)), dim3(EW_THREADS), 0,
+                     ctx().stream, static_cast<const float *>(ws), outer, rows, chunks, out,
+                     accumulate);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+int launch_colsum(const float *src, int rows, int cols, float *out, int accumulate) {
+  hipLaunchKernelGGL(colsum_kernel, dim3(ceil_div(cols, EW_THREADS)), dim3(EW_THREADS), 0,
+                     ctx().stream, src, rows, cols, out, accumulate);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+}  // namespace tdh

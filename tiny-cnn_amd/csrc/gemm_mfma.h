@@ -1,0 +1,371 @@
+// gemm_mfma.h — LDS-tiled fp32 MFMA GEMM for gfx950 with pluggable operand loaders.
+//
+// C[M][N] = sum_k A[m][k] * B[k][n], computed by 256-thread workgroups (four wave64)
+// with v_mfma_f32_32x32x2_f32. Operands are not required to be matrices in memory:
+// each side is a small functor that maps a GEMM coordinate to a global address, which
+// is how convolution gradients (implicit im2col / col2im) and the three fully-connected
+// products share one kernel. Out-of-range coordinates read as zero.
+//
+// Work decomposition
+//   grid.x = N tiles, grid.y = M tiles, grid.z = K splits. With more than one split
+//   every workgroup writes its partial tile to scratch[z][M][N] and a second kernel adds
+//   the splits in index order 0..S-1, so the result does not depend on scheduling.
+//   The number of splits is a function of the problem shape only.
+//
+// Operand loader concept (device side)
+//   struct Op {
+//     struct Fix;                              // per-thread state of its fixed m (or n)
+//     struct KDec;                             // decomposed reduction index
+//     __device__ Fix  fix(int mn) const;       // must tolerate mn >= extent (valid=false)
+//     __device__ KDec kdec(int k) const;       // k < K guaranteed by the caller
+//     __device__ float load(const Fix&, const KDec&) const;   // 0 when fix is invalid
+//   };
+//   LANE_K = true : consecutive lanes walk k (operand contiguous along k)
+//   LANE_K = false: consecutive lanes walk m/n (operand contiguous along m/n); k is then
+//                   wave-uniform and its decomposition runs on the scalar unit.
+//
+// Epilogue concept
+//   struct Epi { struct Col; __device__ Col col(int n) const;
+//                __device__ void store(int m, const Col&, float v) const; };
+#pragma once
+
+#include "common.h"
+
+namespace tdh {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int GEMM_BK      = 16;
+constexpr int GEMM_THREADS = 256;
+constexpr int GEMM_LDS_PAD = 4;
+
+// ------------------------------------------------------------ plain matrices
+// element(mn, k) = p[mn * s_mn + k * s_k]
+struct StridedOperand {
+  const float *p;
+  int s_mn, s_k, extent;
+  struct Fix {
+    int off;
+    bool valid;
+  };
+  struct KDec {
+    int off;
+  };
+  __device__ __forceinline__ Fix fix(int mn) const { return {mn * s_mn, mn < extent}; }
+  __device__ __forceinline__ KDec kdec(int k) const { return {k * s_k}; }
+  __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
+    return f.valid ? p[f.off + k.off] : 0.0f;
+  }
+};
+
+// ------------------------------------------------------------------ epilogues
+// out[m*ld + n] = (accumulate ? out : 0) + (v + bias_n[n]) * act'(y[m*ld + n])
+struct EpiRowMajor {
+  float *out;
+  int ld;
+  const float *bias_n;
+  ActGrad ag;
+  int accumulate;
+  struct Col {
+    int n;
+    float bias;
+  };
+  __device__ __forceinline__ Col col(int n) const { return {n, bias_n ? bias_n[n] : 0.0f}; }
+  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+    const int idx = m * ld + c.n;
+    v += c.bias;
+    if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[idx]);
+    if (accumulate) v += out[idx];
+    out[idx] = v;
+  }
+};
+
+// GEMM column n = (img, p) with p < pix; out[(img*rows + m)*pix + p] = (v + bias_m[m]) * act'
+struct EpiImageRows {
+  float *out;
+  int rows, pix;
+  FastDiv pix_div;
+  const float *bias_m;
+  ActGrad ag;
+  struct Col {
+    int base;  // img*rows*pix + p
+  };
+  __device__ __forceinline__ Col col(int n) const {
+    uint32_t img, p;
+    pix_div.divmod(static_cast<uint32_t>(n), img, p);
+    return {static_cast<int>(img) * rows * pix + static_cast<int>(p)};
+  }
+  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+    const int idx = c.base + m * pix;
+    if (bias_m) v += bias_m[m];
+    if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[idx]);
+    out[idx] = v;
+  }
+};
+
+// --------------------------------------------------------------------- kernel
+template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
+          class Epi>
+__global__ void __launch_bounds__(GEMM_THREADS)
+gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const int N,
+                 const int K, const int k_per_split, float *__restrict__ partial) {
+  constexpr int BK  = GEMM_BK;
+  constexpr int TM  = BM / WM / 32;  // 32x32 MFMA blocks per wave along M
+  constexpr int TN  = BN / WN / 32;
+  constexpr int CA  = BM * BK / GEMM_THREADS;  // elements of A each thread stages per tile
+  constexpr int CB  = BN * BK / GEMM_THREADS;
+  constexpr int LDA = BM + GEMM_LDS_PAD;
+  constexpr int LDB = BN + GEMM_LDS_PAD;
+  static_assert(WM * WN == 4, "four waves per workgroup");
+  static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
+  static_assert(GEMM_THREADS % BM == 0 && GEMM_THREADS % BN == 0, "tile/threads mismatch");
+
+  __shared__ float As[2][BK][LDA];
+  __shared__ float Bs[2][BK][LDB];
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm   = wave % WM;
+  const int wn   = wave / WM;
+  const int m0   = blockIdx.y * BM;
+  const int n0   = blockIdx.x * BN;
+  const int kbeg = blockIdx.z * k_per_split;
+  const int kend = min(K, kbeg + k_per_split);
+
+  // ---- per-thread staging assignment
+  // LANE_K : k_local = tid % 16 (fixed), rows (tid/16) + 16*i
+  // !LANE_K: row = tid % BM (fixed), k_local = tid/BM + (256/BM)*i
+  typename AOp::Fix fa[A_LANE_K ? CA : 1];
+  typename BOp::Fix fb[B_LANE_K ? CB : 1];
+  if (A_LANE_K) {
+#pragma unroll
+    for (int i = 0; i < CA; ++i) fa[i] = aop.fix(m0 + (tid >> 4) + 16 * i);
+  } else {
+    fa[0] = aop.fix(m0 + tid % BM);
+  }
+  if (B_LANE_K) {
+#pragma unroll
+    for (int i = 0; i < CB; ++i) fb[i] = bop.fix(n0 + (tid >> 4) + 16 * i);
+  } else {
+    fb[0] = bop.fix(n0 + tid % BN);
+  }
+
+  float ra[CA], rb[CB];
+
+  auto fetch = [&](int kt) {
+    if (A_LANE_K) {
+      const int k = kt + (tid & 15);
+      if (k < kend) {
+        const typename AOp::KDec kd = aop.kdec(k);
+#pragma unroll
+        for (int i = 0; i < CA; ++i) ra[i] = aop.load(fa[i], kd);
+      } else {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) ra[i] = 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < CA; ++i) {
+        int k = kt + tid / BM + (GEMM_THREADS / BM) * i;
+        if (BM % 64 == 0) k = __builtin_amdgcn_readfirstlane(k);
+        ra[i] = (k < kend) ? aop.load(fa[0], aop.kdec(k)) : 0.0f;
+      }
+    }
+    if (B_LANE_K) {
+      const int k = kt + (tid & 15);
+      if (k < kend) {
+        const typename BOp::KDec kd = bop.kdec(k);
+#pragma unroll
+        for (int i = 0; i < CB; ++i) rb[i] = bop.load(fb[i], kd);
+      } else {
+#pragma unroll
+        for (int i = 0; i < CB; ++i) rb[i] = 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < CB; ++i) {
+        int k = kt + tid / BN + (GEMM_THREADS / BN) * i;
+        if (BN % 64 == 0) k = __builtin_amdgcn_readfirstlane(k);
+        rb[i] = (k < kend) ? bop.load(fb[0], bop.kdec(k)) : 0.0f;
+      }
+    }
+  };
+
+  auto stage = [&](int buf) {
+    if (A_LANE_K) {
+#pragma unroll
+      for (int i = 0; i < CA; ++i) As[buf][tid & 15][(tid >> 4) + 16 * i] = ra[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < CA; ++i) As[buf][tid / BM + (GEMM_THREADS / BM) * i][tid % BM] = ra[i];
+    }
+    if (B_LANE_K) {
+#pragma unroll
+      for (int i = 0; i < CB; ++i) Bs[buf][tid & 15][(tid >> 4) + 16 * i] = rb[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < CB; ++i) Bs[buf][tid / BN + (GEMM_THREADS / BN) * i][tid % BN] = rb[i];
+    }
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int a_col = wm * (BM / WM) + (lane & 31);
+  const int b_col = wn * (BN / WN) + (lane & 31);
+  const int k_sub = lane >> 5;
+
+  int cur = 0;
+  if (kbeg < kend) {
+    fetch(kbeg);
+    stage(0);
+  }
+  __syncthreads();
+
+  for (int kt = kbeg; kt < kend; kt += BK) {
+    const bool has_next = kt + BK < kend;
+    if (has_next) fetch(kt + BK);
+
+#pragma unroll
+    for (int kk = 0; kk < BK / 2; ++kk) {
+      float af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[i] = As[cur][2 * kk + k_sub][a_col + 32 * i];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[j] = Bs[cur][2 * kk + k_sub][b_col + 32 * j];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+
+    if (has_next) stage(cur ^ 1);
+    __syncthreads();
+    cur ^= 1;
+  }
+
+  // ---- epilogue: D[i][j] of a 32x32 block lives in reg r of lane l at
+  //      i = 8*(r/4) + 4*(l/32) + r%4, j = l%32
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
+    if (n >= N) continue;
+    if (partial != nullptr) {
+      float *dst = partial + static_cast<size_t>(blockIdx.z) * M * N + n;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if (m < M) dst[static_cast<size_t>(m) * N] = acc[i][j][r];
+        }
+    } else {
+      const typename Epi::Col c = epi.col(n);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if (m < M) epi.store(m, c, acc[i][j][r]);
+        }
+    }
+  }
+}
+
+// Adds the K-split partial tiles in split order and applies the epilogue.
+template <class Epi>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const int M, const int N,
+                     const Epi epi) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * N) return;
+  const int m = idx / N, n = idx - m * N;
+  float s = 0.0f;
+  for (int z = 0; z < splits; ++z) s += partial[static_cast<size_t>(z) * M * N + idx];
+  epi.store(m, epi.col(n), s);
+}
+
+// ------------------------------------------------------------------- launcher
+struct GemmPlan {
+  int bm, bn;       // tile
+  int splits;       // K splits
+  int k_per_split;  // multiple of GEMM_BK
+};
+
+// Shape-only heuristics (no device queries) so that results are reproducible anywhere.
+inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
+  GemmPlan p;
+  p.bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
+  p.bn = (N <= 64 && p.bm != 32) ? 64 : 128;
+  const long tiles = static_cast<long>(ceil_div(M, p.bm)) * ceil_div(N, p.bn);
+  int splits       = 1;
+  if (allow_split && tiles < 512) {
+    splits = static_cast<int>(1024 / tiles);
+    const int max_by_k = K / 256 > 0 ? K / 256 : 1;
+    if (splits > max_by_k) splits = max_by_k;
+    if (splits > 512) splits = 512;
+    if (splits < 1) splits = 1;
+  }
+  p.k_per_split = ceil_div(ceil_div(K, splits), GEMM_BK) * GEMM_BK;
+  p.splits      = ceil_div(K, p.k_per_split);
+  return p;
+}
+
+inline size_t gemm_workspace_bytes(int M, int N, int K, bool allow_split) {
+  const GemmPlan p = plan_gemm(M, N, K, allow_split);
+  return p.splits > 1 ? ws_align(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
+}
+
+template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
+          class Epi>
+int launch_gemm_tile(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
+                     const GemmPlan &p, float *partial) {
+  dim3 grid(ceil_div(N, BN), ceil_div(M, BM), p.splits);
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, AOp, BOp, Epi>), grid,
+                     dim3(GEMM_THREADS), 0, ctx().stream, a, b, epi, M, N, K, p.k_per_split,
+                     partial);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+template <bool A_LANE_K, bool B_LANE_K, class AOp, class BOp, class Epi>
+int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
+                bool allow_split) {
+  if (M <= 0 || N <= 0) return TDH_OK;
+  TDH_CHECK_ARG(static_cast<long>(M) * N < (1L << 31), "gemm: M*N=%ld too large",
+                static_cast<long>(M) * N);
+  const GemmPlan p = plan_gemm(M, N, K, allow_split);
+  float *partial   = nullptr;
+  if (p.splits > 1) {
+    void *ws = nullptr;
+    TDH_TRY(ws_take(static_cast<size_t>(p.splits) * M * N * sizeof(float), &ws));
+    partial = static_cast<float *>(ws);
+  }
+  int rc;
+  if (p.bm == 128 && p.bn == 128)
+    rc = launch_gemm_tile<128, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+  else if (p.bm == 128 && p.bn == 64)
+    rc = launch_gemm_tile<128, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+  else if (p.bm == 64 && p.bn == 128)
+    rc = launch_gemm_tile<64, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+  else if (p.bm == 64 && p.bn == 64)
+    rc = launch_gemm_tile<64, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+  else
+    rc = launch_gemm_tile<32, 128, 1, 4, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+  TDH_TRY(rc);
+  if (p.splits > 1) {
+    hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, 256)), dim3(256), 0,
+                       ctx().stream, partial, p.splits, M, N, epi);
+    TDH_LAUNCH_CHECK();
+  }
+  return TDH_OK;
+}
+
+}  // namespace tdh

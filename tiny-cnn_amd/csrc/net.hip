@@ -1,0 +1,321 @@
+// net.hip — a sequential network whose tensors never leave the device: the restatement of
+// network<sequential>::train_onebatch (tiny_dnn/network.h:911-926) = fprop
+// (nodes.h:288-303), loss gradient (loss_function.h:191-218), bprop (nodes.h:276-286) and
+// update_weights (nodes.h:103-107, layer.h:663-682), queued on the library stream.
+#include <vector>
+
+#include "common.h"
+
+struct tdh_net {
+  struct Layer {
+    tdh_layer spec;
+    std::vector<uint8_t> tbl;  // private copy of the connection table
+    size_t in_size = 0, out_size = 0, w_size = 0, b_size = 0;
+    float *w = nullptr, *b = nullptr, *dw = nullptr, *db = nullptr;
+    float *s0w = nullptr, *s1w = nullptr, *s0b = nullptr, *s1b = nullptr;
+    float *out  = nullptr;  // [max_batch][out_size]
+    float *dout = nullptr;  // gradient w.r.t. out; the next layer's backward writes it
+    int32_t *argmax = nullptr;
+    bool grad_folded = false;  // activation whose backward runs in the next layer's dX epilogue
+  };
+  std::vector<Layer> layers;
+  int max_batch  = 0;
+  int flags      = 0;
+  float *dx_in   = nullptr;  // gradient w.r.t. the network input
+  size_t scratch = 0;        // largest per-op scratch need
+  std::vector<void *> allocs;
+};
+
+namespace tdh {
+
+namespace {
+
+int layer_sizes(tdh_net::Layer &L) {
+  const tdh_layer &s = L.spec;
+  switch (s.kind) {
+    case TDH_L_CONV: {
+      const int ow = conv_out_length(s.conv.in_w, s.conv.k_w, s.conv.w_stride, s.conv.w_dilation,
+                                     s.conv.pad_same);
+      const int oh = conv_out_length(s.conv.in_h, s.conv.k_h, s.conv.h_stride, s.conv.h_dilation,
+                                     s.conv.pad_same);
+      L.in_size  = static_cast<size_t>(s.conv.in_w) * s.conv.in_h * s.conv.in_c;
+      L.out_size = static_cast<size_t>(ow) * oh * s.conv.out_c;
+      L.w_size   = static_cast<size_t>(s.conv.k_w) * s.conv.k_h * s.conv.in_c * s.conv.out_c;
+      L.b_size   = s.conv.has_bias ? s.conv.out_c : 0;
+    } break;
+    case TDH_L_FC:
+      L.in_size = s.fc_in; L.out_size = s.fc_out;
+      L.w_size = static_cast<size_t>(s.fc_in) * s.fc_out;
+      L.b_size = s.fc_bias ? s.fc_out : 0;
+      break;
+    case TDH_L_MAXPOOL:
+    case TDH_L_AVEPOOL: {
+      const int ow = pool_out_length(s.pool.in_w, s.pool.pool_w, s.pool.stride_w, s.pool.ceil_mode,
+                                     s.pool.pad_same);
+      const int oh = pool_out_length(s.pool.in_h, s.pool.pool_h, s.pool.stride_h, s.pool.ceil_mode,
+                                     s.pool.pad_same);
+      L.in_size  = static_cast<size_t>(s.pool.in_w) * s.pool.in_h * s.pool.in_c;
+      L.out_size = static_cast<size_t>(ow) * oh * s.pool.in_c;
+      L.w_size   = s.kind == TDH_L_AVEPOOL ? s.pool.in_c : 0;
+      L.b_size   = L.w_size;
+    } break;
+    case TDH_L_ACT: L.w_size = L.b_size = 0; break;
+    default: return set_error(TDH_ERR_INVALID, "unknown layer kind %d", s.kind);
+  }
+  return TDH_OK;
+}
+
+int net_alloc(tdh_net *net, size_t floats, float **out, bool zero) {
+  *out = nullptr;
+  if (floats == 0) return TDH_OK;
+  void *p = nullptr;
+  if (hipMalloc(&p, floats * sizeof(float)) != hipSuccess) {
+    (void)hipGetLastError();
+    return set_error(TDH_ERR_OOM, "network: cannot allocate %zu bytes", floats * sizeof(float));
+  }
+  net->allocs.push_back(p);
+  *out = static_cast<float *>(p);
+  if (zero) TDH_TRY(launch_fill_zero(p, floats * sizeof(float)));
+  return TDH_OK;
+}
+
+bool is_pointwise_act(int act) {
+  return act == TDH_ACT_TANH || act == TDH_ACT_RELU || act == TDH_ACT_SIGMOID;
+}
+
+int forward(tdh_net *net, int batch, const float *x) {
+  const float *in = x;
+  for (auto &L : net->layers) {
+    const tdh_layer &s = L.spec;
+    switch (s.kind) {
+      case TDH_L_CONV:
+        TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
+        TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out));
+        break;
+      case TDH_L_FC:
+        TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
+        TDH_TRY(fc_fwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out));
+        break;
+      case TDH_L_MAXPOOL: TDH_TRY(maxpool_fwd(&s.pool, batch, in, L.out, L.argmax)); break;
+      case TDH_L_AVEPOOL: TDH_TRY(avepool_fwd(&s.pool, batch, in, L.w, L.b, L.out)); break;
+      case TDH_L_ACT:
+        TDH_TRY(launch_act_fwd(s.act, batch, static_cast<int>(L.out_size), in, L.out));
+        break;
+    }
+    in = L.out;
+  }
+  return TDH_OK;
+}
+
+}  // namespace
+
+}  // namespace tdh
+
+using namespace tdh;
+
+extern "C" {
+
+int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int flags,
+                   tdh_net **out) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(layers && out && n_layers > 0 && max_batch > 0, "tdh_net_create: bad argument");
+  if (flags & TDH_NET_GRAPH)
+    return set_error(TDH_ERR_UNSUPPORTED, "tdh_net_create: graph replay is not built yet");
+  *out = nullptr;
+  tdh_net *net   = new tdh_net();
+  net->max_batch = max_batch;
+  net->flags     = flags;
+  net->layers.resize(n_layers);
+  int rc = TDH_OK;
+  for (int i = 0; i < n_layers && rc == TDH_OK; ++i) {
+    tdh_net::Layer &L = net->layers[i];
+    L.spec            = layers[i];
+    if (L.spec.kind == TDH_L_CONV && L.spec.conv.tbl) {
+      L.tbl.assign(L.spec.conv.tbl,
+                   L.spec.conv.tbl + static_cast<size_t>(L.spec.conv.in_c) * L.spec.conv.out_c);
+      L.spec.conv.tbl = L.tbl.data();
+    }
+    if (L.spec.kind == TDH_L_ACT) {
+      if (i == 0) {
+        rc = set_error(TDH_ERR_INVALID, "tdh_net_create: an activation cannot be the first layer");
+        break;
+      }
+      L.in_size = L.out_size = net->layers[i - 1].out_size;
+    }
+    rc = layer_sizes(L);
+    if (rc == TDH_OK && i > 0 && L.in_size != net->layers[i - 1].out_size)
+      rc = set_error(TDH_ERR_INVALID, "tdh_net_create: layer %d expects %zu inputs, layer %d gives %zu",
+                     i, L.in_size, i - 1, net->layers[i - 1].out_size);
+    if (rc == TDH_OK && (L.in_size * max_batch >= (1ul << 31) || L.out_size * max_batch >= (1ul << 31)))
+      rc = set_error(TDH_ERR_INVALID, "tdh_net_create: layer %d activations exceed 2^31 elements", i);
+  }
+  for (int i = 0; i < n_layers && rc == TDH_OK; ++i) {
+    tdh_net::Layer &L = net->layers[i];
+    const size_t act  = L.out_size * static_cast<size_t>(max_batch);
+    if ((rc = net_alloc(net, L.w_size, &L.w, true))) break;
+    if ((rc = net_alloc(net, L.w_size, &L.dw, true))) break;
+    if ((rc = net_alloc(net, L.w_size, &L.s0w, true))) break;
+    if ((rc = net_alloc(net, L.w_size, &L.s1w, true))) break;
+    if ((rc = net_alloc(net, L.b_size, &L.b, true))) break;
+    if ((rc = net_alloc(net, L.b_size, &L.db, true))) break;
+    if ((rc = net_alloc(net, L.b_size, &L.s0b, true))) break;
+    if ((rc = net_alloc(net, L.b_size, &L.s1b, true))) break;
+    if ((rc = net_alloc(net, act, &L.out, true))) break;
+    if ((rc = net_alloc(net, act, &L.dout, true))) break;
+    if (L.spec.kind == TDH_L_MAXPOOL) {
+      float *p = nullptr;
+      if ((rc = net_alloc(net, act, &p, true))) break;
+      L.argmax = reinterpret_cast<int32_t *>(p);
+    }
+    size_t need = 0;
+    if (L.spec.kind == TDH_L_CONV) need = conv2d_workspace_bytes(&L.spec.conv, max_batch);
+    if (L.spec.kind == TDH_L_FC) need = fc_workspace_bytes(L.spec.fc_in, L.spec.fc_out, max_batch);
+    if (L.spec.kind == TDH_L_AVEPOOL) need = avepool_workspace_bytes(&L.spec.pool, max_batch);
+    if (need > net->scratch) net->scratch = need;
+    // fold pointwise activation gradients into the following conv/fc dX epilogue
+    if ((flags & TDH_NET_FUSE_ACT_GRAD) && L.spec.kind == TDH_L_ACT &&
+        is_pointwise_act(L.spec.act) && i + 1 < n_layers &&
+        (layers[i + 1].kind == TDH_L_CONV || layers[i + 1].kind == TDH_L_FC))
+      L.grad_folded = true;
+  }
+  if (rc == TDH_OK)
+    rc = net_alloc(net, net->layers[0].in_size * static_cast<size_t>(max_batch), &net->dx_in, true);
+  if (rc != TDH_OK) {
+    for (void *p : net->allocs) (void)hipFree(p);
+    delete net;
+    return rc;
+  }
+  *out = net;
+  return TDH_OK;
+}
+
+int tdh_net_destroy(tdh_net *net) {
+  TDH_REQUIRE_INIT();
+  if (!net) return TDH_OK;
+  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  for (void *p : net->allocs) TDH_HIP(hipFree(p));
+  delete net;
+  return TDH_OK;
+}
+
+size_t tdh_net_in_size(const tdh_net *net) { return net->layers.front().in_size; }
+size_t tdh_net_out_size(const tdh_net *net) { return net->layers.back().out_size; }
+size_t tdh_net_layer_out_size(const tdh_net *net, int layer) {
+  return (layer >= 0 && layer < static_cast<int>(net->layers.size())) ? net->layers[layer].out_size : 0;
+}
+size_t tdh_net_param_size(const tdh_net *net, int layer, int which) {
+  if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return 0;
+  return which == 0 ? net->layers[layer].w_size : (which == 1 ? net->layers[layer].b_size : 0);
+}
+float *tdh_net_param(tdh_net *net, int layer, int which) {
+  if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
+  return which == 0 ? net->layers[layer].w : (which == 1 ? net->layers[layer].b : nullptr);
+}
+int tdh_net_set_param(tdh_net *net, int layer, int which, const float *host_src) {
+  TDH_REQUIRE_INIT();
+  float *dst = tdh_net_param(net, layer, which);
+  const size_t n = tdh_net_param_size(net, layer, which);
+  TDH_CHECK_ARG(n == 0 || (dst && host_src), "tdh_net_set_param: no such parameter");
+  return tdh_memcpy_h2d(dst, host_src, n * sizeof(float));
+}
+int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst) {
+  TDH_REQUIRE_INIT();
+  const float *src = tdh_net_param(net, layer, which);
+  const size_t n   = tdh_net_param_size(net, layer, which);
+  TDH_CHECK_ARG(n == 0 || (src && host_dst), "tdh_net_get_param: no such parameter");
+  return tdh_memcpy_d2h(host_dst, src, n * sizeof(float));
+}
+const float *tdh_net_layer_out(const tdh_net *net, int layer) {
+  return (layer >= 0 && layer < static_cast<int>(net->layers.size())) ? net->layers[layer].out : nullptr;
+}
+const float *tdh_net_layer_dx(const tdh_net *net, int layer) {
+  if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
+  return layer == 0 ? net->dx_in : net->layers[layer - 1].dout;
+}
+const float *tdh_net_layer_grad(const tdh_net *net, int layer, int which) {
+  if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
+  return which == 0 ? net->layers[layer].dw : (which == 1 ? net->layers[layer].db : nullptr);
+}
+const int32_t *tdh_net_layer_argmax(const tdh_net *net, int layer) {
+  return (layer >= 0 && layer < static_cast<int>(net->layers.size())) ? net->layers[layer].argmax : nullptr;
+}
+
+int tdh_net_forward(tdh_net *net, int batch, const float *x) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && x && batch > 0 && batch <= net->max_batch, "tdh_net_forward: bad argument");
+  return forward(net, batch, x);
+}
+
+int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
+                       const float *t, int do_update) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && x && t && batch > 0 && batch <= net->max_batch,
+                "tdh_net_train_step: bad argument");
+  TDH_CHECK_ARG(!do_update || opt, "tdh_net_train_step: update requested without an optimizer");
+  TDH_TRY(forward(net, batch, x));
+  const int n          = static_cast<int>(net->layers.size());
+  tdh_net::Layer &last = net->layers[n - 1];
+  int first_bwd        = n - 1;
+  // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
+  // the full softmax Jacobian
+  if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
+      last.spec.act == TDH_ACT_SOFTMAX && n >= 2) {
+    TDH_TRY(launch_softmax_xent_grad(batch, static_cast<int>(last.out_size), last.out, t,
+                                     net->layers[n - 2].dout));
+    first_bwd = n - 2;
+  } else {
+    TDH_TRY(launch_loss_grad(loss_kind, batch, static_cast<int>(last.out_size), last.out, t,
+                             last.dout));
+  }
+  for (int i = first_bwd; i >= 0; --i) {
+    tdh_net::Layer &L  = net->layers[i];
+    const tdh_layer &s = L.spec;
+    const float *in    = i == 0 ? x : net->layers[i - 1].out;
+    float *dx          = i == 0 ? net->dx_in : net->layers[i - 1].dout;
+    ActGrad fold;
+    if (i >= 1 && net->layers[i - 1].grad_folded) {
+      // write straight into the activation's input gradient, scaled by act'(its output)
+      fold.kind = net->layers[i - 1].spec.act;
+      fold.y    = net->layers[i - 1].out;
+      dx        = i - 1 == 0 ? net->dx_in : net->layers[i - 2].dout;
+    }
+    switch (s.kind) {
+      case TDH_L_CONV:
+        TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
+        TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
+                           fold));
+        break;
+      case TDH_L_FC:
+        TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
+        TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
+                       L.b_size ? L.db : nullptr, 1, fold));
+        break;
+      case TDH_L_MAXPOOL: TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx)); break;
+      case TDH_L_AVEPOOL:
+        TDH_TRY(ws_begin(avepool_workspace_bytes(&s.pool, batch)));
+        TDH_TRY(avepool_bwd(&s.pool, batch, in, L.w, L.dout, dx, L.dw, L.db, 1));
+        break;
+      case TDH_L_ACT:
+        if (!L.grad_folded)
+          TDH_TRY(launch_act_bwd(s.act, batch, static_cast<int>(L.out_size), L.out, L.dout, dx));
+        break;
+    }
+  }
+  if (!do_update) return TDH_OK;
+  // nodes::update_weights visits layers front to back, weight before bias; the gradient
+  // reaches the optimizer unscaled (rcp_batch_size is 1, see tdh_opt_update) and is then
+  // cleared (layer.h:680)
+  for (auto &L : net->layers) {
+    if (L.w_size) {
+      TDH_TRY(launch_opt_update(opt, L.w_size, L.dw, 1.0f, L.w, L.s0w, L.s1w));
+      TDH_TRY(launch_fill_zero(L.dw, L.w_size * sizeof(float)));
+    }
+    if (L.b_size) {
+      TDH_TRY(launch_opt_update(opt, L.b_size, L.db, 1.0f, L.b, L.s0b, L.s1b));
+      TDH_TRY(launch_fill_zero(L.db, L.b_size * sizeof(float)));
+    }
+  }
+  return TDH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,272 @@
+// pool.hip — max pooling (argmax record + gather backward) and tiny-dnn's trainable
+// average pooling, forward and backward. All kernels stream each tensor once.
+// Built with -ffp-contract=off (see elementwise.hip).
+#include <cfloat>
+
+#include "common.h"
+
+namespace tdh {
+
+namespace {
+
+constexpr int PT = 256;
+
+struct PoolGeom {
+  int C, H, W, OH, OW, pw, ph, sw, sh;
+  FastDiv div_ow, div_oh, div_c, div_w, div_h;
+};
+
+PoolGeom make_geom(const tdh_pool_desc *d) {
+  PoolGeom g;
+  g.C = d->in_c; g.H = d->in_h; g.W = d->in_w;
+  g.OW = pool_out_length(d->in_w, d->pool_w, d->stride_w, d->ceil_mode, d->pad_same);
+  g.OH = pool_out_length(d->in_h, d->pool_h, d->stride_h, d->ceil_mode, d->pad_same);
+  g.pw = d->pool_w; g.ph = d->pool_h; g.sw = d->stride_w; g.sh = d->stride_h;
+  g.div_ow = FastDiv(g.OW > 0 ? g.OW : 1); g.div_oh = FastDiv(g.OH > 0 ? g.OH : 1);
+  g.div_c = FastDiv(g.C); g.div_w = FastDiv(g.W); g.div_h = FastDiv(g.H);
+  return g;
+}
+
+// maxpool_op_internal.h:16-40 with the windows of max_pooling_layer::connect_kernel
+// (max_pooling_layer.h:195-222): clipped at the right/bottom edge, scanned row by row,
+// strict '>' from numeric_limits::lowest() so the first maximum wins, NaN never wins and
+// an all-NaN window reports index 0.
+__global__ void __launch_bounds__(PT)
+maxpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
+                   int32_t *__restrict__ argmax, const int total, const PoolGeom g) {
+  const int o = blockIdx.x * PT + threadIdx.x;
+  if (o >= total) return;
+  uint32_t t, ox, oy, c, img;
+  g.div_ow.divmod(o, t, ox);
+  g.div_oh.divmod(t, t, oy);
+  g.div_c.divmod(t, img, c);
+  const int x0 = ox * g.sw, y0 = oy * g.sh;
+  const int dxmax = min(g.pw, g.W - x0), dymax = min(g.ph, g.H - y0);
+  const float *in = x + static_cast<size_t>(img) * g.C * g.H * g.W;
+  float best      = -FLT_MAX;
+  int idx         = 0;
+  for (int wy = 0; wy < dymax; ++wy)
+    for (int wx = 0; wx < dxmax; ++wx) {
+      const int j   = (g.H * c + y0 + wy) * g.W + x0 + wx;
+      const float v = in[j];
+      if (v > best) {
+        best = v;
+        idx  = j;
+      }
+    }
+  y[o] = best;
+  if (argmax) argmax[o] = idx;
+}
+
+// maxpool_grad_op_internal (maxpool_op_internal.h:42-57). in2out[i] is the LAST window, in
+// (c, oy, ox) creation order, that contains input i (max_pooling_layer.h:218), and 0 for
+// inputs no window contains (strides larger than the window).
+__global__ void __launch_bounds__(PT)
+maxpool_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ argmax,
+                   float *__restrict__ dx, const int total, const PoolGeom g) {
+  const int i = blockIdx.x * PT + threadIdx.x;
+  if (i >= total) return;
+  uint32_t t, xx, yy, c, img;
+  g.div_w.divmod(i, t, xx);
+  g.div_h.divmod(t, t, yy);
+  g.div_c.divmod(t, img, c);
+  const int ox = min(g.OW - 1, static_cast<int>(xx) / g.sw);
+  const int oy = min(g.OH - 1, static_cast<int>(yy) / g.sh);
+  const bool covered = (static_cast<int>(xx) < ox * g.sw + g.pw) &&
+                       (static_cast<int>(yy) < oy * g.sh + g.ph);
+  const int outi  = covered ? (g.OH * c + oy) * g.OW + ox : 0;
+  const int local = (g.H * c + yy) * g.W + xx;  // flat CHW index inside the sample
+  const size_t ob = static_cast<size_t>(img) * g.C * g.OH * g.OW;
+  dx[i]           = (argmax[ob + outi] == local) ? dy[ob + outi] : 0.0f;
+}
+
+// tiny_average_pooling_kernel (average_pooling_layer.h:25-55). Window (oy,ox) exists when it
+// lies fully inside the input (init_connection, :270-278); outputs without a window keep
+// the empty sum. value = sum * (W[c]*scale) + b[c], in that order.
+__global__ void __launch_bounds__(PT)
+avepool_fwd_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                   const float *__restrict__ b, float *__restrict__ y, const int total,
+                   const PoolGeom g, const float scale) {
+  const int o = blockIdx.x * PT + threadIdx.x;
+  if (o >= total) return;
+  uint32_t t, ox, oy, c, img;
+  g.div_ow.divmod(o, t, ox);
+  g.div_oh.divmod(t, t, oy);
+  g.div_c.divmod(t, img, c);
+  const int x0 = ox * g.sw, y0 = oy * g.sh;
+  float value  = 0.0f;
+  if (x0 + g.pw <= g.W && y0 + g.ph <= g.H) {
+    const float *in = x + (static_cast<size_t>(img) * g.C + c) * g.H * g.W;
+    for (int wy = 0; wy < g.ph; ++wy)
+      for (int wx = 0; wx < g.pw; ++wx) value += in[(y0 + wy) * g.W + x0 + wx];
+  }
+  const float weight = w[c] * scale;
+  value *= weight;
+  value += b[c];
+  y[o] = value;
+}
+
+// prev_delta[idx] = (W[c]*scale) * curr_delta[first window containing idx]
+// (average_pooling_layer.h:78-85; in2wo[idx][0] is the earliest created window)
+__global__ void __launch_bounds__(PT)
+avepool_bwd_dx_kernel(const float *__restrict__ dy, const float *__restrict__ w,
+                      float *__restrict__ dx, const int total, const PoolGeom g,
+                      const float scale) {
+  const int i = blockIdx.x * PT + threadIdx.x;
+  if (i >= total) return;
+  uint32_t t, xx, yy, c, img;
+  g.div_w.divmod(i, t, xx);
+  g.div_h.divmod(t, t, yy);
+  g.div_c.divmod(t, img, c);
+  const int ix = xx, iy = yy;
+  const int ox = ix < g.pw ? 0 : (ix - g.pw + g.sw) / g.sw;
+  const int oy = iy < g.ph ? 0 : (iy - g.ph + g.sh) / g.sh;
+  const float weight = w[c] * scale;
+  dx[i] = weight * dy[((static_cast<size_t>(img) * g.C + c) * g.OH + oy) * g.OW + ox];
+}
+
+__device__ __forceinline__ float wave_sum_p(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// One block per (sample, channel): partial[(img*C + c)*2 + {0,1}] =
+//   { sum over windows of dy[o] * (sum of x in the window),  sum of dy[o] }
+// (average_pooling_layer.h:87-104, the pair lists regrouped by output)
+__global__ void __launch_bounds__(PT)
+avepool_bwd_param_kernel(const float *__restrict__ x, const float *__restrict__ dy,
+                         float *__restrict__ partial, const PoolGeom g) {
+  __shared__ float sm[8];
+  const int plane = blockIdx.x;  // img*C + c
+  const float *in = x + static_cast<size_t>(plane) * g.H * g.W;
+  const float *d  = dy + static_cast<size_t>(plane) * g.OH * g.OW;
+  float sw_ = 0.0f, sb = 0.0f;
+  for (int o = threadIdx.x; o < g.OH * g.OW; o += PT) {
+    const int oy = o / g.OW, ox = o - oy * g.OW;
+    const int x0 = ox * g.sw, y0 = oy * g.sh;
+    const float dv = d[o];
+    sb += dv;
+    if (x0 + g.pw <= g.W && y0 + g.ph <= g.H) {
+      float win = 0.0f;
+      for (int wy = 0; wy < g.ph; ++wy)
+        for (int wx = 0; wx < g.pw; ++wx) win += in[(y0 + wy) * g.W + x0 + wx];
+      sw_ += win * dv;
+    }
+  }
+  sw_ = wave_sum_p(sw_);
+  sb  = wave_sum_p(sb);
+  if ((threadIdx.x & 63) == 0) {
+    sm[(threadIdx.x >> 6) * 2]     = sw_;
+    sm[(threadIdx.x >> 6) * 2 + 1] = sb;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    partial[plane * 2]     = (sm[0] + sm[2]) + (sm[4] + sm[6]);
+    partial[plane * 2 + 1] = (sm[1] + sm[3]) + (sm[5] + sm[7]);
+  }
+}
+
+// dW[c] (+)= scale * sum_img partial_w, db[c] (+)= sum_img partial_b, samples in order
+__global__ void __launch_bounds__(PT)
+avepool_bwd_param_reduce_kernel(const float *__restrict__ partial, const int batch, const int C,
+                                const float scale, float *__restrict__ dw,
+                                float *__restrict__ db, const int accumulate) {
+  const int c = blockIdx.x * PT + threadIdx.x;
+  if (c >= C) return;
+  float mw = 0.0f, mb = 0.0f;
+  for (int s = 0; s < batch; ++s) {
+    mw += partial[(s * C + c) * 2] * scale;
+    mb += partial[(s * C + c) * 2 + 1];
+  }
+  if (dw) dw[c] = accumulate ? dw[c] + mw : mw;
+  if (db) db[c] = accumulate ? db[c] + mb : mb;
+}
+
+}  // namespace
+
+int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax) {
+  const PoolGeom g = make_geom(d);
+  const long total = static_cast<long>(batch) * g.C * g.OH * g.OW;
+  if (total <= 0) return TDH_OK;
+  hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
+                     y, argmax, static_cast<int>(total), g);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
+                float *dx) {
+  const PoolGeom g = make_geom(d);
+  const long total = static_cast<long>(batch) * g.C * g.H * g.W;
+  TDH_CHECK_ARG(g.OH > 0 && g.OW > 0, "maxpool backward: empty output");
+  hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, dy,
+                     argmax, dx, static_cast<int>(total), g);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+// average_pooling_layer's constructor throws unless the input is a multiple of the window
+// (average_pooling_layer.h:216-218)
+static int check_avepool(const tdh_pool_desc *d) {
+  TDH_CHECK_ARG(d->in_w % d->pool_w == 0 && d->in_h % d->pool_h == 0,
+                "average pooling: input %dx%d is not a multiple of the window %dx%d", d->in_w,
+                d->in_h, d->pool_w, d->pool_h);
+  return TDH_OK;
+}
+
+int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *b,
+                float *y) {
+  TDH_TRY(check_avepool(d));
+  const PoolGeom g = make_geom(d);
+  const long total = static_cast<long>(batch) * g.C * g.OH * g.OW;
+  if (total <= 0) return TDH_OK;
+  const float scale = 1.0f / static_cast<float>(d->pool_w * d->pool_h);
+  hipLaunchKernelGGL(avepool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
+                     w, b, y, static_cast<int>(total), g, scale);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+size_t avepool_workspace_bytes(const tdh_pool_desc *d, int batch) {
+  return ws_align(static_cast<size_t>(batch) * d->in_c * 2 * sizeof(float));
+}
+
+int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,
+                float *dx, float *dw, float *db, int accumulate) {
+  TDH_TRY(check_avepool(d));
+  const PoolGeom g = make_geom(d);
+  // Every input element must lie in at least one window that maps to an existing output;
+  // the reference dereferences in2wo[idx][0] unconditionally.
+  for (int axis = 0; axis < 2; ++axis) {
+    const int len = axis ? g.H : g.W, pool = axis ? g.ph : g.pw, stride = axis ? g.sh : g.sw;
+    const int outs = axis ? g.OH : g.OW;
+    for (int i = 0; i < len; ++i) {
+      const int o = i < pool ? 0 : (i - pool + stride) / stride;
+      const bool ok = o * stride <= i && o * stride + pool <= len && o < outs;
+      TDH_CHECK_ARG(ok, "average pooling backward: input %s %d is covered by no window",
+                    axis ? "row" : "column", i);
+    }
+  }
+  const float scale = 1.0f / static_cast<float>(d->pool_w * d->pool_h);
+  if (dx) {
+    const long total = static_cast<long>(batch) * g.C * g.H * g.W;
+    hipLaunchKernelGGL(avepool_bwd_dx_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream,
+                       dy, w, dx, static_cast<int>(total), g, scale);
+    TDH_LAUNCH_CHECK();
+  }
+  if (dw || db) {
+    void *ws = nullptr;
+    TDH_TRY(ws_take(static_cast<size_t>(batch) * g.C * 2 * sizeof(float), &ws));
+    hipLaunchKernelGGL(avepool_bwd_param_kernel, dim3(batch * g.C), dim3(PT), 0, ctx().stream, x,
+                       dy, static_cast<float *>(ws), g);
+    TDH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(avepool_bwd_param_reduce_kernel, dim3(ceil_div(g.C, PT)), dim3(PT), 0,
+                       ctx().stream, static_cast<const float *>(ws), batch, g.C, scale, dw, db,
+                       accumulate);
+    TDH_LAUNCH_CHECK();
+  }
+  return TDH_OK;
+}
+
+}  // namespace tdh
