@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""Benchmark of the tiny-dnn training hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--others]
+
+Prints ONE JSON line. The default workload is the CIFAR-10-shape CNN train step at batch
+128 (fwd + bwd + update, Adam), the configuration the samples/s target is quoted on; inputs
+are synthetic and resident in HBM before the timed region. Other workloads:
+vgg_stack_b64, lenet5_b16 (train steps), conv2d_bwd_b64 and fc_bwd_adam_b256 (single-op
+backward passes). ``--others`` appends their results under "others".
+
+"roofline" describes the kernel with the largest total time in the workload: its average
+launch duration is measured with HIP events on the library's stream in a second, separately
+timed pass (per-launch events slow the step down, so they are kept out of ``value``).
+"cpu_baseline" times the reference's OpenMP+AVX build (oracle/_ref, kind "reference") or,
+where that library is absent, the scalar restatement (kind "port") on this host's cores.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def load_pkg():
+    T = importlib.import_module("tiny-cnn_amd")
+    W = importlib.import_module("tiny-cnn_amd.workloads")
+    return T, W
+
+
+class NetWorkload:
+    def __init__(self, T, W, name):
+        self.T, self.W, self.name = T, W, name
+        (self.spec, self.params, x, t, self.batch, self.loss, self.opt_kind,
+         self.opt_kw) = W.make_batch(name)
+        self.net = T.Net(W.build_layers(T, self.spec), self.batch, T.NET_FUSE_ACT_GRAD)
+        for (i, which, a) in self.params:
+            self.net.set_param(i, which, a)
+        self.opt = T.opt_desc(self.opt_kind, **self.opt_kw)
+        self.x, self.t = T.to_device(x), T.to_device(t)
+        self.samples = self.batch
+        self.config = {"workload": name, "batch": self.batch, "loss": self.loss,
+                       "optimizer": self.opt_kind, "step": "fwd+bwd+update",
+                       "flop_per_step": 3 * self.batch * W.flops_per_sample(self.spec)}
+
+    def step(self):
+        self.net.train_step(self.opt, self.loss, self.batch, self.x, self.t)
+
+
+class ConvBwdWorkload:
+    """configs[1]: conv2d backward, batch 64, 32x64x64 -> 64 channels, 3x3, pad same."""
+
+    def __init__(self, T, W, name="conv2d_bwd_b64", batch=64):
+        self.T = T
+        (hw, _, c, k, oc), x, w, dy = W.conv_bwd_case(batch=batch)
+        self.d = T.conv_desc(hw, hw, c, k, k, oc, pad_same=True)
+        self.batch = self.samples = batch
+        self.x, self.w, self.dy = T.to_device(x), T.to_device(w), T.to_device(dy)
+        self.dx, self.dw, self.db = T.DevBuf(x.shape), T.DevBuf(w.shape), T.DevBuf((oc,))
+        gemm_flop = 2 * batch * hw * hw * oc * c * k * k
+        self.config = {"workload": name, "batch": batch, "step": "conv2d backward (dX, dW, db)",
+                       "flop_per_step": 2 * gemm_flop}
+
+    def step(self):
+        self.T.conv2d_bwd(self.d, self.batch, self.x, self.w, self.dy, self.dx, self.dw, self.db)
+
+
+class FcBwdWorkload:
+    """configs[2]: tanh-grad -> FC backward (dX, dW, db) -> Adam on W and b, batch 256."""
+
+    def __init__(self, T, W, name="fc_bwd_adam_b256", batch=256, n=4096):
+        self.T = T
+        x, w, b, dy = W.fc_bwd_case(batch, n, n)
+        self.n, self.batch, self.samples = n, batch, batch
+        self.x, self.w, self.b = T.to_device(x), T.to_device(w), T.to_device(b)
+        self.y, self.dy, self.dz = T.DevBuf((batch, n)), T.to_device(dy), T.DevBuf((batch, n))
+        T.fc_fwd(n, n, True, batch, self.x, self.w, self.b, self.dz)
+        T.act_fwd("tanh", batch, n, self.dz, self.y)
+        self.dx, self.dw, self.db = T.DevBuf((batch, n)), T.DevBuf((n * n,)), T.DevBuf((n,))
+        self.s = [T.DevBuf((n * n,), zero=True), T.DevBuf((n * n,), zero=True),
+                  T.DevBuf((n,), zero=True), T.DevBuf((n,), zero=True)]
+        self.opt = T.opt_desc("adam")
+        self.config = {"workload": name, "batch": batch, "step": "tanh-grad + fc backward + adam",
+                       "flop_per_step": 4 * batch * n * n}
+
+    def step(self):
+        T, n, bs = self.T, self.n, self.batch
+        T.act_bwd("tanh", bs, n, self.y, self.dy, self.dz)
+        T.fc_bwd(n, n, True, bs, self.x, self.w, self.dz, self.dx, self.dw, self.db)
+        T.opt_update(self.opt, n * n, self.dw, self.w, self.s[0], self.s[1])
+        T.opt_update(self.opt, n, self.db, self.b, self.s[2], self.s[3])
+
+
+def make_workload(T, W, name):
+    if name in W.WORKLOADS:
+        return NetWorkload(T, W, name)
+    if name == "conv2d_bwd_b64":
+        return ConvBwdWorkload(T, W)
+    if name == "fc_bwd_adam_b256":
+        return FcBwdWorkload(T, W)
+    raise SystemExit(f"unknown workload {name}")
+
+
+def roofline_of(entry):
+    per_s = entry["work"] / (entry["avg_us"] * 1e-6) if entry["avg_us"] > 0 else 0.0
+    if entry["unit"] == "flop":
+        achieved, peak, unit, bound = per_s / 1e12, PEAK_FP32_MFMA_TFLOPS, "TFLOP/s", "mfma"
+    else:
+        achieved, peak, unit, bound = per_s / 1e9, PEAK_HBM_GBS, "GB/s", "hbm"
+    return {"kernel": entry["tag"], "bound": bound, "achieved": round(achieved, 3), "peak": peak,
+            "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
+            "avg_launch_us": round(entry["avg_us"], 2), "launches": entry["launches"],
+            "algorithmic_work_per_launch": entry["work"]}
+
+
+def run_workload(T, wl, steps, warmup, profile_steps):
+    for _ in range(warmup):
+        wl.step()
+    T.sync()
+    e0, e1 = T.Event(), T.Event()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        wl.step()
+    e1.record()
+    T.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = e1.elapsed_ms_since(e0)
+    ms_per_step = wall_ms / steps
+    # second pass: per-kernel durations from events around every launch
+    T.profile_begin()
+    for _ in range(profile_steps):
+        wl.step()
+    prof = T.profile_end()
+    kernels = [roofline_of(e) for e in prof]
+    for k, e in zip(kernels, prof):
+        k["ms_per_step"] = round(e["total_ms"] / profile_steps, 4)
+    return {"ms_per_step": ms_per_step, "gpu_ms_per_step": gpu_ms / steps,
+            "samples_per_s": wl.samples / (ms_per_step * 1e-3), "kernels": kernels}
+
+
+def cpu_baseline(W, name, budget_s=20.0):
+    """Reference CPU figure on a bounded sample of the same workload."""
+    from oracle import oracle as O
+    try:
+        if not os.path.exists(O.ORACLE_SO):
+            O.build()
+    except Exception:
+        pass
+    kind = "reference" if O.ref_lib("avx") is not None else "port"
+    cores = os.cpu_count() or 1
+    if kind == "reference":
+        cores = O.ref_lib("avx").tdr_num_threads()
+    if name in W.WORKLOADS:
+        full_batch = W.WORKLOADS[name][1]
+        batch = {"vgg_stack_b64": 2}.get(name, full_batch)
+        spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch)
+        opt = O.opt_desc(opt_kind, **opt_kw)
+        if kind == "reference":
+            net = O.RefNet(W.build_layers(O, spec), "avx", 1)
+            for (i, which, a) in params:
+                net.set_param(i, which, a)
+            net.fit(opt, loss, x, t, 1)  # warm-up step (allocates the per-sample buffers)
+            steps, spent, per = 0, 0.0, []
+            while spent < budget_s and steps < 20:
+                sec = net.fit(opt, loss, x, t, 1)
+                per.append(sec); spent += sec; steps += 1
+        else:
+            net = O.OracleNet(W.build_layers(O, spec), batch)
+            for (i, which, a) in params:
+                (net.weight(i) if which == 0 else net.bias(i))[:] = a
+            steps, spent, per = 0, 0.0, []
+            while spent < budget_s and steps < 20:
+                t0 = time.perf_counter(); net.train_step(opt, loss, x, t)
+                sec = time.perf_counter() - t0
+                per.append(sec); spent += sec; steps += 1
+        med = float(np.median(per))
+        return {"value": round(batch / med, 2), "unit": "samples/s", "cores": cores, "kind": kind,
+                "sample": f"{steps} train steps at batch {batch} (full workload batch {full_batch}), "
+                          f"median {med * 1e3:.1f} ms/step"}
+    if name == "conv2d_bwd_b64":
+        batch = 8
+        (hw, _, c, k, oc), x, w, dy = W.conv_bwd_case(batch=batch)
+        d = O.conv_desc(hw, hw, c, k, k, oc, pad_same=True)
+        if kind == "reference":
+            *_, sec = O.ref_conv2d_bwd(d, x, w, dy, kind="avx", engine=1, repeat=3, want_time=True)
+        else:
+            t0 = time.perf_counter(); O.conv2d_bwd(d, x, w, dy); sec = time.perf_counter() - t0
+        return {"value": round(batch / sec, 2), "unit": "samples/s", "cores": cores, "kind": kind,
+                "sample": f"layer.backward at batch {batch} (full workload batch 64), best of 3: "
+                          f"{sec * 1e3:.1f} ms"}
+    if name == "fc_bwd_adam_b256":
+        batch = 16
+        x, w, b, dy = W.fc_bwd_case(batch)
+        if kind == "reference":
+            *_, sec = O.ref_fc_bwd(x, w, dy, kind="avx", engine=1, repeat=3, want_time=True)
+        else:
+            t0 = time.perf_counter(); O.fc_bwd(x, w, dy); sec = time.perf_counter() - t0
+        return {"value": round(batch / sec, 2), "unit": "samples/s", "cores": cores, "kind": kind,
+                "sample": f"fc layer.backward only (no tanh-grad/adam) at batch {batch} (full "
+                          f"workload batch 256; per-sample gradient storage needs 67 MB/sample), "
+                          f"best of 3: {sec * 1e3:.1f} ms"}
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cifar10_cnn_b128")
+    ap.add_argument("--others", action="store_true", help="also run the other workloads")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    T, W = load_pkg()
+    T.init(0)
+    dev_name, cus, mem = T.device_info()
+
+    wl = make_workload(T, W, args.workload)
+    prof_steps = max(1, min(args.steps, 10))
+    res = run_workload(T, wl, args.steps, args.warmup, prof_steps)
+    out = {
+        "metric": "train samples/sec (fwd+bwd+update)",
+        "value": round(res["samples_per_s"], 2),
+        "unit": "samples/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(res["ms_per_step"], 4),
+        "gpu_ms_per_step": round(res["gpu_ms_per_step"], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": wl.config,
+        "device": {"name": dev_name, "compute_units": cus},
+        "roofline": res["kernels"][0] if res["kernels"] else None,
+        "kernels": res["kernels"],
+    }
+    if wl.config.get("flop_per_step"):
+        out["step_tflops"] = round(wl.config["flop_per_step"] / (res["ms_per_step"] * 1e-3) / 1e12, 3)
+    del wl
+    if not args.no_cpu_baseline:
+        try:
+            out["cpu_baseline"] = cpu_baseline(W, args.workload)
+            if out["cpu_baseline"]:
+                out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1)
+        except Exception as e:  # the baseline is reported, never required
+            out["cpu_baseline"] = {"error": repr(e)}
+    if args.others:
+        others = {}
+        for name in ("conv2d_bwd_b64", "fc_bwd_adam_b256", "vgg_stack_b64", "lenet5_b16",
+                     "cifar10_cnn_b128"):
+            if name == args.workload:
+                continue
+            w2 = make_workload(T, W, name)
+            r = run_workload(T, w2, max(5, args.steps // 2), max(2, args.warmup // 2), 5)
+            others[name] = {"samples_per_s": round(r["samples_per_s"], 2),
+                            "ms_per_step": round(r["ms_per_step"], 4), "config": w2.config,
+                            "step_tflops": round(w2.config["flop_per_step"] /
+                                                 (r["ms_per_step"] * 1e-3) / 1e12, 3),
+                            "kernels": r["kernels"][:6]}
+            del w2
+        out["others"] = others
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

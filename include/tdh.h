@@ -116,6 +116,16 @@ int tdh_event_destroy(void *event);
 int tdh_event_record(void *event);
 int tdh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
 
+/* Per-kernel timing of everything launched between begin and end: each launch is
+ * bracketed by events on the library stream and booked under a kernel tag with its
+ * algorithmic work (unit 0 = FLOP, 1 = bytes). The events add launch overhead, so
+ * whole-step throughput is measured with profiling off. tdh_profile_end waits for the
+ * GPU; entries are then read back by index, ordered by total time (largest first). */
+int tdh_profile_begin(void);
+int tdh_profile_end(int32_t *n_entries);
+int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launches,
+                      double *total_ms, double *work_per_launch, int32_t *work_unit);
+
 /* shape helpers: conv_out_length / pool_out_length (tiny_dnn/util/util.h:329-363) */
 int tdh_conv_out_w(const tdh_conv_desc *d);
 int tdh_conv_out_h(const tdh_conv_desc *d);

@@ -191,6 +191,32 @@ class Event:
             pass
 
 
+def profile_begin():
+    """Start per-kernel timing (every launch gets a pair of events on the library stream)."""
+    check(lib().tdh_profile_begin(), "tdh_profile_begin")
+
+
+def profile_end():
+    """Stop per-kernel timing. Returns [dict(tag, launches, total_ms, avg_us, work, unit)]
+    sorted by total time; ``work`` is the algorithmic FLOP or bytes of one launch."""
+    n = C.c_int32()
+    check(lib().tdh_profile_end(C.byref(n)), "tdh_profile_end")
+    out = []
+    for i in range(n.value):
+        tag = C.create_string_buffer(128)
+        launches = C.c_int64()
+        total = C.c_double()
+        work = C.c_double()
+        unit = C.c_int32()
+        check(lib().tdh_profile_entry(i, tag, 128, C.byref(launches), C.byref(total),
+                                      C.byref(work), C.byref(unit)), "tdh_profile_entry")
+        out.append({"tag": tag.value.decode(), "launches": launches.value,
+                    "total_ms": total.value,
+                    "avg_us": 1e3 * total.value / max(1, launches.value),
+                    "work": work.value, "unit": "flop" if unit.value == 0 else "byte"})
+    return out
+
+
 # ------------------------------------------------------------------ descriptors
 
 def conv_desc(in_w, in_h, in_c, k_w, k_h, out_c, pad_same=False, has_bias=True, w_stride=1,

@@ -1,7 +1,11 @@
 // api.hip — library state, device memory, events and the thin extern "C" layer that
 // validates arguments before anything is launched.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <map>
+#include <string>
+#include <vector>
 
 #include "common.h"
 
@@ -52,6 +56,60 @@ int ws_take(size_t bytes, void **out) {
   *out = c.workspace + c.workspace_off;
   c.workspace_off += need;
   return TDH_OK;
+}
+
+// ----------------------------------------------------------------- profiler
+namespace {
+struct ProfRecord {
+  std::string tag;
+  double work;
+  WorkUnit unit;
+  hipEvent_t start, stop;
+};
+struct ProfEntry {
+  std::string tag;
+  int64_t launches = 0;
+  double total_ms = 0.0, work = 0.0;
+  int unit = 0;
+};
+bool g_profiling = false;
+std::vector<ProfRecord> g_records;
+std::vector<hipEvent_t> g_event_pool;
+std::vector<ProfEntry> g_entries;
+
+hipEvent_t take_event() {
+  if (!g_event_pool.empty()) {
+    hipEvent_t e = g_event_pool.back();
+    g_event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+}  // namespace
+
+static int open_record(const std::string &tag, double work, WorkUnit unit) {
+  ProfRecord r{tag, work, unit, take_event(), take_event()};
+  if (!r.start || !r.stop) return -1;
+  (void)hipEventRecord(r.start, ctx().stream);
+  g_records.push_back(r);
+  return static_cast<int>(g_records.size()) - 1;
+}
+
+ProfScope::ProfScope(const char *tag, double work, WorkUnit unit) : slot(-1) {
+  if (g_profiling) slot = open_record(tag, work, unit);
+}
+
+ProfScope::ProfScope(const char *tag, int m, int n, int k) : slot(-1) {
+  if (!g_profiling) return;
+  char buf[160];
+  std::snprintf(buf, sizeof(buf), "%s m=%d,n=%d,k=%d", tag, m, n, k);
+  slot = open_record(buf, 2.0 * m * n * k, WORK_FLOP);
+}
+
+ProfScope::~ProfScope() {
+  if (slot >= 0) (void)hipEventRecord(g_records[slot].stop, ctx().stream);
 }
 
 // tiny_dnn/util/util.h:329-344
@@ -239,6 +297,59 @@ int tdh_event_elapsed_ms(void *start, void *stop, float *ms) {
   TDH_CHECK_ARG(start && stop && ms, "tdh_event_elapsed_ms: null argument");
   TDH_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
   TDH_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return TDH_OK;
+}
+
+int tdh_profile_begin(void) {
+  TDH_REQUIRE_INIT();
+  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  for (auto &r : g_records) {
+    g_event_pool.push_back(r.start);
+    g_event_pool.push_back(r.stop);
+  }
+  g_records.clear();
+  g_entries.clear();
+  g_profiling = true;
+  return TDH_OK;
+}
+
+int tdh_profile_end(int32_t *n_entries) {
+  TDH_REQUIRE_INIT();
+  g_profiling = false;
+  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  std::map<std::string, ProfEntry> by_tag;
+  for (auto &r : g_records) {
+    float ms = 0.0f;
+    TDH_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
+    ProfEntry &e = by_tag[r.tag];
+    e.tag        = r.tag;
+    e.launches += 1;
+    e.total_ms += ms;
+    e.work += r.work;
+    e.unit = r.unit;
+    g_event_pool.push_back(r.start);
+    g_event_pool.push_back(r.stop);
+  }
+  g_records.clear();
+  g_entries.clear();
+  for (auto &kv : by_tag) g_entries.push_back(kv.second);
+  std::sort(g_entries.begin(), g_entries.end(),
+            [](const ProfEntry &a, const ProfEntry &b) { return a.total_ms > b.total_ms; });
+  if (n_entries) *n_entries = static_cast<int32_t>(g_entries.size());
+  return TDH_OK;
+}
+
+int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launches,
+                      double *total_ms, double *work_per_launch, int32_t *work_unit) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(index >= 0 && index < static_cast<int32_t>(g_entries.size()),
+                "tdh_profile_entry: index %d of %zu", index, g_entries.size());
+  const ProfEntry &e = g_entries[index];
+  if (tag && tag_len) std::snprintf(tag, tag_len, "%s", e.tag.c_str());
+  if (launches) *launches = e.launches;
+  if (total_ms) *total_ms = e.total_ms;
+  if (work_per_launch) *work_per_launch = e.launches ? e.work / e.launches : 0.0;
+  if (work_unit) *work_unit = e.unit;
   return TDH_OK;
 }
 

@@ -65,6 +65,20 @@ inline size_t ws_align(size_t bytes) { return (bytes + 255) & ~static_cast<size_
     if (rc_ != TDH_OK) return rc_;                                             \
   } while (0)
 
+// ------------------------------------------------------- per-kernel timing
+// When profiling is on (tdh_profile_begin), every kernel launch is bracketed by two
+// events on the library stream and booked under a tag together with its algorithmic
+// work (FLOP for the MFMA GEMMs, bytes for the bandwidth kernels). Off by default:
+// launches then record nothing.
+enum WorkUnit { WORK_FLOP = 0, WORK_BYTE = 1 };
+struct ProfScope {
+  ProfScope(const char *tag, double work, WorkUnit unit);
+  // GEMM launches carry their shape in the tag: "name m=..,n=..,k=.."
+  ProfScope(const char *tag, int m, int n, int k);
+  ~ProfScope();
+  int slot;
+};
+
 // ---------------------------------------------------------------- helpers
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline size_t ceil_div_sz(size_t a, size_t b) { return (a + b - 1) / b; }

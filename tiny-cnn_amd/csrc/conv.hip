@@ -237,6 +237,7 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
   TDH_HIP(hipMemcpyAsync(t, d->tbl, static_cast<size_t>(g.C) * g.Kc, hipMemcpyHostToDevice,
                          ctx().stream));
   TDH_HIP(hipStreamSynchronize(ctx().stream));
+  ProfScope prof("conv_mask_weights", 8.0 * nw, WORK_BYTE);
   hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(nw, 256)), dim3(256), 0, ctx().stream, w,
                      static_cast<const uint8_t *>(t), static_cast<float *>(wm), nw, g.C, g.Kc,
                      g.R * g.S, 0);
@@ -256,7 +257,7 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   StridedOperand A{w_eff, crs, 1, g.Kc};
   FwdInputOperand B{x, g, batch * ohw};
   EpiImageRows epi{y, g.Kc, ohw, g.div_ohw, d->has_bias ? b : nullptr, ActGrad()};
-  return launch_gemm<true, false>(A, B, epi, g.Kc, batch * ohw, crs, true);
+  return launch_gemm<true, false>(A, B, epi, g.Kc, batch * ohw, crs, true, "conv_fwd_gemm", "conv_fwd_splitk_reduce");
 }
 
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
@@ -270,7 +271,7 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
     DxWeightOperand A{w_eff, g.C, g.R * g.S, g.div_rs};
     DxDyOperand B{dy, g, batch * g.H * g.W};
     EpiImageRows epi{dx, g.C, g.H * g.W, g.div_hw, nullptr, dx_act};
-    TDH_TRY((launch_gemm<true, false>(A, B, epi, g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true)));
+    TDH_TRY((launch_gemm<true, false>(A, B, epi, g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true, "conv_dx_gemm", "conv_dx_splitk_reduce")));
   }
   if (dw) {
     DwDyOperand A{dy, g.Kc, ohw, g.div_ohw};
@@ -279,14 +280,15 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       void *tmp = nullptr;
       TDH_TRY(ws_take(sizeof(float) * g.Kc * crs, &tmp));
       EpiRowMajor epi{static_cast<float *>(tmp), crs, nullptr, ActGrad(), 0};
-      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true)));
+      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm", "conv_dw_splitk_reduce")));
+      ProfScope prof("conv_mask_weights", 8.0 * g.Kc * crs, WORK_BYTE);
       hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(g.Kc * crs, 256)), dim3(256), 0,
                          ctx().stream, static_cast<const float *>(tmp), tbl_dev, dw, g.Kc * crs,
                          g.C, g.Kc, g.R * g.S, accumulate);
       TDH_LAUNCH_CHECK();
     } else {
       EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
-      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true)));
+      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm", "conv_dw_splitk_reduce")));
     }
   }
   if (db) TDH_TRY(launch_rowsum(dy, batch, g.Kc, ohw, db, accumulate));

@@ -44,7 +44,8 @@ map_kernel(const float *__restrict__ a, const float *__restrict__ b, float *__re
 
 template <class Op, bool HAS_B>
 int launch_map(const float *a, const float *b, float *out, size_t n,
-               const typename Op::Params &prm) {
+               const typename Op::Params &prm, const char *tag) {
+  ProfScope prof(tag, (HAS_B ? 12.0 : 8.0) * n, WORK_BYTE);
   const bool vec  = aligned16(a) && aligned16(out) && (!HAS_B || aligned16(b));
   const size_t n4 = vec ? n / 4 : 0;
   hipLaunchKernelGGL((map_kernel<Op, HAS_B>), dim3(ew_blocks(vec ? n4 + 3 : n)), dim3(EW_THREADS),
@@ -262,6 +263,9 @@ opt_kernel(const float *__restrict__ g, float *__restrict__ w, float *__restrict
 
 template <int KIND, int NSTATE>
 int launch_opt(size_t n, const float *g, float *w, float *s0, float *s1, const OptScalars &p) {
+  static const char *const tags[] = {"opt_sgd", "opt_momentum", "opt_adam", "opt_adagrad",
+                                     "opt_rmsprop", "opt_adamax", "opt_nesterov"};
+  ProfScope prof(tags[KIND], (12.0 + 8.0 * NSTATE) * n, WORK_BYTE);
   const bool vec = aligned16(g) && aligned16(w) && (NSTATE < 1 || aligned16(s0)) &&
                    (NSTATE < 2 || aligned16(s1));
   const size_t n4 = vec ? n / 4 : 0;
@@ -325,6 +329,7 @@ colsum_kernel(const float *__restrict__ src, const int rows, const int cols,
 }  // namespace
 
 int launch_fill_zero(void *p, size_t bytes) {
+  ProfScope prof("fill_zero", static_cast<double>(bytes), WORK_BYTE);
   const size_t n  = bytes / 4;
   const size_t n4 = aligned16(p) ? n / 4 : 0;
   hipLaunchKernelGGL(fill_zero_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0,
@@ -336,14 +341,16 @@ int launch_fill_zero(void *p, size_t bytes) {
 int launch_act_fwd(int kind, int batch, int len, const float *x, float *y) {
   const size_t n = static_cast<size_t>(batch) * len;
   switch (kind) {
-    case TDH_ACT_TANH: return launch_map<TanhFwd, false>(x, nullptr, y, n, NoParams());
-    case TDH_ACT_RELU: return launch_map<ReluFwd, false>(x, nullptr, y, n, NoParams());
-    case TDH_ACT_SIGMOID: return launch_map<SigmoidFwd, false>(x, nullptr, y, n, NoParams());
-    case TDH_ACT_SOFTMAX:
+    case TDH_ACT_TANH: return launch_map<TanhFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_tanh");
+    case TDH_ACT_RELU: return launch_map<ReluFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_relu");
+    case TDH_ACT_SIGMOID: return launch_map<SigmoidFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_sigmoid");
+    case TDH_ACT_SOFTMAX: {
+      ProfScope prof("act_fwd_softmax", 8.0 * n, WORK_BYTE);
       hipLaunchKernelGGL(softmax_fwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
                          dim3(EW_THREADS), 0, ctx().stream, x, y, batch, len);
       TDH_LAUNCH_CHECK();
       return TDH_OK;
+    }
   }
   return set_error(TDH_ERR_INVALID, "activation kind %d is not supported", kind);
 }
@@ -351,14 +358,16 @@ int launch_act_fwd(int kind, int batch, int len, const float *x, float *y) {
 int launch_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx) {
   const size_t n = static_cast<size_t>(batch) * len;
   switch (kind) {
-    case TDH_ACT_TANH: return launch_map<TanhBwd, true>(y, dy, dx, n, NoParams());
-    case TDH_ACT_RELU: return launch_map<ReluBwd, true>(y, dy, dx, n, NoParams());
-    case TDH_ACT_SIGMOID: return launch_map<SigmoidBwd, true>(y, dy, dx, n, NoParams());
-    case TDH_ACT_SOFTMAX:
+    case TDH_ACT_TANH: return launch_map<TanhBwd, true>(y, dy, dx, n, NoParams(), "act_grad_tanh");
+    case TDH_ACT_RELU: return launch_map<ReluBwd, true>(y, dy, dx, n, NoParams(), "act_grad_relu");
+    case TDH_ACT_SIGMOID: return launch_map<SigmoidBwd, true>(y, dy, dx, n, NoParams(), "act_grad_sigmoid");
+    case TDH_ACT_SOFTMAX: {
+      ProfScope prof("act_grad_softmax", 12.0 * n, WORK_BYTE);
       hipLaunchKernelGGL(softmax_bwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
                          dim3(EW_THREADS), 0, ctx().stream, y, dy, dx, batch, len);
       TDH_LAUNCH_CHECK();
       return TDH_OK;
+    }
   }
   return set_error(TDH_ERR_INVALID, "activation kind %d is not supported", kind);
 }
@@ -369,15 +378,16 @@ int launch_loss_grad(int kind, int batch, int len, const float *y, const float *
     case TDH_LOSS_MSE: {
       MseGrad::Params p;
       p.factor = 2.0f / static_cast<float>(len);
-      return launch_map<MseGrad, true>(y, t, dy, n, p);
+      return launch_map<MseGrad, true>(y, t, dy, n, p, "loss_grad_mse");
     }
-    case TDH_LOSS_CE_MULTICLASS: return launch_map<CeMultiGrad, true>(y, t, dy, n, NoParams());
-    case TDH_LOSS_CE: return launch_map<CeGrad, true>(y, t, dy, n, NoParams());
+    case TDH_LOSS_CE_MULTICLASS: return launch_map<CeMultiGrad, true>(y, t, dy, n, NoParams(), "loss_grad_ce_multiclass");
+    case TDH_LOSS_CE: return launch_map<CeGrad, true>(y, t, dy, n, NoParams(), "loss_grad_ce");
   }
   return set_error(TDH_ERR_INVALID, "loss kind %d is not supported", kind);
 }
 
 int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz) {
+  ProfScope prof("softmax_xent_grad", 12.0 * batch * len, WORK_BYTE);
   hipLaunchKernelGGL(softmax_xent_grad_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
                      dim3(EW_THREADS), 0, ctx().stream, y, t, dz, batch, len);
   TDH_LAUNCH_CHECK();
@@ -440,6 +450,7 @@ int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, i
   rowsum_chunks(cols, chunks, chunk_len);
   void *ws = nullptr;
   TDH_TRY(ws_take(static_cast<size_t>(outer) * rows * chunks * sizeof(float), &ws));
+  ProfScope prof("bias_grad_rowsum", 4.0 * outer * rows * cols, WORK_BYTE);
   hipLaunchKernelGGL(rowsum_stage1_kernel, dim3(outer * rows, chunks), dim3(EW_THREADS), 0,
                      ctx().stream, src, rows, cols, chunks, chunk_len, static_cast<float *>(ws));
   TDH_LAUNCH_CHECK();
@@ -451,6 +462,7 @@ int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, i
 }
 
 int launch_colsum(const float *src, int rows, int cols, float *out, int accumulate) {
+  ProfScope prof("bias_grad_colsum", 4.0 * rows * cols, WORK_BYTE);
   hipLaunchKernelGGL(colsum_kernel, dim3(ceil_div(cols, EW_THREADS)), dim3(EW_THREADS), 0,
                      ctx().stream, src, rows, cols, out, accumulate);
   TDH_LAUNCH_CHECK();

@@ -326,7 +326,8 @@ inline size_t gemm_workspace_bytes(int M, int N, int K, bool allow_split) {
 template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
           class Epi>
 int launch_gemm_tile(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
-                     const GemmPlan &p, float *partial) {
+                     const GemmPlan &p, float *partial, const char *tag) {
+  ProfScope prof(tag, M, N, K);
   dim3 grid(ceil_div(N, BN), ceil_div(M, BM), p.splits);
   hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, AOp, BOp, Epi>), grid,
                      dim3(GEMM_THREADS), 0, ctx().stream, a, b, epi, M, N, K, p.k_per_split,
@@ -337,7 +338,7 @@ int launch_gemm_tile(const AOp &a, const BOp &b, const Epi &epi, int M, int N, i
 
 template <bool A_LANE_K, bool B_LANE_K, class AOp, class BOp, class Epi>
 int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
-                bool allow_split) {
+                bool allow_split, const char *tag, const char *reduce_tag) {
   if (M <= 0 || N <= 0) return TDH_OK;
   TDH_CHECK_ARG(static_cast<long>(M) * N < (1L << 31), "gemm: M*N=%ld too large",
                 static_cast<long>(M) * N);
@@ -350,17 +351,19 @@ int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
   }
   int rc;
   if (p.bm == 128 && p.bn == 128)
-    rc = launch_gemm_tile<128, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+    rc = launch_gemm_tile<128, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
   else if (p.bm == 128 && p.bn == 64)
-    rc = launch_gemm_tile<128, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+    rc = launch_gemm_tile<128, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
   else if (p.bm == 64 && p.bn == 128)
-    rc = launch_gemm_tile<64, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+    rc = launch_gemm_tile<64, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
   else if (p.bm == 64 && p.bn == 64)
-    rc = launch_gemm_tile<64, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+    rc = launch_gemm_tile<64, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
   else
-    rc = launch_gemm_tile<32, 128, 1, 4, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial);
+    rc = launch_gemm_tile<32, 128, 1, 4, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
   TDH_TRY(rc);
   if (p.splits > 1) {
+    // reads every partial tile once and writes the result once
+    ProfScope prof(reduce_tag, 4.0 * M * N * (p.splits + 1), WORK_BYTE);
     hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, 256)), dim3(256), 0,
                        ctx().stream, partial, p.splits, M, N, epi);
     TDH_LAUNCH_CHECK();

@@ -189,6 +189,7 @@ int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.OH * g.OW;
   if (total <= 0) return TDH_OK;
+  ProfScope prof("maxpool_fwd", 4.0 * batch * g.C * g.H * g.W + 8.0 * total, WORK_BYTE);
   hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
                      y, argmax, static_cast<int>(total), g);
   TDH_LAUNCH_CHECK();
@@ -200,6 +201,7 @@ int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.H * g.W;
   TDH_CHECK_ARG(g.OH > 0 && g.OW > 0, "maxpool backward: empty output");
+  ProfScope prof("maxpool_bwd", 8.0 * batch * g.C * g.OH * g.OW + 4.0 * total, WORK_BYTE);
   hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, dy,
                      argmax, dx, static_cast<int>(total), g);
   TDH_LAUNCH_CHECK();
@@ -222,6 +224,7 @@ int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *
   const long total = static_cast<long>(batch) * g.C * g.OH * g.OW;
   if (total <= 0) return TDH_OK;
   const float scale = 1.0f / static_cast<float>(d->pool_w * d->pool_h);
+  ProfScope prof("avepool_fwd", 4.0 * batch * g.C * g.H * g.W + 4.0 * total, WORK_BYTE);
   hipLaunchKernelGGL(avepool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
                      w, b, y, static_cast<int>(total), g, scale);
   TDH_LAUNCH_CHECK();
@@ -251,6 +254,7 @@ int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *
   const float scale = 1.0f / static_cast<float>(d->pool_w * d->pool_h);
   if (dx) {
     const long total = static_cast<long>(batch) * g.C * g.H * g.W;
+    ProfScope prof("avepool_bwd_dx", 4.0 * batch * g.C * g.OH * g.OW + 4.0 * total, WORK_BYTE);
     hipLaunchKernelGGL(avepool_bwd_dx_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream,
                        dy, w, dx, static_cast<int>(total), g, scale);
     TDH_LAUNCH_CHECK();
@@ -258,6 +262,7 @@ int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *
   if (dw || db) {
     void *ws = nullptr;
     TDH_TRY(ws_take(static_cast<size_t>(batch) * g.C * 2 * sizeof(float), &ws));
+    ProfScope prof("avepool_bwd_param", 4.0 * batch * g.C * (g.H * g.W + g.OH * g.OW), WORK_BYTE);
     hipLaunchKernelGGL(avepool_bwd_param_kernel, dim3(batch * g.C), dim3(PT), 0, ctx().stream, x,
                        dy, static_cast<float *>(ws), g);
     TDH_LAUNCH_CHECK();
