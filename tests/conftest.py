@@ -1,0 +1,84 @@
+import importlib
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X; run with -m gpu on the GPU box")
+
+
+# The parity bound of the path: max relative error 1e-4 for floating point, bit-exact for
+# indices. "Relative" is |got - want| / max(|want|, rms(want)): an element much smaller than
+# the tensor's typical magnitude (a sum that happens to cancel) is measured against that
+# magnitude, not against itself.
+REL_TOL = 1e-4
+
+
+def rel_err(got, want):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    if got.size == 0:
+        return 0.0
+    scale = np.maximum(np.abs(want), np.sqrt(np.mean(want * want)) + 1e-30)
+    return float(np.max(np.abs(got - want) / scale))
+
+
+def assert_close(got, want, tol=REL_TOL, what=""):
+    e = rel_err(got, want)
+    assert e <= tol, f"{what}: relative error {e:.3e} > {tol:g}"
+
+
+@pytest.fixture(scope="session")
+def O():
+    """The CPU oracle (test infrastructure)."""
+    from oracle import oracle
+    oracle.oracle_lib()
+    return oracle
+
+
+@pytest.fixture(scope="session")
+def W():
+    return importlib.import_module("tiny-cnn_amd.workloads")
+
+
+@pytest.fixture(scope="session")
+def T():
+    """The product binding, device initialised (GPU tests only)."""
+    mod = importlib.import_module("tiny-cnn_amd")
+    mod.init(0)
+    return mod
+
+
+@pytest.fixture(scope="session")
+def kats():
+    with open(os.path.join(GOLDEN, "reference_kats.json")) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="session")
+def layer_grads():
+    return np.load(os.path.join(GOLDEN, "layer_grads.npz"))
+
+
+@pytest.fixture(scope="session")
+def net_steps():
+    return np.load(os.path.join(GOLDEN, "net_steps.npz"))
+
+
+def load_net_params(net_like, params, setter):
+    for (i, which, a) in params:
+        setter(net_like, i, which, a)
+
+
+def input_checksum(x, t, params):
+    return float(sum(np.asarray(a, np.float64).sum() for a in [x, t] + [p for _, _, p in params]))

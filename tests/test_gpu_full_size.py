@@ -1,0 +1,151 @@
+"""BASELINE.json's configurations at their full sizes on the MI355X, checked through
+size-independent properties and float64 spot checks (the scalar oracle would need minutes
+at these sizes): exact float64 dot products for sampled gradient entries, db against a host
+sum, linearity of the backward pass in dY, and whole fully-connected gradients against
+numpy's float64 matmul."""
+import numpy as np
+import pytest
+
+from conftest import assert_close, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config2_conv_backward_full_size(T, W):
+    """configs[1]: batch 64, 32x64x64 -> 64 channels, 3x3, pad same, stride 1."""
+    (hw, _, c, k, oc), x, w, dy = W.conv_bwd_case()
+    bs = x.shape[0]
+    d = T.conv_desc(hw, hw, c, k, k, oc, pad_same=True)
+    xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+    dx, dw, db = T.DevBuf(x.shape), T.DevBuf(w.shape), T.DevBuf((oc,))
+    T.conv2d_bwd(d, bs, xd, wd, dyd, dx, dw, db)
+    dxh, dwh, dbh = dx.numpy(), dw.numpy().reshape(oc, c, k, k), db.numpy()
+    x4 = x.reshape(bs, c, hw, hw)
+    dy4 = dy.reshape(bs, oc, hw, hw)
+    w4 = w.reshape(oc, c, k, k)
+    # db: exact sum on the host
+    assert_close(dbh, dy4.astype(np.float64).sum(axis=(0, 2, 3)), what="db")
+    # dW: float64 dot products over the whole batch for sampled taps
+    rng = np.random.default_rng(0)
+    xp = np.zeros((bs, c, hw + 2, hw + 2), np.float64)
+    xp[:, :, 1:-1, 1:-1] = x4
+    dw_scale = np.sqrt(np.mean(dwh.astype(np.float64) ** 2))
+    for _ in range(40):
+        o, i, ky, kx = rng.integers(oc), rng.integers(c), rng.integers(k), rng.integers(k)
+        want = np.sum(xp[:, i, ky:ky + hw, kx:kx + hw] * dy4[:, o])
+        assert abs(dwh[o, i, ky, kx] - want) <= 1e-4 * max(abs(want), dw_scale), (o, i, ky, kx)
+    # dX: float64 correlation with the flipped filter at sampled positions
+    dyp = np.zeros((oc, hw + 2, hw + 2), np.float64)
+    dx4 = dxh.reshape(bs, c, hw, hw)
+    dx_scale = np.sqrt(np.mean(dx4.astype(np.float64) ** 2))
+    for _ in range(8):
+        n = rng.integers(bs)
+        dyp[:, 1:-1, 1:-1] = dy4[n]
+        for _ in range(6):
+            i, yy, xx = rng.integers(c), rng.integers(hw), rng.integers(hw)
+            # dX[i,yy,xx] = sum_{o,ky,kx} W[o,i,ky,kx] * dY[o, yy+1-ky, xx+1-kx]
+            win = dyp[:, yy:yy + 3, xx:xx + 3][:, ::-1, ::-1]
+            want = np.sum(w4[:, i].astype(np.float64) * win)
+            assert abs(dx4[n, i, yy, xx] - want) <= 1e-4 * max(abs(want), dx_scale)
+    # linearity in dY: backward(2*dy) == 2*backward(dy), bit for bit (scaling by 2 is exact)
+    dx2, dw2, db2 = T.DevBuf(x.shape), T.DevBuf(w.shape), T.DevBuf((oc,))
+    T.conv2d_bwd(d, bs, xd, wd, T.to_device(dy * 2), dx2, dw2, db2)
+    assert np.array_equal(dx2.numpy(), 2 * dxh)
+    assert np.array_equal(dw2.numpy().reshape(dwh.shape), 2 * dwh)
+    assert np.array_equal(db2.numpy(), 2 * dbh)
+
+
+def test_config3_fc_backward_adam_full_size(T, O, W):
+    """configs[2]: batch 256, 4096 -> 4096, tanh, Adam on W and b."""
+    x, w, b, dy = W.fc_bwd_case()
+    bs, n = x.shape[0], 4096
+    xd, wd, bd = T.to_device(x), T.to_device(w), T.to_device(b)
+    z, y = T.DevBuf((bs, n)), T.DevBuf((bs, n))
+    T.fc_fwd(n, n, True, bs, xd, wd, bd, z)
+    T.act_fwd("tanh", bs, n, z, y)
+    W64 = w.reshape(n, n).astype(np.float64)
+    z_ref = x.astype(np.float64) @ W64 + b
+    assert_close(z.numpy(), z_ref, what="forward")
+    y_ref = np.tanh(z_ref)
+    assert_close(y.numpy(), y_ref, 1e-5, what="tanh")
+    dz, dx, dw, db = T.DevBuf((bs, n)), T.DevBuf((bs, n)), T.DevBuf((n * n,)), T.DevBuf((n,))
+    T.act_bwd("tanh", bs, n, y, T.to_device(dy), dz)
+    yh = y.numpy().astype(np.float64)
+    dz_ref = dy * (1 - yh * yh)
+    assert_close(dz.numpy(), dz_ref, 1e-5, what="tanh gradient")
+    T.fc_bwd(n, n, True, bs, xd, wd, dz, dx, dw, db)
+    dzh = dz.numpy().astype(np.float64)
+    assert_close(dx.numpy(), dzh @ W64.T, what="dx")
+    dw_ref = x.astype(np.float64).T @ dzh
+    assert_close(dw.numpy().reshape(n, n), dw_ref, what="dw (summed over the batch)")
+    assert_close(db.numpy(), dzh.sum(0), what="db")
+    # Adam on W then on b with one optimizer object: b sees the advanced powers
+    opt, ropt = T.opt_desc("adam"), O.opt_desc("adam")
+    s = [T.DevBuf((n * n,), zero=True), T.DevBuf((n * n,), zero=True), T.DevBuf((n,), zero=True),
+         T.DevBuf((n,), zero=True)]
+    dwh, dbh = dw.numpy(), db.numpy()
+    T.opt_update(opt, n * n, dw, wd, s[0], s[1])
+    T.opt_update(opt, n, db, bd, s[2], s[3])
+    rw, rb = w.copy(), b.copy()
+    O.opt_update(ropt, dwh, rw, np.zeros_like(rw), np.zeros_like(rw))
+    O.opt_update(ropt, dbh, rb, np.zeros_like(rb), np.zeros_like(rb))
+    assert_close(wd.numpy(), rw, 1e-6, what="W after Adam")
+    assert_close(bd.numpy(), rb, 1e-6, what="b after Adam")
+    assert opt.b1_t == ropt.b1_t
+
+
+def test_config4_full_batch_step_properties(T, W):
+    """configs[3] at batch 128: a step changes every parameter, stays finite, and the loss
+    gradient rows sum to zero (softmax + cross-entropy)."""
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch("cifar10_cnn_b128")
+    net = T.Net(W.build_layers(T, spec), batch, 1)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+    xd, td = T.to_device(x), T.to_device(t)
+    net.train_step(None, loss, batch, xd, td, do_update=False)
+    n = len(spec)
+    dz = net.layer_dx(n - 1, batch)           # gradient w.r.t. the logits
+    y = net.layer_out(n - 1, batch)
+    assert_close(dz, y.astype(np.float64) - t, 1e-5, what="dz = y - t")
+    assert np.all(np.abs(dz.sum(1)) < 1e-5)
+    # bias gradient of the last fc layer is the column sum of dz
+    assert_close(net.layer_grad(n - 2, 1), dz.astype(np.float64).sum(0), what="db of fc2")
+    # weight gradient of the last fc layer is relu_out^T dz
+    a = net.layer_out(n - 3, batch).astype(np.float64)
+    assert_close(net.layer_grad(n - 2, 0), (a.T @ dz).ravel(), what="dW of fc2")
+    opt = T.opt_desc(opt_kind, **opt_kw)
+    net.train_step(opt, loss, batch, xd, td)
+    for (i, which, a0) in params:
+        got = net.get_param(i, which)
+        assert np.all(np.isfinite(got))
+        assert not np.array_equal(got, a0)
+    net.close()
+
+
+def test_config5_vgg_full_size_one_step(T, W):
+    """configs[4] at its full size (batch 64, 3x128x128): one momentum step; spot-check the
+    big fully-connected gradient (131072 x 256) against float64 and the first conv's bias
+    gradient against a host sum."""
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch("vgg_stack_b64")
+    net = T.Net(W.build_layers(T, spec), batch, 1)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+    xd, td = T.to_device(x), T.to_device(t)
+    net.train_step(None, loss, batch, xd, td, do_update=False)
+    n = len(spec)
+    fc1 = n - 4
+    a = net.layer_out(fc1 - 1, batch).astype(np.float64)      # pooled features [64][131072]
+    dz1 = net.layer_dx(fc1 + 1, batch).astype(np.float64)     # grad w.r.t. fc1 output
+    dw = net.layer_grad(fc1, 0).reshape(-1, 256)
+    rng = np.random.default_rng(1)
+    rows = rng.integers(0, dw.shape[0], 64)
+    want = a[:, rows].T @ dz1
+    scale = np.sqrt(np.mean(dw.astype(np.float64) ** 2))
+    assert np.max(np.abs(dw[rows] - want) / np.maximum(np.abs(want), scale)) <= 1e-4
+    assert_close(net.layer_grad(fc1, 1), dz1.sum(0), what="db of fc1")
+    # first conv: db = sum of its output gradient over batch and pixels
+    g0 = net.layer_dx(1, batch).astype(np.float64).reshape(batch, 64, -1)
+    assert_close(net.layer_grad(0, 1), g0.sum(axis=(0, 2)), what="db of conv1")
+    for (i, which, a0) in params:
+        assert np.all(np.isfinite(net.layer_grad(i, which)))
+    net.close()

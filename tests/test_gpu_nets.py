@@ -1,0 +1,121 @@
+"""Whole train steps (fprop, loss gradient, bprop, update) on the MI355X against the oracle
+and against the parameters tiny-dnn's own network<sequential>::fit produced
+(tests/golden/net_steps.npz). All through the C ABI (tdh_net_*)."""
+import numpy as np
+import pytest
+
+from conftest import assert_close, input_checksum
+
+pytestmark = pytest.mark.gpu
+
+
+def make_pair(T, O, W, name, batch, flags, size=None):
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch, size=size)
+    net = T.Net(W.build_layers(T, spec), batch, flags)
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+        (ref.weight(i) if which == 0 else ref.bias(i))[:] = a
+    return spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref
+
+
+CASES = [("lenet5_b16", 16, None), ("cifar10_cnn_b128", 8, None), ("vgg_stack_b64", 2, 16)]
+
+
+@pytest.mark.parametrize("name,batch,size", CASES)
+@pytest.mark.parametrize("flags", [0, 1])
+def test_gradients_of_every_layer_match_oracle(T, O, W, name, batch, size, flags):
+    spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref = make_pair(T, O, W, name, batch, flags, size)
+    xd, td = T.to_device(x), T.to_device(t)
+    net.train_step(None, loss, batch, xd, td, do_update=False)
+    ref.train_step(O.opt_desc(opt_kind), loss, x, t, do_update=False)
+    for i, l in enumerate(spec):
+        assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{name} layer {i} output")
+        if l[0] == "maxpool":
+            assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64),
+                                  ref.layer_argmax(i, batch)), f"{name} layer {i} argmax"
+        if net.param_size(i, 0):
+            assert_close(net.layer_grad(i, 0), ref.layer_dw(i), what=f"{name} layer {i} dW")
+            assert_close(net.layer_grad(i, 1), ref.layer_db(i), what=f"{name} layer {i} db")
+    assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), what=f"{name} input gradient")
+    net.close()
+
+
+@pytest.mark.parametrize("name,batch,size,steps", [("lenet5_b16", 16, None, 3), ("cifar10_cnn_b128", 8, None, 3),
+                                                   ("vgg_stack_b64", 2, 16, 1)])
+@pytest.mark.parametrize("flags", [0, 1])
+def test_updated_weights_match_oracle(T, O, W, name, batch, size, steps, flags):
+    spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref = make_pair(T, O, W, name, batch, flags, size)
+    opt, ropt = T.opt_desc(opt_kind, **opt_kw), O.opt_desc(opt_kind, **opt_kw)
+    xd, td = T.to_device(x), T.to_device(t)
+    for _ in range(steps):
+        net.train_step(opt, loss, batch, xd, td)
+        ref.train_step(ropt, loss, x, t)
+    for (i, which, a) in params:
+        want = ref.weight(i) if which == 0 else ref.bias(i)
+        assert_close(net.get_param(i, which), want, what=f"{name} updated parameter {i}.{which}")
+    assert opt.b1_t == ropt.b1_t and opt.b2_t == ropt.b2_t
+    # gradients are cleared after the update (layer.h:680)
+    for (i, which, a) in params:
+        assert not net.layer_grad(i, which).any()
+    net.close()
+
+
+@pytest.mark.parametrize("name", ["lenet5_b16", "cifar10_cnn_b128"])
+def test_updated_weights_match_reference_fit(T, W, net_steps, name):
+    """Against what tiny-dnn's network<sequential>::fit itself produced."""
+    g = net_steps
+    batch, steps, stride = int(g[f"{name}.batch"]), int(g[f"{name}.steps"]), int(g[f"{name}.stride"])
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch)
+    assert input_checksum(x, t, params) == float(g[f"{name}.input_checksum"])
+    net = T.Net(W.build_layers(T, spec), batch, 1)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+    opt = T.opt_desc(opt_kind, **opt_kw)
+    xd, td = T.to_device(x), T.to_device(t)
+    for _ in range(steps):
+        net.train_step(opt, loss, batch, xd, td)
+    for (i, which, a) in params:
+        got = net.get_param(i, which)
+        assert_close(got[::stride], g[f"{name}.p{i}.{which}"], what=f"{name} parameter {i}.{which}")
+    net.close()
+
+
+def test_step_is_reproducible_bit_for_bit(T, W):
+    """Fixed-order reductions: the same inputs give the same bits, run after run."""
+    outs = []
+    for _ in range(3):
+        spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch("cifar10_cnn_b128", batch=32)
+        net = T.Net(W.build_layers(T, spec), batch, 1)
+        for (i, which, a) in params:
+            net.set_param(i, which, a)
+        opt = T.opt_desc(opt_kind, **opt_kw)
+        xd, td = T.to_device(x), T.to_device(t)
+        for _ in range(2):
+            net.train_step(opt, loss, batch, xd, td)
+        outs.append([net.get_param(i, which) for (i, which, a) in params])
+        net.close()
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert np.array_equal(a, b)
+
+
+def test_smaller_batch_than_max_and_forward_only(T, O, W):
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch("cifar10_cnn_b128", batch=5)
+    net = T.Net(W.build_layers(T, spec), 16, 0)            # max_batch 16, run 5
+    ref = O.OracleNet(W.build_layers(O, spec), 5)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+        (ref.weight(i) if which == 0 else ref.bias(i))[:] = a
+    net.forward(5, T.to_device(x))
+    assert_close(net.layer_out(len(spec) - 1, 5), ref.forward(x))
+    with pytest.raises(T.TdhError):
+        net.forward(17, T.to_device(np.zeros((17, x.shape[1]), np.float32)))
+    net.close()
+
+
+def test_net_rejects_inconsistent_layers(T):
+    with pytest.raises(T.TdhError, match="expects"):
+        T.Net([T.L_fc(10, 5), T.L_fc(6, 2)], 4)
+    with pytest.raises(T.TdhError, match="first layer"):
+        T.Net([T.L_act("relu"), T.L_fc(6, 2)], 4)

@@ -1,0 +1,367 @@
+"""Parity of every operator of the hot path, called through the C ABI on the MI355X, with
+the CPU oracle on identical seeded inputs, and with the outputs tiny-dnn itself produced
+(tests/golden/layer_grads.npz). Floating point: max relative error 1e-4 (conftest.rel_err);
+max-pool argmax indices and routed gradients: bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from conftest import assert_close, REL_TOL
+
+pytestmark = pytest.mark.gpu
+
+
+def run_conv(T, d, x, w, b, dy, accumulate=False, dw0=None):
+    bs = x.shape[0]
+    ow, oh = T.conv_out_shape(d)
+    xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+    bd = T.to_device(b) if b is not None else None
+    y = T.DevBuf((bs, d.out_c * oh * ow))
+    dx = T.DevBuf(x.shape)
+    dw = T.to_device(dw0) if dw0 is not None else T.DevBuf(w.shape)
+    db = T.DevBuf((d.out_c,), zero=True)
+    T.conv2d_fwd(d, bs, xd, wd, bd, y)
+    T.conv2d_bwd(d, bs, xd, wd, dyd, dx, dw, db if d.has_bias else None, accumulate)
+    return y.numpy(), dx.numpy(), dw.numpy(), db.numpy()
+
+
+CONV = [
+    # in_w, in_h, in_c, k, out_c, same, stride, batch
+    (5, 5, 1, 3, 1, False, 2, 1), (12, 10, 3, 3, 4, True, 1, 3), (9, 9, 2, 5, 3, True, 2, 2),
+    (32, 32, 1, 5, 6, False, 1, 16), (14, 14, 6, 5, 16, False, 1, 16), (5, 5, 16, 5, 120, False, 1, 16),
+    (32, 32, 3, 5, 32, True, 1, 8), (16, 16, 32, 5, 32, True, 1, 8), (8, 8, 32, 5, 64, True, 1, 8),
+    (24, 24, 32, 3, 64, True, 1, 4), (17, 13, 5, 3, 7, True, 1, 3), (11, 11, 4, 3, 6, False, 3, 2),
+    (33, 31, 3, 3, 130, True, 1, 2), (16, 16, 64, 3, 128, True, 1, 2), (7, 7, 3, 7, 5, False, 1, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV)
+def test_conv_fwd_bwd_matches_oracle(T, O, cfg):
+    iw, ih, ic, k, oc, same, st, bs = cfg
+    rng = np.random.default_rng(abs(hash(cfg)) % 2**31)
+    d = T.conv_desc(iw, ih, ic, k, k, oc, pad_same=same, w_stride=st, h_stride=st)
+    do = O.conv_desc(iw, ih, ic, k, k, oc, pad_same=same, w_stride=st, h_stride=st)
+    ow, oh = T.conv_out_shape(d)
+    assert (ow, oh) == O.conv_out_shape(do)
+    x = rng.standard_normal((bs, ic * ih * iw)).astype(np.float32)
+    w = rng.uniform(-0.3, 0.3, oc * ic * k * k).astype(np.float32)
+    b = rng.standard_normal(oc).astype(np.float32)
+    dy = rng.standard_normal((bs, oc * oh * ow)).astype(np.float32)
+    y, dx, dw, db = run_conv(T, d, x, w, b, dy)
+    assert_close(y, O.conv2d_fwd(do, x, w, b), what="y")
+    rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
+    assert_close(dx, rdx, what="dx")
+    assert_close(dw, rdw, what="dw")
+    assert_close(db, rdb, what="db")
+
+
+def test_conv_reference_kat_with_stride(T, kats):
+    k = kats["conv_with_stride"]
+    d = T.conv_desc(5, 5, 1, 3, 3, 1, w_stride=2, h_stride=2)
+    y, dx, dw, db = run_conv(T, d, np.array([k["x"]], np.float32), np.array(k["w"], np.float32),
+                             np.array(k["b"], np.float32), np.array([k["dy"]], np.float32))
+    assert np.array_equal(y[0], np.array(k["y"], np.float32))
+    assert np.array_equal(dx[0], np.array(k["dx"], np.float32))
+    assert np.array_equal(dw, np.array(k["dw"], np.float32))
+    assert np.array_equal(db, np.array(k["db"], np.float32))
+
+
+def test_conv_reference_kats_forward(T, kats):
+    k = kats["conv_fprop"]
+    d = T.conv_desc(5, 5, 1, 3, 3, 2, has_bias=False)
+    y = T.DevBuf((1, 18))
+    T.conv2d_fwd(d, 1, T.to_device(np.array([k["x"]], np.float32)),
+                 T.to_device(np.array(k["w"], np.float32)), None, y)
+    np.testing.assert_allclose(y.numpy()[0, :9], k["y_first9"], atol=k["tol"])
+    k = kats["conv_with_dilation"]
+    d = T.conv_desc(7, 7, 1, 3, 3, 1, has_bias=False, w_dilation=2, h_dilation=2)
+    y = T.DevBuf((1, 9))
+    T.conv2d_fwd(d, 1, T.to_device(np.arange(49, dtype=np.float32)[None]),
+                 T.to_device(np.array(k["w"], np.float32)), None, y)
+    np.testing.assert_allclose(y.numpy()[0], k["y"], atol=1e-3)
+
+
+@pytest.mark.parametrize("name", ["conv5x5_same", "conv3x3_same", "conv5x5_valid", "conv3x3_stride2"])
+def test_conv_matches_reference_outputs(T, layer_grads, name):
+    g = layer_grads
+    iw, ih, ic, k, oc, same, stride, batch = [int(v) for v in g[f"{name}.cfg"]]
+    d = T.conv_desc(iw, ih, ic, k, k, oc, pad_same=bool(same), w_stride=stride, h_stride=stride)
+    y, dx, dw, db = run_conv(T, d, g[f"{name}.x"], g[f"{name}.w"], g[f"{name}.b"], g[f"{name}.dy"])
+    assert_close(y, g[f"{name}.y"], what="y")
+    for eng in ("internal", "avx"):
+        assert_close(dx, g[f"{name}.{eng}.dx"], what=f"dx vs {eng}")
+        assert_close(dw, g[f"{name}.{eng}.dw"], what=f"dw vs {eng}")
+        assert_close(db, g[f"{name}.{eng}.db"], what=f"db vs {eng}")
+
+
+def test_conv_connection_table(T, O):
+    rng = np.random.default_rng(21)
+    tbl = rng.integers(0, 2, (6, 16)).astype(np.uint8)
+    d, do = T.conv_desc(14, 14, 6, 5, 5, 16, tbl=tbl), O.conv_desc(14, 14, 6, 5, 5, 16, tbl=tbl)
+    x = rng.standard_normal((4, 6 * 196)).astype(np.float32)
+    w = rng.uniform(-0.3, 0.3, 16 * 6 * 25).astype(np.float32)
+    b = rng.standard_normal(16).astype(np.float32)
+    dy = rng.standard_normal((4, 1600)).astype(np.float32)
+    y, dx, dw, db = run_conv(T, d, x, w, b, dy)
+    assert_close(y, O.conv2d_fwd(do, x, w, b))
+    rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
+    assert_close(dx, rdx); assert_close(dw, rdw); assert_close(db, rdb)
+    # unconnected pairs get exactly zero gradient
+    mask = np.repeat(tbl.T.reshape(16, 6, 1), 25, axis=2).ravel()
+    assert np.all(dw[mask == 0] == 0.0)
+
+
+def test_conv_accumulate_and_skipped_outputs(T, O):
+    """dW/db are added to when accumulate=1 (the reference's += between clear_grads calls);
+    NULL outputs are skipped; dX is always overwritten."""
+    rng = np.random.default_rng(22)
+    d, do = T.conv_desc(10, 10, 3, 3, 3, 5, pad_same=True), O.conv_desc(10, 10, 3, 3, 3, 5, pad_same=True)
+    x = rng.standard_normal((3, 300)).astype(np.float32)
+    w = rng.standard_normal(135).astype(np.float32)
+    dy = rng.standard_normal((3, 500)).astype(np.float32)
+    dw0 = rng.standard_normal(135).astype(np.float32)
+    _, dx, dw, db = run_conv(T, d, x, w, np.zeros(5, np.float32), dy, accumulate=True, dw0=dw0)
+    rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
+    assert_close(dw, rdw + dw0); assert_close(dx, rdx); assert_close(db, rdb)
+    xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+    dxb = T.to_device(np.full((3, 300), 7.0, np.float32))
+    T.conv2d_bwd(d, 3, xd, wd, dyd, dxb, None, None)
+    assert_close(dxb.numpy(), rdx)
+    dwb = T.DevBuf((135,))
+    T.conv2d_bwd(d, 3, xd, wd, dyd, None, dwb, None)
+    assert_close(dwb.numpy(), rdw)
+
+
+def test_conv_errors_and_empty_batch(T):
+    d = T.conv_desc(8, 8, 2, 3, 3, 4, w_dilation=2, h_dilation=2)
+    buf = T.DevBuf((16,))
+    with pytest.raises(T.TdhError, match="dilation"):
+        T.conv2d_bwd(d, 1, buf, buf, buf, buf, buf, buf)
+    bad = T.conv_desc(2, 2, 1, 3, 3, 1)
+    with pytest.raises(T.TdhError, match="window larger"):
+        T.conv2d_fwd(bad, 1, buf, buf, buf, buf)
+    ok = T.conv_desc(8, 8, 2, 3, 3, 4)
+    T.conv2d_fwd(ok, 0, None, None, None, None)          # empty batch: nothing to do
+    with pytest.raises(T.TdhError, match="null"):
+        T.conv2d_fwd(ok, 1, None, buf, buf, buf)
+
+
+FC = [(1, 4, 2, True), (5, 37, 19, True), (16, 120, 10, True), (128, 1024, 64, True),
+      (64, 300, 257, False), (256, 512, 384, True), (3, 2048, 40, True), (130, 70, 1000, True)]
+
+
+@pytest.mark.parametrize("cfg", FC)
+def test_fc_fwd_bwd_matches_oracle(T, O, cfg):
+    bs, ni, no, bias = cfg
+    rng = np.random.default_rng(abs(hash(cfg)) % 2**31)
+    x = rng.uniform(-1, 1, (bs, ni)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, ni * no).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, no).astype(np.float32)
+    dy = rng.standard_normal((bs, no)).astype(np.float32)
+    xd, wd, bd, dyd = T.to_device(x), T.to_device(w), T.to_device(b), T.to_device(dy)
+    y, dx, dw, db = T.DevBuf((bs, no)), T.DevBuf((bs, ni)), T.DevBuf((ni * no,)), T.DevBuf((no,))
+    T.fc_fwd(ni, no, bias, bs, xd, wd, bd if bias else None, y)
+    assert_close(y.numpy(), O.fc_fwd(x, w, b if bias else None), what="y")
+    T.fc_bwd(ni, no, bias, bs, xd, wd, dyd, dx, dw, db if bias else None)
+    rdx, rdw, rdb = O.fc_bwd(x, w, dy, bias)
+    assert_close(dx.numpy(), rdx, what="dx")
+    assert_close(dw.numpy(), rdw, what="dw")
+    if bias:
+        assert_close(db.numpy(), rdb, what="db")
+
+
+def test_fc_reference_kats_and_outputs(T, kats, layer_grads):
+    k = kats["fc_forward"]
+    y = T.DevBuf((1, 2))
+    T.fc_fwd(4, 2, True, 1, T.to_device(np.array([k["x"]], np.float32)),
+             T.to_device(np.full(8, 1.0, np.float32)), T.to_device(np.full(2, 0.5, np.float32)), y)
+    assert np.array_equal(y.numpy()[0], np.array(k["y"], np.float32))
+    T.fc_fwd(4, 2, False, 1, T.to_device(np.array([k["x"]], np.float32)),
+             T.to_device(np.full(8, 1.0, np.float32)), None, y)
+    assert np.array_equal(y.numpy()[0], np.array(kats["fc_forward_nobias"]["y"], np.float32))
+    g = layer_grads
+    xd, wd, dyd = T.to_device(g["fc.x"]), T.to_device(g["fc.w"]), T.to_device(g["fc.dy"])
+    dx, dw, db = T.DevBuf((6, 37)), T.DevBuf((37 * 19,)), T.DevBuf((19,))
+    T.fc_bwd(37, 19, True, 6, xd, wd, dyd, dx, dw, db)
+    for eng in ("internal", "avx"):
+        assert_close(dx.numpy(), g[f"fc.{eng}.dx"]); assert_close(dw.numpy(), g[f"fc.{eng}.dw"])
+        assert_close(db.numpy(), g[f"fc.{eng}.db"])
+
+
+POOL = [(4, 4, 1, 2, 2, 2, 2, 0, 0), (7, 7, 2, 2, 2, 2, 2, 0, 1), (4, 4, 1, 2, 2, 1, 1, 1, 0),
+        (9, 8, 3, 3, 3, 2, 2, 0, 0), (6, 6, 2, 2, 2, 3, 3, 0, 0), (32, 32, 32, 2, 2, 2, 2, 0, 0),
+        (4, 4, 1, 2, 1, 2, 1, 0, 0), (4, 4, 1, 1, 2, 1, 2, 0, 0), (13, 9, 5, 3, 2, 2, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("cfg", POOL)
+def test_maxpool_bit_exact(T, O, cfg):
+    iw, ih, c = cfg[:3]
+    rng = np.random.default_rng(abs(hash(cfg)) % 2**31)
+    d, do = T.pool_desc(*cfg), O.pool_desc(*cfg)
+    ow, oh = T.pool_out_shape(d)
+    assert (ow, oh) == O.pool_out_shape(do)
+    bs = 5
+    x = rng.integers(-3, 4, (bs, c * ih * iw)).astype(np.float32)     # many ties
+    dy = rng.standard_normal((bs, c * oh * ow)).astype(np.float32)
+    y, am, dx = T.DevBuf((bs, c * oh * ow)), T.DevBuf((bs, c * oh * ow), np.int32), T.DevBuf(x.shape)
+    T.maxpool_fwd(d, bs, T.to_device(x), y, am)
+    T.maxpool_bwd(d, bs, T.to_device(dy), am, dx)
+    ry, ram = O.maxpool_fwd(do, x)
+    assert np.array_equal(y.numpy(), ry)
+    assert np.array_equal(am.numpy().astype(np.int64), ram), "argmax indices must be bit-exact"
+    assert np.array_equal(dx.numpy(), O.maxpool_bwd(do, dy, ram))
+
+
+def test_maxpool_nan_and_reference_outputs(T, O, kats, layer_grads):
+    d, do = T.pool_desc(4, 2, 1, 2), O.pool_desc(4, 2, 1, 2)
+    x = np.array([[5, 5, np.nan, 1, 5, 9, np.nan, np.nan],
+                  [7, 7, np.nan, np.nan, 7, 7, np.nan, np.nan]], np.float32)
+    y, am = T.DevBuf((2, 2)), T.DevBuf((2, 2), np.int32)
+    T.maxpool_fwd(d, 2, T.to_device(x), y, am)
+    ry, ram = O.maxpool_fwd(do, x)
+    assert np.array_equal(am.numpy().astype(np.int64), ram) and np.array_equal(y.numpy(), ry)
+    k = kats["maxpool_backward"]
+    d = T.pool_desc(4, 4, 1, 2)
+    y, am, dx = T.DevBuf((1, 4)), T.DevBuf((1, 4), np.int32), T.DevBuf((1, 16))
+    T.maxpool_fwd(d, 1, T.to_device(np.array([kats["pool_input_4x4"]], np.float32)), y, am)
+    T.maxpool_bwd(d, 1, T.to_device(np.array([k["dy"]], np.float32)), am, dx)
+    assert np.array_equal(dx.numpy()[0], np.array(k["dx"], np.float32))
+    g = layer_grads
+    for name in ("maxpool2x2", "maxpool3x3s2", "maxpool_same_s1", "maxpool_ceil", "maxpool_gap"):
+        cfg = [int(v) for v in g[f"{name}.cfg"]]
+        d = T.pool_desc(*cfg)
+        x, dy = g[f"{name}.x"], g[f"{name}.dy"]
+        y, am, dx = T.DevBuf(g[f"{name}.y"].shape), T.DevBuf(g[f"{name}.y"].shape, np.int32), T.DevBuf(x.shape)
+        T.maxpool_fwd(d, x.shape[0], T.to_device(x), y, am)
+        T.maxpool_bwd(d, x.shape[0], T.to_device(dy), am, dx)
+        assert np.array_equal(y.numpy(), g[f"{name}.y"]), name
+        assert np.array_equal(dx.numpy(), g[f"{name}.dx"]), name
+
+
+@pytest.mark.parametrize("cfg", [(4, 4, 1, 2, 2), (4, 4, 2, 2, 1), (28, 28, 6, 2, 2), (6, 6, 3, 3, 3),
+                                 (10, 10, 16, 2, 2), (64, 64, 8, 2, 2)])
+def test_avepool_matches_oracle(T, O, cfg):
+    iw, ih, c, p, s = cfg
+    rng = np.random.default_rng(abs(hash(cfg)) % 2**31)
+    d, do = T.pool_desc(iw, ih, c, p, p, s, s), O.pool_desc(iw, ih, c, p, p, s, s)
+    ow, oh = T.pool_out_shape(d)
+    bs = 5
+    x = rng.standard_normal((bs, c * ih * iw)).astype(np.float32)
+    w = rng.standard_normal(c).astype(np.float32)
+    b = rng.standard_normal(c).astype(np.float32)
+    dy = rng.standard_normal((bs, c * oh * ow)).astype(np.float32)
+    xd, wd = T.to_device(x), T.to_device(w)
+    y, dx, dw, db = T.DevBuf(dy.shape), T.DevBuf(x.shape), T.DevBuf((c,)), T.DevBuf((c,))
+    T.avepool_fwd(d, bs, xd, wd, T.to_device(b), y)
+    assert_close(y.numpy(), O.avepool_fwd(do, x, w, b), what="y")
+    T.avepool_bwd(d, bs, xd, wd, T.to_device(dy), dx, dw, db)
+    rdx, rdw, rdb = O.avepool_bwd(do, x, w, dy)
+    assert_close(dx.numpy(), rdx, what="dx"); assert_close(dw.numpy(), rdw, what="dw")
+    assert_close(db.numpy(), rdb, what="db")
+
+
+def test_avepool_reference_outputs_and_errors(T, kats, layer_grads):
+    g = layer_grads
+    for name in ("avepool2", "avepool2s1", "avepool3"):
+        iw, ih, c, p, s = [int(v) for v in g[f"{name}.cfg"]]
+        d = T.pool_desc(iw, ih, c, p, p, s, s)
+        x, dy = g[f"{name}.x"], g[f"{name}.dy"]
+        xd, wd = T.to_device(x), T.to_device(g[f"{name}.w"])
+        y, dx, dw, db = T.DevBuf(dy.shape), T.DevBuf(x.shape), T.DevBuf((c,)), T.DevBuf((c,))
+        T.avepool_fwd(d, 3, xd, wd, T.to_device(g[f"{name}.b"]), y)
+        T.avepool_bwd(d, 3, xd, wd, T.to_device(dy), dx, dw, db)
+        assert_close(y.numpy(), g[f"{name}.y"]); assert_close(dx.numpy(), g[f"{name}.dx"])
+        assert_close(dw.numpy(), g[f"{name}.dw"]); assert_close(db.numpy(), g[f"{name}.db"])
+    x = np.array([kats["pool_input_4x4"]], np.float32)
+    for k in kats["avepool_forward"]:
+        d = T.pool_desc(4, 4, 1, k["pool"], k["pool"], k["stride"], k["stride"])
+        y = T.DevBuf((1, len(k["y"])))
+        T.avepool_fwd(d, 1, T.to_device(x), T.to_device(np.ones(1, np.float32)),
+                      T.to_device(np.zeros(1, np.float32)), y)
+        np.testing.assert_allclose(y.numpy()[0], k["y"], rtol=1.2e-5)
+    buf = T.DevBuf((64,))
+    with pytest.raises(T.TdhError, match="multiple of the window"):   # reference ctor throws too
+        T.avepool_fwd(T.pool_desc(5, 5, 1, 2), 1, buf, buf, buf, buf)
+
+
+@pytest.mark.parametrize("kind", ["tanh", "relu", "sigmoid", "softmax"])
+@pytest.mark.parametrize("shape", [(4, 10), (3, 1000), (7, 77), (1, 1), (64, 4099)])
+def test_activations_match_oracle(T, O, kind, shape):
+    rng = np.random.default_rng(shape[1])
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    y, dx = T.DevBuf(shape), T.DevBuf(shape)
+    T.act_fwd(kind, shape[0], shape[1], T.to_device(x), y)
+    ry = O.act_fwd(kind, x)
+    assert_close(y.numpy(), ry, 1e-5, "forward")
+    T.act_bwd(kind, shape[0], shape[1], T.to_device(ry), T.to_device(dy), dx)
+    assert_close(dx.numpy(), O.act_bwd(kind, x, ry, dy), 1e-5, "backward")
+
+
+def test_unaligned_views_take_the_scalar_path(T, O):
+    """Sub-tensors that are not 16-byte aligned still give the same results."""
+    rng = np.random.default_rng(5)
+    n = 1001
+    y = rng.standard_normal((1, n + 1)).astype(np.float32)
+    dy = rng.standard_normal((1, n + 1)).astype(np.float32)
+    yd, dyd, out = T.to_device(y), T.to_device(dy), T.DevBuf((1, n + 1), zero=True)
+    off = lambda b: T.DevBuf.view(b.ptr.value + 4, (1, n))
+    T.act_bwd("tanh", 1, n, off(yd), off(dyd), off(out))
+    want = O.act_bwd("tanh", y[:, 1:], y[:, 1:], dy[:, 1:])
+    got = out.numpy()
+    assert got[0, 0] == 0.0
+    assert_close(got[:, 1:], want, 1e-6)
+
+
+def test_losses_match_oracle(T, O):
+    rng = np.random.default_rng(6)
+    y = O.act_fwd("softmax", rng.standard_normal((33, 10)).astype(np.float32))
+    t = np.eye(10, dtype=np.float32)[rng.integers(0, 10, 33)]
+    yd, td, g = T.to_device(y), T.to_device(t), T.DevBuf((33, 10))
+    for kind in ("mse", "ce_multiclass", "ce"):
+        T.loss_grad(kind, 33, 10, yd, td, g)
+        assert_close(g.numpy(), O.loss_grad(kind, y, t), 1e-6, kind)
+    T.softmax_xent_grad(33, 10, yd, td, g)
+    want = O.act_bwd("softmax", y, y, O.loss_grad("ce_multiclass", y, t))
+    assert_close(g.numpy(), want, 1e-5, "fused softmax + cross-entropy gradient")
+    # soft targets: y*sum(t) - t
+    t2 = rng.uniform(0, 1, (33, 10)).astype(np.float32)
+    T.softmax_xent_grad(33, 10, yd, T.to_device(t2), g)
+    assert_close(g.numpy(), O.act_bwd("softmax", y, y, O.loss_grad("ce_multiclass", y, t2)), 1e-5)
+
+
+@pytest.mark.parametrize("kind", ["sgd", "momentum", "adam", "adagrad", "rmsprop", "adamax", "nesterov"])
+def test_optimizers_match_oracle_and_reference_kats(T, O, kats, kind):
+    rng = np.random.default_rng(17)
+    n = 4099
+    o, ro = T.opt_desc(kind), O.opt_desc(kind)
+    w = rng.standard_normal(n).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    wd, gd = T.to_device(w), T.to_device(g)
+    s0, s1 = T.DevBuf((n,), zero=True), T.DevBuf((n,), zero=True)
+    rw, r0, r1 = w.copy(), np.zeros_like(w), np.zeros_like(w)
+    for _ in range(3):
+        T.opt_update(o, n, gd, wd, s0, s1)
+        O.opt_update(ro, g, rw, r0, r1)
+    assert_close(wd.numpy(), rw, 1e-6, "weights after 3 updates")
+    assert o.b1_t == ro.b1_t and o.b2_t == ro.b2_t, "per-call bias-correction powers"
+    for c in kats["optimizers"]["cases"]:
+        if c["kind"] != kind:
+            continue
+        o = T.opt_desc(kind)
+        wd, gd = T.to_device(np.array(c["w"], np.float32)), T.to_device(np.array(c["g"], np.float32))
+        s0, s1 = T.DevBuf((5,), zero=True), T.DevBuf((5,), zero=True)
+        T.opt_update(o, 5, gd, wd, s0, s1)
+        np.testing.assert_allclose(wd.numpy(), c["first"], atol=1e-3)
+        T.opt_update(o, 5, gd, wd, s0, s1)
+        np.testing.assert_allclose(wd.numpy(), c["second"], atol=1e-3)
+
+
+def test_optimizer_grad_scale_and_state_checks(T, O):
+    o = T.opt_desc("sgd", alpha=0.5)
+    w = T.to_device(np.zeros(3, np.float32))
+    T.opt_update(o, 3, T.to_device(np.array([2, -4, 8], np.float32)), w, grad_scale=0.25)
+    assert np.array_equal(w.numpy(), np.array([-0.25, 0.5, -1.0], np.float32))
+    with pytest.raises(T.TdhError, match="state"):
+        T.opt_update(T.opt_desc("adam"), 3, w, w, None, None)

@@ -1,0 +1,111 @@
+"""Live comparison of the oracle with the compiled reference (oracle/_ref, built from the
+unmodified tiny-dnn headers). Bit-for-bit against the scalar build; within the path's
+tolerance against the OpenMP+AVX build. Skipped where the reference is not built."""
+import numpy as np
+import pytest
+
+from conftest import assert_close
+
+
+@pytest.fixture(scope="module")
+def ref(O):
+    if O.ref_lib("scalar") is None:
+        pytest.skip("oracle/_ref not built (the tiny-dnn tree is not on this machine)")
+    return O
+
+
+CONV = [(5, 5, 1, 3, 1, False, 2, 1), (12, 10, 3, 3, 4, True, 1, 3), (9, 9, 2, 5, 3, True, 2, 2),
+        (32, 32, 1, 5, 6, False, 1, 4), (16, 16, 8, 5, 8, True, 1, 2), (11, 7, 3, 3, 5, True, 1, 5)]
+
+
+@pytest.mark.parametrize("cfg", CONV)
+def test_conv_bit_exact(ref, cfg):
+    O = ref
+    iw, ih, ic, k, oc, same, st, bs = cfg
+    rng = np.random.default_rng(hash(cfg) % 2**31)
+    d = O.conv_desc(iw, ih, ic, k, k, oc, pad_same=same, w_stride=st, h_stride=st)
+    ow, oh = O.conv_out_shape(d)
+    x = rng.standard_normal((bs, ic * ih * iw)).astype(np.float32)
+    w = rng.standard_normal(oc * ic * k * k).astype(np.float32)
+    b = rng.standard_normal(oc).astype(np.float32)
+    dy = rng.standard_normal((bs, oc * oh * ow)).astype(np.float32)
+    assert np.array_equal(O.conv2d_fwd(d, x, w, b), O.ref_conv2d_fwd(d, x, w, b))
+    for got, want in zip(O.conv2d_bwd(d, x, w, dy), O.ref_conv2d_bwd(d, x, w, dy)):
+        assert np.array_equal(got, want)
+    if O.ref_lib("avx") is not None:
+        for got, want in zip(O.conv2d_bwd(d, x, w, dy), O.ref_conv2d_bwd(d, x, w, dy, "avx", 1)):
+            assert_close(got, want, what="vs AVX engine")
+
+
+def test_conv_connection_table_bit_exact(ref):
+    O = ref
+    rng = np.random.default_rng(8)
+    tbl = rng.integers(0, 2, (6, 16)).astype(np.uint8)
+    d = O.conv_desc(14, 14, 6, 5, 5, 16, tbl=tbl)
+    x = rng.standard_normal((3, 6 * 196)).astype(np.float32)
+    w = rng.standard_normal(16 * 6 * 25).astype(np.float32)
+    b = rng.standard_normal(16).astype(np.float32)
+    dy = rng.standard_normal((3, 16 * 100)).astype(np.float32)
+    assert np.array_equal(O.conv2d_fwd(d, x, w, b), O.ref_conv2d_fwd(d, x, w, b))
+    for got, want in zip(O.conv2d_bwd(d, x, w, dy), O.ref_conv2d_bwd(d, x, w, dy)):
+        assert np.array_equal(got, want)
+
+
+def test_fc_pool_act_loss_opt_bit_exact(ref):
+    O = ref
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((5, 37)).astype(np.float32)
+    w = rng.standard_normal(37 * 19).astype(np.float32)
+    b = rng.standard_normal(19).astype(np.float32)
+    dy = rng.standard_normal((5, 19)).astype(np.float32)
+    assert np.array_equal(O.fc_fwd(x, w, b), O.ref_fc_fwd(x, w, b))
+    for got, want in zip(O.fc_bwd(x, w, dy), O.ref_fc_bwd(x, w, dy)):
+        assert np.array_equal(got, want)
+    for cfg in [(4, 4, 1, 2, 2, 2, 2, 0, 0), (7, 7, 2, 2, 2, 2, 2, 0, 1), (4, 4, 1, 2, 2, 1, 1, 1, 0),
+                (9, 8, 3, 3, 3, 2, 2, 0, 0), (6, 6, 2, 2, 2, 3, 3, 0, 0)]:
+        d = O.pool_desc(*cfg)
+        ow, oh = O.pool_out_shape(d)
+        xi = rng.integers(-3, 4, (3, cfg[2] * cfg[1] * cfg[0])).astype(np.float32)
+        g = rng.standard_normal((3, cfg[2] * oh * ow)).astype(np.float32)
+        y, am = O.maxpool_fwd(d, xi)
+        yr, dxr = O.ref_maxpool_fwd_bwd(d, xi, g)
+        assert np.array_equal(y, yr) and np.array_equal(O.maxpool_bwd(d, g, am), dxr)
+    for kind in ("tanh", "relu", "softmax", "sigmoid"):
+        xa = rng.standard_normal((4, 10)).astype(np.float32)
+        g = rng.standard_normal((4, 10)).astype(np.float32)
+        y = O.act_fwd(kind, xa)
+        yr, dxr = O.ref_act(kind, xa, g)
+        assert np.array_equal(y, yr) and np.array_equal(O.act_bwd(kind, xa, y, g), dxr)
+    y = O.act_fwd("softmax", rng.standard_normal((4, 10)).astype(np.float32))
+    t = np.eye(10, dtype=np.float32)[[1, 3, 5, 7]]
+    for kind in ("mse", "ce_multiclass", "ce"):
+        assert np.array_equal(O.loss_grad(kind, y, t), O.ref_loss_grad(kind, y, t))
+    for kind in O.OPT:
+        o, o2 = O.opt_desc(kind), O.opt_desc(kind)
+        w0 = rng.standard_normal(17).astype(np.float32)
+        g = rng.standard_normal(17).astype(np.float32)
+        want = O.ref_opt_updates(o2, g, w0, 3)
+        w1, s0, s1 = w0.copy(), np.zeros_like(w0), np.zeros_like(w0)
+        for _ in range(3):
+            O.opt_update(o, g, w1, s0, s1)
+        assert np.array_equal(w1, want), kind
+
+
+def test_vgg_style_step_bit_exact(ref, W):
+    """A shrunken VGG stack (16x16 input, batch 2): one momentum SGD step through fit().
+    (A second step already overflows in the reference itself: its update uses the gradient
+    summed over the batch, and softmax outputs that underflow to 0 turn -t/y into NaN.)"""
+    O = ref
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch("vgg_stack_b64", batch=2, size=16)
+    net = O.OracleNet(W.build_layers(O, spec), batch)
+    rn = O.RefNet(W.build_layers(O, spec), "scalar", 0)
+    for (i, which, a) in params:
+        (net.weight(i) if which == 0 else net.bias(i))[:] = a
+        rn.set_param(i, which, a)
+    o, o2 = O.opt_desc(opt_kind, **opt_kw), O.opt_desc(opt_kind, **opt_kw)
+    net.train_step(o, loss, x, t)
+    rn.fit(o2, loss, x, t, 1)
+    for (i, which, a) in params:
+        got = net.weight(i) if which == 0 else net.bias(i)
+        assert np.all(np.isfinite(got))
+        assert np.array_equal(got, rn.get_param(i, which)[:a.size]), (i, which)
