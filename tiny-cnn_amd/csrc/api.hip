@@ -2,6 +2,7 @@
 // validates arguments before anything is launched.
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <string>
@@ -56,6 +57,16 @@ int ws_take(size_t bytes, void **out) {
   *out = c.workspace + c.workspace_off;
   c.workspace_off += need;
   return TDH_OK;
+}
+
+// tdh_tune_gemm_plan forces one tile configuration and split count for every GEMM (tuning
+// sweeps only; in normal use the plan is a function of the shape alone).
+static int g_force_cfg = -1, g_force_splits = 1;
+
+bool gemm_plan_override(int *cfg, int *splits) {
+  *cfg    = g_force_cfg;
+  *splits = g_force_splits;
+  return g_force_cfg >= 0;
 }
 
 // ----------------------------------------------------------------- profiler
@@ -297,6 +308,14 @@ int tdh_event_elapsed_ms(void *start, void *stop, float *ms) {
   TDH_CHECK_ARG(start && stop && ms, "tdh_event_elapsed_ms: null argument");
   TDH_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
   TDH_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return TDH_OK;
+}
+
+int tdh_tune_gemm_plan(int32_t tile_cfg, int32_t splits) {
+  TDH_CHECK_ARG(tile_cfg < 10 && splits >= 1, "tdh_tune_gemm_plan: cfg %d splits %d", tile_cfg,
+                splits);
+  g_force_cfg    = tile_cfg;
+  g_force_splits = splits;
   return TDH_OK;
 }
 

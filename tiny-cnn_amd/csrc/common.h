@@ -36,6 +36,7 @@ int set_error(int code, const char *fmt, ...);
 int ws_begin(size_t total);
 // Next 256-byte aligned piece of the reserved scratch.
 int ws_take(size_t bytes, void **out);
+bool gemm_plan_override(int *cfg, int *splits);
 inline size_t ws_align(size_t bytes) { return (bytes + 255) & ~static_cast<size_t>(255); }
 
 #define TDH_REQUIRE_INIT()                                                     \
@@ -120,6 +121,17 @@ int launch_loss_grad(int kind, int batch, int len, const float *y, const float *
 int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz);
 int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, float *w, float *s0,
                       float *s1);
+// One launch for every trainable tensor of a network (update order = table order). Entry j
+// sees the optimizer's bias-correction powers advanced j times, as j earlier update() calls
+// would have left them; gradients are cleared after use when zero_grad is set.
+struct OptTensor {
+  float *g, *w, *s0, *s1;
+  uint32_t n, first_block;
+};
+constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 4096;
+int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
+                            int total_blocks, double total_params, float grad_scale,
+                            int zero_grad);
 // deterministic reductions: out[r] (+)= sum over `cols` contiguous values of row r,
 // rows laid out as [outer][rows][cols] and summed over outer in order
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate);

@@ -209,6 +209,130 @@ mask_weights_kernel(const float *__restrict__ src, const uint8_t *__restrict__ t
   dst[i]        = accumulate ? dst[i] + v : v;
 }
 
+// dX for convolutions with very few input channels (the first layer of an image network:
+// M = Cin = 1..4 would leave 7/8 of every 32-row MFMA block empty). Direct form on the vector
+// ALUs, stride 1: a workgroup owns a band of input rows of one image, stages the dY rows that
+// can reach it (with zero halo) in LDS eight output channels at a time, and every thread
+// accumulates its pixels for all Cin channels. Filter taps are wave-uniform reads.
+constexpr int DXS_MAX_CIN  = 4;
+constexpr int DXS_CO_CHUNK = 8;
+constexpr int DXS_PX       = 4;  // pixels per thread
+
+// KR, KS: compile-time window (0 = use the run-time g.R, g.S)
+template <int KR, int KS>
+__global__ void __launch_bounds__(256)
+conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__ w,
+                         float *__restrict__ dx, const ConvGeom g, const int tile_rows,
+                         const int bands, const ActGrad ag) {
+  extern __shared__ float smem[];  // dY tile [DXS_CO_CHUNK][trows][tcols], then weights
+  const int R = KR ? KR : g.R, S = KS ? KS : g.S;
+  const int img   = blockIdx.x / bands;
+  const int y0    = (blockIdx.x - img * bands) * tile_rows;
+  const int rows  = min(tile_rows, g.H - y0);
+  const int trows = tile_rows + R - 1, tcols = g.W + S - 1;
+  const int oy0 = y0 + g.pad_h - (R - 1), ox0 = g.pad_w - (S - 1);
+  const int ohw = g.OH * g.OW, rs = R * S;
+  const float *dy_img = dy + static_cast<size_t>(img) * g.Kc * ohw;
+  float *tile = smem;
+  float4 *wl  = reinterpret_cast<float4 *>(smem + ((DXS_CO_CHUNK * trows * tcols + 3) & ~3));
+
+  float acc[DXS_MAX_CIN][DXS_PX];
+#pragma unroll
+  for (int c = 0; c < DXS_MAX_CIN; ++c)
+#pragma unroll
+    for (int i = 0; i < DXS_PX; ++i) acc[c][i] = 0.0f;
+
+  // pixel i of this thread: p = tid + 256*i -> (py, px); its tile offset for tap (R-1, S-1)
+  int toff[DXS_PX];
+  bool live[DXS_PX];
+#pragma unroll
+  for (int i = 0; i < DXS_PX; ++i) {
+    const int p  = threadIdx.x + 256 * i;
+    const int py = p / g.W, px = p - py * g.W;
+    live[i] = py < rows;
+    toff[i] = live[i] ? py * tcols + px : 0;
+  }
+
+  for (int co0 = 0; co0 < g.Kc; co0 += DXS_CO_CHUNK) {
+    const int nco = min(DXS_CO_CHUNK, g.Kc - co0);
+    __syncthreads();
+    for (int e = threadIdx.x; e < nco * trows * tcols; e += 256) {
+      const int c = e / (trows * tcols);
+      const int r = (e - c * trows * tcols) / tcols;
+      const int q = e - c * trows * tcols - r * tcols;
+      const int oy = oy0 + r, ox = ox0 + q;
+      float v = 0.0f;
+      if (static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
+          static_cast<unsigned>(ox) < static_cast<unsigned>(g.OW))
+        v = dy_img[(co0 + c) * ohw + oy * g.OW + ox];
+      tile[e] = v;
+    }
+    // weights of the chunk as [c][tap] -> (w[ci=0..3]); tap stored flipped so that the
+    // inner loops walk the tile forwards
+    for (int e = threadIdx.x; e < nco * rs; e += 256) {
+      const int c = e / rs, t = e - c * rs;
+      const float *wc = w + (static_cast<size_t>(co0 + c) * g.C) * rs + (rs - 1 - t);
+      float4 v;
+      v.x = wc[0];
+      v.y = g.C > 1 ? wc[rs] : 0.0f;
+      v.z = g.C > 2 ? wc[2 * rs] : 0.0f;
+      v.w = g.C > 3 ? wc[3 * rs] : 0.0f;
+      wl[e] = v;
+    }
+    __syncthreads();
+    for (int c = 0; c < nco; ++c) {
+      const float *t = tile + c * trows * tcols;
+#pragma unroll
+      for (int fy = 0; fy < (KR ? KR : 1); ++fy)
+        for (int fyy = fy; fyy < R; fyy += (KR ? R : 1)) {
+#pragma unroll
+          for (int fx = 0; fx < (KS ? KS : 1); ++fx)
+            for (int fxx = fx; fxx < S; fxx += (KS ? S : 1)) {
+              // flipped tap (fyy, fxx) reads tile[(py + fyy)][px + fxx]
+              const float4 wv = wl[c * rs + fyy * S + fxx];
+#pragma unroll
+              for (int i = 0; i < DXS_PX; ++i) {
+                const float v = t[toff[i] + fyy * tcols + fxx];
+                acc[0][i] += wv.x * v;
+                acc[1][i] += wv.y * v;
+                acc[2][i] += wv.z * v;
+                acc[3][i] += wv.w * v;
+              }
+            }
+        }
+    }
+  }
+  float *dx_img = dx + static_cast<size_t>(img) * g.C * g.H * g.W;
+#pragma unroll
+  for (int i = 0; i < DXS_PX; ++i) {
+    if (!live[i]) continue;
+    const int p  = threadIdx.x + 256 * i;
+    const int py = p / g.W, px = p - py * g.W;
+#pragma unroll
+    for (int ci = 0; ci < DXS_MAX_CIN; ++ci) {
+      if (ci >= g.C) break;
+      const size_t idx = (static_cast<size_t>(ci) * g.H + y0 + py) * g.W + px;
+      float v = acc[ci][i];
+      if (ag.kind != TDH_ACT_NONE)
+        v *= act_grad_factor(ag.kind, ag.y[static_cast<size_t>(img) * g.C * g.H * g.W + idx]);
+      dx_img[idx] = v;
+    }
+  }
+}
+
+// true when the direct kernel applies; fills the launch geometry
+static bool small_cin_dx_plan(const ConvGeom &g, int &tile_rows, int &bands, size_t &lds_bytes) {
+  if (g.C > DXS_MAX_CIN || g.sh != 1 || g.sw != 1 || g.W > 256 * DXS_PX) return false;
+  tile_rows = (256 * DXS_PX) / g.W;
+  if (tile_rows > g.H) tile_rows = g.H;
+  // keep at least ~2 workgroups per image so that small batches still fill the chip
+  if (tile_rows > 8 && tile_rows * 2 > g.H) tile_rows = (g.H + 1) / 2;
+  bands     = ceil_div(g.H, tile_rows);
+  lds_bytes = sizeof(float) * (((DXS_CO_CHUNK * (tile_rows + g.R - 1) * (g.W + g.S - 1) + 3) & ~3) +
+                               4 * DXS_CO_CHUNK * g.R * g.S);
+  return lds_bytes <= 64 * 1024;
+}
+
 }  // namespace
 
 size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
@@ -267,7 +391,21 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, &tbl_dev, &w_eff));
-  if (dx) {
+  int tile_rows = 0, bands = 0;
+  size_t lds_bytes = 0;
+  if (dx && small_cin_dx_plan(g, tile_rows, bands, lds_bytes)) {
+    ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
+    if (g.R == 3 && g.S == 3)
+      hipLaunchKernelGGL((conv_dx_small_cin_kernel<3, 3>), dim3(batch * bands), dim3(256),
+                         lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
+    else if (g.R == 5 && g.S == 5)
+      hipLaunchKernelGGL((conv_dx_small_cin_kernel<5, 5>), dim3(batch * bands), dim3(256),
+                         lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
+    else
+      hipLaunchKernelGGL((conv_dx_small_cin_kernel<0, 0>), dim3(batch * bands), dim3(256),
+                         lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
+    TDH_LAUNCH_CHECK();
+  } else if (dx) {
     DxWeightOperand A{w_eff, g.C, g.R * g.S, g.div_rs};
     DxDyOperand B{dy, g, batch * g.H * g.W};
     EpiImageRows epi{dx, g.C, g.H * g.W, g.div_hw, nullptr, dx_act};

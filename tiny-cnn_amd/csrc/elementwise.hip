@@ -275,6 +275,54 @@ int launch_opt(size_t n, const float *g, float *w, float *s0, float *s1, const O
   return TDH_OK;
 }
 
+// Multi-tensor form: block b works on tensor j = the table entry whose block range holds b.
+template <int KIND, int NSTATE>
+__global__ void __launch_bounds__(EW_THREADS)
+opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptScalars p,
+                 const float b1_t, const float b2_t, const int zero_grad) {
+  int j = 0;
+  while (j + 1 < n_tensors && table[j + 1].first_block <= blockIdx.x) ++j;
+  const OptTensor t = table[j];
+  // the reference multiplies b1_t by b1 after every update() call (optimizer.h:125-126)
+  float p1 = b1_t, p2 = b2_t;
+  for (int i = 0; i < j; ++i) {
+    p1 *= p.b1;
+    p2 *= p.b2;
+  }
+  p.omb1t     = 1.0f - p1;
+  p.omb2t     = 1.0f - p2;
+  p.adamax_lr = static_cast<double>(p.alpha) / (1.0 - static_cast<double>(p1));
+  const uint32_t beg = (blockIdx.x - t.first_block) * OPT_MULTI_ELEMS_PER_BLOCK;
+  const uint32_t end = min(t.n, beg + OPT_MULTI_ELEMS_PER_BLOCK);
+  // tensors come from separate allocations (256-byte aligned): 16-byte accesses are safe
+  const uint32_t end4 = beg + ((end - beg) & ~3u);
+  for (uint32_t i = beg + threadIdx.x * 4; i < end4; i += EW_THREADS * 4) {
+    const float4 vg = *reinterpret_cast<const float4 *>(t.g + i);
+    float4 vw       = *reinterpret_cast<float4 *>(t.w + i);
+    float4 v0       = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
+    if (NSTATE >= 1) v0 = *reinterpret_cast<float4 *>(t.s0 + i);
+    if (NSTATE >= 2) v1 = *reinterpret_cast<float4 *>(t.s1 + i);
+    opt_one<KIND>(vg.x, vw.x, v0.x, v1.x, p);
+    opt_one<KIND>(vg.y, vw.y, v0.y, v1.y, p);
+    opt_one<KIND>(vg.z, vw.z, v0.z, v1.z, p);
+    opt_one<KIND>(vg.w, vw.w, v0.w, v1.w, p);
+    *reinterpret_cast<float4 *>(t.w + i) = vw;
+    if (NSTATE >= 1) *reinterpret_cast<float4 *>(t.s0 + i) = v0;
+    if (NSTATE >= 2) *reinterpret_cast<float4 *>(t.s1 + i) = v1;
+    if (zero_grad) *reinterpret_cast<float4 *>(t.g + i) = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  for (uint32_t i = end4 + threadIdx.x; i < end; i += EW_THREADS) {
+    float ww = t.w[i], a = 0.0f, b = 0.0f;
+    if (NSTATE >= 1) a = t.s0[i];
+    if (NSTATE >= 2) b = t.s1[i];
+    opt_one<KIND>(t.g[i], ww, a, b, p);
+    t.w[i] = ww;
+    if (NSTATE >= 1) t.s0[i] = a;
+    if (NSTATE >= 2) t.s1[i] = b;
+    if (zero_grad) t.g[i] = 0.0f;
+  }
+}
+
 // ---------------------------------------------------------------- reductions
 // Block-wide sum with a fixed shape: wave butterflies, then wave 0 adds the four wave
 // totals in order. Every thread of the block must call it.
@@ -287,32 +335,34 @@ __device__ __forceinline__ float block_sum(float v, float *smem4) {
   return r;
 }
 
-// stage 1: partial[(o*rows + r)*chunks + c] = sum of a slice of row r in image o
+// Bias gradient of a convolution: out[r] (+)= sum over images o and pixels of
+// src[(o*rows + r)*cols + c]. Stage 1: workgroup (r, g) adds the planes of images
+// o = g, g+G, ... in order, each plane with a fixed block-wide tree. Stage 2: one wave per
+// row adds the G group sums with a fixed butterfly.
 __global__ void __launch_bounds__(EW_THREADS)
-rowsum_stage1_kernel(const float *__restrict__ src, const int rows, const int cols,
-                     const int chunks, const int chunk_len, float *__restrict__ partial) {
+rowsum_stage1_kernel(const float *__restrict__ src, const int outer, const int rows,
+                     const int cols, const int groups, float *__restrict__ partial) {
   __shared__ float smem4[4];
-  const int row = blockIdx.x;  // o*rows + r
-  const int c   = blockIdx.y;
-  const float *p = src + static_cast<size_t>(row) * cols;
-  const int beg = c * chunk_len;
-  const int end = min(cols, beg + chunk_len);
+  const int r = blockIdx.x, g = blockIdx.y;
   float s = 0.0f;
-  for (int i = beg + threadIdx.x; i < end; i += EW_THREADS) s += p[i];
+  for (int o = g; o < outer; o += groups) {
+    const float *p = src + (static_cast<size_t>(o) * rows + r) * cols;
+    for (int i = threadIdx.x; i < cols; i += EW_THREADS) s += p[i];
+  }
   s = block_sum(s, smem4);
-  if (threadIdx.x == 0) partial[static_cast<size_t>(row) * chunks + c] = s;
+  if (threadIdx.x == 0) partial[r * groups + g] = s;
 }
 
-// stage 2: out[r] (+)= sum over o (outer) and chunks, in index order
 __global__ void __launch_bounds__(EW_THREADS)
-rowsum_stage2_kernel(const float *__restrict__ partial, const int outer, const int rows,
-                     const int chunks, float *__restrict__ out, const int accumulate) {
-  const int r = blockIdx.x * EW_THREADS + threadIdx.x;
+rowsum_stage2_kernel(const float *__restrict__ partial, const int rows, const int groups,
+                     float *__restrict__ out, const int accumulate) {
+  const int r    = blockIdx.x * (EW_THREADS / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   if (r >= rows) return;
   float s = 0.0f;
-  for (int o = 0; o < outer; ++o)
-    for (int c = 0; c < chunks; ++c) s += partial[(static_cast<size_t>(o) * rows + r) * chunks + c];
-  out[r] = accumulate ? out[r] + s : s;
+  for (int g = lane; g < groups; g += 64) s += partial[r * groups + g];
+  s = wave_sum(s);
+  if (lane == 0) out[r] = accumulate ? out[r] + s : s;
 }
 
 // out[c] (+)= sum_s src[s*cols + c], s ascending (fully_connected bias gradient)
@@ -431,32 +481,70 @@ int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, fl
   return TDH_OK;
 }
 
-// chunking depends on the shape only
-static void rowsum_chunks(int cols, int &chunks, int &chunk_len) {
-  chunks = ceil_div(cols, 4096);
-  if (chunks > 64) chunks = 64;
-  chunk_len = ceil_div(cols, chunks);
-  chunks    = ceil_div(cols, chunk_len);
-}
+// grouping depends on the shape only
+static int rowsum_groups(int outer) { return outer < 64 ? outer : 64; }
 
 size_t rowsum_workspace_bytes(int outer, int rows, int cols) {
-  int chunks, chunk_len;
-  rowsum_chunks(cols, chunks, chunk_len);
-  return ws_align(static_cast<size_t>(outer) * rows * chunks * sizeof(float));
+  (void)cols;
+  return ws_align(static_cast<size_t>(rows) * rowsum_groups(outer) * sizeof(float));
+}
+
+int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
+                            int total_blocks, double total_params, float grad_scale,
+                            int zero_grad) {
+  if (n_tensors <= 0) return TDH_OK;
+  OptScalars p;
+  p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; p.b1 = o->b1; p.b2 = o->b2;
+  p.eps = o->eps;
+  p.omb1 = 1.0f - o->b1; p.omb2 = 1.0f - o->b2;
+  p.omb1t = p.omb2t = 0.0f;
+  p.grad_scale = grad_scale;
+  p.adamax_lr  = 0.0;
+  static const char *const tags[] = {"opt_sgd_multi", "opt_momentum_multi", "opt_adam_multi",
+                                     "opt_adagrad_multi", "opt_rmsprop_multi", "opt_adamax_multi",
+                                     "opt_nesterov_multi"};
+  TDH_CHECK_ARG(o->kind >= 0 && o->kind <= TDH_OPT_NESTEROV, "optimizer kind %d is not supported",
+                o->kind);
+  const int nstate = (o->kind == TDH_OPT_SGD) ? 0
+                     : (o->kind == TDH_OPT_ADAM || o->kind == TDH_OPT_ADAMAX) ? 2 : 1;
+  // gradient read (+ cleared), weight read+write, states read+write
+  ProfScope prof(tags[o->kind], (12.0 + 8.0 * nstate + (zero_grad ? 4.0 : 0.0)) * total_params,
+                 WORK_BYTE);
+#define TDH_LAUNCH_MULTI(KIND, NS)                                                            \
+  hipLaunchKernelGGL((opt_multi_kernel<KIND, NS>), dim3(total_blocks), dim3(EW_THREADS), 0,   \
+                     ctx().stream, dev_table, n_tensors, p, o->b1_t, o->b2_t, zero_grad)
+  switch (o->kind) {
+    case TDH_OPT_SGD: TDH_LAUNCH_MULTI(TDH_OPT_SGD, 0); break;
+    case TDH_OPT_MOMENTUM: TDH_LAUNCH_MULTI(TDH_OPT_MOMENTUM, 1); break;
+    case TDH_OPT_NESTEROV: TDH_LAUNCH_MULTI(TDH_OPT_NESTEROV, 1); break;
+    case TDH_OPT_ADAM: TDH_LAUNCH_MULTI(TDH_OPT_ADAM, 2); break;
+    case TDH_OPT_ADAGRAD: TDH_LAUNCH_MULTI(TDH_OPT_ADAGRAD, 1); break;
+    case TDH_OPT_RMSPROP: TDH_LAUNCH_MULTI(TDH_OPT_RMSPROP, 1); break;
+    case TDH_OPT_ADAMAX: TDH_LAUNCH_MULTI(TDH_OPT_ADAMAX, 2); break;
+  }
+#undef TDH_LAUNCH_MULTI
+  TDH_LAUNCH_CHECK();
+  for (int j = 0; j < n_tensors; ++j) {
+    if (o->kind == TDH_OPT_ADAM) {
+      o->b1_t *= o->b1;
+      o->b2_t *= o->b2;
+    } else if (o->kind == TDH_OPT_ADAMAX) {
+      o->b1_t *= o->b1;
+    }
+  }
+  return TDH_OK;
 }
 
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate) {
-  int chunks, chunk_len;
-  rowsum_chunks(cols, chunks, chunk_len);
+  const int groups = rowsum_groups(outer);
   void *ws = nullptr;
-  TDH_TRY(ws_take(static_cast<size_t>(outer) * rows * chunks * sizeof(float), &ws));
+  TDH_TRY(ws_take(static_cast<size_t>(rows) * groups * sizeof(float), &ws));
   ProfScope prof("bias_grad_rowsum", 4.0 * outer * rows * cols, WORK_BYTE);
-  hipLaunchKernelGGL(rowsum_stage1_kernel, dim3(outer * rows, chunks), dim3(EW_THREADS), 0,
-                     ctx().stream, src, rows, cols, chunks, chunk_len, static_cast<float *>(ws));
+  hipLaunchKernelGGL(rowsum_stage1_kernel, dim3(rows, groups), dim3(EW_THREADS), 0, ctx().stream,
+                     src, outer, rows, cols, groups, static_cast<float *>(ws));
   TDH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(rowsum_stage2_kernel, dim3(ceil_div(rows, EW_THREADS)), dim3(EW_THREADS), 0,
-                     ctx().stream, static_cast<const float *>(ws), outer, rows, chunks, out,
-                     accumulate);
+  hipLaunchKernelGGL(rowsum_stage2_kernel, dim3(ceil_div(rows, EW_THREADS / 64)), dim3(EW_THREADS),
+                     0, ctx().stream, static_cast<const float *>(ws), rows, groups, out, accumulate);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }

@@ -36,7 +36,6 @@ namespace tdh {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int GEMM_BK      = 16;
-constexpr int GEMM_THREADS = 256;
 constexpr int GEMM_LDS_PAD = 4;
 
 // ------------------------------------------------------------ plain matrices
@@ -106,19 +105,20 @@ struct EpiImageRows {
 // --------------------------------------------------------------------- kernel
 template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
           class Epi>
-__global__ void __launch_bounds__(GEMM_THREADS)
+__global__ void __launch_bounds__(64 * WM * WN)
 gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const int N,
                  const int K, const int k_per_split, float *__restrict__ partial) {
   constexpr int BK  = GEMM_BK;
+  constexpr int NT  = 64 * WM * WN;  // threads per workgroup
   constexpr int TM  = BM / WM / 32;  // 32x32 MFMA blocks per wave along M
   constexpr int TN  = BN / WN / 32;
-  constexpr int CA  = BM * BK / GEMM_THREADS;  // elements of A each thread stages per tile
-  constexpr int CB  = BN * BK / GEMM_THREADS;
+  constexpr int CA  = BM * BK / NT;  // elements of A each thread stages per tile
+  constexpr int CB  = BN * BK / NT;
   constexpr int LDA = BM + GEMM_LDS_PAD;
   constexpr int LDB = BN + GEMM_LDS_PAD;
-  static_assert(WM * WN == 4, "four waves per workgroup");
   static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
-  static_assert(GEMM_THREADS % BM == 0 && GEMM_THREADS % BN == 0, "tile/threads mismatch");
+  static_assert(TM * 32 * WM == BM && TN * 32 * WN == BN, "tile is not a whole number of blocks");
+  static_assert((BM * BK) % NT == 0 && (BN * BK) % NT == 0, "tile/threads mismatch");
 
   __shared__ float As[2][BK][LDA];
   __shared__ float Bs[2][BK][LDB];
@@ -134,21 +134,30 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   const int kend = min(K, kbeg + k_per_split);
 
   // ---- per-thread staging assignment
-  // LANE_K : k_local = tid % 16 (fixed), rows (tid/16) + 16*i
-  // !LANE_K: row = tid % BM (fixed), k_local = tid/BM + (256/BM)*i
-  typename AOp::Fix fa[A_LANE_K ? CA : 1];
-  typename BOp::Fix fb[B_LANE_K ? CB : 1];
+  // LANE_K : k_local = tid % 16 (fixed), rows (tid/16) + (NT/16)*i
+  // !LANE_K: element e = tid + NT*i of the tile, row = e % BM, k_local = e / BM; when the
+  //          tile width is a multiple of NT the row is the same for every i
+  constexpr bool A_ONE_ROW = (NT % BM) == 0;
+  constexpr bool B_ONE_ROW = (NT % BN) == 0;
+  typename AOp::Fix fa[(A_LANE_K || !A_ONE_ROW) ? CA : 1];
+  typename BOp::Fix fb[(B_LANE_K || !B_ONE_ROW) ? CB : 1];
   if (A_LANE_K) {
 #pragma unroll
-    for (int i = 0; i < CA; ++i) fa[i] = aop.fix(m0 + (tid >> 4) + 16 * i);
-  } else {
+    for (int i = 0; i < CA; ++i) fa[i] = aop.fix(m0 + (tid >> 4) + (NT / 16) * i);
+  } else if (A_ONE_ROW) {
     fa[0] = aop.fix(m0 + tid % BM);
+  } else {
+#pragma unroll
+    for (int i = 0; i < CA; ++i) fa[i] = aop.fix(m0 + (tid + NT * i) % BM);
   }
   if (B_LANE_K) {
 #pragma unroll
-    for (int i = 0; i < CB; ++i) fb[i] = bop.fix(n0 + (tid >> 4) + 16 * i);
-  } else {
+    for (int i = 0; i < CB; ++i) fb[i] = bop.fix(n0 + (tid >> 4) + (NT / 16) * i);
+  } else if (B_ONE_ROW) {
     fb[0] = bop.fix(n0 + tid % BN);
+  } else {
+#pragma unroll
+    for (int i = 0; i < CB; ++i) fb[i] = bop.fix(n0 + (tid + NT * i) % BN);
   }
 
   float ra[CA], rb[CB];
@@ -167,9 +176,9 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
     } else {
 #pragma unroll
       for (int i = 0; i < CA; ++i) {
-        int k = kt + tid / BM + (GEMM_THREADS / BM) * i;
+        int k = kt + (tid + NT * i) / BM;
         if (BM % 64 == 0) k = __builtin_amdgcn_readfirstlane(k);
-        ra[i] = (k < kend) ? aop.load(fa[0], aop.kdec(k)) : 0.0f;
+        ra[i] = (k < kend) ? aop.load(fa[A_ONE_ROW ? 0 : i], aop.kdec(k)) : 0.0f;
       }
     }
     if (B_LANE_K) {
@@ -185,9 +194,9 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
     } else {
 #pragma unroll
       for (int i = 0; i < CB; ++i) {
-        int k = kt + tid / BN + (GEMM_THREADS / BN) * i;
+        int k = kt + (tid + NT * i) / BN;
         if (BN % 64 == 0) k = __builtin_amdgcn_readfirstlane(k);
-        rb[i] = (k < kend) ? bop.load(fb[0], bop.kdec(k)) : 0.0f;
+        rb[i] = (k < kend) ? bop.load(fb[B_ONE_ROW ? 0 : i], bop.kdec(k)) : 0.0f;
       }
     }
   };
@@ -195,17 +204,17 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   auto stage = [&](int buf) {
     if (A_LANE_K) {
 #pragma unroll
-      for (int i = 0; i < CA; ++i) As[buf][tid & 15][(tid >> 4) + 16 * i] = ra[i];
+      for (int i = 0; i < CA; ++i) As[buf][tid & 15][(tid >> 4) + (NT / 16) * i] = ra[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < CA; ++i) As[buf][tid / BM + (GEMM_THREADS / BM) * i][tid % BM] = ra[i];
+      for (int i = 0; i < CA; ++i) As[buf][(tid + NT * i) / BM][(tid + NT * i) % BM] = ra[i];
     }
     if (B_LANE_K) {
 #pragma unroll
-      for (int i = 0; i < CB; ++i) Bs[buf][tid & 15][(tid >> 4) + 16 * i] = rb[i];
+      for (int i = 0; i < CB; ++i) Bs[buf][tid & 15][(tid >> 4) + (NT / 16) * i] = rb[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < CB; ++i) Bs[buf][tid / BN + (GEMM_THREADS / BN) * i][tid % BN] = rb[i];
+      for (int i = 0; i < CB; ++i) Bs[buf][(tid + NT * i) / BN][(tid + NT * i) % BN] = rb[i];
     }
   };
 
@@ -279,48 +288,121 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   }
 }
 
-// Adds the K-split partial tiles in split order and applies the epilogue.
+// Adds the K-split partial tiles and applies the epilogue. A workgroup owns 32 consecutive
+// outputs; its eight 32-lane groups each add every eighth slice (g, g+8, ...) and the eight
+// group sums are then added in group order, so the summation tree depends on the split
+// count only.
+constexpr int REDUCE_OUTPUTS = 32;
+constexpr int REDUCE_GROUPS  = 8;
+
 template <class Epi>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const int M, const int N,
                      const Epi epi) {
-  const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= M * N) return;
-  const int m = idx / N, n = idx - m * N;
+  __shared__ float sm[REDUCE_GROUPS][REDUCE_OUTPUTS];
+  const int o   = threadIdx.x & (REDUCE_OUTPUTS - 1);
+  const int g   = threadIdx.x / REDUCE_OUTPUTS;
+  const int idx = blockIdx.x * REDUCE_OUTPUTS + o;
+  const size_t mn = static_cast<size_t>(M) * N;
   float s = 0.0f;
-  for (int z = 0; z < splits; ++z) s += partial[static_cast<size_t>(z) * M * N + idx];
-  epi.store(m, epi.col(n), s);
+  if (idx < M * N)
+    for (int z = g; z < splits; z += REDUCE_GROUPS) s += partial[z * mn + idx];
+  sm[g][o] = s;
+  __syncthreads();
+  if (g == 0 && idx < M * N) {
+    float t = sm[0][o];
+#pragma unroll
+    for (int i = 1; i < REDUCE_GROUPS; ++i) t += sm[i][o];
+    const int m = idx / N, n = idx - m * N;
+    epi.store(m, epi.col(n), t);
+  }
 }
 
 // ------------------------------------------------------------------- launcher
 struct GemmPlan {
+  int cfg;          // index into the tile table below
   int bm, bn;       // tile
   int splits;       // K splits
   int k_per_split;  // multiple of GEMM_BK
 };
 
+// tile table: {BM, BN, waves along M, waves along N}
+struct TileCfg {
+  int bm, bn, wm, wn;
+};
+constexpr TileCfg kTiles[] = {
+  {128, 128, 2, 2},  // 0
+  {128, 64, 2, 2},   // 1
+  {64, 128, 2, 2},   // 2
+  {64, 64, 2, 2},    // 3
+  {32, 128, 1, 4},   // 4
+  {32, 256, 1, 4},   // 5
+  {32, 64, 1, 2},    // 6
+  {64, 32, 2, 1},    // 7
+  {32, 32, 1, 1},    // 8
+  {64, 96, 2, 1},    // 9
+};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
+// Optional override "cfg,splits" from the environment (tuning runs only).
+bool gemm_plan_override(int *cfg, int *splits);
+
 // Shape-only heuristics (no device queries) so that results are reproducible anywhere.
 inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
-  GemmPlan p;
-  p.bm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
-  p.bn = (N <= 64 && p.bm != 32) ? 64 : 128;
-  const long tiles = static_cast<long>(ceil_div(M, p.bm)) * ceil_div(N, p.bn);
-  int splits       = 1;
-  if (allow_split && tiles < 512) {
-    splits = static_cast<int>(1024 / tiles);
-    const int max_by_k = K / 256 > 0 ? K / 256 : 1;
-    if (splits > max_by_k) splits = max_by_k;
-    if (splits > 512) splits = 512;
-    if (splits < 1) splits = 1;
+  // relative MFMA efficiency of a tile (operand fetches per MFMA, prologue share)
+  static const double kEff[kNumTiles] = {1.00, 0.88, 0.88, 0.72, 0.62, 0.80, 0.50, 0.50, 0.36, 0.84};
+  const double kSlots = 512.0;  // workgroups of 256 threads the chip runs at full rate
+  int best = 0, best_splits = 1;
+  double best_cost = 1e300;
+  for (int c = 0; c < kNumTiles; ++c) {
+    const TileCfg &t = kTiles[c];
+    if (t.bm > 32 && t.bm >= 2 * M && M > 0 && t.bm / 2 >= 32) continue;  // half the rows empty
+    if (t.bn > 32 && t.bn >= 2 * N && t.bn / 2 >= 32) continue;
+    const double tiles = static_cast<double>(ceil_div(M, t.bm)) * ceil_div(N, t.bn);
+    const double slots = kSlots * 256.0 / (64.0 * t.wm * t.wn);
+    int splits = 1;
+    if (allow_split && tiles < slots) {
+      splits = static_cast<int>(slots / tiles);
+      const int max_by_k = K / 96 > 0 ? K / 96 : 1;
+      if (splits > max_by_k) splits = max_by_k;
+      if (splits < 1) splits = 1;
+    }
+    const double work  = tiles * t.bm * t.bn * static_cast<double>(K);  // padded MACs
+    const double waves = tiles * splits / slots;
+    const double fill  = waves >= 1.0 ? waves / static_cast<double>(static_cast<long>(waves + 0.999)) : waves;
+    double cost = work / (kEff[c] * (fill > 1.0 ? 1.0 : fill));
+    if (splits > 1) cost += 3.0 * tiles * t.bm * t.bn * splits * 64.0;  // partial tile traffic
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = c;
+      best_splits = splits;
+    }
   }
-  p.k_per_split = ceil_div(ceil_div(K, splits), GEMM_BK) * GEMM_BK;
+  int ocfg, osplits;
+  if (gemm_plan_override(&ocfg, &osplits)) {
+    best = ocfg;
+    best_splits = allow_split ? osplits : 1;
+    if (best_splits > K / GEMM_BK && K >= GEMM_BK) best_splits = K / GEMM_BK;
+    if (best_splits < 1) best_splits = 1;
+  }
+  GemmPlan p;
+  p.cfg = best;
+  p.bm = kTiles[best].bm;
+  p.bn = kTiles[best].bn;
+  p.k_per_split = ceil_div(ceil_div(K, best_splits), GEMM_BK) * GEMM_BK;
   p.splits      = ceil_div(K, p.k_per_split);
+  if (p.splits < 1) p.splits = 1;
   return p;
 }
 
 inline size_t gemm_workspace_bytes(int M, int N, int K, bool allow_split) {
+  // the plan can be overridden at run time, so reserve for the largest split count any
+  // plan may use for this shape
   const GemmPlan p = plan_gemm(M, N, K, allow_split);
-  return p.splits > 1 ? ws_align(static_cast<size_t>(p.splits) * M * N * sizeof(float)) : 0;
+  int ocfg, osplits;
+  int splits = p.splits;
+  if (gemm_plan_override(&ocfg, &osplits) && osplits > splits) splits = osplits;
+  return splits > 1 ? ws_align(static_cast<size_t>(splits) * M * N * sizeof(float)) : 0;
 }
 
 template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
@@ -330,7 +412,7 @@ int launch_gemm_tile(const AOp &a, const BOp &b, const Epi &epi, int M, int N, i
   ProfScope prof(tag, M, N, K);
   dim3 grid(ceil_div(N, BN), ceil_div(M, BM), p.splits);
   hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, AOp, BOp, Epi>), grid,
-                     dim3(GEMM_THREADS), 0, ctx().stream, a, b, epi, M, N, K, p.k_per_split,
+                     dim3(64 * WM * WN), 0, ctx().stream, a, b, epi, M, N, K, p.k_per_split,
                      partial);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -349,22 +431,27 @@ int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
     TDH_TRY(ws_take(static_cast<size_t>(p.splits) * M * N * sizeof(float), &ws));
     partial = static_cast<float *>(ws);
   }
-  int rc;
-  if (p.bm == 128 && p.bn == 128)
-    rc = launch_gemm_tile<128, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
-  else if (p.bm == 128 && p.bn == 64)
-    rc = launch_gemm_tile<128, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
-  else if (p.bm == 64 && p.bn == 128)
-    rc = launch_gemm_tile<64, 128, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
-  else if (p.bm == 64 && p.bn == 64)
-    rc = launch_gemm_tile<64, 64, 2, 2, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
-  else
-    rc = launch_gemm_tile<32, 128, 1, 4, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag);
+  int rc = TDH_OK;
+#define TDH_TILE(BM, BN, WM, WN) \
+  rc = launch_gemm_tile<BM, BN, WM, WN, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag)
+  switch (p.cfg) {
+    case 0: TDH_TILE(128, 128, 2, 2); break;
+    case 1: TDH_TILE(128, 64, 2, 2); break;
+    case 2: TDH_TILE(64, 128, 2, 2); break;
+    case 3: TDH_TILE(64, 64, 2, 2); break;
+    case 4: TDH_TILE(32, 128, 1, 4); break;
+    case 5: TDH_TILE(32, 256, 1, 4); break;
+    case 6: TDH_TILE(32, 64, 1, 2); break;
+    case 7: TDH_TILE(64, 32, 2, 1); break;
+    case 8: TDH_TILE(32, 32, 1, 1); break;
+    default: TDH_TILE(64, 96, 2, 1); break;
+  }
+#undef TDH_TILE
   TDH_TRY(rc);
   if (p.splits > 1) {
     // reads every partial tile once and writes the result once
     ProfScope prof(reduce_tag, 4.0 * M * N * (p.splits + 1), WORK_BYTE);
-    hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, 256)), dim3(256), 0,
+    hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, REDUCE_OUTPUTS)), dim3(256), 0,
                        ctx().stream, partial, p.splits, M, N, epi);
     TDH_LAUNCH_CHECK();
   }

@@ -22,6 +22,9 @@ struct tdh_net {
   int max_batch  = 0;
   int flags      = 0;
   float *dx_in   = nullptr;  // gradient w.r.t. the network input
+  tdh::OptTensor *opt_table = nullptr;  // device table of trainable tensors, update order
+  int opt_tensors = 0, opt_blocks = 0;
+  double opt_params = 0.0;
   size_t scratch = 0;        // largest per-op scratch need
   std::vector<void *> allocs;
 };
@@ -180,6 +183,37 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
   }
   if (rc == TDH_OK)
     rc = net_alloc(net, net->layers[0].in_size * static_cast<size_t>(max_batch), &net->dx_in, true);
+  if (rc == TDH_OK) {
+    // nodes::update_weights order: layers front to back, weight before bias
+    std::vector<OptTensor> table;
+    uint32_t block = 0;
+    for (auto &L : net->layers) {
+      for (int which = 0; which < 2; ++which) {
+        const size_t n = which ? L.b_size : L.w_size;
+        if (!n) continue;
+        OptTensor t;
+        t.g  = which ? L.db : L.dw;
+        t.w  = which ? L.b : L.w;
+        t.s0 = which ? L.s0b : L.s0w;
+        t.s1 = which ? L.s1b : L.s1w;
+        t.n  = static_cast<uint32_t>(n);
+        t.first_block = block;
+        block += static_cast<uint32_t>(ceil_div_sz(n, OPT_MULTI_ELEMS_PER_BLOCK));
+        net->opt_params += static_cast<double>(n);
+        table.push_back(t);
+      }
+    }
+    net->opt_tensors = static_cast<int>(table.size());
+    net->opt_blocks  = static_cast<int>(block);
+    if (!table.empty()) {
+      float *p = nullptr;
+      rc = net_alloc(net, ceil_div_sz(table.size() * sizeof(OptTensor), sizeof(float)), &p, false);
+      if (rc == TDH_OK) {
+        net->opt_table = reinterpret_cast<OptTensor *>(p);
+        rc = tdh_memcpy_h2d(net->opt_table, table.data(), table.size() * sizeof(OptTensor));
+      }
+    }
+  }
   if (rc != TDH_OK) {
     for (void *p : net->allocs) (void)hipFree(p);
     delete net;
@@ -305,17 +339,8 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   // nodes::update_weights visits layers front to back, weight before bias; the gradient
   // reaches the optimizer unscaled (rcp_batch_size is 1, see tdh_opt_update) and is then
   // cleared (layer.h:680)
-  for (auto &L : net->layers) {
-    if (L.w_size) {
-      TDH_TRY(launch_opt_update(opt, L.w_size, L.dw, 1.0f, L.w, L.s0w, L.s1w));
-      TDH_TRY(launch_fill_zero(L.dw, L.w_size * sizeof(float)));
-    }
-    if (L.b_size) {
-      TDH_TRY(launch_opt_update(opt, L.b_size, L.db, 1.0f, L.b, L.s0b, L.s1b));
-      TDH_TRY(launch_fill_zero(L.db, L.b_size * sizeof(float)));
-    }
-  }
-  return TDH_OK;
+  return launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
+                                 net->opt_params, 1.0f, 1);
 }
 
 }  // extern "C"
