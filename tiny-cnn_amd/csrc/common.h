@@ -154,6 +154,13 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
            const float *b, float *y);
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act);
+// conv_s1.hip: stride-1 forward / dX with LDS halo tiles (3x3 and 5x5 windows)
+bool conv_s1_applicable(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
+                        int ph, int pw);
+size_t conv_s1_workspace_bytes(int R, int S, int C, int Kc);
+int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
+                const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
+                int OW, int ph, int pw, ActGrad ag, const char *tag);
 // workspace bytes the op may ask for (so a net can reserve it before graph capture)
 size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
 size_t fc_workspace_bytes(int in, int out, int batch);

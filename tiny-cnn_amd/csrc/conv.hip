@@ -344,6 +344,7 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   total += gemm_workspace_bytes(g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true);  // dX
   total += rowsum_workspace_bytes(batch, g.Kc, ohw);                  // db
   if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
+  total += 2 * conv_s1_workspace_bytes(g.R, g.S, g.C, g.Kc);          // repacked filters
   return total;
 }
 
@@ -378,6 +379,11 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, &tbl_dev, &w_eff));
+  if (g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 &&
+      conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w))
+    return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w_eff, nullptr,
+                       d->has_bias ? b : nullptr, y, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w,
+                       ActGrad(), "conv_fwd_s1");
   StridedOperand A{w_eff, crs, 1, g.Kc};
   FwdInputOperand B{x, g, batch * ohw};
   EpiImageRows epi{y, g.Kc, ohw, g.div_ohw, d->has_bias ? b : nullptr, ActGrad()};
@@ -405,6 +411,12 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       hipLaunchKernelGGL((conv_dx_small_cin_kernel<0, 0>), dim3(batch * bands), dim3(256),
                          lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
     TDH_LAUNCH_CHECK();
+  } else if (dx && g.sh == 1 && g.sw == 1 &&
+             conv_s1_applicable(g.R, g.S, batch, g.Kc, g.C, g.OH, g.OW, g.H, g.W,
+                                g.R - 1 - g.pad_h, g.S - 1 - g.pad_w)) {
+    TDH_TRY(conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 1, dy, w_eff, nullptr, nullptr, dx, g.OH,
+                        g.OW, g.H, g.W, g.R - 1 - g.pad_h, g.S - 1 - g.pad_w, dx_act,
+                        "conv_dx_s1"));
   } else if (dx) {
     DxWeightOperand A{w_eff, g.C, g.R * g.S, g.div_rs};
     DxDyOperand B{dy, g, batch * g.H * g.W};
