@@ -42,7 +42,8 @@ class NetWorkload:
         self.T, self.W, self.name = T, W, name
         (self.spec, self.params, x, t, self.batch, self.loss, self.opt_kind,
          self.opt_kw) = W.make_batch(name)
-        self.net = T.Net(W.build_layers(T, self.spec), self.batch, T.NET_FUSE_ACT_GRAD)
+        self.net = T.Net(W.build_layers(T, self.spec), self.batch,
+                         T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
         for (i, which, a) in self.params:
             self.net.set_param(i, which, a)
         self.opt = T.opt_desc(self.opt_kind, **self.opt_kw)
@@ -50,6 +51,7 @@ class NetWorkload:
         self.samples = self.batch
         self.config = {"workload": name, "batch": self.batch, "loss": self.loss,
                        "optimizer": self.opt_kind, "step": "fwd+bwd+update",
+                       "launch": "captured HIP graph (per-kernel pass runs the same kernels eagerly)",
                        "flop_per_step": 3 * self.batch * W.flops_per_sample(self.spec)}
 
     def step(self):

@@ -119,3 +119,47 @@ def test_net_rejects_inconsistent_layers(T):
         T.Net([T.L_fc(10, 5), T.L_fc(6, 2)], 4)
     with pytest.raises(T.TdhError, match="first layer"):
         T.Net([T.L_act("relu"), T.L_fc(6, 2)], 4)
+
+
+@pytest.mark.parametrize("name,batch", [("cifar10_cnn_b128", 16), ("lenet5_b16", 16)])
+def test_graph_replay_matches_eager_on_every_step(T, W, name, batch):
+    """TDH_NET_GRAPH: the captured step is replayed five times with eager work, readbacks and
+    synchronisations in between; after every replay all parameters equal the eager net's bit
+    for bit (same kernels, same order), including Adam's per-tensor bias-correction powers."""
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch)
+    eager = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD)
+    graph = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
+    for (i, which, a) in params:
+        eager.set_param(i, which, a)
+        graph.set_param(i, which, a)
+    o1, o2 = T.opt_desc(opt_kind, **opt_kw), T.opt_desc(opt_kind, **opt_kw)
+    xd, td = T.to_device(x), T.to_device(t)
+    side_in = T.to_device(np.linspace(-2, 2, 4096, dtype=np.float32)[None])
+    side_out = T.DevBuf((1, 4096))
+    for step in range(5):
+        eager.train_step(o1, loss, batch, xd, td)
+        graph.train_step(o2, loss, batch, xd, td)
+        T.act_fwd("tanh", 1, 4096, side_in, side_out)      # unrelated eager work in between
+        T.sync()
+        assert side_out.numpy()[0, 0] == np.float32(np.tanh(np.float32(-2.0)))
+        for (i, which, a) in params:
+            assert np.array_equal(eager.get_param(i, which), graph.get_param(i, which)), (step, i, which)
+        assert o1.b1_t == o2.b1_t and o1.b2_t == o2.b2_t
+    # a changed optimizer object (new hyper-parameter, reset powers) is honoured
+    o1.alpha = o2.alpha = 0.5 * o1.alpha
+    o1.b1_t = o2.b1_t = 0.9
+    eager.train_step(o1, loss, batch, xd, td)
+    graph.train_step(o2, loss, batch, xd, td)
+    for (i, which, a) in params:
+        assert np.array_equal(eager.get_param(i, which), graph.get_param(i, which)), (i, which)
+    # another batch size re-captures
+    eager.train_step(o1, loss, batch // 2, xd, td)
+    graph.train_step(o2, loss, batch // 2, xd, td)
+    for (i, which, a) in params:
+        assert np.array_equal(eager.get_param(i, which), graph.get_param(i, which)), (i, which)
+    # gradients without update through the graph path as well
+    eager.train_step(None, loss, batch, xd, td, do_update=False)
+    graph.train_step(None, loss, batch, xd, td, do_update=False)
+    for (i, which, a) in params:
+        assert np.array_equal(eager.layer_grad(i, which), graph.layer_grad(i, which))
+    eager.close(); graph.close()

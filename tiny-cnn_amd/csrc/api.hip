@@ -108,6 +108,8 @@ static int open_record(const std::string &tag, double work, WorkUnit unit) {
   return static_cast<int>(g_records.size()) - 1;
 }
 
+bool profiling_active() { return g_profiling; }
+
 ProfScope::ProfScope(const char *tag, double work, WorkUnit unit) : slot(-1) {
   if (g_profiling) slot = open_record(tag, work, unit);
 }

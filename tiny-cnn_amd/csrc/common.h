@@ -129,9 +129,12 @@ struct OptTensor {
   uint32_t n, first_block;
 };
 constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 4096;
+// dev_powers: NULL, or two device floats {b1_t, b2_t} that the kernel reads instead of the
+// host values and that a follow-up kernel advances n_tensors times (graph replay).
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
-                            int zero_grad);
+                            int zero_grad, float *dev_powers);
+bool profiling_active();
 // deterministic reductions: out[r] (+)= sum over `cols` contiguous values of row r,
 // rows laid out as [outer][rows][cols] and summed over outer in order
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate);
@@ -147,9 +150,10 @@ struct ActGrad {
 
 // conv.hip / fc.hip
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
-               float *y);
+               float *y, const uint8_t *tbl_resident = nullptr);
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
-               float *dx, float *dw, float *db, int accumulate, ActGrad dx_act);
+               float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
+               const uint8_t *tbl_resident = nullptr);
 int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *b, float *y);
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,

@@ -345,12 +345,16 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   total += rowsum_workspace_bytes(batch, g.Kc, ohw);                  // db
   if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
   total += 2 * conv_s1_workspace_bytes(g.R, g.S, g.C, g.Kc);          // repacked filters
+
   return total;
 }
 
 // Uploads the connection table (if any) and returns masked weights in scratch.
+// `tbl_resident`: a device copy the caller keeps (a network does, so that a captured graph
+// holds no host copies); otherwise the host table is uploaded into scratch here.
 static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float *w,
-                         const uint8_t **tbl_dev, const float **w_eff) {
+                         const uint8_t *tbl_resident, const uint8_t **tbl_dev,
+                         const float **w_eff) {
   *tbl_dev = nullptr;
   *w_eff   = w;
   if (!d->tbl) return TDH_OK;
@@ -358,10 +362,14 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
   const int nw = g.Kc * g.C * g.R * g.S;
   TDH_TRY(ws_take(static_cast<size_t>(g.C) * g.Kc, &t));
   TDH_TRY(ws_take(sizeof(float) * nw, &wm));
-  // pageable source: the copy is staged before the call returns
-  TDH_HIP(hipMemcpyAsync(t, d->tbl, static_cast<size_t>(g.C) * g.Kc, hipMemcpyHostToDevice,
-                         ctx().stream));
-  TDH_HIP(hipStreamSynchronize(ctx().stream));
+  if (tbl_resident) {
+    t = const_cast<uint8_t *>(tbl_resident);
+  } else {
+    // pageable source: the copy is staged before the call returns
+    TDH_HIP(hipMemcpyAsync(t, d->tbl, static_cast<size_t>(g.C) * g.Kc, hipMemcpyHostToDevice,
+                           ctx().stream));
+    TDH_HIP(hipStreamSynchronize(ctx().stream));
+  }
   ProfScope prof("conv_mask_weights", 8.0 * nw, WORK_BYTE);
   hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(nw, 256)), dim3(256), 0, ctx().stream, w,
                      static_cast<const uint8_t *>(t), static_cast<float *>(wm), nw, g.C, g.Kc,
@@ -373,12 +381,12 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
 }
 
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
-               float *y) {
+               float *y, const uint8_t *tbl_resident) {
   const ConvGeom g = make_geom(d);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
-  TDH_TRY(prepare_table(d, g, w, &tbl_dev, &w_eff));
+  TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
   if (g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 &&
       conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w))
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w_eff, nullptr,
@@ -391,12 +399,13 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
 }
 
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
-               float *dx, float *dw, float *db, int accumulate, ActGrad dx_act) {
+               float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
+               const uint8_t *tbl_resident) {
   const ConvGeom g = make_geom(d);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
-  TDH_TRY(prepare_table(d, g, w, &tbl_dev, &w_eff));
+  TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
   int tile_rows = 0, bands = 0;
   size_t lds_bytes = 0;
   if (dx && small_cin_dx_plan(g, tile_rows, bands, lds_bytes)) {
@@ -438,7 +447,8 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       TDH_LAUNCH_CHECK();
     } else {
       EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
-      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm", "conv_dw_splitk_reduce")));
+      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm",
+                                       "conv_dw_splitk_reduce")));
     }
   }
   if (db) TDH_TRY(launch_rowsum(dy, batch, g.Kc, ohw, db, accumulate));

@@ -279,7 +279,12 @@ int launch_opt(size_t n, const float *g, float *w, float *s0, float *s1, const O
 template <int KIND, int NSTATE>
 __global__ void __launch_bounds__(EW_THREADS)
 opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptScalars p,
-                 const float b1_t, const float b2_t, const int zero_grad) {
+                 float b1_t, float b2_t, const float *__restrict__ dev_powers,
+                 const int zero_grad) {
+  if (dev_powers) {
+    b1_t = dev_powers[0];
+    b2_t = dev_powers[1];
+  }
   int j = 0;
   while (j + 1 < n_tensors && table[j + 1].first_block <= blockIdx.x) ++j;
   const OptTensor t = table[j];
@@ -321,6 +326,19 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
     if (NSTATE >= 2) t.s1[i] = b;
     if (zero_grad) t.g[i] = 0.0f;
   }
+}
+
+// advances the device copy of the bias-correction powers as n update() calls would
+__global__ void opt_advance_powers_kernel(float *powers, const int n, const float b1,
+                                          const float b2, const int adam) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float p1 = powers[0], p2 = powers[1];
+  for (int i = 0; i < n; ++i) {
+    p1 *= b1;
+    if (adam) p2 *= b2;
+  }
+  powers[0] = p1;
+  powers[1] = p2;
 }
 
 // ---------------------------------------------------------------- reductions
@@ -365,15 +383,25 @@ rowsum_stage2_kernel(const float *__restrict__ partial, const int rows, const in
   if (lane == 0) out[r] = accumulate ? out[r] + s : s;
 }
 
-// out[c] (+)= sum_s src[s*cols + c], s ascending (fully_connected bias gradient)
+// out[c] (+)= sum_s src[s*cols + c] (fully_connected bias gradient). A workgroup owns 32
+// columns; its eight row groups add rows g, g+8, ... and the group sums are added in order.
 __global__ void __launch_bounds__(EW_THREADS)
 colsum_kernel(const float *__restrict__ src, const int rows, const int cols,
               float *__restrict__ out, const int accumulate) {
-  const int c = blockIdx.x * EW_THREADS + threadIdx.x;
-  if (c >= cols) return;
+  __shared__ float sm[8][32];
+  const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
+  const int c  = blockIdx.x * 32 + cl;
   float s = 0.0f;
-  for (int r = 0; r < rows; ++r) s += src[static_cast<size_t>(r) * cols + c];
-  out[c] = accumulate ? out[c] + s : s;
+  if (c < cols)
+    for (int r = g; r < rows; r += 8) s += src[static_cast<size_t>(r) * cols + c];
+  sm[g][cl] = s;
+  __syncthreads();
+  if (g == 0 && c < cols) {
+    float t = sm[0][cl];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) t += sm[i][cl];
+    out[c] = accumulate ? out[c] + t : t;
+  }
 }
 
 }  // namespace
@@ -491,7 +519,7 @@ size_t rowsum_workspace_bytes(int outer, int rows, int cols) {
 
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
-                            int zero_grad) {
+                            int zero_grad, float *dev_powers) {
   if (n_tensors <= 0) return TDH_OK;
   OptScalars p;
   p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; p.b1 = o->b1; p.b2 = o->b2;
@@ -512,7 +540,8 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
                  WORK_BYTE);
 #define TDH_LAUNCH_MULTI(KIND, NS)                                                            \
   hipLaunchKernelGGL((opt_multi_kernel<KIND, NS>), dim3(total_blocks), dim3(EW_THREADS), 0,   \
-                     ctx().stream, dev_table, n_tensors, p, o->b1_t, o->b2_t, zero_grad)
+                     ctx().stream, dev_table, n_tensors, p, o->b1_t, o->b2_t,                  \
+                     static_cast<const float *>(dev_powers), zero_grad)
   switch (o->kind) {
     case TDH_OPT_SGD: TDH_LAUNCH_MULTI(TDH_OPT_SGD, 0); break;
     case TDH_OPT_MOMENTUM: TDH_LAUNCH_MULTI(TDH_OPT_MOMENTUM, 1); break;
@@ -524,6 +553,11 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
   }
 #undef TDH_LAUNCH_MULTI
   TDH_LAUNCH_CHECK();
+  if (dev_powers && (o->kind == TDH_OPT_ADAM || o->kind == TDH_OPT_ADAMAX)) {
+    hipLaunchKernelGGL(opt_advance_powers_kernel, dim3(1), dim3(64), 0, ctx().stream, dev_powers,
+                       n_tensors, o->b1, o->b2, o->kind == TDH_OPT_ADAM ? 1 : 0);
+    TDH_LAUNCH_CHECK();
+  }
   for (int j = 0; j < n_tensors; ++j) {
     if (o->kind == TDH_OPT_ADAM) {
       o->b1_t *= o->b1;
@@ -551,7 +585,7 @@ int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, i
 
 int launch_colsum(const float *src, int rows, int cols, float *out, int accumulate) {
   ProfScope prof("bias_grad_colsum", 4.0 * rows * cols, WORK_BYTE);
-  hipLaunchKernelGGL(colsum_kernel, dim3(ceil_div(cols, EW_THREADS)), dim3(EW_THREADS), 0,
+  hipLaunchKernelGGL(colsum_kernel, dim3(ceil_div(cols, 32)), dim3(EW_THREADS), 0,
                      ctx().stream, src, rows, cols, out, accumulate);
   TDH_LAUNCH_CHECK();
   return TDH_OK;

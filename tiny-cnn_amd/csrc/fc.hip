@@ -19,7 +19,8 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
   StridedOperand A{x, in, 1, batch};   // X[s][k], k contiguous
   StridedOperand B{w, 1, out, out};    // W[k][n], n contiguous
   EpiRowMajor epi{y, out, has_bias ? b : nullptr, ActGrad(), 0};
-  return launch_gemm<true, false>(A, B, epi, batch, out, in, true, "fc_fwd_gemm", "fc_fwd_splitk_reduce");
+  return launch_gemm<true, false, false, true>(A, B, epi, batch, out, in, true, "fc_fwd_gemm",
+                                              "fc_fwd_splitk_reduce");
 }
 
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
@@ -28,13 +29,15 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     StridedOperand A{dy, out, 1, batch};  // dY[s][k]
     StridedOperand B{w, out, 1, in};      // W[n][k], k contiguous
     EpiRowMajor epi{dx, in, nullptr, dx_act, 0};
-    TDH_TRY((launch_gemm<true, true>(A, B, epi, batch, in, out, true, "fc_dx_gemm", "fc_dx_splitk_reduce")));
+    TDH_TRY((launch_gemm<true, true, false, false>(A, B, epi, batch, in, out, true, "fc_dx_gemm",
+                                                 "fc_dx_splitk_reduce")));
   }
   if (dw) {
     StridedOperand A{x, 1, in, in};      // X[k][m], m contiguous
     StridedOperand B{dy, 1, out, out};   // dY[k][n], n contiguous
     EpiRowMajor epi{dw, out, nullptr, ActGrad(), accumulate};
-    TDH_TRY((launch_gemm<false, false>(A, B, epi, in, out, batch, true, "fc_dw_gemm", "fc_dw_splitk_reduce")));
+    TDH_TRY((launch_gemm<false, false, true, true>(A, B, epi, in, out, batch, true, "fc_dw_gemm",
+                                                   "fc_dw_splitk_reduce")));
   }
   if (db && has_bias) TDH_TRY(launch_colsum(dy, batch, out, db, accumulate));
   return TDH_OK;

@@ -38,6 +38,12 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int GEMM_BK      = 16;
 constexpr int GEMM_LDS_PAD = 4;
 
+// four floats with 4-byte alignment: lets the compiler emit one dwordx4 access where the
+// address is only float-aligned (global memory tolerates it)
+struct __attribute__((packed, aligned(4))) float4u {
+  float x, y, z, w;
+};
+
 // ------------------------------------------------------------ plain matrices
 // element(mn, k) = p[mn * s_mn + k * s_k]
 struct StridedOperand {
@@ -54,6 +60,25 @@ struct StridedOperand {
   __device__ __forceinline__ KDec kdec(int k) const { return {k * s_k}; }
   __device__ __forceinline__ float load(const Fix &f, const KDec &k) const {
     return f.valid ? p[f.off + k.off] : 0.0f;
+  }
+  // four consecutive k (needs s_k == 1)
+  __device__ __forceinline__ float4 load4k(const Fix &f, const KDec &k) const {
+    if (!f.valid) return make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4u v = *reinterpret_cast<const float4u *>(p + f.off + k.off);
+    return make_float4(v.x, v.y, v.z, v.w);
+  }
+  // four consecutive m/n starting at f (needs s_mn == 1); `count` of them are in range
+  __device__ __forceinline__ float4 load4m(const Fix &f, const KDec &k, int mn) const {
+    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (mn + 3 < extent) {
+      const float4u v = *reinterpret_cast<const float4u *>(p + f.off + k.off);
+      r = make_float4(v.x, v.y, v.z, v.w);
+    } else {
+      if (mn < extent) r.x = p[f.off + k.off];
+      if (mn + 1 < extent) r.y = p[f.off + k.off + 1];
+      if (mn + 2 < extent) r.z = p[f.off + k.off + 2];
+    }
+    return r;
   }
 };
 
@@ -103,8 +128,8 @@ struct EpiImageRows {
 };
 
 // --------------------------------------------------------------------- kernel
-template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
-          class Epi>
+template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, bool A_VEC, bool B_VEC,
+          class AOp, class BOp, class Epi>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const int N,
                  const int K, const int k_per_split, float *__restrict__ partial) {
@@ -119,9 +144,13 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
   static_assert(TM * 32 * WM == BM && TN * 32 * WN == BN, "tile is not a whole number of blocks");
   static_assert((BM * BK) % NT == 0 && (BN * BK) % NT == 0, "tile/threads mismatch");
+  // vectorised staging: a thread moves groups of four floats (four k of one row, or four rows
+  // of one k). Groups per thread: CA/4, CB/4.
+  static_assert(!A_VEC || (CA % 4 == 0 && (A_LANE_K || (4 * NT) % BM == 0)), "A vec4 shape");
+  static_assert(!B_VEC || (CB % 4 == 0 && (B_LANE_K || (4 * NT) % BN == 0)), "B vec4 shape");
 
-  __shared__ float As[2][BK][LDA];
-  __shared__ float Bs[2][BK][LDB];
+  __shared__ __attribute__((aligned(16))) float As[2][BK][LDA];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDB];
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -141,7 +170,14 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   constexpr bool B_ONE_ROW = (NT % BN) == 0;
   typename AOp::Fix fa[(A_LANE_K || !A_ONE_ROW) ? CA : 1];
   typename BOp::Fix fb[(B_LANE_K || !B_ONE_ROW) ? CB : 1];
-  if (A_LANE_K) {
+  if constexpr (A_VEC && A_LANE_K) {
+    // k group = tid % 4, rows (tid/4) + (NT/4)*i
+#pragma unroll
+    for (int i = 0; i < CA / 4; ++i) fa[i] = aop.fix(m0 + (tid >> 2) + (NT / 4) * i);
+  } else if constexpr (A_VEC) {
+    // row group = tid % (BM/4) (rows 4g..4g+3), k_local = tid/(BM/4) + (4*NT/BM)*i
+    fa[0] = aop.fix(m0 + 4 * (tid % (BM / 4)));
+  } else if (A_LANE_K) {
 #pragma unroll
     for (int i = 0; i < CA; ++i) fa[i] = aop.fix(m0 + (tid >> 4) + (NT / 16) * i);
   } else if (A_ONE_ROW) {
@@ -150,7 +186,12 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
 #pragma unroll
     for (int i = 0; i < CA; ++i) fa[i] = aop.fix(m0 + (tid + NT * i) % BM);
   }
-  if (B_LANE_K) {
+  if constexpr (B_VEC && B_LANE_K) {
+#pragma unroll
+    for (int i = 0; i < CB / 4; ++i) fb[i] = bop.fix(n0 + (tid >> 2) + (NT / 4) * i);
+  } else if constexpr (B_VEC) {
+    fb[0] = bop.fix(n0 + 4 * (tid % (BN / 4)));
+  } else if (B_LANE_K) {
 #pragma unroll
     for (int i = 0; i < CB; ++i) fb[i] = bop.fix(n0 + (tid >> 4) + (NT / 16) * i);
   } else if (B_ONE_ROW) {
@@ -163,7 +204,29 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   float ra[CA], rb[CB];
 
   auto fetch = [&](int kt) {
-    if (A_LANE_K) {
+    if constexpr (A_VEC && A_LANE_K) {
+      const int k = kt + 4 * (tid & 3);
+#pragma unroll
+      for (int i = 0; i < CA / 4; ++i) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k + 3 < kend) {
+          v = aop.load4k(fa[i], aop.kdec(k));
+        } else {
+          if (k < kend) v.x = aop.load(fa[i], aop.kdec(k));
+          if (k + 1 < kend) v.y = aop.load(fa[i], aop.kdec(k + 1));
+          if (k + 2 < kend) v.z = aop.load(fa[i], aop.kdec(k + 2));
+        }
+        ra[4 * i] = v.x; ra[4 * i + 1] = v.y; ra[4 * i + 2] = v.z; ra[4 * i + 3] = v.w;
+      }
+    } else if constexpr (A_VEC) {
+#pragma unroll
+      for (int i = 0; i < CA / 4; ++i) {
+        int k = kt + tid / (BM / 4) + (4 * NT / BM) * i;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k < kend) v = aop.load4m(fa[0], aop.kdec(k), m0 + 4 * (tid % (BM / 4)));
+        ra[4 * i] = v.x; ra[4 * i + 1] = v.y; ra[4 * i + 2] = v.z; ra[4 * i + 3] = v.w;
+      }
+    } else if (A_LANE_K) {
       const int k = kt + (tid & 15);
       if (k < kend) {
         const typename AOp::KDec kd = aop.kdec(k);
@@ -181,7 +244,29 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
         ra[i] = (k < kend) ? aop.load(fa[A_ONE_ROW ? 0 : i], aop.kdec(k)) : 0.0f;
       }
     }
-    if (B_LANE_K) {
+    if constexpr (B_VEC && B_LANE_K) {
+      const int k = kt + 4 * (tid & 3);
+#pragma unroll
+      for (int i = 0; i < CB / 4; ++i) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k + 3 < kend) {
+          v = bop.load4k(fb[i], bop.kdec(k));
+        } else {
+          if (k < kend) v.x = bop.load(fb[i], bop.kdec(k));
+          if (k + 1 < kend) v.y = bop.load(fb[i], bop.kdec(k + 1));
+          if (k + 2 < kend) v.z = bop.load(fb[i], bop.kdec(k + 2));
+        }
+        rb[4 * i] = v.x; rb[4 * i + 1] = v.y; rb[4 * i + 2] = v.z; rb[4 * i + 3] = v.w;
+      }
+    } else if constexpr (B_VEC) {
+#pragma unroll
+      for (int i = 0; i < CB / 4; ++i) {
+        int k = kt + tid / (BN / 4) + (4 * NT / BN) * i;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k < kend) v = bop.load4m(fb[0], bop.kdec(k), n0 + 4 * (tid % (BN / 4)));
+        rb[4 * i] = v.x; rb[4 * i + 1] = v.y; rb[4 * i + 2] = v.z; rb[4 * i + 3] = v.w;
+      }
+    } else if (B_LANE_K) {
       const int k = kt + (tid & 15);
       if (k < kend) {
         const typename BOp::KDec kd = bop.kdec(k);
@@ -202,14 +287,36 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   };
 
   auto stage = [&](int buf) {
-    if (A_LANE_K) {
+    if constexpr (A_VEC && A_LANE_K) {
+#pragma unroll
+      for (int i = 0; i < CA / 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          As[buf][4 * (tid & 3) + j][(tid >> 2) + (NT / 4) * i] = ra[4 * i + j];
+    } else if constexpr (A_VEC) {
+#pragma unroll
+      for (int i = 0; i < CA / 4; ++i)
+        *reinterpret_cast<float4 *>(&As[buf][tid / (BM / 4) + (4 * NT / BM) * i][4 * (tid % (BM / 4))]) =
+          make_float4(ra[4 * i], ra[4 * i + 1], ra[4 * i + 2], ra[4 * i + 3]);
+    } else if (A_LANE_K) {
 #pragma unroll
       for (int i = 0; i < CA; ++i) As[buf][tid & 15][(tid >> 4) + (NT / 16) * i] = ra[i];
     } else {
 #pragma unroll
       for (int i = 0; i < CA; ++i) As[buf][(tid + NT * i) / BM][(tid + NT * i) % BM] = ra[i];
     }
-    if (B_LANE_K) {
+    if constexpr (B_VEC && B_LANE_K) {
+#pragma unroll
+      for (int i = 0; i < CB / 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          Bs[buf][4 * (tid & 3) + j][(tid >> 2) + (NT / 4) * i] = rb[4 * i + j];
+    } else if constexpr (B_VEC) {
+#pragma unroll
+      for (int i = 0; i < CB / 4; ++i)
+        *reinterpret_cast<float4 *>(&Bs[buf][tid / (BN / 4) + (4 * NT / BN) * i][4 * (tid % (BN / 4))]) =
+          make_float4(rb[4 * i], rb[4 * i + 1], rb[4 * i + 2], rb[4 * i + 3]);
+    } else if (B_LANE_K) {
 #pragma unroll
       for (int i = 0; i < CB; ++i) Bs[buf][tid & 15][(tid >> 4) + (NT / 16) * i] = rb[i];
     } else {
@@ -405,20 +512,24 @@ inline size_t gemm_workspace_bytes(int M, int N, int K, bool allow_split) {
   return splits > 1 ? ws_align(static_cast<size_t>(splits) * M * N * sizeof(float)) : 0;
 }
 
-template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, class AOp, class BOp,
-          class Epi>
+template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, bool A_VEC, bool B_VEC,
+          class AOp, class BOp, class Epi>
 int launch_gemm_tile(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
                      const GemmPlan &p, float *partial, const char *tag) {
   ProfScope prof(tag, M, N, K);
   dim3 grid(ceil_div(N, BN), ceil_div(M, BM), p.splits);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, AOp, BOp, Epi>), grid,
+  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, A_VEC, B_VEC, AOp, BOp,
+                                       Epi>), grid,
                      dim3(64 * WM * WN), 0, ctx().stream, a, b, epi, M, N, K, p.k_per_split,
                      partial);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }
 
-template <bool A_LANE_K, bool B_LANE_K, class AOp, class BOp, class Epi>
+// A_VEC / B_VEC: the operand provides load4k (LANE_K) or load4m (otherwise) and its layout
+// allows groups of four; used by the tiles wide enough for it (the rest stage scalars).
+template <bool A_LANE_K, bool B_LANE_K, bool A_VEC = false, bool B_VEC = false, class AOp,
+          class BOp, class Epi>
 int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
                 bool allow_split, const char *tag, const char *reduce_tag) {
   if (M <= 0 || N <= 0) return TDH_OK;
@@ -432,19 +543,21 @@ int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
     partial = static_cast<float *>(ws);
   }
   int rc = TDH_OK;
-#define TDH_TILE(BM, BN, WM, WN) \
-  rc = launch_gemm_tile<BM, BN, WM, WN, A_LANE_K, B_LANE_K>(a, b, epi, M, N, K, p, partial, tag)
+#define TDH_TILE(BM, BN, WM, WN, AV, BV)                                                  \
+  rc = launch_gemm_tile<BM, BN, WM, WN, A_LANE_K, B_LANE_K, AV, BV>(a, b, epi, M, N, K, p, \
+                                                                    partial, tag)
+  // vector staging needs at least four floats per thread and operand
   switch (p.cfg) {
-    case 0: TDH_TILE(128, 128, 2, 2); break;
-    case 1: TDH_TILE(128, 64, 2, 2); break;
-    case 2: TDH_TILE(64, 128, 2, 2); break;
-    case 3: TDH_TILE(64, 64, 2, 2); break;
-    case 4: TDH_TILE(32, 128, 1, 4); break;
-    case 5: TDH_TILE(32, 256, 1, 4); break;
-    case 6: TDH_TILE(32, 64, 1, 2); break;
-    case 7: TDH_TILE(64, 32, 2, 1); break;
-    case 8: TDH_TILE(32, 32, 1, 1); break;
-    default: TDH_TILE(64, 96, 2, 1); break;
+    case 0: TDH_TILE(128, 128, 2, 2, A_VEC, B_VEC); break;
+    case 1: TDH_TILE(128, 64, 2, 2, A_VEC, B_VEC); break;
+    case 2: TDH_TILE(64, 128, 2, 2, A_VEC, B_VEC); break;
+    case 3: TDH_TILE(64, 64, 2, 2, A_VEC, B_VEC); break;
+    case 4: TDH_TILE(32, 128, 1, 4, false, B_VEC); break;
+    case 5: TDH_TILE(32, 256, 1, 4, false, B_VEC); break;
+    case 6: TDH_TILE(32, 64, 1, 2, A_VEC, B_VEC); break;
+    case 7: TDH_TILE(64, 32, 2, 1, A_VEC, B_VEC); break;
+    case 8: TDH_TILE(32, 32, 1, 1, A_VEC, B_VEC); break;
+    default: TDH_TILE(64, 96, 2, 1, A_VEC &&A_LANE_K, B_VEC &&B_LANE_K); break;
   }
 #undef TDH_TILE
   TDH_TRY(rc);

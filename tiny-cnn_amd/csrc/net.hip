@@ -2,6 +2,7 @@
 // network<sequential>::train_onebatch (tiny_dnn/network.h:911-926) = fprop
 // (nodes.h:288-303), loss gradient (loss_function.h:191-218), bprop (nodes.h:276-286) and
 // update_weights (nodes.h:103-107, layer.h:663-682), queued on the library stream.
+#include <cstring>
 #include <vector>
 
 #include "common.h"
@@ -10,6 +11,7 @@ struct tdh_net {
   struct Layer {
     tdh_layer spec;
     std::vector<uint8_t> tbl;  // private copy of the connection table
+    uint8_t *tbl_dev = nullptr;
     size_t in_size = 0, out_size = 0, w_size = 0, b_size = 0;
     float *w = nullptr, *b = nullptr, *dw = nullptr, *db = nullptr;
     float *s0w = nullptr, *s1w = nullptr, *s0b = nullptr, *s1b = nullptr;
@@ -25,6 +27,16 @@ struct tdh_net {
   tdh::OptTensor *opt_table = nullptr;  // device table of trainable tensors, update order
   int opt_tensors = 0, opt_blocks = 0;
   double opt_params = 0.0;
+  // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
+  float *dev_powers = nullptr;          // {b1_t, b2_t} as the captured optimizer kernel reads them
+  hipGraphExec_t graph_exec = nullptr;
+  struct GraphKey {
+    int batch = 0, loss = 0, do_update = 0;
+    const float *x = nullptr, *t = nullptr;
+    const void *scratch = nullptr;      // the library scratch buffer the captured kernels use
+    tdh_opt hyper = {};                 // hyper-parameters only (powers zeroed)
+  } graph_key;
+  float mirror_b1_t = 0.0f, mirror_b2_t = 0.0f;  // what the device copy of the powers holds
   size_t scratch = 0;        // largest per-op scratch need
   std::vector<void *> allocs;
 };
@@ -93,7 +105,7 @@ int forward(tdh_net *net, int batch, const float *x) {
     switch (s.kind) {
       case TDH_L_CONV:
         TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
-        TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out));
+        TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev));
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
@@ -122,8 +134,6 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
                    tdh_net **out) {
   TDH_REQUIRE_INIT();
   TDH_CHECK_ARG(layers && out && n_layers > 0 && max_batch > 0, "tdh_net_create: bad argument");
-  if (flags & TDH_NET_GRAPH)
-    return set_error(TDH_ERR_UNSUPPORTED, "tdh_net_create: graph replay is not built yet");
   *out = nullptr;
   tdh_net *net   = new tdh_net();
   net->max_batch = max_batch;
@@ -170,6 +180,12 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       if ((rc = net_alloc(net, act, &p, true))) break;
       L.argmax = reinterpret_cast<int32_t *>(p);
     }
+    if (!L.tbl.empty()) {
+      float *p = nullptr;
+      if ((rc = net_alloc(net, ceil_div_sz(L.tbl.size(), sizeof(float)), &p, false))) break;
+      L.tbl_dev = reinterpret_cast<uint8_t *>(p);
+      if ((rc = tdh_memcpy_h2d(L.tbl_dev, L.tbl.data(), L.tbl.size()))) break;
+    }
     size_t need = 0;
     if (L.spec.kind == TDH_L_CONV) need = conv2d_workspace_bytes(&L.spec.conv, max_batch);
     if (L.spec.kind == TDH_L_FC) need = fc_workspace_bytes(L.spec.fc_in, L.spec.fc_out, max_batch);
@@ -214,6 +230,9 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       }
     }
   }
+  if (rc == TDH_OK) rc = net_alloc(net, 2, &net->dev_powers, true);
+  // reserve the scratch every layer may need, so that no op ever has to grow it
+  if (rc == TDH_OK) rc = ws_begin(net->scratch);
   if (rc != TDH_OK) {
     for (void *p : net->allocs) (void)hipFree(p);
     delete net;
@@ -227,6 +246,7 @@ int tdh_net_destroy(tdh_net *net) {
   TDH_REQUIRE_INIT();
   if (!net) return TDH_OK;
   TDH_HIP(hipStreamSynchronize(ctx().stream));
+  if (net->graph_exec) TDH_HIP(hipGraphExecDestroy(net->graph_exec));
   for (void *p : net->allocs) TDH_HIP(hipFree(p));
   delete net;
   return TDH_OK;
@@ -280,12 +300,9 @@ int tdh_net_forward(tdh_net *net, int batch, const float *x) {
   return forward(net, batch, x);
 }
 
-int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
-                       const float *t, int do_update) {
-  TDH_REQUIRE_INIT();
-  TDH_CHECK_ARG(net && x && t && batch > 0 && batch <= net->max_batch,
-                "tdh_net_train_step: bad argument");
-  TDH_CHECK_ARG(!do_update || opt, "tdh_net_train_step: update requested without an optimizer");
+// Queues one whole train step on the library stream.
+static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
+                        const float *t, int do_update, float *dev_powers) {
   TDH_TRY(forward(net, batch, x));
   const int n          = static_cast<int>(net->layers.size());
   tdh_net::Layer &last = net->layers[n - 1];
@@ -317,7 +334,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
       case TDH_L_CONV:
         TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
         TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
-                           fold));
+                           fold, L.tbl_dev));
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
@@ -340,7 +357,89 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   // reaches the optimizer unscaled (rcp_batch_size is 1, see tdh_opt_update) and is then
   // cleared (layer.h:680)
   return launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
-                                 net->opt_params, 1.0f, 1);
+                                 net->opt_params, 1.0f, 1, dev_powers);
+}
+
+static bool same_key(const tdh_net::GraphKey &a, const tdh_net::GraphKey &b) {
+  return a.batch == b.batch && a.loss == b.loss && a.do_update == b.do_update && a.x == b.x &&
+         a.t == b.t && a.scratch == b.scratch &&
+         std::memcmp(&a.hyper, &b.hyper, sizeof(tdh_opt)) == 0;
+}
+
+int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
+                       const float *t, int do_update) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && x && t && batch > 0 && batch <= net->max_batch,
+                "tdh_net_train_step: bad argument");
+  TDH_CHECK_ARG(!do_update || opt, "tdh_net_train_step: update requested without an optimizer");
+  // per-kernel timing needs the launches themselves, not a replay
+  if (!(net->flags & TDH_NET_GRAPH) || profiling_active())
+    return enqueue_step(net, opt, loss_kind, batch, x, t, do_update, nullptr);
+
+  tdh_net::GraphKey key;
+  key.batch = batch; key.loss = loss_kind; key.do_update = do_update; key.x = x; key.t = t;
+  if (opt) {
+    key.hyper      = *opt;
+    key.hyper.b1_t = key.hyper.b2_t = 0.0f;
+  }
+  TDH_TRY(ws_begin(net->scratch));  // may move the scratch buffer if another op outgrew it
+  key.scratch = ctx().workspace;
+  if (!net->graph_exec || !same_key(key, net->graph_key)) {
+    if (net->graph_exec) {
+      TDH_HIP(hipGraphExecDestroy(net->graph_exec));
+      net->graph_exec = nullptr;
+    }
+    Context &c  = ctx();
+    c.ws_locked = true;  // nothing may allocate while the stream is capturing
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal);
+    int rc = TDH_OK;
+    if (e == hipSuccess) {
+      tdh_opt capture_opt;
+      if (opt) capture_opt = *opt;
+      rc = enqueue_step(net, opt ? &capture_opt : nullptr, loss_kind, batch, x, t, do_update,
+                        net->dev_powers);
+      e = hipStreamEndCapture(c.stream, &graph);
+    }
+    c.ws_locked = false;
+    if (rc != TDH_OK) {
+      if (graph) (void)hipGraphDestroy(graph);
+      return rc;
+    }
+    if (e != hipSuccess || !graph)
+      return set_error(TDH_ERR_HIP, "tdh_net_train_step: graph capture failed: %s",
+                       hipGetErrorString(e));
+    e = hipGraphInstantiate(&net->graph_exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+      net->graph_exec = nullptr;
+      return set_error(TDH_ERR_HIP, "tdh_net_train_step: graph instantiation failed: %s",
+                       hipGetErrorString(e));
+    }
+    net->graph_key   = key;
+    net->mirror_b1_t = net->mirror_b2_t = -1.0f;  // forces the upload below
+  }
+  // the captured optimizer kernel reads the powers from device memory; bring that copy in
+  // line with the caller's optimizer object whenever the two have drifted apart
+  if (opt && do_update && (opt->b1_t != net->mirror_b1_t || opt->b2_t != net->mirror_b2_t)) {
+    const float h[2] = {opt->b1_t, opt->b2_t};
+    TDH_TRY(tdh_memcpy_h2d(net->dev_powers, h, sizeof(h)));
+  }
+  TDH_HIP(hipGraphLaunch(net->graph_exec, ctx().stream));
+  if (opt && do_update) {
+    // advance the host object exactly as the eager path does
+    for (int j = 0; j < net->opt_tensors; ++j) {
+      if (opt->kind == TDH_OPT_ADAM) {
+        opt->b1_t *= opt->b1;
+        opt->b2_t *= opt->b2;
+      } else if (opt->kind == TDH_OPT_ADAMAX) {
+        opt->b1_t *= opt->b1;
+      }
+    }
+    net->mirror_b1_t = opt->b1_t;
+    net->mirror_b2_t = opt->b2_t;
+  }
+  return TDH_OK;
 }
 
 }  // extern "C"
