@@ -223,6 +223,9 @@ size_t tdh_net_layer_out_size(const tdh_net *net, int layer);
 size_t tdh_net_param_size(const tdh_net *net, int layer, int which);
 int tdh_net_set_param(tdh_net *net, int layer, int which, const float *host_src);
 int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst);
+/* optimizer::reset() as network::fit calls it before training (tiny_dnn/network.h:856,
+ * tiny_dnn/optimizers/optimizer.h:36-38): clears the per-weight state vectors */
+int tdh_net_reset_optimizer(tdh_net *net);
 /* device views valid until the net is destroyed */
 float *tdh_net_param(tdh_net *net, int layer, int which);
 const float *tdh_net_layer_out(const tdh_net *net, int layer);

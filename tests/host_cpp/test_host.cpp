@@ -1,0 +1,380 @@
+// Tests of the C++ host mirror (tiny_dnn_hip.h) on a GPU: the reference's own known-answer
+// tests for this path, written against the same class names, plus random cases checked against
+// the CPU oracle (oracle/td_oracle.h). Built by tests/host_cpp/Makefile, run by
+// tests/test_gpu_host_cpp.py.
+//
+// Known answers come from the reference's test-suite:
+//   convolutional.with_stride   test/test_convolutional_layer.h:133-200
+//   fully_connected.forward     test/test_fully_connected_layer.h:48-64
+//   max_pool.forward/backward   test/test_max_pooling_layer.h:25-39, 85-110, 251-281
+//   optimizers                  test/test_optimizers.h:15-190
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+
+#include "td_oracle.h"
+#include "tiny_dnn_hip.h"
+
+using namespace tiny_dnn;
+
+static int g_failed = 0, g_checks = 0;
+
+#define EXPECT(cond)                                                       \
+  do {                                                                     \
+    ++g_checks;                                                            \
+    if (!(cond)) {                                                         \
+      ++g_failed;                                                          \
+      std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);      \
+    }                                                                      \
+  } while (0)
+
+static void expect_near(const float *got, const float *want, size_t n, float tol, const char *what) {
+  double rms = 0;
+  for (size_t i = 0; i < n; ++i) rms += double(want[i]) * want[i];
+  rms = n ? std::sqrt(rms / n) : 0;
+  double worst = 0;
+  for (size_t i = 0; i < n; ++i) {
+    const double scale = std::max(std::fabs(double(want[i])), rms);
+    const double err   = std::fabs(double(got[i]) - want[i]) / (scale > 0 ? scale : 1);
+    if (!(err <= worst)) worst = err;  // NaN sticks
+  }
+  ++g_checks;
+  if (!(worst <= tol)) {
+    ++g_failed;
+    std::printf("  FAILED %s: max rel err %.3g > %.3g over %zu values\n", what, worst, double(tol), n);
+  }
+}
+static void expect_near(const vec_t &got, const vec_t &want, float tol, const char *what) {
+  EXPECT(got.size() >= want.size());
+  if (got.size() >= want.size()) expect_near(got.data(), want.data(), want.size(), tol, what);
+}
+
+static vec_t random_vec(size_t n, unsigned seed, float lo = -1.f, float hi = 1.f) {
+  std::mt19937 gen(seed);
+  std::uniform_real_distribution<float> dist(lo, hi);
+  vec_t v(n);
+  for (auto &x : v) x = dist(gen);
+  return v;
+}
+static tensor_t random_tensor(size_t samples, size_t len, unsigned seed) {
+  tensor_t t(samples);
+  for (size_t s = 0; s < samples; ++s) t[s] = random_vec(len, seed + 7919u * unsigned(s));
+  return t;
+}
+static std::vector<float> flat(const tensor_t &t) {
+  std::vector<float> f;
+  for (auto &r : t) f.insert(f.end(), r.begin(), r.end());
+  return f;
+}
+
+// ---------------------------------------------------------------- known answers
+static void conv_with_stride() {
+  std::puts("convolutional.with_stride");
+  convolutional_layer l(5, 5, 3, 1, 1, padding::valid, true, 2, 2);
+  tensor_t in{{0, 1, 2, 3, 4, 1, 2, 3, 4, 5, 2, 3, 4, 5, 6, 3, 4, 5, 6, 7, 4, 5, 6, 7, 8}};
+  tensor_t weight{vec_t(9, 0.5f)}, bias{{0.5f}};
+  tensor_t out{vec_t(4)}, out_grad{{-1, 2, 3, 0}};
+  tensor_t in_grad{vec_t(25)}, weight_grad{vec_t(9, 0.f)}, bias_grad{vec_t(1, 0.f)};
+  std::vector<tensor_t *> in_data{&in, &weight, &bias}, out_data{&out};
+  std::vector<tensor_t *> og{&out_grad}, ig{&in_grad, &weight_grad, &bias_grad};
+  l.forward_propagation(in_data, out_data);
+  expect_near(out[0], {9.5f, 18.5f, 18.5f, 27.5f}, 1e-6f, "forward");
+  l.back_propagation(in_data, out_data, og, ig);
+  expect_near(in_grad[0], {-0.5f, -0.5f, 0.5f, 1, 1, -0.5f, -0.5f, 0.5f, 1, 1, 1, 1, 2, 1, 1,
+                           1.5f, 1.5f, 1.5f, 0, 0, 1.5f, 1.5f, 1.5f, 0, 0}, 1e-6f, "dX");
+  expect_near(weight_grad[0], {10, 14, 18, 14, 18, 22, 18, 22, 26}, 1e-6f, "dW");
+  expect_near(bias_grad[0], {4}, 1e-6f, "db");
+  // a second backward pass adds into dW/db and overwrites dX, as the reference's += does
+  l.back_propagation(in_data, out_data, og, ig);
+  expect_near(weight_grad[0], {20, 28, 36, 28, 36, 44, 36, 44, 52}, 1e-6f, "dW accumulates");
+  expect_near(bias_grad[0], {8}, 1e-6f, "db accumulates");
+  EXPECT(std::fabs(in_grad[0][12] - 2.f) < 1e-6f);
+}
+
+static void fc_forward() {
+  std::puts("fully_connected.forward");
+  fully_connected_layer l(4, 2);
+  tensor_t in{{0, 1, 2, 3}}, w{vec_t(8, 1.f)}, b{vec_t(2, 0.5f)}, out{vec_t(2)};
+  std::vector<tensor_t *> in_data{&in, &w, &b}, out_data{&out};
+  l.forward_propagation(in_data, out_data);
+  expect_near(out[0], {6.5f, 6.5f}, 1e-6f, "forward");
+  fully_connected_layer nb(4, 2, false);
+  std::vector<tensor_t *> in_nb{&in, &w};
+  nb.forward_propagation(in_nb, out_data);
+  expect_near(out[0], {6.f, 6.f}, 1e-6f, "forward without bias");
+}
+
+static void max_pool_kats() {
+  std::puts("max_pool.forward / forward_padding_same / backward");
+  const vec_t image{0, 1, 2, 3, 8, 7, 5, 6, 4, 3, 1, 2, 0, -1, -2, -3};
+  {
+    max_pooling_layer l(4, 4, 1, 2);
+    tensor_t in{image}, out{vec_t(4)};
+    std::vector<tensor_t *> in_data{&in}, out_data{&out};
+    l.forward_propagation(in_data, out_data);
+    expect_near(out[0], {8, 6, 4, 2}, 0.f, "forward");
+    tensor_t out_grad{{1, 2, 3, 4}}, in_grad{vec_t(16, -1.f)};
+    std::vector<tensor_t *> og{&out_grad}, ig{&in_grad};
+    l.back_propagation(in_data, out_data, og, ig);
+    expect_near(in_grad[0], {0, 0, 0, 0, 1, 0, 0, 2, 3, 0, 0, 4, 0, 0, 0, 0}, 0.f, "backward");
+  }
+  {
+    max_pooling_layer l(4, 4, 1, 2, 2, 1, 1, false, padding::same);
+    tensor_t in{image}, out{vec_t(16)};
+    std::vector<tensor_t *> in_data{&in}, out_data{&out};
+    l.forward_propagation(in_data, out_data);
+    expect_near(out[0], {8, 7, 6, 6, 8, 7, 6, 6, 4, 3, 2, 2, 0, -1, -2, -3}, 0.f, "padding same");
+  }
+  {
+    max_pooling_layer l(4, 4, 1, 2, 1, 2, 1, false);  // forward_stride_x
+    tensor_t in{image}, out{vec_t(8)};
+    std::vector<tensor_t *> in_data{&in}, out_data{&out};
+    l.forward_propagation(in_data, out_data);
+    expect_near(out[0], {1, 3, 8, 6, 4, 2, 0, -2}, 0.f, "stride x");
+  }
+}
+
+struct opt_case {
+  const char *name;
+  vec_t w, g, first, second;
+};
+template <typename Opt>
+static void run_opt(const opt_case &c) {
+  Opt o;
+  vec_t w = c.w;
+  o.update(c.g, w, false);
+  expect_near(w, c.first, 2e-2f, c.name);   // the reference's own tolerance is 1e-3 absolute
+  for (size_t i = 0; i < w.size(); ++i) EXPECT(std::fabs(w[i] - c.first[i]) < 1e-3f);
+  o.update(c.g, w, false);
+  for (size_t i = 0; i < w.size(); ++i) EXPECT(std::fabs(w[i] - c.second[i]) < 1e-3f);
+}
+static void optimizer_kats() {
+  std::puts("optimizers (two consecutive updates)");
+  const vec_t g1{1.0f, -3.24f, -0.6f, 2.79f, 1.82f}, g2{6.45f, -3.24f, -0.6f, 2.79f, 1.82f},
+    g3{-2.24f, -3.24f, 0.6f, 0.39f, 0.82f};
+  run_opt<adagrad>({"adagrad", {0.2f, 0.4f, 0.006f, -0.77f, -0.01f}, g1,
+                    {0.19f, 0.41f, 0.016f, -0.78f, -0.02f}, {0.1829f, 0.417f, 0.023f, -0.787f, -0.027f}});
+  run_opt<RMSprop>({"rmsprop", {-0.021f, 1.03f, -0.05f, -0.749f, 0.009f}, g1,
+                    {-0.022f, 1.031f, -0.049f, -0.75f, 0.008f}, {-0.0227f, 1.0317f, -0.0482f, -0.7507f, 0.0072f}});
+  run_opt<adam>({"adam", {1.0f, 0.081f, -0.6201f, 0.96f, -0.007f}, g2,
+                 {0.9992f, 0.0817f, -0.6193f, 0.9592f, -0.0077f}, {0.9983f, 0.0826f, -0.6184f, 0.9583f, -0.0086f}});
+  run_opt<adamax>({"adamax", {1.0f, 0.081f, -0.6201f, 0.96f, -0.007f}, g2,
+                   {0.998f, 0.083f, -0.6181f, 0.958f, -0.009f}, {0.996f, 0.085f, -0.6161f, 0.956f, -0.0109f}});
+  run_opt<gradient_descent>({"sgd", {-0.001f, -0.9f, 0.005f, -0.74f, 0.003f}, g3,
+                             {0.0214f, -0.8676f, -0.001f, -0.7439f, -0.0052f}, {0.0438f, -0.8352f, -0.007f, -0.7478f, -0.0134f}});
+  run_opt<momentum>({"momentum", {-0.001f, -0.9f, 0.005f, -0.74f, 0.003f}, g3,
+                     {0.0214f, -0.8676f, -0.001f, -0.7439f, -0.0052f}, {0.0639f, -0.806f, -0.0124f, -0.7513f, -0.0207f}});
+  run_opt<nesterov_momentum>({"nesterov", {0.1f, 0.3f, 0.005f, -0.74f, -0.008f}, g1,
+                              {0.081f, 0.3615f, 0.0164f, -0.793f, -0.0425f}, {0.0539f, 0.4493f, 0.0326f, -0.8686f, -0.0919f}});
+  // adam's powers advance once per update() call, like the reference's members
+  adam a;
+  vec_t w(3, 0.f);
+  a.update(vec_t(3, 1.f), w, false);
+  EXPECT(std::fabs(a.b1_t - 0.81f) < 1e-6f && std::fabs(a.b2_t - 0.998001f) < 1e-6f);
+}
+
+// ------------------------------------------------- operators against the oracle
+static void conv_ops_vs_oracle() {
+  std::puts("Conv2dOp / Conv2dGradOp through OpKernelContext vs oracle (same, 3->5 ch, batch 3)");
+  bool tbl[3 * 5];
+  for (int i = 0; i < 15; ++i) tbl[i] = (i % 4) != 1;
+  convolutional_layer l(9, 7, 3, 3, 3, 5, core::connection_table(tbl, 3, 5), padding::same);
+  const core::conv_params &p = l.params();
+  const size_t n = 3;
+  tensor_t in = random_tensor(n, p.in.size(), 11), w{random_vec(p.weight.size(), 12)},
+           b{random_vec(5, 13)}, out(n, vec_t(p.out.size())), dy = random_tensor(n, p.out.size(), 14);
+  tensor_t dx(n, vec_t(p.in.size())), dw(n, vec_t(p.weight.size(), 0.f)), db(n, vec_t(5, 0.f));
+  std::vector<tensor_t *> in_data{&in, &w, &b}, out_data{&out}, og{&dy}, ig{&dx, &dw, &db};
+
+  core::conv_params params = p;
+  core::OpKernelConstruction construction(nullptr, &params);
+  Conv2dOp fwd(construction);
+  Conv2dGradOp bwd(construction);
+  core::OpKernelContext ctx;
+  ctx.setEngine(core::backend_t::hip);
+  ctx.set_in_out(in_data, out_data);
+  fwd.compute(ctx);
+  ctx.set_in_out(in_data, out_data, og, ig);
+  bwd.compute(ctx);
+
+  uint8_t tbl8[15];
+  for (int i = 0; i < 15; ++i) tbl8[i] = tbl[i];
+  tdo_conv_desc d{9, 7, 3, 3, 3, 5, 1, 1, 1, 1, 1, 1, tbl8};
+  std::vector<float> x = flat(in), gy = flat(dy), y(n * p.out.size()), gx(n * p.in.size()),
+                     gw(p.weight.size()), gb(5);
+  EXPECT(tdo_conv2d_fwd(&d, n, x.data(), w[0].data(), b[0].data(), y.data()) == 0);
+  EXPECT(tdo_conv2d_bwd(&d, n, x.data(), w[0].data(), gy.data(), gx.data(), gw.data(), gb.data()) == 0);
+  expect_near(flat(out).data(), y.data(), y.size(), 1e-4f, "Y");
+  expect_near(flat(dx).data(), gx.data(), gx.size(), 1e-4f, "dX");
+  expect_near(dw[0].data(), gw.data(), gw.size(), 1e-4f, "dW (slot 0 = sum over the batch)");
+  expect_near(db[0].data(), gb.data(), gb.size(), 1e-4f, "db");
+  for (size_t s = 1; s < n; ++s)
+    for (float v : dw[s]) EXPECT(v == 0.f);
+
+  // any other engine is refused like the reference refuses an unknown one
+  ctx.setEngine(core::backend_t::avx);
+  bool threw = false;
+  try {
+    bwd.compute(ctx);
+  } catch (const nn_error &e) {
+    threw = std::string(e.what()).find("Not supported engine") != std::string::npos;
+  }
+  EXPECT(threw);
+}
+
+static void fc_pool_ops_vs_oracle() {
+  std::puts("FullyConnectedGradOp / MaxPoolGradOp / AvePoolGradOp vs oracle");
+  {
+    const size_t n = 5, in = 37, out = 19;
+    core::fully_params params;
+    params.in_size_ = in; params.out_size_ = out; params.has_bias_ = true;
+    FullyConnectedGradOp op(core::OpKernelConstruction(nullptr, &params));
+    tensor_t x = random_tensor(n, in, 21), w{random_vec(in * out, 22)}, b{vec_t(out)},
+             y(n, vec_t(out)), dy = random_tensor(n, out, 23);
+    tensor_t dx(n, vec_t(in)), dw(n, vec_t(in * out, 0.f)), db(n, vec_t(out, 0.f));
+    std::vector<tensor_t *> in_data{&x, &w, &b}, out_data{&y}, og{&dy}, ig{&dx, &dw, &db};
+    core::OpKernelContext ctx;
+    ctx.set_in_out(in_data, out_data, og, ig);
+    op.compute(ctx);
+    std::vector<float> gx(n * in), gw(in * out), gb(out);
+    EXPECT(tdo_fc_bwd(in, out, 1, n, flat(x).data(), w[0].data(), flat(dy).data(), gx.data(), gw.data(),
+                      gb.data()) == 0);
+    expect_near(flat(dx).data(), gx.data(), gx.size(), 1e-4f, "fc dX");
+    expect_near(dw[0].data(), gw.data(), gw.size(), 1e-4f, "fc dW");
+    expect_near(db[0].data(), gb.data(), gb.size(), 1e-4f, "fc db");
+  }
+  {
+    const size_t n = 4;
+    max_pooling_layer l(11, 9, 3, 3, 3, 2, 2, true);  // overlapping windows, ceil mode
+    tdo_pool_desc d{11, 9, 3, 3, 3, 2, 2, 0, 1};
+    const size_t isz = 11 * 9 * 3, osz = size_t(tdo_pool_out_w(&d)) * tdo_pool_out_h(&d) * 3;
+    EXPECT(l.out_shape()[0].size() == osz);
+    tensor_t x = random_tensor(n, isz, 31), y(n, vec_t(osz)), dy = random_tensor(n, osz, 32), dx(n, vec_t(isz));
+    std::vector<tensor_t *> in_data{&x}, out_data{&y}, og{&dy}, ig{&dx};
+    l.forward_propagation(in_data, out_data);
+    l.back_propagation(in_data, out_data, og, ig);
+    std::vector<float> wy(n * osz), wx(n * isz);
+    std::vector<int64_t> arg(n * osz);
+    EXPECT(tdo_maxpool_fwd(&d, n, flat(x).data(), wy.data(), arg.data()) == 0);
+    EXPECT(tdo_maxpool_bwd(&d, n, flat(dy).data(), arg.data(), wx.data()) == 0);
+    expect_near(flat(y).data(), wy.data(), wy.size(), 0.f, "max-pool Y (exact)");
+    expect_near(flat(dx).data(), wx.data(), wx.size(), 0.f, "max-pool dX (exact)");
+  }
+  {
+    const size_t n = 3, c = 4;
+    average_pooling_layer l(8, 6, c, 2);
+    tdo_pool_desc d{8, 6, 4, 2, 2, 2, 2, 0, 0};
+    const size_t isz = 8 * 6 * c, osz = 4 * 3 * c;
+    tensor_t x = random_tensor(n, isz, 41), w{random_vec(c, 42)}, b{random_vec(c, 43)}, y(n, vec_t(osz)),
+             dy = random_tensor(n, osz, 44), dx(n, vec_t(isz)), dw(n, vec_t(c, 0.f)), db(n, vec_t(c, 0.f));
+    std::vector<tensor_t *> in_data{&x, &w, &b}, out_data{&y}, og{&dy}, ig{&dx, &dw, &db};
+    l.forward_propagation(in_data, out_data);
+    l.back_propagation(in_data, out_data, og, ig);
+    std::vector<float> wy(n * osz), wx(n * isz), ww(c), wb(c);
+    EXPECT(tdo_avepool_fwd(&d, n, flat(x).data(), w[0].data(), b[0].data(), wy.data()) == 0);
+    EXPECT(tdo_avepool_bwd(&d, n, flat(x).data(), w[0].data(), flat(dy).data(), wx.data(), ww.data(),
+                           wb.data()) == 0);
+    expect_near(flat(y).data(), wy.data(), wy.size(), 1e-4f, "ave-pool Y");
+    expect_near(flat(dx).data(), wx.data(), wx.size(), 1e-4f, "ave-pool dX");
+    expect_near(dw[0].data(), ww.data(), c, 1e-4f, "ave-pool dW");
+    expect_near(db[0].data(), wb.data(), c, 1e-4f, "ave-pool db");
+    bool threw = false;
+    try {
+      average_pooling_layer bad(7, 6, 1, 2);
+    } catch (const nn_error &) {
+      threw = true;
+    }
+    EXPECT(threw);
+  }
+}
+
+// -------------------------------------------------- network<sequential>::fit
+template <typename Opt>
+static void net_fit_vs_oracle(const char *name, int opt_kind) {
+  std::printf("network<sequential>::fit<cross_entropy_multiclass> with %s vs oracle (short last batch)\n", name);
+  network<sequential> nn;
+  nn << convolutional_layer(12, 12, 3, 1, 4, padding::same) << tanh_layer()
+     << max_pooling_layer(12, 12, 4, 2) << convolutional_layer(6, 6, 3, 4, 6) << relu_layer()
+     << average_pooling_layer(4, 4, 6, 2) << fully_connected_layer(24, 10) << softmax_layer();
+  EXPECT(nn.layer_size() == 8);
+  EXPECT(nn.in_data_size() == 144 && nn.out_data_size() == 10);
+
+  tdo_layer L[8] = {};
+  L[0].kind = TDO_L_CONV; L[0].conv = tdo_conv_desc{12, 12, 1, 3, 3, 4, 1, 1, 1, 1, 1, 1, nullptr};
+  L[1].kind = TDO_L_ACT;  L[1].act = TDO_ACT_TANH;
+  L[2].kind = TDO_L_MAXPOOL; L[2].pool = tdo_pool_desc{12, 12, 4, 2, 2, 2, 2, 0, 0};
+  L[3].kind = TDO_L_CONV; L[3].conv = tdo_conv_desc{6, 6, 4, 3, 3, 6, 1, 1, 1, 1, 0, 1, nullptr};
+  L[4].kind = TDO_L_ACT;  L[4].act = TDO_ACT_RELU;
+  L[5].kind = TDO_L_AVEPOOL; L[5].pool = tdo_pool_desc{4, 4, 6, 2, 2, 2, 2, 0, 0};
+  L[6].kind = TDO_L_FC; L[6].fc_in = 24; L[6].fc_out = 10; L[6].fc_bias = 1;
+  L[7].kind = TDO_L_ACT;  L[7].act = TDO_ACT_SOFTMAX;
+  const size_t batch = 4, samples = 10;  // batches of 4, 4, 2
+  tdo_net *ref = tdo_net_create(L, 8, batch);
+  EXPECT(ref != nullptr);
+  for (int i = 0; i < 8; ++i) {
+    const size_t nw = tdo_net_weight_size(ref, i), nb = tdo_net_bias_size(ref, i);
+    if (nw) {
+      vec_t w = random_vec(nw, 100 + i, -0.3f, 0.3f);
+      std::copy(w.begin(), w.end(), tdo_net_weight(ref, i));
+      nn.set_weights(i, 0, w);
+    }
+    if (nb) {
+      vec_t b = random_vec(nb, 200 + i, -0.1f, 0.1f);
+      std::copy(b.begin(), b.end(), tdo_net_bias(ref, i));
+      nn.set_weights(i, 1, b);
+    }
+  }
+  std::vector<vec_t> inputs = random_tensor(samples, 144, 51);
+  std::vector<label_t> labels(samples);
+  for (size_t i = 0; i < samples; ++i) labels[i] = (i * 7) % 10;
+
+  Opt opt;
+  int batches = 0, epochs = 0;
+  std::vector<vec_t> targets(samples, vec_t(10, 0.f));
+  for (size_t i = 0; i < samples; ++i) targets[i][labels[i]] = 1.f;
+  EXPECT((nn.fit<cross_entropy_multiclass>(opt, inputs, targets, batch, 2, [&]() { ++batches; },
+                                           [&]() { ++epochs; })));
+  EXPECT(batches == 6 && epochs == 2);
+
+  tdo_opt o;
+  tdo_opt_default(&o, opt_kind);
+  for (int e = 0; e < 2; ++e)
+    for (size_t i = 0; i < samples; i += batch) {
+      const size_t n = std::min(batch, samples - i);
+      tensor_t xb(inputs.begin() + i, inputs.begin() + i + n), tb(targets.begin() + i, targets.begin() + i + n);
+      EXPECT(tdo_net_train_step(ref, &o, TDO_LOSS_CE_MULTICLASS, n, flat(xb).data(), flat(tb).data(), 1) == 0);
+    }
+  for (int i = 0; i < 8; ++i) {
+    const size_t nw = tdo_net_weight_size(ref, i), nb = tdo_net_bias_size(ref, i);
+    if (nw) expect_near(nn.weights(i, 0).data(), tdo_net_weight(ref, i), nw, 1e-4f, "weights after fit");
+    if (nb) expect_near(nn.weights(i, 1).data(), tdo_net_bias(ref, i), nb, 1e-4f, "biases after fit");
+  }
+  vec_t y = nn.predict(inputs[3]);
+  EXPECT(tdo_net_forward(ref, 1, inputs[3].data()) == 0);
+  expect_near(y.data(), tdo_net_layer_out(ref, 7), 10, 1e-4f, "predict");
+
+  // train() with labels builds the same one-hot targets; mismatched sizes are refused
+  std::vector<label_t> too_few(samples - 1);
+  EXPECT(!(nn.train<cross_entropy_multiclass>(opt, inputs, too_few, batch, 1)));
+  EXPECT((nn.train<cross_entropy_multiclass>(opt, inputs, labels, batch, 1)));
+  tdo_net_destroy(ref);
+}
+
+int main() {
+  try {
+    conv_with_stride();
+    fc_forward();
+    max_pool_kats();
+    optimizer_kats();
+    conv_ops_vs_oracle();
+    fc_pool_ops_vs_oracle();
+    net_fit_vs_oracle<gradient_descent>("gradient_descent", TDO_OPT_SGD);
+    net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM);
+  } catch (const std::exception &e) {
+    std::printf("EXCEPTION: %s\n", e.what());
+    return 2;
+  }
+  std::printf("%d checks, %d failed\n", g_checks, g_failed);
+  return g_failed ? 1 : 0;
+}

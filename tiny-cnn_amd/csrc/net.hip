@@ -272,6 +272,17 @@ int tdh_net_set_param(tdh_net *net, int layer, int which, const float *host_src)
   TDH_CHECK_ARG(n == 0 || (dst && host_src), "tdh_net_set_param: no such parameter");
   return tdh_memcpy_h2d(dst, host_src, n * sizeof(float));
 }
+int tdh_net_reset_optimizer(tdh_net *net) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net != nullptr, "tdh_net_reset_optimizer: null net");
+  for (tdh_net::Layer &L : net->layers) {
+    float *state[4]      = {L.s0w, L.s1w, L.s0b, L.s1b};
+    const size_t size[4] = {L.w_size, L.w_size, L.b_size, L.b_size};
+    for (int i = 0; i < 4; ++i)
+      if (state[i] && size[i]) TDH_TRY(launch_fill_zero(state[i], size[i] * sizeof(float)));
+  }
+  return TDH_OK;
+}
 int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst) {
   TDH_REQUIRE_INIT();
   const float *src = tdh_net_param(net, layer, which);
