@@ -150,6 +150,36 @@ def run_workload(T, wl, steps, warmup, profile_steps):
             "samples_per_s": wl.samples / (ms_per_step * 1e-3), "kernels": kernels}
 
 
+def copy_yardstick(T, mib=256, reps=5):
+    """Achieved bandwidth of the library's plain copy kernel (reads and writes `mib` MiB each):
+    what a bandwidth-bound kernel can reach on this device, and the dispatch of known size
+    that hardware byte counters are scaled by."""
+    n = mib << 20
+    a, b = T.DevBuf((n // 4,), zero=True), T.DevBuf((n // 4,))
+    T.copy_d2d(b, a)
+    T.sync()
+    e0, e1 = T.Event(), T.Event()
+    e0.record()
+    for _ in range(reps):
+        T.copy_d2d(b, a)
+    e1.record()
+    T.sync()
+    us = e1.elapsed_ms_since(e0) * 1e3 / reps
+    return {"kernel": "copy_kernel", "read_bytes": n, "write_bytes": n, "avg_launch_us": round(us, 2),
+            "GB/s": round(2 * n / (us * 1e-6) / 1e9, 1)}
+
+
+def measured_traffic(tag):
+    """HBM bytes per launch of kernel `tag` from hardware counters, when a counter run of this
+    workload has been recorded in profiles/hbm_traffic.json (null otherwise)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            rec = json.load(f)["kernels"].get(tag)
+        return rec and rec["hbm_bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        return None
+
+
 def cpu_baseline(W, name, budget_s=20.0):
     """Reference CPU figure on a bounded sample of the same workload."""
     from oracle import oracle as O
@@ -246,9 +276,12 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": wl.config,
         "device": {"name": dev_name, "compute_units": cus},
-        "roofline": res["kernels"][0] if res["kernels"] else None,
+        "roofline": dict(res["kernels"][0]) if res["kernels"] else None,
         "kernels": res["kernels"],
     }
+    if out["roofline"]:
+        out["roofline"]["traffic"] = measured_traffic(out["roofline"]["kernel"])
+    out["copy_yardstick"] = copy_yardstick(T)
     if wl.config.get("flop_per_step"):
         out["step_tflops"] = round(wl.config["flop_per_step"] / (res["ms_per_step"] * 1e-3) / 1e12, 3)
     del wl

@@ -365,3 +365,18 @@ def test_optimizer_grad_scale_and_state_checks(T, O):
     assert np.array_equal(w.numpy(), np.array([-0.25, 0.5, -1.0], np.float32))
     with pytest.raises(T.TdhError, match="state"):
         T.opt_update(T.opt_desc("adam"), 3, w, w, None, None)
+
+
+@pytest.mark.parametrize("n,dst_off,src_off", [(1, 0, 0), (1023, 0, 0), (4096, 4, 8), (100003, 12, 0),
+                                               (1 << 20, 0, 4)])
+def test_device_copy_is_exact(T, n, dst_off, src_off):
+    """tdh_memcpy_d2d (a copy kernel): every word arrives, nothing outside the range is written."""
+    rng = np.random.default_rng(n)
+    src = rng.integers(0, 2**32, n + 8, dtype=np.uint32)
+    dst0 = rng.integers(0, 2**32, n + 8, dtype=np.uint32)
+    s, d = T.to_device(src, np.uint32), T.to_device(dst0, np.uint32)
+    T.copy_d2d(d, s, nbytes=4 * n, dst_offset=dst_off, src_offset=src_off)
+    got = d.numpy()
+    want = dst0.copy()
+    want[dst_off // 4: dst_off // 4 + n] = src[src_off // 4: src_off // 4 + n]
+    assert np.array_equal(got, want)

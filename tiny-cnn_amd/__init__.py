@@ -164,6 +164,16 @@ class DevBuf:
             pass
 
 
+def copy_d2d(dst, src, nbytes=None, dst_offset=0, src_offset=0):
+    """Device-to-device copy on the library's stream (a copy kernel for 4-byte-aligned sizes)."""
+    n = src.nbytes if nbytes is None else int(nbytes)
+    if n + dst_offset > dst.nbytes or n + src_offset > src.nbytes:
+        raise ValueError("copy_d2d: range exceeds a buffer")
+    check(lib().tdh_memcpy_d2d(C.c_void_p(dst.ptr.value + dst_offset),
+                               C.c_void_p(src.ptr.value + src_offset), C.c_size_t(n)),
+          "tdh_memcpy_d2d")
+
+
 def to_device(a, dtype=np.float32):
     a = np.ascontiguousarray(a, dtype=dtype)
     return DevBuf(a.shape, dtype).upload(a)

@@ -115,6 +115,7 @@ int pool_out_length(int in_length, int window, int stride, int ceil_mode, int pa
 // ------------------------------------------------- internal launchers (device ptrs)
 // elementwise.hip
 int launch_fill_zero(void *p, size_t bytes);
+int launch_copy(void *dst, const void *src, size_t bytes);  // bytes % 4 == 0
 int launch_act_fwd(int kind, int batch, int len, const float *x, float *y);
 int launch_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx);
 int launch_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);

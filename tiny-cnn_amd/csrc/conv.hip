@@ -211,65 +211,88 @@ mask_weights_kernel(const float *__restrict__ src, const uint8_t *__restrict__ t
 
 // dX for convolutions with very few input channels (the first layer of an image network:
 // M = Cin = 1..4 would leave 7/8 of every 32-row MFMA block empty). Direct form on the vector
-// ALUs, stride 1: a workgroup owns a band of input rows of one image, stages the dY rows that
-// can reach it (with zero halo) in LDS eight output channels at a time, and every thread
-// accumulates its pixels for all Cin channels. Filter taps are wave-uniform reads.
+// ALUs, stride 1. A workgroup of four waves owns a band of input rows of one image: lane l of
+// EVERY wave owns the same DXS_PX adjacent pixels of the band, and the waves split the output
+// channels between them (the pixels alone would not fill the chip), so the four partial sums
+// are added through LDS at the end, always in wave order. dY rows that can reach the band are
+// staged in LDS (zero halo) DXS_CO_CHUNK channels at a time, the next chunk travelling in
+// registers while the current one is used; a lane reads its 4+S-1 tile values of a filter row
+// as 16-byte words and reuses them for all S taps and Cin channels.
 constexpr int DXS_MAX_CIN  = 4;
-constexpr int DXS_CO_CHUNK = 8;
-constexpr int DXS_PX       = 4;  // pixels per thread
+constexpr int DXS_WAVES    = 4;
+constexpr int DXS_CPW      = 2;                      // output channels per wave in a chunk
+constexpr int DXS_CO_CHUNK = DXS_WAVES * DXS_CPW;
+constexpr int DXS_PX       = 4;                      // adjacent pixels per lane
+constexpr int DXS_NT       = 64 * DXS_WAVES;
+constexpr int DXS_MAX_STAGE = 20;                    // staged tile elements per thread and chunk
 
-// KR, KS: compile-time window (0 = use the run-time g.R, g.S)
-template <int KR, int KS>
-__global__ void __launch_bounds__(256)
+struct DxsPlan {
+  int tile_rows, bands, gw, trows, tcols;  // gw: pixel groups per row; tile = [trows][tcols]
+  FastDiv div_gw, div_tcols, div_tile;
+  size_t lds_bytes;
+};
+
+// KR, KS: compile-time window (0 = use the run-time g.R, g.S); CIN: input channels computed
+template <int KR, int KS, int CIN>
+__global__ void __launch_bounds__(DXS_NT)
 conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__ w,
-                         float *__restrict__ dx, const ConvGeom g, const int tile_rows,
-                         const int bands, const ActGrad ag) {
-  extern __shared__ float smem[];  // dY tile [DXS_CO_CHUNK][trows][tcols], then weights
+                         float *__restrict__ dx, const ConvGeom g, const DxsPlan p,
+                         const ActGrad ag) {
+  extern __shared__ __align__(16) float smem[];
   const int R = KR ? KR : g.R, S = KS ? KS : g.S;
-  const int img   = blockIdx.x / bands;
-  const int y0    = (blockIdx.x - img * bands) * tile_rows;
-  const int rows  = min(tile_rows, g.H - y0);
-  const int trows = tile_rows + R - 1, tcols = g.W + S - 1;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int img = blockIdx.x / p.bands;
+  const int y0  = (blockIdx.x - img * p.bands) * p.tile_rows;
+  const int tsz = p.trows * p.tcols, rs = R * S;
   const int oy0 = y0 + g.pad_h - (R - 1), ox0 = g.pad_w - (S - 1);
-  const int ohw = g.OH * g.OW, rs = R * S;
+  const int ohw = g.OH * g.OW;
   const float *dy_img = dy + static_cast<size_t>(img) * g.Kc * ohw;
-  float *tile = smem;
-  float4 *wl  = reinterpret_cast<float4 *>(smem + ((DXS_CO_CHUNK * trows * tcols + 3) & ~3));
+  float *tile = smem;                                                  // [DXS_CO_CHUNK][tsz]
+  float4 *wl  = reinterpret_cast<float4 *>(smem + DXS_CO_CHUNK * tsz);  // [DXS_CO_CHUNK][rs]
 
-  float acc[DXS_MAX_CIN][DXS_PX];
+  // this lane's pixels: row prow of the band, columns 4*grp .. 4*grp+3
+  uint32_t prow, grp;
+  p.div_gw.divmod(lane, prow, grp);
+  const bool lane_live = static_cast<int>(prow) < p.tile_rows;
+  const int toff       = lane_live ? prow * p.tcols + 4 * grp : 0;
+
+  float acc[CIN][DXS_PX];
 #pragma unroll
-  for (int c = 0; c < DXS_MAX_CIN; ++c)
+  for (int c = 0; c < CIN; ++c)
 #pragma unroll
     for (int i = 0; i < DXS_PX; ++i) acc[c][i] = 0.0f;
 
-  // pixel i of this thread: p = tid + 256*i -> (py, px); its tile offset for tap (R-1, S-1)
-  int toff[DXS_PX];
-  bool live[DXS_PX];
-#pragma unroll
-  for (int i = 0; i < DXS_PX; ++i) {
-    const int p  = threadIdx.x + 256 * i;
-    const int py = p / g.W, px = p - py * g.W;
-    live[i] = py < rows;
-    toff[i] = live[i] ? py * tcols + px : 0;
-  }
-
-  for (int co0 = 0; co0 < g.Kc; co0 += DXS_CO_CHUNK) {
+  // staging plan: element e = tid + DXS_NT*j of the chunk tile -> global offset or -1
+  float stage[DXS_MAX_STAGE];
+  auto fetch = [&](int co0) {
     const int nco = min(DXS_CO_CHUNK, g.Kc - co0);
-    __syncthreads();
-    for (int e = threadIdx.x; e < nco * trows * tcols; e += 256) {
-      const int c = e / (trows * tcols);
-      const int r = (e - c * trows * tcols) / tcols;
-      const int q = e - c * trows * tcols - r * tcols;
-      const int oy = oy0 + r, ox = ox0 + q;
+#pragma unroll
+    for (int j = 0; j < DXS_MAX_STAGE; ++j) {
+      const uint32_t e = tid + DXS_NT * j;
+      uint32_t c, rem, r, q;
+      p.div_tile.divmod(e, c, rem);
+      p.div_tcols.divmod(rem, r, q);
+      const int oy = oy0 + static_cast<int>(r), ox = ox0 + static_cast<int>(q);
       float v = 0.0f;
-      if (static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
+      if (static_cast<int>(c) < nco && static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
           static_cast<unsigned>(ox) < static_cast<unsigned>(g.OW))
         v = dy_img[(co0 + c) * ohw + oy * g.OW + ox];
-      tile[e] = v;
+      stage[j] = v;
     }
-    // weights of the chunk as [c][tap] -> (w[ci=0..3]); tap stored flipped so that the
+  };
+
+  fetch(0);
+  for (int co0 = 0; co0 < g.Kc; co0 += DXS_CO_CHUNK) {
+    const int nco = min(DXS_CO_CHUNK, g.Kc - co0);
+    __syncthreads();  // the previous chunk has been consumed
+#pragma unroll
+    for (int j = 0; j < DXS_MAX_STAGE; ++j) {
+      const int e = tid + DXS_NT * j;
+      if (e < DXS_CO_CHUNK * tsz) tile[e] = stage[j];
+    }
+    // weights of the chunk as [c][tap] -> (w[ci=0..3]); taps stored flipped so that the
     // inner loops walk the tile forwards
-    for (int e = threadIdx.x; e < nco * rs; e += 256) {
+    for (int e = tid; e < nco * rs; e += DXS_NT) {
       const int c = e / rs, t = e - c * rs;
       const float *wc = w + (static_cast<size_t>(co0 + c) * g.C) * rs + (rs - 1 - t);
       float4 v;
@@ -280,57 +303,108 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
       wl[e] = v;
     }
     __syncthreads();
-    for (int c = 0; c < nco; ++c) {
-      const float *t = tile + c * trows * tcols;
+    if (co0 + DXS_CO_CHUNK < g.Kc) fetch(co0 + DXS_CO_CHUNK);  // in flight during the math
+
 #pragma unroll
-      for (int fy = 0; fy < (KR ? KR : 1); ++fy)
-        for (int fyy = fy; fyy < R; fyy += (KR ? R : 1)) {
+    for (int cc = 0; cc < DXS_CPW; ++cc) {
+      const int c = wv * DXS_CPW + cc;
+      if (c >= nco) break;
+      const float *t   = tile + c * tsz + toff;
+      const float4 *wc = wl + c * rs;
+      if (KR != 0) {
+        constexpr int NV = (DXS_PX + (KS ? KS : 1) - 1 + 3) / 4;  // 16-byte words per filter row
 #pragma unroll
-          for (int fx = 0; fx < (KS ? KS : 1); ++fx)
-            for (int fxx = fx; fxx < S; fxx += (KS ? S : 1)) {
-              // flipped tap (fyy, fxx) reads tile[(py + fyy)][px + fxx]
-              const float4 wv = wl[c * rs + fyy * S + fxx];
+        for (int fy = 0; fy < KR; ++fy) {
+          float v[4 * NV];
 #pragma unroll
-              for (int i = 0; i < DXS_PX; ++i) {
-                const float v = t[toff[i] + fyy * tcols + fxx];
-                acc[0][i] += wv.x * v;
-                acc[1][i] += wv.y * v;
-                acc[2][i] += wv.z * v;
-                acc[3][i] += wv.w * v;
-              }
-            }
+          for (int q = 0; q < NV; ++q) {
+            const float4 f = *reinterpret_cast<const float4 *>(t + fy * p.tcols + 4 * q);
+            v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+          }
+#pragma unroll
+          for (int fx = 0; fx < KS; ++fx) {
+            const float4 wq  = wc[fy * KS + fx];
+            const float wa[4] = {wq.x, wq.y, wq.z, wq.w};
+#pragma unroll
+            for (int ci = 0; ci < CIN; ++ci)
+#pragma unroll
+              for (int i = 0; i < DXS_PX; ++i) acc[ci][i] += wa[ci] * v[i + fx];
+          }
         }
+      } else {
+        for (int fy = 0; fy < R; ++fy)
+          for (int fx = 0; fx < S; ++fx) {
+            const float4 wq  = wc[fy * S + fx];
+            const float wa[4] = {wq.x, wq.y, wq.z, wq.w};
+#pragma unroll
+            for (int i = 0; i < DXS_PX; ++i) {
+              const float v = t[fy * p.tcols + fx + i];
+#pragma unroll
+              for (int ci = 0; ci < CIN; ++ci) acc[ci][i] += wa[ci] * v;
+            }
+          }
+      }
     }
   }
-  float *dx_img = dx + static_cast<size_t>(img) * g.C * g.H * g.W;
+
+  // partial sums of the four waves -> red[wave][ci][lane*4 + i], then one fixed-order add
+  __syncthreads();
+  float *red = smem;
 #pragma unroll
-  for (int i = 0; i < DXS_PX; ++i) {
-    if (!live[i]) continue;
-    const int p  = threadIdx.x + 256 * i;
-    const int py = p / g.W, px = p - py * g.W;
+  for (int ci = 0; ci < CIN; ++ci)
+    *reinterpret_cast<float4 *>(red + (wv * CIN + ci) * (64 * DXS_PX) + lane * DXS_PX) =
+      make_float4(acc[ci][0], acc[ci][1], acc[ci][2], acc[ci][3]);
+  __syncthreads();
+  {
+    uint32_t orow, ogrp;
+    p.div_gw.divmod(tid >> 2, orow, ogrp);  // tid = lane*4 + i of the pixel it finishes
+    const int y = y0 + static_cast<int>(orow), x = 4 * static_cast<int>(ogrp) + (tid & 3);
+    if (static_cast<int>(orow) < p.tile_rows && y < g.H && x < g.W) {
+      const size_t img_off = static_cast<size_t>(img) * g.C * g.H * g.W;
 #pragma unroll
-    for (int ci = 0; ci < DXS_MAX_CIN; ++ci) {
-      if (ci >= g.C) break;
-      const size_t idx = (static_cast<size_t>(ci) * g.H + y0 + py) * g.W + px;
-      float v = acc[ci][i];
-      if (ag.kind != TDH_ACT_NONE)
-        v *= act_grad_factor(ag.kind, ag.y[static_cast<size_t>(img) * g.C * g.H * g.W + idx]);
-      dx_img[idx] = v;
+      for (int ci = 0; ci < CIN; ++ci) {
+        if (ci >= g.C) break;
+        float v = red[ci * (64 * DXS_PX) + tid];
+#pragma unroll
+        for (int k = 1; k < DXS_WAVES; ++k) v += red[(k * CIN + ci) * (64 * DXS_PX) + tid];
+        const size_t idx = img_off + (static_cast<size_t>(ci) * g.H + y) * g.W + x;
+        if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[idx]);
+        dx[idx] = v;
+      }
     }
   }
 }
 
 // true when the direct kernel applies; fills the launch geometry
-static bool small_cin_dx_plan(const ConvGeom &g, int &tile_rows, int &bands, size_t &lds_bytes) {
-  if (g.C > DXS_MAX_CIN || g.sh != 1 || g.sw != 1 || g.W > 256 * DXS_PX) return false;
-  tile_rows = (256 * DXS_PX) / g.W;
-  if (tile_rows > g.H) tile_rows = g.H;
-  // keep at least ~2 workgroups per image so that small batches still fill the chip
-  if (tile_rows > 8 && tile_rows * 2 > g.H) tile_rows = (g.H + 1) / 2;
-  bands     = ceil_div(g.H, tile_rows);
-  lds_bytes = sizeof(float) * (((DXS_CO_CHUNK * (tile_rows + g.R - 1) * (g.W + g.S - 1) + 3) & ~3) +
-                               4 * DXS_CO_CHUNK * g.R * g.S);
-  return lds_bytes <= 64 * 1024;
+static bool small_cin_dx_plan(const ConvGeom &g, DxsPlan &p) {
+  if (g.C > DXS_MAX_CIN || g.sh != 1 || g.sw != 1) return false;
+  p.gw = ceil_div(g.W, DXS_PX);
+  if (p.gw > 64) return false;
+  p.tile_rows = std::min(64 / p.gw, g.H);
+  p.bands     = ceil_div(g.H, p.tile_rows);
+  p.trows     = p.tile_rows + g.R - 1;
+  p.tcols     = (DXS_PX * p.gw + g.S - 1 + 3) & ~3;  // lanes read whole 16-byte words
+  const int tsz = p.trows * p.tcols;
+  if (DXS_CO_CHUNK * tsz > DXS_MAX_STAGE * DXS_NT) return false;
+  p.div_gw    = FastDiv(p.gw);
+  p.div_tcols = FastDiv(p.tcols);
+  p.div_tile  = FastDiv(tsz);
+  const size_t stage_floats = static_cast<size_t>(DXS_CO_CHUNK) * tsz + 4 * DXS_CO_CHUNK * g.R * g.S;
+  const size_t red_floats   = static_cast<size_t>(DXS_WAVES) * DXS_MAX_CIN * 64 * DXS_PX;
+  p.lds_bytes = sizeof(float) * std::max(stage_floats, red_floats);
+  return p.lds_bytes <= 64 * 1024;
+}
+
+template <int KR, int KS>
+static void launch_small_cin_dx(const ConvGeom &g, const DxsPlan &p, int batch, const float *dy,
+                                const float *w, float *dx, ActGrad ag) {
+  const dim3 grid(batch * p.bands), block(DXS_NT);
+  switch (KR ? g.C : DXS_MAX_CIN) {
+    case 1: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 1>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    case 2: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 2>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    case 3: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 3>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    default: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 4>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+  }
 }
 
 }  // namespace
@@ -406,19 +480,15 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
-  int tile_rows = 0, bands = 0;
-  size_t lds_bytes = 0;
-  if (dx && small_cin_dx_plan(g, tile_rows, bands, lds_bytes)) {
+  DxsPlan dxs;
+  if (dx && small_cin_dx_plan(g, dxs)) {
     ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
     if (g.R == 3 && g.S == 3)
-      hipLaunchKernelGGL((conv_dx_small_cin_kernel<3, 3>), dim3(batch * bands), dim3(256),
-                         lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
+      launch_small_cin_dx<3, 3>(g, dxs, batch, dy, w_eff, dx, dx_act);
     else if (g.R == 5 && g.S == 5)
-      hipLaunchKernelGGL((conv_dx_small_cin_kernel<5, 5>), dim3(batch * bands), dim3(256),
-                         lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
+      launch_small_cin_dx<5, 5>(g, dxs, batch, dy, w_eff, dx, dx_act);
     else
-      hipLaunchKernelGGL((conv_dx_small_cin_kernel<0, 0>), dim3(batch * bands), dim3(256),
-                         lds_bytes, ctx().stream, dy, w_eff, dx, g, tile_rows, bands, dx_act);
+      launch_small_cin_dx<0, 0>(g, dxs, batch, dy, w_eff, dx, dx_act);
     TDH_LAUNCH_CHECK();
   } else if (dx && g.sh == 1 && g.sw == 1 &&
              conv_s1_applicable(g.R, g.S, batch, g.Kc, g.C, g.OH, g.OW, g.H, g.W,

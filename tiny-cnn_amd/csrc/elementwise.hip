@@ -121,6 +121,17 @@ fill_zero_kernel(uint32_t *__restrict__ p, const size_t n4, const size_t n) {
   for (size_t j = n4 * 4 + t0; j < n; j += stride) p[j] = 0u;
 }
 
+// plain device-to-device copy: one 16-byte load and store per lane and iteration
+__global__ void __launch_bounds__(EW_THREADS)
+copy_kernel(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, const size_t n4,
+            const size_t n) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * EW_THREADS;
+  const size_t t0     = static_cast<size_t>(blockIdx.x) * EW_THREADS + threadIdx.x;
+  for (size_t i = t0; i < n4; i += stride)
+    reinterpret_cast<uint4 *>(dst)[i] = reinterpret_cast<const uint4 *>(src)[i];
+  for (size_t j = n4 * 4 + t0; j < n; j += stride) dst[j] = src[j];
+}
+
 // ------------------------------------------------------------------ softmax
 // One wave64 per sample row; reductions by butterfly shuffles (every lane ends with the
 // same value, summed in a fixed tree).
@@ -412,6 +423,16 @@ int launch_fill_zero(void *p, size_t bytes) {
   const size_t n4 = aligned16(p) ? n / 4 : 0;
   hipLaunchKernelGGL(fill_zero_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0,
                      ctx().stream, static_cast<uint32_t *>(p), n4, n);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+int launch_copy(void *dst, const void *src, size_t bytes) {
+  ProfScope prof("copy", 2.0 * static_cast<double>(bytes), WORK_BYTE);
+  const size_t n  = bytes / 4;
+  const size_t n4 = (aligned16(dst) && aligned16(src)) ? n / 4 : 0;
+  hipLaunchKernelGGL(copy_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0, ctx().stream,
+                     static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), n4, n);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }
