@@ -162,7 +162,8 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
 // conv_s1.hip: stride-1 forward / dX with LDS halo tiles (3x3 and 5x5 windows)
 bool conv_s1_applicable(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
                         int ph, int pw);
-size_t conv_s1_workspace_bytes(int R, int S, int C, int Kc);
+size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip, int IH, int IW,
+                               int OH, int OW, int ph, int pw);
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
                 int OW, int ph, int pw, ActGrad ag, const char *tag);

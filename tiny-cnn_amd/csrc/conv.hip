@@ -418,7 +418,11 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   total += gemm_workspace_bytes(g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true);  // dX
   total += rowsum_workspace_bytes(batch, g.Kc, ohw);                  // db
   if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
-  total += 2 * conv_s1_workspace_bytes(g.R, g.S, g.C, g.Kc);          // repacked filters
+  if (g.sh == 1 && g.sw == 1) {  // LDS-halo kernel: repacked filters and split partial sums
+    total += conv_s1_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, 0, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
+    total += conv_s1_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, 1, g.OH, g.OW, g.H, g.W,
+                                     g.R - 1 - g.pad_h, g.S - 1 - g.pad_w);
+  }
 
   return total;
 }

@@ -37,6 +37,11 @@ struct ConvS1Args {
   int log_tr, log_ti;
   int tiles_x, tiles_y;        // tiles per image row / column direction
   FastDiv div_rows, div_pitch; // by (TR+R-1)*(TC+S-1) and by (TC+S-1)
+  // split over the reduction channels: workgroup z sums channels [z*kc_split, (z+1)*kc_split)
+  // into part[z][...] (laid out like out); part == nullptr: one pass, written to out
+  int kc_split;
+  float *part;
+  size_t part_stride;
 };
 
 template <int R, int S, int TC, int KCH, int TM, int TN>
@@ -69,6 +74,8 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
   const int x0    = tx * TC;
   const int m0    = blockIdx.y * BM;
   const int ihw   = a.IH * a.IW;
+  const int kc_lo = blockIdx.z * a.kc_split;
+  const int kc_hi = min(a.KC, kc_lo + a.kc_split);
 
   // ---- staging plan of the input patch: thread -> channel kcl, elements tl + TPC*i of a plane
   const int kcl = tid / TPC, tl = tid % TPC;
@@ -118,7 +125,7 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
   float rin[S1_NI_MAX], rw[NW];
 
   auto fetch = [&](int kc0) {
-    const bool ch_ok  = kc0 + kcl < a.KC;
+    const bool ch_ok  = kc0 + kcl < kc_hi;
     const float *base = a.in + static_cast<size_t>(kc0 + kcl) * ihw;
 #pragma unroll
     for (int i = 0; i < S1_NI_MAX; ++i)
@@ -127,7 +134,7 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
     for (int i = 0; i < NW; ++i) {
       const int e = tid + 256 * i;
       const int m = e % BM, kcw = (e / BM) % KCH, t = e / (BM * KCH);
-      const bool ok = (e < NWT) && (kc0 + kcw < a.KC) && (m0 + m < a.MC);
+      const bool ok = (e < NWT) && (kc0 + kcw < kc_hi) && (m0 + m < a.MC);
       rw[i] = ok ? a.wp[(static_cast<size_t>(t) * a.KC + kc0 + kcw) * a.MC + m0 + m] : 0.0f;
     }
   };
@@ -142,12 +149,12 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
       if (tid + 256 * i < NWT) w_l[tid + 256 * i] = rw[i];
   };
 
-  fetch(0);
-  for (int kc0 = 0; kc0 < a.KC; kc0 += KCH) {
-    if (kc0 > 0) __syncthreads();  // everyone is done reading the previous chunk
+  fetch(kc_lo);
+  for (int kc0 = kc_lo; kc0 < kc_hi; kc0 += KCH) {
+    if (kc0 > kc_lo) __syncthreads();  // everyone is done reading the previous chunk
     stage();
     __syncthreads();
-    if (kc0 + KCH < a.KC) fetch(kc0 + KCH);
+    if (kc0 + KCH < kc_hi) fetch(kc0 + KCH);
 #pragma unroll
     for (int p = 0; p < KCH / 2; ++p) {
       const float *inp = in_l + 2 * p * plane;
@@ -188,11 +195,48 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
         if (m >= a.MC) continue;
         const size_t idx = pbase + static_cast<size_t>(m) * ohw;
         float v = acc[i][j][rr];
+        if (a.part) {
+          a.part[blockIdx.z * a.part_stride + idx] = v;
+          continue;
+        }
         if (a.bias) v += a.bias[m];
         if (a.ag.kind != TDH_ACT_NONE) v *= act_grad_factor(a.ag.kind, a.ag.y[idx]);
         a.out[idx] = v;
       }
   }
+}
+
+// out = part[0] + part[1] + ... (in this order) (+ bias[m]) (* act'(y)); four elements per
+// thread when a channel plane is a multiple of four
+template <int VEC>
+__global__ void __launch_bounds__(256)
+s1_split_reduce_kernel(const float *__restrict__ part, const int splits, const size_t stride,
+                       float *__restrict__ out, const float *__restrict__ bias, const ActGrad ag,
+                       const int MC, const FastDiv div_plane, const size_t total) {
+  const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
+  if (i >= total) return;
+  float v[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) v[e] = 0.0f;
+  for (int z = 0; z < splits; ++z) {
+    if (VEC == 4) {
+      const float4 f = *reinterpret_cast<const float4 *>(part + z * stride + i);
+      v[0] += f.x; v[1] += f.y; v[2] += f.z; v[VEC - 1] += f.w;
+    } else {
+      v[0] += part[z * stride + i];
+    }
+  }
+  const int m = div_plane.div(static_cast<uint32_t>(i)) % MC;  // the plane of all VEC elements
+  const float b = bias ? bias[m] : 0.0f;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    v[e] += b;
+    if (ag.kind != TDH_ACT_NONE) v[e] *= act_grad_factor(ag.kind, ag.y[i + e]);
+  }
+  if (VEC == 4)
+    *reinterpret_cast<float4 *>(out + i) = make_float4(v[0], v[1], v[2], v[VEC - 1]);
+  else
+    out[i] = v[0];
 }
 
 // wp[t][kc][m]: forward (flip = 0): kc = ci, m = co, t as is; dX (flip = 1): kc = co, m = ci,
@@ -231,7 +275,24 @@ struct S1Plan {
   ConvS1Args args;
   size_t lds_bytes;
   dim3 grid;
+  int splits;
 };
+
+// Splits the reduction channels over grid.z when the tiles alone leave most of the chip idle.
+void choose_split(S1Plan &p, long blocks) {
+  const int nchunks = ceil_div(p.args.KC, p.kch);
+  int splits = 1;
+  if (blocks < 384 && nchunks >= 4) {
+    splits = static_cast<int>(std::min<long>(8, (512 + blocks - 1) / blocks));
+    splits = std::min(splits, nchunks / 2);
+  }
+  const int per      = ceil_div(nchunks, splits) * p.kch;
+  p.splits           = ceil_div(p.args.KC, per);
+  p.args.kc_split    = p.splits > 1 ? per : p.args.KC;
+  p.args.part        = nullptr;
+  p.args.part_stride = static_cast<size_t>(p.args.batch) * p.args.MC * p.args.OH * p.args.OW;
+  p.grid.z           = p.splits;
+}
 
 // Shape-only choice of the tile geometry; ok = false sends the caller to the generic GEMM.
 // Candidates run from the largest workgroup tile to the smallest; the first one that yields
@@ -276,13 +337,14 @@ S1Plan make_plan(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH
     if (tiles > 2000000000L) continue;
     p.grid = dim3(static_cast<unsigned>(tiles), ceil_div(MC, 32 * p.tm), 1);
     p.ok   = true;
+    choose_split(p, blocks);
     if (blocks >= 256) return p;
     if (blocks > best_blocks) {
       best_blocks = blocks;
       best        = p;
     }
   }
-  if (best_blocks < 64) best.ok = false;
+  if (best_blocks * (best.ok ? best.splits : 1) < 128) best.ok = false;
   return best;
 }
 
@@ -332,8 +394,14 @@ bool conv_s1_applicable(int R, int S, int batch, int KC, int MC, int IH, int IW,
   return make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw).ok;
 }
 
-size_t conv_s1_workspace_bytes(int R, int S, int C, int Kc) {
-  return ws_align(sizeof(float) * static_cast<size_t>(R) * S * C * Kc);
+size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip, int IH, int IW,
+                               int OH, int OW, int ph, int pw) {
+  const int KC = flip ? Kc : C, MC = flip ? C : Kc;
+  const S1Plan p = make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw);
+  if (!p.ok) return 0;
+  size_t total = ws_align(sizeof(float) * static_cast<size_t>(R) * S * C * Kc);  // repacked filter
+  if (p.splits > 1) total += ws_align(sizeof(float) * p.splits * p.args.part_stride);
+  return total;
 }
 
 // Runs out = conv(in, repack(w)) (+ bias) (* act'(y)); the caller has checked applicability
@@ -354,8 +422,31 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
   }
   p.args.in = in; p.args.wp = static_cast<const float *>(wp); p.args.bias = bias;
   p.args.out = out; p.args.ag = ag;
-  ProfScope prof(tag, MC, batch * OH * OW, KC * R * S);
-  return R == 3 ? launch_s1_rs<3, 3>(p) : launch_s1_rs<5, 5>(p);
+  if (p.splits > 1) {
+    void *part = nullptr;
+    TDH_TRY(ws_take(sizeof(float) * p.splits * p.args.part_stride, &part));
+    p.args.part = static_cast<float *>(part);
+  }
+  {
+    ProfScope prof(tag, MC, batch * OH * OW, KC * R * S);
+    TDH_TRY(R == 3 ? (launch_s1_rs<3, 3>(p)) : (launch_s1_rs<5, 5>(p)));
+  }
+  if (p.splits > 1) {
+    const size_t total = p.args.part_stride;
+    const int plane    = OH * OW;
+    ProfScope prof("conv_s1_split_reduce", 4.0 * total * (p.splits + 1 + (ag.kind != TDH_ACT_NONE)),
+                   WORK_BYTE);
+    if (plane % 4 == 0)
+      hipLaunchKernelGGL((s1_split_reduce_kernel<4>), dim3(static_cast<unsigned>(ceil_div_sz(total / 4, 256))), dim3(256), 0,
+                         ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
+                         FastDiv(plane), total);
+    else
+      hipLaunchKernelGGL((s1_split_reduce_kernel<1>), dim3(static_cast<unsigned>(ceil_div_sz(total, 256))), dim3(256), 0,
+                         ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
+                         FastDiv(plane), total);
+    TDH_LAUNCH_CHECK();
+  }
+  return TDH_OK;
 }
 
 }  // namespace tdh
