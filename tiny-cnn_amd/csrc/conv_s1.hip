@@ -338,7 +338,9 @@ S1Plan make_plan(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH
     p.grid = dim3(static_cast<unsigned>(tiles), ceil_div(MC, 32 * p.tm), 1);
     p.ok   = true;
     choose_split(p, blocks);
-    if (blocks >= 256) return p;
+    // short reductions have nothing to overlap their loads with inside a workgroup: ask for
+    // more, smaller workgroups then
+    if (blocks >= (KC * R * S < 256 ? 1024 : 256)) return p;
     if (blocks > best_blocks) {
       best_blocks = blocks;
       best        = p;

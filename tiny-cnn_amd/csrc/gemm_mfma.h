@@ -157,9 +157,23 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
   const int wave = tid >> 6;
   const int wm   = wave % WM;
   const int wn   = wave / WM;
-  const int m0   = blockIdx.y * BM;
-  const int n0   = blockIdx.x * BN;
-  const int kbeg = blockIdx.z * k_per_split;
+  // Workgroups are handed to the eight XCDs (each with its own L2) round-robin in launch
+  // order. Renumber them so that workgroups that are neighbours in (n-tile, m-tile, split)
+  // order, which read the same rows of A or columns of B, run on the same XCD.
+  int bx, by, bz;
+  {
+    const int gx = gridDim.x, gy = gridDim.y;
+    const int total = gx * gy * gridDim.z, per = total >> 3;
+    int id = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
+    bx = id % gx;
+    id /= gx;
+    by = id % gy;
+    bz = id / gy;
+  }
+  const int m0   = by * BM;
+  const int n0   = bx * BN;
+  const int kbeg = bz * k_per_split;
   const int kend = min(K, kbeg + k_per_split);
 
   // ---- per-thread staging assignment
@@ -374,7 +388,7 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
     const int n = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
     if (n >= N) continue;
     if (partial != nullptr) {
-      float *dst = partial + static_cast<size_t>(blockIdx.z) * M * N + n;
+      float *dst = partial + static_cast<size_t>(bz) * M * N + n;
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -412,8 +426,18 @@ splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const 
   const int idx = blockIdx.x * REDUCE_OUTPUTS + o;
   const size_t mn = static_cast<size_t>(M) * N;
   float s = 0.0f;
-  if (idx < M * N)
-    for (int z = g; z < splits; z += REDUCE_GROUPS) s += partial[z * mn + idx];
+  if (idx < M * N) {
+    // eight slices per trip: the loads are issued together, the adds keep slice order
+    int z = g;
+    for (; z + 7 * REDUCE_GROUPS < splits; z += 8 * REDUCE_GROUPS) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = partial[(z + u * REDUCE_GROUPS) * mn + idx];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; z < splits; z += REDUCE_GROUPS) s += partial[z * mn + idx];
+  }
   sm[g][o] = s;
   __syncthreads();
   if (g == 0 && idx < M * N) {

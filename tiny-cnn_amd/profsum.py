@@ -49,7 +49,10 @@ def kernels(dirname, top):
         with open(path, newline="") as f:
             for r in csv.DictReader(f):
                 dur = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
-                grid = int(r.get("Grid_Size") or r.get("Grid_Size_X") or 0)
+                if "Grid_Size" in r:
+                    grid = int(r["Grid_Size"])
+                else:
+                    grid = int(r["Grid_Size_X"]) * int(r["Grid_Size_Y"]) * int(r["Grid_Size_Z"])
                 rows[(short_name(r["Kernel_Name"]), grid)].append(dur)
     total = sum(sum(v) for v in rows.values())
     print(f"| kernel | grid (work-items) | launches | avg us | min us | max us | % of GPU time |")
@@ -75,11 +78,12 @@ def counters(dirs, top, copy_mib):
     mean = lambda xs: sum(xs) / len(xs) if xs else float("nan")
     scale = {}
     copy_bytes = copy_mib * (1 << 20)
-    for (name, grid), v in acc.items():
-        if name.startswith("copy_kernel") and grid >= copy_bytes // 64:
-            for c in ("FETCH_SIZE", "WRITE_SIZE"):
-                if c in v:
-                    scale[c] = copy_bytes / (mean(v[c]) * 1024.0)
+    copies = [k for k in acc if k[0].startswith("copy_kernel")]
+    if copies:
+        v = acc[max(copies, key=lambda k: k[1])]  # the yardstick is the largest copy of the run
+        for c in ("FETCH_SIZE", "WRITE_SIZE"):
+            if c in v:
+                scale[c] = copy_bytes / (mean(v[c]) * 1024.0)
     if scale:
         print("counter scale from copy_kernel (%d MiB read, %d MiB written; counters in KiB): "
               % (copy_mib, copy_mib) + ", ".join(f"{c} x{s:.4f}" for c, s in sorted(scale.items())) + "\n")
