@@ -33,6 +33,9 @@ CONV = [
     (32, 32, 3, 5, 32, True, 1, 8), (16, 16, 32, 5, 32, True, 1, 8), (8, 8, 32, 5, 64, True, 1, 8),
     (24, 24, 32, 3, 64, True, 1, 4), (17, 13, 5, 3, 7, True, 1, 3), (11, 11, 4, 3, 6, False, 3, 2),
     (33, 31, 3, 3, 130, True, 1, 2), (16, 16, 64, 3, 128, True, 1, 2), (7, 7, 3, 7, 5, False, 1, 1),
+    # LDS-staged dW kernel: ragged widths, partial channel blocks, valid padding, column tiles
+    (13, 11, 16, 3, 40, True, 1, 3), (18, 18, 20, 5, 24, False, 1, 2), (70, 9, 33, 3, 65, True, 1, 2),
+    (12, 12, 48, 5, 16, True, 1, 5), (40, 6, 16, 3, 16, False, 1, 1),
 ]
 
 

@@ -167,6 +167,13 @@ size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip,
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
                 int OW, int ph, int pw, ActGrad ag, const char *tag);
+// conv_dw.hip: stride-1 weight gradient from LDS-staged tiles (3x3 and 5x5 windows)
+bool conv_dw_halo_applicable(int R, int S, int batch, int C, int Kc, int H, int W, int OH, int OW,
+                             int ph, int pw);
+size_t conv_dw_halo_workspace_bytes(int R, int S, int batch, int C, int Kc, int H, int W, int OH,
+                                    int OW, int ph, int pw);
+int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, const float *dy,
+                     float *dw, int H, int W, int OH, int OW, int ph, int pw, int accumulate);
 // workspace bytes the op may ask for (so a net can reserve it before graph capture)
 size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
 size_t fc_workspace_bytes(int in, int out, int batch);

@@ -418,6 +418,8 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   total += gemm_workspace_bytes(g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true);  // dX
   total += rowsum_workspace_bytes(batch, g.Kc, ohw);                  // db
   if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
+  if (g.sh == 1 && g.sw == 1)
+    total += conv_dw_halo_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
   if (g.sh == 1 && g.sw == 1) {  // LDS-halo kernel: repacked filters and split partial sums
     total += conv_s1_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, 0, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
     total += conv_s1_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, 1, g.OH, g.OW, g.H, g.W,
@@ -509,16 +511,26 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   if (dw) {
     DwDyOperand A{dy, g.Kc, ohw, g.div_ohw};
     DwInputOperand B{x, g, crs};
+    const bool halo = g.sh == 1 && g.sw == 1 &&
+                      conv_dw_halo_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW,
+                                              g.pad_h, g.pad_w);
     if (tbl_dev) {
       void *tmp = nullptr;
       TDH_TRY(ws_take(sizeof(float) * g.Kc * crs, &tmp));
       EpiRowMajor epi{static_cast<float *>(tmp), crs, nullptr, ActGrad(), 0};
-      TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm", "conv_dw_splitk_reduce")));
+      if (halo)
+        TDH_TRY(conv_dw_halo_run(g.R, g.S, batch, g.C, g.Kc, x, dy, static_cast<float *>(tmp), g.H,
+                                 g.W, g.OH, g.OW, g.pad_h, g.pad_w, 0));
+      else
+        TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm", "conv_dw_splitk_reduce")));
       ProfScope prof("conv_mask_weights", 8.0 * g.Kc * crs, WORK_BYTE);
       hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(g.Kc * crs, 256)), dim3(256), 0,
                          ctx().stream, static_cast<const float *>(tmp), tbl_dev, dw, g.Kc * crs,
                          g.C, g.Kc, g.R * g.S, accumulate);
       TDH_LAUNCH_CHECK();
+    } else if (halo) {
+      TDH_TRY(conv_dw_halo_run(g.R, g.S, batch, g.C, g.Kc, x, dy, dw, g.H, g.W, g.OH, g.OW, g.pad_h,
+                               g.pad_w, accumulate));
     } else {
       EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
       TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm",
