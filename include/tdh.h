@@ -46,7 +46,9 @@ typedef enum tdh_status {
 } tdh_status;
 
 /* activation_layer subclasses (tiny_dnn/activations/) */
-enum { TDH_ACT_TANH = 0, TDH_ACT_RELU = 1, TDH_ACT_SOFTMAX = 2, TDH_ACT_SIGMOID = 3, TDH_ACT_NONE = -1 };
+enum { TDH_ACT_TANH = 0, TDH_ACT_RELU = 1, TDH_ACT_SOFTMAX = 2, TDH_ACT_SIGMOID = 3,
+       TDH_ACT_LEAKY_RELU = 4, TDH_ACT_ELU = 5, TDH_ACT_SELU = 6, TDH_ACT_SOFTPLUS = 7,
+       TDH_ACT_SOFTSIGN = 8, TDH_ACT_ASINH = 9, TDH_ACT_TANH_P1M2 = 10, TDH_ACT_NONE = -1 };
 /* loss functions (tiny_dnn/lossfunctions/loss_function.h) */
 enum { TDH_LOSS_MSE = 0, TDH_LOSS_CE_MULTICLASS = 1, TDH_LOSS_CE = 2 };
 /* optimizers (tiny_dnn/optimizers/optimizer.h) */
@@ -91,6 +93,7 @@ typedef struct tdh_layer {
   tdh_conv_desc conv;
   tdh_pool_desc pool;
   int32_t fc_in, fc_out, fc_bias;
+  float act_p[2]; /* TDH_L_ACT: constructor parameters of the kinds that have them (see tdh_act_fwd_p) */
 } tdh_layer;
 
 /* ------------------------------------------------------------ library state */
@@ -186,6 +189,18 @@ int tdh_avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const flo
  * len = per-sample vector length; the backward uses the layer OUTPUT y. */
 int tdh_act_fwd(int kind, int batch, int len, const float *x, float *y);
 int tdh_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx);
+/* The same for every activation layer, with the layer's constructor parameters p[2]:
+ * leaky_relu {epsilon} (leaky_relu_layer.h:74-88), elu {alpha} (elu_layer.h:37-52),
+ * selu {lambda, alpha} (selu_layer.h:82-99), softplus {beta, threshold}
+ * (softplus_layer.h:84-102), softsign (softsign_layer.h:24-40), asinh (asinh_layer.h:24-38),
+ * tanh_p1m2 (tanh_p1m2_layer.h:24-40); p is ignored by the other kinds and NULL selects the
+ * constructor defaults. The backward takes the layer input x as well, as the reference's
+ * backward_activation does: selu and softsign read it (x may be NULL for the others).
+ * tdh_act_fwd / tdh_act_bwd are these calls with p = NULL and x = NULL. */
+void tdh_act_default_params(int kind, float *p);
+int tdh_act_fwd_p(int kind, const float *p, int batch, int len, const float *x, float *y);
+int tdh_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, const float *y,
+                  const float *dy, float *dx);
 /* gradient<E> for a mini-batch (tiny_dnn/lossfunctions/loss_function.h:191-218) */
 int tdh_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
 /* softmax_layer backward applied to cross_entropy_multiclass::df in one kernel:

@@ -15,7 +15,18 @@ ORACLE_SO = os.path.join(HERE, "libtd_oracle.so")
 REF_SCALAR_SO = os.path.join(HERE, "_ref", "libtd_ref_scalar.so")
 REF_AVX_SO = os.path.join(HERE, "_ref", "libtd_ref_avx.so")
 
-ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3}
+ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3, "leaky_relu": 4, "elu": 5, "selu": 6,
+       "softplus": 7, "softsign": 8, "asinh": 9, "tanh_p1m2": 10}
+# constructor defaults of the parameterised activation layers (leaky_relu_layer.h:25,
+# elu_layer.h:18, selu_layer.h:26-27, softplus_layer.h:26-27)
+ACT_DEFAULTS = {"leaky_relu": (0.01, 0.0), "elu": (1.0, 0.0), "selu": (1.05070, 1.67326),
+                "softplus": (1.0, 20.0)}
+
+
+def act_params(kind, params=None):
+    p = list(params) if params is not None else list(ACT_DEFAULTS.get(kind, (0.0, 0.0)))
+    p += [0.0] * (2 - len(p))
+    return (C.c_float * 2)(*p)
 LOSS = {"mse": 0, "ce_multiclass": 1, "ce": 2}
 OPT = {"sgd": 0, "momentum": 1, "adam": 2, "adagrad": 3, "rmsprop": 4, "adamax": 5, "nesterov": 6}
 L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT = range(5)
@@ -42,7 +53,8 @@ class OptDesc(C.Structure):
 
 class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("act", C.c_int32), ("conv", ConvDesc), ("pool", PoolDesc),
-                ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32)]
+                ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32),
+                ("act_p", C.c_float * 2)]
 
 
 def conv_desc(in_w, in_h, in_c, k_w, k_h, out_c, pad_same=False, has_bias=True, w_stride=1,
@@ -240,20 +252,21 @@ def avepool_bwd(d, x, w, dy):
     return dx, dw, db
 
 
-def act_fwd(kind, x):
+def act_fwd(kind, x, params=None):
     lib = oracle_lib()
     x, xp = _f(x)
     y = np.empty_like(x)
-    _chk(lib.tdo_act_fwd(ACT[kind], x.shape[0], x.shape[1], xp, y.ctypes.data_as(f32p)), "act_fwd")
+    _chk(lib.tdo_act_fwd_p(ACT[kind], act_params(kind, params), x.shape[0], x.shape[1], xp,
+                           y.ctypes.data_as(f32p)), "act_fwd")
     return y
 
 
-def act_bwd(kind, x, y, dy):
+def act_bwd(kind, x, y, dy, params=None):
     lib = oracle_lib()
     x, xp = _f(x); y, yp = _f(y); dy, dyp = _f(dy)
     dx = np.empty_like(x)
-    _chk(lib.tdo_act_bwd(ACT[kind], x.shape[0], x.shape[1], xp, yp, dyp,
-                         dx.ctypes.data_as(f32p)), "act_bwd")
+    _chk(lib.tdo_act_bwd_p(ACT[kind], act_params(kind, params), x.shape[0], x.shape[1], xp, yp, dyp,
+                           dx.ctypes.data_as(f32p)), "act_bwd")
     return dx
 
 
@@ -317,9 +330,10 @@ def L_avepool(in_w, in_h, in_c, pool, stride=None):
     return l
 
 
-def L_act(kind):
+def L_act(kind, params=None):
     l = LayerDesc()
     l.kind, l.act = L_ACT, ACT[kind]
+    l.act_p = act_params(kind, params)
     return l
 
 
@@ -550,18 +564,19 @@ def ref_avepool_bwd(d, x, w, dy, kind="scalar"):
     return dx, dw, db
 
 
-def ref_act(kind_name, x, dy=None, kind="scalar"):
+def ref_act(kind_name, x, dy=None, kind="scalar", params=None):
     lib = ref_lib(kind)
     x, xp = _f(x)
     y = np.empty_like(x)
+    prm = act_params(kind_name, params)
     if dy is None:
-        _chk(lib.tdr_act(ACT[kind_name], x.shape[0], x.shape[1], xp, y.ctypes.data_as(f32p),
-                         None, None), "ref act")
+        _chk(lib.tdr_act_p(ACT[kind_name], prm, x.shape[0], x.shape[1], xp, y.ctypes.data_as(f32p),
+                           None, None), "ref act")
         return y
     dy, dyp = _f(dy)
     dx = np.empty_like(x)
-    _chk(lib.tdr_act(ACT[kind_name], x.shape[0], x.shape[1], xp, y.ctypes.data_as(f32p), dyp,
-                     dx.ctypes.data_as(f32p)), "ref act")
+    _chk(lib.tdr_act_p(ACT[kind_name], prm, x.shape[0], x.shape[1], xp, y.ctypes.data_as(f32p), dyp,
+                       dx.ctypes.data_as(f32p)), "ref act")
     return y, dx
 
 

@@ -53,6 +53,7 @@ struct layer_desc {
   conv_desc conv;
   pool_desc pool;
   int32_t fc_in, fc_out, fc_bias;
+  float act_p[2];
 };
 
 core::backend_t engine_of(int engine) {
@@ -143,9 +144,9 @@ double layer_bwd(layer &l, int batch, const float *dy, size_t out_len, float *dx
   return std::chrono::duration<double>(t1 - t0).count();
 }
 
-template <typename Act>
-int act_run(int batch, int len, const float *x, float *y, const float *dy, float *dx) {
-  Act a((size_t)len);
+template <typename Act, typename... P>
+int act_run(int batch, int len, const float *x, float *y, const float *dy, float *dx, P... prm) {
+  Act a((size_t)len, prm...);
   layer_fwd(a, batch, x, len, y, len);
   if (dy) layer_bwd(a, batch, dy, len, dx, len);
   return 0;
@@ -276,17 +277,31 @@ int tdr_avepool_bwd(const pool_desc *d, int batch, const float *x, const float *
   } catch (const std::exception &) { return -1; }
 }
 
-/* kind: 0 tanh, 1 relu, 2 softmax, 3 sigmoid; dy/dx may be NULL (forward only) */
-int tdr_act(int kind, int batch, int len, const float *x, float *y, const float *dy, float *dx) {
+/* kind: 0 tanh, 1 relu, 2 softmax, 3 sigmoid, 4 leaky_relu {epsilon}, 5 elu {alpha},
+ * 6 selu {lambda, alpha}, 7 softplus {beta, threshold}, 8 softsign, 9 asinh, 10 tanh_p1m2;
+ * p: the constructor parameters in braces; dy/dx may be NULL (forward only) */
+int tdr_act_p(int kind, const float *p, int batch, int len, const float *x, float *y,
+              const float *dy, float *dx) {
   try {
     switch (kind) {
       case 0: return act_run<tanh_layer>(batch, len, x, y, dy, dx);
       case 1: return act_run<relu_layer>(batch, len, x, y, dy, dx);
       case 2: return act_run<softmax_layer>(batch, len, x, y, dy, dx);
       case 3: return act_run<sigmoid_layer>(batch, len, x, y, dy, dx);
+      case 4: return act_run<leaky_relu_layer>(batch, len, x, y, dy, dx, p[0]);
+      case 5: return act_run<elu_layer>(batch, len, x, y, dy, dx, p[0]);
+      case 6: return act_run<selu_layer>(batch, len, x, y, dy, dx, p[0], p[1]);
+      case 7: return act_run<softplus_layer>(batch, len, x, y, dy, dx, p[0], p[1]);
+      case 8: return act_run<softsign_layer>(batch, len, x, y, dy, dx);
+      case 9: return act_run<asinh_layer>(batch, len, x, y, dy, dx);
+      case 10: return act_run<tanh_p1m2_layer>(batch, len, x, y, dy, dx);
     }
     return -2;
   } catch (const std::exception &) { return -1; }
+}
+int tdr_act(int kind, int batch, int len, const float *x, float *y, const float *dy, float *dx) {
+  const float none[2] = {0.0f, 0.0f};
+  return kind <= 3 ? tdr_act_p(kind, none, batch, len, x, y, dy, dx) : -2;
 }
 
 /* kind: 0 mse, 1 cross_entropy_multiclass, 2 cross_entropy */
@@ -373,6 +388,13 @@ tdr_net *tdr_net_create(const layer_desc *layers, int n_layers, int engine) {
             case 1: h->net << relu_layer(); break;
             case 2: h->net << softmax_layer(); break;
             case 3: h->net << sigmoid_layer(); break;
+            case 4: h->net << leaky_relu_layer(s.act_p[0]); break;
+            case 5: h->net << elu_layer(s.act_p[0]); break;
+            case 6: h->net << selu_layer(s.act_p[0], s.act_p[1]); break;
+            case 7: h->net << softplus_layer(s.act_p[0], s.act_p[1]); break;
+            case 8: h->net << softsign_layer(); break;
+            case 9: h->net << asinh_layer(); break;
+            case 10: h->net << tanh_p1m2_layer(); break;
             default: return nullptr;
           }
           break;

@@ -560,10 +560,35 @@ int tdo_avepool_bwd(const tdo_pool_desc *d, int batch, const float *x, const flo
 
 /* activation_layer::forward_propagation, tiny_dnn/activations/activation_layer.h:74-79;
  * tanh_layer.h:24-28, relu_layer.h:25-29, softmax_layer.h:24-34, sigmoid_layer.h:24-28 */
+void tdo_act_default_params(int kind, float *p) {
+  p[0] = p[1] = 0.0f;
+  switch (kind) {
+    case TDO_ACT_LEAKY_RELU: p[0] = 0.01f; break;                 /* epsilon, leaky_relu_layer.h:25 */
+    case TDO_ACT_ELU: p[0] = 1.0f; break;                         /* alpha, elu_layer.h:18 */
+    case TDO_ACT_SELU: p[0] = 1.05070f; p[1] = 1.67326f; break;   /* lambda, alpha, selu_layer.h:26-27 */
+    case TDO_ACT_SOFTPLUS: p[0] = 1.0f; p[1] = 20.0f; break;      /* beta, threshold, softplus_layer.h:26-27 */
+  }
+}
+
 int tdo_act_fwd(int kind, int batch, int len, const float *x, float *y) {
-  if (kind != TDO_ACT_TANH && kind != TDO_ACT_RELU && kind != TDO_ACT_SOFTMAX &&
-      kind != TDO_ACT_SIGMOID)
-    return -2;
+  float p[2];
+  tdo_act_default_params(kind, p);
+  return tdo_act_fwd_p(kind, p, batch, len, x, y);
+}
+
+int tdo_act_bwd(int kind, int batch, int len, const float *x, const float *y, const float *dy,
+                float *dx) {
+  float p[2];
+  tdo_act_default_params(kind, p);
+  return tdo_act_bwd_p(kind, p, batch, len, x, y, dy, dx);
+}
+
+/* forward_activation of leaky_relu_layer.h:74-78, elu_layer.h:37-42, selu_layer.h:82-88,
+ * softplus_layer.h:84-90, softsign_layer.h:24-28 (computed in double: `1.0 + std::abs`),
+ * asinh_layer.h:24-28, tanh_p1m2_layer.h:24-30, beside the four kinds above */
+int tdo_act_fwd_p(int kind, const float *p, int batch, int len, const float *x, float *y) {
+  if (kind < TDO_ACT_TANH || kind > TDO_ACT_TANH_P1M2) return -2;
+  const float p0 = p[0], p1 = p[1];
 #pragma omp parallel for schedule(static)
   for (int s = 0; s < batch; s++) {
     const float *xi = x + (size_t)len * s;
@@ -589,6 +614,34 @@ int tdo_act_fwd(int kind, int batch, int len, const float *x, float *y) {
         }
         for (int j = 0; j < len; j++) yo[j] /= denominator;
       } break;
+      case TDO_ACT_LEAKY_RELU:
+        for (int j = 0; j < len; j++) yo[j] = xi[j] > 0.0f ? xi[j] : p0 * xi[j];
+        break;
+      case TDO_ACT_ELU:
+        for (int j = 0; j < len; j++) yo[j] = xi[j] < 0.0f ? (p0 * (expf(xi[j]) - 1.0f)) : xi[j];
+        break;
+      case TDO_ACT_SELU:
+        for (int j = 0; j < len; j++)
+          yo[j] = p0 * (xi[j] > 0.0f ? xi[j] : p1 * (expf(xi[j]) - 1.0f));
+        break;
+      case TDO_ACT_SOFTPLUS:
+        for (int j = 0; j < len; j++) {
+          const float betain = p0 * xi[j];
+          yo[j] = (betain > p1) ? xi[j] : (1 / p0) * log1pf(expf(betain));
+        }
+        break;
+      case TDO_ACT_SOFTSIGN:
+        for (int j = 0; j < len; j++) yo[j] = (float)(xi[j] / (1.0 + fabsf(xi[j])));
+        break;
+      case TDO_ACT_ASINH:
+        for (int j = 0; j < len; j++) yo[j] = asinhf(xi[j]);
+        break;
+      case TDO_ACT_TANH_P1M2:
+        for (int j = 0; j < len; j++) {
+          const float ep = expf(xi[j]);
+          yo[j] = ep / (ep + (1.0f / ep));
+        }
+        break;
     }
   }
   return 0;
@@ -597,14 +650,18 @@ int tdo_act_fwd(int kind, int batch, int len, const float *x, float *y) {
 /* activation_layer::back_propagation, activation_layer.h:81-91; tanh_layer.h:30-38,
  * relu_layer.h:31-39, softmax_layer.h:36-55 (full Jacobian row dotted with dy),
  * sigmoid_layer.h:30-38 */
-int tdo_act_bwd(int kind, int batch, int len, const float *x, const float *y, const float *dy,
-                float *dx) {
-  (void)x;
-  if (kind != TDO_ACT_TANH && kind != TDO_ACT_RELU && kind != TDO_ACT_SOFTMAX &&
-      kind != TDO_ACT_SIGMOID)
-    return -2;
+/* ... and backward_activation of leaky_relu_layer.h:80-88, elu_layer.h:44-52,
+ * selu_layer.h:90-99 (uses x; the product runs in double because of the literal 1.0),
+ * softplus_layer.h:92-102, softsign_layer.h:30-40 (uses x, double), asinh_layer.h:30-38,
+ * tanh_p1m2_layer.h:32-40 */
+int tdo_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, const float *y,
+                  const float *dy, float *dx) {
+  if (kind < TDO_ACT_TANH || kind > TDO_ACT_TANH_P1M2) return -2;
+  if ((kind == TDO_ACT_SELU || kind == TDO_ACT_SOFTSIGN) && !x) return -2;
+  const float p0 = p[0], p1 = p[1];
 #pragma omp parallel for schedule(static)
   for (int s = 0; s < batch; s++) {
+    const float *xi = x ? x + (size_t)len * s : NULL;
     const float *yo = y + (size_t)len * s;
     const float *d  = dy + (size_t)len * s;
     float *o        = dx + (size_t)len * s;
@@ -627,6 +684,35 @@ int tdo_act_bwd(int kind, int batch, int len, const float *x, const float *y, co
         }
         free(df);
       } break;
+      case TDO_ACT_LEAKY_RELU:
+        for (int j = 0; j < len; j++) o[j] = d[j] * (yo[j] > 0.0f ? 1.0f : p0);
+        break;
+      case TDO_ACT_ELU:
+        for (int j = 0; j < len; j++) o[j] = d[j] * (yo[j] > 0.0f ? 1.0f : (p0 + yo[j]));
+        break;
+      case TDO_ACT_SELU:
+        for (int j = 0; j < len; j++)
+          o[j] = (float)(d[j] * p0 * (xi[j] > 0.0f ? 1.0 : (double)(p1 * expf(xi[j]))));
+        break;
+      case TDO_ACT_SOFTPLUS:
+        for (int j = 0; j < len; j++) {
+          const float betaout = p0 * yo[j];
+          const float exp_bo  = expf(betaout);
+          o[j] = (betaout > p1) ? d[j] : d[j] * (exp_bo - 1) / exp_bo;
+        }
+        break;
+      case TDO_ACT_SOFTSIGN:
+        for (int j = 0; j < len; j++) {
+          const double dd = 1.0 + fabsf(xi[j]);
+          o[j] = (float)(d[j] / (dd * dd));
+        }
+        break;
+      case TDO_ACT_ASINH:
+        for (int j = 0; j < len; j++) o[j] = d[j] / coshf(yo[j]);
+        break;
+      case TDO_ACT_TANH_P1M2:
+        for (int j = 0; j < len; j++) o[j] = d[j] * (2 * yo[j] * (1.0f - yo[j]));
+        break;
     }
   }
   return 0;
@@ -904,7 +990,9 @@ int tdo_net_forward(tdo_net *net, int batch, const float *x) {
         break;
       case TDO_L_MAXPOOL: rc = tdo_maxpool_fwd(&L->spec.pool, batch, in, L->out, L->argmax); break;
       case TDO_L_AVEPOOL: rc = tdo_avepool_fwd(&L->spec.pool, batch, in, L->w, L->b, L->out); break;
-      case TDO_L_ACT: rc = tdo_act_fwd(L->spec.act, batch, (int)L->out_size, in, L->out); break;
+      case TDO_L_ACT:
+        rc = tdo_act_fwd_p(L->spec.act, L->spec.act_p, batch, (int)L->out_size, in, L->out);
+        break;
     }
     if (rc) return rc;
     in = L->out;
@@ -939,7 +1027,8 @@ int tdo_net_train_step(tdo_net *net, tdo_opt *opt, int loss_kind, int batch, con
         rc = tdo_avepool_bwd(&L->spec.pool, batch, in, L->w, L->dout, L->dx, L->dw, L->db);
         break;
       case TDO_L_ACT:
-        rc = tdo_act_bwd(L->spec.act, batch, (int)L->out_size, in, L->out, L->dout, L->dx);
+        rc = tdo_act_bwd_p(L->spec.act, L->spec.act_p, batch, (int)L->out_size, in, L->out, L->dout,
+                           L->dx);
         break;
     }
     if (rc) return rc;

@@ -47,7 +47,9 @@ typedef struct tdo_pool_desc {
   int32_t ceil_mode;
 } tdo_pool_desc;
 
-enum { TDO_ACT_TANH = 0, TDO_ACT_RELU = 1, TDO_ACT_SOFTMAX = 2, TDO_ACT_SIGMOID = 3 };
+enum { TDO_ACT_TANH = 0, TDO_ACT_RELU = 1, TDO_ACT_SOFTMAX = 2, TDO_ACT_SIGMOID = 3,
+       TDO_ACT_LEAKY_RELU = 4, TDO_ACT_ELU = 5, TDO_ACT_SELU = 6, TDO_ACT_SOFTPLUS = 7,
+       TDO_ACT_SOFTSIGN = 8, TDO_ACT_ASINH = 9, TDO_ACT_TANH_P1M2 = 10 };
 enum { TDO_LOSS_MSE = 0, TDO_LOSS_CE_MULTICLASS = 1, TDO_LOSS_CE = 2 };
 enum { TDO_OPT_SGD = 0, TDO_OPT_MOMENTUM = 1, TDO_OPT_ADAM = 2, TDO_OPT_ADAGRAD = 3,
        TDO_OPT_RMSPROP = 4, TDO_OPT_ADAMAX = 5, TDO_OPT_NESTEROV = 6 };
@@ -98,6 +100,12 @@ int tdo_avepool_bwd(const tdo_pool_desc *d, int batch, const float *x, const flo
 int tdo_act_fwd(int kind, int batch, int len, const float *x, float *y);
 int tdo_act_bwd(int kind, int batch, int len, const float *x, const float *y,
                 const float *dy, float *dx);
+/* the same with the layer's constructor parameters p[2]: leaky-relu {epsilon}, elu {alpha},
+ * selu {lambda, alpha}, softplus {beta, threshold}; ignored by the other kinds */
+void tdo_act_default_params(int kind, float *p);
+int tdo_act_fwd_p(int kind, const float *p, int batch, int len, const float *x, float *y);
+int tdo_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, const float *y,
+                  const float *dy, float *dx);
 
 /* loss gradient for a mini-batch (no 1/batch factor, as in the reference) */
 int tdo_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
@@ -119,6 +127,7 @@ typedef struct tdo_layer {
   tdo_conv_desc conv;
   tdo_pool_desc pool;
   int32_t fc_in, fc_out, fc_bias;
+  float act_p[2]; /* TDO_L_ACT: parameters of the kinds that have them */
 } tdo_layer;
 
 typedef struct tdo_net tdo_net;

@@ -71,6 +71,11 @@ def layer_grads():
 
 
 @pytest.fixture(scope="session")
+def act_golden():
+    return np.load(os.path.join(GOLDEN, "activations.npz"))
+
+
+@pytest.fixture(scope="session")
 def net_steps():
     return np.load(os.path.join(GOLDEN, "net_steps.npz"))
 

@@ -289,13 +289,53 @@ static void fc_pool_ops_vs_oracle() {
   }
 }
 
+// activation layers: forward_activation / backward_activation against the oracle
+template <typename Layer>
+static void activation_case(Layer l, int kind, const float *prm, const char *name) {
+  const size_t n = 257;
+  vec_t x = random_vec(n, 61, -4.f, 4.f), dy = random_vec(n, 62), y, dx;
+  x[0] = 0.f;
+  if (kind != TDO_ACT_SOFTMAX) {  // a saturated softmax has gradients of rounding-error size only
+    x[1] = 30.f;
+    x[2] = -30.f;
+  }
+  l.forward_activation(x, y);
+  l.backward_activation(x, y, dx, dy);
+  float p[2];
+  tdo_act_default_params(kind, p);
+  if (prm) { p[0] = prm[0]; p[1] = prm[1]; }
+  vec_t wy(n), wdx(n);
+  EXPECT(tdo_act_fwd_p(kind, p, 1, n, x.data(), wy.data()) == 0);
+  EXPECT(tdo_act_bwd_p(kind, p, 1, n, x.data(), wy.data(), dy.data(), wdx.data()) == 0);
+  expect_near(y, wy, 1e-4f, name);
+  expect_near(dx, wdx, 1e-4f, name);
+}
+static void activations_vs_oracle() {
+  std::puts("activation layers vs oracle");
+  const float leaky[2] = {0.2f, 0.f}, elu[2] = {0.5f, 0.f}, sp[2] = {2.f, 5.f};
+  activation_case(tanh_layer(), TDO_ACT_TANH, nullptr, "tanh");
+  activation_case(relu_layer(), TDO_ACT_RELU, nullptr, "relu");
+  activation_case(sigmoid_layer(), TDO_ACT_SIGMOID, nullptr, "sigmoid");
+  activation_case(softmax_layer(), TDO_ACT_SOFTMAX, nullptr, "softmax");
+  activation_case(leaky_relu_layer(), TDO_ACT_LEAKY_RELU, nullptr, "leaky_relu");
+  activation_case(leaky_relu_layer(0.2f), TDO_ACT_LEAKY_RELU, leaky, "leaky_relu(0.2)");
+  activation_case(elu_layer(0.5f), TDO_ACT_ELU, elu, "elu(0.5)");
+  activation_case(selu_layer(), TDO_ACT_SELU, nullptr, "selu");
+  activation_case(softplus_layer(2.f, 5.f), TDO_ACT_SOFTPLUS, sp, "softplus(2,5)");
+  activation_case(softsign_layer(), TDO_ACT_SOFTSIGN, nullptr, "softsign");
+  activation_case(asinh_layer(), TDO_ACT_ASINH, nullptr, "asinh");
+  activation_case(tanh_p1m2_layer(), TDO_ACT_TANH_P1M2, nullptr, "tanh_p1m2");
+  EXPECT(leaky_relu_layer(0.3f).epsilon_value() == 0.3f);
+  EXPECT(elu_layer().layer_type() == "elu-activation");
+}
+
 // -------------------------------------------------- network<sequential>::fit
 template <typename Opt>
 static void net_fit_vs_oracle(const char *name, int opt_kind) {
   std::printf("network<sequential>::fit<cross_entropy_multiclass> with %s vs oracle (short last batch)\n", name);
   network<sequential> nn;
   nn << convolutional_layer(12, 12, 3, 1, 4, padding::same) << tanh_layer()
-     << max_pooling_layer(12, 12, 4, 2) << convolutional_layer(6, 6, 3, 4, 6) << relu_layer()
+     << max_pooling_layer(12, 12, 4, 2) << convolutional_layer(6, 6, 3, 4, 6) << leaky_relu_layer(0.1f)
      << average_pooling_layer(4, 4, 6, 2) << fully_connected_layer(24, 10) << softmax_layer();
   EXPECT(nn.layer_size() == 8);
   EXPECT(nn.in_data_size() == 144 && nn.out_data_size() == 10);
@@ -305,7 +345,7 @@ static void net_fit_vs_oracle(const char *name, int opt_kind) {
   L[1].kind = TDO_L_ACT;  L[1].act = TDO_ACT_TANH;
   L[2].kind = TDO_L_MAXPOOL; L[2].pool = tdo_pool_desc{12, 12, 4, 2, 2, 2, 2, 0, 0};
   L[3].kind = TDO_L_CONV; L[3].conv = tdo_conv_desc{6, 6, 4, 3, 3, 6, 1, 1, 1, 1, 0, 1, nullptr};
-  L[4].kind = TDO_L_ACT;  L[4].act = TDO_ACT_RELU;
+  L[4].kind = TDO_L_ACT;  L[4].act = TDO_ACT_LEAKY_RELU; L[4].act_p[0] = 0.1f;
   L[5].kind = TDO_L_AVEPOOL; L[5].pool = tdo_pool_desc{4, 4, 6, 2, 2, 2, 2, 0, 0};
   L[6].kind = TDO_L_FC; L[6].fc_in = 24; L[6].fc_out = 10; L[6].fc_bias = 1;
   L[7].kind = TDO_L_ACT;  L[7].act = TDO_ACT_SOFTMAX;
@@ -369,6 +409,7 @@ int main() {
     optimizer_kats();
     conv_ops_vs_oracle();
     fc_pool_ops_vs_oracle();
+    activations_vs_oracle();
     net_fit_vs_oracle<gradient_descent>("gradient_descent", TDO_OPT_SGD);
     net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM);
   } catch (const std::exception &e) {

@@ -4,7 +4,7 @@ and against the parameters tiny-dnn's own network<sequential>::fit produced
 import numpy as np
 import pytest
 
-from conftest import assert_close, input_checksum
+from conftest import assert_close, input_checksum, REL_TOL
 
 pytestmark = pytest.mark.gpu
 
@@ -163,3 +163,36 @@ def test_graph_replay_matches_eager_on_every_step(T, W, name, batch):
     for (i, which, a) in params:
         assert np.array_equal(eager.layer_grad(i, which), graph.layer_grad(i, which))
     eager.close(); graph.close()
+
+
+def test_net_with_every_other_activation_matches_oracle(T, O, W):
+    """A small net that chains the parameterised and remaining activation layers: two Adam
+    steps, every layer output, gradient and updated weight against the oracle."""
+    spec = [("conv", 10, 10, 2, 3, 4, True), ("act", "leaky_relu", (0.1,)), ("conv", 10, 10, 4, 3, 4, False),
+            ("act", "elu", (0.7,)), ("avepool", 8, 8, 4, 2), ("act", "selu"), ("fc", 64, 24), ("act", "softplus"),
+            ("fc", 24, 20), ("act", "softsign"), ("fc", 20, 16), ("act", "asinh"), ("fc", 16, 10),
+            ("act", "tanh_p1m2")]
+    batch = 6
+    rng = np.random.default_rng(5)
+    for flags in (0, T.NET_FUSE_ACT_GRAD):
+        net = T.Net(W.build_layers(T, spec), batch, flags)
+        ref = O.OracleNet(W.build_layers(O, spec), batch)
+        for i, l in enumerate(spec):
+            nw, nb, fan_in, _ = W.layer_fans(l)
+            if nw:
+                w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+                b = rng.uniform(-0.1, 0.1, nb).astype(np.float32)
+                net.set_param(i, 0, w); net.set_param(i, 1, b)
+                ref.weight(i)[:] = w; ref.bias(i)[:] = b
+        x = rng.standard_normal((batch, 200)).astype(np.float32)
+        t = rng.uniform(0.1, 0.9, (batch, 10)).astype(np.float32)
+        xd, td = T.to_device(x), T.to_device(t)
+        opt, ropt = T.opt_desc("adam"), O.opt_desc("adam")
+        for step in range(2):
+            net.train_step(opt, "mse", batch, xd, td)
+            ref.train_step(ropt, "mse", x, t)
+            for i, l in enumerate(spec):
+                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"step {step} out {i}")
+                if W.layer_fans(l)[0]:
+                    assert_close(net.get_param(i, 0), ref.weight(i), REL_TOL, f"step {step} w {i}")
+                    assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} b {i}")

@@ -288,6 +288,25 @@ def test_avepool_reference_outputs_and_errors(T, kats, layer_grads):
         T.avepool_fwd(T.pool_desc(5, 5, 1, 2), 1, buf, buf, buf, buf)
 
 
+def test_activation_layers_match_reference_outputs(T, act_golden):
+    """Every activation layer against what the compiled reference produced for the same input."""
+    g = act_golden
+    x, dy = g["x"], g["dy"]
+    xd, dyd = T.to_device(x), T.to_device(dy)
+    names = sorted({f.rsplit(".", 1)[0] for f in g.files if "." in f})
+    assert len(names) == 14
+    for name in names:
+        kind, prm = name.split(".", 1)[1], tuple(float(v) for v in g[name + ".p"])
+        y, dx = T.DevBuf(x.shape), T.DevBuf(x.shape)
+        T.act_fwd(kind, x.shape[0], x.shape[1], xd, y, params=prm)
+        assert_close(y.numpy(), g[name + ".y"], REL_TOL, name + " forward")
+        T.act_bwd(kind, x.shape[0], x.shape[1], T.to_device(g[name + ".y"]), dyd, dx, x=xd, params=prm)
+        assert_close(dx.numpy(), g[name + ".dx"], REL_TOL, name + " backward")
+    # the gradients of selu and softsign read the layer input: refused without it
+    with pytest.raises(T.TdhError, match="reads the layer input"):
+        T.act_bwd("selu", x.shape[0], x.shape[1], xd, dyd, T.DevBuf(x.shape))
+
+
 @pytest.mark.parametrize("kind", ["tanh", "relu", "sigmoid", "softmax"])
 @pytest.mark.parametrize("shape", [(4, 10), (3, 1000), (7, 77), (1, 1), (64, 4099)])
 def test_activations_match_oracle(T, O, kind, shape):

@@ -207,6 +207,47 @@ def test_activation_closed_forms(O, kind):
     assert_close(O.act_bwd(kind, x, got_y, dy), dx, 1e-5, "backward")
 
 
+ACT_FORMS = {
+    # kind: (params, y(x), dy/dx as a function of (x, y)) in float64; formulas are the textbook ones
+    "leaky_relu": ((0.2,), lambda x: np.where(x > 0, x, 0.2 * x), lambda x, y: np.where(x > 0, 1.0, 0.2)),
+    "elu": ((0.5,), lambda x: np.where(x < 0, 0.5 * np.expm1(x), x), lambda x, y: np.where(x > 0, 1.0, 0.5 * np.exp(x))),
+    "selu": (None, lambda x: 1.05070 * np.where(x > 0, x, 1.67326 * np.expm1(x)),
+             lambda x, y: 1.05070 * np.where(x > 0, 1.0, 1.67326 * np.exp(x))),
+    "softplus": ((2.0, 5.0), lambda x: np.where(2 * x > 5, x, np.log1p(np.exp(2 * x)) / 2),
+                 lambda x, y: np.where(2 * y > 5, 1.0, -np.expm1(-2 * y))),
+    "softsign": (None, lambda x: x / (1 + np.abs(x)), lambda x, y: 1 / (1 + np.abs(x)) ** 2),
+    "asinh": (None, np.arcsinh, lambda x, y: 1 / np.sqrt(1 + x * x)),
+    "tanh_p1m2": (None, lambda x: (np.tanh(x) + 1) / 2, lambda x, y: (1 - np.tanh(x) ** 2) / 2),
+}
+
+
+@pytest.mark.parametrize("kind", sorted(ACT_FORMS))
+def test_more_activation_closed_forms(O, kind):
+    """Each layer against its textbook definition and derivative in float64 (the derivative as a
+    function of x, where the layers compute it from y: a dropped term or wrong sign shows)."""
+    prm, f, df = ACT_FORMS[kind]
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((4, 50)) * 2).astype(np.float32)
+    x[np.abs(x) < 1e-3] = 0.5
+    dy = rng.standard_normal((4, 50)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    y = O.act_fwd(kind, x, prm)
+    assert_close(y, f(x64), 2e-6, "forward")
+    assert_close(O.act_bwd(kind, x, y, dy, prm), dy * df(x64, f(x64)), 2e-5, "backward")
+
+
+def test_activation_layers_match_reference_outputs(O, act_golden):
+    """The committed outputs of the compiled reference (tests/golden/make_fixtures.py): bit for bit."""
+    g = act_golden
+    names = sorted({f.rsplit(".", 1)[0] for f in g.files if "." in f})
+    assert len(names) == 14
+    for name in names:
+        kind, prm = name.split(".", 1)[1], tuple(g[name + ".p"])
+        y = O.act_fwd(kind, g["x"], prm)
+        assert np.array_equal(y, g[name + ".y"]), name
+        assert np.array_equal(O.act_bwd(kind, g["x"], y, g["dy"], prm), g[name + ".dx"]), name
+
+
 def test_loss_gradients_and_softmax_xent_identity(O):
     rng = np.random.default_rng(6)
     z = rng.standard_normal((7, 10)).astype(np.float32)

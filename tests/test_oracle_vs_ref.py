@@ -76,6 +76,14 @@ def test_fc_pool_act_loss_opt_bit_exact(ref):
         y = O.act_fwd(kind, xa)
         yr, dxr = O.ref_act(kind, xa, g)
         assert np.array_equal(y, yr) and np.array_equal(O.act_bwd(kind, xa, y, g), dxr)
+    for kind, prm in (("leaky_relu", None), ("leaky_relu", (0.3,)), ("elu", (0.7,)), ("selu", None),
+                      ("selu", (1.2, 0.9)), ("softplus", None), ("softplus", (3.0, 4.0)),
+                      ("softsign", None), ("asinh", None), ("tanh_p1m2", None)):
+        xa = (rng.standard_normal((4, 33)) * 3).astype(np.float32)
+        g = rng.standard_normal((4, 33)).astype(np.float32)
+        y = O.act_fwd(kind, xa, prm)
+        yr, dxr = O.ref_act(kind, xa, g, params=prm)
+        assert np.array_equal(y, yr) and np.array_equal(O.act_bwd(kind, xa, y, g, prm), dxr), kind
     y = O.act_fwd("softmax", rng.standard_normal((4, 10)).astype(np.float32))
     t = np.eye(10, dtype=np.float32)[[1, 3, 5, 7]]
     for kind in ("mse", "ce_multiclass", "ce"):

@@ -20,7 +20,8 @@ LIB_PATH = os.path.join(HERE, "lib", "libtdh.so")
 CSRC = os.path.join(HERE, "csrc")
 HEADER = os.path.join(os.path.dirname(HERE), "include", "tdh.h")
 
-ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3}
+ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3, "leaky_relu": 4, "elu": 5, "selu": 6,
+       "softplus": 7, "softsign": 8, "asinh": 9, "tanh_p1m2": 10}
 LOSS = {"mse": 0, "ce_multiclass": 1, "ce": 2}
 OPT = {"sgd": 0, "momentum": 1, "adam": 2, "adagrad": 3, "rmsprop": 4, "adamax": 5, "nesterov": 6}
 L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT = range(5)
@@ -52,7 +53,8 @@ class OptDesc(C.Structure):
 
 class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("act", C.c_int32), ("conv", ConvDesc), ("pool", PoolDesc),
-                ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32)]
+                ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32),
+                ("act_p", C.c_float * 2)]
 
 
 def build(verbose=False):
@@ -85,6 +87,7 @@ def lib():
                   "tdh_net_layer_argmax"):
             getattr(l, n).restype = C.c_void_p
         l.tdh_opt_default.restype = None
+        l.tdh_act_default_params.restype = None
         _lib = l
     return _lib
 
@@ -307,12 +310,25 @@ def avepool_bwd(d, batch, x, w, dy, dx, dw, db, accumulate=False):
                                 int(accumulate)), "tdh_avepool_bwd")
 
 
-def act_fwd(kind, batch, length, x, y):
-    check(lib().tdh_act_fwd(ACT[kind], batch, length, _p(x), _p(y)), "tdh_act_fwd")
+def act_params(kind, params=None):
+    """The two constructor parameters of an activation layer (the reference's defaults when
+    `params` is None): leaky_relu (epsilon,), elu (alpha,), selu (lambda, alpha), softplus
+    (beta, threshold)."""
+    p = (C.c_float * 2)()
+    lib().tdh_act_default_params(ACT[kind], p)
+    for i, v in enumerate(params or ()):
+        p[i] = v
+    return p
 
 
-def act_bwd(kind, batch, length, y, dy, dx):
-    check(lib().tdh_act_bwd(ACT[kind], batch, length, _p(y), _p(dy), _p(dx)), "tdh_act_bwd")
+def act_fwd(kind, batch, length, x, y, params=None):
+    check(lib().tdh_act_fwd_p(ACT[kind], act_params(kind, params), batch, length, _p(x), _p(y)),
+          "tdh_act_fwd_p")
+
+
+def act_bwd(kind, batch, length, y, dy, dx, x=None, params=None):
+    check(lib().tdh_act_bwd_p(ACT[kind], act_params(kind, params), batch, length, _p(x), _p(y),
+                              _p(dy), _p(dx)), "tdh_act_bwd_p")
 
 
 def loss_grad(kind, batch, length, y, t, dy):
@@ -359,9 +375,10 @@ def L_avepool(in_w, in_h, in_c, pool, stride=None):
     return l
 
 
-def L_act(kind):
+def L_act(kind, params=None):
     l = LayerDesc()
     l.kind, l.act = L_ACT, ACT[kind]
+    l.act_p = act_params(kind, params)
     return l
 
 

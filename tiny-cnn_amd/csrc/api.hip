@@ -482,22 +482,46 @@ int tdh_avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const flo
   return avepool_bwd(d, batch, x, w, dy, dx, dw, db, accumulate);
 }
 
-int tdh_act_fwd(int kind, int batch, int len, const float *x, float *y) {
+void tdh_act_default_params(int kind, float *p) {
+  if (!p) return;
+  p[0] = p[1] = 0.0f;
+  switch (kind) {
+    case TDH_ACT_LEAKY_RELU: p[0] = 0.01f; break;                // leaky_relu_layer.h:25
+    case TDH_ACT_ELU: p[0] = 1.0f; break;                        // elu_layer.h:18
+    case TDH_ACT_SELU: p[0] = 1.05070f; p[1] = 1.67326f; break;  // selu_layer.h:26-27
+    case TDH_ACT_SOFTPLUS: p[0] = 1.0f; p[1] = 20.0f; break;     // softplus_layer.h:26-27
+  }
+}
+
+int tdh_act_fwd_p(int kind, const float *p, int batch, int len, const float *x, float *y) {
   TDH_REQUIRE_INIT();
   TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_act_fwd: negative size");
   if (batch == 0 || len == 0) return TDH_OK;
   TDH_CHECK_ARG(x && y, "tdh_act_fwd: null tensor");
   TDH_CHECK_ARG(static_cast<long>(batch) * len < (1L << 31), "tdh_act_fwd: tensor too large");
-  return launch_act_fwd(kind, batch, len, x, y);
+  float def[2];
+  tdh_act_default_params(kind, def);
+  return launch_act_fwd(kind, p ? p : def, batch, len, x, y);
 }
 
-int tdh_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx) {
+int tdh_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, const float *y,
+                  const float *dy, float *dx) {
   TDH_REQUIRE_INIT();
   TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_act_bwd: negative size");
   if (batch == 0 || len == 0) return TDH_OK;
   TDH_CHECK_ARG(y && dy && dx, "tdh_act_bwd: null tensor");
   TDH_CHECK_ARG(static_cast<long>(batch) * len < (1L << 31), "tdh_act_bwd: tensor too large");
-  return launch_act_bwd(kind, batch, len, y, dy, dx);
+  float def[2];
+  tdh_act_default_params(kind, def);
+  return launch_act_bwd(kind, p ? p : def, batch, len, x, y, dy, dx);
+}
+
+int tdh_act_fwd(int kind, int batch, int len, const float *x, float *y) {
+  return tdh_act_fwd_p(kind, nullptr, batch, len, x, y);
+}
+
+int tdh_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx) {
+  return tdh_act_bwd_p(kind, nullptr, batch, len, nullptr, y, dy, dx);
 }
 
 int tdh_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy) {

@@ -116,8 +116,10 @@ int pool_out_length(int in_length, int window, int stride, int ceil_mode, int pa
 // elementwise.hip
 int launch_fill_zero(void *p, size_t bytes);
 int launch_copy(void *dst, const void *src, size_t bytes);  // bytes % 4 == 0
-int launch_act_fwd(int kind, int batch, int len, const float *x, float *y);
-int launch_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx);
+// p: two constructor parameters (never null); x may be null unless the kind's gradient reads it
+int launch_act_fwd(int kind, const float *p, int batch, int len, const float *x, float *y);
+int launch_act_bwd(int kind, const float *p, int batch, int len, const float *x, const float *y,
+                   const float *dy, float *dx);
 int launch_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
 int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz);
 int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, float *w, float *s0,

@@ -93,6 +93,88 @@ struct SigmoidBwd {
     return dy * y * (1.0f - y);
   }
 };
+// parameterised and remaining pointwise activations; Params = the layer's constructor
+// arguments. Forward: a = x. Backward: a = y (or x where the reference reads x), b = dy.
+struct Act2 {
+  float p0, p1;
+};
+struct LeakyReluFwd {  // leaky_relu_layer.h:74-78, p0 = epsilon
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params p) { return x > 0.0f ? x : p.p0 * x; }
+};
+struct LeakyReluBwd {  // leaky_relu_layer.h:80-88
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params p) { return dy * (y > 0.0f ? 1.0f : p.p0); }
+};
+struct EluFwd {  // elu_layer.h:37-42, p0 = alpha
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params p) {
+    return x < 0.0f ? (p.p0 * (expf(x) - 1.0f)) : x;
+  }
+};
+struct EluBwd {  // elu_layer.h:44-52
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params p) { return dy * (y > 0.0f ? 1.0f : (p.p0 + y)); }
+};
+struct SeluFwd {  // selu_layer.h:82-88, p0 = lambda, p1 = alpha
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params p) {
+    return p.p0 * (x > 0.0f ? x : p.p1 * (expf(x) - 1.0f));
+  }
+};
+struct SeluBwd {  // selu_layer.h:90-99: reads x; the product is a double one in the reference
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float dy, Params p) {
+    return static_cast<float>(dy * p.p0 * (x > 0.0f ? 1.0 : static_cast<double>(p.p1 * expf(x))));
+  }
+};
+struct SoftplusFwd {  // softplus_layer.h:84-90, p0 = beta, p1 = threshold
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params p) {
+    const float betain = p.p0 * x;
+    return betain > p.p1 ? x : (1.0f / p.p0) * log1pf(expf(betain));
+  }
+};
+struct SoftplusBwd {  // softplus_layer.h:92-102
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params p) {
+    const float betaout = p.p0 * y;
+    const float exp_bo  = expf(betaout);
+    return betaout > p.p1 ? dy : dy * (exp_bo - 1.0f) / exp_bo;
+  }
+};
+struct SoftsignFwd {  // softsign_layer.h:24-28 (double arithmetic: `1.0 + std::abs(x)`)
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params) {
+    return static_cast<float>(x / (1.0 + fabsf(x)));
+  }
+};
+struct SoftsignBwd {  // softsign_layer.h:30-40: reads x
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float dy, Params) {
+    const double d = 1.0 + fabsf(x);
+    return static_cast<float>(dy / (d * d));
+  }
+};
+struct AsinhFwd {  // asinh_layer.h:24-28
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params) { return asinhf(x); }
+};
+struct AsinhBwd {  // asinh_layer.h:30-38
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params) { return dy / coshf(y); }
+};
+struct TanhP1m2Fwd {  // tanh_p1m2_layer.h:24-30
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float x, float, Params) {
+    const float ep = expf(x);
+    return ep / (ep + (1.0f / ep));
+  }
+};
+struct TanhP1m2Bwd {  // tanh_p1m2_layer.h:32-40
+  typedef Act2 Params;
+  static __device__ __forceinline__ float apply(float y, float dy, Params) { return dy * (2.0f * y * (1.0f - y)); }
+};
 // loss gradients: loss_function.h:28-36, :143-150, :120-128.  a = y, b = t
 struct MseGrad {
   struct Params {
@@ -437,9 +519,17 @@ int launch_copy(void *dst, const void *src, size_t bytes) {
   return TDH_OK;
 }
 
-int launch_act_fwd(int kind, int batch, int len, const float *x, float *y) {
+int launch_act_fwd(int kind, const float *p, int batch, int len, const float *x, float *y) {
   const size_t n = static_cast<size_t>(batch) * len;
+  const Act2 prm{p[0], p[1]};
   switch (kind) {
+    case TDH_ACT_LEAKY_RELU: return launch_map<LeakyReluFwd, false>(x, nullptr, y, n, prm, "act_fwd_leaky_relu");
+    case TDH_ACT_ELU: return launch_map<EluFwd, false>(x, nullptr, y, n, prm, "act_fwd_elu");
+    case TDH_ACT_SELU: return launch_map<SeluFwd, false>(x, nullptr, y, n, prm, "act_fwd_selu");
+    case TDH_ACT_SOFTPLUS: return launch_map<SoftplusFwd, false>(x, nullptr, y, n, prm, "act_fwd_softplus");
+    case TDH_ACT_SOFTSIGN: return launch_map<SoftsignFwd, false>(x, nullptr, y, n, prm, "act_fwd_softsign");
+    case TDH_ACT_ASINH: return launch_map<AsinhFwd, false>(x, nullptr, y, n, prm, "act_fwd_asinh");
+    case TDH_ACT_TANH_P1M2: return launch_map<TanhP1m2Fwd, false>(x, nullptr, y, n, prm, "act_fwd_tanh_p1m2");
     case TDH_ACT_TANH: return launch_map<TanhFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_tanh");
     case TDH_ACT_RELU: return launch_map<ReluFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_relu");
     case TDH_ACT_SIGMOID: return launch_map<SigmoidFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_sigmoid");
@@ -454,9 +544,20 @@ int launch_act_fwd(int kind, int batch, int len, const float *x, float *y) {
   return set_error(TDH_ERR_INVALID, "activation kind %d is not supported", kind);
 }
 
-int launch_act_bwd(int kind, int batch, int len, const float *y, const float *dy, float *dx) {
+int launch_act_bwd(int kind, const float *p, int batch, int len, const float *x, const float *y,
+                   const float *dy, float *dx) {
   const size_t n = static_cast<size_t>(batch) * len;
+  const Act2 prm{p[0], p[1]};
+  if ((kind == TDH_ACT_SELU || kind == TDH_ACT_SOFTSIGN) && x == nullptr)
+    return set_error(TDH_ERR_INVALID, "the gradient of activation kind %d reads the layer input x", kind);
   switch (kind) {
+    case TDH_ACT_LEAKY_RELU: return launch_map<LeakyReluBwd, true>(y, dy, dx, n, prm, "act_grad_leaky_relu");
+    case TDH_ACT_ELU: return launch_map<EluBwd, true>(y, dy, dx, n, prm, "act_grad_elu");
+    case TDH_ACT_SELU: return launch_map<SeluBwd, true>(x, dy, dx, n, prm, "act_grad_selu");
+    case TDH_ACT_SOFTPLUS: return launch_map<SoftplusBwd, true>(y, dy, dx, n, prm, "act_grad_softplus");
+    case TDH_ACT_SOFTSIGN: return launch_map<SoftsignBwd, true>(x, dy, dx, n, prm, "act_grad_softsign");
+    case TDH_ACT_ASINH: return launch_map<AsinhBwd, true>(y, dy, dx, n, prm, "act_grad_asinh");
+    case TDH_ACT_TANH_P1M2: return launch_map<TanhP1m2Bwd, true>(y, dy, dx, n, prm, "act_grad_tanh_p1m2");
     case TDH_ACT_TANH: return launch_map<TanhBwd, true>(y, dy, dx, n, NoParams(), "act_grad_tanh");
     case TDH_ACT_RELU: return launch_map<ReluBwd, true>(y, dy, dx, n, NoParams(), "act_grad_relu");
     case TDH_ACT_SIGMOID: return launch_map<SigmoidBwd, true>(y, dy, dx, n, NoParams(), "act_grad_sigmoid");

@@ -114,7 +114,7 @@ int forward(tdh_net *net, int batch, const float *x) {
       case TDH_L_MAXPOOL: TDH_TRY(maxpool_fwd(&s.pool, batch, in, L.out, L.argmax)); break;
       case TDH_L_AVEPOOL: TDH_TRY(avepool_fwd(&s.pool, batch, in, L.w, L.b, L.out)); break;
       case TDH_L_ACT:
-        TDH_TRY(launch_act_fwd(s.act, batch, static_cast<int>(L.out_size), in, L.out));
+        TDH_TRY(launch_act_fwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out));
         break;
     }
     in = L.out;
@@ -359,7 +359,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         break;
       case TDH_L_ACT:
         if (!L.grad_folded)
-          TDH_TRY(launch_act_bwd(s.act, batch, static_cast<int>(L.out_size), L.out, L.dout, dx));
+          TDH_TRY(launch_act_bwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out, L.dout, dx));
         break;
     }
   }

@@ -877,27 +877,85 @@ class average_pooling_layer : public layer {
   std::shared_ptr<core::OpKernel> kernel_fwd_, kernel_back_;
 };
 
-// activation layers (tiny_dnn/activations/*.h): shape is inherited from the previous layer
-template <int KIND>
-class activation_layer_t : public layer {
+// activation layers (tiny_dnn/activations/*.h): shape is inherited from the previous layer;
+// forward_activation / backward_activation keep the reference's signatures
+// (activation_layer.h:93-112) on single samples
+class activation_layer : public layer {
  public:
-  activation_layer_t() {}
-  std::string layer_type() const override {
-    return KIND == TDH_ACT_TANH ? "tanh-activation" : KIND == TDH_ACT_RELU ? "relu-activation"
-           : KIND == TDH_ACT_SOFTMAX ? "softmax-activation" : "sigmoid-activation";
-  }
+  std::string layer_type() const override { return type_; }
   layer_desc describe(const shape3d &) const override {
     layer_desc r;
     std::memset(&r.l, 0, sizeof(r.l));
-    r.l.kind = TDH_L_ACT;
-    r.l.act  = KIND;
+    r.l.kind     = TDH_L_ACT;
+    r.l.act      = kind_;
+    r.l.act_p[0] = p_[0];
+    r.l.act_p[1] = p_[1];
     return r;
   }
+  void forward_activation(const vec_t &x, vec_t &y) {
+    detail::ensure_init();
+    const int n = static_cast<int>(x.size());
+    y.resize(x.size());
+    buffers &s = scratch();
+    s.b.resize(x.size());
+    detail::check(tdh_act_fwd_p(kind_, p_, 1, n, s.a.upload(x, x.size()), s.b.get()));
+    if (n) detail::check(tdh_memcpy_d2h(y.data(), s.b.get(), x.size() * sizeof(float)));
+  }
+  void backward_activation(const vec_t &x, const vec_t &y, vec_t &dx, const vec_t &dy) {
+    detail::ensure_init();
+    const int n = static_cast<int>(y.size());
+    dx.resize(y.size());
+    buffers &s = scratch();
+    s.d.resize(y.size());
+    detail::check(tdh_act_bwd_p(kind_, p_, 1, n, s.a.upload(x, x.size()), s.b.upload(y, y.size()),
+                                s.c.upload(dy, dy.size()), s.d.get()));
+    if (n) detail::check(tdh_memcpy_d2h(dx.data(), s.d.get(), y.size() * sizeof(float)));
+  }
+
+ protected:
+  activation_layer(int kind, const char *type, float p0 = 0.f, float p1 = 0.f)
+    : kind_(kind), type_(type) {
+    p_[0] = p0;
+    p_[1] = p1;
+  }
+  int kind_;
+  const char *type_;
+  float p_[2];
+
+ private:
+  struct buffers {
+    detail::device_tensor a, b, c, d;
+  };
+  buffers &scratch() {
+    if (!buf_) buf_.reset(new buffers());
+    return *buf_;
+  }
+  std::shared_ptr<buffers> buf_;  // copies of a layer share their device scratch, like the ops
 };
-typedef activation_layer_t<TDH_ACT_TANH> tanh_layer;
-typedef activation_layer_t<TDH_ACT_RELU> relu_layer;
-typedef activation_layer_t<TDH_ACT_SOFTMAX> softmax_layer;
-typedef activation_layer_t<TDH_ACT_SIGMOID> sigmoid_layer;
+struct tanh_layer : activation_layer { tanh_layer() : activation_layer(TDH_ACT_TANH, "tanh-activation") {} };
+struct relu_layer : activation_layer { relu_layer() : activation_layer(TDH_ACT_RELU, "relu-activation") {} };
+struct softmax_layer : activation_layer { softmax_layer() : activation_layer(TDH_ACT_SOFTMAX, "softmax-activation") {} };
+struct sigmoid_layer : activation_layer { sigmoid_layer() : activation_layer(TDH_ACT_SIGMOID, "sigmoid-activation") {} };
+// leaky_relu_layer.h:25, elu_layer.h:18, selu_layer.h:26-27, softplus_layer.h:26-27
+struct leaky_relu_layer : activation_layer {
+  explicit leaky_relu_layer(const float_t epsilon = float_t(0.01))
+    : activation_layer(TDH_ACT_LEAKY_RELU, "leaky-relu-activation", epsilon) {}
+  float_t epsilon_value() const { return p_[0]; }
+};
+struct elu_layer : activation_layer {
+  explicit elu_layer(const float_t alpha = float_t(1.0)) : activation_layer(TDH_ACT_ELU, "elu-activation", alpha) {}
+};
+struct selu_layer : activation_layer {
+  explicit selu_layer(const float_t lambda = float_t(1.05070), const float_t alpha = float_t(1.67326))
+    : activation_layer(TDH_ACT_SELU, "selu-activation", lambda, alpha) {}
+};
+struct softplus_layer : activation_layer {
+  explicit softplus_layer(const float_t beta = float_t(1.0), const float_t threshold = float_t(20.0))
+    : activation_layer(TDH_ACT_SOFTPLUS, "softplus-activation", beta, threshold) {}
+};
+struct softsign_layer : activation_layer { softsign_layer() : activation_layer(TDH_ACT_SOFTSIGN, "softsign-activation") {} };
+struct asinh_layer : activation_layer { asinh_layer() : activation_layer(TDH_ACT_ASINH, "asinh-activation") {} };
+struct tanh_p1m2_layer : activation_layer { tanh_p1m2_layer() : activation_layer(TDH_ACT_TANH_P1M2, "tanh-scaled-activation") {} };
 
 struct sequential {};
 

@@ -66,7 +66,7 @@ def build_layers(api, spec):
         elif kind == "avepool":
             out.append(api.L_avepool(l[1], l[2], l[3], l[4]))
         elif kind == "act":
-            out.append(api.L_act(l[1]))
+            out.append(api.L_act(l[1], l[2] if len(l) > 2 else None))
         else:
             raise ValueError(kind)
     return out
