@@ -1,13 +1,17 @@
 // Tests of the C++ host mirror (tiny_dnn_hip.h) on a GPU: the reference's own known-answer
 // tests for this path, written against the same class names, plus random cases checked against
 // the CPU oracle (oracle/td_oracle.h). Built by tests/host_cpp/Makefile, run by
-// tests/test_gpu_host_cpp.py.
+// tests/test_gpu_zz_host_cpp.py.
 //
 // Known answers come from the reference's test-suite:
 //   convolutional.with_stride   test/test_convolutional_layer.h:133-200
 //   fully_connected.forward     test/test_fully_connected_layer.h:48-64
 //   max_pool.forward/backward   test/test_max_pooling_layer.h:25-39, 85-110, 251-281
 //   optimizers                  test/test_optimizers.h:15-190
+#include <execinfo.h>
+#include <signal.h>
+#include <unistd.h>
+
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -401,7 +405,21 @@ static void net_fit_vs_oracle(const char *name, int opt_kind) {
   tdo_net_destroy(ref);
 }
 
+// a crash of the host process names its call chain instead of dying silently
+static void on_fatal_signal(int sig) {
+  void *frames[64];
+  const int n = backtrace(frames, 64);
+  const char msg[] = "FATAL SIGNAL, backtrace:\n";
+  (void)!write(2, msg, sizeof(msg) - 1);
+  backtrace_symbols_fd(frames, n, 2);
+  _exit(128 + sig);
+}
+
 int main() {
+  setvbuf(stdout, nullptr, _IONBF, 0);  // every case is named before it runs
+  signal(SIGSEGV, on_fatal_signal);
+  signal(SIGBUS, on_fatal_signal);
+  signal(SIGABRT, on_fatal_signal);
   try {
     conv_with_stride();
     fc_forward();

@@ -5,7 +5,8 @@ tests/host_cpp/test_host.cpp re-states the reference's own tests for this path
 test/test_max_pooling_layer.h:25-39,85-110,251-281, test/test_optimizers.h:15-190) against the
 mirrored class names and checks random cases and network<sequential>::fit against the CPU oracle,
 tolerance 1e-4 relative (max-pool exact). The binary is built beforehand by
-`make -C tests/host_cpp` (done by __graft_entry__.build()).
+`make -C tests/host_cpp` (done by __graft_entry__.build()). The file name sorts after the other
+GPU tests: the binary is a child process, and `pytest -x` should not let its failure hide them.
 """
 import os
 import subprocess

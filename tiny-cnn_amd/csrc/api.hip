@@ -27,8 +27,16 @@ int set_error(int code, const char *fmt, ...) {
   return code;
 }
 
+StreamSwap::StreamSwap(hipStream_t s) : saved(ctx().stream) { ctx().stream = s; }
+StreamSwap::~StreamSwap() { ctx().stream = saved; }
+
 int ws_begin(size_t total) {
   Context &c = ctx();
+  if (c.ws_keep) {
+    if (c.workspace_off + total <= c.workspace_size) return TDH_OK;
+    return set_error(TDH_ERR_INVALID, "scratch reservation of %zu more bytes exceeds the locked %zu",
+                     total, c.workspace_size);
+  }
   c.workspace_off = 0;
   if (total <= c.workspace_size) return TDH_OK;
   if (c.ws_locked)
@@ -212,6 +220,8 @@ int tdh_shutdown(void) {
   if (!c.ready) return TDH_OK;
   TDH_HIP(hipStreamSynchronize(c.stream));
   if (c.workspace) TDH_HIP(hipFree(c.workspace));
+  for (hipStream_t s : c.side)
+    if (s) TDH_HIP(hipStreamDestroy(s));
   TDH_HIP(hipStreamDestroy(c.stream));
   c = Context();
   return TDH_OK;

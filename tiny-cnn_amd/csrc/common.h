@@ -27,6 +27,17 @@ struct Context {
   size_t workspace_size = 0;
   size_t workspace_off  = 0;
   bool ws_locked        = false;  // a network owns the reservation: ops must fit, never grow
+  bool ws_keep          = false;  // ws_begin does not rewind: pieces handed out stay disjoint
+  // two more streams (default priority) for work that branches off the main one inside a
+  // captured train step; created on first use
+  hipStream_t side[2]   = {nullptr, nullptr};
+};
+
+// Runs the launches of a scope on another stream of the context.
+struct StreamSwap {
+  hipStream_t saved;
+  explicit StreamSwap(hipStream_t s);
+  ~StreamSwap();
 };
 
 Context &ctx();
@@ -152,11 +163,17 @@ struct ActGrad {
 };
 
 // conv.hip / fc.hip
+// prepacked: filters already packed by conv_pack_filters for this direction (and only then)
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
-               float *y, const uint8_t *tbl_resident = nullptr);
+               float *y, const uint8_t *tbl_resident = nullptr, const float *prepacked = nullptr);
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
-               const uint8_t *tbl_resident = nullptr);
+               const uint8_t *tbl_resident = nullptr, const float *prepacked_dx = nullptr);
+// true when forward (flip = 0) / dX (flip = 1) of this layer reads packed filters
+bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip);
+// packs w (masked by the device-resident connection table, if any) into wp[k_w*k_h*in_c*out_c]
+int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const uint8_t *tbl_resident,
+                      float *wp);
 int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *b, float *y);
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
@@ -168,7 +185,10 @@ size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip,
                                int OH, int OW, int ph, int pw);
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
-                int OW, int ph, int pw, ActGrad ag, const char *tag);
+                int OW, int ph, int pw, ActGrad ag, const char *tag,
+                const float *prepacked = nullptr);
+int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const uint8_t *tbl_dev,
+                   float *wp);
 // conv_dw.hip: stride-1 weight gradient from LDS-staged tiles (3x3 and 5x5 windows)
 bool conv_dw_halo_applicable(int R, int S, int batch, int C, int Kc, int H, int W, int OH, int OW,
                              int ph, int pw);

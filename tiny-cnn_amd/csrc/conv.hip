@@ -460,9 +460,29 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
   return TDH_OK;
 }
 
-int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
-               float *y, const uint8_t *tbl_resident) {
+bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip) {
   const ConvGeom g = make_geom(d);
+  if (g.sh != 1 || g.sw != 1) return false;
+  if (!flip)
+    return g.dh == 1 && g.dw == 1 &&
+           conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
+  DxsPlan dxs;
+  if (small_cin_dx_plan(g, dxs)) return false;
+  return conv_s1_applicable(g.R, g.S, batch, g.Kc, g.C, g.OH, g.OW, g.H, g.W, g.R - 1 - g.pad_h,
+                            g.S - 1 - g.pad_w);
+}
+
+int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const uint8_t *tbl_resident,
+                      float *wp) {
+  return conv_s1_repack(d->k_h, d->k_w, d->in_c, d->out_c, flip, w, d->tbl ? tbl_resident : nullptr, wp);
+}
+
+int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
+               float *y, const uint8_t *tbl_resident, const float *prepacked) {
+  const ConvGeom g = make_geom(d);
+  if (prepacked)
+    return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
+                       g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
@@ -480,9 +500,15 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
 
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
-               const uint8_t *tbl_resident) {
+               const uint8_t *tbl_resident, const float *prepacked_dx) {
   const ConvGeom g = make_geom(d);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
+  if (dx && prepacked_dx) {
+    TDH_TRY(conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 1, dy, w, nullptr, nullptr, dx, g.OH, g.OW, g.H,
+                        g.W, g.R - 1 - g.pad_h, g.S - 1 - g.pad_w, dx_act, "conv_dx_s1", prepacked_dx));
+    dx = nullptr;
+    if (!dw && !db) return TDH_OK;
+  }
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));

@@ -406,21 +406,31 @@ size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip,
   return total;
 }
 
+// wp = the filter in the kernel's layout [tap][kc][m] (R*S*C*Kc floats); flip as in conv_s1_run
+int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const uint8_t *tbl_dev,
+                   float *wp) {
+  ProfScope prof("conv_repack_weights", 8.0 * R * S * C * Kc, WORK_BYTE);
+  hipLaunchKernelGGL(repack_weights_kernel, dim3(ceil_div(R * S * C * Kc, 256)), dim3(256), 0,
+                     ctx().stream, w, tbl_dev, wp, C, Kc, R * S, flip);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
 // Runs out = conv(in, repack(w)) (+ bias) (* act'(y)); the caller has checked applicability
-// and reserved conv_s1_workspace_bytes of scratch. flip = 0: forward, 1: dX.
+// and reserved conv_s1_workspace_bytes of scratch. flip = 0: forward, 1: dX. prepacked: the
+// result of conv_s1_repack for this filter, when the caller already has it (w is not read).
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
-                int OW, int ph, int pw, ActGrad ag, const char *tag) {
+                int OW, int ph, int pw, ActGrad ag, const char *tag, const float *prepacked) {
   const int KC = flip ? Kc : C, MC = flip ? C : Kc;
   S1Plan p = make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw);
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_s1_run: shape not supported");
-  void *wp = nullptr;
-  TDH_TRY(ws_take(sizeof(float) * static_cast<size_t>(R) * S * C * Kc, &wp));
-  {
-    ProfScope prof("conv_repack_weights", 8.0 * R * S * C * Kc, WORK_BYTE);
-    hipLaunchKernelGGL(repack_weights_kernel, dim3(ceil_div(R * S * C * Kc, 256)), dim3(256), 0,
-                       ctx().stream, w, tbl_dev, static_cast<float *>(wp), C, Kc, R * S, flip);
-    TDH_LAUNCH_CHECK();
+  const void *wp = prepacked;
+  if (!prepacked) {
+    void *fresh = nullptr;
+    TDH_TRY(ws_take(sizeof(float) * static_cast<size_t>(R) * S * C * Kc, &fresh));
+    TDH_TRY(conv_s1_repack(R, S, C, Kc, flip, w, tbl_dev, static_cast<float *>(fresh)));
+    wp = fresh;
   }
   p.args.in = in; p.args.wp = static_cast<const float *>(wp); p.args.bias = bias;
   p.args.out = out; p.args.ag = ag;

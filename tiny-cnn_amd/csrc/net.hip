@@ -19,6 +19,9 @@ struct tdh_net {
     float *dout = nullptr;  // gradient w.r.t. out; the next layer's backward writes it
     int32_t *argmax = nullptr;
     bool grad_folded = false;  // activation whose backward runs in the next layer's dX epilogue
+    // filters in the LDS-halo kernels' layout for forward / dX, packed on a side stream at the
+    // start of a captured step (stride-1 conv layers of a TDH_NET_GRAPH net)
+    float *wp_fwd = nullptr, *wp_dx = nullptr;
   };
   std::vector<Layer> layers;
   int max_batch  = 0;
@@ -37,7 +40,9 @@ struct tdh_net {
     tdh_opt hyper = {};                 // hyper-parameters only (powers zeroed)
   } graph_key;
   float mirror_b1_t = 0.0f, mirror_b2_t = 0.0f;  // what the device copy of the powers holds
-  size_t scratch = 0;        // largest per-op scratch need
+  size_t scratch = 0;        // largest per-op scratch need; with TDH_NET_GRAPH the sum over the
+                             // layers, because branches of the captured step run side by side
+  std::vector<hipEvent_t> events;  // fork/join points of the captured step
   std::vector<void *> allocs;
 };
 
@@ -98,14 +103,42 @@ bool is_pointwise_act(int act) {
   return act == TDH_ACT_TANH || act == TDH_ACT_RELU || act == TDH_ACT_SIGMOID;
 }
 
-int forward(tdh_net *net, int batch, const float *x) {
+// Whether the captured step of this net branches (weight and bias gradients and filter
+// packing beside the main chain): mid-sized steps only. With tiny kernels the cross-queue
+// synchronisation costs more than it hides, and products that fill the chip for hundreds of
+// microseconds only fight the main chain for its caches (measured: LeNet-style net 5 % slower,
+// VGG-style 1 % slower, CIFAR-10-shape net 12 % faster with branches).
+bool net_forks(const tdh_net *net, int batch) {
+  double macs = 0.0;
+  for (const tdh_net::Layer &L : net->layers) {
+    if (L.spec.kind == TDH_L_CONV)
+      macs += static_cast<double>(L.out_size) * L.spec.conv.in_c * L.spec.conv.k_w * L.spec.conv.k_h;
+    else if (L.spec.kind == TDH_L_FC)
+      macs += static_cast<double>(L.spec.fc_in) * L.spec.fc_out;
+  }
+  const double flop = 2.0 * batch * macs;  // of the forward pass
+  return flop >= 1e8 && flop <= 3e10;
+}
+bool layer_forks(const tdh_net::Layer &L) {
+  return L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC;
+}
+
+// packed: the layers' wp_fwd are being filled on side stream 0 (events n+i mark them ready)
+int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
   const float *in = x;
-  for (auto &L : net->layers) {
+  const int n     = static_cast<int>(net->layers.size());
+  for (int i = 0; i < n; ++i) {
+    tdh_net::Layer &L  = net->layers[i];
     const tdh_layer &s = L.spec;
     switch (s.kind) {
       case TDH_L_CONV:
         TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
-        TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev));
+        if (packed && L.wp_fwd && layer_forks(L) && conv_uses_packed(&s.conv, batch, 0)) {
+          TDH_HIP(hipStreamWaitEvent(ctx().stream, net->events[n + i], 0));
+          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, L.wp_fwd));
+        } else {
+          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev));
+        }
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
@@ -180,6 +213,11 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       if ((rc = net_alloc(net, act, &p, true))) break;
       L.argmax = reinterpret_cast<int32_t *>(p);
     }
+    if ((flags & TDH_NET_GRAPH) && L.spec.kind == TDH_L_CONV && L.spec.conv.w_stride == 1 &&
+        L.spec.conv.h_stride == 1) {
+      if ((rc = net_alloc(net, L.w_size, &L.wp_fwd, false))) break;
+      if ((rc = net_alloc(net, L.w_size, &L.wp_dx, false))) break;
+    }
     if (!L.tbl.empty()) {
       float *p = nullptr;
       if ((rc = net_alloc(net, ceil_div_sz(L.tbl.size(), sizeof(float)), &p, false))) break;
@@ -190,7 +228,10 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
     if (L.spec.kind == TDH_L_CONV) need = conv2d_workspace_bytes(&L.spec.conv, max_batch);
     if (L.spec.kind == TDH_L_FC) need = fc_workspace_bytes(L.spec.fc_in, L.spec.fc_out, max_batch);
     if (L.spec.kind == TDH_L_AVEPOOL) need = avepool_workspace_bytes(&L.spec.pool, max_batch);
-    if (need > net->scratch) net->scratch = need;
+    if (flags & TDH_NET_GRAPH)  // three times: dX, dW and db are separate calls of the operator there
+      net->scratch += 3 * ws_align(need);
+    else if (need > net->scratch)
+      net->scratch = need;
     // fold pointwise activation gradients into the following conv/fc dX epilogue
     if ((flags & TDH_NET_FUSE_ACT_GRAD) && L.spec.kind == TDH_L_ACT &&
         is_pointwise_act(L.spec.act) && i + 1 < n_layers &&
@@ -231,9 +272,25 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
     }
   }
   if (rc == TDH_OK) rc = net_alloc(net, 2, &net->dev_powers, true);
+  if (rc == TDH_OK && (flags & TDH_NET_GRAPH)) {
+    Context &c = ctx();
+    for (hipStream_t &s : c.side)
+      if (!s && hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess)
+        rc = set_error(TDH_ERR_HIP, "tdh_net_create: cannot create a side stream");
+    // events: [0,n) gradient forks, [n,2n) packed forward filters, 2n and 2n+1 joins,
+    // 2n+2 start of the step, 2n+3 packed dX filters
+    for (int i = 0; rc == TDH_OK && i < 2 * n_layers + 4; ++i) {
+      hipEvent_t e = nullptr;
+      if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess)
+        rc = set_error(TDH_ERR_HIP, "tdh_net_create: cannot create an event");
+      else
+        net->events.push_back(e);
+    }
+  }
   // reserve the scratch every layer may need, so that no op ever has to grow it
   if (rc == TDH_OK) rc = ws_begin(net->scratch);
   if (rc != TDH_OK) {
+    for (hipEvent_t e : net->events) (void)hipEventDestroy(e);
     for (void *p : net->allocs) (void)hipFree(p);
     delete net;
     return rc;
@@ -247,6 +304,7 @@ int tdh_net_destroy(tdh_net *net) {
   if (!net) return TDH_OK;
   TDH_HIP(hipStreamSynchronize(ctx().stream));
   if (net->graph_exec) TDH_HIP(hipGraphExecDestroy(net->graph_exec));
+  for (hipEvent_t e : net->events) TDH_HIP(hipEventDestroy(e));
   for (void *p : net->allocs) TDH_HIP(hipFree(p));
   delete net;
   return TDH_OK;
@@ -311,12 +369,57 @@ int tdh_net_forward(tdh_net *net, int batch, const float *x) {
   return forward(net, batch, x);
 }
 
-// Queues one whole train step on the library stream.
+// Queues one whole train step on the library stream. forked (only while the stream is being
+// captured): the weight and bias gradients of every conv / fc layer branch off onto the side
+// stream, because nothing before the optimizer waits for them; the main stream carries only
+// the chain forward -> loss -> dX ... -> dX, and the two join in front of the optimizer. The
+// kernels and their arguments are the same either way, so are the results.
 static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
-                        const float *t, int do_update, float *dev_powers) {
-  TDH_TRY(forward(net, batch, x));
-  const int n          = static_cast<int>(net->layers.size());
+                        const float *t, int do_update, float *dev_powers, bool forked = false) {
+  Context &c = ctx();
+  struct KeepScratch {  // hands out disjoint scratch pieces for the whole backward pass
+    Context &c;
+    bool on;
+    KeepScratch(Context &cc, bool o) : c(cc), on(o) {}
+    void start() { if (on) { c.workspace_off = 0; c.ws_keep = true; } }
+    ~KeepScratch() { c.ws_keep = false; }
+  } keep(c, forked);
+  bool side_used[2] = {false, false};
+  const int n   = static_cast<int>(net->layers.size());
+  bool packed_dx = false;
+  if (forked) {
+    // the filters do not change until the optimizer runs: pack them for every layer now, beside
+    // the forward pass, instead of in front of each convolution
+    bool any = false;
+    for (int i = 0; i < n; ++i) {
+      tdh_net::Layer &L = net->layers[i];
+      if (!L.wp_fwd || !layer_forks(L)) continue;
+      const bool f = conv_uses_packed(&L.spec.conv, batch, 0), b = conv_uses_packed(&L.spec.conv, batch, 1);
+      if (!f && !b) continue;
+      if (!any) {
+        TDH_HIP(hipEventRecord(net->events[2 * n + 2], c.stream));
+        TDH_HIP(hipStreamWaitEvent(c.side[0], net->events[2 * n + 2], 0));
+        any = true;
+      }
+      StreamSwap on_side(c.side[0]);
+      if (f) {
+        TDH_TRY(conv_pack_filters(&L.spec.conv, 0, L.w, L.tbl_dev, L.wp_fwd));
+        TDH_HIP(hipEventRecord(net->events[n + i], c.side[0]));
+      }
+    }
+    for (int i = 0; i < n; ++i) {
+      tdh_net::Layer &L = net->layers[i];
+      if (!L.wp_dx || !layer_forks(L) || !conv_uses_packed(&L.spec.conv, batch, 1)) continue;
+      StreamSwap on_side(c.side[0]);
+      TDH_TRY(conv_pack_filters(&L.spec.conv, 1, L.w, L.tbl_dev, L.wp_dx));
+      packed_dx = true;
+    }
+    if (packed_dx) TDH_HIP(hipEventRecord(net->events[2 * n + 3], c.side[0]));
+    side_used[0] = any;
+  }
+  TDH_TRY(forward(net, batch, x, forked));
   tdh_net::Layer &last = net->layers[n - 1];
+  bool waited_dx = false;
   int first_bwd        = n - 1;
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
   // the full softmax Jacobian
@@ -329,12 +432,21 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     TDH_TRY(launch_loss_grad(loss_kind, batch, static_cast<int>(last.out_size), last.out, t,
                              last.dout));
   }
+  keep.start();
   for (int i = first_bwd; i >= 0; --i) {
     tdh_net::Layer &L  = net->layers[i];
     const tdh_layer &s = L.spec;
     const float *in    = i == 0 ? x : net->layers[i - 1].out;
     float *dx          = i == 0 ? net->dx_in : net->layers[i - 1].dout;
     ActGrad fold;
+    const bool fork = forked && layer_forks(L);
+    if (fork) {
+      // this layer's output gradient is complete here: let the side streams start from it
+      TDH_HIP(hipEventRecord(net->events[i], c.stream));
+      TDH_HIP(hipStreamWaitEvent(c.side[0], net->events[i], 0));
+      TDH_HIP(hipStreamWaitEvent(c.side[1], net->events[i], 0));
+      side_used[0] = side_used[1] = true;
+    }
     if (i >= 1 && net->layers[i - 1].grad_folded) {
       // write straight into the activation's input gradient, scaled by act'(its output)
       fold.kind = net->layers[i - 1].spec.act;
@@ -343,14 +455,48 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     }
     switch (s.kind) {
       case TDH_L_CONV:
-        TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
-        TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
-                           fold, L.tbl_dev));
+        TDH_TRY(ws_begin((forked ? 3 : 1) * conv2d_workspace_bytes(&s.conv, batch)));
+        if (forked) {
+          const float *wp = packed_dx && fork && L.wp_dx && conv_uses_packed(&s.conv, batch, 1) ? L.wp_dx : nullptr;
+          if (wp && !waited_dx) {
+            TDH_HIP(hipStreamWaitEvent(c.stream, net->events[2 * n + 3], 0));
+            waited_dx = true;
+          }
+          if (!fork) {
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1, fold,
+                               L.tbl_dev, wp));
+            break;
+          }
+          TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+          {
+            StreamSwap on_side(c.side[0]);
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad(), L.tbl_dev));
+          }
+          if (L.b_size) {
+            StreamSwap on_side(c.side[1]);
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));
+          }
+        } else {
+          TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
+                             fold, L.tbl_dev));
+        }
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
-        TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
-                       L.b_size ? L.db : nullptr, 1, fold));
+        if (fork) {
+          TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
+          {
+            StreamSwap on_side(c.side[0]);
+            TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad()));
+          }
+          if (L.b_size) {
+            StreamSwap on_side(c.side[1]);
+            TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad()));
+          }
+        } else {
+          TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
+                         L.b_size ? L.db : nullptr, 1, fold));
+        }
         break;
       case TDH_L_MAXPOOL: TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx)); break;
       case TDH_L_AVEPOOL:
@@ -362,6 +508,11 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           TDH_TRY(launch_act_bwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out, L.dout, dx));
         break;
     }
+  }
+  for (int k = 0; k < 2; ++k) {  // the optimizer (and the end of the capture) wait for the branches
+    if (!side_used[k]) continue;
+    TDH_HIP(hipEventRecord(net->events[2 * n + k], c.side[k]));
+    TDH_HIP(hipStreamWaitEvent(c.stream, net->events[2 * n + k], 0));
   }
   if (!do_update) return TDH_OK;
   // nodes::update_weights visits layers front to back, weight before bias; the gradient
@@ -409,7 +560,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
       tdh_opt capture_opt;
       if (opt) capture_opt = *opt;
       rc = enqueue_step(net, opt ? &capture_opt : nullptr, loss_kind, batch, x, t, do_update,
-                        net->dev_powers);
+                        net->dev_powers, /*forked=*/net_forks(net, batch));
       e = hipStreamEndCapture(c.stream, &graph);
     }
     c.ws_locked = false;
