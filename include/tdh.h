@@ -253,6 +253,23 @@ int tdh_net_forward(tdh_net *net, int batch, const float *x);
 int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
                        const float *t, int do_update);
 
+/* ------------------------------------------------ batches from host memory */
+/* network::fit hands each mini-batch over as host vectors (tiny_dnn/network.h:866-879;
+ * layer::set_in_data copies them into the first layer, tiny_dnn/layers/layer.h:230-251).
+ * A feeder uploads them double-buffered: tdh_feeder_stage copies batch k+1 from pageable
+ * host memory into a pinned slot and queues its upload on a copy stream while the step on
+ * batch k runs; tdh_feeder_acquire makes the library stream wait for that upload and returns
+ * the device pointers to hand to tdh_net_train_step / tdh_net_forward. Calls alternate
+ * stage, acquire, stage, acquire ...; x: [batch][x_len], t: [batch][t_len] floats. The host
+ * copy runs on a worker thread of the feeder: x_host / t_host must stay valid and unchanged
+ * until the matching tdh_feeder_acquire returns. The device pointers stay valid until the
+ * second-next acquire. */
+typedef struct tdh_feeder tdh_feeder;
+int tdh_feeder_create(size_t x_len, size_t t_len, int max_batch, tdh_feeder **feeder);
+int tdh_feeder_destroy(tdh_feeder *feeder);
+int tdh_feeder_stage(tdh_feeder *feeder, int batch, const float *x_host, const float *t_host);
+int tdh_feeder_acquire(tdh_feeder *feeder, const float **x_dev, const float **t_dev, int *batch);
+
 #ifdef __cplusplus
 }
 #endif

@@ -196,3 +196,35 @@ def test_net_with_every_other_activation_matches_oracle(T, O, W):
                 if W.layer_fans(l)[0]:
                     assert_close(net.get_param(i, 0), ref.weight(i), REL_TOL, f"step {step} w {i}")
                     assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} b {i}")
+
+
+def test_feeder_double_buffered_batches_match_oracle(T, O, W):
+    """tdh_feeder_*: different host batches every step, a short last batch, graph replay from
+    the two alternating device slots; updated weights against the oracle after every step."""
+    spec, params, _, _, _, loss, opt_kind, opt_kw = W.make_batch("cifar10_cnn_b128", batch=8)
+    batch = 8
+    net = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+        (ref.weight(i) if which == 0 else ref.bias(i))[:] = a
+    rng = np.random.default_rng(9)
+    sizes = [8, 8, 8, 3, 8, 8, 8, 3]   # two "epochs" with a short last batch
+    xs = [rng.standard_normal((n, 3072)).astype(np.float32) for n in sizes]
+    ts = [np.eye(10, dtype=np.float32)[rng.integers(0, 10, n)] for n in sizes]
+    opt, ropt = T.opt_desc(opt_kind, **opt_kw), O.opt_desc(opt_kind, **opt_kw)
+    feed = T.Feeder(3072, 10, batch)
+    feed.stage(xs[0], ts[0])
+    for k in range(len(sizes)):
+        xd, td, n = feed.acquire()
+        assert n == sizes[k]
+        net.train_step(opt, loss, n, xd, td)
+        if k + 1 < len(sizes):
+            feed.stage(xs[k + 1], ts[k + 1])
+        with pytest.raises(T.TdhError, match="nothing has been staged|has not been acquired"):
+            feed.acquire() if k + 1 == len(sizes) else feed.stage(xs[k], ts[k])
+        ref.train_step(ropt, loss, xs[k], ts[k])
+        for (i, which, _) in params:
+            want = ref.weight(i) if which == 0 else ref.bias(i)
+            assert_close(net.get_param(i, which), want, REL_TOL, f"step {k} layer {i}.{which}")
+    feed.close()

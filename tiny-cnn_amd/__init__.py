@@ -177,6 +177,44 @@ def copy_d2d(dst, src, nbytes=None, dst_offset=0, src_offset=0):
           "tdh_memcpy_d2d")
 
 
+class Feeder:
+    """Double-buffered upload of host batches (tdh_feeder_*): stage(x, t) copies the next batch
+    while the current step runs, acquire() returns device views of the batch staged last."""
+
+    def __init__(self, x_len, t_len, max_batch):
+        self.x_len, self.t_len, self.max_batch = int(x_len), int(t_len), int(max_batch)
+        self.h = C.c_void_p()
+        check(lib().tdh_feeder_create(C.c_size_t(self.x_len), C.c_size_t(self.t_len), self.max_batch,
+                                      C.byref(self.h)), "tdh_feeder_create")
+
+    def stage(self, x, t):
+        x = np.ascontiguousarray(x, np.float32)
+        t = np.ascontiguousarray(t, np.float32)
+        batch = x.shape[0]
+        assert x.size == batch * self.x_len and t.size == batch * self.t_len
+        self._staged = (x, t)  # the worker thread reads them until acquire() returns
+        check(lib().tdh_feeder_stage(self.h, batch, x.ctypes.data_as(C.c_void_p),
+                                     t.ctypes.data_as(C.c_void_p)), "tdh_feeder_stage")
+
+    def acquire(self):
+        xp, tp, b = C.c_void_p(), C.c_void_p(), C.c_int()
+        check(lib().tdh_feeder_acquire(self.h, C.byref(xp), C.byref(tp), C.byref(b)),
+              "tdh_feeder_acquire")
+        return (DevBuf.view(xp.value, (b.value, self.x_len)), DevBuf.view(tp.value, (b.value, self.t_len)),
+                b.value)
+
+    def close(self):
+        if self.h:
+            check(lib().tdh_feeder_destroy(self.h), "tdh_feeder_destroy")
+            self.h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def to_device(a, dtype=np.float32):
     a = np.ascontiguousarray(a, dtype=dtype)
     return DevBuf(a.shape, dtype).upload(a)

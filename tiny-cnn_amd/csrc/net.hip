@@ -32,13 +32,21 @@ struct tdh_net {
   double opt_params = 0.0;
   // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
   float *dev_powers = nullptr;          // {b1_t, b2_t} as the captured optimizer kernel reads them
-  hipGraphExec_t graph_exec = nullptr;
   struct GraphKey {
     int batch = 0, loss = 0, do_update = 0;
     const float *x = nullptr, *t = nullptr;
     const void *scratch = nullptr;      // the library scratch buffer the captured kernels use
     tdh_opt hyper = {};                 // hyper-parameters only (powers zeroed)
-  } graph_key;
+  };
+  // a few captured steps are kept, so that alternating input buffers (double-buffered
+  // uploads) or batch sizes (the short last batch of an epoch) do not re-capture every step
+  static constexpr int kGraphSlots = 4;
+  struct GraphSlot {
+    hipGraphExec_t exec = nullptr;
+    GraphKey key;
+    uint64_t last_use = 0;
+  } graphs[kGraphSlots];
+  uint64_t graph_clock = 0;
   float mirror_b1_t = 0.0f, mirror_b2_t = 0.0f;  // what the device copy of the powers holds
   size_t scratch = 0;        // largest per-op scratch need; with TDH_NET_GRAPH the sum over the
                              // layers, because branches of the captured step run side by side
@@ -303,7 +311,8 @@ int tdh_net_destroy(tdh_net *net) {
   TDH_REQUIRE_INIT();
   if (!net) return TDH_OK;
   TDH_HIP(hipStreamSynchronize(ctx().stream));
-  if (net->graph_exec) TDH_HIP(hipGraphExecDestroy(net->graph_exec));
+  for (auto &g : net->graphs)
+    if (g.exec) TDH_HIP(hipGraphExecDestroy(g.exec));
   for (hipEvent_t e : net->events) TDH_HIP(hipEventDestroy(e));
   for (void *p : net->allocs) TDH_HIP(hipFree(p));
   delete net;
@@ -546,10 +555,23 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   }
   TDH_TRY(ws_begin(net->scratch));  // may move the scratch buffer if another op outgrew it
   key.scratch = ctx().workspace;
-  if (!net->graph_exec || !same_key(key, net->graph_key)) {
-    if (net->graph_exec) {
-      TDH_HIP(hipGraphExecDestroy(net->graph_exec));
-      net->graph_exec = nullptr;
+  tdh_net::GraphSlot *slot = nullptr;
+  for (auto &g : net->graphs)
+    if (g.exec && same_key(key, g.key)) slot = &g;
+  if (!slot) {
+    for (auto &g : net->graphs)  // an empty slot, else the least recently used one
+      if (!g.exec) {
+        slot = &g;
+        break;
+      }
+    if (!slot) {
+      slot = &net->graphs[0];
+      for (auto &g : net->graphs)
+        if (g.last_use < slot->last_use) slot = &g;
+    }
+    if (slot->exec) {
+      TDH_HIP(hipGraphExecDestroy(slot->exec));
+      slot->exec = nullptr;
     }
     Context &c  = ctx();
     c.ws_locked = true;  // nothing may allocate while the stream is capturing
@@ -571,14 +593,14 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
     if (e != hipSuccess || !graph)
       return set_error(TDH_ERR_HIP, "tdh_net_train_step: graph capture failed: %s",
                        hipGetErrorString(e));
-    e = hipGraphInstantiate(&net->graph_exec, graph, nullptr, nullptr, 0);
+    e = hipGraphInstantiate(&slot->exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     if (e != hipSuccess) {
-      net->graph_exec = nullptr;
+      slot->exec = nullptr;
       return set_error(TDH_ERR_HIP, "tdh_net_train_step: graph instantiation failed: %s",
                        hipGetErrorString(e));
     }
-    net->graph_key   = key;
+    slot->key = key;
     net->mirror_b1_t = net->mirror_b2_t = -1.0f;  // forces the upload below
   }
   // the captured optimizer kernel reads the powers from device memory; bring that copy in
@@ -587,7 +609,8 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
     const float h[2] = {opt->b1_t, opt->b2_t};
     TDH_TRY(tdh_memcpy_h2d(net->dev_powers, h, sizeof(h)));
   }
-  TDH_HIP(hipGraphLaunch(net->graph_exec, ctx().stream));
+  slot->last_use = ++net->graph_clock;
+  TDH_HIP(hipGraphLaunch(slot->exec, ctx().stream));
   if (opt && do_update) {
     // advance the host object exactly as the eager path does
     for (int j = 0; j < net->opt_tensors; ++j) {

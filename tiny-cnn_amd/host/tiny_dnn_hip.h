@@ -957,6 +957,38 @@ struct softsign_layer : activation_layer { softsign_layer() : activation_layer(T
 struct asinh_layer : activation_layer { asinh_layer() : activation_layer(TDH_ACT_ASINH, "asinh-activation") {} };
 struct tanh_p1m2_layer : activation_layer { tanh_p1m2_layer() : activation_layer(TDH_ACT_TANH_P1M2, "tanh-scaled-activation") {} };
 
+namespace detail {
+// RAII handle of a tdh_feeder plus the flattening of vector-of-vectors batches
+class feeder {
+ public:
+  feeder(size_t x_len, size_t t_len, size_t max_batch) : x_len_(x_len), t_len_(t_len) {
+    check(tdh_feeder_create(x_len, t_len, static_cast<int>(max_batch), &f_));
+    x_.resize(x_len * max_batch);
+    t_.resize(t_len * max_batch);
+  }
+  feeder(const feeder &) = delete;
+  feeder &operator=(const feeder &) = delete;
+  ~feeder() {
+    if (f_) tdh_feeder_destroy(f_);
+  }
+  void stage(const std::vector<vec_t> &x, const std::vector<vec_t> &t, size_t first, size_t n) {
+    for (size_t s = 0; s < n; ++s) {
+      if (x[first + s].size() < x_len_ || t[first + s].size() < t_len_)
+        throw nn_error("fit: sample shorter than the network's input / output");
+      std::memcpy(x_.data() + s * x_len_, x[first + s].data(), x_len_ * sizeof(float));
+      std::memcpy(t_.data() + s * t_len_, t[first + s].data(), t_len_ * sizeof(float));
+    }
+    check(tdh_feeder_stage(f_, static_cast<int>(n), x_.data(), t_.data()));
+  }
+  tdh_feeder *get() const { return f_; }
+
+ private:
+  tdh_feeder *f_ = nullptr;
+  size_t x_len_, t_len_;
+  std::vector<float> x_, t_;
+};
+}  // namespace detail
+
 struct sequential {};
 
 // network<sequential> (tiny_dnn/network.h:148-1105): operator<<, fit, train, predict. Weights
@@ -1019,16 +1051,25 @@ class network<sequential> {
     opt.reset();  // network.h:856; the device copy of the state vectors is cleared with it
     detail::check(tdh_net_reset_optimizer(net_));
     tdh_opt o = opt.descriptor();
-    for (int iter = 0; iter < epoch; ++iter) {
-      for (size_t i = 0; i < inputs.size(); i += batch_size) {
-        const size_t n = std::min(batch_size, inputs.size() - i);
-        tensor_t xb(inputs.begin() + i, inputs.begin() + i + n);
-        tensor_t tb(desired_outputs.begin() + i, desired_outputs.begin() + i + n);
-        detail::check(tdh_net_train_step(net_, &o, Error::kind, static_cast<int>(n),
-                                         x_.upload(xb, n, in_len), t_.upload(tb, n, out_len), 1));
-        on_batch_enumerate();
-      }
-      on_epoch_enumerate();
+    // batches travel double-buffered: while a step runs, the next batch is flattened, copied
+    // to pinned memory and uploaded
+    detail::feeder feed(in_len, out_len, batch_size);
+    const size_t per_epoch = (inputs.size() + batch_size - 1) / batch_size;
+    const size_t total     = per_epoch * static_cast<size_t>(epoch);
+    auto stage = [&](size_t k) {
+      const size_t i = (k % per_epoch) * batch_size;
+      const size_t n = std::min(batch_size, inputs.size() - i);
+      feed.stage(inputs, desired_outputs, i, n);
+    };
+    if (total) stage(0);
+    for (size_t k = 0; k < total; ++k) {
+      const float *xd = nullptr, *td = nullptr;
+      int n = 0;
+      detail::check(tdh_feeder_acquire(feed.get(), &xd, &td, &n));
+      if (k + 1 < total) stage(k + 1);  // the feeder's thread copies while this one launches
+      detail::check(tdh_net_train_step(net_, &o, Error::kind, n, xd, td, 1));
+      on_batch_enumerate();
+      if ((k + 1) % per_epoch == 0) on_epoch_enumerate();
     }
     opt.absorb(o);
     return true;
@@ -1083,7 +1124,7 @@ class network<sequential> {
     }
     tdh_net *fresh = nullptr;
     detail::check(tdh_net_create(raw.data(), static_cast<int>(raw.size()), static_cast<int>(batch),
-                                 TDH_NET_FUSE_ACT_GRAD, &fresh));
+                                 TDH_NET_FUSE_ACT_GRAD | TDH_NET_GRAPH, &fresh));
     if (net_) {
       for (size_t i = 0; i < layers_.size(); ++i)
         for (int which = 0; which < 2; ++which) {
