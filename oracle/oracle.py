@@ -455,6 +455,12 @@ class RefNet:
         _chk(self.lib.tdr_net_get_param(self.h, layer, which, a.ctypes.data_as(f32p)), "get_param")
         return a
 
+    def save_weights(self, path):
+        _chk(self.lib.tdr_net_save_weights(self.h, str(path).encode()), "save_weights")
+
+    def load_weights(self, path):
+        _chk(self.lib.tdr_net_load_weights(self.h, str(path).encode()), "load_weights")
+
     def fit(self, opt, loss, x, t, steps=1):
         x, xp = _f(x); t, tp = _f(t)
         sec = self.lib.tdr_net_fit(self.h, C.byref(opt), LOSS[loss], x.shape[0], xp,
@@ -596,3 +602,41 @@ def ref_opt_updates(o, g, w, steps, kind="scalar"):
     _chk(lib.tdr_opt_updates(C.byref(o), C.c_size_t(w.size), gp, w.ctypes.data_as(f32p), steps),
          "ref opt_updates")
     return w
+
+
+# ---- the reference's dataset readers (io/mnist_parser.h, io/cifar10_parser.h)
+def ref_parse_mnist_images(path, scale_min, scale_max, x_pad, y_pad, kind="scalar"):
+    lib = ref_lib(kind)
+    lib.tdr_parse_mnist_images.restype = C.c_long
+    n_len = C.c_size_t()
+    args = (str(path).encode(), C.c_float(scale_min), C.c_float(scale_max), x_pad, y_pad)
+    n = lib.tdr_parse_mnist_images(*args, None, C.byref(n_len))
+    if n < 0:
+        raise ValueError("reference parser raised nn_error")
+    out = np.empty((n, n_len.value), np.float32)
+    lib.tdr_parse_mnist_images(*args, out.ctypes.data_as(f32p), None)
+    return out
+
+
+def ref_parse_mnist_labels(path, kind="scalar"):
+    lib = ref_lib(kind)
+    lib.tdr_parse_mnist_labels.restype = C.c_long
+    n = lib.tdr_parse_mnist_labels(str(path).encode(), None)
+    if n < 0:
+        raise ValueError("reference parser raised nn_error")
+    out = np.empty(n, np.int64)
+    lib.tdr_parse_mnist_labels(str(path).encode(), out.ctypes.data_as(i64p))
+    return out
+
+
+def ref_parse_cifar10(path, scale_min, scale_max, x_pad, y_pad, kind="scalar"):
+    lib = ref_lib(kind)
+    lib.tdr_parse_cifar10.restype = C.c_long
+    n_len = C.c_size_t()
+    args = (str(path).encode(), C.c_float(scale_min), C.c_float(scale_max), x_pad, y_pad)
+    n = lib.tdr_parse_cifar10(*args, None, None, C.byref(n_len))
+    if n < 0:
+        raise ValueError("reference parser raised nn_error")
+    img, lab = np.empty((n, n_len.value), np.float32), np.empty(n, np.int64)
+    lib.tdr_parse_cifar10(*args, img.ctypes.data_as(f32p), lab.ctypes.data_as(i64p), None)
+    return img, lab

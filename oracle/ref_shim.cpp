@@ -16,6 +16,7 @@
  * Include order works around tiny_dnn/tiny_dnn.h:122 naming linear_layer
  * without including its header.
  */
+#include <fstream>
 #include <iostream>
 #ifdef CNN_USE_OMP
 #include <omp.h>
@@ -471,6 +472,62 @@ int tdr_net_predict(tdr_net *h, int batch, const float *x, size_t in_len, float 
       std::memcpy(y + out_len * s, out.data(), sizeof(float) * out_len);
     }
     return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* network::save(std::ostream&) / load(std::istream&) of the weights as text
+ * (tiny_dnn/network.h:762-771, layer::save/load tiny_dnn/layers/layer.h:361-385) */
+int tdr_net_save_weights(tdr_net *h, const char *path) {
+  try {
+    std::ofstream os(path);
+    h->net.save(os);
+    return os.good() ? 0 : -1;
+  } catch (const std::exception &) { return -1; }
+}
+int tdr_net_load_weights(tdr_net *h, const char *path) {
+  try {
+    std::ifstream is(path);
+    if (!is.good()) return -1;
+    h->net.load(is);
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* io/mnist_parser.h, io/cifar10_parser.h. out_images: [count][len] floats (may be NULL to
+ * query), out_labels: [count] int64. Returns the number of items, -1 on nn_error. */
+long tdr_parse_mnist_images(const char *path, float scale_min, float scale_max, int x_pad, int y_pad,
+                            float *out_images, size_t *len) {
+  try {
+    std::vector<vec_t> images;
+    parse_mnist_images(path, &images, scale_min, scale_max, x_pad, y_pad);
+    if (len) *len = images.empty() ? 0 : images[0].size();
+    if (out_images)
+      for (size_t i = 0; i < images.size(); i++)
+        std::memcpy(out_images + i * images[0].size(), images[i].data(), sizeof(float) * images[0].size());
+    return (long)images.size();
+  } catch (const std::exception &) { return -1; }
+}
+long tdr_parse_mnist_labels(const char *path, int64_t *out_labels) {
+  try {
+    std::vector<label_t> labels;
+    parse_mnist_labels(path, &labels);
+    if (out_labels)
+      for (size_t i = 0; i < labels.size(); i++) out_labels[i] = (int64_t)labels[i];
+    return (long)labels.size();
+  } catch (const std::exception &) { return -1; }
+}
+long tdr_parse_cifar10(const char *path, float scale_min, float scale_max, int x_pad, int y_pad,
+                       float *out_images, int64_t *out_labels, size_t *len) {
+  try {
+    std::vector<vec_t> images;
+    std::vector<label_t> labels;
+    parse_cifar10(path, &images, &labels, scale_min, scale_max, x_pad, y_pad);
+    if (len) *len = images.empty() ? 0 : images[0].size();
+    for (size_t i = 0; i < images.size(); i++) {
+      if (out_images) std::memcpy(out_images + i * images[0].size(), images[i].data(), sizeof(float) * images[0].size());
+      if (out_labels) out_labels[i] = (int64_t)labels[i];
+    }
+    return (long)images.size();
   } catch (const std::exception &) { return -1; }
 }
 

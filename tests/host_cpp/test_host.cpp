@@ -15,7 +15,9 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <fstream>
 #include <random>
+#include <sstream>
 
 #include "td_oracle.h"
 #include "tiny_dnn_hip.h"
@@ -415,6 +417,53 @@ static void on_fatal_signal(int sig) {
   _exit(128 + sig);
 }
 
+// weights as text: save -> load into a second network, stream operators, fast_load
+static void weight_files() {
+  std::puts("network save / load / fast_load");
+  auto make = [](network<sequential> &nn) {
+    nn << convolutional_layer(8, 8, 3, 2, 3, padding::same) << tanh_layer()
+       << average_pooling_layer(8, 8, 3, 2) << fully_connected_layer(48, 5);
+  };
+  network<sequential> a, b, c;
+  make(a); make(b); make(c);
+  const size_t sizes[4][2] = {{54, 3}, {0, 0}, {3, 3}, {240, 5}};
+  for (size_t i = 0; i < 4; ++i)
+    for (int which = 0; which < 2; ++which)
+      if (sizes[i][which]) a.set_weights(i, which, random_vec(sizes[i][which], 300 + 2 * i + which, -2.f, 2.f));
+  std::stringstream ss;
+  ss << a;
+  const std::string text = ss.str();
+  // 54+3 conv, 12+3 pooling (3 used + 9 written as 0), 240+5 fc = 317 numbers
+  size_t blanks = 0;
+  for (char ch : text) blanks += ch == ' ';
+  EXPECT(blanks == 317);
+  ss >> b;
+  const char *path = "/tmp/tdh_test_weights.txt";
+  {
+    std::ofstream f(path);
+    f << text;
+  }
+  c.fast_load(path);
+  for (size_t i = 0; i < 4; ++i)
+    for (int which = 0; which < 2; ++which) {
+      if (!sizes[i][which]) continue;
+      const vec_t wa = a.weights(i, which);
+      expect_near(b.weights(i, which), wa, 1e-7f, "load");
+      expect_near(c.weights(i, which), wa, 1e-7f, "fast_load");
+    }
+  std::stringstream second;
+  second << b;  // what was loaded prints as the same text
+  EXPECT(second.str() == text);
+  std::stringstream few("1 2 3");
+  bool threw = false;
+  try {
+    few >> c;
+  } catch (const nn_error &) {
+    threw = true;
+  }
+  EXPECT(threw);
+}
+
 int main() {
   setvbuf(stdout, nullptr, _IONBF, 0);  // every case is named before it runs
   signal(SIGSEGV, on_fatal_signal);
@@ -428,6 +477,7 @@ int main() {
     conv_ops_vs_oracle();
     fc_pool_ops_vs_oracle();
     activations_vs_oracle();
+    weight_files();
     net_fit_vs_oracle<gradient_descent>("gradient_descent", TDO_OPT_SGD);
     net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM);
   } catch (const std::exception &e) {

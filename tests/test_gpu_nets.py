@@ -228,3 +228,27 @@ def test_feeder_double_buffered_batches_match_oracle(T, O, W):
             want = ref.weight(i) if which == 0 else ref.bias(i)
             assert_close(net.get_param(i, which), want, REL_TOL, f"step {k} layer {i}.{which}")
     feed.close()
+
+
+def test_weight_files_round_trip_with_the_reference(T, tmp_path):
+    """A weight file written by the reference's network::save loads into the device network,
+    and the file the device network writes is byte for byte the reference's."""
+    import importlib, os
+    io = importlib.import_module("tiny-cnn_amd.io")
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "io.npz"))
+    nets = {"weights_avepool": [T.L_conv(8, 8, 2, 3, 3, pad_same=True), T.L_act("tanh"),
+                                T.L_avepool(8, 8, 3, 2), T.L_fc(48, 5)],
+            "weights_plain": [T.L_conv(6, 6, 1, 3, 4), T.L_act("relu"), T.L_fc(64, 3)]}
+    for name, layers in nets.items():
+        path = str(tmp_path / (name + ".txt"))
+        g[name + ".text"].tofile(path)
+        net = T.Net(layers, 2)
+        io.load_weights(net, path)
+        for k, (i, which, n) in enumerate(net.params()):
+            want = g[f"{name}.param{k}"]
+            assert np.allclose(net.get_param(i, which), want, rtol=1e-7, atol=0), (name, k)
+        out = str(tmp_path / (name + ".out.txt"))
+        io.save_weights(net, out)
+        assert open(out).read() == open(path).read(), name
+    with pytest.raises(ValueError, match="fewer weights"):
+        io.load_weights(T.Net(nets["weights_avepool"], 2), str(tmp_path / "weights_plain.txt"))

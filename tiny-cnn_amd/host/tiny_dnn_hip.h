@@ -31,9 +31,15 @@
 #include <algorithm>
 #include <cstddef>
 #include <cstdint>
+#include <cstdio>
 #include <cstring>
 #include <exception>
+#include <fstream>
+#include <iomanip>
+#include <istream>
+#include <limits>
 #include <map>
+#include <ostream>
 #include <memory>
 #include <string>
 #include <vector>
@@ -1091,6 +1097,55 @@ class network<sequential> {
     return fit<Error>(opt, inputs, t, batch_size, epoch);
   }
 
+  // Weights as text, the reference's stream format (network::save / load, tiny_dnn/network.h:
+  // 762-771; layer::save / load, tiny_dnn/layers/layer.h:361-385): every trainable vector of
+  // every layer in order, each value printed with 8 significant digits and followed by a
+  // blank. An average-pooling layer's weight vector has pool_w*pool_h*channels entries in the
+  // reference's files although only the first `channels` are ever read
+  // (average_pooling_layer.h:222-226): the extra ones are written as 0 and skipped on load.
+  void save(std::ostream &os) {
+    build(max_batch_ ? max_batch_ : 1);
+    os << std::setprecision(std::numeric_limits<float_t>::digits10 + 2);
+    for (size_t i = 0; i < layers_.size(); ++i)
+      for (int which = 0; which < 2; ++which) {
+        const vec_t v = weights(i, which);
+        for (float_t w : v) os << w << " ";
+        for (size_t k = v.size(); k < file_length(i, which); ++k) os << float_t(0) << " ";
+      }
+  }
+  void load(std::istream &is) {
+    build(max_batch_ ? max_batch_ : 1);
+    for (size_t i = 0; i < layers_.size(); ++i)
+      for (int which = 0; which < 2; ++which) {
+        vec_t v(tdh_net_param_size(net_, static_cast<int>(i), which));
+        for (float_t &w : v) is >> w;
+        float_t skipped;
+        for (size_t k = v.size(); k < file_length(i, which); ++k) is >> skipped;
+        if (is.fail()) throw nn_error("load: the stream holds fewer weights than the network");
+        if (!v.empty()) set_weights(i, which, v);
+      }
+    initialized_ = true;
+  }
+  // network::fast_load (tiny_dnn/network.h:777-785): the same file through fscanf
+  void fast_load(const char *filepath) {
+    FILE *stream = std::fopen(filepath, "r");
+    if (!stream) throw nn_error(std::string("failed to open file:") + filepath);
+    std::vector<float_t> data;
+    double temp;
+    while (std::fscanf(stream, "%lf", &temp) > 0) data.push_back(float_t(temp));
+    std::fclose(stream);
+    build(max_batch_ ? max_batch_ : 1);
+    size_t idx = 0;
+    for (size_t i = 0; i < layers_.size(); ++i)
+      for (int which = 0; which < 2; ++which) {
+        const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which), len = file_length(i, which);
+        if (idx + len > data.size()) throw nn_error("fast_load: the file holds fewer weights than the network");
+        if (n) set_weights(i, which, vec_t(data.begin() + idx, data.begin() + idx + n));
+        idx += len;
+      }
+    initialized_ = true;
+  }
+
   // network::predict (tiny_dnn/network.h:226-230)
   vec_t predict(const vec_t &in) {
     build(max_batch_ ? max_batch_ : 1);
@@ -1104,6 +1159,13 @@ class network<sequential> {
   }
 
  private:
+  // entries of trainable vector `which` of layer i in a weight file
+  size_t file_length(size_t i, int which) {
+    const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which);
+    const layer_desc d = layers_[i]->describe(shape3d());
+    if (d.l.kind == TDH_L_AVEPOOL && which == 0) return n * d.l.pool.pool_w * d.l.pool.pool_h;
+    return n;
+  }
   void drop() {
     if (net_) tdh_net_destroy(net_);
     net_ = nullptr;
@@ -1149,6 +1211,89 @@ class network<sequential> {
 template <typename Layer>
 network<sequential> &operator<<(network<sequential> &n, Layer &&l) {
   return n.add(std::forward<Layer>(l));
+}
+// tiny_dnn/network.h:1153-1165
+inline std::ostream &operator<<(std::ostream &os, network<sequential> &n) {
+  n.save(os);
+  return os;
+}
+inline std::istream &operator>>(std::istream &is, network<sequential> &n) {
+  n.load(is);
+  return is;
+}
+
+// ---- data ingest: the reference's dataset readers (tiny_dnn/io/mnist_parser.h,
+// tiny_dnn/io/cifar10_parser.h) with their signatures, scaling arithmetic and errors; the
+// batches they produce travel to the device through network::fit's double-buffered feeder.
+namespace detail {
+inline std::vector<uint8_t> read_file(const std::string &path) {
+  std::ifstream ifs(path.c_str(), std::ios::in | std::ios::binary);
+  if (ifs.bad() || ifs.fail()) throw nn_error("failed to open file:" + path);
+  return std::vector<uint8_t>((std::istreambuf_iterator<char>(ifs)), std::istreambuf_iterator<char>());
+}
+// big-endian 32-bit field at byte `at`; bytes past the end read as 0, like a failed ifstream::read
+inline uint32_t be32(const std::vector<uint8_t> &b, size_t at) {
+  uint32_t v = 0;
+  for (size_t i = 0; i < 4; ++i) v = (v << 8) | (at + i < b.size() ? b[at + i] : 0u);
+  return v;
+}
+}  // namespace detail
+
+// mnist_parser.h:77-102: idx1 file, magic 0x00000801
+inline void parse_mnist_labels(const std::string &label_file, std::vector<label_t> *labels) {
+  const std::vector<uint8_t> b = detail::read_file(label_file);
+  const uint32_t magic = detail::be32(b, 0), num_items = detail::be32(b, 4);
+  if (magic != 0x00000801 || num_items <= 0) throw nn_error("MNIST label-file format error");
+  labels->resize(num_items);
+  for (uint32_t i = 0; i < num_items; ++i)
+    (*labels)[i] = static_cast<label_t>(8 + static_cast<size_t>(i) < b.size() ? b[8 + i] : 0);
+}
+
+// mnist_parser.h:121-147 (+ :26-75): idx3 file, magic 0x00000803; pixel p becomes
+// (p / 255) * (scale_max - scale_min) + scale_min, the border added by the paddings scale_min
+inline void parse_mnist_images(const std::string &image_file, std::vector<vec_t> *images,
+                               float_t scale_min, float_t scale_max, int x_padding, int y_padding) {
+  if (x_padding < 0 || y_padding < 0) throw nn_error("padding size must not be negative");
+  if (scale_min >= scale_max) throw nn_error("scale_max must be greater than scale_min");
+  const std::vector<uint8_t> b = detail::read_file(image_file);
+  const uint32_t magic = detail::be32(b, 0), num_items = detail::be32(b, 4);
+  const uint32_t rows = detail::be32(b, 8), cols = detail::be32(b, 12);
+  if (magic != 0x00000803 || num_items <= 0) throw nn_error("MNIST label-file format error");
+  const size_t width = cols + 2 * static_cast<size_t>(x_padding), height = rows + 2 * static_cast<size_t>(y_padding);
+  images->resize(num_items);
+  for (uint32_t i = 0; i < num_items; ++i) {
+    vec_t &dst = (*images)[i];
+    dst.assign(width * height, scale_min);
+    const size_t base = 16 + static_cast<size_t>(i) * rows * cols;
+    for (uint32_t y = 0; y < rows; ++y)
+      for (uint32_t x = 0; x < cols; ++x) {
+        const size_t at = base + static_cast<size_t>(y) * cols + x;
+        const uint8_t p = at < b.size() ? b[at] : 0;
+        dst[width * (y + y_padding) + x + x_padding] = (p / float_t(255)) * (scale_max - scale_min) + scale_min;
+      }
+  }
+}
+
+// cifar10_parser.h:38-86: records of one label byte and 3 x 32 x 32 pixel bytes, appended to
+// the vectors; pixel c becomes scale_min + (scale_max - scale_min) * c / 255
+inline void parse_cifar10(const std::string &filename, std::vector<vec_t> *train_images,
+                          std::vector<label_t> *train_labels, float_t scale_min, float_t scale_max,
+                          int x_padding, int y_padding) {
+  if (x_padding < 0 || y_padding < 0) throw nn_error("padding size must not be negative");
+  if (scale_min >= scale_max) throw nn_error("scale_max must be greater than scale_min");
+  const std::vector<uint8_t> b = detail::read_file(filename);
+  const size_t depth = 3, side = 32, area = side * side, record = 1 + depth * area;
+  const size_t w = side + 2 * static_cast<size_t>(x_padding), h = side + 2 * static_cast<size_t>(y_padding);
+  for (size_t at = 0; at + record <= b.size(); at += record) {
+    vec_t img(w * h * depth, scale_min);
+    for (size_t c = 0; c < depth; ++c)
+      for (size_t y = 0; y < side; ++y)
+        for (size_t x = 0; x < side; ++x)
+          img[c * w * h + (y + y_padding) * w + x + x_padding] =
+            scale_min + (scale_max - scale_min) * b[at + 1 + c * area + y * side + x] / 255;
+    train_images->push_back(std::move(img));
+    train_labels->push_back(b[at]);
+  }
 }
 
 }  // namespace tiny_dnn
