@@ -201,7 +201,9 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
 size_t fc_workspace_bytes(int in, int out, int batch);
 
 // pool.hip
-int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax);
+// act_out: also writes act(y) there (tanh / relu / sigmoid), the activation layer behind the pool
+int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax,
+                float *act_out = nullptr, int act_kind = TDH_ACT_NONE);
 int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
                 float *dx);
 int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *b,
@@ -209,6 +211,17 @@ int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *
 int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,
                 float *dx, float *dw, float *db, int accumulate);
 size_t avepool_workspace_bytes(const tdh_pool_desc *d, int batch);
+
+// forward of the three parameter-free pointwise activations (tanh_layer.h:24-28,
+// relu_layer.h:25-29, sigmoid_layer.h:24-28), for kernels that apply one on their way out
+__device__ __forceinline__ float act_apply(int kind, float x) {
+  switch (kind) {
+    case TDH_ACT_TANH: return tanhf(x);
+    case TDH_ACT_RELU: return x > 0.0f ? x : 0.0f;
+    case TDH_ACT_SIGMOID: return 1.0f / (1.0f + expf(-x));
+    default: return x;
+  }
+}
 
 __device__ __forceinline__ float act_grad_factor(int kind, float y) {
   switch (kind) {

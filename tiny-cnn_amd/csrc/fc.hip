@@ -9,6 +9,93 @@
 
 namespace tdh {
 
+namespace {
+
+// Products of a small network's fully-connected layers (a few million MACs, K <= 256): the
+// tiled MFMA kernel pays one exposed memory latency per 16-deep K tile with only a handful of
+// workgroups to hide it behind, 7-16 us for microseconds of arithmetic. Here a workgroup
+// stages 64-deep panels of both operands with every load in flight at once (20 per thread),
+// and the four waves multiply out of LDS on the vector ALUs: wave w owns rows 4w..4w+3 of a
+// 16 x 64 tile, so its A values are wave-uniform LDS broadcasts and its B values one
+// conflict-free read per k. k ascends, one FMA per term: the summation order is fixed.
+constexpr int SFC_TM = 16, SFC_TN = 64, SFC_KC = 64, SFC_NT = 256;
+constexpr int SFC_NA = SFC_TM * SFC_KC / SFC_NT, SFC_NB = SFC_TN * SFC_KC / SFC_NT;
+
+template <class Epi>
+__global__ void __launch_bounds__(SFC_NT)
+small_fc_gemm_kernel(const StridedOperand a, const StridedOperand b, const Epi epi, const int M,
+                     const int N, const int K) {
+  __shared__ __attribute__((aligned(16))) float As[SFC_KC][SFC_TM + 4];
+  __shared__ float Bs[SFC_KC][SFC_TN + 1];
+  const int tid = threadIdx.x, tn = tid & 63, tmg = tid >> 6;
+  const int m0 = blockIdx.y * SFC_TM, n0 = blockIdx.x * SFC_TN;
+  // staging coordinates: consecutive threads walk the operand's contiguous direction
+  const bool a_k_fast = a.s_k == 1, b_k_fast = b.s_k == 1;
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k0 = 0; k0 < K; k0 += SFC_KC) {
+    float ra[SFC_NA], rb[SFC_NB];
+#pragma unroll
+    for (int i = 0; i < SFC_NA; ++i) {
+      const int e = tid + SFC_NT * i;
+      const int m = a_k_fast ? e / SFC_KC : e % SFC_TM, k = a_k_fast ? e % SFC_KC : e / SFC_TM;
+      ra[i] = (m0 + m < M && k0 + k < K) ? a.p[(m0 + m) * a.s_mn + (k0 + k) * a.s_k] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < SFC_NB; ++i) {
+      const int e = tid + SFC_NT * i;
+      const int n = b_k_fast ? e / SFC_KC : e % SFC_TN, k = b_k_fast ? e % SFC_KC : e / SFC_TN;
+      rb[i] = (n0 + n < N && k0 + k < K) ? b.p[(n0 + n) * b.s_mn + (k0 + k) * b.s_k] : 0.0f;
+    }
+    if (k0 > 0) __syncthreads();  // the previous panel has been consumed
+#pragma unroll
+    for (int i = 0; i < SFC_NA; ++i) {
+      const int e = tid + SFC_NT * i;
+      As[a_k_fast ? e % SFC_KC : e / SFC_TM][a_k_fast ? e / SFC_KC : e % SFC_TM] = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < SFC_NB; ++i) {
+      const int e = tid + SFC_NT * i;
+      Bs[b_k_fast ? e % SFC_KC : e / SFC_TN][b_k_fast ? e / SFC_KC : e % SFC_TN] = rb[i];
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < SFC_KC; ++k) {
+      const float4 av = *reinterpret_cast<const float4 *>(&As[k][4 * tmg]);
+      const float bv  = Bs[k][tn];
+      acc[0] += av.x * bv;
+      acc[1] += av.y * bv;
+      acc[2] += av.z * bv;
+      acc[3] += av.w * bv;
+    }
+  }
+  const int n = n0 + tn;
+  if (n < N) {
+    const typename Epi::Col c = epi.col(n);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 4 * tmg + i;
+      if (m < M) epi.store(m, c, acc[i]);
+    }
+  }
+}
+
+bool small_fc_applies(int M, int N, int K) {
+  return K <= 4 * SFC_KC && static_cast<long>(M) * N <= (1L << 18) &&
+         static_cast<long>(M) * N * K <= (1L << 24);
+}
+
+template <class Epi>
+int launch_small_fc(const StridedOperand &a, const StridedOperand &b, const Epi &epi, int M, int N,
+                    int K, const char *tag) {
+  ProfScope prof(tag, M, N, K);
+  hipLaunchKernelGGL((small_fc_gemm_kernel<Epi>), dim3(ceil_div(N, SFC_TN), ceil_div(M, SFC_TM)),
+                     dim3(SFC_NT), 0, ctx().stream, a, b, epi, M, N, K);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
+}  // namespace
+
 size_t fc_workspace_bytes(int in, int out, int batch) {
   return gemm_workspace_bytes(batch, out, in, true) + gemm_workspace_bytes(batch, in, out, true) +
          gemm_workspace_bytes(in, out, batch, true);
@@ -19,6 +106,7 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
   StridedOperand A{x, in, 1, batch};   // X[s][k], k contiguous
   StridedOperand B{w, 1, out, out};    // W[k][n], n contiguous
   EpiRowMajor epi{y, out, has_bias ? b : nullptr, ActGrad(), 0};
+  if (small_fc_applies(batch, out, in)) return launch_small_fc(A, B, epi, batch, out, in, "fc_fwd_small");
   return launch_gemm<true, false, false, true>(A, B, epi, batch, out, in, true, "fc_fwd_gemm",
                                               "fc_fwd_splitk_reduce");
 }
@@ -29,14 +117,20 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     StridedOperand A{dy, out, 1, batch};  // dY[s][k]
     StridedOperand B{w, out, 1, in};      // W[n][k], k contiguous
     EpiRowMajor epi{dx, in, nullptr, dx_act, 0};
-    TDH_TRY((launch_gemm<true, true, false, false>(A, B, epi, batch, in, out, true, "fc_dx_gemm",
+    if (small_fc_applies(batch, in, out))
+      TDH_TRY(launch_small_fc(A, B, epi, batch, in, out, "fc_dx_small"));
+    else
+      TDH_TRY((launch_gemm<true, true, false, false>(A, B, epi, batch, in, out, true, "fc_dx_gemm",
                                                  "fc_dx_splitk_reduce")));
   }
   if (dw) {
     StridedOperand A{x, 1, in, in};      // X[k][m], m contiguous
     StridedOperand B{dy, 1, out, out};   // dY[k][n], n contiguous
     EpiRowMajor epi{dw, out, nullptr, ActGrad(), accumulate};
-    TDH_TRY((launch_gemm<false, false, true, true>(A, B, epi, in, out, batch, true, "fc_dw_gemm",
+    if (small_fc_applies(in, out, batch))
+      TDH_TRY(launch_small_fc(A, B, epi, in, out, batch, "fc_dw_small"));
+    else
+      TDH_TRY((launch_gemm<false, false, true, true>(A, B, epi, in, out, batch, true, "fc_dw_gemm",
                                                    "fc_dw_splitk_reduce")));
   }
   if (db && has_bias) TDH_TRY(launch_colsum(dy, batch, out, db, accumulate));

@@ -152,13 +152,23 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
         TDH_TRY(fc_fwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out));
         break;
-      case TDH_L_MAXPOOL: TDH_TRY(maxpool_fwd(&s.pool, batch, in, L.out, L.argmax)); break;
+      case TDH_L_MAXPOOL:
+        if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
+            is_pointwise_act(net->layers[i + 1].spec.act)) {
+          // the activation layer behind the pool leaves the same kernel
+          TDH_TRY(maxpool_fwd(&s.pool, batch, in, L.out, L.argmax, net->layers[i + 1].out,
+                              net->layers[i + 1].spec.act));
+          ++i;
+        } else {
+          TDH_TRY(maxpool_fwd(&s.pool, batch, in, L.out, L.argmax));
+        }
+        break;
       case TDH_L_AVEPOOL: TDH_TRY(avepool_fwd(&s.pool, batch, in, L.w, L.b, L.out)); break;
       case TDH_L_ACT:
         TDH_TRY(launch_act_fwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out));
         break;
     }
-    in = L.out;
+    in = net->layers[i].out;  // of the activation layer when one was fused
   }
   return TDH_OK;
 }

@@ -33,7 +33,8 @@ PoolGeom make_geom(const tdh_pool_desc *d) {
 // an all-NaN window reports index 0.
 __global__ void __launch_bounds__(PT)
 maxpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
-                   int32_t *__restrict__ argmax, const int total, const PoolGeom g) {
+                   int32_t *__restrict__ argmax, const int total, const PoolGeom g,
+                   float *__restrict__ act_out, const int act_kind) {
   const int o = blockIdx.x * PT + threadIdx.x;
   if (o >= total) return;
   uint32_t t, ox, oy, c, img;
@@ -56,6 +57,7 @@ maxpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
     }
   y[o] = best;
   if (argmax) argmax[o] = idx;
+  if (act_out) act_out[o] = act_apply(act_kind, best);  // the activation layer that follows
 }
 
 // maxpool_grad_op_internal (maxpool_op_internal.h:42-57). in2out[i] is the LAST window, in
@@ -185,13 +187,15 @@ avepool_bwd_param_reduce_kernel(const float *__restrict__ partial, const int bat
 
 }  // namespace
 
-int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax) {
+int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax,
+                float *act_out, int act_kind) {
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.OH * g.OW;
   if (total <= 0) return TDH_OK;
-  ProfScope prof("maxpool_fwd", 4.0 * batch * g.C * g.H * g.W + 8.0 * total, WORK_BYTE);
+  ProfScope prof(act_out ? "maxpool_fwd_act" : "maxpool_fwd",
+                 4.0 * batch * g.C * g.H * g.W + (act_out ? 12.0 : 8.0) * total, WORK_BYTE);
   hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
-                     y, argmax, static_cast<int>(total), g);
+                     y, argmax, static_cast<int>(total), g, act_out, act_kind);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }
