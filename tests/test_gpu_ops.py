@@ -36,6 +36,8 @@ CONV = [
     # LDS-staged dW kernel: ragged widths, partial channel blocks, valid padding, column tiles
     (13, 11, 16, 3, 40, True, 1, 3), (18, 18, 20, 5, 24, False, 1, 2), (70, 9, 33, 3, 65, True, 1, 2),
     (12, 12, 48, 5, 16, True, 1, 5), (40, 6, 16, 3, 16, False, 1, 1),
+    # 5x5 windows split by filter row: stacked small images with a ragged last chunk, row chunks
+    (10, 10, 16, 5, 40, True, 1, 7), (36, 36, 16, 5, 16, False, 1, 2), (8, 8, 32, 5, 64, True, 1, 11),
     # direct small-Cin forward kernel: ragged tiles, one and two channel blocks
     (20, 17, 3, 3, 40, True, 1, 3), (23, 22, 1, 5, 33, False, 1, 2), (37, 9, 3, 5, 64, True, 1, 2),
 ]

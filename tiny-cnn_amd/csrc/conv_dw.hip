@@ -1,4 +1,4 @@
-// conv_dw.hip — weight gradient of a stride-1 3x3 convolution from LDS-staged tiles.
+// conv_dw.hip — weight gradient of a stride-1 3x3 or 5x5 convolution from LDS-staged tiles.
 //
 //   dW[co][ci][fy][fx] = sum_{img,oy,ox} dY[img][co][oy][ox] * X[img][ci][oy+fy-ph][ox+fx-pw]
 //
@@ -9,18 +9,32 @@
 //
 // The two pixels of an instruction are NOT neighbours: within a tile row of TC pixels, k = 0
 // lanes walk the left half and k = 1 lanes the right half. A lane therefore needs consecutive
-// pixels in consecutive instructions, so both fragments come out of LDS as 16-byte words in the
-// tensors' own (pixel-fastest) layout: per four pixels and filter row one dY word and two X
-// words serve 4*S instructions. Channel planes are padded to 4 (mod 32) floats, which spreads
-// eight lanes' words over all banks.
+// pixels in consecutive instructions: per four pixels and filter row one 16-byte dY word and
+// 4+S-1 X floats serve 4*S instructions. dY channel planes are padded to 4 (mod 32) floats (eight
+// lanes' 16-byte words cover all banks), X channel planes to an odd stride (32 lanes' floats
+// cover all banks).
 //
-// A workgroup owns 32*WCO output channels x 32 input channels x all taps for a range of pixel
-// chunks (one image, TRw*WK output rows x TC columns). Waves: WCO channel blocks x WK row
-// groups of the chunk x WFY filter-row groups; a wave keeps (R/WFY)*S accumulators, up to 144
-// registers, so the kernel runs one workgroup per CU with the full register file. The next
-// chunk's global loads are issued before the current chunk's MFMAs and parked in registers.
-// At the end the WK row-group sums are added in wave order through LDS and the workgroup
-// writes one slice [slice][co][ci][tap]; splitk_reduce_kernel adds the slices in order.
+// Staging is by aligned 16-byte words of the tensors' own rows: the staged X patch starts at
+// the image column x0 - pwa, pwa the padding rounded up to 4, so that every word is either
+// wholly inside a row or wholly outside; the fragment reads start pwa - pw floats in. A thread
+// keeps one relative offset per word; whether the word exists for a given chunk (row inside the
+// image, image inside the batch) is ONE unsigned compare of offset + chunk base against a
+// limit, and words that do not exist are read from a zero word instead, which keeps the loads
+// free of branches. Tensors whose rows are not multiples of four floats take the same words as
+// four scalar loads.
+//
+// A workgroup owns 32*WCO output channels x 32 input channels x its taps for a range of pixel
+// chunks (WK row groups of 64/TC output rows x TC columns). Waves: WCO channel blocks x WK row groups of the
+// chunk x WFY filter-row groups; a wave keeps (R/WFY)*S accumulators, up to 144 registers, so
+// the kernel runs one workgroup per CU with the full register file. The next chunk's global
+// loads are issued before the current chunk's MFMAs and parked in registers. At the end the
+// WK row-group sums are added pairwise through LDS and the workgroup writes one slice
+// [slice][co][ci][tap]; splitk_reduce_kernel adds the slices in order.
+//
+// 5x5 windows: 25 accumulators do not fit one wave, so the filter rows go to different
+// WORKGROUPS (grid z = channel block x filter row) and the kernel runs as a 1x5 window whose
+// input rows are shifted by the filter row. Such a window needs no halo rows, so on small
+// images a chunk holds TI whole images stacked as rows.
 #include "gemm_mfma.h"
 
 namespace tdh {
@@ -28,34 +42,53 @@ namespace tdh {
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int DWH_NX_MAX  = 36;  // X elements a thread stages per chunk (at most)
-constexpr int DWH_NDY_MAX = 8;   // dY 16-byte words a thread stages per chunk (at most)
+constexpr int DWH_NDY = 8;   // dY words a thread stages per chunk
+constexpr int DWH_NEVER = -(1 << 30);  // relative offset of a word that never exists
+
+// a word that does not exist is loaded from here (not const: the loads must stay in the global
+// address space, like those of the tensors)
+__device__ __align__(16) float dwh_zero_word[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 
 struct DwHaloArgs {
   const float *x, *dy;
-  float *partial;  // [slices][Kc][C*R*S]
+  float *partial;  // [slices][Kc][C*RF*S]
   int batch, C, Kc, H, W, OH, OW, ph, pw;
-  int TRw;         // output rows one wave row-group takes per chunk
+  int TI;          // whole images stacked in a chunk (1: a chunk is WK*64/TC rows of one image)
   int tiles_x, chunks_total, chunks_per_slice;
-  int plane, plane_p, dyp;  // staged X plane (rows*PITCH), its padded stride, dY channel stride
-  int nx, ndy;              // staging trips per thread
-  int dy_vec;               // dY rows allow aligned 16-byte loads
-  FastDiv div_pitch, div_rowchunks, div_dyq;  // by PITCH, chunks per image, words per dY channel
+  int plane_p;     // channel stride of the staged X planes (odd)
+  int dyp;         // channel stride of the staged dY planes (4 mod 32)
+  int pwa;         // staged X column 0 is image column x0 - pwa
+  FastDiv div_rowchunks, div_oh;
 };
 
-template <int R, int S, int TC, int WCO, int WK, int WFY>
+// R: filter rows one workgroup covers, RF: filter rows of the window (RF/R workgroups share a
+// channel block), VEC: the rows of X and dY allow aligned 16-byte loads
+template <int R, int S, int TC, int WCO, int WK, int WFY, int RF, bool VEC>
 __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(const DwHaloArgs a) {
   constexpr int NT    = 64 * WCO * WK * WFY;
+  constexpr int FYB   = RF / R;
   constexpr int RPW   = R / WFY;  // filter rows per wave
   constexpr int NACC  = RPW * S;
   constexpr int BCO   = 32 * WCO;
-  constexpr int PITCH = (TC + S - 1 + 3) & ~3;
-  constexpr int NG    = TC / 8;   // 4-pixel groups per row and half
+  constexpr int NQ    = (3 + TC + S - 1 + 3) / 4;  // words per staged X row
+  constexpr int PITCH = 4 * NQ;
   constexpr int TPC   = NT / 32;  // threads staging one X channel plane
+  constexpr int NG    = TC / 8;   // 4-pixel groups per row and half
+  constexpr int TRW   = 64 / TC;  // output rows one wave row-group takes per chunk
+  constexpr int STEPS = TRW * NG; // (row, group) steps of a chunk's MFMA loop: always 8
+  constexpr int TR    = TRW * WK;
+  constexpr int PRQ   = (TR + R - 1) * NQ;        // words of a staged X plane
+  constexpr int NXI   = (PRQ + TPC - 1) / TPC;    // X words a thread stages per chunk
+  static_assert(NXI <= 16, "the keep bits of the scalar loads cover 16 words");
   constexpr int LOG_TC = TC == 64 ? 6 : TC == 32 ? 5 : TC == 16 ? 4 : 3;
+  constexpr int DQ    = 16 * WK;  // words per staged dY channel: 64 pixels per row group
+  constexpr int DCO   = NT / DQ;  // dY channels one staging trip covers
   static_assert(R % WFY == 0, "filter rows must divide among the waves");
-  static_assert(S <= 5, "two 16-byte words per filter row hold 4+S-1 <= 8 pixels");
+  static_assert(RF % R == 0, "filter rows must divide among the workgroups");
+  static_assert(BCO * DQ == NT * DWH_NDY, "dY staging trips");
+  static_assert(WFY == 1 || WK == 1, "row groups and filter-row groups are not combined");
 
   extern __shared__ __align__(16) float smem[];
   float *dy_l = smem;                // [BCO][dyp]
@@ -64,48 +97,139 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wco = wave % WCO, wk = (wave / WCO) % WK, wfy = wave / (WCO * WK);
   const int tx = blockIdx.x % a.tiles_x, slice = blockIdx.x / a.tiles_x;
-  const int x0 = tx * TC, co0 = blockIdx.y * BCO, ci0 = blockIdx.z * 32;
-  const int TR = a.TRw * WK;
+  const int x0 = tx * TC, co0 = blockIdx.y * BCO;
+  const int ci0 = (blockIdx.z / FYB) * 32, fy0 = (blockIdx.z % FYB) * R;
   const int hw = a.H * a.W, ohw = a.OH * a.OW;
+  const int chw = a.C * hw, kohw = a.Kc * ohw;
 
-  // ---- X staging plan: thread -> channel xc, elements xl + TPC*i of the plane [rows][PITCH]
+  // ---- X staging plan: thread -> channel xc, words xl + TPC*i of the plane [rows][NQ]
   const int xc = tid / TPC, xl = tid % TPC;
-  const bool xch_ok = ci0 + xc < a.C;
-  int xrel[DWH_NX_MAX];
-  unsigned long long xcol = 0;  // element i lies in a column inside the image
+  int xrel[NXI];            // offset of word i from the chunk's base, or DWH_NEVER
+  unsigned long long xkeep = 0; // scalar loads: 4 bits per word, float k lies inside the row
 #pragma unroll
-  for (int i = 0; i < DWH_NX_MAX; ++i) {
-    xrel[i] = 0;
+  for (int i = 0; i < NXI; ++i) {
+    xrel[i] = DWH_NEVER;
     const int pe = xl + TPC * i;
-    if (i < a.nx && pe < a.plane) {
-      uint32_t r, c;
-      a.div_pitch.divmod(pe, r, c);
-      const int ix = x0 - a.pw + static_cast<int>(c);
-      xrel[i]      = static_cast<int>(r) * a.W + ix;
-      if (static_cast<int>(c) < TC + S - 1 && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W))
-        xcol |= 1ull << i;
+    if (pe < PRQ && ci0 + xc < a.C) {
+      int r = pe / NQ;
+      const int q = pe - r * NQ;
+      const int ix = x0 - a.pwa + 4 * q;
+      unsigned keep = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (static_cast<unsigned>(ix + k) < static_cast<unsigned>(a.W)) keep |= 1u << k;
+      bool ok = VEC ? keep == 15u : keep != 0u;
+      int base = 0;
+      if (a.TI > 1) {
+        // stacked whole images: the row inside its image is fixed, the chunk only picks images
+        uint32_t il, rr;
+        a.div_oh.divmod(static_cast<uint32_t>(r), il, rr);
+        r = static_cast<int>(rr) + fy0 - a.ph;
+        ok = ok && static_cast<int>(il) < a.TI && static_cast<unsigned>(r) < static_cast<unsigned>(a.H);
+        base = static_cast<int>(il) * chw;
+      }
+      if (ok) {
+        xrel[i] = base + r * a.W + ix;
+        if (!VEC) xkeep |= static_cast<unsigned long long>(keep) << (4 * i);
+      }
     }
   }
   const float *x_chan = a.x + static_cast<size_t>(ci0 + xc) * hw;
 
-  // ---- dY staging plan: word e4 = tid + NT*i -> channel co, row r, columns c..c+3
-  int dyoff[DWH_NDY_MAX], dyrow[DWH_NDY_MAX], dylds[DWH_NDY_MAX], dycol[DWH_NDY_MAX];
+  // ---- dY staging plan: word tid + NT*i -> channel dco + DCO*i, the same row and column for
+  //      every i
+  const int dq = tid % DQ, dco = tid / DQ;
+  const int dcol = x0 + ((4 * dq) & (TC - 1));
+  int dyrel = DWH_NEVER;
+  {
+    int r = (4 * dq) >> LOG_TC, base = 0;
+    bool ok = VEC ? dcol + 3 < a.OW : dcol < a.OW;
+    if (a.TI > 1) {
+      uint32_t il, rr;
+      a.div_oh.divmod(static_cast<uint32_t>(r), il, rr);
+      ok   = ok && static_cast<int>(il) < a.TI;
+      base = static_cast<int>(il) * kohw;
+      r    = static_cast<int>(rr);
+    }
+    if (ok) dyrel = base + r * a.OW + dcol;
+  }
+  const float *dy_chan = a.dy + static_cast<size_t>(co0 + dco) * ohw;
+  const float *zero = dwh_zero_word;
+
+  floatx4 rx[NXI];
+  floatx4 rdy[DWH_NDY];
+
+  // The loads of a chunk are issued in STEPS parts, one per step of the MFMA loop of the chunk
+  // before: every workgroup of the grid fetches at the same time, and a chunk's words issued
+  // in one go wait for HBM while the matrix cores idle.
+  const float *xb = nullptr, *dyb = nullptr;  // the chunk's image, this thread's channel
+  int xbase = 0, dybase = 0;                  // added to the words' relative offsets
+  unsigned xlimit = 0, dylimit = 0;
+  auto fetch_begin = [&](int chunk) {
+    uint32_t img, rc;
+    a.div_rowchunks.divmod(chunk, img, rc);
+    img *= a.TI;
+    const int y0   = a.TI > 1 ? 0 : rc * TR;
+    const int nimg = min(a.TI, a.batch - static_cast<int>(img));
+    xb      = x_chan + static_cast<size_t>(img) * chw;
+    xbase   = a.TI > 1 ? 0 : (y0 - a.ph + fy0) * a.W;
+    xlimit  = a.TI > 1 ? nimg * chw : hw;
+    dyb     = dy_chan + static_cast<size_t>(img) * kohw;
+    dybase  = y0 * a.OW;
+    dylimit = a.TI > 1 ? nimg * kohw : ohw;
+  };
+  auto fetch_part = [&](int part) {
 #pragma unroll
-  for (int i = 0; i < DWH_NDY_MAX; ++i) {
-    dyoff[i] = 0; dylds[i] = 0; dycol[i] = 0;
-    dyrow[i] = 1 << 20;  // never inside the image
-    const int e4 = tid + NT * i;
-    if (i < a.ndy && e4 < BCO * (TR << LOG_TC) / 4) {
-      uint32_t co, q;
-      a.div_dyq.divmod(e4, co, q);
-      const int r = static_cast<int>(4 * q) >> LOG_TC, c = static_cast<int>(4 * q) & (TC - 1);
-      dylds[i] = co * a.dyp + 4 * q;
-      if (co0 + static_cast<int>(co) < a.Kc && x0 + c < a.OW) {
-        dyrow[i] = r;
-        dycol[i] = x0 + c;
-        dyoff[i] = (co0 + co) * ohw + r * a.OW + x0 + c;
+    for (int i = 0; i < NXI; ++i) {
+      if (i % STEPS != part) continue;
+      const int rel = xrel[i] + xbase;
+      const bool ok = static_cast<unsigned>(rel) < xlimit;
+      if (VEC) {
+        rx[i] = *reinterpret_cast<const floatx4 *>(ok ? xb + rel : zero);
+      } else {
+        const unsigned keep = ok ? static_cast<unsigned>(xkeep >> (4 * (i & 15))) & 15u : 0u;
+        rx[i].x = *((keep & 1u) ? xb + rel : zero);
+        rx[i].y = *((keep & 2u) ? xb + rel + 1 : zero);
+        rx[i].z = *((keep & 4u) ? xb + rel + 2 : zero);
+        rx[i].w = *((keep & 8u) ? xb + rel + 3 : zero);
       }
     }
+#pragma unroll
+    for (int i = 0; i < DWH_NDY; ++i) {
+      if (i % STEPS != part) continue;
+      const int rel  = dyrel + dybase;
+      const bool oki = static_cast<unsigned>(rel) < dylimit && co0 + dco + DCO * i < a.Kc;
+      const float *p = dyb + static_cast<size_t>(DCO * i) * ohw + rel;
+      if (VEC) {
+        rdy[i] = *reinterpret_cast<const floatx4 *>(oki ? p : zero);
+      } else {
+        rdy[i].x = *(oki ? p : zero);
+        rdy[i].y = *((oki && dcol + 1 < a.OW) ? p + 1 : zero);
+        rdy[i].z = *((oki && dcol + 2 < a.OW) ? p + 2 : zero);
+        rdy[i].w = *((oki && dcol + 3 < a.OW) ? p + 3 : zero);
+      }
+    }
+  };
+  auto stage = [&]() {
+    float *xd = x_l + xc * a.plane_p + 4 * xl;
+#pragma unroll
+    for (int i = 0; i < NXI; ++i) {
+      if (xl + TPC * i < PRQ) {
+        float *d = xd + 4 * TPC * i;
+        d[0] = rx[i].x; d[1] = rx[i].y; d[2] = rx[i].z; d[3] = rx[i].w;
+      }
+    }
+    float *dd = dy_l + dco * a.dyp + 4 * dq;
+#pragma unroll
+    for (int i = 0; i < DWH_NDY; ++i) *reinterpret_cast<floatx4 *>(dd + DCO * i * a.dyp) = rdy[i];
+  };
+
+  const int c_begin = slice * a.chunks_per_slice;
+  const int c_end   = min(a.chunks_total, c_begin + a.chunks_per_slice);
+  if (c_begin < c_end) {
+    fetch_begin(c_begin);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) fetch_part(s);
   }
 
   floatx16 acc[NACC];
@@ -114,77 +238,29 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
 
-  float rx[DWH_NX_MAX];
-  float4 rdy[DWH_NDY_MAX];
-
-  auto fetch = [&](int chunk) {
-    uint32_t img, rc;
-    a.div_rowchunks.divmod(chunk, img, rc);
-    const int y0    = rc * TR;
-    const float *xb = x_chan + static_cast<size_t>(img) * a.C * hw;
-    const int ybase = (y0 - a.ph) * a.W;
-#pragma unroll
-    for (int i = 0; i < DWH_NX_MAX; ++i) {
-      const int rel = xrel[i] + ybase;
-      const bool ok = i < a.nx && xch_ok && ((xcol >> i) & 1ull) &&
-                      static_cast<unsigned>(rel) < static_cast<unsigned>(hw);
-      rx[i] = ok ? xb[rel] : 0.0f;
-    }
-    const float *dyb = a.dy + static_cast<size_t>(img) * a.Kc * ohw + y0 * a.OW;
-#pragma unroll
-    for (int i = 0; i < DWH_NDY_MAX; ++i) {
-      float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      if (i < a.ndy && y0 + dyrow[i] < a.OH) {
-        const float *p = dyb + dyoff[i];
-        if (a.dy_vec) {
-          v = *reinterpret_cast<const float4 *>(p);
-        } else {
-          v.x = p[0];
-          if (dycol[i] + 1 < a.OW) v.y = p[1];
-          if (dycol[i] + 2 < a.OW) v.z = p[2];
-          if (dycol[i] + 3 < a.OW) v.w = p[3];
-        }
-      }
-      rdy[i] = v;
-    }
-  };
-  auto stage = [&]() {
-#pragma unroll
-    for (int i = 0; i < DWH_NX_MAX; ++i) {
-      const int pe = xl + TPC * i;
-      if (i < a.nx && pe < a.plane) x_l[xc * a.plane_p + pe] = rx[i];
-    }
-#pragma unroll
-    for (int i = 0; i < DWH_NDY_MAX; ++i)
-      if (i < a.ndy && tid + NT * i < BCO * (TR << LOG_TC) / 4)
-        *reinterpret_cast<float4 *>(dy_l + dylds[i]) = rdy[i];
-  };
-
   // fragment bases of this lane: half k = lane/32 starts TC/2 pixels into the row
-  const float *ap = dy_l + (wco * 32 + (lane & 31)) * a.dyp + ((wk * a.TRw) << LOG_TC) + (lane >> 5) * (TC / 2);
-  const float *bp = x_l + (lane & 31) * a.plane_p + (wk * a.TRw + wfy * RPW) * PITCH + (lane >> 5) * (TC / 2);
+  const float *ap = dy_l + (wco * 32 + (lane & 31)) * a.dyp + ((wk * TRW) << LOG_TC) + (lane >> 5) * (TC / 2);
+  const float *bp = x_l + (lane & 31) * a.plane_p + (wk * TRW + wfy * RPW) * PITCH + (a.pwa - a.pw) +
+                    (lane >> 5) * (TC / 2);
 
-  const int c_begin = slice * a.chunks_per_slice;
-  const int c_end   = min(a.chunks_total, c_begin + a.chunks_per_slice);
-  if (c_begin < c_end) fetch(c_begin);
   for (int chunk = c_begin; chunk < c_end; ++chunk) {
     if (chunk > c_begin) __syncthreads();  // everyone is done reading the previous chunk
     stage();
     __syncthreads();
-    if (chunk + 1 < c_end) fetch(chunk + 1);
-    for (int r = 0; r < a.TRw; ++r) {
+    const bool more = chunk + 1 < c_end;
+    if (more) fetch_begin(chunk + 1);
 #pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        const float4 av4 = *reinterpret_cast<const float4 *>(ap + (r << LOG_TC) + 4 * g);
+    for (int s = 0; s < STEPS; ++s) {
+      {
+        const int r = s / NG, g = s % NG;
+        if (more) fetch_part(s);
+        const floatx4 av4 = *reinterpret_cast<const floatx4 *>(ap + (r << LOG_TC) + 4 * g);
         const float av[4] = {av4.x, av4.y, av4.z, av4.w};
-        float bv[RPW][8];
+        float bv[RPW][4 + S - 1];
 #pragma unroll
-        for (int fy = 0; fy < RPW; ++fy) {
-          const float4 b0 = *reinterpret_cast<const float4 *>(bp + (r + fy) * PITCH + 4 * g);
-          const float4 b1 = *reinterpret_cast<const float4 *>(bp + (r + fy) * PITCH + 4 * g + 4);
-          bv[fy][0] = b0.x; bv[fy][1] = b0.y; bv[fy][2] = b0.z; bv[fy][3] = b0.w;
-          bv[fy][4] = b1.x; bv[fy][5] = b1.y; bv[fy][6] = b1.z; bv[fy][7] = b1.w;
-        }
+        for (int fy = 0; fy < RPW; ++fy)
+#pragma unroll
+          for (int k = 0; k < 4 + S - 1; ++k) bv[fy][k] = bp[(r + fy) * PITCH + 4 * g + k];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -197,21 +273,21 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     }
   }
 
-  // ---- add the WK row-group sums in wave order, then write the slice
+  // ---- add the WK row-group sums pairwise (upper half of the groups onto the lower half)
   if (WK > 1) {
-    float *red = smem;  // [WCO*WFY][NACC*16][64]
-    for (int s = 1; s < WK; ++s) {
+    float *red = smem;  // [WK/2][WCO][NACC*16][64]
+    for (int h = WK / 2; h >= 1; h >>= 1) {
       __syncthreads();
-      if (wk == s) {
-        float *dst = red + static_cast<size_t>(wco + WCO * wfy) * (NACC * 16 * 64) + lane;
+      if (wk >= h && wk < 2 * h) {
+        float *dst = red + static_cast<size_t>((wk - h) * WCO + wco) * (NACC * 16 * 64) + lane;
 #pragma unroll
         for (int t = 0; t < NACC; ++t)
 #pragma unroll
           for (int r = 0; r < 16; ++r) dst[(t * 16 + r) * 64] = acc[t][r];
       }
       __syncthreads();
-      if (wk == 0) {
-        const float *src = red + static_cast<size_t>(wco + WCO * wfy) * (NACC * 16 * 64) + lane;
+      if (wk < h) {
+        const float *src = red + static_cast<size_t>(wk * WCO + wco) * (NACC * 16 * 64) + lane;
 #pragma unroll
         for (int t = 0; t < NACC; ++t)
 #pragma unroll
@@ -222,9 +298,10 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
   if (wk == 0) {
     // reg r of lane l: row (co) 8*(r/4) + 4*(l/32) + r%4, column (ci) l%32
     const int ci = ci0 + (lane & 31);
-    const int crs = a.C * R * S;
+    const int crs = a.C * RF * S;
     if (ci < a.C) {
-      float *dst = a.partial + static_cast<size_t>(blockIdx.x) * a.Kc * crs + ci * (R * S) + wfy * RPW * S;
+      float *dst = a.partial + static_cast<size_t>(blockIdx.x) * a.Kc * crs + ci * (RF * S) +
+                   (fy0 + wfy * RPW) * S;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int co = co0 + wco * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -239,6 +316,7 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
 struct DwHaloPlan {
   bool ok;
   int tc, wco, wk, wfy, nt;
+  int rows_block;  // filter rows one workgroup covers
   DwHaloArgs args;
   size_t lds_bytes;
   dim3 grid;
@@ -254,35 +332,38 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
                         int pw) {
   DwHaloPlan p;
   p.ok = false;
-  // 3x3 windows only: with 25 taps the accumulators of a channel block no longer fit one wave,
-  // and splitting the filter rows over five waves measured slower than the generic GEMM on
-  // the small images such layers see here
-  if (!(R == 3 && S == 3)) return p;
-  if (C < 16 || Kc < 16 || OW < 8 || OH < 2) return p;
+  const bool five = R == 5 && S == 5;
+  if (!(R == 3 && S == 3) && !five) return p;
+  if (C < 16 || Kc < 16 || OW < 8 || OH < 2 || pw > 4) return p;
   p.tc = OW >= 48 ? 64 : OW >= 24 ? 32 : OW >= 12 ? 16 : 8;
   p.wfy = 1;
-  p.wco = Kc > 32 ? 2 : 1;
+  p.wco = (Kc > 32 && !five) ? 2 : 1;
   p.wk  = 4 / p.wco;
   p.nt = 64 * p.wco * p.wk * p.wfy;
+  p.rows_block = five ? 1 : R;
   DwHaloArgs &a = p.args;
   a.batch = batch; a.C = C; a.Kc = Kc; a.H = H; a.W = W; a.OH = OH; a.OW = OW; a.ph = ph; a.pw = pw;
-  a.TRw = std::max(1, 64 / p.tc);
-  const int tr    = a.TRw * p.wk;
-  const int pitch = (p.tc + S - 1 + 3) & ~3;
-  a.plane   = (tr + R - 1) * pitch;
-  a.plane_p = pad_to_4_mod_32(a.plane);
+  const int tr = (64 / p.tc) * p.wk;
+  const int nq = (3 + p.tc + S - 1 + 3) / 4;
+  a.pwa = (pw + 3) & ~3;
+  a.TI = 1;
+  // whole images stacked as rows; rows past the last whole image stay empty
+  if (five && tr > OH) a.TI = tr / OH;
+  const int prq = (tr + p.rows_block - 1) * nq;
+  a.plane_p = (4 * prq) | 1;
   a.dyp     = pad_to_4_mod_32(tr * p.tc);
-  a.nx      = ceil_div(a.plane, p.nt / 32);
-  a.ndy     = ceil_div(32 * p.wco * tr * p.tc / 4, p.nt);
-  if (a.nx > DWH_NX_MAX || a.ndy > DWH_NDY_MAX) return p;
-  a.dy_vec        = (OW % 4 == 0) ? 1 : 0;
-  a.tiles_x       = ceil_div(OW, p.tc);
-  const int row_chunks = ceil_div(OH, tr);
-  a.chunks_total  = batch * row_chunks;
-  a.div_pitch     = FastDiv(pitch);
+  // the keep bits of the scalar loads cover 16 words a thread
+  if (ceil_div(prq, p.nt / 32) > 16) return p;
+  // offsets inside a chunk are 32-bit and must stay clear of the never-exists marker
+  if (static_cast<long>(a.TI) * std::max<long>(static_cast<long>(C) * H * W, static_cast<long>(Kc) * OH * OW) >=
+      (1L << 29))
+    return p;
+  a.tiles_x = ceil_div(OW, p.tc);
+  const int row_chunks = a.TI > 1 ? 1 : ceil_div(OH, tr);
+  a.chunks_total  = a.TI > 1 ? ceil_div(batch, a.TI) : batch * row_chunks;
   a.div_rowchunks = FastDiv(row_chunks);
-  a.div_dyq       = FastDiv(tr * p.tc / 4);
-  const int co_blocks = ceil_div(Kc, 32 * p.wco), ci_blocks = ceil_div(C, 32);
+  a.div_oh        = FastDiv(OH);
+  const int co_blocks = ceil_div(Kc, 32 * p.wco), ci_blocks = ceil_div(C, 32) * (R / p.rows_block);
   const long base = static_cast<long>(a.tiles_x) * co_blocks * ci_blocks;
   // one workgroup per CU; a slice should still cover a few chunks so that its prologue and
   // its partial tile are paid for
@@ -290,8 +371,9 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
   slices = std::min<long>(slices, std::max(1, a.chunks_total / 2));
   a.chunks_per_slice = ceil_div(a.chunks_total, static_cast<int>(slices));
   p.slices           = ceil_div(a.chunks_total, a.chunks_per_slice);
+  const int nacc = (p.rows_block / p.wfy) * S;
   const size_t stage_floats = static_cast<size_t>(32 * p.wco) * a.dyp + 32 * static_cast<size_t>(a.plane_p);
-  const size_t red_floats   = p.wk > 1 ? static_cast<size_t>(p.wco * p.wfy) * (R / p.wfy) * S * 16 * 64 : 0;
+  const size_t red_floats   = static_cast<size_t>(p.wk / 2) * p.wco * nacc * 16 * 64;
   p.lds_bytes = sizeof(float) * std::max(stage_floats, red_floats);
   if (p.lds_bytes > 150 * 1024) return p;
   if (static_cast<long>(a.tiles_x) * p.slices > 65535L * 16) return p;
@@ -300,9 +382,9 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
   return p;
 }
 
-template <int R, int S, int TC, int WCO, int WK, int WFY>
+template <int R, int S, int TC, int WCO, int WK, int WFY, int RF, bool VEC>
 int launch_dw_inst(const DwHaloPlan &p) {
-  auto kernel = conv_dw_halo_kernel<R, S, TC, WCO, WK, WFY>;
+  auto kernel = conv_dw_halo_kernel<R, S, TC, WCO, WK, WFY, RF, VEC>;
   if (p.lds_bytes > 64 * 1024) {
     // raised once per kernel instance and size: the default dynamic LDS limit is 64 KiB
     static size_t raised = 0;
@@ -318,11 +400,26 @@ int launch_dw_inst(const DwHaloPlan &p) {
   return TDH_OK;
 }
 
-template <int TC>
+template <int TC, bool VEC>
 int launch_dw_tc(const DwHaloPlan &p) {
-  if (p.wco == 2) return launch_dw_inst<3, 3, TC, 2, 2, 1>(p);
-  return launch_dw_inst<3, 3, TC, 1, 4, 1>(p);
+  if (p.rows_block == 1) return launch_dw_inst<1, 5, TC, 1, 4, 1, 5, VEC>(p);
+  if (p.wco == 2) return launch_dw_inst<3, 3, TC, 2, 2, 1, 3, VEC>(p);
+  // 8 columns x 4 row groups would stage 17 words a thread; the plan leaves that tile out
+  if (TC == 8) return set_error(TDH_ERR_INVALID, "conv_dw_halo_run: tile not built");
+  return launch_dw_inst<3, 3, (TC == 8 ? 16 : TC), 1, 4, 1, 3, VEC>(p);
 }
+
+template <bool VEC>
+int launch_dw_vec(const DwHaloPlan &p) {
+  switch (p.tc) {
+    case 64: return launch_dw_tc<64, VEC>(p);
+    case 32: return launch_dw_tc<32, VEC>(p);
+    case 16: return launch_dw_tc<16, VEC>(p);
+    default: return launch_dw_tc<8, VEC>(p);
+  }
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace
 
@@ -347,14 +444,11 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
   void *part = nullptr;
   TDH_TRY(ws_take(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc * crs, &part));
   p.args.x = x; p.args.dy = dy; p.args.partial = static_cast<float *>(part);
+  const bool vec = W % 4 == 0 && OW % 4 == 0 && aligned16(x) && aligned16(dy);
   {
     ProfScope prof("conv_dw_halo", Kc, crs, batch * OH * OW);
-    switch (p.tc) {
-      case 64: TDH_TRY(launch_dw_tc<64>(p)); break;
-      case 32: TDH_TRY(launch_dw_tc<32>(p)); break;
-      case 16: TDH_TRY(launch_dw_tc<16>(p)); break;
-      default: TDH_TRY(launch_dw_tc<8>(p)); break;
-    }
+    if (vec) TDH_TRY(launch_dw_vec<true>(p));
+    else TDH_TRY(launch_dw_vec<false>(p));
   }
   const int slices = static_cast<int>(p.grid.x);
   ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
