@@ -38,6 +38,9 @@ CONV = [
     (12, 12, 48, 5, 16, True, 1, 5), (40, 6, 16, 3, 16, False, 1, 1),
     # 5x5 windows split by filter row: stacked small images with a ragged last chunk, row chunks
     (10, 10, 16, 5, 40, True, 1, 7), (36, 36, 16, 5, 16, False, 1, 2), (8, 8, 32, 5, 64, True, 1, 11),
+    # stride-1 MFMA kernel with scalar loads: rows or channel counts that are not multiples of 4,
+    # a last chunk of reduction channels that is not full
+    (26, 26, 16, 3, 32, True, 1, 32), (14, 14, 16, 5, 32, True, 1, 64), (16, 16, 16, 3, 30, True, 1, 64),
     # direct small-Cin forward kernel: ragged tiles, one and two channel blocks
     (20, 17, 3, 3, 40, True, 1, 3), (23, 22, 1, 5, 33, False, 1, 2), (37, 9, 3, 5, 64, True, 1, 2),
 ]
