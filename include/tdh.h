@@ -201,6 +201,28 @@ void tdh_act_default_params(int kind, float *p);
 int tdh_act_fwd_p(int kind, const float *p, int batch, int len, const float *x, float *y);
 int tdh_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, const float *y,
                   const float *dy, float *dx);
+/* batch_normalization_layer (tiny_dnn/layers/batch_normalization_layer.h:127-169): tensors are
+ * [batch][channels][spatial]. train != 0: mean and variance receive this batch's moments
+ * (util/math_functions.h:25-96: variance over max(1, batch*spatial - 1)); train == 0: they are
+ * read (the moving averages). stddev[c] = sqrt(variance[c] + eps) is written either way and is
+ * what the backward pass divides by. y = (x - mean) / stddev. */
+int tdh_batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,
+                      float *mean, float *variance, float *stddev, float *y);
+/* batch_normalization_layer::back_propagation (batch_normalization_layer.h:87-125):
+ * dx = (dy - mean(dy) - mean(dy*y) * y) / stddev, means per channel over batch and space */
+int tdh_batchnorm_bwd(int channels, int spatial, int batch, const float *y, const float *dy,
+                      const float *stddev, float *dx);
+/* batch_normalization_layer::post_update (batch_normalization_layer.h:171-177):
+ * mean = momentum*mean + (1-momentum)*mean_cur, the same for the variance */
+int tdh_batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
+                                const float *var_cur, float *mean, float *variance);
+/* dropout_layer (tiny_dnn/layers/dropout_layer.h:84-117): mask is [batch][len] bytes of 0/1, drawn
+ * by the caller as the reference draws it (bernoulli(rate) per element, sample after sample);
+ * train != 0: y = mask * scale * x with scale = 1/(1-rate), else y = x (mask may be NULL).
+ * Backward (dropout_layer.h:62-82): dx = mask * dy, without the scale. */
+int tdh_dropout_fwd(int batch, int len, int train, float scale, const uint8_t *mask, const float *x,
+                    float *y);
+int tdh_dropout_bwd(int batch, int len, const uint8_t *mask, const float *dy, float *dx);
 /* gradient<E> for a mini-batch (tiny_dnn/lossfunctions/loss_function.h:191-218) */
 int tdh_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
 /* softmax_layer backward applied to cross_entropy_multiclass::df in one kernel:

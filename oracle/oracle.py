@@ -270,6 +270,72 @@ def act_bwd(kind, x, y, dy, params=None):
     return dx
 
 
+def batchnorm_fwd(channels, spatial, x, eps=1e-5, train=True, mean=None, variance=None):
+    """Returns (y, mean, variance, stddev); train=False reads mean/variance."""
+    lib = oracle_lib()
+    x, xp = _f(x)
+    mean = np.zeros(channels, np.float32) if mean is None else np.array(mean, np.float32)
+    variance = np.zeros(channels, np.float32) if variance is None else np.array(variance, np.float32)
+    stddev = np.zeros(channels, np.float32)
+    y = np.empty_like(x)
+    _chk(lib.tdo_batchnorm_fwd(channels, spatial, x.shape[0], C.c_float(eps), int(bool(train)), xp,
+                               mean.ctypes.data_as(f32p), variance.ctypes.data_as(f32p),
+                               stddev.ctypes.data_as(f32p), y.ctypes.data_as(f32p)), "batchnorm_fwd")
+    return y, mean, variance, stddev
+
+
+def batchnorm_bwd(channels, spatial, y, dy, stddev):
+    lib = oracle_lib()
+    y, yp = _f(y); dy, dyp = _f(dy); stddev, sp = _f(stddev)
+    dx = np.empty_like(y)
+    _chk(lib.tdo_batchnorm_bwd(channels, spatial, y.shape[0], yp, dyp, sp, dx.ctypes.data_as(f32p)),
+         "batchnorm_bwd")
+    return dx
+
+
+def batchnorm_update_moving(momentum, mean_cur, var_cur, mean, variance):
+    lib = oracle_lib()
+    mean = np.array(mean, np.float32); variance = np.array(variance, np.float32)
+    mc, mcp = _f(mean_cur); vc, vcp = _f(var_cur)
+    lib.tdo_batchnorm_update_moving(mean.size, C.c_float(momentum), mcp, vcp,
+                                    mean.ctypes.data_as(f32p), variance.ctypes.data_as(f32p))
+    return mean, variance
+
+
+def dropout_mask(seed, rate, batch, length, state=None):
+    """The mask dropout_layer draws after set_random_seed(seed) (one worker thread)."""
+    lib = oracle_lib()
+    st = np.zeros(625, np.uint32) if state is None else state
+    if state is None:
+        lib.tdo_mt_seed(st.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_uint32(seed))
+    mask = np.zeros((batch, length), np.uint8)
+    lib.tdo_dropout_mask(st.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_float(rate),
+                         C.c_size_t(batch * length), mask.ctypes.data_as(C.POINTER(C.c_uint8)))
+    return mask
+
+
+def dropout_fwd(mask, x, rate=0.5, train=True):
+    lib = oracle_lib()
+    x, xp = _f(x)
+    mask = np.ascontiguousarray(mask, np.uint8)
+    y = np.empty_like(x)
+    scale = np.float32(1) / (np.float32(1) - np.float32(rate))
+    _chk(lib.tdo_dropout_fwd(x.shape[0], x.shape[1], int(bool(train)), C.c_float(scale),
+                             mask.ctypes.data_as(C.POINTER(C.c_uint8)), xp, y.ctypes.data_as(f32p)),
+         "dropout_fwd")
+    return y
+
+
+def dropout_bwd(mask, dy):
+    lib = oracle_lib()
+    dy, dyp = _f(dy)
+    mask = np.ascontiguousarray(mask, np.uint8)
+    dx = np.empty_like(dy)
+    _chk(lib.tdo_dropout_bwd(dy.shape[0], dy.shape[1], mask.ctypes.data_as(C.POINTER(C.c_uint8)), dyp,
+                             dx.ctypes.data_as(f32p)), "dropout_bwd")
+    return dx
+
+
 def loss_grad(kind, y, t):
     lib = oracle_lib()
     y, yp = _f(y); t, tp = _f(t)
@@ -584,6 +650,46 @@ def ref_act(kind_name, x, dy=None, kind="scalar", params=None):
     _chk(lib.tdr_act_p(ACT[kind_name], prm, x.shape[0], x.shape[1], xp, y.ctypes.data_as(f32p), dyp,
                        dx.ctypes.data_as(f32p)), "ref act")
     return y, dx
+
+
+def ref_batchnorm(channels, spatial, x, dy=None, eps=1e-5, train=True, mean=None, variance=None,
+                  kind="scalar"):
+    """The compiled reference's batch_normalization_layer: (y, mean, variance[, dx])."""
+    lib = ref_lib(kind)
+    x, xp = _f(x)
+    mean = np.zeros(channels, np.float32) if mean is None else np.array(mean, np.float32)
+    variance = np.zeros(channels, np.float32) if variance is None else np.array(variance, np.float32)
+    y = np.empty_like(x)
+    dx = np.empty_like(x) if dy is not None else None
+    dyp = _f(dy)[1] if dy is not None else None
+    _chk(lib.tdr_batchnorm(channels, spatial, x.shape[0], C.c_float(eps), int(bool(train)), xp,
+                           mean.ctypes.data_as(f32p), variance.ctypes.data_as(f32p),
+                           y.ctypes.data_as(f32p), dyp,
+                           dx.ctypes.data_as(f32p) if dx is not None else None), "ref batchnorm")
+    return (y, mean, variance) if dy is None else (y, mean, variance, dx)
+
+
+def ref_batchnorm_post_update(channels, spatial, x, mean, variance, eps=1e-5, momentum=0.999,
+                              kind="scalar"):
+    lib = ref_lib(kind)
+    x, xp = _f(x)
+    mean = np.array(mean, np.float32); variance = np.array(variance, np.float32)
+    _chk(lib.tdr_batchnorm_post_update(channels, spatial, x.shape[0], C.c_float(eps),
+                                       C.c_float(momentum), xp, mean.ctypes.data_as(f32p),
+                                       variance.ctypes.data_as(f32p)), "ref batchnorm post_update")
+    return mean, variance
+
+
+def ref_dropout(x, dy, rate, seed, kind="scalar"):
+    """The compiled reference's dropout_layer after set_random_seed(seed): (mask, y, dx)."""
+    lib = ref_lib(kind)
+    x, xp = _f(x); dy, dyp = _f(dy)
+    mask = np.zeros(x.shape, np.uint8)
+    y = np.empty_like(x); dx = np.empty_like(x)
+    _chk(lib.tdr_dropout(x.shape[1], x.shape[0], C.c_float(rate), C.c_uint32(seed), xp,
+                         mask.ctypes.data_as(C.POINTER(C.c_uint8)), y.ctypes.data_as(f32p), dyp,
+                         dx.ctypes.data_as(f32p)), "ref dropout")
+    return mask, y, dx
 
 
 def ref_loss_grad(kind_name, y, t, kind="scalar"):

@@ -31,6 +31,7 @@
 #include <cstdint>
 #include <cstring>
 #include <memory>
+#include <sstream>
 #include <vector>
 
 using namespace tiny_dnn;
@@ -303,6 +304,74 @@ int tdr_act_p(int kind, const float *p, int batch, int len, const float *x, floa
 int tdr_act(int kind, int batch, int len, const float *x, float *y, const float *dy, float *dx) {
   const float none[2] = {0.0f, 0.0f};
   return kind <= 3 ? tdr_act_p(kind, none, batch, len, x, y, dy, dx) : -2;
+}
+
+/* batch_normalization_layer: forward in the given phase, then backward. In the train phase the
+ * layer's batch moments come back in mean/variance; in the test phase mean/variance are set on
+ * the layer first. stddev comes back as sqrt(variance + eps) (the layer keeps it private). */
+int tdr_batchnorm(int channels, int spatial, int batch, float eps, int train, const float *x,
+                  float *mean, float *variance, float *y, const float *dy, float *dx) {
+  try {
+    batch_normalization_layer bn((size_t)spatial, (size_t)channels, eps, 0.999f,
+                                 train ? net_phase::train : net_phase::test);
+    if (!train) {
+      bn.set_mean(vec_t(mean, mean + channels));
+      bn.set_variance(vec_t(variance, variance + channels));
+    } else {
+      bn.update_immidiately(true);  /* copies the batch moments into mean_/variance_, read by save() */
+    }
+    const size_t len = (size_t)channels * spatial;
+    layer_fwd(bn, batch, x, len, y, len);
+    if (train) {
+      std::ostringstream os;
+      bn.save(os);
+      std::istringstream is(os.str());
+      for (int i = 0; i < channels; i++) is >> mean[i];
+      for (int i = 0; i < channels; i++) is >> variance[i];
+    }
+    if (dy) layer_bwd(bn, batch, dy, len, dx, len);
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* batch_normalization_layer::post_update after one train-phase forward of x, starting from the
+ * moving averages mean/variance (in and out) */
+int tdr_batchnorm_post_update(int channels, int spatial, int batch, float eps, float momentum,
+                              const float *x, float *mean, float *variance) {
+  try {
+    batch_normalization_layer bn((size_t)spatial, (size_t)channels, eps, momentum, net_phase::train);
+    bn.set_mean(vec_t(mean, mean + channels));
+    bn.set_variance(vec_t(variance, variance + channels));
+    const size_t len = (size_t)channels * spatial;
+    layer_fwd(bn, batch, x, len, nullptr, len);
+    bn.post_update();
+    std::ostringstream os;
+    bn.save(os);
+    std::istringstream is(os.str());
+    for (int i = 0; i < channels; i++) is >> mean[i];
+    for (int i = 0; i < channels; i++) is >> variance[i];
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
+/* dropout_layer in the train phase after set_random_seed(seed): forward (mask and y come back),
+ * then backward. Meaningful with one worker thread only: the samples draw from one generator. */
+int tdr_dropout(int len, int batch, float rate, unsigned int seed, const float *x,
+                unsigned char *mask, float *y, const float *dy, float *dx) {
+  try {
+    dropout_layer dl((size_t)len, rate, net_phase::train);
+    set_random_seed(seed);
+    const int threads = omp_get_max_threads();
+    omp_set_num_threads(1);  /* the samples share one generator: any other count races */
+    layer_fwd(dl, batch, x, len, y, len);
+    omp_set_num_threads(threads);
+    for (int s = 0; s < batch; s++) {
+      const std::vector<uint8_t> &m = dl.get_mask((size_t)s);
+      std::memcpy(mask + (size_t)len * s, m.data(), len);
+    }
+    if (dy) layer_bwd(dl, batch, dy, len, dx, len);
+    return 0;
+  } catch (const std::exception &) { return -1; }
 }
 
 /* kind: 0 mse, 1 cross_entropy_multiclass, 2 cross_entropy */

@@ -720,8 +720,152 @@ int tdo_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, 
 
 /* ------------------------------------------------------------------ losses */
 
-/* gradient<E> for a mini-batch, tiny_dnn/lossfunctions/loss_function.h:191-218;
- * mse::df :28-36, cross_entropy::df :120-128, cross_entropy_multiclass::df :143-150 */
+/* ------------------------------------------------- batch normalization, dropout */
+
+/* tiny_dnn/util/math_functions.h:25-37 and 68-79: per channel, the samples' runs are added one
+ * after the other onto one float (std::accumulate), then divided by (float)batch*spatial */
+static void moments_mean(int channels, int spatial, int batch, const float *in, float *mean) {
+  for (int j = 0; j < channels; j++) mean[j] = 0.0f;
+  for (int i = 0; i < batch; i++)
+    for (int j = 0; j < channels; j++) {
+      const float *p = in + ((size_t)i * channels + j) * spatial;
+      float r = mean[j];
+      for (int k = 0; k < spatial; k++) r = r + p[k];
+      mean[j] = r;
+    }
+  const float denom = (float)batch * spatial;
+  for (int j = 0; j < channels; j++) mean[j] = mean[j] / denom;
+}
+
+/* tiny_dnn/util/math_functions.h:39-61: sum of pow(x - mean, 2) over max(1, batch*spatial - 1) */
+static void moments_variance(int channels, int spatial, int batch, const float *in,
+                             const float *mean, float *variance) {
+  for (int j = 0; j < channels; j++) variance[j] = 0.0f;
+  for (int i = 0; i < batch; i++)
+    for (int j = 0; j < channels; j++) {
+      const float *p = in + ((size_t)i * channels + j) * spatial;
+      const float ex = mean[j];
+      float r = variance[j];
+      /* the unqualified pow(x - ex, float_t{2.0}) of the reference is the C library's
+       * pow(double, double): the square and the addition are carried out in double and
+       * rounded to float once per element */
+      for (int k = 0; k < spatial; k++) {
+        const double d = (double)(p[k] - ex);
+        r = (float)((double)r + d * d);
+      }
+      variance[j] = r;
+    }
+  float denom = (float)((size_t)batch * spatial) - 1.0f;
+  if (denom < 1.0f) denom = 1.0f;
+  for (int j = 0; j < channels; j++) variance[j] = variance[j] / denom;
+}
+
+/* batch_normalization_layer.h:127-169 */
+int tdo_batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,
+                      float *mean, float *variance, float *stddev, float *y) {
+  if (channels < 0 || spatial < 0 || batch < 0) return -1;
+  if (train) {
+    moments_mean(channels, spatial, batch, x, mean);
+    moments_variance(channels, spatial, batch, x, mean, variance);
+  }
+  for (int j = 0; j < channels; j++) stddev[j] = sqrtf(variance[j] + eps);
+  for (int i = 0; i < batch; i++)
+    for (int j = 0; j < channels; j++) {
+      const float m = mean[j];
+      for (int k = 0; k < spatial; k++) {
+        const size_t idx = ((size_t)i * channels + j) * spatial + k;
+        y[idx] = (x[idx] - m) / stddev[j];
+      }
+    }
+  return 0;
+}
+
+/* batch_normalization_layer.h:87-125 */
+int tdo_batchnorm_bwd(int channels, int spatial, int batch, const float *y, const float *dy,
+                      const float *stddev, float *dx) {
+  if (channels < 0 || spatial < 0 || batch < 0) return -1;
+  const size_t total = (size_t)batch * channels * spatial;
+  float *prod = (float *)malloc(sizeof(float) * (total ? total : 1));
+  float *m_prod = (float *)malloc(sizeof(float) * (channels ? channels : 1));
+  float *m_dy = (float *)malloc(sizeof(float) * (channels ? channels : 1));
+  if (!prod || !m_prod || !m_dy) { free(prod); free(m_prod); free(m_dy); return -1; }
+  for (size_t i = 0; i < total; i++) prod[i] = y[i] * dy[i];
+  moments_mean(channels, spatial, batch, prod, m_prod);
+  moments_mean(channels, spatial, batch, dy, m_dy);
+  for (int i = 0; i < batch; i++)
+    for (int j = 0; j < channels; j++)
+      for (int k = 0; k < spatial; k++) {
+        const size_t idx = ((size_t)i * channels + j) * spatial + k;
+        float v = dy[idx] - m_dy[j] - m_prod[j] * y[idx];
+        dx[idx] = v / stddev[j];
+      }
+  free(prod); free(m_prod); free(m_dy);
+  return 0;
+}
+
+/* batch_normalization_layer.h:171-177 */
+void tdo_batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
+                                 const float *var_cur, float *mean, float *variance) {
+  for (int i = 0; i < channels; i++) {
+    mean[i]     = momentum * mean[i] + (1 - momentum) * mean_cur[i];
+    variance[i] = momentum * variance[i] + (1 - momentum) * var_cur[i];
+  }
+}
+
+/* dropout_layer.h:84-117 */
+int tdo_dropout_fwd(int batch, int len, int train, float scale, const unsigned char *mask,
+                    const float *x, float *y) {
+  if (batch < 0 || len < 0) return -1;
+  const size_t total = (size_t)batch * len;
+  for (size_t i = 0; i < total; i++) y[i] = train ? mask[i] * scale * x[i] : x[i];
+  return 0;
+}
+
+/* dropout_layer.h:62-82 */
+int tdo_dropout_bwd(int batch, int len, const unsigned char *mask, const float *dy, float *dx) {
+  if (batch < 0 || len < 0) return -1;
+  const size_t total = (size_t)batch * len;
+  for (size_t i = 0; i < total; i++) dx[i] = mask[i] * dy[i];
+  return 0;
+}
+
+/* MT19937 (Matsumoto & Nishimura 1998) as std::mt19937 specifies it: seeding by the linear
+ * recurrence 1812433253, tempering (11, 7/0x9d2c5680, 15/0xefc60000, 18) */
+void tdo_mt_seed(unsigned int *state, unsigned int seed) {
+  state[0] = seed;
+  for (unsigned int i = 1; i < 624; i++) state[i] = 1812433253u * (state[i - 1] ^ (state[i - 1] >> 30)) + i;
+  state[624] = 624;
+}
+
+static unsigned int mt_next(unsigned int *mt) {
+  if (mt[624] >= 624) {
+    for (int k = 0; k < 624; k++) {
+      const unsigned int yv = (mt[k] & 0x80000000u) | (mt[(k + 1) % 624] & 0x7fffffffu);
+      mt[k] = mt[(k + 397) % 624] ^ (yv >> 1) ^ ((yv & 1u) ? 0x9908b0dfu : 0u);
+    }
+    mt[624] = 0;
+  }
+  unsigned int v = mt[mt[624]++];
+  v ^= v >> 11;
+  v ^= (v << 7) & 0x9d2c5680u;
+  v ^= (v << 15) & 0xefc60000u;
+  v ^= v >> 18;
+  return v;
+}
+
+/* util/random.h:67-69 with libstdc++'s uniform_real_distribution<float>(0,1): one 32-bit draw
+ * converted to float, divided by 2^32, and clamped below 1 */
+void tdo_dropout_mask(unsigned int *state, float rate, size_t n, unsigned char *mask) {
+  for (size_t i = 0; i < n; i++) {
+    float u = (float)mt_next(state) / 4294967296.0f;
+    if (u >= 1.0f) u = nextafterf(1.0f, 0.0f);
+    mask[i] = u <= rate ? 1 : 0;
+  }
+}
+
+
+
+/* gradient<E> for a mini-batch, tiny_dnn/lossfunctions/loss_function.h:191-218; * mse::df :28-36, cross_entropy::df :120-128, cross_entropy_multiclass::df :143-150 */
 int tdo_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy) {
   const size_t n = (size_t)batch * len;
   switch (kind) {

@@ -107,6 +107,25 @@ int tdo_act_fwd_p(int kind, const float *p, int batch, int len, const float *x, 
 int tdo_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, const float *y,
                   const float *dy, float *dx);
 
+/* batch normalization over [batch][channels][spatial] (batch_normalization_layer.h,
+ * util/math_functions.h:25-96); train != 0 computes mean/variance from x, else reads them */
+int tdo_batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,
+                      float *mean, float *variance, float *stddev, float *y);
+int tdo_batchnorm_bwd(int channels, int spatial, int batch, const float *y, const float *dy,
+                      const float *stddev, float *dx);
+void tdo_batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
+                                 const float *var_cur, float *mean, float *variance);
+/* dropout (dropout_layer.h): mask [batch][len] of 0/1 */
+int tdo_dropout_fwd(int batch, int len, int train, float scale, const unsigned char *mask,
+                    const float *x, float *y);
+int tdo_dropout_bwd(int batch, int len, const unsigned char *mask, const float *dy, float *dx);
+/* The reference's generator (util/random.h:19-69): one std::mt19937, seeded with 1 unless
+ * set_random_seed is called, and bernoulli(p) = uniform_real_distribution<float>(0,1) <= p.
+ * state: 625 words (624 of MT19937 state, then the position); tdo_mt_seed fills it. */
+void tdo_mt_seed(unsigned int *state, unsigned int seed);
+/* mask[i] = bernoulli(rate) for n elements, advancing state */
+void tdo_dropout_mask(unsigned int *state, float rate, size_t n, unsigned char *mask);
+
 /* loss gradient for a mini-batch (no 1/batch factor, as in the reference) */
 int tdo_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
 float tdo_loss_value(int kind, int batch, int len, const float *y, const float *t);

@@ -76,6 +76,11 @@ def act_golden():
 
 
 @pytest.fixture(scope="session")
+def norm_golden():
+    return np.load(os.path.join(GOLDEN, "norm.npz"))
+
+
+@pytest.fixture(scope="session")
 def net_steps():
     return np.load(os.path.join(GOLDEN, "net_steps.npz"))
 

@@ -409,3 +409,74 @@ def test_device_copy_is_exact(T, n, dst_off, src_off):
     want = dst0.copy()
     want[dst_off // 4: dst_off // 4 + n] = src[src_off // 4: src_off // 4 + n]
     assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- batch normalization, dropout
+@pytest.mark.parametrize("shape", [(5, 7, 4), (3, 100, 9), (64, 256, 128), (4, 1, 1), (130, 33, 70)])
+def test_batchnorm_matches_oracle(T, O, shape):
+    c, s, b = shape
+    rng = np.random.default_rng(c + s)
+    x = (rng.standard_normal((b, c * s)) * 2 + 0.5).astype(np.float32)
+    dy = rng.standard_normal((b, c * s)).astype(np.float32)
+    xd, dyd = T.to_device(x), T.to_device(dy)
+    y, dx = T.DevBuf(x.shape), T.DevBuf(x.shape)
+    mean, var, sd = T.DevBuf((c,)), T.DevBuf((c,)), T.DevBuf((c,))
+    T.batchnorm_fwd(c, s, b, xd, mean, var, sd, y)
+    ry, rmean, rvar, rsd = O.batchnorm_fwd(c, s, x)
+    assert_close(mean.numpy(), rmean, 1e-5, "mean")
+    assert_close(var.numpy(), rvar, 1e-5, "variance")
+    assert_close(sd.numpy(), rsd, 1e-5, "stddev")
+    assert_close(y.numpy(), ry, REL_TOL, "y")
+    T.batchnorm_bwd(c, s, b, T.to_device(ry), dyd, T.to_device(rsd), dx)
+    assert_close(dx.numpy(), O.batchnorm_bwd(c, s, ry, dy, rsd), REL_TOL, "dx")
+    # test phase: the given moving averages are read, not written
+    m0, v0 = rng.standard_normal(c).astype(np.float32), rng.uniform(0.5, 2, c).astype(np.float32)
+    md, vd = T.to_device(m0), T.to_device(v0)
+    T.batchnorm_fwd(c, s, b, xd, md, vd, sd, y, train=False)
+    assert_close(y.numpy(), O.batchnorm_fwd(c, s, x, train=False, mean=m0, variance=v0)[0], REL_TOL, "test phase")
+    assert np.array_equal(md.numpy(), m0) and np.array_equal(vd.numpy(), v0)
+    T.batchnorm_update_moving(c, 0.9, mean, var, md, vd)
+    rm1, rv1 = O.batchnorm_update_moving(0.9, rmean, rvar, m0, v0)
+    assert_close(md.numpy(), rm1, 1e-5, "moving mean")
+    assert_close(vd.numpy(), rv1, 1e-5, "moving variance")
+
+
+def test_norm_layers_match_reference_outputs(T, norm_golden):
+    """Against outputs of the compiled reference itself (tests/golden/norm.npz)."""
+    g = norm_golden
+    i = 0
+    while f"bn{i}.x" in g:
+        x, dy = g[f"bn{i}.x"], g[f"bn{i}.dy"]
+        c = g[f"bn{i}.mean"].size
+        s, b = x.shape[1] // c, x.shape[0]
+        y, dx = T.DevBuf(x.shape), T.DevBuf(x.shape)
+        mean, var, sd = T.DevBuf((c,)), T.DevBuf((c,)), T.DevBuf((c,))
+        T.batchnorm_fwd(c, s, b, T.to_device(x), mean, var, sd, y)
+        assert_close(y.numpy(), g[f"bn{i}.y"], REL_TOL, "y")
+        assert_close(var.numpy(), g[f"bn{i}.var"], 1e-5, "variance")
+        T.batchnorm_bwd(c, s, b, T.to_device(g[f"bn{i}.y"]), T.to_device(dy), sd, dx)
+        assert_close(dx.numpy(), g[f"bn{i}.dx"], REL_TOL, "dx")
+        i += 1
+    from tests.golden.make_fixtures import DROPOUT_CASES
+    x, dy = g["do.x"], g["do.dy"]
+    for k, (seed, rate) in enumerate(DROPOUT_CASES):
+        mask = T.dropout_mask(T.Mt19937(seed), rate, *x.shape)
+        assert np.array_equal(mask, g[f"do{k}.mask"])           # host-side draw, bit for bit
+        md = T.to_device(mask, np.uint8)
+        y, dx = T.DevBuf(x.shape), T.DevBuf(x.shape)
+        T.dropout_fwd(x.shape[0], x.shape[1], md, T.to_device(x), y, rate=rate)
+        assert np.array_equal(y.numpy(), g[f"do{k}.y"])
+        T.dropout_bwd(x.shape[0], x.shape[1], md, T.to_device(dy), dx)
+        assert np.array_equal(dx.numpy(), g[f"do{k}.dx"])
+    T.dropout_fwd(x.shape[0], x.shape[1], None, T.to_device(x), y, train=False)
+    assert np.array_equal(y.numpy(), x)
+
+
+def test_norm_argument_errors(T):
+    buf = T.DevBuf((4,))
+    with pytest.raises(T.TdhError, match="null tensor"):
+        T.batchnorm_fwd(2, 2, 1, None, buf, buf, buf, buf)
+    with pytest.raises(T.TdhError, match="null tensor"):
+        T.dropout_fwd(1, 4, None, buf, buf, train=True)
+    T.batchnorm_fwd(0, 2, 1, None, None, None, None, None)      # empty tensors: nothing to do
+    T.dropout_bwd(0, 4, None, None, None)

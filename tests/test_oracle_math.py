@@ -296,3 +296,94 @@ def test_update_weight_feeds_the_sum_not_the_mean(O):
     w = np.zeros(2, np.float32)
     O.update_weight(o, 1, merged, w)
     assert np.array_equal(w, -0.5 * merged)
+
+
+# ---------------------------------------------------------------- batch normalization, dropout
+def test_mt19937_known_answer(O):
+    """std::mt19937 is specified by its 10000th output for the default seed 5489: 4123659995
+    (ISO C++ [rand.predef]). The mask generator's engine must reproduce it."""
+    lib = O.oracle_lib()
+    import ctypes as C
+    st = np.zeros(625, np.uint32)
+    lib.tdo_mt_seed(st.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_uint32(5489))
+    # tdo_dropout_mask draws one word per element: rate 1 accepts every draw, so only the state moves
+    mask = np.zeros(9999, np.uint8)
+    lib.tdo_dropout_mask(st.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_float(1.0), C.c_size_t(9999),
+                         mask.ctypes.data_as(C.POINTER(C.c_uint8)))
+    assert mask.all()
+    # the 10000th word decides one more element against a threshold just below / above it
+    want = np.float32(4123659995) / np.float32(4294967296.0)
+    for rate, expect in ((np.nextafter(want, np.float32(0)), 0), (want, 1)):
+        s2 = st.copy()
+        one = np.zeros(1, np.uint8)
+        lib.tdo_dropout_mask(s2.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_float(rate), C.c_size_t(1),
+                             one.ctypes.data_as(C.POINTER(C.c_uint8)))
+        assert one[0] == expect
+
+
+def test_batchnorm_closed_forms(O):
+    rng = np.random.default_rng(5)
+    c, s, b = 6, 40, 10
+    x = (rng.standard_normal((b, c * s)) * 3 + 1).astype(np.float32)
+    y, mean, var, sd = O.batchnorm_fwd(c, s, x, eps=1e-5)
+    xs = x.reshape(b, c, s).astype(np.float64)
+    # moments: plain mean, variance over n-1 (util/math_functions.h:57-60)
+    np.testing.assert_allclose(mean, xs.mean(axis=(0, 2)), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(var, xs.var(axis=(0, 2), ddof=1), rtol=1e-5)
+    np.testing.assert_allclose(sd, np.sqrt(var.astype(np.float64) + 1e-5), rtol=1e-6)
+    ys = y.reshape(b, c, s).astype(np.float64)
+    assert np.abs(ys.mean(axis=(0, 2))).max() < 1e-5
+    np.testing.assert_allclose(ys.var(axis=(0, 2), ddof=1), var / (var + 1e-5), rtol=1e-4)
+    # backward: a gradient that is constant per channel, or proportional to y, is annihilated
+    const = np.repeat(rng.standard_normal(c).astype(np.float32), s)[None].repeat(b, 0)
+    assert np.abs(O.batchnorm_bwd(c, s, y, const, sd)).max() < 1e-5
+    dy = rng.standard_normal((b, c * s)).astype(np.float32)
+    dx = O.batchnorm_bwd(c, s, y, dy, sd).reshape(b, c, s).astype(np.float64)
+    assert np.abs(dx.sum(axis=(0, 2))).max() < 1e-3                  # sum of dx is zero
+    want = (dy.reshape(b, c, s) - dy.reshape(b, c, s).mean(axis=(0, 2), keepdims=True)
+            - (dy.reshape(b, c, s) * ys).mean(axis=(0, 2), keepdims=True) * ys) / sd[None, :, None]
+    np.testing.assert_allclose(dx, want, rtol=1e-4, atol=1e-5)
+    # one element per channel: variance over max(1, n-1) = 1 is zero, y = 0
+    y1, m1, v1, sd1 = O.batchnorm_fwd(3, 1, np.array([[1.0, -2.0, 3.0]], np.float32))
+    assert np.array_equal(m1, [1.0, -2.0, 3.0]) and not v1.any() and not y1.any()
+
+
+def test_dropout_quirks(O):
+    """dropout_layer keeps an element when bernoulli(rate) is TRUE, scales the kept ones by
+    1/(1-rate) on the way forward and by nothing on the way back (dropout_layer.h:62-113)."""
+    x = np.arange(1, 9, dtype=np.float32)[None]
+    mask = np.array([[1, 0, 1, 1, 0, 0, 1, 0]], np.uint8)
+    y = O.dropout_fwd(mask, x, rate=0.75)
+    assert np.array_equal(y, mask * np.float32(4.0) * x)
+    assert np.array_equal(O.dropout_fwd(mask, x, rate=0.75, train=False), x)
+    assert np.array_equal(O.dropout_bwd(mask, x), mask * x)
+    m = O.dropout_mask(1, 0.2, 50, 400)
+    assert abs(m.mean() - 0.2) < 0.01          # kept with probability `rate`
+    assert np.array_equal(m, O.dropout_mask(1, 0.2, 50, 400)) and not np.array_equal(m, O.dropout_mask(2, 0.2, 50, 400))
+
+
+def test_norm_layers_match_reference_outputs(O, norm_golden):
+    g = norm_golden
+    i = 0
+    while f"bn{i}.x" in g:
+        x, dy = g[f"bn{i}.x"], g[f"bn{i}.dy"]
+        c = g[f"bn{i}.mean"].size
+        s = x.shape[1] // c
+        y, mean, var, sd = O.batchnorm_fwd(c, s, x)
+        assert np.array_equal(y, g[f"bn{i}.y"]) and np.array_equal(mean, g[f"bn{i}.mean"])
+        assert np.array_equal(var, g[f"bn{i}.var"])
+        assert np.array_equal(O.batchnorm_bwd(c, s, y, dy, sd), g[f"bn{i}.dx"])
+        yt, _, _, _ = O.batchnorm_fwd(c, s, x, train=False, mean=g[f"bn{i}.m0"], variance=g[f"bn{i}.v0"])
+        assert np.array_equal(yt, g[f"bn{i}.y_test"])
+        m1, v1 = O.batchnorm_update_moving(0.9, mean, var, g[f"bn{i}.m0"], g[f"bn{i}.v0"])
+        # the reference prints the moving averages with 8 significant digits
+        np.testing.assert_allclose(m1, g[f"bn{i}.m1"], rtol=2e-7, atol=1e-9)
+        np.testing.assert_allclose(v1, g[f"bn{i}.v1"], rtol=2e-7, atol=1e-9)
+        i += 1
+    assert i == 4
+    from tests.golden.make_fixtures import DROPOUT_CASES
+    for k, (seed, rate) in enumerate(DROPOUT_CASES):
+        mask = O.dropout_mask(seed, rate, *g["do.x"].shape)
+        assert np.array_equal(mask, g[f"do{k}.mask"])
+        assert np.array_equal(O.dropout_fwd(mask, g["do.x"], rate), g[f"do{k}.y"])
+        assert np.array_equal(O.dropout_bwd(mask, g["do.dy"]), g[f"do{k}.dx"])

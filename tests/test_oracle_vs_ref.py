@@ -117,3 +117,36 @@ def test_vgg_style_step_bit_exact(ref, W):
         got = net.weight(i) if which == 0 else net.bias(i)
         assert np.all(np.isfinite(got))
         assert np.array_equal(got, rn.get_param(i, which)[:a.size]), (i, which)
+
+
+@pytest.mark.parametrize("shape", [(5, 7, 4), (3, 100, 9), (16, 64, 32), (4, 1, 1), (2, 3, 1)])
+def test_batchnorm_bit_exact(ref, shape):
+    O = ref
+    c, s, b = shape
+    rng = np.random.default_rng(c * 1000 + s)
+    x = (rng.standard_normal((b, c * s)) * 2 + 0.5).astype(np.float32)
+    dy = rng.standard_normal((b, c * s)).astype(np.float32)
+    y, mean, var, sd = O.batchnorm_fwd(c, s, x)
+    ry, rmean, rvar, rdx = O.ref_batchnorm(c, s, x, dy)
+    assert np.array_equal(y, ry) and np.array_equal(mean, rmean) and np.array_equal(var, rvar)
+    assert np.array_equal(O.batchnorm_bwd(c, s, y, dy, sd), rdx)
+    m0, v0 = rng.standard_normal(c).astype(np.float32), rng.uniform(0.5, 2, c).astype(np.float32)
+    yt = O.batchnorm_fwd(c, s, x, train=False, mean=m0, variance=v0)[0]
+    assert np.array_equal(yt, O.ref_batchnorm(c, s, x, train=False, mean=m0, variance=v0)[0])
+    m1, v1 = O.batchnorm_update_moving(0.9, mean, var, m0, v0)
+    rm1, rv1 = O.ref_batchnorm_post_update(c, s, x, m0, v0, momentum=0.9)
+    np.testing.assert_allclose(m1, rm1, rtol=2e-7, atol=1e-9)   # read back through the text format
+    np.testing.assert_allclose(v1, rv1, rtol=2e-7, atol=1e-9)
+
+
+@pytest.mark.parametrize("seed,rate", [(1, 0.3), (7, 0.5), (3, 0.9), (11, 0.0)])
+def test_dropout_bit_exact(ref, seed, rate):
+    O = ref
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((9, 333)).astype(np.float32)
+    dy = rng.standard_normal((9, 333)).astype(np.float32)
+    mask = O.dropout_mask(seed, rate, 9, 333)
+    rmask, ry, rdx = O.ref_dropout(x, dy, rate, seed)
+    assert np.array_equal(mask, rmask)
+    assert np.array_equal(O.dropout_fwd(mask, x, rate), ry)
+    assert np.array_equal(O.dropout_bwd(mask, dy), rdx)

@@ -369,6 +369,57 @@ def act_bwd(kind, batch, length, y, dy, dx, x=None, params=None):
                               _p(dy), _p(dx)), "tdh_act_bwd_p")
 
 
+def batchnorm_fwd(channels, spatial, batch, x, mean, variance, stddev, y, eps=1e-5, train=True):
+    """batch_normalization_layer::forward_propagation; train: mean/variance are written."""
+    check(lib().tdh_batchnorm_fwd(channels, spatial, batch, C.c_float(eps), int(bool(train)), _p(x),
+                                  _p(mean), _p(variance), _p(stddev), _p(y)), "tdh_batchnorm_fwd")
+
+
+def batchnorm_bwd(channels, spatial, batch, y, dy, stddev, dx):
+    check(lib().tdh_batchnorm_bwd(channels, spatial, batch, _p(y), _p(dy), _p(stddev), _p(dx)),
+          "tdh_batchnorm_bwd")
+
+
+def batchnorm_update_moving(channels, momentum, mean_cur, var_cur, mean, variance):
+    check(lib().tdh_batchnorm_update_moving(channels, C.c_float(momentum), _p(mean_cur), _p(var_cur),
+                                            _p(mean), _p(variance)), "tdh_batchnorm_update_moving")
+
+
+def dropout_fwd(batch, length, mask, x, y, rate=0.5, train=True):
+    """dropout_layer::forward_propagation; mask: device bytes [batch][length] (see dropout_mask)."""
+    scale = np.float32(1) / (np.float32(1) - np.float32(rate))
+    check(lib().tdh_dropout_fwd(batch, length, int(bool(train)), C.c_float(scale), _p(mask), _p(x),
+                                _p(y)), "tdh_dropout_fwd")
+
+
+def dropout_bwd(batch, length, mask, dy, dx):
+    check(lib().tdh_dropout_bwd(batch, length, _p(mask), _p(dy), _p(dx)), "tdh_dropout_bwd")
+
+
+class Mt19937:
+    """The reference's random generator (tiny_dnn/util/random.h:19-37): one std::mt19937, seed 1
+    unless set_random_seed is called. Draws 32-bit words like std::mt19937 does."""
+
+    def __init__(self, seed=1):
+        self._rs = np.random.RandomState()
+        mt = np.empty(624, dtype=np.uint32)
+        mt[0] = seed
+        for i in range(1, 624):
+            mt[i] = (1812433253 * (int(mt[i - 1]) ^ (int(mt[i - 1]) >> 30)) + i) & 0xFFFFFFFF
+        self._rs.set_state(("MT19937", mt, 624))
+
+    def words(self, n):
+        return self._rs.randint(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32)
+
+
+def dropout_mask(rng, rate, batch, length):
+    """mask[s][i] = bernoulli(rate) (tiny_dnn/util/random.h:67-69, dropout_layer.h:99-102): one draw
+    of uniform_real_distribution<float>(0,1) per element, sample after sample; 1 where u <= rate."""
+    u = rng.words(batch * length).astype(np.float32) / np.float32(4294967296.0)
+    u = np.minimum(u, np.nextafter(np.float32(1), np.float32(0)))
+    return (u <= np.float32(rate)).astype(np.uint8).reshape(batch, length)
+
+
 def loss_grad(kind, batch, length, y, t, dy):
     check(lib().tdh_loss_grad(LOSS[kind], batch, length, _p(y), _p(t), _p(dy)), "tdh_loss_grad")
 

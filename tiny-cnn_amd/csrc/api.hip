@@ -526,6 +526,54 @@ int tdh_act_bwd_p(int kind, const float *p, int batch, int len, const float *x, 
   return launch_act_bwd(kind, p ? p : def, batch, len, x, y, dy, dx);
 }
 
+int tdh_batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,
+                      float *mean, float *variance, float *stddev, float *y) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(channels >= 0 && spatial >= 0 && batch >= 0, "tdh_batchnorm_fwd: negative size");
+  if (channels == 0 || spatial == 0 || batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && y && mean && variance && stddev, "tdh_batchnorm_fwd: null tensor");
+  TDH_CHECK_ARG(static_cast<long>(batch) * channels * spatial < (1L << 31), "tdh_batchnorm_fwd: tensor too large");
+  TDH_TRY(ws_begin(batchnorm_workspace_bytes(channels, batch)));
+  return batchnorm_fwd(channels, spatial, batch, eps, train, x, mean, variance, stddev, y);
+}
+
+int tdh_batchnorm_bwd(int channels, int spatial, int batch, const float *y, const float *dy,
+                      const float *stddev, float *dx) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(channels >= 0 && spatial >= 0 && batch >= 0, "tdh_batchnorm_bwd: negative size");
+  if (channels == 0 || spatial == 0 || batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(y && dy && stddev && dx, "tdh_batchnorm_bwd: null tensor");
+  TDH_CHECK_ARG(static_cast<long>(batch) * channels * spatial < (1L << 31), "tdh_batchnorm_bwd: tensor too large");
+  TDH_TRY(ws_begin(batchnorm_workspace_bytes(channels, batch)));
+  return batchnorm_bwd(channels, spatial, batch, y, dy, stddev, dx);
+}
+
+int tdh_batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
+                                const float *var_cur, float *mean, float *variance) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(channels >= 0, "tdh_batchnorm_update_moving: negative size");
+  if (channels == 0) return TDH_OK;
+  TDH_CHECK_ARG(mean_cur && var_cur && mean && variance, "tdh_batchnorm_update_moving: null tensor");
+  return batchnorm_update_moving(channels, momentum, mean_cur, var_cur, mean, variance);
+}
+
+int tdh_dropout_fwd(int batch, int len, int train, float scale, const uint8_t *mask, const float *x,
+                    float *y) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_dropout_fwd: negative size");
+  if (batch == 0 || len == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && y && (mask || !train), "tdh_dropout_fwd: null tensor");
+  return dropout_fwd(static_cast<size_t>(batch) * len, train, scale, mask, x, y);
+}
+
+int tdh_dropout_bwd(int batch, int len, const uint8_t *mask, const float *dy, float *dx) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(batch >= 0 && len >= 0, "tdh_dropout_bwd: negative size");
+  if (batch == 0 || len == 0) return TDH_OK;
+  TDH_CHECK_ARG(mask && dy && dx, "tdh_dropout_bwd: null tensor");
+  return dropout_bwd(static_cast<size_t>(batch) * len, mask, dy, dx);
+}
+
 int tdh_act_fwd(int kind, int batch, int len, const float *x, float *y) {
   return tdh_act_fwd_p(kind, nullptr, batch, len, x, y);
 }

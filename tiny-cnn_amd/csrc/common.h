@@ -152,6 +152,16 @@ bool profiling_active();
 // deterministic reductions: out[r] (+)= sum over `cols` contiguous values of row r,
 // rows laid out as [outer][rows][cols] and summed over outer in order
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate);
+// norm.hip
+size_t batchnorm_workspace_bytes(int channels, int batch);
+int batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,
+                  float *mean, float *variance, float *stddev, float *y);
+int batchnorm_bwd(int channels, int spatial, int batch, const float *y, const float *dy,
+                  const float *stddev, float *dx);
+int batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
+                            const float *var_cur, float *mean, float *var);
+int dropout_fwd(size_t total, int train, float scale, const uint8_t *mask, const float *x, float *y);
+int dropout_bwd(size_t total, const uint8_t *mask, const float *dy, float *dx);
 size_t rowsum_workspace_bytes(int outer, int rows, int cols);
 // out[c] (+)= sum_s src[s*cols + c]
 int launch_colsum(const float *src, int rows, int cols, float *out, int accumulate);
