@@ -335,6 +335,78 @@ static void activations_vs_oracle() {
   EXPECT(elu_layer().layer_type() == "elu-activation");
 }
 
+// batch_normalization_layer / dropout_layer: forward_propagation / back_propagation on host
+// tensors against the oracle; the dropout mask must be the one the reference's generator draws
+static void norm_layers_vs_oracle() {
+  std::puts("batch-norm / dropout layers vs oracle");
+  const size_t c = 6, sp = 35, n = 9, len = c * sp;
+  tensor_t x = random_tensor(n, len, 71), dy = random_tensor(n, len, 72), y, dx;
+  for (auto &r : x) for (auto &v : r) v = 2.f * v + 0.5f;
+  batch_normalization_layer bn(sp, c);
+  std::vector<tensor_t *> in{&x}, out{&y}, og{&dy}, ig{&dx};
+  bn.update_immidiately(true);
+  bn.forward_propagation(in, out);
+  bn.back_propagation(in, out, og, ig);
+  std::vector<float> fx = flat(x), fdy = flat(dy), wy(n * len), wdx(n * len);
+  vec_t mean(c), var(c), sd(c);
+  EXPECT(tdo_batchnorm_fwd(c, sp, n, 1e-5f, 1, fx.data(), mean.data(), var.data(), sd.data(), wy.data()) == 0);
+  EXPECT(tdo_batchnorm_bwd(c, sp, n, wy.data(), fdy.data(), sd.data(), wdx.data()) == 0);
+  expect_near(flat(y).data(), wy.data(), wy.size(), 1e-4f, "batch-norm y");
+  expect_near(flat(dx).data(), wdx.data(), wdx.size(), 1e-4f, "batch-norm dx");
+  expect_near(bn.mean(), mean, 1e-5f, "batch-norm mean");
+  expect_near(bn.variance(), var, 1e-5f, "batch-norm variance");
+  // test phase reads the moving averages; post_update blends them
+  vec_t m0 = random_vec(c, 73), v0 = random_vec(c, 74, 0.5f, 2.f);
+  batch_normalization_layer bt(sp, c, 1e-5f, 0.9f, net_phase::test);
+  bt.set_mean(m0);
+  bt.set_variance(v0);
+  bt.forward_propagation(in, out);
+  vec_t tm = m0, tv = v0;
+  EXPECT(tdo_batchnorm_fwd(c, sp, n, 1e-5f, 0, fx.data(), tm.data(), tv.data(), sd.data(), wy.data()) == 0);
+  expect_near(flat(y).data(), wy.data(), wy.size(), 1e-4f, "batch-norm test phase");
+  bt.set_context(net_phase::train);
+  bt.forward_propagation(in, out);
+  bt.post_update();
+  tdo_batchnorm_update_moving(c, 0.9f, mean.data(), var.data(), tm.data(), tv.data());
+  expect_near(bt.mean(), tm, 1e-5f, "batch-norm moving mean");
+  expect_near(bt.variance(), tv, 1e-5f, "batch-norm moving variance");
+  EXPECT(bn.layer_type() == "batch-norm" && bn.epsilon() == 1e-5f && bt.momentum() == 0.9f);
+
+  const size_t dl_len = 333;
+  tensor_t dxin = random_tensor(n, dl_len, 75), ddy = random_tensor(n, dl_len, 76), dyo, ddx;
+  dropout_layer dl(dl_len, 0.3f);
+  set_random_seed(7);
+  std::vector<tensor_t *> din{&dxin}, dout{&dyo}, dog{&ddy}, dig{&ddx};
+  dl.forward_propagation(din, dout);
+  dl.back_propagation(din, dout, dog, dig);
+  std::vector<unsigned int> st(625);
+  std::vector<unsigned char> mask(n * dl_len);
+  tdo_mt_seed(st.data(), 7);
+  tdo_dropout_mask(st.data(), 0.3f, mask.size(), mask.data());
+  bool same_mask = true;
+  for (size_t s = 0; s < n; ++s)
+    same_mask = same_mask && std::memcmp(dl.get_mask(s).data(), mask.data() + s * dl_len, dl_len) == 0;
+  EXPECT(same_mask);
+  std::vector<float> wdy(n * dl_len), wddx(n * dl_len), fdx = flat(dxin), fddy = flat(ddy);
+  const float scale = 1.f / (1.f - 0.3f);
+  EXPECT(tdo_dropout_fwd(n, dl_len, 1, scale, mask.data(), fdx.data(), wdy.data()) == 0);
+  EXPECT(tdo_dropout_bwd(n, dl_len, mask.data(), fddy.data(), wddx.data()) == 0);
+  EXPECT(flat(dyo) == wdy);
+  EXPECT(flat(ddx) == wddx);
+  dl.set_context(net_phase::test);
+  dl.forward_propagation(din, dout);
+  EXPECT(flat(dyo) == fdx);
+  dl.set_dropout_rate(0.5f);
+  EXPECT(dl.dropout_rate() == 0.5f && dl.layer_type() == "dropout");
+  bool refused = false;
+  try {
+    network<sequential> net;
+    net << fully_connected_layer(4, 4) << dropout_layer(4, 0.5f);
+    net.in_data_size();
+  } catch (const nn_error &) { refused = true; }
+  EXPECT(refused);
+}
+
 // -------------------------------------------------- network<sequential>::fit
 template <typename Opt>
 static void net_fit_vs_oracle(const char *name, int opt_kind) {
@@ -477,6 +549,7 @@ int main() {
     conv_ops_vs_oracle();
     fc_pool_ops_vs_oracle();
     activations_vs_oracle();
+    norm_layers_vs_oracle();
     weight_files();
     net_fit_vs_oracle<gradient_descent>("gradient_descent", TDO_OPT_SGD);
     net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM);

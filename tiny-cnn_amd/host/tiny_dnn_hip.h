@@ -29,6 +29,7 @@
 #pragma once
 
 #include <algorithm>
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
@@ -40,6 +41,7 @@
 #include <limits>
 #include <map>
 #include <ostream>
+#include <random>
 #include <memory>
 #include <string>
 #include <vector>
@@ -962,6 +964,242 @@ struct softplus_layer : activation_layer {
 struct softsign_layer : activation_layer { softsign_layer() : activation_layer(TDH_ACT_SOFTSIGN, "softsign-activation") {} };
 struct asinh_layer : activation_layer { asinh_layer() : activation_layer(TDH_ACT_ASINH, "asinh-activation") {} };
 struct tanh_p1m2_layer : activation_layer { tanh_p1m2_layer() : activation_layer(TDH_ACT_TANH_P1M2, "tanh-scaled-activation") {} };
+
+// ---- the reference's random source (tiny_dnn/util/random.h:19-69): one std::mt19937 for the
+// whole process, seeded with 1 until set_random_seed is called; bernoulli(p) is one draw of
+// uniform_real_distribution<float_t>(0, 1) compared with p ----
+class random_generator {
+ public:
+  static random_generator &get_instance() {
+    static random_generator g;
+    return g;
+  }
+  std::mt19937 &operator()() { return engine_; }
+  void set_seed(unsigned int seed) { engine_.seed(seed); }
+
+ private:
+  random_generator() : engine_(1) {}
+  std::mt19937 engine_;
+};
+inline void set_random_seed(unsigned int seed) { random_generator::get_instance().set_seed(seed); }
+inline bool bernoulli(float_t p) {
+  std::uniform_real_distribution<float_t> unit(float_t(0), float_t(1));
+  return unit(random_generator::get_instance()()) <= p;
+}
+
+enum class net_phase { train, test };  // tiny_dnn/util/util.h:71
+
+// The two layers below run on the device through their own operators. The device-resident
+// train step of network<sequential> does not include them (describe() says so); they are used
+// the way the reference's tests use a single layer: forward_propagation / back_propagation on
+// host tensors.
+namespace detail {
+struct norm_buffers {
+  device_tensor x, y, dy, dx, mean, var, stddev, mean_cur, var_cur;
+  void *mask     = nullptr;
+  size_t mask_cap = 0;
+  ~norm_buffers() {
+    if (mask) tdh_free(mask);
+  }
+  void *mask_upload(const std::vector<uint8_t> &m) {
+    if (m.size() > mask_cap) {
+      if (mask) check(tdh_free(mask));
+      mask = nullptr;
+      check(tdh_malloc(&mask, m.size()));
+      mask_cap = m.size();
+    }
+    if (!m.empty()) check(tdh_memcpy_h2d(mask, m.data(), m.size()));
+    return mask;
+  }
+};
+inline void download_vec(vec_t &v, const float *dev, size_t n) {
+  v.resize(n);
+  if (n) check(tdh_memcpy_d2h(v.data(), dev, n * sizeof(float)));
+}
+}  // namespace detail
+
+// tiny_dnn/layers/batch_normalization_layer.h:54-72 (the constructor that takes the shape)
+class batch_normalization_layer : public layer {
+ public:
+  batch_normalization_layer(size_t in_spatial_size, size_t in_channels, float_t epsilon = 1e-5,
+                            float_t momentum = 0.999, net_phase phase = net_phase::train)
+    : channels_(in_channels), spatial_(in_spatial_size), phase_(phase), momentum_(momentum),
+      eps_(epsilon), update_immidiately_(false), mean_(in_channels), variance_(in_channels),
+      mean_current_(in_channels), variance_current_(in_channels), stddev_(in_channels),
+      buf_(new detail::norm_buffers()) {}
+
+  std::string layer_type() const override { return "batch-norm"; }
+  layer_desc describe(const shape3d &) const override {
+    throw nn_error("batch_normalization_layer is not part of the device-resident train step");
+  }
+  std::vector<shape3d> in_shape() const { return {shape3d(spatial_, 1, channels_)}; }
+  std::vector<shape3d> out_shape() const { return {shape3d(spatial_, 1, channels_)}; }
+
+  // batch_normalization_layer.h:127-169
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+    detail::ensure_init();
+    const tensor_t &in = *in_data[0];
+    tensor_t &out      = *out_data[0];
+    const size_t n = in.size(), len = channels_ * spatial_;
+    const bool train = phase_ == net_phase::train;
+    detail::norm_buffers &b = *buf_;
+    float *mean = train ? b.mean_cur.resize(channels_) : b.mean.upload(mean_, channels_);
+    float *var  = train ? b.var_cur.resize(channels_) : b.var.upload(variance_, channels_);
+    b.y.resize(n * len);
+    detail::check(tdh_batchnorm_fwd(static_cast<int>(channels_), static_cast<int>(spatial_),
+                                    static_cast<int>(n), eps_, train ? 1 : 0, b.x.upload(in, n, len),
+                                    mean, var, b.stddev.resize(channels_), b.y.get()));
+    out.resize(n);
+    b.y.download(out, n, len);
+    detail::download_vec(stddev_, b.stddev.get(), channels_);
+    if (train) {
+      detail::download_vec(mean_current_, mean, channels_);
+      detail::download_vec(variance_current_, var, channels_);
+      if (update_immidiately_) {
+        mean_     = mean_current_;
+        variance_ = variance_current_;
+      }
+    }
+  }
+
+  // batch_normalization_layer.h:87-125
+  void back_propagation(const std::vector<tensor_t *> &, const std::vector<tensor_t *> &out_data,
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+    detail::ensure_init();
+    const tensor_t &curr_out = *out_data[0];
+    tensor_t &prev_delta     = *in_grad[0];
+    const size_t n = curr_out.size(), len = channels_ * spatial_;
+    detail::norm_buffers &b = *buf_;
+    b.dx.resize(n * len);
+    detail::check(tdh_batchnorm_bwd(static_cast<int>(channels_), static_cast<int>(spatial_),
+                                    static_cast<int>(n), b.y.upload(curr_out, n, len),
+                                    b.dy.upload(*out_grad[0], n, len),
+                                    b.stddev.upload(stddev_, channels_), b.dx.get()));
+    prev_delta.resize(n);
+    b.dx.download(prev_delta, n, len);
+  }
+
+  void set_context(net_phase ctx) { phase_ = ctx; }
+  // batch_normalization_layer.h:171-177
+  void post_update() {
+    detail::ensure_init();
+    detail::norm_buffers &b = *buf_;
+    detail::check(tdh_batchnorm_update_moving(
+      static_cast<int>(channels_), momentum_, b.mean_cur.upload(mean_current_, channels_),
+      b.var_cur.upload(variance_current_, channels_), b.mean.upload(mean_, channels_),
+      b.var.upload(variance_, channels_)));
+    detail::download_vec(mean_, b.mean.get(), channels_);
+    detail::download_vec(variance_, b.var.get(), channels_);
+  }
+  // batch_normalization_layer.h:179-202: the moving averages follow the (absent) weights
+  void save(std::ostream &os, const int precision = std::numeric_limits<float_t>::digits10 + 2) const {
+    os << std::setprecision(precision);
+    for (auto m : mean_) os << m << " ";
+    for (auto v : variance_) os << v << " ";
+  }
+  void load(std::istream &is) {
+    for (auto &m : mean_) is >> m;
+    for (auto &v : variance_) is >> v;
+  }
+  void update_immidiately(bool update) { update_immidiately_ = update; }
+  void set_stddev(const vec_t &stddev) { stddev_ = stddev; }
+  void set_mean(const vec_t &mean) { mean_ = mean; }
+  void set_variance(const vec_t &variance) {
+    variance_ = variance;
+    for (size_t i = 0; i < channels_; ++i) stddev_[i] = std::sqrt(variance_[i] + eps_);
+  }
+  const vec_t &mean() const { return mean_; }
+  const vec_t &variance() const { return variance_; }
+  float_t epsilon() const { return eps_; }
+  float_t momentum() const { return momentum_; }
+
+ private:
+  size_t channels_, spatial_;
+  net_phase phase_;
+  float_t momentum_, eps_;
+  bool update_immidiately_;
+  vec_t mean_, variance_, mean_current_, variance_current_, stddev_;
+  std::shared_ptr<detail::norm_buffers> buf_;
+};
+
+// tiny_dnn/layers/dropout_layer.h:22-147
+class dropout_layer : public layer {
+ public:
+  dropout_layer(size_t in_dim, float_t dropout_rate, net_phase phase = net_phase::train)
+    : phase_(phase), dropout_rate_(dropout_rate), scale_(float_t(1) / (float_t(1) - dropout_rate)),
+      in_size_(in_dim), mask_(1, std::vector<uint8_t>(in_dim)), buf_(new detail::norm_buffers()) {}
+
+  std::string layer_type() const override { return "dropout"; }
+  layer_desc describe(const shape3d &) const override {
+    throw nn_error("dropout_layer is not part of the device-resident train step");
+  }
+  std::vector<shape3d> in_shape() const { return {shape3d(in_size_, 1, 1)}; }
+  std::vector<shape3d> out_shape() const { return {shape3d(in_size_, 1, 1)}; }
+  void set_dropout_rate(float_t rate) {
+    dropout_rate_ = rate;
+    scale_        = float_t(1) / (float_t(1) - dropout_rate_);
+  }
+  float_t dropout_rate() const { return dropout_rate_; }
+
+  // dropout_layer.h:84-117: in the train phase every element of every sample draws its own
+  // bernoulli(rate), sample after sample; the products run on the device
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+    detail::ensure_init();
+    const tensor_t &in = *in_data[0];
+    tensor_t &out      = *out_data[0];
+    const size_t n = in.size();
+    if (mask_.size() < n) mask_.resize(n, mask_[0]);
+    const bool train = phase_ == net_phase::train;
+    detail::norm_buffers &b = *buf_;
+    void *mask = nullptr;
+    if (train) {
+      flat_.resize(n * in_size_);
+      for (size_t s = 0; s < n; ++s) {
+        for (size_t i = 0; i < in_size_; ++i) mask_[s][i] = bernoulli(dropout_rate_);
+        std::memcpy(flat_.data() + s * in_size_, mask_[s].data(), in_size_);
+      }
+      mask = b.mask_upload(flat_);
+    }
+    b.y.resize(n * in_size_);
+    detail::check(tdh_dropout_fwd(static_cast<int>(n), static_cast<int>(in_size_), train ? 1 : 0, scale_,
+                                  static_cast<const uint8_t *>(mask), b.x.upload(in, n, in_size_), b.y.get()));
+    out.resize(n);
+    b.y.download(out, n, in_size_);
+  }
+
+  // dropout_layer.h:62-82
+  void back_propagation(const std::vector<tensor_t *> &, const std::vector<tensor_t *> &,
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+    detail::ensure_init();
+    const tensor_t &curr_delta = *out_grad[0];
+    tensor_t &prev_delta       = *in_grad[0];
+    const size_t n = curr_delta.size();
+    if (n > mask_.size()) throw nn_error("dropout_layer: backward over more samples than forward");
+    detail::norm_buffers &b = *buf_;
+    flat_.resize(n * in_size_);
+    for (size_t s = 0; s < n; ++s) std::memcpy(flat_.data() + s * in_size_, mask_[s].data(), in_size_);
+    b.dx.resize(n * in_size_);
+    detail::check(tdh_dropout_bwd(static_cast<int>(n), static_cast<int>(in_size_),
+                                  static_cast<const uint8_t *>(b.mask_upload(flat_)),
+                                  b.dy.upload(curr_delta, n, in_size_), b.dx.get()));
+    prev_delta.resize(n);
+    b.dx.download(prev_delta, n, in_size_);
+  }
+
+  void set_context(net_phase ctx) { phase_ = ctx; }
+  const std::vector<uint8_t> &get_mask(size_t sample_index) const { return mask_[sample_index]; }
+  void clear_mask() {
+    for (auto &sample : mask_) std::fill(sample.begin(), sample.end(), 0);
+  }
+
+ private:
+  net_phase phase_;
+  float_t dropout_rate_, scale_;
+  size_t in_size_;
+  std::vector<std::vector<uint8_t>> mask_;
+  std::vector<uint8_t> flat_;
+  std::shared_ptr<detail::norm_buffers> buf_;
+};
 
 namespace detail {
 // RAII handle of a tdh_feeder plus the flattening of vector-of-vectors batches
