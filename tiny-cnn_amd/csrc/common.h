@@ -209,6 +209,7 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
 // workspace bytes the op may ask for (so a net can reserve it before graph capture)
 size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
 size_t fc_workspace_bytes(int in, int out, int batch);
+bool fc_bwd_fuses(int in, int out, int batch);
 
 // pool.hip
 // act_out: also writes act(y) there (tanh / relu / sigmoid), the activation layer behind the pool

@@ -21,19 +21,24 @@ namespace {
 constexpr int SFC_TM = 16, SFC_TN = 64, SFC_KC = 64, SFC_NT = 256;
 constexpr int SFC_NA = SFC_TM * SFC_KC / SFC_NT, SFC_NB = SFC_TN * SFC_KC / SFC_NT;
 
+struct SfcSmem {
+  __attribute__((aligned(16))) float As[SFC_KC][SFC_TM + 4];
+  float Bs[SFC_KC][SFC_TN + 1];
+};
+
+// One 16 x 64 tile (bx, by) of C = A * B with the epilogue applied. The next panel's loads are
+// issued before the current panel is multiplied.
 template <class Epi>
-__global__ void __launch_bounds__(SFC_NT)
-small_fc_gemm_kernel(const StridedOperand a, const StridedOperand b, const Epi epi, const int M,
-                     const int N, const int K) {
-  __shared__ __attribute__((aligned(16))) float As[SFC_KC][SFC_TM + 4];
-  __shared__ float Bs[SFC_KC][SFC_TN + 1];
+__device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const StridedOperand &b,
+                                              const Epi &epi, const int M, const int N, const int K,
+                                              const int bx, const int by, SfcSmem &sm) {
   const int tid = threadIdx.x, tn = tid & 63, tmg = tid >> 6;
-  const int m0 = blockIdx.y * SFC_TM, n0 = blockIdx.x * SFC_TN;
+  const int m0 = by * SFC_TM, n0 = bx * SFC_TN;
   // staging coordinates: consecutive threads walk the operand's contiguous direction
   const bool a_k_fast = a.s_k == 1, b_k_fast = b.s_k == 1;
   float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int k0 = 0; k0 < K; k0 += SFC_KC) {
-    float ra[SFC_NA], rb[SFC_NB];
+  float ra[SFC_NA], rb[SFC_NB];
+  auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < SFC_NA; ++i) {
       const int e = tid + SFC_NT * i;
@@ -46,22 +51,26 @@ small_fc_gemm_kernel(const StridedOperand a, const StridedOperand b, const Epi e
       const int n = b_k_fast ? e / SFC_KC : e % SFC_TN, k = b_k_fast ? e % SFC_KC : e / SFC_TN;
       rb[i] = (n0 + n < N && k0 + k < K) ? b.p[(n0 + n) * b.s_mn + (k0 + k) * b.s_k] : 0.0f;
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += SFC_KC) {
     if (k0 > 0) __syncthreads();  // the previous panel has been consumed
 #pragma unroll
     for (int i = 0; i < SFC_NA; ++i) {
       const int e = tid + SFC_NT * i;
-      As[a_k_fast ? e % SFC_KC : e / SFC_TM][a_k_fast ? e / SFC_KC : e % SFC_TM] = ra[i];
+      sm.As[a_k_fast ? e % SFC_KC : e / SFC_TM][a_k_fast ? e / SFC_KC : e % SFC_TM] = ra[i];
     }
 #pragma unroll
     for (int i = 0; i < SFC_NB; ++i) {
       const int e = tid + SFC_NT * i;
-      Bs[b_k_fast ? e % SFC_KC : e / SFC_TN][b_k_fast ? e / SFC_KC : e % SFC_TN] = rb[i];
+      sm.Bs[b_k_fast ? e % SFC_KC : e / SFC_TN][b_k_fast ? e / SFC_KC : e % SFC_TN] = rb[i];
     }
     __syncthreads();
+    if (k0 + SFC_KC < K) fetch(k0 + SFC_KC);
 #pragma unroll 8
     for (int k = 0; k < SFC_KC; ++k) {
-      const float4 av = *reinterpret_cast<const float4 *>(&As[k][4 * tmg]);
-      const float bv  = Bs[k][tn];
+      const float4 av = *reinterpret_cast<const float4 *>(&sm.As[k][4 * tmg]);
+      const float bv  = sm.Bs[k][tn];
       acc[0] += av.x * bv;
       acc[1] += av.y * bv;
       acc[2] += av.z * bv;
@@ -75,6 +84,54 @@ small_fc_gemm_kernel(const StridedOperand a, const StridedOperand b, const Epi e
     for (int i = 0; i < 4; ++i) {
       const int m = m0 + 4 * tmg + i;
       if (m < M) epi.store(m, c, acc[i]);
+    }
+  }
+}
+
+template <class Epi>
+__global__ void __launch_bounds__(SFC_NT)
+small_fc_gemm_kernel(const StridedOperand a, const StridedOperand b, const Epi epi, const int M,
+                     const int N, const int K) {
+  __shared__ SfcSmem sm;
+  small_fc_tile(a, b, epi, M, N, K, blockIdx.x, blockIdx.y, sm);
+}
+
+// The whole backward pass of a small fully-connected layer in one launch: the first nx
+// workgroups take the tiles of dX, the next nw those of dW, the rest 32 columns each of the bias
+// gradient (rows g, g+8, ... per 32-lane group, group sums added in order, as the stand-alone
+// column sum does). The three products only share their inputs, and none of them fills the chip.
+struct FcBwdFused {
+  StridedOperand xa, xb, wa, wb;
+  EpiRowMajor xepi, wepi;
+  int xM, xN, xK, x_tiles_n, nx;
+  int wM, wN, wK, w_tiles_n, nw;
+  const float *dy;
+  float *db;
+  int batch, out, db_accumulate;
+};
+
+__global__ void __launch_bounds__(SFC_NT) fc_bwd_fused_kernel(const FcBwdFused f) {
+  __shared__ SfcSmem sm;
+  const int b = blockIdx.x;
+  if (b < f.nx) {
+    small_fc_tile(f.xa, f.xb, f.xepi, f.xM, f.xN, f.xK, b % f.x_tiles_n, b / f.x_tiles_n, sm);
+  } else if (b < f.nx + f.nw) {
+    const int t = b - f.nx;
+    small_fc_tile(f.wa, f.wb, f.wepi, f.wM, f.wN, f.wK, t % f.w_tiles_n, t / f.w_tiles_n, sm);
+  } else {
+    float(*part)[32] = reinterpret_cast<float(*)[32]>(&sm.Bs[0][0]);
+    const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int c  = (b - f.nx - f.nw) * 32 + cl;
+    float s = 0.0f;
+    if (c < f.out)
+      for (int r = g; r < f.batch; r += 8) s += f.dy[static_cast<size_t>(r) * f.out + c];
+    part[g][cl] = s;
+    __syncthreads();
+    if (g == 0 && c < f.out) {
+      float t = part[0][cl];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) t += part[i][cl];
+      f.db[c] = f.db_accumulate ? f.db[c] + t : t;
     }
   }
 }
@@ -96,6 +153,11 @@ int launch_small_fc(const StridedOperand &a, const StridedOperand &b, const Epi 
 
 }  // namespace
 
+// dX, dW and db of this layer leave one launch (when all three are asked for)
+bool fc_bwd_fuses(int in, int out, int batch) {
+  return small_fc_applies(batch, in, out) && small_fc_applies(in, out, batch);
+}
+
 size_t fc_workspace_bytes(int in, int out, int batch) {
   return gemm_workspace_bytes(batch, out, in, true) + gemm_workspace_bytes(batch, in, out, true) +
          gemm_workspace_bytes(in, out, batch, true);
@@ -113,6 +175,28 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
 
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act) {
+  if (dx && dw && fc_bwd_fuses(in, out, batch)) {
+    FcBwdFused f;
+    f.xa = StridedOperand{dy, out, 1, batch};
+    f.xb = StridedOperand{w, out, 1, in};
+    f.xepi = EpiRowMajor{dx, in, nullptr, dx_act, 0};
+    f.xM = batch; f.xN = in; f.xK = out;
+    f.x_tiles_n = ceil_div(in, SFC_TN);
+    f.nx = f.x_tiles_n * ceil_div(batch, SFC_TM);
+    f.wa = StridedOperand{x, 1, in, in};
+    f.wb = StridedOperand{dy, 1, out, out};
+    f.wepi = EpiRowMajor{dw, out, nullptr, ActGrad(), accumulate};
+    f.wM = in; f.wN = out; f.wK = batch;
+    f.w_tiles_n = ceil_div(out, SFC_TN);
+    f.nw = f.w_tiles_n * ceil_div(in, SFC_TM);
+    const bool bias = db && has_bias;
+    f.dy = dy; f.db = db; f.batch = batch; f.out = out; f.db_accumulate = accumulate;
+    ProfScope prof("fc_bwd_small", 4.0 * batch * in * out, WORK_FLOP);
+    hipLaunchKernelGGL(fc_bwd_fused_kernel, dim3(f.nx + f.nw + (bias ? ceil_div(out, 32) : 0)),
+                       dim3(SFC_NT), 0, ctx().stream, f);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   if (dx) {
     StridedOperand A{dy, out, 1, batch};  // dY[s][k]
     StridedOperand B{w, out, 1, in};      // W[n][k], k contiguous
