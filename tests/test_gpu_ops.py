@@ -201,7 +201,10 @@ def test_fc_reference_kats_and_outputs(T, kats, layer_grads):
 
 POOL = [(4, 4, 1, 2, 2, 2, 2, 0, 0), (7, 7, 2, 2, 2, 2, 2, 0, 1), (4, 4, 1, 2, 2, 1, 1, 1, 0),
         (9, 8, 3, 3, 3, 2, 2, 0, 0), (6, 6, 2, 2, 2, 3, 3, 0, 0), (32, 32, 32, 2, 2, 2, 2, 0, 0),
-        (4, 4, 1, 2, 1, 2, 1, 0, 0), (4, 4, 1, 1, 2, 1, 2, 0, 0), (13, 9, 5, 3, 2, 2, 1, 1, 1)]
+        (4, 4, 1, 2, 1, 2, 1, 0, 0), (4, 4, 1, 1, 2, 1, 2, 0, 0), (13, 9, 5, 3, 2, 2, 1, 1, 1),
+        # 2x2 stride-2 windows over rows of whole 16-byte words (two outputs a thread), and not
+        (8, 6, 3, 2, 2, 2, 2, 0, 0), (12, 4, 5, 2, 2, 2, 2, 0, 0), (6, 6, 2, 2, 2, 2, 2, 0, 0),
+        (16, 16, 7, 2, 2, 2, 2, 1, 0)]
 
 
 @pytest.mark.parametrize("cfg", POOL)

@@ -215,9 +215,10 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
 #pragma unroll
           for (int j = 0; j < TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
-        // keep the steps apart: LDS reads moved ahead over many steps cost more registers than
-        // two resident workgroups have, and the other workgroup covers the read latency anyway
-        __builtin_amdgcn_sched_barrier(0);
+        // Tiles of several accumulator blocks keep the steps apart: LDS reads moved ahead over
+        // many steps cost more registers than two resident workgroups have. A single-block tile
+        // has the registers, and often the CU to itself, so there the reads may run ahead.
+        if (TM * TN > 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
   };

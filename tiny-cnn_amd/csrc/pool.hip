@@ -60,6 +60,80 @@ maxpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
   if (act_out) act_out[o] = act_apply(act_kind, best);  // the activation layer that follows
 }
 
+// The same for the common geometry: 2x2 windows, stride 2, width a multiple of 4 and even
+// height, 16-byte aligned tensors. A thread owns two neighbouring outputs, i.e. two input rows
+// of four floats, read as 16-byte words; the window scan order (row by row, left to right) and
+// the strict '>' are those of the general kernel.
+__global__ void __launch_bounds__(PT)
+maxpool2x2_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
+                      int32_t *__restrict__ argmax, const int pairs, const int W, const int OW2,
+                      const FastDiv div_ow2, const int rows_per_sample, float *__restrict__ act_out,
+                      const int act_kind) {
+  const int t = blockIdx.x * PT + threadIdx.x;  // pair index: (plane*OH + oy)*OW2 + ox2
+  if (t >= pairs) return;
+  uint32_t row, ox2;
+  div_ow2.divmod(t, row, ox2);                   // row = plane*OH + oy
+  // input rows 2*row and 2*row+1 of the [planes*H][W] image, columns 4*ox2 .. 4*ox2+3
+  const float *p   = x + (static_cast<size_t>(2 * row) * W + 4 * ox2);
+  const float4 r0  = *reinterpret_cast<const float4 *>(p);
+  const float4 r1  = *reinterpret_cast<const float4 *>(p + W);
+  const float v[2][4] = {{r0.x, r0.y, r1.x, r1.y}, {r0.z, r0.w, r1.z, r1.w}};
+  float best[2];
+  int idx[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    best[k] = -FLT_MAX;
+    int sel = -1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (v[k][j] > best[k]) {
+        best[k] = v[k][j];
+        sel     = j;
+      }
+    idx[k] = sel;
+  }
+  const size_t o = static_cast<size_t>(row) * (2 * OW2) + 2 * ox2;
+  *reinterpret_cast<float2 *>(y + o) = make_float2(best[0], best[1]);
+  if (act_out)
+    *reinterpret_cast<float2 *>(act_out + o) =
+      make_float2(act_apply(act_kind, best[0]), act_apply(act_kind, best[1]));
+  if (argmax) {
+    // flat CHW index inside the sample (rows_per_sample = C*H input rows a sample)
+    int2 a;
+    const int base = (static_cast<int>(2 * row) % rows_per_sample) * W + 4 * static_cast<int>(ox2);
+    a.x = idx[0] < 0 ? 0 : base + (idx[0] >> 1) * W + (idx[0] & 1);
+    a.y = idx[1] < 0 ? 0 : base + 2 + (idx[1] >> 1) * W + (idx[1] & 1);
+    *reinterpret_cast<int2 *>(argmax + o) = a;
+  }
+}
+
+// dx rows 2*row, 2*row+1, columns 4*ox2..4*ox2+3 from two outputs and their argmax records
+__global__ void __launch_bounds__(PT)
+maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ argmax,
+                      float *__restrict__ dx, const int pairs, const int W, const int OW2,
+                      const FastDiv div_ow2, const int rows_per_sample) {
+  const int t = blockIdx.x * PT + threadIdx.x;
+  if (t >= pairs) return;
+  uint32_t row, ox2;
+  div_ow2.divmod(t, row, ox2);
+  const size_t o  = static_cast<size_t>(row) * (2 * OW2) + 2 * ox2;
+  const float2 g  = *reinterpret_cast<const float2 *>(dy + o);
+  const int2 a    = *reinterpret_cast<const int2 *>(argmax + o);
+  const int base  = (static_cast<int>(2 * row) % rows_per_sample) * W + 4 * static_cast<int>(ox2);
+  float4 r0, r1;
+  r0.x = a.x == base ? g.x : 0.0f;
+  r0.y = a.x == base + 1 ? g.x : 0.0f;
+  r0.z = a.y == base + 2 ? g.y : 0.0f;
+  r0.w = a.y == base + 3 ? g.y : 0.0f;
+  r1.x = a.x == base + W ? g.x : 0.0f;
+  r1.y = a.x == base + W + 1 ? g.x : 0.0f;
+  r1.z = a.y == base + W + 2 ? g.y : 0.0f;
+  r1.w = a.y == base + W + 3 ? g.y : 0.0f;
+  float *p = dx + (static_cast<size_t>(2 * row) * W + 4 * ox2);
+  *reinterpret_cast<float4 *>(p)     = r0;
+  *reinterpret_cast<float4 *>(p + W) = r1;
+}
+
 // maxpool_grad_op_internal (maxpool_op_internal.h:42-57). in2out[i] is the LAST window, in
 // (c, oy, ox) creation order, that contains input i (max_pooling_layer.h:218), and 0 for
 // inputs no window contains (strides larger than the window).
@@ -185,6 +259,14 @@ avepool_bwd_param_reduce_kernel(const float *__restrict__ partial, const int bat
   if (db) db[c] = accumulate ? db[c] + mb : mb;
 }
 
+// 2x2 windows at stride 2 that tile the input exactly, rows of whole 16-byte words
+bool is_2x2_tiling(const PoolGeom &g) {
+  return g.pw == 2 && g.ph == 2 && g.sw == 2 && g.sh == 2 && g.W % 4 == 0 && g.H % 2 == 0 &&
+         g.OW * 2 == g.W && g.OH * 2 == g.H;
+}
+bool aligned8(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 }  // namespace
 
 int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax,
@@ -194,6 +276,14 @@ int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int
   if (total <= 0) return TDH_OK;
   ProfScope prof(act_out ? "maxpool_fwd_act" : "maxpool_fwd",
                  4.0 * batch * g.C * g.H * g.W + (act_out ? 12.0 : 8.0) * total, WORK_BYTE);
+  if (is_2x2_tiling(g) && aligned16(x) && aligned8(y) && aligned8(argmax) && aligned8(act_out) &&
+      total / 2 < (1L << 31)) {
+    const int pairs = static_cast<int>(total / 2);
+    hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, x,
+                       y, argmax, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, act_out, act_kind);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
                      y, argmax, static_cast<int>(total), g, act_out, act_kind);
   TDH_LAUNCH_CHECK();
@@ -206,6 +296,13 @@ int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_
   const long total = static_cast<long>(batch) * g.C * g.H * g.W;
   TDH_CHECK_ARG(g.OH > 0 && g.OW > 0, "maxpool backward: empty output");
   ProfScope prof("maxpool_bwd", 8.0 * batch * g.C * g.OH * g.OW + 4.0 * total, WORK_BYTE);
+  if (is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) && total / 8 < (1L << 31)) {
+    const int pairs = static_cast<int>(total / 8);
+    hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
+                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, dy,
                      argmax, dx, static_cast<int>(total), g);
   TDH_LAUNCH_CHECK();
