@@ -141,6 +141,12 @@ int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, fl
 struct OptTensor {
   float *g, *w, *s0, *s1;
   uint32_t n, first_block;
+  // A convolution's OIHW weight tensor whose filters the stride-1 kernels read in their own
+  // layout: the update also writes the new value into those copies (wp_fwd[t][ci][co],
+  // wp_dx[rs-1-t][co][ci]; unconnected pairs of the connection table as zero). NULL: none.
+  float *wp_fwd, *wp_dx;
+  const uint8_t *tbl;
+  uint32_t C, Kc, rs;
 };
 constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 4096;
 // dev_powers: NULL, or two device floats {b1_t, b2_t} that the kernel reads instead of the

@@ -368,6 +368,15 @@ int launch_opt(size_t n, const float *g, float *w, float *s0, float *s1, const O
   return TDH_OK;
 }
 
+// The packed copies of element e = (co*C + ci)*rs + t of a convolution's weight tensor
+__device__ __forceinline__ void opt_pack_store(const OptTensor &t, const uint32_t e, float v) {
+  const uint32_t tap = e % t.rs, pair = e / t.rs;
+  const uint32_t co = pair / t.C, ci = pair - co * t.C;
+  if (t.tbl && !t.tbl[ci * t.Kc + co]) v = 0.0f;
+  t.wp_fwd[(static_cast<size_t>(tap) * t.C + ci) * t.Kc + co] = v;
+  t.wp_dx[(static_cast<size_t>(t.rs - 1 - tap) * t.Kc + co) * t.C + ci] = v;
+}
+
 // Multi-tensor form: block b works on tensor j = the table entry whose block range holds b.
 template <int KIND, int NSTATE>
 __global__ void __launch_bounds__(EW_THREADS)
@@ -405,6 +414,12 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
     opt_one<KIND>(vg.z, vw.z, v0.z, v1.z, p);
     opt_one<KIND>(vg.w, vw.w, v0.w, v1.w, p);
     *reinterpret_cast<float4 *>(t.w + i) = vw;
+    if (t.wp_fwd) {
+      opt_pack_store(t, i, vw.x);
+      opt_pack_store(t, i + 1, vw.y);
+      opt_pack_store(t, i + 2, vw.z);
+      opt_pack_store(t, i + 3, vw.w);
+    }
     if (NSTATE >= 1) *reinterpret_cast<float4 *>(t.s0 + i) = v0;
     if (NSTATE >= 2) *reinterpret_cast<float4 *>(t.s1 + i) = v1;
     if (zero_grad) *reinterpret_cast<float4 *>(t.g + i) = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -415,6 +430,7 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
     if (NSTATE >= 2) b = t.s1[i];
     opt_one<KIND>(t.g[i], ww, a, b, p);
     t.w[i] = ww;
+    if (t.wp_fwd) opt_pack_store(t, i, ww);
     if (NSTATE >= 1) t.s0[i] = a;
     if (NSTATE >= 2) t.s1[i] = b;
     if (zero_grad) t.g[i] = 0.0f;

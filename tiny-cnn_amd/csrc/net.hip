@@ -21,13 +21,14 @@ struct tdh_net {
     bool grad_folded = false;  // activation whose backward runs in the next layer's dX epilogue
     // filters in the LDS-halo kernels' layout for forward / dX, packed on a side stream at the
     // start of a captured step (stride-1 conv layers of a TDH_NET_GRAPH net)
-    float *wp_fwd = nullptr, *wp_dx = nullptr;
+    float *wp_fwd = nullptr, *wp_dx = nullptr;  // kept current by the optimizer kernel
   };
   std::vector<Layer> layers;
   int max_batch  = 0;
   int flags      = 0;
   float *dx_in   = nullptr;  // gradient w.r.t. the network input
   tdh::OptTensor *opt_table = nullptr;  // device table of trainable tensors, update order
+  bool packs_valid = false;  // wp_fwd / wp_dx of every layer match its weights
   int opt_tensors = 0, opt_blocks = 0;
   double opt_params = 0.0;
   // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
@@ -131,7 +132,7 @@ bool layer_forks(const tdh_net::Layer &L) {
   return L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC;
 }
 
-// packed: the layers' wp_fwd are being filled on side stream 0 (events n+i mark them ready)
+// packed: the layers' wp_fwd hold the current filters in the stride-1 kernels' layout
 int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
   const float *in = x;
   const int n     = static_cast<int>(net->layers.size());
@@ -141,8 +142,7 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
     switch (s.kind) {
       case TDH_L_CONV:
         TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
-        if (packed && L.wp_fwd && layer_forks(L) && conv_uses_packed(&s.conv, batch, 0)) {
-          TDH_HIP(hipStreamWaitEvent(ctx().stream, net->events[n + i], 0));
+        if (packed && L.wp_fwd && conv_uses_packed(&s.conv, batch, 0)) {
           TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, L.wp_fwd));
         } else {
           TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev));
@@ -267,6 +267,17 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
         const size_t n = which ? L.b_size : L.w_size;
         if (!n) continue;
         OptTensor t;
+        t.wp_fwd = t.wp_dx = nullptr;
+        t.tbl = nullptr;
+        t.C = t.Kc = t.rs = 1;
+        if (!which && L.wp_fwd) {
+          t.wp_fwd = L.wp_fwd;
+          t.wp_dx  = L.wp_dx;
+          t.tbl    = L.spec.conv.tbl ? L.tbl_dev : nullptr;
+          t.C      = static_cast<uint32_t>(L.spec.conv.in_c);
+          t.Kc     = static_cast<uint32_t>(L.spec.conv.out_c);
+          t.rs     = static_cast<uint32_t>(L.spec.conv.k_w * L.spec.conv.k_h);
+        }
         t.g  = which ? L.db : L.dw;
         t.w  = which ? L.b : L.w;
         t.s0 = which ? L.s0b : L.s0w;
@@ -338,13 +349,17 @@ size_t tdh_net_param_size(const tdh_net *net, int layer, int which) {
   if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return 0;
   return which == 0 ? net->layers[layer].w_size : (which == 1 ? net->layers[layer].b_size : 0);
 }
-float *tdh_net_param(tdh_net *net, int layer, int which) {
+static float *net_param_ptr(tdh_net *net, int layer, int which) {
   if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
   return which == 0 ? net->layers[layer].w : (which == 1 ? net->layers[layer].b : nullptr);
 }
+float *tdh_net_param(tdh_net *net, int layer, int which) {
+  if (net) net->packs_valid = false;  // the caller may write through the pointer
+  return net ? net_param_ptr(net, layer, which) : nullptr;
+}
 int tdh_net_set_param(tdh_net *net, int layer, int which, const float *host_src) {
   TDH_REQUIRE_INIT();
-  float *dst = tdh_net_param(net, layer, which);
+  float *dst = tdh_net_param(net, layer, which);  // marks the packed filters stale
   const size_t n = tdh_net_param_size(net, layer, which);
   TDH_CHECK_ARG(n == 0 || (dst && host_src), "tdh_net_set_param: no such parameter");
   return tdh_memcpy_h2d(dst, host_src, n * sizeof(float));
@@ -362,7 +377,7 @@ int tdh_net_reset_optimizer(tdh_net *net) {
 }
 int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst) {
   TDH_REQUIRE_INIT();
-  const float *src = tdh_net_param(net, layer, which);
+  const float *src = net_param_ptr(net, layer, which);
   const size_t n   = tdh_net_param_size(net, layer, which);
   TDH_CHECK_ARG(n == 0 || (src && host_dst), "tdh_net_get_param: no such parameter");
   return tdh_memcpy_d2h(host_dst, src, n * sizeof(float));
@@ -404,41 +419,14 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     ~KeepScratch() { c.ws_keep = false; }
   } keep(c, forked);
   bool side_used[2] = {false, false};
+  // the per-kernel timing pass of a net whose captured step branches launches what that step
+  // launches (a branching step computes dX, dW and db of a layer separately)
+  const bool as_forked = !forked && profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch);
   const int n   = static_cast<int>(net->layers.size());
-  bool packed_dx = false;
-  if (forked) {
-    // the filters do not change until the optimizer runs: pack them for every layer now, beside
-    // the forward pass, instead of in front of each convolution
-    bool any = false;
-    for (int i = 0; i < n; ++i) {
-      tdh_net::Layer &L = net->layers[i];
-      if (!L.wp_fwd || !layer_forks(L)) continue;
-      const bool f = conv_uses_packed(&L.spec.conv, batch, 0), b = conv_uses_packed(&L.spec.conv, batch, 1);
-      if (!f && !b) continue;
-      if (!any) {
-        TDH_HIP(hipEventRecord(net->events[2 * n + 2], c.stream));
-        TDH_HIP(hipStreamWaitEvent(c.side[0], net->events[2 * n + 2], 0));
-        any = true;
-      }
-      StreamSwap on_side(c.side[0]);
-      if (f) {
-        TDH_TRY(conv_pack_filters(&L.spec.conv, 0, L.w, L.tbl_dev, L.wp_fwd));
-        TDH_HIP(hipEventRecord(net->events[n + i], c.side[0]));
-      }
-    }
-    for (int i = 0; i < n; ++i) {
-      tdh_net::Layer &L = net->layers[i];
-      if (!L.wp_dx || !layer_forks(L) || !conv_uses_packed(&L.spec.conv, batch, 1)) continue;
-      StreamSwap on_side(c.side[0]);
-      TDH_TRY(conv_pack_filters(&L.spec.conv, 1, L.w, L.tbl_dev, L.wp_dx));
-      packed_dx = true;
-    }
-    if (packed_dx) TDH_HIP(hipEventRecord(net->events[2 * n + 3], c.side[0]));
-    side_used[0] = any;
-  }
-  TDH_TRY(forward(net, batch, x, forked));
+  // the optimizer kernel keeps the packed filters of the stride-1 kernels current
+  const bool packed = net->packs_valid;
+  TDH_TRY(forward(net, batch, x, packed));
   tdh_net::Layer &last = net->layers[n - 1];
-  bool waited_dx = false;
   int first_bwd        = n - 1;
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
   // the full softmax Jacobian
@@ -475,12 +463,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     switch (s.kind) {
       case TDH_L_CONV:
         TDH_TRY(ws_begin((forked ? 3 : 1) * conv2d_workspace_bytes(&s.conv, batch)));
+      {
+        const float *wp = packed && L.wp_dx && conv_uses_packed(&s.conv, batch, 1) ? L.wp_dx : nullptr;
         if (forked) {
-          const float *wp = packed_dx && fork && L.wp_dx && conv_uses_packed(&s.conv, batch, 1) ? L.wp_dx : nullptr;
-          if (wp && !waited_dx) {
-            TDH_HIP(hipStreamWaitEvent(c.stream, net->events[2 * n + 3], 0));
-            waited_dx = true;
-          }
           if (!fork) {
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1, fold,
                                L.tbl_dev, wp));
@@ -497,9 +482,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           }
         } else {
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
-                             fold, L.tbl_dev));
+                             fold, L.tbl_dev, wp));
         }
-        break;
+      } break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
         if (fork) {
@@ -512,6 +497,12 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             StreamSwap on_side(c.side[1]);
             TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad()));
           }
+        } else if (as_forked) {
+          // the launches of the captured, branching step, one after the other
+          TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
+          TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad()));
+          if (L.b_size)
+            TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad()));
         } else {
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
                          L.b_size ? L.db : nullptr, 1, fold));
@@ -553,6 +544,17 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   TDH_CHECK_ARG(net && x && t && batch > 0 && batch <= net->max_batch,
                 "tdh_net_train_step: bad argument");
   TDH_CHECK_ARG(!do_update || opt, "tdh_net_train_step: update requested without an optimizer");
+  // The filters in the stride-1 kernels' layout: packed here when the weights came from
+  // outside (creation, tdh_net_set_param, a pointer handed out), by the optimizer kernel after
+  // that.
+  if ((net->flags & TDH_NET_GRAPH) && !net->packs_valid) {
+    for (tdh_net::Layer &L : net->layers) {
+      if (!L.wp_fwd) continue;
+      TDH_TRY(conv_pack_filters(&L.spec.conv, 0, L.w, L.tbl_dev, L.wp_fwd));
+      TDH_TRY(conv_pack_filters(&L.spec.conv, 1, L.w, L.tbl_dev, L.wp_dx));
+    }
+    net->packs_valid = true;
+  }
   // per-kernel timing needs the launches themselves, not a replay
   if (!(net->flags & TDH_NET_GRAPH) || profiling_active())
     return enqueue_step(net, opt, loss_kind, batch, x, t, do_update, nullptr);
