@@ -133,6 +133,8 @@ int launch_act_bwd(int kind, const float *p, int batch, int len, const float *x,
                    const float *dy, float *dx);
 int launch_loss_grad(int kind, int batch, int len, const float *y, const float *t, float *dy);
 int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz);
+// softmax forward (y) and the gradient above (dz) in one launch
+int launch_softmax_fwd_xent(int batch, int len, const float *x, const float *t, float *y, float *dz);
 int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, float *w, float *s0,
                       float *s1);
 // One launch for every trainable tensor of a network (update order = table order). Entry j
@@ -191,7 +193,7 @@ bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip);
 int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const uint8_t *tbl_resident,
                       float *wp);
 int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
-           const float *b, float *y);
+           const float *b, float *y, float *act_out = nullptr, int act_kind = 0);
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act);
 // conv_s1.hip: stride-1 forward / dX with LDS halo tiles (3x3 and 5x5 windows)

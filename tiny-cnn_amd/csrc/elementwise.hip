@@ -282,6 +282,38 @@ softmax_xent_grad_kernel(const float *__restrict__ y, const float *__restrict__ 
   for (int j = lane; j < len; j += 64) dz[static_cast<size_t>(row) * len + j] = yr[j] * st - tr[j];
 }
 
+// softmax forward and the gradient above in one pass over the row: the values and their order
+// of evaluation are those of softmax_fwd_kernel followed by softmax_xent_grad_kernel
+__global__ void __launch_bounds__(EW_THREADS)
+softmax_fwd_xent_kernel(const float *__restrict__ x, const float *__restrict__ t,
+                        float *__restrict__ y, float *__restrict__ dz, const int batch,
+                        const int len) {
+  const int row  = blockIdx.x * (EW_THREADS / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= batch) return;
+  const float *xr = x + static_cast<size_t>(row) * len;
+  const float *tr = t + static_cast<size_t>(row) * len;
+  float *yr       = y + static_cast<size_t>(row) * len;
+  float *dr       = dz + static_cast<size_t>(row) * len;
+  float m         = -FLT_MAX;
+  for (int j = lane; j < len; j += 64) m = fmaxf(m, xr[j]);
+  m       = wave_max(m);
+  float s = 0.0f, st = 0.0f;
+  for (int j = lane; j < len; j += 64) {
+    const float e = expf(xr[j] - m);
+    yr[j]         = e;
+    s += e;
+    st += tr[j];
+  }
+  s  = wave_sum(s);
+  st = wave_sum(st);
+  for (int j = lane; j < len; j += 64) {
+    const float v = yr[j] / s;
+    yr[j]         = v;
+    dr[j]         = v * st - tr[j];
+  }
+}
+
 // --------------------------------------------------------------- optimizers
 // tiny_dnn/optimizers/optimizer.h; g = merged * grad_scale is layer::update_weight's
 // diff (tiny_dnn/layers/layer.h:668-673). Scalars that the reference derives once per
@@ -600,6 +632,14 @@ int launch_loss_grad(int kind, int batch, int len, const float *y, const float *
     case TDH_LOSS_CE: return launch_map<CeGrad, true>(y, t, dy, n, NoParams(), "loss_grad_ce");
   }
   return set_error(TDH_ERR_INVALID, "loss kind %d is not supported", kind);
+}
+
+int launch_softmax_fwd_xent(int batch, int len, const float *x, const float *t, float *y, float *dz) {
+  ProfScope prof("softmax_fwd_xent_grad", 20.0 * batch * len, WORK_BYTE);
+  hipLaunchKernelGGL(softmax_fwd_xent_kernel, dim3(ceil_div(batch, EW_THREADS / 64)), dim3(EW_THREADS),
+                     0, ctx().stream, x, t, y, dz, batch, len);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
 }
 
 int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz) {

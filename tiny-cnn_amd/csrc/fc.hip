@@ -164,9 +164,15 @@ size_t fc_workspace_bytes(int in, int out, int batch) {
 }
 
 int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
-           const float *b, float *y) {
+           const float *b, float *y, float *act_out, int act_kind) {
   StridedOperand A{x, in, 1, batch};   // X[s][k], k contiguous
   StridedOperand B{w, 1, out, out};    // W[k][n], n contiguous
+  if (act_out) {  // the pointwise activation layer that follows leaves the same kernel
+    EpiRowMajorAct epi{y, out, has_bias ? b : nullptr, act_out, act_kind};
+    if (small_fc_applies(batch, out, in)) return launch_small_fc(A, B, epi, batch, out, in, "fc_fwd_small");
+    return launch_gemm<true, false, false, true>(A, B, epi, batch, out, in, true, "fc_fwd_gemm",
+                                                "fc_fwd_splitk_reduce");
+  }
   EpiRowMajor epi{y, out, has_bias ? b : nullptr, ActGrad(), 0};
   if (small_fc_applies(batch, out, in)) return launch_small_fc(A, B, epi, batch, out, in, "fc_fwd_small");
   return launch_gemm<true, false, false, true>(A, B, epi, batch, out, in, true, "fc_fwd_gemm",

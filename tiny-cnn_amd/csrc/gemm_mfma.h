@@ -104,6 +104,27 @@ struct EpiRowMajor {
   }
 };
 
+// forward product followed by a pointwise activation layer:
+// out[m*ld + n] = v + bias_n[n], act_out[m*ld + n] = act(out[m*ld + n])
+struct EpiRowMajorAct {
+  float *out;
+  int ld;
+  const float *bias_n;
+  float *act_out;
+  int act_kind;
+  struct Col {
+    int n;
+    float bias;
+  };
+  __device__ __forceinline__ Col col(int n) const { return {n, bias_n ? bias_n[n] : 0.0f}; }
+  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+    const int idx = m * ld + c.n;
+    v += c.bias;
+    out[idx]     = v;
+    act_out[idx] = act_apply(act_kind, v);
+  }
+};
+
 // GEMM column n = (img, p) with p < pix; out[(img*rows + m)*pix + p] = (v + bias_m[m]) * act'
 struct EpiImageRows {
   float *out;

@@ -133,7 +133,10 @@ bool layer_forks(const tdh_net::Layer &L) {
 }
 
 // packed: the layers' wp_fwd hold the current filters in the stride-1 kernels' layout
-int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
+// xent_t / xent_dz: the net ends in softmax and the step's loss is cross_entropy_multiclass: the
+// last layer's kernel also writes the loss gradient with respect to the softmax input
+int forward(tdh_net *net, int batch, const float *x, bool packed = false, const float *xent_t = nullptr,
+            float *xent_dz = nullptr) {
   const float *in = x;
   const int n     = static_cast<int>(net->layers.size());
   for (int i = 0; i < n; ++i) {
@@ -150,7 +153,15 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
-        TDH_TRY(fc_fwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out));
+        if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
+            is_pointwise_act(net->layers[i + 1].spec.act)) {
+          // the activation layer behind the product leaves the same kernel
+          TDH_TRY(fc_fwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out, net->layers[i + 1].out,
+                         net->layers[i + 1].spec.act));
+          ++i;
+        } else {
+          TDH_TRY(fc_fwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out));
+        }
         break;
       case TDH_L_MAXPOOL:
         if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
@@ -165,7 +176,10 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false) {
         break;
       case TDH_L_AVEPOOL: TDH_TRY(avepool_fwd(&s.pool, batch, in, L.w, L.b, L.out)); break;
       case TDH_L_ACT:
-        TDH_TRY(launch_act_fwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out));
+        if (xent_t && i == n - 1 && s.act == TDH_ACT_SOFTMAX)
+          TDH_TRY(launch_softmax_fwd_xent(batch, static_cast<int>(L.out_size), in, xent_t, L.out, xent_dz));
+        else
+          TDH_TRY(launch_act_fwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out));
         break;
     }
     in = net->layers[i].out;  // of the activation layer when one was fused
@@ -425,17 +439,16 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   const int n   = static_cast<int>(net->layers.size());
   // the optimizer kernel keeps the packed filters of the stride-1 kernels current
   const bool packed = net->packs_valid;
-  TDH_TRY(forward(net, batch, x, packed));
   tdh_net::Layer &last = net->layers[n - 1];
   int first_bwd        = n - 1;
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
-  // the full softmax Jacobian
+  // the full softmax Jacobian, and that kernel is the softmax layer's forward kernel
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
       last.spec.act == TDH_ACT_SOFTMAX && n >= 2) {
-    TDH_TRY(launch_softmax_xent_grad(batch, static_cast<int>(last.out_size), last.out, t,
-                                     net->layers[n - 2].dout));
+    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout));
     first_bwd = n - 2;
   } else {
+    TDH_TRY(forward(net, batch, x, packed));
     TDH_TRY(launch_loss_grad(loss_kind, batch, static_cast<int>(last.out_size), last.out, t,
                              last.dout));
   }
