@@ -459,7 +459,10 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     const float *in    = i == 0 ? x : net->layers[i - 1].out;
     float *dx          = i == 0 ? net->dx_in : net->layers[i - 1].dout;
     ActGrad fold;
-    const bool fork = forked && layer_forks(L);
+    // a small fully-connected layer computes its three gradients in one launch on the main
+    // chain: its weight and bias products are too small to be worth a branch
+    const bool fc_one_launch = s.kind == TDH_L_FC && fc_bwd_fuses(s.fc_in, s.fc_out, batch);
+    const bool fork = forked && layer_forks(L) && !fc_one_launch;
     if (fork) {
       // this layer's output gradient is complete here: let the side streams start from it
       TDH_HIP(hipEventRecord(net->events[i], c.stream));
@@ -510,7 +513,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             StreamSwap on_side(c.side[1]);
             TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad()));
           }
-        } else if (as_forked) {
+        } else if (as_forked && !fc_one_launch) {
           // the launches of the captured, branching step, one after the other
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad()));
