@@ -183,12 +183,14 @@ struct ActGrad {
 // conv.hip / fc.hip
 // prepacked: filters already packed by conv_pack_filters for this direction (and only then)
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
-               float *y, const uint8_t *tbl_resident = nullptr, const float *prepacked = nullptr);
+               float *y, const uint8_t *tbl_resident = nullptr, const float *prepacked = nullptr,
+               float *act_out = nullptr, int act_kind = 0);
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
                const uint8_t *tbl_resident = nullptr, const float *prepacked_dx = nullptr);
 // true when forward (flip = 0) / dX (flip = 1) of this layer reads packed filters
 bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip);
+bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked);
 // packs w (masked by the device-resident connection table, if any) into wp[k_w*k_h*in_c*out_c]
 int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const uint8_t *tbl_resident,
                       float *wp);
@@ -204,7 +206,7 @@ size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip,
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
                 int OW, int ph, int pw, ActGrad ag, const char *tag,
-                const float *prepacked = nullptr);
+                const float *prepacked = nullptr, float *act_out = nullptr, int act_kind = 0);
 int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const uint8_t *tbl_dev,
                    float *wp);
 // conv_dw.hip: stride-1 weight gradient from LDS-staged tiles (3x3 and 5x5 windows)
@@ -224,7 +226,7 @@ bool fc_bwd_fuses(int in, int out, int batch);
 int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax,
                 float *act_out = nullptr, int act_kind = TDH_ACT_NONE);
 int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
-                float *dx);
+                float *dx, ActGrad ag = ActGrad());
 int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *b,
                 float *y);
 int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,

@@ -422,6 +422,8 @@ constexpr int FSC_TR = 4 * FSC_TN;
 struct FwdSmallCinArgs {
   const float *x, *w, *bias;
   float *y;
+  float *act_out;  // act(y) of the pointwise activation layer that follows, or NULL
+  int act_kind;
   int batch, Kc, H, W, OH, OW, ph, pw;
   int tiles_x, tiles_y;
 };
@@ -527,7 +529,10 @@ conv_fwd_small_cin_kernel(const FwdSmallCinArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int co = 32 * mb + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (co < a.Kc) out[static_cast<size_t>(co) * ohw] = acc[mb][j][r] + (a.bias ? a.bias[co] : 0.0f);
+        if (co >= a.Kc) continue;
+        const float v = acc[mb][j][r] + (a.bias ? a.bias[co] : 0.0f);
+        out[static_cast<size_t>(co) * ohw] = v;
+        if (a.act_out) a.act_out[(out - a.y) + static_cast<size_t>(co) * ohw] = act_apply(a.act_kind, v);
       }
   }
 }
@@ -538,9 +543,10 @@ static bool small_cin_fwd_applies(const ConvGeom &g) {
 }
 
 static int launch_small_cin_fwd(const ConvGeom &g, int batch, const float *x, const float *w,
-                                const float *bias, float *y) {
+                                const float *bias, float *y, float *act_out, int act_kind) {
   FwdSmallCinArgs a;
   a.x = x; a.w = w; a.bias = bias; a.y = y;
+  a.act_out = act_out; a.act_kind = act_kind;
   a.batch = batch; a.Kc = g.Kc; a.H = g.H; a.W = g.W; a.OH = g.OH; a.OW = g.OW; a.ph = g.pad_h; a.pw = g.pad_w;
   a.tiles_x = ceil_div(g.OW, FSC_TC);
   a.tiles_y = ceil_div(g.OH, FSC_TR);
@@ -615,6 +621,12 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
   return TDH_OK;
 }
 
+// the forward kernel of this layer can write a following pointwise activation as well
+// (prepacked: the caller passes the filters in the stride-1 kernel's layout)
+bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked) {
+  return prepacked ? conv_uses_packed(d, batch, 0) : small_cin_fwd_applies(make_geom(d));
+}
+
 bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip) {
   const ConvGeom g = make_geom(d);
   if (g.sh != 1 || g.sw != 1) return false;
@@ -633,16 +645,21 @@ int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const ui
 }
 
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
-               float *y, const uint8_t *tbl_resident, const float *prepacked) {
+               float *y, const uint8_t *tbl_resident, const float *prepacked, float *act_out,
+               int act_kind) {
   const ConvGeom g = make_geom(d);
   if (prepacked)
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
-                       g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked);
+                       g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked, act_out,
+                       act_kind);
+  if (act_out && !small_cin_fwd_applies(g))
+    return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not apply a following activation");
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
-  if (small_cin_fwd_applies(g)) return launch_small_cin_fwd(g, batch, x, w_eff, d->has_bias ? b : nullptr, y);
+  if (small_cin_fwd_applies(g))
+    return launch_small_cin_fwd(g, batch, x, w_eff, d->has_bias ? b : nullptr, y, act_out, act_kind);
   if (g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 &&
       conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w))
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w_eff, nullptr,

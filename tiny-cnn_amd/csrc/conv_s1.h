@@ -24,6 +24,8 @@ struct ConvS1Args {
   const float *in, *wp, *bias;
   float *out;
   ActGrad ag;
+  float *act_out;              // forward: act(out) of the pointwise activation layer that follows
+  int act_kind;
   int batch, KC, MC, IH, IW, OH, OW, ph, pw;
   int pwa;                     // staged column 0 is image column x0 - pwa
   int TR, TI;                  // tile rows, images per tile (TI*TR*TC = PIX), powers of two

@@ -12,7 +12,8 @@ template <int VEC>
 __global__ void __launch_bounds__(256)
 s1_split_reduce_kernel(const float *__restrict__ part, const int splits, const size_t stride,
                        float *__restrict__ out, const float *__restrict__ bias, const ActGrad ag,
-                       const int MC, const FastDiv div_plane, const size_t total) {
+                       const int MC, const FastDiv div_plane, const size_t total,
+                       float *__restrict__ act_out, const int act_kind) {
   const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
   if (i >= total) return;
   float v[VEC];
@@ -37,6 +38,10 @@ s1_split_reduce_kernel(const float *__restrict__ part, const int splits, const s
     *reinterpret_cast<float4 *>(out + i) = make_float4(v[0], v[1], v[2], v[VEC - 1]);
   else
     out[i] = v[0];
+  if (act_out) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) act_out[i + e] = act_apply(act_kind, v[e]);
+  }
 }
 
 // wp[t][kc][m]: forward (flip = 0): kc = ci, m = co, t as is; dX (flip = 1): kc = co, m = ci,
@@ -177,7 +182,8 @@ int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const 
 // result of conv_s1_repack for this filter, when the caller already has it (w is not read).
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
-                int OW, int ph, int pw, ActGrad ag, const char *tag, const float *prepacked) {
+                int OW, int ph, int pw, ActGrad ag, const char *tag, const float *prepacked,
+                float *act_out, int act_kind) {
   const int KC = flip ? Kc : C, MC = flip ? C : Kc;
   S1Plan p = make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw);
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_s1_run: shape not supported");
@@ -190,6 +196,7 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
   }
   p.args.in = in; p.args.wp = static_cast<const float *>(wp); p.args.bias = bias;
   p.args.out = out; p.args.ag = ag;
+  p.args.act_out = act_out; p.args.act_kind = act_kind;
   if (p.splits > 1) {
     void *part = nullptr;
     TDH_TRY(ws_take(sizeof(float) * p.splits * p.args.part_stride, &part));
@@ -209,11 +216,11 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
     if (plane % 4 == 0)
       hipLaunchKernelGGL((s1_split_reduce_kernel<4>), dim3(static_cast<unsigned>(ceil_div_sz(total / 4, 256))), dim3(256), 0,
                          ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
-                         FastDiv(plane), total);
+                         FastDiv(plane), total, act_out, act_kind);
     else
       hipLaunchKernelGGL((s1_split_reduce_kernel<1>), dim3(static_cast<unsigned>(ceil_div_sz(total, 256))), dim3(256), 0,
                          ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
-                         FastDiv(plane), total);
+                         FastDiv(plane), total, act_out, act_kind);
     TDH_LAUNCH_CHECK();
   }
   return TDH_OK;

@@ -278,6 +278,13 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
         const int m = mb + 8 * (rr >> 2) + (rr & 3);
         if (m < a.MC) dst[pbase + static_cast<size_t>(m) * ohw] = v[rr];
       }
+      if (!a.part && a.act_out) {
+#pragma unroll
+        for (int rr = 0; rr < 16; ++rr) {
+          const int m = mb + 8 * (rr >> 2) + (rr & 3);
+          if (m < a.MC) a.act_out[pbase + static_cast<size_t>(m) * ohw] = act_apply(a.act_kind, v[rr]);
+        }
+      }
     }
   }
 }

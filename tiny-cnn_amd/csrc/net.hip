@@ -145,11 +145,18 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
     switch (s.kind) {
       case TDH_L_CONV:
         TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
-        if (packed && L.wp_fwd && conv_uses_packed(&s.conv, batch, 0)) {
-          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, L.wp_fwd));
+      {
+        const float *wp = packed && L.wp_fwd && conv_uses_packed(&s.conv, batch, 0) ? L.wp_fwd : nullptr;
+        if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
+            is_pointwise_act(net->layers[i + 1].spec.act) && conv_fwd_applies_act(&s.conv, batch, wp != nullptr)) {
+          // the activation layer behind the convolution leaves the same kernel
+          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp, net->layers[i + 1].out,
+                             net->layers[i + 1].spec.act));
+          ++i;
         } else {
-          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev));
+          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp));
         }
+      }
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
@@ -264,10 +271,12 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       net->scratch += 3 * ws_align(need);
     else if (need > net->scratch)
       net->scratch = need;
-    // fold pointwise activation gradients into the following conv/fc dX epilogue
+    // fold pointwise activation gradients into the following layer's backward kernel (the dX
+    // epilogue of a conv / fc layer, the scatter of a max-pool)
     if ((flags & TDH_NET_FUSE_ACT_GRAD) && L.spec.kind == TDH_L_ACT &&
         is_pointwise_act(L.spec.act) && i + 1 < n_layers &&
-        (layers[i + 1].kind == TDH_L_CONV || layers[i + 1].kind == TDH_L_FC))
+        (layers[i + 1].kind == TDH_L_CONV || layers[i + 1].kind == TDH_L_FC ||
+         layers[i + 1].kind == TDH_L_MAXPOOL))
       L.grad_folded = true;
   }
   if (rc == TDH_OK)
@@ -524,7 +533,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
                          L.b_size ? L.db : nullptr, 1, fold));
         }
         break;
-      case TDH_L_MAXPOOL: TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx)); break;
+      case TDH_L_MAXPOOL: TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold)); break;
       case TDH_L_AVEPOOL:
         TDH_TRY(ws_begin(avepool_workspace_bytes(&s.pool, batch)));
         TDH_TRY(avepool_bwd(&s.pool, batch, in, L.w, L.dout, dx, L.dw, L.db, 1));

@@ -111,7 +111,7 @@ maxpool2x2_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
 __global__ void __launch_bounds__(PT)
 maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ argmax,
                       float *__restrict__ dx, const int pairs, const int W, const int OW2,
-                      const FastDiv div_ow2, const int rows_per_sample) {
+                      const FastDiv div_ow2, const int rows_per_sample, const ActGrad ag) {
   const int t = blockIdx.x * PT + threadIdx.x;
   if (t >= pairs) return;
   uint32_t row, ox2;
@@ -129,7 +129,16 @@ maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ 
   r1.y = a.x == base + W + 1 ? g.x : 0.0f;
   r1.z = a.y == base + W + 2 ? g.y : 0.0f;
   r1.w = a.y == base + W + 3 ? g.y : 0.0f;
-  float *p = dx + (static_cast<size_t>(2 * row) * W + 4 * ox2);
+  const size_t at = static_cast<size_t>(2 * row) * W + 4 * ox2;
+  if (ag.kind != TDH_ACT_NONE) {  // the activation layer in front of the pool: dx *= act'(its output)
+    const float4 y0 = *reinterpret_cast<const float4 *>(ag.y + at);
+    const float4 y1 = *reinterpret_cast<const float4 *>(ag.y + at + W);
+    r0.x *= act_grad_factor(ag.kind, y0.x); r0.y *= act_grad_factor(ag.kind, y0.y);
+    r0.z *= act_grad_factor(ag.kind, y0.z); r0.w *= act_grad_factor(ag.kind, y0.w);
+    r1.x *= act_grad_factor(ag.kind, y1.x); r1.y *= act_grad_factor(ag.kind, y1.y);
+    r1.z *= act_grad_factor(ag.kind, y1.z); r1.w *= act_grad_factor(ag.kind, y1.w);
+  }
+  float *p = dx + at;
   *reinterpret_cast<float4 *>(p)     = r0;
   *reinterpret_cast<float4 *>(p + W) = r1;
 }
@@ -139,7 +148,7 @@ maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ 
 // inputs no window contains (strides larger than the window).
 __global__ void __launch_bounds__(PT)
 maxpool_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ argmax,
-                   float *__restrict__ dx, const int total, const PoolGeom g) {
+                   float *__restrict__ dx, const int total, const PoolGeom g, const ActGrad ag) {
   const int i = blockIdx.x * PT + threadIdx.x;
   if (i >= total) return;
   uint32_t t, xx, yy, c, img;
@@ -153,7 +162,9 @@ maxpool_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ arg
   const int outi  = covered ? (g.OH * c + oy) * g.OW + ox : 0;
   const int local = (g.H * c + yy) * g.W + xx;  // flat CHW index inside the sample
   const size_t ob = static_cast<size_t>(img) * g.C * g.OH * g.OW;
-  dx[i]           = (argmax[ob + outi] == local) ? dy[ob + outi] : 0.0f;
+  float v         = (argmax[ob + outi] == local) ? dy[ob + outi] : 0.0f;
+  if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[i]);
+  dx[i] = v;
 }
 
 // tiny_average_pooling_kernel (average_pooling_layer.h:25-55). Window (oy,ox) exists when it
@@ -291,20 +302,22 @@ int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int
 }
 
 int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
-                float *dx) {
+                float *dx, ActGrad ag) {
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.H * g.W;
   TDH_CHECK_ARG(g.OH > 0 && g.OW > 0, "maxpool backward: empty output");
-  ProfScope prof("maxpool_bwd", 8.0 * batch * g.C * g.OH * g.OW + 4.0 * total, WORK_BYTE);
-  if (is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) && total / 8 < (1L << 31)) {
+  ProfScope prof(ag.kind != TDH_ACT_NONE ? "maxpool_bwd_act" : "maxpool_bwd",
+                 8.0 * batch * g.C * g.OH * g.OW + (ag.kind != TDH_ACT_NONE ? 8.0 : 4.0) * total, WORK_BYTE);
+  if (is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) && total / 8 < (1L << 31) &&
+      (ag.kind == TDH_ACT_NONE || aligned16(ag.y))) {
     const int pairs = static_cast<int>(total / 8);
     hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
-                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H);
+                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag);
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
   hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, dy,
-                     argmax, dx, static_cast<int>(total), g);
+                     argmax, dx, static_cast<int>(total), g, ag);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }
