@@ -96,9 +96,24 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wco = wave % WCO, wk = (wave / WCO) % WK, wfy = wave / (WCO * WK);
-  const int tx = blockIdx.x % a.tiles_x, slice = blockIdx.x / a.tiles_x;
-  const int x0 = tx * TC, co0 = blockIdx.y * BCO;
-  const int ci0 = (blockIdx.z / FYB) * 32, fy0 = (blockIdx.z % FYB) * R;
+  // Workgroups are handed to the eight XCDs (each with its own L2) round-robin in launch
+  // order. Renumber them so that the workgroups that read the same tiles (the filter rows of a
+  // channel block share dY and X, the input-channel blocks share dY, the output-channel blocks
+  // share X) are neighbours on one XCD.
+  int bx, by, bz;
+  {
+    const int gy = gridDim.y, gz = gridDim.z;
+    const int total = gridDim.x * gy * gz, per = total >> 3;
+    int id = blockIdx.x + gridDim.x * (blockIdx.y + gy * blockIdx.z);
+    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
+    bz = id % gz;  // filter row fastest, then input-channel block
+    id /= gz;
+    by = id % gy;
+    bx = id / gy;
+  }
+  const int tx = bx % a.tiles_x, slice = bx / a.tiles_x;
+  const int x0 = tx * TC, co0 = by * BCO;
+  const int ci0 = (bz / FYB) * 32, fy0 = (bz % FYB) * R;
   const int hw = a.H * a.W, ohw = a.OH * a.OW;
   const int chw = a.C * hw, kohw = a.Kc * ohw;
 
@@ -300,7 +315,7 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     const int ci = ci0 + (lane & 31);
     const int crs = a.C * RF * S;
     if (ci < a.C) {
-      float *dst = a.partial + static_cast<size_t>(blockIdx.x) * a.Kc * crs + ci * (RF * S) +
+      float *dst = a.partial + static_cast<size_t>(bx) * a.Kc * crs + ci * (RF * S) +
                    (fy0 + wfy * RPW) * S;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
