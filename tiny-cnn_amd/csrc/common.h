@@ -28,6 +28,9 @@ struct Context {
   size_t workspace_off  = 0;
   bool ws_locked        = false;  // a network owns the reservation: ops must fit, never grow
   bool ws_keep          = false;  // ws_begin does not rewind: pieces handed out stay disjoint
+  // a train step collects the split reductions of its weight gradients and the row sums of its
+  // bias gradients and launches each kind once (flush_deferred_*)
+  bool defer_reduce = false, defer_rowsum = false;
   // two more streams (default priority) for work that branches off the main one inside a
   // captured train step; created on first use
   hipStream_t side[2]   = {nullptr, nullptr};
@@ -160,6 +163,9 @@ bool profiling_active();
 // deterministic reductions: out[r] (+)= sum over `cols` contiguous values of row r,
 // rows laid out as [outer][rows][cols] and summed over outer in order
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate);
+// launch what was recorded on the current stream (launch = false: forget it)
+int flush_deferred_rowsums(bool launch = true);   // elementwise.hip
+int flush_deferred_reduces(bool launch = true);   // conv.hip
 // norm.hip
 size_t batchnorm_workspace_bytes(int channels, int batch);
 int batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,

@@ -12,6 +12,9 @@
 //   db       row sums of dY per output channel, fixed two-stage order
 //
 // Reference: conv2d_op_internal.h:13-74 (forward), :78-181 (backward).
+#include <algorithm>
+#include <vector>
+
 #include "gemm_mfma.h"
 
 namespace tdh {
@@ -623,6 +626,52 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
 
 // the forward kernel of this layer can write a following pointwise activation as well
 // (prepacked: the caller passes the filters in the stride-1 kernel's layout)
+__global__ void __launch_bounds__(256) splitk_reduce_multi_kernel(const ReduceJobs jobs) {
+  __shared__ float sm[REDUCE_GROUPS][REDUCE_OUTPUTS];
+  int j = 0;
+  while (j + 1 < jobs.n && jobs.first_block[j + 1] <= static_cast<int>(blockIdx.x)) ++j;
+  const ReduceJob &r = jobs.job[j];
+  splitk_reduce_block(r.partial, r.splits, r.M, r.N, r.epi, static_cast<int>(blockIdx.x) - jobs.first_block[j], sm);
+}
+
+static std::vector<ReduceJob> &deferred_reduces() {
+  static std::vector<ReduceJob> jobs;
+  return jobs;
+}
+
+int flush_deferred_reduces(bool launch) {
+  std::vector<ReduceJob> &all = deferred_reduces();
+  if (!launch) all.clear();
+  for (size_t at = 0; at < all.size(); at += REDUCE_MULTI_MAX) {
+    ReduceJobs jobs;
+    jobs.n = static_cast<int>(std::min<size_t>(REDUCE_MULTI_MAX, all.size() - at));
+    int blocks = 0;
+    double bytes = 0.0;
+    for (int j = 0; j < jobs.n; ++j) {
+      jobs.job[j]         = all[at + j];
+      jobs.first_block[j] = blocks;
+      blocks += ceil_div(jobs.job[j].M * jobs.job[j].N, REDUCE_OUTPUTS);
+      bytes += 4.0 * jobs.job[j].M * jobs.job[j].N * (jobs.job[j].splits + 1);
+    }
+    jobs.first_block[jobs.n] = blocks;
+    ProfScope prof("conv_dw_splitk_reduce_multi", bytes, WORK_BYTE);
+    hipLaunchKernelGGL(splitk_reduce_multi_kernel, dim3(blocks), dim3(256), 0, ctx().stream, jobs);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      all.clear();
+      return set_error(TDH_ERR_HIP, "splitk_reduce_multi_kernel: %s", hipGetErrorString(e));
+    }
+  }
+  all.clear();
+  return TDH_OK;
+}
+
+bool defer_reduce(const float *partial, int splits, int M, int N, const EpiRowMajor &epi) {
+  if (!ctx().defer_reduce) return false;
+  deferred_reduces().push_back(ReduceJob{partial, splits, M, N, epi});
+  return true;
+}
+
 bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked) {
   return prepacked ? conv_uses_packed(d, batch, 0) : small_cin_fwd_applies(make_geom(d));
 }

@@ -466,8 +466,9 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
     else TDH_TRY(launch_dw_vec<false>(p));
   }
   const int slices = static_cast<int>(p.grid.x);
-  ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
   EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
+  if (defer_reduce(p.args.partial, slices, Kc, crs, epi)) return TDH_OK;
+  ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
   hipLaunchKernelGGL((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * crs, REDUCE_OUTPUTS)),
                      dim3(256), 0, ctx().stream, p.args.partial, slices, Kc, crs, epi);
   TDH_LAUNCH_CHECK();

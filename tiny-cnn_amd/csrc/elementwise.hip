@@ -2,7 +2,9 @@
 // loss gradients, optimizer updates and the fixed-order reductions used for bias
 // gradients. One pass over each array, 16-byte accesses where alignment allows.
 // Built with -ffp-contract=off so that a*b+c rounds twice, as in the scalar reference.
+#include <algorithm>
 #include <cfloat>
+#include <vector>
 
 #include "common.h"
 
@@ -498,11 +500,10 @@ __device__ __forceinline__ float block_sum(float v, float *smem4) {
 // src[(o*rows + r)*cols + c]. Stage 1: workgroup (r, g) adds the planes of images
 // o = g, g+G, ... in order, each plane with a fixed block-wide tree. Stage 2: one wave per
 // row adds the G group sums with a fixed butterfly.
-__global__ void __launch_bounds__(EW_THREADS)
-rowsum_stage1_kernel(const float *__restrict__ src, const int outer, const int rows,
-                     const int cols, const int groups, float *__restrict__ partial) {
-  __shared__ float smem4[4];
-  const int r = blockIdx.x, g = blockIdx.y;
+__device__ __forceinline__ void rowsum_stage1_block(const float *__restrict__ src, const int outer,
+                                                    const int rows, const int cols, const int groups,
+                                                    float *__restrict__ partial, const int r,
+                                                    const int g, float *smem4) {
   float s = 0.0f;
   for (int o = g; o < outer; o += groups) {
     const float *p = src + (static_cast<size_t>(o) * rows + r) * cols;
@@ -512,16 +513,62 @@ rowsum_stage1_kernel(const float *__restrict__ src, const int outer, const int r
   if (threadIdx.x == 0) partial[r * groups + g] = s;
 }
 
-__global__ void __launch_bounds__(EW_THREADS)
-rowsum_stage2_kernel(const float *__restrict__ partial, const int rows, const int groups,
-                     float *__restrict__ out, const int accumulate) {
-  const int r    = blockIdx.x * (EW_THREADS / 64) + (threadIdx.x >> 6);
+__device__ __forceinline__ void rowsum_stage2_block(const float *__restrict__ partial, const int rows,
+                                                    const int groups, float *__restrict__ out,
+                                                    const int accumulate, const int block) {
+  const int r    = block * (EW_THREADS / 64) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (r >= rows) return;
   float s = 0.0f;
   for (int g = lane; g < groups; g += 64) s += partial[r * groups + g];
   s = wave_sum(s);
   if (lane == 0) out[r] = accumulate ? out[r] + s : s;
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+rowsum_stage1_kernel(const float *__restrict__ src, const int outer, const int rows,
+                     const int cols, const int groups, float *__restrict__ partial) {
+  __shared__ float smem4[4];
+  rowsum_stage1_block(src, outer, rows, cols, groups, partial, blockIdx.x, blockIdx.y, smem4);
+}
+
+__global__ void __launch_bounds__(EW_THREADS)
+rowsum_stage2_kernel(const float *__restrict__ partial, const int rows, const int groups,
+                     float *__restrict__ out, const int accumulate) {
+  rowsum_stage2_block(partial, rows, groups, out, accumulate, blockIdx.x);
+}
+
+// The bias gradients of several layers in one pair of launches. Job j owns the workgroups
+// [first1[j], first1[j+1]) of stage 1, numbered g*rows + r, and [first2[j], first2[j+1]) of
+// stage 2; every job keeps the grouping and the order of additions of a launch of its own.
+constexpr int ROWSUM_MULTI_MAX = 8;
+struct RowsumJob {
+  const float *src;
+  float *partial, *out;
+  int outer, rows, cols, groups, accumulate;
+};
+struct RowsumJobs {
+  RowsumJob job[ROWSUM_MULTI_MAX];
+  int first1[ROWSUM_MULTI_MAX + 1], first2[ROWSUM_MULTI_MAX + 1];
+  int n;
+};
+
+__global__ void __launch_bounds__(EW_THREADS) rowsum_multi_stage1_kernel(const RowsumJobs jobs) {
+  __shared__ float smem4[4];
+  int j = 0;
+  while (j + 1 < jobs.n && jobs.first1[j + 1] <= static_cast<int>(blockIdx.x)) ++j;
+  const RowsumJob &q = jobs.job[j];
+  const int b = static_cast<int>(blockIdx.x) - jobs.first1[j];
+  const int g = b / q.rows, r = b - g * q.rows;
+  rowsum_stage1_block(q.src, q.outer, q.rows, q.cols, q.groups, q.partial, r, g, smem4);
+}
+
+__global__ void __launch_bounds__(EW_THREADS) rowsum_multi_stage2_kernel(const RowsumJobs jobs) {
+  int j = 0;
+  while (j + 1 < jobs.n && jobs.first2[j + 1] <= static_cast<int>(blockIdx.x)) ++j;
+  const RowsumJob &q = jobs.job[j];
+  rowsum_stage2_block(q.partial, q.rows, q.groups, q.out, q.accumulate,
+                      static_cast<int>(blockIdx.x) - jobs.first2[j]);
 }
 
 // out[c] (+)= sum_s src[s*cols + c] (fully_connected bias gradient). A workgroup owns 32
@@ -747,10 +794,55 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
   return TDH_OK;
 }
 
+static std::vector<RowsumJob> &deferred_rowsums() {
+  static std::vector<RowsumJob> jobs;
+  return jobs;
+}
+
+int flush_deferred_rowsums(bool launch) {
+  std::vector<RowsumJob> &all = deferred_rowsums();
+  if (!launch) all.clear();
+  for (size_t at = 0; at < all.size(); at += ROWSUM_MULTI_MAX) {
+    RowsumJobs jobs;
+    jobs.n = static_cast<int>(std::min<size_t>(ROWSUM_MULTI_MAX, all.size() - at));
+    int b1 = 0, b2 = 0;
+    double bytes = 0.0;
+    for (int j = 0; j < jobs.n; ++j) {
+      const RowsumJob &q = jobs.job[j] = all[at + j];
+      jobs.first1[j] = b1;
+      jobs.first2[j] = b2;
+      b1 += q.rows * q.groups;
+      b2 += ceil_div(q.rows, EW_THREADS / 64);
+      bytes += 4.0 * q.outer * q.rows * q.cols;
+    }
+    jobs.first1[jobs.n] = b1;
+    jobs.first2[jobs.n] = b2;
+    ProfScope prof("bias_grad_rowsum_multi", bytes, WORK_BYTE);
+    hipLaunchKernelGGL(rowsum_multi_stage1_kernel, dim3(b1), dim3(EW_THREADS), 0, ctx().stream, jobs);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(rowsum_multi_stage2_kernel, dim3(b2), dim3(EW_THREADS), 0, ctx().stream,
+                         jobs);
+      e = hipGetLastError();
+    }
+    if (e != hipSuccess) {
+      all.clear();
+      return set_error(TDH_ERR_HIP, "rowsum_multi kernels: %s", hipGetErrorString(e));
+    }
+  }
+  all.clear();
+  return TDH_OK;
+}
+
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate) {
   const int groups = rowsum_groups(outer);
   void *ws = nullptr;
   TDH_TRY(ws_take(static_cast<size_t>(rows) * groups * sizeof(float), &ws));
+  if (ctx().defer_rowsum) {
+    deferred_rowsums().push_back(
+        RowsumJob{src, static_cast<float *>(ws), out, outer, rows, cols, groups, accumulate});
+    return TDH_OK;
+  }
   ProfScope prof("bias_grad_rowsum", 4.0 * outer * rows * cols, WORK_BYTE);
   hipLaunchKernelGGL(rowsum_stage1_kernel, dim3(rows, groups), dim3(EW_THREADS), 0, ctx().stream,
                      src, outer, rows, cols, groups, static_cast<float *>(ws));

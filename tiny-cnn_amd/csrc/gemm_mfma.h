@@ -438,13 +438,12 @@ constexpr int REDUCE_OUTPUTS = 32;
 constexpr int REDUCE_GROUPS  = 8;
 
 template <class Epi>
-__global__ void __launch_bounds__(256)
-splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const int M, const int N,
-                     const Epi epi) {
-  __shared__ float sm[REDUCE_GROUPS][REDUCE_OUTPUTS];
+__device__ __forceinline__ void splitk_reduce_block(const float *__restrict__ partial, const int splits,
+                                                    const int M, const int N, const Epi &epi,
+                                                    const int block, float (*sm)[REDUCE_OUTPUTS]) {
   const int o   = threadIdx.x & (REDUCE_OUTPUTS - 1);
   const int g   = threadIdx.x / REDUCE_OUTPUTS;
-  const int idx = blockIdx.x * REDUCE_OUTPUTS + o;
+  const int idx = block * REDUCE_OUTPUTS + o;
   const size_t mn = static_cast<size_t>(M) * N;
   float s = 0.0f;
   if (idx < M * N) {
@@ -469,6 +468,36 @@ splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const 
     epi.store(m, epi.col(n), t);
   }
 }
+
+template <class Epi>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const int M, const int N,
+                     const Epi epi) {
+  __shared__ float sm[REDUCE_GROUPS][REDUCE_OUTPUTS];
+  splitk_reduce_block(partial, splits, M, N, epi, blockIdx.x, sm);
+}
+
+// Several reductions in one launch: the weight gradients of a train step's layers, whose
+// partial tiles are all complete when the last dW kernel ends. Job j owns the workgroups
+// [first_block[j], first_block[j+1]).
+constexpr int REDUCE_MULTI_MAX = 8;
+struct ReduceJob {
+  const float *partial;
+  int splits, M, N;
+  EpiRowMajor epi;
+};
+struct ReduceJobs {
+  ReduceJob job[REDUCE_MULTI_MAX];
+  int first_block[REDUCE_MULTI_MAX + 1];
+  int n;
+};
+__global__ void __launch_bounds__(256) splitk_reduce_multi_kernel(const ReduceJobs jobs);
+
+// While ctx().defer_reduce is set, a split reduction with the row-major epilogue is recorded
+// instead of launched; flush_deferred_reduces() (common.h) launches what was recorded.
+bool defer_reduce(const float *partial, int splits, int M, int N, const EpiRowMajor &epi);
+template <class Epi>
+inline bool defer_reduce(const float *, int, int, int, const Epi &) { return false; }
 
 // ------------------------------------------------------------------- launcher
 struct GemmPlan {
@@ -608,6 +637,7 @@ int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
   TDH_TRY(rc);
   if (p.splits > 1) {
     // reads every partial tile once and writes the result once
+    if (defer_reduce(partial, p.splits, M, N, epi)) return TDH_OK;
     ProfScope prof(reduce_tag, 4.0 * M * N * (p.splits + 1), WORK_BYTE);
     hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, REDUCE_OUTPUTS)), dim3(256), 0,
                        ctx().stream, partial, p.splits, M, N, epi);

@@ -442,6 +442,19 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     ~KeepScratch() { c.ws_keep = false; }
   } keep(c, forked);
   bool side_used[2] = {false, false};
+  // The split reductions behind the weight-gradient kernels and the row sums of the bias
+  // gradients of a branching step are collected and launched once each behind the last layer:
+  // one launch per layer would sit at the end of its side stream's queue anyway, and every
+  // launch there costs its own dispatch latency.
+  struct Deferred {
+    Context &c;
+    explicit Deferred(Context &cc) : c(cc) {}
+    ~Deferred() {
+      c.defer_reduce = c.defer_rowsum = false;
+      flush_deferred_reduces(false);
+      flush_deferred_rowsums(false);
+    }
+  } deferred(c);
   // the per-kernel timing pass of a net whose captured step branches launches what that step
   // launches (a branching step computes dX, dW and db of a layer separately)
   const bool as_forked = !forked && profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch);
@@ -499,11 +512,15 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
           {
             StreamSwap on_side(c.side[0]);
+            c.defer_reduce = true;
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad(), L.tbl_dev));
+            c.defer_reduce = false;
           }
           if (L.b_size) {
             StreamSwap on_side(c.side[1]);
+            c.defer_rowsum = true;
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));
+            c.defer_rowsum = false;
           }
         } else {
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
@@ -516,7 +533,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
           {
             StreamSwap on_side(c.side[0]);
+            c.defer_reduce = true;
             TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad()));
+            c.defer_reduce = false;
           }
           if (L.b_size) {
             StreamSwap on_side(c.side[1]);
@@ -543,6 +562,14 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           TDH_TRY(launch_act_bwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out, L.dout, dx));
         break;
     }
+  }
+  if (side_used[0]) {
+    StreamSwap on_side(c.side[0]);
+    TDH_TRY(flush_deferred_reduces());
+  }
+  if (side_used[1]) {
+    StreamSwap on_side(c.side[1]);
+    TDH_TRY(flush_deferred_rowsums());
   }
   for (int k = 0; k < 2; ++k) {  // the optimizer (and the end of the capture) wait for the branches
     if (!side_used[k]) continue;
