@@ -198,6 +198,54 @@ def test_net_with_every_other_activation_matches_oracle(T, O, W):
                     assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} b {i}")
 
 
+@pytest.mark.parametrize("spec", [
+    # conv -> pool -> act, ragged width of the 32-column tiles, partial channel tile
+    [("conv", 40, 12, 3, 5, 20, True), ("maxpool", 40, 12, 20, 2), ("act", "tanh"), ("fc", 20 * 20 * 6, 10)],
+    # conv -> act -> pool (the pool reads the activation), two channel tiles, valid padding
+    [("conv", 14, 18, 2, 3, 40, False), ("act", "relu"), ("maxpool", 12, 16, 40, 2), ("fc", 40 * 6 * 8, 10)],
+    # conv -> pool without any activation, one input channel
+    [("conv", 36, 8, 1, 5, 6, True), ("maxpool", 36, 8, 6, 2), ("fc", 6 * 18 * 4, 10)],
+    # conv -> act -> pool -> act
+    [("conv", 16, 16, 3, 3, 33, True), ("act", "sigmoid"), ("maxpool", 16, 16, 33, 2), ("act", "relu"),
+     ("fc", 33 * 64, 10)],
+])
+def test_first_conv_with_pool_in_its_kernel_matches_oracle(T, O, W, spec):
+    """The first convolution of a fusing net also computes the 2x2 max-pool (and the activations)
+    behind it: every layer output, the argmax records (bit-exact) and all gradients against the
+    oracle, and the same net without fusion gives the same outputs."""
+    batch = 5
+    rng = np.random.default_rng(len(spec) * 131 + spec[0][1])
+    nets = [T.Net(W.build_layers(T, spec), batch, f) for f in (0, T.NET_FUSE_ACT_GRAD)]
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for i, l in enumerate(spec):
+        nw, nb, fan_in, _ = W.layer_fans(l)
+        if nw:
+            w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+            b = rng.uniform(-0.5, 0.5, nb).astype(np.float32)
+            for net in nets:
+                net.set_param(i, 0, w); net.set_param(i, 1, b)
+            ref.weight(i)[:] = w; ref.bias(i)[:] = b
+    first = spec[0]
+    x = rng.standard_normal((batch, first[1] * first[2] * first[3])).astype(np.float32)
+    t = rng.uniform(0.1, 0.9, (batch, 10)).astype(np.float32)
+    xd, td = T.to_device(x), T.to_device(t)
+    ref.train_step(O.opt_desc("sgd"), "mse", x, t, do_update=False)
+    for net in nets:
+        net.train_step(None, "mse", batch, xd, td, do_update=False)
+        for i, l in enumerate(spec):
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+            if l[0] == "maxpool":
+                assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64), ref.layer_argmax(i, batch))
+            if net.param_size(i, 0):
+                assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
+                assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")
+        assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, "input gradient")
+    for i in range(len(spec)):
+        assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
+    for net in nets:
+        net.close()
+
+
 def test_feeder_double_buffered_batches_match_oracle(T, O, W):
     """tdh_feeder_*: different host batches every step, a short last batch, graph replay from
     the two alternating device slots; updated weights against the oracle after every step."""

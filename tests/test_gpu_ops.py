@@ -43,6 +43,10 @@ CONV = [
     (26, 26, 16, 3, 32, True, 1, 32), (14, 14, 16, 5, 32, True, 1, 64), (16, 16, 16, 3, 30, True, 1, 64),
     # direct small-Cin forward kernel: ragged tiles, one and two channel blocks
     (20, 17, 3, 3, 40, True, 1, 3), (23, 22, 1, 5, 33, False, 1, 2), (37, 9, 3, 5, 64, True, 1, 2),
+    # small-Cin dW + db kernel: strides, several bands with a ragged last one, partial and
+    # several output-channel tiles, one to three column tiles
+    (16, 16, 3, 3, 8, True, 2, 4), (19, 14, 2, 5, 33, False, 2, 3), (64, 64, 3, 5, 16, True, 1, 2),
+    (32, 37, 3, 3, 70, True, 1, 5), (32, 32, 3, 5, 32, True, 1, 128), (28, 28, 2, 5, 6, True, 1, 40),
 ]
 
 

@@ -84,6 +84,7 @@ struct ProfRecord {
   double work;
   WorkUnit unit;
   hipEvent_t start, stop;
+  bool started = false, launched = false;
 };
 struct ProfEntry {
   std::string tag;
@@ -92,6 +93,7 @@ struct ProfEntry {
   int unit = 0;
 };
 bool g_profiling = false;
+int g_open_scope = -1;  // index into g_records of the innermost open ProfScope
 std::vector<ProfRecord> g_records;
 std::vector<hipEvent_t> g_event_pool;
 std::vector<ProfEntry> g_entries;
@@ -111,26 +113,40 @@ hipEvent_t take_event() {
 static int open_record(const std::string &tag, double work, WorkUnit unit) {
   ProfRecord r{tag, work, unit, take_event(), take_event()};
   if (!r.start || !r.stop) return -1;
-  (void)hipEventRecord(r.start, ctx().stream);
   g_records.push_back(r);
   return static_cast<int>(g_records.size()) - 1;
 }
 
 bool profiling_active() { return g_profiling; }
 
-ProfScope::ProfScope(const char *tag, double work, WorkUnit unit) : slot(-1) {
-  if (g_profiling) slot = open_record(tag, work, unit);
+ProfScope::ProfScope(const char *tag, double work, WorkUnit unit) : slot(-1), outer(g_open_scope) {
+  if (!g_profiling) return;
+  slot = open_record(tag, work, unit);
+  g_open_scope = slot;
 }
 
-ProfScope::ProfScope(const char *tag, int m, int n, int k) : slot(-1) {
+ProfScope::ProfScope(const char *tag, int m, int n, int k) : slot(-1), outer(g_open_scope) {
   if (!g_profiling) return;
   char buf[160];
   std::snprintf(buf, sizeof(buf), "%s m=%d,n=%d,k=%d", tag, m, n, k);
   slot = open_record(buf, 2.0 * m * n * k, WORK_FLOP);
+  g_open_scope = slot;
 }
 
 ProfScope::~ProfScope() {
-  if (slot >= 0) (void)hipEventRecord(g_records[slot].stop, ctx().stream);
+  if (g_profiling) g_open_scope = outer;
+}
+
+hipEvent_t prof_launch_start() {
+  if (!g_profiling || g_open_scope < 0 || g_records[g_open_scope].started) return nullptr;
+  g_records[g_open_scope].started = true;
+  return g_records[g_open_scope].start;
+}
+
+hipEvent_t prof_launch_stop() {
+  if (!g_profiling || g_open_scope < 0) return nullptr;
+  g_records[g_open_scope].launched = true;
+  return g_records[g_open_scope].stop;
 }
 
 // tiny_dnn/util/util.h:329-344
@@ -344,7 +360,8 @@ int tdh_profile_begin(void) {
   }
   g_records.clear();
   g_entries.clear();
-  g_profiling = true;
+  g_open_scope = -1;
+  g_profiling  = true;
   return TDH_OK;
 }
 
@@ -353,8 +370,14 @@ int tdh_profile_end(int32_t *n_entries) {
   g_profiling = false;
   TDH_HIP(hipStreamSynchronize(ctx().stream));
   std::map<std::string, ProfEntry> by_tag;
+  g_open_scope = -1;
   for (auto &r : g_records) {
     float ms = 0.0f;
+    if (!r.launched) {  // a scope that launched nothing (its work was deferred or empty)
+      g_event_pool.push_back(r.start);
+      g_event_pool.push_back(r.stop);
+      continue;
+    }
     TDH_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
     ProfEntry &e = by_tag[r.tag];
     e.tag        = r.tag;

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -91,8 +92,23 @@ struct ProfScope {
   // GEMM launches carry their shape in the tag: "name m=..,n=..,k=.."
   ProfScope(const char *tag, int m, int n, int k);
   ~ProfScope();
-  int slot;
+  int slot, outer;
 };
+bool profiling_active();
+// The duration of a profiled scope comes from the dispatches themselves: while a scope is
+// open, TDH_LAUNCH hands its events to hipExtLaunchKernelGGL, which stamps them with the
+// start of the scope's first kernel and the end of its last one. (Events recorded around a
+// launch would add the latency of their own packets, a few microseconds per kernel.)
+hipEvent_t prof_launch_start();
+hipEvent_t prof_launch_stop();
+#define TDH_LAUNCH(kernel, grid, block, shmem, stream, ...)                                  \
+  do {                                                                                       \
+    if (::tdh::profiling_active())                                                           \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, ::tdh::prof_launch_start(),  \
+                            ::tdh::prof_launch_stop(), 0, __VA_ARGS__);                       \
+    else                                                                                     \
+      hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                   \
+  } while (0)
 
 // ---------------------------------------------------------------- helpers
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -154,7 +170,7 @@ struct OptTensor {
   uint32_t C, Kc, rs;
 };
 constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 4096;
-// dev_powers: NULL, or two device floats {b1_t, b2_t} that the kernel reads instead of the
+// dev_powers: NULL, or device floats {b1_t, b2_t, ticket (zero), unused} that the kernel reads instead of the
 // host values and that a follow-up kernel advances n_tensors times (graph replay).
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
@@ -166,6 +182,16 @@ int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, i
 // launch what was recorded on the current stream (launch = false: forget it)
 int flush_deferred_rowsums(bool launch = true);   // elementwise.hip
 int flush_deferred_reduces(bool launch = true);   // conv.hip
+// conv_dw_small.hip: dW (+ db) of a convolution with few input channels
+bool conv_dw_small_applicable(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
+                              int sh, int sw, int dh, int dw, int ph, int pw);
+size_t conv_dw_small_workspace_bytes(int batch, int C, int Kc, int H, int W, int OH, int OW, int R,
+                                     int S, int sh, int sw, int dh, int dw, int ph, int pw);
+int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy, float *dw_out,
+                      float *db_out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
+                      int dw, int ph, int pw, int accumulate);
+// the weight-gradient kernel of this layer also produces the bias gradient when asked for both
+bool conv_dw_gives_db(const tdh_conv_desc *d, int batch);
 // norm.hip
 size_t batchnorm_workspace_bytes(int channels, int batch);
 int batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, const float *x,
@@ -188,9 +214,25 @@ struct ActGrad {
 
 // conv.hip / fc.hip
 // prepacked: filters already packed by conv_pack_filters for this direction (and only then)
+// A 2x2 / stride-2 max-pool layer (and the pointwise activation behind it) computed by the
+// forward kernel of the layer in front of it
+struct PoolFuse {
+  float *out;
+  int32_t *argmax;
+  float *act_out;  // or null
+  int act_kind;
+};
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
                float *y, const uint8_t *tbl_resident = nullptr, const float *prepacked = nullptr,
-               float *act_out = nullptr, int act_kind = 0);
+               float *act_out = nullptr, int act_kind = 0, const PoolFuse *pool = nullptr);
+// the forward kernel of this convolution can also compute the max-pool layer `pool` behind it
+bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked);
+// conv_fwd_small.hip
+bool conv_fwd_small_applicable(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
+                               int sh, int sw, int dh, int dw, int ph, int pw);
+int conv_fwd_small_run(int batch, int C, int Kc, const float *x, const float *w, const float *bias,
+                       float *out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
+                       int dw, int ph, int pw, float *act_out, int act_kind, const PoolFuse *pool);
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
                const uint8_t *tbl_resident = nullptr, const float *prepacked_dx = nullptr);

@@ -403,172 +403,17 @@ static void launch_small_cin_dx(const ConvGeom &g, const DxsPlan &p, int batch, 
                                 const float *w, float *dx, ActGrad ag) {
   const dim3 grid(batch * p.bands), block(DXS_NT);
   switch (KR ? g.C : DXS_MAX_CIN) {
-    case 1: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 1>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
-    case 2: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 2>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
-    case 3: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 3>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
-    default: hipLaunchKernelGGL((conv_dx_small_cin_kernel<KR, KS, 4>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    case 1: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 1>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    case 2: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 2>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    case 3: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 3>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    default: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 4>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
   }
 }
 
 
-// Forward for convolutions with very few input channels (the first layer of an image network),
-// stride 1: the whole reduction is K = Cin*R*S <= 100 deep, so nothing is chunked. M = output
-// channels, N = pixels, K = (ci, fy, fx). A lane keeps its filter values for every k pair in
-// registers for the whole kernel (A operand: m = l%32, k = 2p + l/32), the input patch of the
-// pixel tile (with halo, zero outside the image) sits in LDS once, and the B operand of pair p
-// is one ds_read at a compile-time offset from the lane's pixel. A workgroup of four waves
-// owns FSC_TN*4 rows x 32 columns of one image; wave w takes rows w*FSC_TN ...
-constexpr int FSC_TC = 32;  // tile columns = pixels of one MFMA block
-constexpr int FSC_TN = 2;   // 32-pixel row blocks per wave
-constexpr int FSC_TR = 4 * FSC_TN;
-
-struct FwdSmallCinArgs {
-  const float *x, *w, *bias;
-  float *y;
-  float *act_out;  // act(y) of the pointwise activation layer that follows, or NULL
-  int act_kind;
-  int batch, Kc, H, W, OH, OW, ph, pw;
-  int tiles_x, tiles_y;
-};
-
-template <int R, int S, int CIN, int MB>
-__global__ void __launch_bounds__(256)
-conv_fwd_small_cin_kernel(const FwdSmallCinArgs a) {
-  constexpr int KTOT  = CIN * R * S;
-  constexpr int KP    = (KTOT + 1) / 2;  // MFMA k pairs
-  constexpr int PITCH = FSC_TC + S - 1;
-  constexpr int ROWS  = FSC_TR + R - 1;
-  constexpr int PLANE = ROWS * PITCH;
-  __shared__ float patch[CIN * PLANE];
-  __shared__ float wl[32 * MB * KTOT];  // the filters as they lie in memory: [co][k]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
-  int bt       = blockIdx.x;
-  const int tx = bt % a.tiles_x;
-  bt /= a.tiles_x;
-  const int ty  = bt % a.tiles_y;
-  const int img = bt / a.tiles_y;
-  const int x0 = tx * FSC_TC, y0 = ty * FSC_TR;
-
-  // ---- input patch with halo
-  const float *xin = a.x + static_cast<size_t>(img) * CIN * a.H * a.W;
-  constexpr int NE = (CIN * PLANE + 255) / 256;  // every load is in flight before the first store
-  float staged[NE];
-#pragma unroll
-  for (int i = 0; i < NE; ++i) {
-    const int e  = tid + 256 * i;
-    const int ci = e / PLANE, rem = e - ci * PLANE;
-    const int r = rem / PITCH, c = rem - r * PITCH;
-    const int iy = y0 - a.ph + r, ix = x0 - a.pw + c;
-    const bool ok = e < CIN * PLANE && static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) &&
-                    static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
-    staged[i] = ok ? xin[(ci * a.H + iy) * a.W + ix] : 0.0f;
-  }
-  // the filters come in with coalesced loads; a lane then picks its fragments out of LDS
-  // (rows KTOT apart: an odd stride, no bank conflicts)
-  constexpr int NWL = (32 * MB * KTOT + 255) / 256;
-  float wstaged[NWL];
-#pragma unroll
-  for (int i = 0; i < NWL; ++i) {
-    const int e = tid + 256 * i;
-    wstaged[i]  = (e < 32 * MB * KTOT && e < a.Kc * KTOT) ? a.w[e] : 0.0f;
-  }
-#pragma unroll
-  for (int i = 0; i < NE; ++i)
-    if (tid + 256 * i < CIN * PLANE) patch[tid + 256 * i] = staged[i];
-#pragma unroll
-  for (int i = 0; i < NWL; ++i)
-    if (tid + 256 * i < 32 * MB * KTOT) wl[tid + 256 * i] = wstaged[i];
-  __syncthreads();
-
-  // ---- filter fragments: af[mb][p] = w[co = 32*mb + l%32][k = 2p + l/32]
-  float af[MB][KP];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int co = 32 * mb + (lane & 31);
-#pragma unroll
-    for (int p = 0; p < KP; ++p) {
-      const int k = 2 * p + half;
-      af[mb][p]   = k < KTOT ? wl[co * KTOT + k] : 0.0f;
-    }
-  }
-
-  floatx16 acc[MB][FSC_TN];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int j = 0; j < FSC_TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][j][r] = 0.0f;
-
-  const float *bp = patch + (wave * FSC_TN) * PITCH + (lane & 31);
-#pragma unroll
-  for (int p = 0; p < KP; ++p) {
-    // patch offset of k = 2p (+1 for the upper half of the wave); a k beyond KTOT has a zero filter
-    constexpr int RS = R * S;
-    const int k0 = 2 * p, k1 = 2 * p + 1 < KTOT ? 2 * p + 1 : 2 * p;
-    const int off0 = (k0 / RS) * PLANE + ((k0 % RS) / S) * PITCH + (k0 % RS) % S;
-    const int off1 = (k1 / RS) * PLANE + ((k1 % RS) / S) * PITCH + (k1 % RS) % S;
-    const int off  = half ? off1 : off0;
-#pragma unroll
-    for (int j = 0; j < FSC_TN; ++j) {
-      const float bf = bp[j * PITCH + off];
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        acc[mb][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mb][p], bf, acc[mb][j], 0, 0, 0);
-    }
-  }
-
-  // ---- reg r of lane l: channel 8*(r/4) + 4*(l/32) + r%4 (+32*mb), pixel l%32 of row block j
-  const int ohw = a.OH * a.OW;
-  const int ox  = x0 + (lane & 31);
-#pragma unroll
-  for (int j = 0; j < FSC_TN; ++j) {
-    const int oy = y0 + wave * FSC_TN + j;
-    if (oy >= a.OH || ox >= a.OW) continue;
-    float *out = a.y + static_cast<size_t>(img) * a.Kc * ohw + oy * a.OW + ox;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int co = 32 * mb + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (co >= a.Kc) continue;
-        const float v = acc[mb][j][r] + (a.bias ? a.bias[co] : 0.0f);
-        out[static_cast<size_t>(co) * ohw] = v;
-        if (a.act_out) a.act_out[(out - a.y) + static_cast<size_t>(co) * ohw] = act_apply(a.act_kind, v);
-      }
-  }
-}
-
-static bool small_cin_fwd_applies(const ConvGeom &g) {
-  if (g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1 || g.Kc > 64 || g.OW < 16) return false;
-  return (g.R == 5 && g.S == 5 && (g.C == 3 || g.C == 1)) || (g.R == 3 && g.S == 3 && (g.C == 3 || g.C == 1));
-}
-
-static int launch_small_cin_fwd(const ConvGeom &g, int batch, const float *x, const float *w,
-                                const float *bias, float *y, float *act_out, int act_kind) {
-  FwdSmallCinArgs a;
-  a.x = x; a.w = w; a.bias = bias; a.y = y;
-  a.act_out = act_out; a.act_kind = act_kind;
-  a.batch = batch; a.Kc = g.Kc; a.H = g.H; a.W = g.W; a.OH = g.OH; a.OW = g.OW; a.ph = g.pad_h; a.pw = g.pad_w;
-  a.tiles_x = ceil_div(g.OW, FSC_TC);
-  a.tiles_y = ceil_div(g.OH, FSC_TR);
-  const long blocks = static_cast<long>(a.tiles_x) * a.tiles_y * batch;
-  TDH_CHECK_ARG(blocks < (1L << 31), "convolution forward: too many tiles");
-  const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-  ProfScope prof("conv_fwd_small_cin", g.Kc, batch * g.OH * g.OW, g.C * g.R * g.S);
-#define TDH_FSC(R_, S_, C_)                                                                       \
-  if (g.Kc > 32)                                                                                  \
-    hipLaunchKernelGGL((conv_fwd_small_cin_kernel<R_, S_, C_, 2>), grid, block, 0, ctx().stream, a); \
-  else                                                                                            \
-    hipLaunchKernelGGL((conv_fwd_small_cin_kernel<R_, S_, C_, 1>), grid, block, 0, ctx().stream, a)
-  if (g.R == 5 && g.C == 3) { TDH_FSC(5, 5, 3); }
-  else if (g.R == 5) { TDH_FSC(5, 5, 1); }
-  else if (g.C == 3) { TDH_FSC(3, 3, 3); }
-  else { TDH_FSC(3, 3, 1); }
-#undef TDH_FSC
-  TDH_LAUNCH_CHECK();
-  return TDH_OK;
+static bool fwd_small_applies(const ConvGeom &g, int batch) {
+  return conv_fwd_small_applicable(batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw, g.dh,
+                                   g.dw, g.pad_h, g.pad_w);
 }
 
 }  // namespace
@@ -582,6 +427,8 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   total += gemm_workspace_bytes(g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true);  // dX
   total += rowsum_workspace_bytes(batch, g.Kc, ohw);                  // db
   if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
+  total += conv_dw_small_workspace_bytes(batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw,
+                                         g.dh, g.dw, g.pad_h, g.pad_w);
   if (g.sh == 1 && g.sw == 1)
     total += conv_dw_halo_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
   if (g.sh == 1 && g.sw == 1) {  // LDS-halo kernel: repacked filters and split partial sums
@@ -615,7 +462,7 @@ static int prepare_table(const tdh_conv_desc *d, const ConvGeom &g, const float 
     TDH_HIP(hipStreamSynchronize(ctx().stream));
   }
   ProfScope prof("conv_mask_weights", 8.0 * nw, WORK_BYTE);
-  hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(nw, 256)), dim3(256), 0, ctx().stream, w,
+  TDH_LAUNCH(mask_weights_kernel, dim3(ceil_div(nw, 256)), dim3(256), 0, ctx().stream, w,
                      static_cast<const uint8_t *>(t), static_cast<float *>(wm), nw, g.C, g.Kc,
                      g.R * g.S, 0);
   TDH_LAUNCH_CHECK();
@@ -655,7 +502,7 @@ int flush_deferred_reduces(bool launch) {
     }
     jobs.first_block[jobs.n] = blocks;
     ProfScope prof("conv_dw_splitk_reduce_multi", bytes, WORK_BYTE);
-    hipLaunchKernelGGL(splitk_reduce_multi_kernel, dim3(blocks), dim3(256), 0, ctx().stream, jobs);
+    TDH_LAUNCH(splitk_reduce_multi_kernel, dim3(blocks), dim3(256), 0, ctx().stream, jobs);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       all.clear();
@@ -672,15 +519,29 @@ bool defer_reduce(const float *partial, int splits, int M, int N, const EpiRowMa
   return true;
 }
 
+static bool dw_small_applies(const tdh_conv_desc *d, const ConvGeom &g, int batch) {
+  return !d->tbl && conv_dw_small_applicable(batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw,
+                                             g.dh, g.dw, g.pad_h, g.pad_w);
+}
+
+bool conv_dw_gives_db(const tdh_conv_desc *d, int batch) { return dw_small_applies(d, make_geom(d), batch); }
+
 bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked) {
-  return prepacked ? conv_uses_packed(d, batch, 0) : small_cin_fwd_applies(make_geom(d));
+  return prepacked ? conv_uses_packed(d, batch, 0) : fwd_small_applies(make_geom(d), batch);
+}
+
+bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked) {
+  const ConvGeom g = make_geom(d);
+  if (prepacked || !fwd_small_applies(g, batch)) return false;
+  return pool->pool_w == 2 && pool->pool_h == 2 && pool->stride_w == 2 && pool->stride_h == 2 &&
+         pool->in_w == g.OW && pool->in_h == g.OH && pool->in_c == g.Kc && g.OW % 2 == 0 && g.OH % 2 == 0;
 }
 
 bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip) {
   const ConvGeom g = make_geom(d);
   if (g.sh != 1 || g.sw != 1) return false;
   if (!flip)
-    return g.dh == 1 && g.dw == 1 && !small_cin_fwd_applies(g) &&
+    return g.dh == 1 && g.dw == 1 && !fwd_small_applies(g, batch) &&
            conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
   DxsPlan dxs;
   if (small_cin_dx_plan(g, dxs)) return false;
@@ -695,20 +556,21 @@ int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const ui
 
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
                float *y, const uint8_t *tbl_resident, const float *prepacked, float *act_out,
-               int act_kind) {
+               int act_kind, const PoolFuse *pool) {
   const ConvGeom g = make_geom(d);
   if (prepacked)
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
                        g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked, act_out,
                        act_kind);
-  if (act_out && !small_cin_fwd_applies(g))
-    return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not apply a following activation");
+  if ((act_out || pool) && !fwd_small_applies(g, batch))
+    return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not apply the layers behind it");
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
-  if (small_cin_fwd_applies(g))
-    return launch_small_cin_fwd(g, batch, x, w_eff, d->has_bias ? b : nullptr, y, act_out, act_kind);
+  if (fwd_small_applies(g, batch))
+    return conv_fwd_small_run(batch, g.C, g.Kc, x, w_eff, d->has_bias ? b : nullptr, y, g.H, g.W, g.OH, g.OW,
+                              g.R, g.S, g.sh, g.sw, g.dh, g.dw, g.pad_h, g.pad_w, act_out, act_kind, pool);
   if (g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 &&
       conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w))
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w_eff, nullptr,
@@ -756,6 +618,11 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
     EpiImageRows epi{dx, g.C, g.H * g.W, g.div_hw, nullptr, dx_act};
     TDH_TRY((launch_gemm<true, false>(A, B, epi, g.C, batch * g.H * g.W, g.Kc * g.R * g.S, true, "conv_dx_gemm", "conv_dx_splitk_reduce")));
   }
+  if (dw && dw_small_applies(d, g, batch) && !(reinterpret_cast<uintptr_t>(dy) & 15)) {
+    TDH_TRY(conv_dw_small_run(batch, g.C, g.Kc, x, dy, dw, db, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw,
+                              g.dh, g.dw, g.pad_h, g.pad_w, accumulate));
+    return TDH_OK;
+  }
   if (dw) {
     DwDyOperand A{dy, g.Kc, ohw, g.div_ohw};
     DwInputOperand B{x, g, crs};
@@ -763,6 +630,12 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
                       conv_dw_halo_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW,
                                               g.pad_h, g.pad_w);
     if (tbl_dev) {
+      // the masking kernel below reads the reduced gradient: its reduction cannot wait
+      struct NoDefer {
+        bool was = ctx().defer_reduce;
+        NoDefer() { ctx().defer_reduce = false; }
+        ~NoDefer() { ctx().defer_reduce = was; }
+      } no_defer;
       void *tmp = nullptr;
       TDH_TRY(ws_take(sizeof(float) * g.Kc * crs, &tmp));
       EpiRowMajor epi{static_cast<float *>(tmp), crs, nullptr, ActGrad(), 0};
@@ -772,7 +645,7 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       else
         TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm", "conv_dw_splitk_reduce")));
       ProfScope prof("conv_mask_weights", 8.0 * g.Kc * crs, WORK_BYTE);
-      hipLaunchKernelGGL(mask_weights_kernel, dim3(ceil_div(g.Kc * crs, 256)), dim3(256), 0,
+      TDH_LAUNCH(mask_weights_kernel, dim3(ceil_div(g.Kc * crs, 256)), dim3(256), 0,
                          ctx().stream, static_cast<const float *>(tmp), tbl_dev, dw, g.Kc * crs,
                          g.C, g.Kc, g.R * g.S, accumulate);
       TDH_LAUNCH_CHECK();

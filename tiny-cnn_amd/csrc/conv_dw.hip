@@ -410,7 +410,7 @@ int launch_dw_inst(const DwHaloPlan &p) {
       raised = p.lds_bytes;
     }
   }
-  hipLaunchKernelGGL(kernel, p.grid, dim3(p.nt), p.lds_bytes, ctx().stream, p.args);
+  TDH_LAUNCH(kernel, p.grid, dim3(p.nt), p.lds_bytes, ctx().stream, p.args);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }
@@ -469,7 +469,7 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
   EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
   if (defer_reduce(p.args.partial, slices, Kc, crs, epi)) return TDH_OK;
   ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
-  hipLaunchKernelGGL((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * crs, REDUCE_OUTPUTS)),
+  TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * crs, REDUCE_OUTPUTS)),
                      dim3(256), 0, ctx().stream, p.args.partial, slices, Kc, crs, epi);
   TDH_LAUNCH_CHECK();
   return TDH_OK;

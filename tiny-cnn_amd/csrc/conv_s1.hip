@@ -171,7 +171,7 @@ size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip,
 int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const uint8_t *tbl_dev,
                    float *wp) {
   ProfScope prof("conv_repack_weights", 8.0 * R * S * C * Kc, WORK_BYTE);
-  hipLaunchKernelGGL(repack_weights_kernel, dim3(ceil_div(R * S * C * Kc, 256)), dim3(256), 0,
+  TDH_LAUNCH(repack_weights_kernel, dim3(ceil_div(R * S * C * Kc, 256)), dim3(256), 0,
                      ctx().stream, w, tbl_dev, wp, C, Kc, R * S, flip);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -214,11 +214,11 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
     ProfScope prof("conv_s1_split_reduce", 4.0 * total * (p.splits + 1 + (ag.kind != TDH_ACT_NONE)),
                    WORK_BYTE);
     if (plane % 4 == 0)
-      hipLaunchKernelGGL((s1_split_reduce_kernel<4>), dim3(static_cast<unsigned>(ceil_div_sz(total / 4, 256))), dim3(256), 0,
+      TDH_LAUNCH((s1_split_reduce_kernel<4>), dim3(static_cast<unsigned>(ceil_div_sz(total / 4, 256))), dim3(256), 0,
                          ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
                          FastDiv(plane), total, act_out, act_kind);
     else
-      hipLaunchKernelGGL((s1_split_reduce_kernel<1>), dim3(static_cast<unsigned>(ceil_div_sz(total, 256))), dim3(256), 0,
+      TDH_LAUNCH((s1_split_reduce_kernel<1>), dim3(static_cast<unsigned>(ceil_div_sz(total, 256))), dim3(256), 0,
                          ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
                          FastDiv(plane), total, act_out, act_kind);
     TDH_LAUNCH_CHECK();

@@ -302,7 +302,7 @@ int launch_s1_inst(const S1Plan &p) {
       raised = p.lds_bytes;
     }
   }
-  hipLaunchKernelGGL(kernel, p.grid, dim3(256), p.lds_bytes, ctx().stream, p.args);
+  TDH_LAUNCH(kernel, p.grid, dim3(256), p.lds_bytes, ctx().stream, p.args);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }

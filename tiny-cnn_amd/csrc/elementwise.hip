@@ -50,7 +50,7 @@ int launch_map(const float *a, const float *b, float *out, size_t n,
   ProfScope prof(tag, (HAS_B ? 12.0 : 8.0) * n, WORK_BYTE);
   const bool vec  = aligned16(a) && aligned16(out) && (!HAS_B || aligned16(b));
   const size_t n4 = vec ? n / 4 : 0;
-  hipLaunchKernelGGL((map_kernel<Op, HAS_B>), dim3(ew_blocks(vec ? n4 + 3 : n)), dim3(EW_THREADS),
+  TDH_LAUNCH((map_kernel<Op, HAS_B>), dim3(ew_blocks(vec ? n4 + 3 : n)), dim3(EW_THREADS),
                      0, ctx().stream, a, b, out, n4, n, prm);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -396,7 +396,7 @@ int launch_opt(size_t n, const float *g, float *w, float *s0, float *s1, const O
   const bool vec = aligned16(g) && aligned16(w) && (NSTATE < 1 || aligned16(s0)) &&
                    (NSTATE < 2 || aligned16(s1));
   const size_t n4 = vec ? n / 4 : 0;
-  hipLaunchKernelGGL((opt_kernel<KIND, NSTATE>), dim3(ew_blocks(vec ? n4 + 3 : n)),
+  TDH_LAUNCH((opt_kernel<KIND, NSTATE>), dim3(ew_blocks(vec ? n4 + 3 : n)),
                      dim3(EW_THREADS), 0, ctx().stream, g, w, s0, s1, n4, n, p);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -415,7 +415,7 @@ __device__ __forceinline__ void opt_pack_store(const OptTensor &t, const uint32_
 template <int KIND, int NSTATE>
 __global__ void __launch_bounds__(EW_THREADS)
 opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptScalars p,
-                 float b1_t, float b2_t, const float *__restrict__ dev_powers,
+                 float b1_t, float b2_t, float *dev_powers, const int advance,
                  const int zero_grad) {
   if (dev_powers) {
     b1_t = dev_powers[0];
@@ -469,19 +469,27 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
     if (NSTATE >= 2) t.s1[i] = b;
     if (zero_grad) t.g[i] = 0.0f;
   }
-}
-
-// advances the device copy of the bias-correction powers as n update() calls would
-__global__ void opt_advance_powers_kernel(float *powers, const int n, const float b1,
-                                          const float b2, const int adam) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  float p1 = powers[0], p2 = powers[1];
-  for (int i = 0; i < n; ++i) {
-    p1 *= b1;
-    if (adam) p2 *= b2;
+  // The device copy of the powers advances as n_tensors update() calls would. The workgroup
+  // that draws the last ticket does it: by then every workgroup has read the old values.
+  // advance: 0 = leave them, 1 = b1_t only (adamax), 2 = both (adam).
+  if (advance) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned int *ticket = reinterpret_cast<unsigned int *>(dev_powers + 2);
+      const unsigned int drawn =
+          __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (drawn == gridDim.x - 1) {
+        float q1 = b1_t, q2 = b2_t;
+        for (int i = 0; i < n_tensors; ++i) {
+          q1 *= p.b1;
+          if (advance == 2) q2 *= p.b2;
+        }
+        dev_powers[0] = q1;
+        dev_powers[1] = q2;
+        __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
   }
-  powers[0] = p1;
-  powers[1] = p2;
 }
 
 // ---------------------------------------------------------------- reductions
@@ -598,7 +606,7 @@ int launch_fill_zero(void *p, size_t bytes) {
   ProfScope prof("fill_zero", static_cast<double>(bytes), WORK_BYTE);
   const size_t n  = bytes / 4;
   const size_t n4 = aligned16(p) ? n / 4 : 0;
-  hipLaunchKernelGGL(fill_zero_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0,
+  TDH_LAUNCH(fill_zero_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0,
                      ctx().stream, static_cast<uint32_t *>(p), n4, n);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -608,7 +616,7 @@ int launch_copy(void *dst, const void *src, size_t bytes) {
   ProfScope prof("copy", 2.0 * static_cast<double>(bytes), WORK_BYTE);
   const size_t n  = bytes / 4;
   const size_t n4 = (aligned16(dst) && aligned16(src)) ? n / 4 : 0;
-  hipLaunchKernelGGL(copy_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0, ctx().stream,
+  TDH_LAUNCH(copy_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0, ctx().stream,
                      static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), n4, n);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -630,7 +638,7 @@ int launch_act_fwd(int kind, const float *p, int batch, int len, const float *x,
     case TDH_ACT_SIGMOID: return launch_map<SigmoidFwd, false>(x, nullptr, y, n, NoParams(), "act_fwd_sigmoid");
     case TDH_ACT_SOFTMAX: {
       ProfScope prof("act_fwd_softmax", 8.0 * n, WORK_BYTE);
-      hipLaunchKernelGGL(softmax_fwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
+      TDH_LAUNCH(softmax_fwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
                          dim3(EW_THREADS), 0, ctx().stream, x, y, batch, len);
       TDH_LAUNCH_CHECK();
       return TDH_OK;
@@ -658,7 +666,7 @@ int launch_act_bwd(int kind, const float *p, int batch, int len, const float *x,
     case TDH_ACT_SIGMOID: return launch_map<SigmoidBwd, true>(y, dy, dx, n, NoParams(), "act_grad_sigmoid");
     case TDH_ACT_SOFTMAX: {
       ProfScope prof("act_grad_softmax", 12.0 * n, WORK_BYTE);
-      hipLaunchKernelGGL(softmax_bwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
+      TDH_LAUNCH(softmax_bwd_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
                          dim3(EW_THREADS), 0, ctx().stream, y, dy, dx, batch, len);
       TDH_LAUNCH_CHECK();
       return TDH_OK;
@@ -683,7 +691,7 @@ int launch_loss_grad(int kind, int batch, int len, const float *y, const float *
 
 int launch_softmax_fwd_xent(int batch, int len, const float *x, const float *t, float *y, float *dz) {
   ProfScope prof("softmax_fwd_xent_grad", 20.0 * batch * len, WORK_BYTE);
-  hipLaunchKernelGGL(softmax_fwd_xent_kernel, dim3(ceil_div(batch, EW_THREADS / 64)), dim3(EW_THREADS),
+  TDH_LAUNCH(softmax_fwd_xent_kernel, dim3(ceil_div(batch, EW_THREADS / 64)), dim3(EW_THREADS),
                      0, ctx().stream, x, t, y, dz, batch, len);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -691,7 +699,7 @@ int launch_softmax_fwd_xent(int batch, int len, const float *x, const float *t, 
 
 int launch_softmax_xent_grad(int batch, int len, const float *y, const float *t, float *dz) {
   ProfScope prof("softmax_xent_grad", 12.0 * batch * len, WORK_BYTE);
-  hipLaunchKernelGGL(softmax_xent_grad_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
+  TDH_LAUNCH(softmax_xent_grad_kernel, dim3(ceil_div(batch, EW_THREADS / 64)),
                      dim3(EW_THREADS), 0, ctx().stream, y, t, dz, batch, len);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -763,10 +771,11 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
   // gradient read (+ cleared), weight read+write, states read+write
   ProfScope prof(tags[o->kind], (12.0 + 8.0 * nstate + (zero_grad ? 4.0 : 0.0)) * total_params,
                  WORK_BYTE);
+  const int advance = !dev_powers ? 0 : o->kind == TDH_OPT_ADAM ? 2 : o->kind == TDH_OPT_ADAMAX ? 1 : 0;
 #define TDH_LAUNCH_MULTI(KIND, NS)                                                            \
-  hipLaunchKernelGGL((opt_multi_kernel<KIND, NS>), dim3(total_blocks), dim3(EW_THREADS), 0,   \
+  TDH_LAUNCH((opt_multi_kernel<KIND, NS>), dim3(total_blocks), dim3(EW_THREADS), 0,   \
                      ctx().stream, dev_table, n_tensors, p, o->b1_t, o->b2_t,                  \
-                     static_cast<const float *>(dev_powers), zero_grad)
+                     dev_powers, advance, zero_grad)
   switch (o->kind) {
     case TDH_OPT_SGD: TDH_LAUNCH_MULTI(TDH_OPT_SGD, 0); break;
     case TDH_OPT_MOMENTUM: TDH_LAUNCH_MULTI(TDH_OPT_MOMENTUM, 1); break;
@@ -778,11 +787,6 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
   }
 #undef TDH_LAUNCH_MULTI
   TDH_LAUNCH_CHECK();
-  if (dev_powers && (o->kind == TDH_OPT_ADAM || o->kind == TDH_OPT_ADAMAX)) {
-    hipLaunchKernelGGL(opt_advance_powers_kernel, dim3(1), dim3(64), 0, ctx().stream, dev_powers,
-                       n_tensors, o->b1, o->b2, o->kind == TDH_OPT_ADAM ? 1 : 0);
-    TDH_LAUNCH_CHECK();
-  }
   for (int j = 0; j < n_tensors; ++j) {
     if (o->kind == TDH_OPT_ADAM) {
       o->b1_t *= o->b1;
@@ -818,10 +822,10 @@ int flush_deferred_rowsums(bool launch) {
     jobs.first1[jobs.n] = b1;
     jobs.first2[jobs.n] = b2;
     ProfScope prof("bias_grad_rowsum_multi", bytes, WORK_BYTE);
-    hipLaunchKernelGGL(rowsum_multi_stage1_kernel, dim3(b1), dim3(EW_THREADS), 0, ctx().stream, jobs);
+    TDH_LAUNCH(rowsum_multi_stage1_kernel, dim3(b1), dim3(EW_THREADS), 0, ctx().stream, jobs);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess) {
-      hipLaunchKernelGGL(rowsum_multi_stage2_kernel, dim3(b2), dim3(EW_THREADS), 0, ctx().stream,
+      TDH_LAUNCH(rowsum_multi_stage2_kernel, dim3(b2), dim3(EW_THREADS), 0, ctx().stream,
                          jobs);
       e = hipGetLastError();
     }
@@ -844,10 +848,10 @@ int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, i
     return TDH_OK;
   }
   ProfScope prof("bias_grad_rowsum", 4.0 * outer * rows * cols, WORK_BYTE);
-  hipLaunchKernelGGL(rowsum_stage1_kernel, dim3(rows, groups), dim3(EW_THREADS), 0, ctx().stream,
+  TDH_LAUNCH(rowsum_stage1_kernel, dim3(rows, groups), dim3(EW_THREADS), 0, ctx().stream,
                      src, outer, rows, cols, groups, static_cast<float *>(ws));
   TDH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(rowsum_stage2_kernel, dim3(ceil_div(rows, EW_THREADS / 64)), dim3(EW_THREADS),
+  TDH_LAUNCH(rowsum_stage2_kernel, dim3(ceil_div(rows, EW_THREADS / 64)), dim3(EW_THREADS),
                      0, ctx().stream, static_cast<const float *>(ws), rows, groups, out, accumulate);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -855,7 +859,7 @@ int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, i
 
 int launch_colsum(const float *src, int rows, int cols, float *out, int accumulate) {
   ProfScope prof("bias_grad_colsum", 4.0 * rows * cols, WORK_BYTE);
-  hipLaunchKernelGGL(colsum_kernel, dim3(ceil_div(cols, 32)), dim3(EW_THREADS), 0,
+  TDH_LAUNCH(colsum_kernel, dim3(ceil_div(cols, 32)), dim3(EW_THREADS), 0,
                      ctx().stream, src, rows, cols, out, accumulate);
   TDH_LAUNCH_CHECK();
   return TDH_OK;

@@ -145,7 +145,7 @@ template <class Epi>
 int launch_small_fc(const StridedOperand &a, const StridedOperand &b, const Epi &epi, int M, int N,
                     int K, const char *tag) {
   ProfScope prof(tag, M, N, K);
-  hipLaunchKernelGGL((small_fc_gemm_kernel<Epi>), dim3(ceil_div(N, SFC_TN), ceil_div(M, SFC_TM)),
+  TDH_LAUNCH((small_fc_gemm_kernel<Epi>), dim3(ceil_div(N, SFC_TN), ceil_div(M, SFC_TM)),
                      dim3(SFC_NT), 0, ctx().stream, a, b, epi, M, N, K);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -198,7 +198,7 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     const bool bias = db && has_bias;
     f.dy = dy; f.db = db; f.batch = batch; f.out = out; f.db_accumulate = accumulate;
     ProfScope prof("fc_bwd_small", 4.0 * batch * in * out, WORK_FLOP);
-    hipLaunchKernelGGL(fc_bwd_fused_kernel, dim3(f.nx + f.nw + (bias ? ceil_div(out, 32) : 0)),
+    TDH_LAUNCH(fc_bwd_fused_kernel, dim3(f.nx + f.nw + (bias ? ceil_div(out, 32) : 0)),
                        dim3(SFC_NT), 0, ctx().stream, f);
     TDH_LAUNCH_CHECK();
     return TDH_OK;

@@ -592,7 +592,7 @@ int launch_gemm_tile(const AOp &a, const BOp &b, const Epi &epi, int M, int N, i
                      const GemmPlan &p, float *partial, const char *tag) {
   ProfScope prof(tag, M, N, K);
   dim3 grid(ceil_div(N, BN), ceil_div(M, BM), p.splits);
-  hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, A_VEC, B_VEC, AOp, BOp,
+  TDH_LAUNCH((gemm_mfma_kernel<BM, BN, WM, WN, A_LANE_K, B_LANE_K, A_VEC, B_VEC, AOp, BOp,
                                        Epi>), grid,
                      dim3(64 * WM * WN), 0, ctx().stream, a, b, epi, M, N, K, p.k_per_split,
                      partial);
@@ -639,7 +639,7 @@ int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
     // reads every partial tile once and writes the result once
     if (defer_reduce(partial, p.splits, M, N, epi)) return TDH_OK;
     ProfScope prof(reduce_tag, 4.0 * M * N * (p.splits + 1), WORK_BYTE);
-    hipLaunchKernelGGL((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, REDUCE_OUTPUTS)), dim3(256), 0,
+    TDH_LAUNCH((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, REDUCE_OUTPUTS)), dim3(256), 0,
                        ctx().stream, partial, p.splits, M, N, epi);
     TDH_LAUNCH_CHECK();
   }

@@ -32,7 +32,7 @@ struct tdh_net {
   int opt_tensors = 0, opt_blocks = 0;
   double opt_params = 0.0;
   // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
-  float *dev_powers = nullptr;          // {b1_t, b2_t} as the captured optimizer kernel reads them
+  float *dev_powers = nullptr;          // {b1_t, b2_t, ticket} as the captured optimizer kernel uses them
   struct GraphKey {
     int batch = 0, loss = 0, do_update = 0;
     const float *x = nullptr, *t = nullptr;
@@ -147,15 +147,36 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
         TDH_TRY(ws_begin(conv2d_workspace_bytes(&s.conv, batch)));
       {
         const float *wp = packed && L.wp_fwd && conv_uses_packed(&s.conv, batch, 0) ? L.wp_fwd : nullptr;
-        if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
-            is_pointwise_act(net->layers[i + 1].spec.act) && conv_fwd_applies_act(&s.conv, batch, wp != nullptr)) {
-          // the activation layer behind the convolution leaves the same kernel
-          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp, net->layers[i + 1].out,
-                             net->layers[i + 1].spec.act));
-          ++i;
-        } else {
-          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp));
+        const bool fuse = (net->flags & TDH_NET_FUSE_ACT_GRAD) != 0;
+        auto pointwise = [&](int k) {
+          return k < n && net->layers[k].spec.kind == TDH_L_ACT && is_pointwise_act(net->layers[k].spec.act);
+        };
+        // the layers behind the convolution that leave the same kernel: a pointwise activation,
+        // then a 2x2 max-pool, then the activation behind the pool
+        int last = i;
+        float *act_out = nullptr;
+        int act_kind   = TDH_ACT_NONE;
+        if (fuse && pointwise(i + 1) && conv_fwd_applies_act(&s.conv, batch, wp != nullptr)) {
+          last     = i + 1;
+          act_out  = net->layers[last].out;
+          act_kind = net->layers[last].spec.act;
         }
+        PoolFuse pf{nullptr, nullptr, nullptr, TDH_ACT_NONE};
+        if (fuse && !(pointwise(i + 1) && last == i) && last + 1 < n &&
+            net->layers[last + 1].spec.kind == TDH_L_MAXPOOL &&
+            conv_fwd_fuses_pool(&s.conv, &net->layers[last + 1].spec.pool, batch, wp != nullptr)) {
+          ++last;
+          pf.out    = net->layers[last].out;
+          pf.argmax = net->layers[last].argmax;
+          if (pointwise(last + 1)) {
+            ++last;
+            pf.act_out  = net->layers[last].out;
+            pf.act_kind = net->layers[last].spec.act;
+          }
+        }
+        TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp, act_out, act_kind,
+                           pf.out ? &pf : nullptr));
+        i = last;
       }
         break;
       case TDH_L_FC:
@@ -323,7 +344,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       }
     }
   }
-  if (rc == TDH_OK) rc = net_alloc(net, 2, &net->dev_powers, true);
+  if (rc == TDH_OK) rc = net_alloc(net, 4, &net->dev_powers, true);  // powers, ticket (zero)
   if (rc == TDH_OK && (flags & TDH_NET_GRAPH)) {
     Context &c = ctx();
     for (hipStream_t &s : c.side)
@@ -489,8 +510,13 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
       // this layer's output gradient is complete here: let the side streams start from it
       TDH_HIP(hipEventRecord(net->events[i], c.stream));
       TDH_HIP(hipStreamWaitEvent(c.side[0], net->events[i], 0));
-      TDH_HIP(hipStreamWaitEvent(c.side[1], net->events[i], 0));
-      side_used[0] = side_used[1] = true;
+      side_used[0] = true;
+      // the second side stream carries the bias gradient where that is a launch of its own
+      const bool own_db = L.b_size && !(s.kind == TDH_L_CONV && conv_dw_gives_db(&s.conv, batch));
+      if (own_db) {
+        TDH_HIP(hipStreamWaitEvent(c.side[1], net->events[i], 0));
+        side_used[1] = true;
+      }
     }
     if (i >= 1 && net->layers[i - 1].grad_folded) {
       // write straight into the activation's input gradient, scaled by act'(its output)
@@ -510,13 +536,15 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             break;
           }
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+          const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
           {
             StreamSwap on_side(c.side[0]);
             c.defer_reduce = true;
-            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad(), L.tbl_dev));
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, db_with_dw ? L.db : nullptr, 1,
+                               ActGrad(), L.tbl_dev));
             c.defer_reduce = false;
           }
-          if (L.b_size) {
+          if (L.b_size && !db_with_dw) {
             StreamSwap on_side(c.side[1]);
             c.defer_rowsum = true;
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));

@@ -158,26 +158,26 @@ int batchnorm_fwd(int channels, int spatial, int batch, float eps, int train, co
     float *partial = static_cast<float *>(ws);
     const float n  = static_cast<float>(batch) * static_cast<float>(spatial);
     ProfScope prof("batchnorm_moments", 8.0 * total, WORK_BYTE);
-    hipLaunchKernelGGL((bn_partial_kernel<0>), dim3(channels, groups), dim3(NT), 0, ctx().stream, x,
+    TDH_LAUNCH((bn_partial_kernel<0>), dim3(channels, groups), dim3(NT), 0, ctx().stream, x,
                        nullptr, nullptr, batch, channels, spatial, groups, partial);
     TDH_LAUNCH_CHECK();
-    hipLaunchKernelGGL((bn_finish_kernel<0>), dim3(ceil_div(channels, NT / 64)), dim3(NT), 0,
+    TDH_LAUNCH((bn_finish_kernel<0>), dim3(ceil_div(channels, NT / 64)), dim3(NT), 0,
                        ctx().stream, partial, channels, groups, n, 0.0f, mean, nullptr);
     TDH_LAUNCH_CHECK();
-    hipLaunchKernelGGL((bn_partial_kernel<1>), dim3(channels, groups), dim3(NT), 0, ctx().stream, x,
+    TDH_LAUNCH((bn_partial_kernel<1>), dim3(channels, groups), dim3(NT), 0, ctx().stream, x,
                        nullptr, mean, batch, channels, spatial, groups, partial);
     TDH_LAUNCH_CHECK();
-    hipLaunchKernelGGL((bn_finish_kernel<1>), dim3(ceil_div(channels, NT / 64)), dim3(NT), 0,
+    TDH_LAUNCH((bn_finish_kernel<1>), dim3(ceil_div(channels, NT / 64)), dim3(NT), 0,
                        ctx().stream, partial, channels, groups, std::max(1.0f, n - 1.0f), eps,
                        variance, stddev);
     TDH_LAUNCH_CHECK();
   } else {
-    hipLaunchKernelGGL(bn_stddev_kernel, dim3(ceil_div(channels, NT)), dim3(NT), 0, ctx().stream,
+    TDH_LAUNCH(bn_stddev_kernel, dim3(ceil_div(channels, NT)), dim3(NT), 0, ctx().stream,
                        variance, channels, eps, stddev);
     TDH_LAUNCH_CHECK();
   }
   ProfScope prof("batchnorm_fwd", 8.0 * total, WORK_BYTE);
-  hipLaunchKernelGGL(bn_apply_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))), dim3(NT),
+  TDH_LAUNCH(bn_apply_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))), dim3(NT),
                      0, ctx().stream, x, mean, stddev, channels, FastDiv(spatial), total, y);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -194,15 +194,15 @@ int batchnorm_bwd(int channels, int spatial, int batch, const float *y, const fl
   const float n  = static_cast<float>(batch) * static_cast<float>(spatial);
   {
     ProfScope prof("batchnorm_bwd_moments", 8.0 * total, WORK_BYTE);
-    hipLaunchKernelGGL((bn_partial_kernel<2>), dim3(channels, groups), dim3(NT), 0, ctx().stream, dy,
+    TDH_LAUNCH((bn_partial_kernel<2>), dim3(channels, groups), dim3(NT), 0, ctx().stream, dy,
                        y, nullptr, batch, channels, spatial, groups, partial);
     TDH_LAUNCH_CHECK();
-    hipLaunchKernelGGL((bn_finish_kernel<0>), dim3(ceil_div(2 * channels, NT / 64)), dim3(NT), 0,
+    TDH_LAUNCH((bn_finish_kernel<0>), dim3(ceil_div(2 * channels, NT / 64)), dim3(NT), 0,
                        ctx().stream, partial, 2 * channels, groups, n, 0.0f, means, nullptr);
     TDH_LAUNCH_CHECK();
   }
   ProfScope prof("batchnorm_bwd", 12.0 * total, WORK_BYTE);
-  hipLaunchKernelGGL(bn_bwd_apply_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))),
+  TDH_LAUNCH(bn_bwd_apply_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))),
                      dim3(NT), 0, ctx().stream, y, dy, means, stddev, channels, FastDiv(spatial),
                      total, dx);
   TDH_LAUNCH_CHECK();
@@ -211,7 +211,7 @@ int batchnorm_bwd(int channels, int spatial, int batch, const float *y, const fl
 
 int batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
                             const float *var_cur, float *mean, float *var) {
-  hipLaunchKernelGGL(bn_moving_kernel, dim3(ceil_div(channels, NT)), dim3(NT), 0, ctx().stream,
+  TDH_LAUNCH(bn_moving_kernel, dim3(ceil_div(channels, NT)), dim3(NT), 0, ctx().stream,
                      mean_cur, var_cur, channels, momentum, mean, var);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -219,7 +219,7 @@ int batchnorm_update_moving(int channels, float momentum, const float *mean_cur,
 
 int dropout_fwd(size_t total, int train, float scale, const uint8_t *mask, const float *x, float *y) {
   ProfScope prof("dropout_fwd", (train ? 9.0 : 8.0) * total, WORK_BYTE);
-  hipLaunchKernelGGL(dropout_fwd_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))),
+  TDH_LAUNCH(dropout_fwd_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))),
                      dim3(NT), 0, ctx().stream, train ? mask : nullptr, scale, x, total, y);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -227,7 +227,7 @@ int dropout_fwd(size_t total, int train, float scale, const uint8_t *mask, const
 
 int dropout_bwd(size_t total, const uint8_t *mask, const float *dy, float *dx) {
   ProfScope prof("dropout_bwd", 9.0 * total, WORK_BYTE);
-  hipLaunchKernelGGL(dropout_bwd_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))),
+  TDH_LAUNCH(dropout_bwd_kernel, dim3(static_cast<unsigned>(ceil_div_sz(total, NT))),
                      dim3(NT), 0, ctx().stream, mask, dy, total, dx);
   TDH_LAUNCH_CHECK();
   return TDH_OK;

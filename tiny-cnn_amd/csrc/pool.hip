@@ -290,12 +290,12 @@ int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int
   if (is_2x2_tiling(g) && aligned16(x) && aligned8(y) && aligned8(argmax) && aligned8(act_out) &&
       total / 2 < (1L << 31)) {
     const int pairs = static_cast<int>(total / 2);
-    hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, x,
+    TDH_LAUNCH(maxpool2x2_fwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, x,
                        y, argmax, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, act_out, act_kind);
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
-  hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
+  TDH_LAUNCH(maxpool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
                      y, argmax, static_cast<int>(total), g, act_out, act_kind);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -311,12 +311,12 @@ int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_
   if (is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) && total / 8 < (1L << 31) &&
       (ag.kind == TDH_ACT_NONE || aligned16(ag.y))) {
     const int pairs = static_cast<int>(total / 8);
-    hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
+    TDH_LAUNCH(maxpool2x2_bwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
                        argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag);
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
-  hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, dy,
+  TDH_LAUNCH(maxpool_bwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, dy,
                      argmax, dx, static_cast<int>(total), g, ag);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -339,7 +339,7 @@ int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *
   if (total <= 0) return TDH_OK;
   const float scale = 1.0f / static_cast<float>(d->pool_w * d->pool_h);
   ProfScope prof("avepool_fwd", 4.0 * batch * g.C * g.H * g.W + 4.0 * total, WORK_BYTE);
-  hipLaunchKernelGGL(avepool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
+  TDH_LAUNCH(avepool_fwd_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream, x,
                      w, b, y, static_cast<int>(total), g, scale);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
@@ -369,7 +369,7 @@ int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *
   if (dx) {
     const long total = static_cast<long>(batch) * g.C * g.H * g.W;
     ProfScope prof("avepool_bwd_dx", 4.0 * batch * g.C * g.OH * g.OW + 4.0 * total, WORK_BYTE);
-    hipLaunchKernelGGL(avepool_bwd_dx_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream,
+    TDH_LAUNCH(avepool_bwd_dx_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream,
                        dy, w, dx, static_cast<int>(total), g, scale);
     TDH_LAUNCH_CHECK();
   }
@@ -377,10 +377,10 @@ int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *
     void *ws = nullptr;
     TDH_TRY(ws_take(static_cast<size_t>(batch) * g.C * 2 * sizeof(float), &ws));
     ProfScope prof("avepool_bwd_param", 4.0 * batch * g.C * (g.H * g.W + g.OH * g.OW), WORK_BYTE);
-    hipLaunchKernelGGL(avepool_bwd_param_kernel, dim3(batch * g.C), dim3(PT), 0, ctx().stream, x,
+    TDH_LAUNCH(avepool_bwd_param_kernel, dim3(batch * g.C), dim3(PT), 0, ctx().stream, x,
                        dy, static_cast<float *>(ws), g);
     TDH_LAUNCH_CHECK();
-    hipLaunchKernelGGL(avepool_bwd_param_reduce_kernel, dim3(ceil_div(g.C, PT)), dim3(PT), 0,
+    TDH_LAUNCH(avepool_bwd_param_reduce_kernel, dim3(ceil_div(g.C, PT)), dim3(PT), 0,
                        ctx().stream, static_cast<const float *>(ws), batch, g.C, scale, dw, db,
                        accumulate);
     TDH_LAUNCH_CHECK();
