@@ -82,6 +82,10 @@ void choose_split(S1Plan &p, int rs, long blocks) {
   if (blocks < 384 && nchunks >= 4) {
     splits = static_cast<int>(std::min<long>(8, (512 + blocks - 1) / blocks));
     splits = std::min(splits, nchunks / 2);
+    // still under half the chip: one chunk per workgroup
+    if (blocks * splits <= 128) splits = static_cast<int>(std::min<long>(nchunks, 256 / blocks));
+  } else if (blocks <= 128 && nchunks >= 2) {
+    splits = 2;  // half the chip would idle: one chunk per workgroup is still the better deal
   }
   const int per      = ceil_div(nchunks, splits) * kch;
   p.splits           = ceil_div(p.args.KC, per);
