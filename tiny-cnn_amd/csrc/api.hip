@@ -95,13 +95,15 @@ struct ProfEntry {
 bool g_profiling = false;
 int g_open_scope = -1;  // index into g_records of the innermost open ProfScope
 std::vector<ProfRecord> g_records;
-std::vector<hipEvent_t> g_event_pool;
+// Events go back to the pool of the role they had: the runtime remembers on an event handed to
+// hipExtLaunchKernelGGL whether it stands for the begin or the end of the dispatch.
+std::vector<hipEvent_t> g_event_pool[2];  // [0] start events, [1] stop events
 std::vector<ProfEntry> g_entries;
 
-hipEvent_t take_event() {
-  if (!g_event_pool.empty()) {
-    hipEvent_t e = g_event_pool.back();
-    g_event_pool.pop_back();
+hipEvent_t take_event(int role) {
+  if (!g_event_pool[role].empty()) {
+    hipEvent_t e = g_event_pool[role].back();
+    g_event_pool[role].pop_back();
     return e;
   }
   hipEvent_t e = nullptr;
@@ -111,7 +113,7 @@ hipEvent_t take_event() {
 }  // namespace
 
 static int open_record(const std::string &tag, double work, WorkUnit unit) {
-  ProfRecord r{tag, work, unit, take_event(), take_event()};
+  ProfRecord r{tag, work, unit, take_event(0), take_event(1)};
   if (!r.start || !r.stop) return -1;
   g_records.push_back(r);
   return static_cast<int>(g_records.size()) - 1;
@@ -355,8 +357,8 @@ int tdh_profile_begin(void) {
   TDH_REQUIRE_INIT();
   TDH_HIP(hipStreamSynchronize(ctx().stream));
   for (auto &r : g_records) {
-    g_event_pool.push_back(r.start);
-    g_event_pool.push_back(r.stop);
+    g_event_pool[0].push_back(r.start);
+    g_event_pool[1].push_back(r.stop);
   }
   g_records.clear();
   g_entries.clear();
@@ -374,8 +376,8 @@ int tdh_profile_end(int32_t *n_entries) {
   for (auto &r : g_records) {
     float ms = 0.0f;
     if (!r.launched) {  // a scope that launched nothing (its work was deferred or empty)
-      g_event_pool.push_back(r.start);
-      g_event_pool.push_back(r.stop);
+      g_event_pool[0].push_back(r.start);
+      g_event_pool[1].push_back(r.stop);
       continue;
     }
     TDH_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
@@ -385,8 +387,8 @@ int tdh_profile_end(int32_t *n_entries) {
     e.total_ms += ms;
     e.work += r.work;
     e.unit = r.unit;
-    g_event_pool.push_back(r.start);
-    g_event_pool.push_back(r.stop);
+    g_event_pool[0].push_back(r.start);
+    g_event_pool[1].push_back(r.stop);
   }
   g_records.clear();
   g_entries.clear();

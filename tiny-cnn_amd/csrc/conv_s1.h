@@ -7,9 +7,11 @@
 namespace tdh {
 
 // Reduction channels per chunk. Tiles of four accumulator blocks a wave take 8 (4 with 25
-// taps): two workgroups share a CU's 512 registers, and with 64 accumulators the staged words
-// of 16 channels no longer fit beside them.
-constexpr int s1_kch(int RS, int TM, int TN) { return TM * TN >= 4 ? (RS >= 25 ? 4 : 8) : 16; }
+// taps), tiles of two channel blocks with 25 taps 8: two workgroups share a CU's 512 registers, and
+// beside that many accumulators the staged words of 16 channels no longer fit.
+constexpr int s1_kch(int RS, int TM, int TN) {
+  return TM * TN >= 4 ? (RS >= 25 ? 4 : 8) : (TM == 2 && TN == 1 && RS >= 25 ? 8 : 16);
+}
 
 // Input-patch words a thread stages per chunk at most: a tile of 128*TN pixels in rows of TC,
 // cut into at most two images (two halos), 256/KCH threads to a channel plane.

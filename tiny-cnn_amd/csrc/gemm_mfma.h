@@ -551,8 +551,12 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
     const double work  = tiles * t.bm * t.bn * static_cast<double>(K);  // padded MACs
     const double waves = tiles * splits / slots;
     const double fill  = waves >= 1.0 ? waves / static_cast<double>(static_cast<long>(waves + 0.999)) : waves;
-    double cost = work / (kEff[c] * (fill > 1.0 ? 1.0 : fill));
-    if (splits > 1) cost += 3.0 * tiles * t.bm * t.bn * splits * 64.0;  // partial tile traffic
+    // a workgroup's prologue and epilogue weigh like bm*bn/80 more steps of K: large tiles
+    // lose on short reductions (4096 x 4096 x 256: 64x64 tiles 92 us, 128x128 tiles 108 us)
+    // (unsplit products only: split ones keep every workgroup resident at once)
+    const double eff = splits > 1 ? kEff[c] : kEff[c] * K / (K + t.bm * t.bn / 80.0);
+    double cost = work / (eff * (fill > 1.0 ? 1.0 : fill));
+    if (splits > 1) cost += 2.0 * tiles * t.bm * t.bn * splits * 64.0;  // partial tile traffic
     if (cost < best_cost) {
       best_cost = cost;
       best = c;
