@@ -263,7 +263,8 @@ bool conv_dw_halo_applicable(int R, int S, int batch, int C, int Kc, int H, int 
 size_t conv_dw_halo_workspace_bytes(int R, int S, int batch, int C, int Kc, int H, int W, int OH,
                                     int OW, int ph, int pw);
 int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, const float *dy,
-                     float *dw, int H, int W, int OH, int OW, int ph, int pw, int accumulate);
+                     float *dw, int H, int W, int OH, int OW, int ph, int pw, int accumulate,
+                     float *db = nullptr);
 // workspace bytes the op may ask for (so a net can reserve it before graph capture)
 size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
 size_t fc_workspace_bytes(int in, int out, int batch);

@@ -524,7 +524,12 @@ static bool dw_small_applies(const tdh_conv_desc *d, const ConvGeom &g, int batc
                                              g.dh, g.dw, g.pad_h, g.pad_w);
 }
 
-bool conv_dw_gives_db(const tdh_conv_desc *d, int batch) { return dw_small_applies(d, make_geom(d), batch); }
+bool conv_dw_gives_db(const tdh_conv_desc *d, int batch) {
+  const ConvGeom g = make_geom(d);
+  if (dw_small_applies(d, g, batch)) return true;
+  return !d->tbl && g.sh == 1 && g.sw == 1 &&
+         conv_dw_halo_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
+}
 
 bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked) {
   return prepacked ? conv_uses_packed(d, batch, 0) : fwd_small_applies(make_geom(d), batch);
@@ -650,8 +655,10 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
                          g.C, g.Kc, g.R * g.S, accumulate);
       TDH_LAUNCH_CHECK();
     } else if (halo) {
+      // the kernel adds up the dY words it stages: the bias gradient needs no pass of its own
       TDH_TRY(conv_dw_halo_run(g.R, g.S, batch, g.C, g.Kc, x, dy, dw, g.H, g.W, g.OH, g.OW, g.pad_h,
-                               g.pad_w, accumulate));
+                               g.pad_w, accumulate, db));
+      db = nullptr;
     } else {
       EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
       TDH_TRY((launch_gemm<true, true>(A, B, epi, g.Kc, crs, batch * ohw, true, "conv_dw_gemm",

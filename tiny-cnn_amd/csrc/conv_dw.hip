@@ -54,6 +54,9 @@ __device__ __align__(16) float dwh_zero_word[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 struct DwHaloArgs {
   const float *x, *dy;
   float *partial;  // [slices][Kc][C*RF*S]
+  // Bias gradient on the way (or null): the workgroups of input-channel block 0 / filter row 0
+  // add up the dY words they stage anyway; [slices][Kc], reduced like the dW slices.
+  float *partial_db;
   int batch, C, Kc, H, W, OH, OW, ph, pw;
   int TI;          // whole images stacked in a chunk (1: a chunk is WK*64/TC rows of one image)
   int tiles_x, chunks_total, chunks_per_slice;
@@ -173,6 +176,10 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
 
   floatx4 rx[NXI];
   floatx4 rdy[DWH_NDY];
+  const bool sums_dy = a.partial_db != nullptr && bz == 0;
+  float dbs[DWH_NDY];  // this thread's share of the bias gradient of channels dco + DCO*i
+#pragma unroll
+  for (int i = 0; i < DWH_NDY; ++i) dbs[i] = 0.0f;
 
   // The loads of a chunk are issued in STEPS parts, one per step of the MFMA loop of the chunk
   // before: every workgroup of the grid fetches at the same time, and a chunk's words issued
@@ -237,6 +244,10 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     float *dd = dy_l + dco * a.dyp + 4 * dq;
 #pragma unroll
     for (int i = 0; i < DWH_NDY; ++i) *reinterpret_cast<floatx4 *>(dd + DCO * i * a.dyp) = rdy[i];
+    if (sums_dy) {
+#pragma unroll
+      for (int i = 0; i < DWH_NDY; ++i) dbs[i] += (rdy[i].x + rdy[i].y) + (rdy[i].z + rdy[i].w);
+    }
   };
 
   const int c_begin = slice * a.chunks_per_slice;
@@ -324,6 +335,21 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
 #pragma unroll
         for (int t = 0; t < NACC; ++t) dst[static_cast<size_t>(co) * crs + t] = acc[t][r];
       }
+    }
+  }
+  if (sums_dy) {
+    // channel c = dco + DCO*i was summed by the DQ threads dco*DQ .. dco*DQ + DQ-1: add their
+    // shares in thread order
+    float *sh = smem;  // [DWH_NDY][NT]
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < DWH_NDY; ++i) sh[i * NT + tid] = dbs[i];
+    __syncthreads();
+    if (tid < BCO && co0 + tid < a.Kc) {
+      const float *src = sh + (tid / DCO) * NT + (tid % DCO) * DQ;
+      float s = 0.0f;
+      for (int q = 0; q < DQ; ++q) s += src[q];
+      a.partial_db[static_cast<size_t>(bx) * a.Kc + co0 + tid] = s;
     }
   }
 }
@@ -447,31 +473,51 @@ size_t conv_dw_halo_workspace_bytes(int R, int S, int batch, int C, int Kc, int 
                                     int OW, int ph, int pw) {
   const DwHaloPlan p = make_dw_plan(R, S, batch, C, Kc, H, W, OH, OW, ph, pw);
   if (!p.ok) return 0;
-  return ws_align(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc * C * R * S);
+  return ws_align(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc * C * R * S) +
+         ws_align(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc);
 }
 
 // dw (+)= sum over the batch; the caller has checked applicability and reserved the workspace
 int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, const float *dy,
-                     float *dw, int H, int W, int OH, int OW, int ph, int pw, int accumulate) {
+                     float *dw, int H, int W, int OH, int OW, int ph, int pw, int accumulate,
+                     float *db) {
   DwHaloPlan p = make_dw_plan(R, S, batch, C, Kc, H, W, OH, OW, ph, pw);
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_dw_halo_run: shape not supported");
   const int crs = C * R * S;
   void *part = nullptr;
   TDH_TRY(ws_take(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc * crs, &part));
   p.args.x = x; p.args.dy = dy; p.args.partial = static_cast<float *>(part);
+  p.args.partial_db = nullptr;
+  if (db) {
+    void *part_db = nullptr;
+    TDH_TRY(ws_take(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc, &part_db));
+    p.args.partial_db = static_cast<float *>(part_db);
+  }
   const bool vec = W % 4 == 0 && OW % 4 == 0 && aligned16(x) && aligned16(dy);
   {
-    ProfScope prof("conv_dw_halo", Kc, crs, batch * OH * OW);
+    ProfScope prof(db ? "conv_dw_db_halo" : "conv_dw_halo", Kc, crs, batch * OH * OW);
     if (vec) TDH_TRY(launch_dw_vec<true>(p));
     else TDH_TRY(launch_dw_vec<false>(p));
   }
   const int slices = static_cast<int>(p.grid.x);
   EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
-  if (defer_reduce(p.args.partial, slices, Kc, crs, epi)) return TDH_OK;
-  ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
-  TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * crs, REDUCE_OUTPUTS)),
-                     dim3(256), 0, ctx().stream, p.args.partial, slices, Kc, crs, epi);
-  TDH_LAUNCH_CHECK();
+  EpiRowMajor epi_b{db, 1, nullptr, ActGrad(), accumulate};
+  if (defer_reduce(p.args.partial, slices, Kc, crs, epi)) {
+    if (db) defer_reduce(p.args.partial_db, slices, Kc, 1, epi_b);
+    return TDH_OK;
+  }
+  {
+    ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
+    TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * crs, REDUCE_OUTPUTS)), dim3(256), 0,
+               ctx().stream, p.args.partial, slices, Kc, crs, epi);
+    TDH_LAUNCH_CHECK();
+  }
+  if (db) {
+    ProfScope prof("conv_db_splitk_reduce", 4.0 * Kc * (slices + 1), WORK_BYTE);
+    TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc, REDUCE_OUTPUTS)), dim3(256), 0,
+               ctx().stream, static_cast<const float *>(p.args.partial_db), slices, Kc, 1, epi_b);
+    TDH_LAUNCH_CHECK();
+  }
   return TDH_OK;
 }
 
