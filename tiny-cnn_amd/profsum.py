@@ -44,23 +44,38 @@ def find(dirname, suffix):
 
 
 def kernels(dirname, top):
-    rows = collections.defaultdict(list)
+    """One row per kernel symbol and grid size. A replayed train step runs its weight-gradient
+    kernels beside the main chain, and a kernel that shares the device takes longer than the
+    same kernel alone; the "alone" columns average only the dispatches that overlap no other
+    dispatch in time (the per-kernel pass of bench.py launches every kernel that way)."""
+    disp = []
     for path in find(dirname, "_kernel_trace.csv"):
         with open(path, newline="") as f:
             for r in csv.DictReader(f):
-                dur = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
                 if "Grid_Size" in r:
                     grid = int(r["Grid_Size"])
                 else:
                     grid = int(r["Grid_Size_X"]) * int(r["Grid_Size_Y"]) * int(r["Grid_Size_Z"])
-                rows[(short_name(r["Kernel_Name"]), grid)].append(dur)
+                disp.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]),
+                             (short_name(r["Kernel_Name"]), grid)))
+    disp.sort()
+    rows, alone = collections.defaultdict(list), collections.defaultdict(list)
+    latest_end = 0  # of all earlier dispatches
+    for k, (start, end, key) in enumerate(disp):
+        rows[key].append(end - start)
+        overlaps = start < latest_end or (k + 1 < len(disp) and disp[k + 1][0] < end)
+        if not overlaps:
+            alone[key].append(end - start)
+        latest_end = max(latest_end, end)
     total = sum(sum(v) for v in rows.values())
-    print(f"| kernel | grid (work-items) | launches | avg us | min us | max us | % of GPU time |")
-    print("|---|---:|---:|---:|---:|---:|---:|")
+    print("| kernel | grid (work-items) | launches | avg us | min us | max us | % of GPU time | alone: launches | alone: avg us |")
+    print("|---|---:|---:|---:|---:|---:|---:|---:|---:|")
     order = sorted(rows.items(), key=lambda kv: -sum(kv[1]))
     for (name, grid), d in order[:top]:
+        a = alone.get((name, grid), [])
+        a_avg = f"{sum(a) / len(a) / 1e3:.2f}" if a else "-"
         print(f"| `{name}` | {grid} | {len(d)} | {sum(d) / len(d) / 1e3:.2f} | {min(d) / 1e3:.2f} | "
-              f"{max(d) / 1e3:.2f} | {100.0 * sum(d) / total:.1f} |")
+              f"{max(d) / 1e3:.2f} | {100.0 * sum(d) / total:.1f} | {len(a)} | {a_avg} |")
     print(f"\n{sum(len(v) for v in rows.values())} dispatches, {total / 1e6:.3f} ms of kernel time in total")
 
 
