@@ -7,8 +7,9 @@
 // As a product the shape is M = Cout, N = Cin*KH*KW (75 for 3 channels and 5x5), K = batch*OH*OW:
 // a tile of a general GEMM kernel is mostly padding in N, and its B operand is gathered from
 // global memory element by element. Here a workgroup owns a band of output rows of one image.
-// It stages the input patch under the band (zero-filled where the window leaves the image) and
-// the band of dY into LDS once, with all loads in flight together, and then every MFMA
+// It stages the input patch under the band (zero-filled where the window leaves the image) once
+// and the band of dY chunk by chunk into LDS, a thread's loads all in flight together and the
+// next chunk's issued before the current chunk is multiplied, and then every MFMA
 // (v_mfma_f32_32x32x2_f32: A lane = (co, k), B lane = (n, k)) takes its B value with one LDS read
 // at patch[pos(k)] + offset(n); offset(n) is a per-lane constant. Column N of the product has
 // B = 1: it is the bias gradient, which so costs no pass over dY of its own. The four waves of
