@@ -169,7 +169,7 @@ struct OptTensor {
   const uint8_t *tbl;
   uint32_t C, Kc, rs;
 };
-constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 4096;
+constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 1024;  // one 16-byte access per thread: a pass of a small net is latency, not bandwidth
 // dev_powers: NULL, or device floats {b1_t, b2_t, ticket (zero), unused} that the kernel reads instead of the
 // host values and that a follow-up kernel advances n_tensors times (graph replay).
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
