@@ -11,14 +11,16 @@ namespace tdh {
 
 namespace {
 
-// Products of a small network's fully-connected layers (a few million MACs, K <= 256): the
+// Products of a small network's fully-connected layers (a few million MACs, K <= 512): the
 // tiled MFMA kernel pays one exposed memory latency per 16-deep K tile with only a handful of
 // workgroups to hide it behind, 7-16 us for microseconds of arithmetic. Here a workgroup
-// stages 64-deep panels of both operands with every load in flight at once (20 per thread),
+// stages 128-deep panels of both operands with every load in flight at once (40 per thread;
+// a panel costs one exposed memory latency, so the fewer the better: 64-deep panels made the
+// backward kernels of the CIFAR net's two layers 10.6 us, 128-deep ones 8.6 us),
 // and the four waves multiply out of LDS on the vector ALUs: wave w owns rows 4w..4w+3 of a
 // 16 x 64 tile, so its A values are wave-uniform LDS broadcasts and its B values one
 // conflict-free read per k. k ascends, one FMA per term: the summation order is fixed.
-constexpr int SFC_TM = 16, SFC_TN = 64, SFC_KC = 64, SFC_NT = 256;
+constexpr int SFC_TM = 16, SFC_TN = 64, SFC_KC = 128, SFC_NT = 256;
 constexpr int SFC_NA = SFC_TM * SFC_KC / SFC_NT, SFC_NB = SFC_TN * SFC_KC / SFC_NT;
 
 struct SfcSmem {
