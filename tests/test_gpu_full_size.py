@@ -1,4 +1,4 @@
-"""BASELINE.json's configurations at their full sizes on the MI355X, checked through
+"""The five benchmark configurations at their full sizes on the MI355X, checked through
 size-independent properties and float64 spot checks (the scalar oracle would need minutes
 at these sizes): exact float64 dot products for sampled gradient entries, db against a host
 sum, linearity of the backward pass in dY, and whole fully-connected gradients against
