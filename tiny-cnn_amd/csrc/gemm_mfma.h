@@ -544,7 +544,7 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
     int splits = 1;
     if (allow_split && tiles < slots) {
       splits = static_cast<int>(slots / tiles);
-      const int max_by_k = K / 96 > 0 ? K / 96 : 1;
+      const int max_by_k = K / 16 > 0 ? K / 16 : 1;
       if (splits > max_by_k) splits = max_by_k;
       if (splits < 1) splits = 1;
     }
