@@ -83,8 +83,7 @@ struct ProfRecord {
   std::string tag;
   double work;
   WorkUnit unit;
-  hipEvent_t start, stop;
-  bool started = false, launched = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> launches;  // (begin, end) of every kernel
 };
 struct ProfEntry {
   std::string tag;
@@ -113,9 +112,7 @@ hipEvent_t take_event(int role) {
 }  // namespace
 
 static int open_record(const std::string &tag, double work, WorkUnit unit) {
-  ProfRecord r{tag, work, unit, take_event(0), take_event(1)};
-  if (!r.start || !r.stop) return -1;
-  g_records.push_back(r);
+  g_records.push_back(ProfRecord{tag, work, unit, {}});
   return static_cast<int>(g_records.size()) - 1;
 }
 
@@ -139,16 +136,14 @@ ProfScope::~ProfScope() {
   if (g_profiling) g_open_scope = outer;
 }
 
-hipEvent_t prof_launch_start() {
-  if (!g_profiling || g_open_scope < 0 || g_records[g_open_scope].started) return nullptr;
-  g_records[g_open_scope].started = true;
-  return g_records[g_open_scope].start;
-}
-
-hipEvent_t prof_launch_stop() {
-  if (!g_profiling || g_open_scope < 0) return nullptr;
-  g_records[g_open_scope].launched = true;
-  return g_records[g_open_scope].stop;
+void prof_launch_events(hipEvent_t *start, hipEvent_t *stop) {
+  *start = *stop = nullptr;
+  if (!g_profiling || g_open_scope < 0) return;
+  hipEvent_t b = take_event(0), e = take_event(1);
+  if (!b || !e) return;
+  g_records[g_open_scope].launches.emplace_back(b, e);
+  *start = b;
+  *stop  = e;
 }
 
 // tiny_dnn/util/util.h:329-344
@@ -356,10 +351,11 @@ int tdh_tune_gemm_plan(int32_t tile_cfg, int32_t splits) {
 int tdh_profile_begin(void) {
   TDH_REQUIRE_INIT();
   TDH_HIP(hipStreamSynchronize(ctx().stream));
-  for (auto &r : g_records) {
-    g_event_pool[0].push_back(r.start);
-    g_event_pool[1].push_back(r.stop);
-  }
+  for (auto &r : g_records)
+    for (auto &l : r.launches) {
+      g_event_pool[0].push_back(l.first);
+      g_event_pool[1].push_back(l.second);
+    }
   g_records.clear();
   g_entries.clear();
   g_open_scope = -1;
@@ -374,21 +370,21 @@ int tdh_profile_end(int32_t *n_entries) {
   std::map<std::string, ProfEntry> by_tag;
   g_open_scope = -1;
   for (auto &r : g_records) {
-    float ms = 0.0f;
-    if (!r.launched) {  // a scope that launched nothing (its work was deferred or empty)
-      g_event_pool[0].push_back(r.start);
-      g_event_pool[1].push_back(r.stop);
-      continue;
+    if (r.launches.empty()) continue;  // a scope that launched nothing (its work was deferred)
+    double ms_sum = 0.0;
+    for (auto &l : r.launches) {
+      float ms = 0.0f;
+      TDH_HIP(hipEventElapsedTime(&ms, l.first, l.second));
+      ms_sum += ms;
+      g_event_pool[0].push_back(l.first);
+      g_event_pool[1].push_back(l.second);
     }
-    TDH_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
     ProfEntry &e = by_tag[r.tag];
     e.tag        = r.tag;
     e.launches += 1;
-    e.total_ms += ms;
+    e.total_ms += ms_sum;
     e.work += r.work;
     e.unit = r.unit;
-    g_event_pool[0].push_back(r.start);
-    g_event_pool[1].push_back(r.stop);
   }
   g_records.clear();
   g_entries.clear();

@@ -96,18 +96,21 @@ struct ProfScope {
 };
 bool profiling_active();
 // The duration of a profiled scope comes from the dispatches themselves: while a scope is
-// open, TDH_LAUNCH hands its events to hipExtLaunchKernelGGL, which stamps them with the
-// start of the scope's first kernel and the end of its last one. (Events recorded around a
-// launch would add the latency of their own packets, a few microseconds per kernel.)
-hipEvent_t prof_launch_start();
-hipEvent_t prof_launch_stop();
+// open, TDH_LAUNCH hands every launch a pair of events to hipExtLaunchKernelGGL, which stamps
+// them with the begin and the end of that kernel's execution; a scope's duration is the sum
+// over its launches. (Events recorded around a launch would add the latency of their own
+// packets, a few microseconds per kernel, and idle time between two launches of a scope.)
+void prof_launch_events(hipEvent_t *start, hipEvent_t *stop);  // nulls outside a scope
 #define TDH_LAUNCH(kernel, grid, block, shmem, stream, ...)                                  \
   do {                                                                                       \
-    if (::tdh::profiling_active())                                                           \
-      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, ::tdh::prof_launch_start(),  \
-                            ::tdh::prof_launch_stop(), 0, __VA_ARGS__);                       \
-    else                                                                                     \
+    if (::tdh::profiling_active()) {                                                         \
+      hipEvent_t tdh_ev0_, tdh_ev1_;                                                         \
+      ::tdh::prof_launch_events(&tdh_ev0_, &tdh_ev1_);                                       \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, tdh_ev0_, tdh_ev1_, 0,       \
+                            __VA_ARGS__);                                                    \
+    } else {                                                                                 \
       hipLaunchKernelGGL(kernel, grid, block, shmem, stream, __VA_ARGS__);                   \
+    }                                                                                        \
   } while (0)
 
 // ---------------------------------------------------------------- helpers

@@ -502,23 +502,15 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
   const int slices = static_cast<int>(p.grid.x);
   EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
   EpiRowMajor epi_b{db, 1, nullptr, ActGrad(), accumulate};
-  if (defer_reduce(p.args.partial, slices, Kc, crs, epi)) {
-    if (db) defer_reduce(p.args.partial_db, slices, Kc, 1, epi_b);
-    return TDH_OK;
-  }
-  {
-    ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * crs * (slices + 1), WORK_BYTE);
-    TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * crs, REDUCE_OUTPUTS)), dim3(256), 0,
-               ctx().stream, p.args.partial, slices, Kc, crs, epi);
-    TDH_LAUNCH_CHECK();
-  }
-  if (db) {
-    ProfScope prof("conv_db_splitk_reduce", 4.0 * Kc * (slices + 1), WORK_BYTE);
-    TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc, REDUCE_OUTPUTS)), dim3(256), 0,
-               ctx().stream, static_cast<const float *>(p.args.partial_db), slices, Kc, 1, epi_b);
-    TDH_LAUNCH_CHECK();
-  }
-  return TDH_OK;
+  // the two reductions leave as one launch: collected by the train step, or here
+  const bool collect_here = !ctx().defer_reduce;
+  if (collect_here) flush_deferred_reduces(false);  // nothing may be left from a failed call
+  ctx().defer_reduce = true;
+  defer_reduce(p.args.partial, slices, Kc, crs, epi);
+  if (db) defer_reduce(p.args.partial_db, slices, Kc, 1, epi_b);
+  if (!collect_here) return TDH_OK;
+  ctx().defer_reduce = false;
+  return flush_deferred_reduces();
 }
 
 }  // namespace tdh

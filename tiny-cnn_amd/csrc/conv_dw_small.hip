@@ -320,25 +320,15 @@ int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy,
   }
   EpiRowMajor epi_w{dw_out, p.a.crs, nullptr, ActGrad(), accumulate};
   EpiRowMajor epi_b{db_out, 1, nullptr, ActGrad(), accumulate};
-  const bool deferred = defer_reduce(p.a.partial_dw, blocks, Kc, p.a.crs, epi_w);
-  if (deferred) {
-    if (db_out) defer_reduce(p.a.partial_db, blocks, Kc, 1, epi_b);
-    return TDH_OK;
-  }
-  {
-    ProfScope prof("conv_dw_splitk_reduce", 4.0 * Kc * p.a.crs * (blocks + 1), WORK_BYTE);
-    TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc * p.a.crs, REDUCE_OUTPUTS)),
-                       dim3(256), 0, ctx().stream, static_cast<const float *>(p.a.partial_dw), blocks, Kc,
-                       p.a.crs, epi_w);
-    TDH_LAUNCH_CHECK();
-  }
-  if (db_out) {
-    ProfScope prof("conv_db_splitk_reduce", 4.0 * Kc * (blocks + 1), WORK_BYTE);
-    TDH_LAUNCH((splitk_reduce_kernel<EpiRowMajor>), dim3(ceil_div(Kc, REDUCE_OUTPUTS)), dim3(256), 0,
-                       ctx().stream, static_cast<const float *>(p.a.partial_db), blocks, Kc, 1, epi_b);
-    TDH_LAUNCH_CHECK();
-  }
-  return TDH_OK;
+  // the two reductions leave as one launch: collected by the train step, or here
+  const bool collect_here = !ctx().defer_reduce;
+  if (collect_here) flush_deferred_reduces(false);  // nothing may be left from a failed call
+  ctx().defer_reduce = true;
+  defer_reduce(p.a.partial_dw, blocks, Kc, p.a.crs, epi_w);
+  if (db_out) defer_reduce(p.a.partial_db, blocks, Kc, 1, epi_b);
+  if (!collect_here) return TDH_OK;
+  ctx().defer_reduce = false;
+  return flush_deferred_reduces();
 }
 
 }  // namespace tdh
