@@ -119,11 +119,13 @@ int tdh_event_destroy(void *event);
 int tdh_event_record(void *event);
 int tdh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
 
-/* Per-kernel timing of everything launched between begin and end: each launch is
- * bracketed by events on the library stream and booked under a kernel tag with its
- * algorithmic work (unit 0 = FLOP, 1 = bytes). The events add launch overhead, so
- * whole-step throughput is measured with profiling off. tdh_profile_end waits for the
- * GPU; entries are then read back by index, ordered by total time (largest first). */
+/* Per-kernel timing of everything launched between begin and end: each launch carries
+ * a pair of events that the runtime stamps with the begin and the end of that kernel's
+ * execution, and is booked under a kernel tag with its algorithmic work (unit 0 = FLOP,
+ * 1 = bytes); a tag's time is the sum over its kernels. A captured train step runs
+ * eagerly while profiling is on, so whole-step throughput is measured with profiling
+ * off. tdh_profile_end waits for the GPU; entries are then read back by index, ordered
+ * by total time (largest first). */
 int tdh_profile_begin(void);
 int tdh_profile_end(int32_t *n_entries);
 int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launches,
