@@ -282,7 +282,7 @@ int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_
 int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *b,
                 float *y);
 int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,
-                float *dx, float *dw, float *db, int accumulate);
+                float *dx, float *dw, float *db, int accumulate, ActGrad ag = ActGrad());
 size_t avepool_workspace_bytes(const tdh_pool_desc *d, int batch);
 
 // forward of the three parameter-free pointwise activations (tanh_layer.h:24-28,

@@ -532,7 +532,9 @@ bool conv_dw_gives_db(const tdh_conv_desc *d, int batch) {
 }
 
 bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked) {
-  return prepacked ? conv_uses_packed(d, batch, 0) : fwd_small_applies(make_geom(d), batch);
+  // every forward kernel does: the packed stride-1 kernel, the first-layer kernel, the
+  // stride-1 kernel that packs for itself and the GEMM (in its epilogue or its split reduction)
+  return prepacked ? conv_uses_packed(d, batch, 0) : true;
 }
 
 bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked) {
@@ -567,8 +569,8 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
                        g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked, act_out,
                        act_kind);
-  if ((act_out || pool) && !fwd_small_applies(g, batch))
-    return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not apply the layers behind it");
+  if (pool && !fwd_small_applies(g, batch))
+    return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not compute the pool layer behind it");
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
@@ -580,9 +582,13 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w))
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w_eff, nullptr,
                        d->has_bias ? b : nullptr, y, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w,
-                       ActGrad(), "conv_fwd_s1");
+                       ActGrad(), "conv_fwd_s1", nullptr, act_out, act_kind);
   StridedOperand A{w_eff, crs, 1, g.Kc};
   FwdInputOperand B{x, g, batch * ohw};
+  if (act_out) {  // the pointwise activation layer that follows leaves the same kernel
+    EpiImageRowsAct epi{y, g.Kc, ohw, g.div_ohw, d->has_bias ? b : nullptr, act_out, act_kind};
+    return launch_gemm<true, false>(A, B, epi, g.Kc, batch * ohw, crs, true, "conv_fwd_gemm", "conv_fwd_splitk_reduce");
+  }
   EpiImageRows epi{y, g.Kc, ohw, g.div_ohw, d->has_bias ? b : nullptr, ActGrad()};
   return launch_gemm<true, false>(A, B, epi, g.Kc, batch * ohw, crs, true, "conv_fwd_gemm", "conv_fwd_splitk_reduce");
 }

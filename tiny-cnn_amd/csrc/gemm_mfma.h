@@ -148,6 +148,31 @@ struct EpiImageRows {
   }
 };
 
+// forward convolution followed by a pointwise activation layer:
+// out = v + bias_m[m], act_out = act(out), both laid out like EpiImageRows
+struct EpiImageRowsAct {
+  float *out;
+  int rows, pix;
+  FastDiv pix_div;
+  const float *bias_m;
+  float *act_out;
+  int act_kind;
+  struct Col {
+    int base;
+  };
+  __device__ __forceinline__ Col col(int n) const {
+    uint32_t img, p;
+    pix_div.divmod(static_cast<uint32_t>(n), img, p);
+    return {static_cast<int>(img) * rows * pix + static_cast<int>(p)};
+  }
+  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+    const int idx = c.base + m * pix;
+    if (bias_m) v += bias_m[m];
+    out[idx]     = v;
+    act_out[idx] = act_apply(act_kind, v);
+  }
+};
+
 // --------------------------------------------------------------------- kernel
 template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, bool A_VEC, bool B_VEC,
           class AOp, class BOp, class Epi>

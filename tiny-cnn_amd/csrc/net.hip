@@ -293,11 +293,11 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
     else if (need > net->scratch)
       net->scratch = need;
     // fold pointwise activation gradients into the following layer's backward kernel (the dX
-    // epilogue of a conv / fc layer, the scatter of a max-pool)
+    // epilogue of a conv / fc layer, the scatter of a max-pool, the dX kernel of an average pool)
     if ((flags & TDH_NET_FUSE_ACT_GRAD) && L.spec.kind == TDH_L_ACT &&
         is_pointwise_act(L.spec.act) && i + 1 < n_layers &&
         (layers[i + 1].kind == TDH_L_CONV || layers[i + 1].kind == TDH_L_FC ||
-         layers[i + 1].kind == TDH_L_MAXPOOL))
+         layers[i + 1].kind == TDH_L_MAXPOOL || layers[i + 1].kind == TDH_L_AVEPOOL))
       L.grad_folded = true;
   }
   if (rc == TDH_OK)
@@ -583,7 +583,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
       case TDH_L_MAXPOOL: TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold)); break;
       case TDH_L_AVEPOOL:
         TDH_TRY(ws_begin(avepool_workspace_bytes(&s.pool, batch)));
-        TDH_TRY(avepool_bwd(&s.pool, batch, in, L.w, L.dout, dx, L.dw, L.db, 1));
+        TDH_TRY(avepool_bwd(&s.pool, batch, in, L.w, L.dout, dx, L.dw, L.db, 1, fold));
         break;
       case TDH_L_ACT:
         if (!L.grad_folded)

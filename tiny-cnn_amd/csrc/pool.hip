@@ -198,7 +198,7 @@ avepool_fwd_kernel(const float *__restrict__ x, const float *__restrict__ w,
 __global__ void __launch_bounds__(PT)
 avepool_bwd_dx_kernel(const float *__restrict__ dy, const float *__restrict__ w,
                       float *__restrict__ dx, const int total, const PoolGeom g,
-                      const float scale) {
+                      const float scale, const ActGrad ag) {
   const int i = blockIdx.x * PT + threadIdx.x;
   if (i >= total) return;
   uint32_t t, xx, yy, c, img;
@@ -209,7 +209,10 @@ avepool_bwd_dx_kernel(const float *__restrict__ dy, const float *__restrict__ w,
   const int ox = ix < g.pw ? 0 : (ix - g.pw + g.sw) / g.sw;
   const int oy = iy < g.ph ? 0 : (iy - g.ph + g.sh) / g.sh;
   const float weight = w[c] * scale;
-  dx[i] = weight * dy[((static_cast<size_t>(img) * g.C + c) * g.OH + oy) * g.OW + ox];
+  float v = weight * dy[((static_cast<size_t>(img) * g.C + c) * g.OH + oy) * g.OW + ox];
+  // the gradient of the activation layer in front of the pool, folded in
+  if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[i]);
+  dx[i] = v;
 }
 
 __device__ __forceinline__ float wave_sum_p(float v) {
@@ -350,7 +353,7 @@ size_t avepool_workspace_bytes(const tdh_pool_desc *d, int batch) {
 }
 
 int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,
-                float *dx, float *dw, float *db, int accumulate) {
+                float *dx, float *dw, float *db, int accumulate, ActGrad ag) {
   TDH_TRY(check_avepool(d));
   const PoolGeom g = make_geom(d);
   // Every input element must lie in at least one window that maps to an existing output;
@@ -368,9 +371,10 @@ int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *
   const float scale = 1.0f / static_cast<float>(d->pool_w * d->pool_h);
   if (dx) {
     const long total = static_cast<long>(batch) * g.C * g.H * g.W;
-    ProfScope prof("avepool_bwd_dx", 4.0 * batch * g.C * g.OH * g.OW + 4.0 * total, WORK_BYTE);
+    ProfScope prof(ag.kind != TDH_ACT_NONE ? "avepool_bwd_dx_act" : "avepool_bwd_dx",
+                   4.0 * batch * g.C * g.OH * g.OW + (ag.kind != TDH_ACT_NONE ? 8.0 : 4.0) * total, WORK_BYTE);
     TDH_LAUNCH(avepool_bwd_dx_kernel, dim3(ceil_div(total, PT)), dim3(PT), 0, ctx().stream,
-                       dy, w, dx, static_cast<int>(total), g, scale);
+                       dy, w, dx, static_cast<int>(total), g, scale, ag);
     TDH_LAUNCH_CHECK();
   }
   if (dw || db) {
