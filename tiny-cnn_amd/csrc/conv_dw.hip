@@ -200,10 +200,13 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     dybase  = y0 * a.OW;
     dylimit = a.TI > 1 ? nimg * kohw : ohw;
   };
+  // (in the first half of the steps: a load issued in the last steps has no MFMAs left to hide
+  // behind, and the next stage() would wait a whole trip to memory for it)
+  constexpr int LOAD_STEPS = STEPS / 2;
   auto fetch_part = [&](int part) {
 #pragma unroll
     for (int i = 0; i < NXI; ++i) {
-      if (i % STEPS != part) continue;
+      if (i % LOAD_STEPS != part) continue;
       const int rel = xrel[i] + xbase;
       const bool ok = static_cast<unsigned>(rel) < xlimit;
       if (VEC) {
@@ -218,7 +221,7 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     }
 #pragma unroll
     for (int i = 0; i < DWH_NDY; ++i) {
-      if (i % STEPS != part) continue;
+      if (i % LOAD_STEPS != part) continue;
       const int rel  = dyrel + dybase;
       const bool oki = static_cast<unsigned>(rel) < dylimit && co0 + dco + DCO * i < a.Kc;
       const float *p = dyb + static_cast<size_t>(DCO * i) * ohw + rel;
