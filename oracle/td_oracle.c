@@ -126,6 +126,10 @@ int tdo_conv2d_fwd(const tdo_conv_desc *d, int batch, const float *x, const floa
   const int ow = tdo_conv_out_w(d), oh = tdo_conv_out_h(d);
   const int id = d->in_c, od = d->out_c, kw = d->k_w, kh = d->k_h;
   const size_t psz = (size_t)iw * ih * id, osz = (size_t)ow * oh * od;
+  /* padding::same pads by the undilated window (convolutional_layer.h:470-474), so with a
+   * dilation the loop below would read past the padded rows, as the reference does: there is
+   * no defined result to restate. */
+  if (d->pad_same && (d->w_dilation != 1 || d->h_dilation != 1)) return -2;
   float *xp = pad_input(d, batch, x);
   if (!xp) return -1;
 #pragma omp parallel for schedule(static)

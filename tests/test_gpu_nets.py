@@ -119,6 +119,11 @@ def test_net_rejects_inconsistent_layers(T):
         T.Net([T.L_fc(10, 5), T.L_fc(6, 2)], 4)
     with pytest.raises(T.TdhError, match="first layer"):
         T.Net([T.L_act("relu"), T.L_fc(6, 2)], 4)
+    # a net is trained, and the reference's backward pass has no defined result with a dilation
+    dilated = T.L_conv(8, 8, 2, 3, 4)
+    dilated.conv.w_dilation = dilated.conv.h_dilation = 2
+    with pytest.raises(T.TdhError, match="dilation"):
+        T.Net([dilated, T.L_fc(4 * 4 * 4, 2)], 4)
 
 
 @pytest.mark.parametrize("name,batch", [("cifar10_cnn_b128", 16), ("lenet5_b16", 16)])

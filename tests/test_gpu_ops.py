@@ -152,6 +152,9 @@ def test_conv_errors_and_empty_batch(T):
     buf = T.DevBuf((16,))
     with pytest.raises(T.TdhError, match="dilation"):
         T.conv2d_bwd(d, 1, buf, buf, buf, buf, buf, buf)
+    same_dilated = T.conv_desc(8, 8, 2, 3, 3, 4, pad_same=True, w_dilation=2, h_dilation=2)
+    with pytest.raises(T.TdhError, match="padding::same and dilation"):
+        T.conv2d_fwd(same_dilated, 1, buf, buf, buf, buf)
     bad = T.conv_desc(2, 2, 1, 3, 3, 1)
     with pytest.raises(T.TdhError, match="window larger"):
         T.conv2d_fwd(bad, 1, buf, buf, buf, buf)

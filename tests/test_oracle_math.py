@@ -387,3 +387,13 @@ def test_norm_layers_match_reference_outputs(O, norm_golden):
         assert np.array_equal(mask, g[f"do{k}.mask"])
         assert np.array_equal(O.dropout_fwd(mask, g["do.x"], rate), g[f"do{k}.y"])
         assert np.array_equal(O.dropout_bwd(mask, g["do.dy"]), g[f"do{k}.dx"])
+
+
+def test_oracle_refuses_same_padding_with_dilation(O):
+    """The reference pads by the undilated window, so its forward loop reads past the padded
+    rows when a dilation is set: the oracle restates no result for that case."""
+    d = O.conv_desc(8, 8, 2, 3, 3, 4, pad_same=True, w_dilation=2, h_dilation=2)
+    x = np.zeros((1, 128), np.float32)
+    w = np.zeros(72, np.float32)
+    with pytest.raises(RuntimeError, match="code -2"):
+        O.conv2d_fwd(d, x, w)

@@ -159,7 +159,7 @@ int pool_out_length(int in_length, int window, int stride, int ceil_mode, int pa
   return static_cast<int>(ceil_mode ? std::ceil(tmp) : std::floor(tmp));
 }
 
-static int check_conv_desc(const tdh_conv_desc *d, int batch, bool backward) {
+int check_conv_desc(const tdh_conv_desc *d, int batch, bool backward) {
   TDH_CHECK_ARG(d != nullptr, "conv: null descriptor");
   TDH_CHECK_ARG(batch >= 0, "conv: negative batch %d", batch);
   TDH_CHECK_ARG(d->in_w > 0 && d->in_h > 0 && d->in_c > 0 && d->out_c > 0 && d->k_w > 0 &&
@@ -171,6 +171,12 @@ static int check_conv_desc(const tdh_conv_desc *d, int batch, bool backward) {
     return set_error(TDH_ERR_UNSUPPORTED,
                      "conv backward with dilation %dx%d: the reference's backward kernel ignores "
                      "dilation, so no defined result exists to match",
+                     d->w_dilation, d->h_dilation);
+  if (d->pad_same && (d->w_dilation != 1 || d->h_dilation != 1))
+    return set_error(TDH_ERR_UNSUPPORTED,
+                     "conv with padding::same and dilation %dx%d: the reference pads by the undilated "
+                     "window (convolutional_layer.h:470-474) and its kernel then reads past the padded "
+                     "rows, so no defined result exists to match",
                      d->w_dilation, d->h_dilation);
   if (!d->pad_same)
     TDH_CHECK_ARG(d->in_w >= d->w_dilation * (d->k_w - 1) + 1 &&

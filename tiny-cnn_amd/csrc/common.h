@@ -179,6 +179,9 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
                             int total_blocks, double total_params, float grad_scale,
                             int zero_grad, float *dev_powers);
 bool profiling_active();
+// api.hip: the argument checks of the convolution entry points (backward: also what only the
+// backward pass refuses)
+int check_conv_desc(const tdh_conv_desc *d, int batch, bool backward);
 // deterministic reductions: out[r] (+)= sum over `cols` contiguous values of row r,
 // rows laid out as [outer][rows][cols] and summed over outer in order
 int launch_rowsum(const float *src, int outer, int rows, int cols, float *out, int accumulate);

@@ -63,6 +63,7 @@ int layer_sizes(tdh_net::Layer &L) {
   const tdh_layer &s = L.spec;
   switch (s.kind) {
     case TDH_L_CONV: {
+      TDH_TRY(check_conv_desc(&s.conv, 1, /*backward=*/true));  // a net is there to be trained
       const int ow = conv_out_length(s.conv.in_w, s.conv.k_w, s.conv.w_stride, s.conv.w_dilation,
                                      s.conv.pad_same);
       const int oh = conv_out_length(s.conv.in_h, s.conv.k_h, s.conv.h_stride, s.conv.h_dilation,
