@@ -490,3 +490,97 @@ def test_norm_argument_errors(T):
         T.dropout_fwd(1, 4, None, buf, buf, train=True)
     T.batchnorm_fwd(0, 2, 1, None, None, None, None, None)      # empty tensors: nothing to do
     T.dropout_bwd(0, 4, None, None, None)
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_randomized_conv_shapes_match_oracle(T, O, seed):
+    """A seeded sweep over window, channel counts, image sizes, padding, stride, dilation
+    (forward only, as in the reference) and batch: whichever kernel the shape selects, forward
+    and all three gradients agree with the oracle."""
+    rng = np.random.default_rng(seed)
+    done = 0
+    while done < 60:
+        k = int(rng.choice([3, 5]))
+        ic = int(rng.choice([1, 2, 3, 4, 8, 16, 20, 32, 48]))
+        oc = int(rng.choice([1, 5, 16, 32, 33, 40, 64, 70]))
+        iw, ih = int(rng.integers(k, 44)), int(rng.integers(k, 30))
+        same = bool(rng.integers(0, 2))
+        st = int(rng.choice([1, 1, 1, 2, 3]))
+        dil = 1 if same else int(rng.choice([1, 1, 1, 2]))
+        bs = int(rng.choice([1, 2, 3, 5, 8, 17]))
+        if not same and (iw < dil * (k - 1) + 1 or ih < dil * (k - 1) + 1):
+            continue
+        kw = dict(pad_same=same, w_stride=st, h_stride=st, w_dilation=dil, h_dilation=dil)
+        d, do = T.conv_desc(iw, ih, ic, k, k, oc, **kw), O.conv_desc(iw, ih, ic, k, k, oc, **kw)
+        ow, oh = T.conv_out_shape(d)
+        if ow < 1 or oh < 1:
+            continue
+        what = f"{(iw, ih, ic, k, oc, same, st, dil, bs)}"
+        x = rng.standard_normal((bs, ic * ih * iw)).astype(np.float32)
+        w = rng.uniform(-0.3, 0.3, oc * ic * k * k).astype(np.float32)
+        b = rng.standard_normal(oc).astype(np.float32)
+        dy = rng.standard_normal((bs, oc * oh * ow)).astype(np.float32)
+        xd, wd, bd, dyd = T.to_device(x), T.to_device(w), T.to_device(b), T.to_device(dy)
+        y = T.DevBuf((bs, oc * oh * ow))
+        T.conv2d_fwd(d, bs, xd, wd, bd, y)
+        assert_close(y.numpy(), O.conv2d_fwd(do, x, w, b), what=what + " y")
+        if dil == 1:
+            dx, dw, db = T.DevBuf(x.shape), T.DevBuf(w.shape), T.DevBuf((oc,), zero=True)
+            T.conv2d_bwd(d, bs, xd, wd, dyd, dx, dw, db, 0)
+            rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
+            assert_close(dx.numpy(), rdx, what=what + " dx")
+            assert_close(dw.numpy(), rdw, what=what + " dw")
+            assert_close(db.numpy(), rdb, what=what + " db")
+        done += 1
+
+
+def test_randomized_fc_and_maxpool_shapes_match_oracle(T, O):
+    """Seeded sweeps: fully-connected layers across the small / tiled / split products, and
+    max-pool windows, strides, padding modes with tied values (outputs, argmax and routed
+    gradients bit-exact)."""
+    rng = np.random.default_rng(21)
+    for _ in range(30):
+        ni = int(rng.choice([1, 7, 10, 64, 100, 120, 256, 300, 512, 1000, 1024, 2048]))
+        no = int(rng.choice([1, 2, 10, 33, 64, 100, 256, 500]))
+        bs = int(rng.choice([1, 2, 5, 16, 17, 64, 128]))
+        what = f"fc {(ni, no, bs)}"
+        x = rng.standard_normal((bs, ni)).astype(np.float32)
+        w = rng.uniform(-0.2, 0.2, ni * no).astype(np.float32)
+        b = rng.standard_normal(no).astype(np.float32)
+        dy = rng.standard_normal((bs, no)).astype(np.float32)
+        xd, wd, bd, dyd = T.to_device(x), T.to_device(w), T.to_device(b), T.to_device(dy)
+        y, dx, dw, db = T.DevBuf((bs, no)), T.DevBuf((bs, ni)), T.DevBuf((ni * no,)), T.DevBuf((no,))
+        T.fc_fwd(ni, no, True, bs, xd, wd, bd, y)
+        T.fc_bwd(ni, no, True, bs, xd, wd, dyd, dx, dw, db)
+        rdx, rdw, rdb = O.fc_bwd(x, w, dy)
+        assert_close(y.numpy(), O.fc_fwd(x, w, b), what=what + " y")
+        assert_close(dx.numpy(), rdx, what=what + " dx")
+        assert_close(dw.numpy(), rdw, what=what + " dw")
+        assert_close(db.numpy(), rdb, what=what + " db")
+    done = 0
+    while done < 40:
+        c = int(rng.choice([1, 3, 8, 33]))
+        iw, ih = int(rng.integers(2, 40)), int(rng.integers(2, 30))
+        pw, ph = int(rng.choice([2, 2, 3])), int(rng.choice([2, 2, 3]))
+        sw, sh = int(rng.choice([1, 2, 2, 3])), int(rng.choice([1, 2, 2, 3]))
+        same, ceil = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        bs = int(rng.choice([1, 3, 8]))
+        if not same and (iw < pw or ih < ph):
+            continue
+        kw = dict(pad_same=same, ceil_mode=ceil)
+        d, do = T.pool_desc(iw, ih, c, pw, ph, sw, sh, **kw), O.pool_desc(iw, ih, c, pw, ph, sw, sh, **kw)
+        ow, oh = T.pool_out_shape(d)
+        if ow < 1 or oh < 1:
+            continue
+        what = f"maxpool {(iw, ih, c, pw, ph, sw, sh, same, ceil, bs)}"
+        x = rng.standard_normal((bs, c * ih * iw)).astype(np.float32)
+        x[rng.random(x.shape) < 0.2] = 0.5  # ties
+        dy = rng.standard_normal((bs, c * oh * ow)).astype(np.float32)
+        ry, ram = O.maxpool_fwd(do, x)
+        y, am, dx = T.DevBuf((bs, c * oh * ow)), T.DevBuf((bs, c * oh * ow), np.int32), T.DevBuf(x.shape)
+        T.maxpool_fwd(d, bs, T.to_device(x), y, am)
+        T.maxpool_bwd(d, bs, T.to_device(dy), am, dx)
+        assert np.array_equal(y.numpy(), ry), what
+        assert np.array_equal(am.numpy().astype(np.int64), ram), what
+        assert np.array_equal(dx.numpy(), O.maxpool_bwd(do, dy, ram)), what
+        done += 1
