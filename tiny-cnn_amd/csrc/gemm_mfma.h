@@ -26,6 +26,8 @@
 //
 // Epilogue concept
 //   struct Epi { struct Col; __device__ Col col(int n) const;
+//                __device__ float prior(int m, const Col&) const;   // old value if the store adds
+//                __device__ void store(int m, const Col&, float v, float prior) const;
 //                __device__ void store(int m, const Col&, float v) const; };
 #pragma once
 
@@ -95,13 +97,19 @@ struct EpiRowMajor {
     float bias;
   };
   __device__ __forceinline__ Col col(int n) const { return {n, bias_n ? bias_n[n] : 0.0f}; }
-  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+  // what the output holds before the store, when the store adds to it (else 0). A kernel that
+  // stores several values a lane asks for all of them first: loads between its stores would
+  // each wait for the store before (they may alias), one trip to memory per value.
+  __device__ __forceinline__ float prior(int m, const Col &c) const {
+    return accumulate ? out[m * ld + c.n] : 0.0f;
+  }
+  __device__ __forceinline__ void store(int m, const Col &c, float v, float before) const {
     const int idx = m * ld + c.n;
     v += c.bias;
     if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[idx]);
-    if (accumulate) v += out[idx];
-    out[idx] = v;
+    out[idx] = v + before;
   }
+  __device__ __forceinline__ void store(int m, const Col &c, float v) const { store(m, c, v, prior(m, c)); }
 };
 
 // forward product followed by a pointwise activation layer:
@@ -117,7 +125,8 @@ struct EpiRowMajorAct {
     float bias;
   };
   __device__ __forceinline__ Col col(int n) const { return {n, bias_n ? bias_n[n] : 0.0f}; }
-  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+  __device__ __forceinline__ float prior(int, const Col &) const { return 0.0f; }
+  __device__ __forceinline__ void store(int m, const Col &c, float v, float = 0.0f) const {
     const int idx = m * ld + c.n;
     v += c.bias;
     out[idx]     = v;
@@ -140,7 +149,8 @@ struct EpiImageRows {
     pix_div.divmod(static_cast<uint32_t>(n), img, p);
     return {static_cast<int>(img) * rows * pix + static_cast<int>(p)};
   }
-  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+  __device__ __forceinline__ float prior(int, const Col &) const { return 0.0f; }
+  __device__ __forceinline__ void store(int m, const Col &c, float v, float = 0.0f) const {
     const int idx = c.base + m * pix;
     if (bias_m) v += bias_m[m];
     if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[idx]);
@@ -165,7 +175,8 @@ struct EpiImageRowsAct {
     pix_div.divmod(static_cast<uint32_t>(n), img, p);
     return {static_cast<int>(img) * rows * pix + static_cast<int>(p)};
   }
-  __device__ __forceinline__ void store(int m, const Col &c, float v) const {
+  __device__ __forceinline__ float prior(int, const Col &) const { return 0.0f; }
+  __device__ __forceinline__ void store(int m, const Col &c, float v, float = 0.0f) const {
     const int idx = c.base + m * pix;
     if (bias_m) v += bias_m[m];
     out[idx]     = v;
@@ -445,12 +456,19 @@ gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const
     } else {
       const typename Epi::Col c = epi.col(n);
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i) {
+        float before[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-          if (m < M) epi.store(m, c, acc[i][j][r]);
+          before[r]   = m < M ? epi.prior(m, c) : 0.0f;
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if (m < M) epi.store(m, c, acc[i][j][r], before[r]);
+        }
+      }
     }
   }
 }
