@@ -82,10 +82,16 @@ __device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const Str
   const int n = n0 + tn;
   if (n < N) {
     const typename Epi::Col c = epi.col(n);
+    float before[4];  // all loads before the first store: a load behind a store waits for it
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = m0 + 4 * tmg + i;
-      if (m < M) epi.store(m, c, acc[i]);
+      before[i]   = m < M ? epi.prior(m, c) : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 4 * tmg + i;
+      if (m < M) epi.store(m, c, acc[i], before[i]);
     }
   }
 }
