@@ -265,23 +265,28 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
 #pragma unroll
     for (int i = 0; i < DXS_PX; ++i) acc[c][i] = 0.0f;
 
-  // staging plan: element e = tid + DXS_NT*j of the chunk tile -> global offset or -1
+  // staging plan, the same for every chunk: element e = tid + DXS_NT*j of the chunk tile ->
+  // channel inside the chunk and offset inside that channel's plane (-1: outside the image)
   float stage[DXS_MAX_STAGE];
-  auto fetch = [&](int co0) {
-    const int nco = min(DXS_CO_CHUNK, g.Kc - co0);
+  int soff[DXS_MAX_STAGE], sch[DXS_MAX_STAGE];
 #pragma unroll
-    for (int j = 0; j < DXS_MAX_STAGE; ++j) {
-      const uint32_t e = tid + DXS_NT * j;
-      uint32_t c, rem, r, q;
-      p.div_tile.divmod(e, c, rem);
-      p.div_tcols.divmod(rem, r, q);
-      const int oy = oy0 + static_cast<int>(r), ox = ox0 + static_cast<int>(q);
-      float v = 0.0f;
-      if (static_cast<int>(c) < nco && static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
-          static_cast<unsigned>(ox) < static_cast<unsigned>(g.OW))
-        v = dy_img[(co0 + c) * ohw + oy * g.OW + ox];
-      stage[j] = v;
-    }
+  for (int j = 0; j < DXS_MAX_STAGE; ++j) {
+    const uint32_t e = tid + DXS_NT * j;
+    uint32_t c, rem, r, q;
+    p.div_tile.divmod(e, c, rem);
+    p.div_tcols.divmod(rem, r, q);
+    const int oy = oy0 + static_cast<int>(r), ox = ox0 + static_cast<int>(q);
+    const bool in = static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
+                    static_cast<unsigned>(ox) < static_cast<unsigned>(g.OW);
+    sch[j]  = static_cast<int>(c);
+    soff[j] = in ? static_cast<int>(c) * ohw + oy * g.OW + ox : -1;
+  }
+  auto fetch = [&](int co0) {
+    const int nco     = min(DXS_CO_CHUNK, g.Kc - co0);
+    const float *base = dy_img + co0 * ohw;
+#pragma unroll
+    for (int j = 0; j < DXS_MAX_STAGE; ++j)
+      stage[j] = (soff[j] >= 0 && sch[j] < nco) ? base[soff[j]] : 0.0f;
   };
 
   fetch(0);
