@@ -281,12 +281,31 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
     sch[j]  = static_cast<int>(c);
     soff[j] = in ? static_cast<int>(c) * ohw + oy * g.OW + ox : -1;
   }
+  // The chunk's weights as [c][tap] -> (w[ci=0..3]), taps flipped so that the inner loops walk
+  // the tile forwards. The first two per thread travel with the tile (512 cover 8 channels of
+  // up to 8x8 taps); loaded behind the barrier they would cost a trip to memory per chunk.
+  float4 wreg[2];
+  auto load_w = [&](int co0, int e) {
+    const int c = e / rs, t = e - c * rs;
+    const float *wc = w + (static_cast<size_t>(co0 + c) * g.C) * rs + (rs - 1 - t);
+    float4 v;
+    v.x = wc[0];
+    v.y = g.C > 1 ? wc[rs] : 0.0f;
+    v.z = g.C > 2 ? wc[2 * rs] : 0.0f;
+    v.w = g.C > 3 ? wc[3 * rs] : 0.0f;
+    return v;
+  };
   auto fetch = [&](int co0) {
     const int nco     = min(DXS_CO_CHUNK, g.Kc - co0);
     const float *base = dy_img + co0 * ohw;
 #pragma unroll
     for (int j = 0; j < DXS_MAX_STAGE; ++j)
       stage[j] = (soff[j] >= 0 && sch[j] < nco) ? base[soff[j]] : 0.0f;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int e = tid + DXS_NT * k;
+      wreg[k]     = e < nco * rs ? load_w(co0, e) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
   };
 
   fetch(0);
@@ -298,18 +317,12 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
       const int e = tid + DXS_NT * j;
       if (e < DXS_CO_CHUNK * tsz) tile[e] = stage[j];
     }
-    // weights of the chunk as [c][tap] -> (w[ci=0..3]); taps stored flipped so that the
-    // inner loops walk the tile forwards
-    for (int e = tid; e < nco * rs; e += DXS_NT) {
-      const int c = e / rs, t = e - c * rs;
-      const float *wc = w + (static_cast<size_t>(co0 + c) * g.C) * rs + (rs - 1 - t);
-      float4 v;
-      v.x = wc[0];
-      v.y = g.C > 1 ? wc[rs] : 0.0f;
-      v.z = g.C > 2 ? wc[2 * rs] : 0.0f;
-      v.w = g.C > 3 ? wc[3 * rs] : 0.0f;
-      wl[e] = v;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int e = tid + DXS_NT * k;
+      if (e < nco * rs) wl[e] = wreg[k];
     }
+    for (int e = tid + 2 * DXS_NT; e < nco * rs; e += DXS_NT) wl[e] = load_w(co0, e);  // larger windows
     __syncthreads();
     if (co0 + DXS_CO_CHUNK < g.Kc) fetch(co0 + DXS_CO_CHUNK);  // in flight during the math
 
