@@ -338,6 +338,24 @@ def test_activations_match_oracle(T, O, kind, shape):
     assert_close(dx.numpy(), O.act_bwd(kind, x, ry, dy), 1e-5, "backward")
 
 
+@pytest.mark.parametrize("shape,scale", [((1, 255), 20.0), ((3, 10), 50.0), ((16, 1000), 8.0)])
+def test_softmax_backward_of_saturated_rows_matches_oracle(T, O, shape, scale):
+    """Rows whose largest output is next to 1: every term of the reference's Jacobian row is
+    small there, and y*(dy - <dy, y>) in float would lose the element of the largest output."""
+    rng = np.random.default_rng(int(scale))
+    x = (rng.standard_normal(shape) * scale).astype(np.float32)
+    x[np.arange(shape[0]), rng.integers(0, shape[1], shape[0])] += 5 * scale
+    dy = rng.standard_normal(shape).astype(np.float32)
+    ry = O.act_fwd("softmax", x)
+    assert ry.max(axis=1).min() > 0.9
+    dx = T.DevBuf(shape)
+    T.act_bwd("softmax", shape[0], shape[1], T.to_device(ry), T.to_device(dy), dx)
+    want = O.act_bwd("softmax", x, ry, dy)
+    got = dx.numpy()
+    for r in range(shape[0]):   # row by row: a saturated row's gradient is tiny beside the others'
+        assert_close(got[r], want[r], REL_TOL, f"row {r}")
+
+
 def test_unaligned_views_take_the_scalar_path(T, O):
     """Sub-tensors that are not 16-byte aligned still give the same results."""
     rng = np.random.default_rng(5)

@@ -252,7 +252,13 @@ softmax_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, const int
   for (int j = lane; j < len; j += 64) yr[j] = yr[j] / s;
 }
 
-// softmax_layer.h:36-55: dx_j = sum_k dy_k * (delta_jk*y_j - y_j*y_k) = y_j * (dy_j - <dy, y>)
+// softmax_layer.h:36-55: dx_j = sum_k dy_k * df_k with df_j = y_j*(1 - y_j), df_k = -y_k*y_j,
+// that is dx_j = dy_j*y_j*(1 - y_j) - y_j * sum_{k != j} dy_k*y_k. The reference adds the terms
+// one by one, so a term that dwarfs the others (a saturated row: one y next to 1, the rest
+// 1e-20) does not disturb the sums it is not part of. In one pass over the row the same is
+// had by leaving the largest term t_m = dy_m*y_m out of the row sum (kept in double):
+// sum_{k != m} is that sum itself, and sum_{k != j} = that sum - t_j + t_m for the others,
+// where t_m dominates whatever the subtraction lost.
 __global__ void __launch_bounds__(EW_THREADS)
 softmax_bwd_kernel(const float *__restrict__ y, const float *__restrict__ dy,
                    float *__restrict__ dx, const int batch, const int len) {
@@ -261,11 +267,31 @@ softmax_bwd_kernel(const float *__restrict__ y, const float *__restrict__ dy,
   if (row >= batch) return;
   const float *yr  = y + static_cast<size_t>(row) * len;
   const float *dyr = dy + static_cast<size_t>(row) * len;
-  float dot        = 0.0f;
-  for (int j = lane; j < len; j += 64) dot += dyr[j] * yr[j];
-  dot = wave_sum(dot);
+  // the largest |dy_k*y_k| of the row; of equal ones the first
+  float big = -1.0f;
+  int m     = len;
+  for (int j = lane; j < len; j += 64) {
+    const float t = fabsf(dyr[j] * yr[j]);
+    if (t > big) { big = t; m = j; }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(big, off, 64);
+    const int om   = __shfl_xor(m, off, 64);
+    if (ob > big || (ob == big && om < m)) { big = ob; m = om; }
+  }
+  double rest_m = 0.0;  // sum over k != m
   for (int j = lane; j < len; j += 64)
-    dx[static_cast<size_t>(row) * len + j] = yr[j] * (dyr[j] - dot);
+    if (j != m) rest_m += static_cast<double>(dyr[j]) * static_cast<double>(yr[j]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) rest_m += __shfl_xor(rest_m, off, 64);
+  const double tm = m < len ? static_cast<double>(dyr[m]) * static_cast<double>(yr[m]) : 0.0;
+  for (int j = lane; j < len; j += 64) {
+    const float yj = yr[j], dj = dyr[j];
+    const double own  = static_cast<double>(dj) * static_cast<double>(yj * (1.0f - yj));
+    const double rest = j == m ? rest_m : rest_m - static_cast<double>(dj) * static_cast<double>(yj) + tm;
+    dx[static_cast<size_t>(row) * len + j] = static_cast<float>(own - static_cast<double>(yj) * rest);
+  }
 }
 
 // softmax backward of cross_entropy_multiclass::df (= -t/y) in closed form:
