@@ -552,6 +552,84 @@ def test_randomized_conv_shapes_match_oracle(T, O, seed):
         done += 1
 
 
+def test_randomized_conv_and_fc_options_match_oracle(T, O):
+    """A seeded sweep over what a caller may leave out or ask for: no bias, any subset of the
+    three gradients (NULL outputs are skipped), accumulation onto prior dW/db, windows that are
+    not square (1x1 up to 7x7), different strides along the two axes; on shapes that pick the
+    few-channel kernels as well as the tiled ones."""
+    rng = np.random.default_rng(31)
+    done = 0
+    while done < 70:
+        kw = int(rng.choice([1, 2, 3, 3, 5, 5, 7]))
+        kh = kw if rng.random() < 0.6 else int(rng.choice([1, 2, 3, 5]))
+        big = rng.random() < 0.5
+        ic = int(rng.choice([16, 32, 48, 64] if big else [1, 2, 3, 4, 6, 8, 20]))
+        oc = int(rng.choice([16, 32, 64, 96] if big else [1, 3, 6, 16, 33]))
+        iw, ih = int(rng.integers(max(kw, 4), 36)), int(rng.integers(max(kh, 4), 28))
+        if big and rng.random() < 0.6:
+            iw, ih = int(rng.choice([8, 12, 16, 24, 32])), int(rng.choice([8, 16, 24, 32]))
+        same = bool(rng.integers(0, 2))
+        sw = int(rng.choice([1, 1, 1, 2]))
+        sh = sw if rng.random() < 0.7 else int(rng.choice([1, 2, 3]))
+        bias, acc = bool(rng.random() < 0.7), bool(rng.integers(0, 2))
+        want = [bool(v) for v in rng.integers(0, 2, 3)]   # dx, dw, db
+        if not any(want):
+            want[1] = True
+        want[2] = want[2] and bias
+        bs = int(rng.choice([1, 2, 4, 7, 16]))
+        if iw < kw or ih < kh:
+            continue
+        opts = dict(pad_same=same, has_bias=bias, w_stride=sw, h_stride=sh)
+        d, do = T.conv_desc(iw, ih, ic, kw, kh, oc, **opts), O.conv_desc(iw, ih, ic, kw, kh, oc, **opts)
+        ow, oh = T.conv_out_shape(d)
+        if ow < 1 or oh < 1:
+            continue
+        what = f"conv {(iw, ih, ic, kw, kh, oc, same, sw, sh, bias, acc, want, bs)}"
+        x = rng.standard_normal((bs, ic * ih * iw)).astype(np.float32)
+        w = rng.uniform(-0.3, 0.3, oc * ic * kh * kw).astype(np.float32)
+        b = rng.standard_normal(oc).astype(np.float32)
+        dy = rng.standard_normal((bs, oc * oh * ow)).astype(np.float32)
+        prior = [rng.standard_normal(n).astype(np.float32) for n in (x.shape, w.shape, (oc,))]
+        xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+        y = T.DevBuf((bs, oc * oh * ow))
+        T.conv2d_fwd(d, bs, xd, wd, T.to_device(b) if bias else None, y)
+        assert_close(y.numpy(), O.conv2d_fwd(do, x, w, b if bias else None), what=what + " y")
+        out = [T.to_device(p0) if wanted else None for p0, wanted in zip(prior, want)]
+        T.conv2d_bwd(d, bs, xd, wd, dyd, out[0], out[1], out[2], acc)
+        ref = O.conv2d_bwd(do, x, w, dy)
+        for k, name in enumerate(("dx", "dw", "db")):
+            if want[k]:
+                base = prior[k] if acc and k > 0 else 0.0     # dX is always overwritten
+                assert_close(out[k].numpy(), ref[k] + base, what=f"{what} {name}")
+        done += 1
+    for _ in range(40):
+        ni = int(rng.choice([1, 7, 64, 120, 256, 512, 1000, 2048]))
+        no = int(rng.choice([1, 10, 33, 64, 256, 1024]))
+        bs = int(rng.choice([1, 2, 16, 17, 128]))
+        bias, acc = bool(rng.random() < 0.7), bool(rng.integers(0, 2))
+        want = [bool(v) for v in rng.integers(0, 2, 3)]
+        if not any(want):
+            want[0] = True
+        want[2] = want[2] and bias
+        what = f"fc {(ni, no, bs, bias, acc, want)}"
+        x = rng.standard_normal((bs, ni)).astype(np.float32)
+        w = rng.uniform(-0.2, 0.2, ni * no).astype(np.float32)
+        b = rng.standard_normal(no).astype(np.float32)
+        dy = rng.standard_normal((bs, no)).astype(np.float32)
+        prior = [rng.standard_normal(n).astype(np.float32) for n in (x.shape, w.shape, (no,))]
+        xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+        y = T.DevBuf((bs, no))
+        T.fc_fwd(ni, no, bias, bs, xd, wd, T.to_device(b) if bias else None, y)
+        assert_close(y.numpy(), O.fc_fwd(x, w, b if bias else None), what=what + " y")
+        out = [T.to_device(p0) if wanted else None for p0, wanted in zip(prior, want)]
+        T.fc_bwd(ni, no, bias, bs, xd, wd, dyd, out[0], out[1], out[2], acc)
+        ref = O.fc_bwd(x, w, dy)
+        for k, name in enumerate(("dx", "dw", "db")):
+            if want[k]:
+                base = prior[k] if acc and k > 0 else 0.0
+                assert_close(out[k].numpy(), ref[k] + base, what=f"{what} {name}")
+
+
 def test_randomized_fc_and_maxpool_shapes_match_oracle(T, O):
     """Seeded sweeps: fully-connected layers across the small / tiled / split products, and
     max-pool windows, strides, padding modes with tied values (outputs, argmax and routed
