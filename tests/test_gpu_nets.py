@@ -251,6 +251,66 @@ def test_first_conv_with_pool_in_its_kernel_matches_oracle(T, O, W, spec):
         net.close()
 
 
+@pytest.mark.parametrize("spec,batch", [
+    # both limits of the one-launch kernel (128 inputs, 64 outputs), relu folded, ragged batch
+    ([("fc", 100, 128), ("act", "relu"), ("fc", 128, 64), ("act", "softmax")], 37),
+    # the fully-connected layer is the first layer: its dX is the net's input gradient
+    ([("fc", 30, 10), ("act", "softmax")], 5),
+    # 70 inputs: a second, partial block of dX columns; tanh folded
+    ([("fc", 50, 70), ("act", "tanh"), ("fc", 70, 3), ("act", "softmax")], 16),
+    # a pool in front: nothing to fold
+    ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("fc", 64, 10), ("act", "softmax")], 9),
+    # too wide for the one-launch kernel: the three separate launches
+    ([("fc", 20, 200), ("act", "relu"), ("fc", 200, 10), ("act", "softmax")], 8),
+])
+@pytest.mark.parametrize("targets", ["one_hot", "soft"])
+def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch, targets):
+    """A fusing net trained with cross_entropy_multiclass runs its last fully-connected layer,
+    the softmax, the loss gradient and that layer's dX as one kernel: outputs and gradients
+    against the oracle, and bit for bit against the same net without fusion (same terms, same
+    order), for one-hot and for soft targets."""
+    rng = np.random.default_rng(len(spec) * 17 + batch)
+    nets = [T.Net(W.build_layers(T, spec), batch, f) for f in (0, T.NET_FUSE_ACT_GRAD)]
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for i, l in enumerate(spec):
+        nw, nb, fan_in, _ = W.layer_fans(l)
+        if nw:
+            w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+            b = rng.uniform(-0.5, 0.5, nb).astype(np.float32)
+            for net in nets:
+                net.set_param(i, 0, w); net.set_param(i, 1, b)
+            ref.weight(i)[:] = w; ref.bias(i)[:] = b
+    first, classes = spec[0], spec[-2][2]
+    n_in = first[1] if first[0] == "fc" else first[1] * first[2] * first[3]
+    x = rng.standard_normal((batch, n_in)).astype(np.float32)
+    one_hot = np.eye(classes, dtype=np.float32)[rng.integers(0, classes, batch)]
+    soft = rng.uniform(0.0, 1.0, (batch, classes)).astype(np.float32)
+    xd = T.to_device(x)
+    for t in ((one_hot,) if targets == "one_hot" else (soft,)):
+        td = T.to_device(t)
+        ref.train_step(O.opt_desc("sgd"), "ce_multiclass", x, t, do_update=False)
+        for net in nets:
+            net.train_step(None, "ce_multiclass", batch, xd, td, do_update=False)
+            for i, l in enumerate(spec):
+                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+                if net.param_size(i, 0):
+                    assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
+                    assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")
+            assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, "input gradient")
+        for i in range(len(spec)):
+            assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
+        # (a folded activation gradient rounds differently from the activation layer's own kernel,
+        # so the layers in front agree to rounding only)
+        last_fc = len(spec) - 2
+        for which in (0, 1):
+            assert np.array_equal(nets[0].layer_grad(last_fc, which), nets[1].layer_grad(last_fc, which)), \
+                f"last layer's gradient {which} fused vs not"
+        if last_fc == 0:
+            assert np.array_equal(nets[0].layer_dx(0, batch), nets[1].layer_dx(0, batch)), "input gradient fused vs not"
+    for net in nets:
+        net.close()
+
+
 def test_feeder_double_buffered_batches_match_oracle(T, O, W):
     """tdh_feeder_*: different host batches every step, a short last batch, graph replay from
     the two alternating device slots; updated weights against the oracle after every step."""

@@ -295,7 +295,8 @@ softmax_bwd_kernel(const float *__restrict__ y, const float *__restrict__ dy,
 }
 
 // softmax backward of cross_entropy_multiclass::df (= -t/y) in closed form:
-// dz_j = y_j * (-t_j/y_j + sum_k t_k) = y_j * sum(t) - t_j
+// dz_j = y_j * (-t_j/y_j + sum_k t_k) = y_j * sum(t) - t_j, as one fused multiply-add in every
+// kernel that computes it (left to the compiler, one kernel fused it and another did not)
 __global__ void __launch_bounds__(EW_THREADS)
 softmax_xent_grad_kernel(const float *__restrict__ y, const float *__restrict__ t,
                          float *__restrict__ dz, const int batch, const int len) {
@@ -307,7 +308,7 @@ softmax_xent_grad_kernel(const float *__restrict__ y, const float *__restrict__ 
   float st        = 0.0f;
   for (int j = lane; j < len; j += 64) st += tr[j];
   st = wave_sum(st);
-  for (int j = lane; j < len; j += 64) dz[static_cast<size_t>(row) * len + j] = yr[j] * st - tr[j];
+  for (int j = lane; j < len; j += 64) dz[static_cast<size_t>(row) * len + j] = fmaf(yr[j], st, -tr[j]);
 }
 
 // softmax forward and the gradient above in one pass over the row: the values and their order
@@ -338,7 +339,7 @@ softmax_fwd_xent_kernel(const float *__restrict__ x, const float *__restrict__ t
   for (int j = lane; j < len; j += 64) {
     const float v = yr[j] / s;
     yr[j]         = v;
-    dr[j]         = v * st - tr[j];
+    dr[j]         = fmaf(v, st, -tr[j]);
   }
 }
 

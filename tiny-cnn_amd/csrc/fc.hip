@@ -5,6 +5,8 @@
 //   dW       dW[c][o] = sum_s X[s][c] * dY[s][o]              M=in    N=out K=batch
 // dW is reduced over the batch inside the GEMM (K spans the samples) instead of being stored
 // per sample and merged afterwards (fully_connected_op_internal.h:54-60, node.h:89-103).
+#include <cfloat>
+
 #include "gemm_mfma.h"
 
 namespace tdh {
@@ -28,17 +30,18 @@ struct SfcSmem {
   float Bs[SFC_KC][SFC_TN + 1];
 };
 
-// One 16 x 64 tile (bx, by) of C = A * B with the epilogue applied. The next panel's loads are
-// issued before the current panel is multiplied.
-template <class Epi>
-__device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const StridedOperand &b,
-                                              const Epi &epi, const int M, const int N, const int K,
-                                              const int bx, const int by, SfcSmem &sm) {
+// One 16 x 64 tile (bx, by) of C = A * B: acc[i] is row 4*(tid/64) + i, column tid%64 of the
+// tile. The next panel's loads are issued before the current panel is multiplied. The last
+// panel stays in LDS (rows past K hold zeros).
+__device__ __forceinline__ void small_fc_accumulate(const StridedOperand &a, const StridedOperand &b,
+                                                    const int M, const int N, const int K,
+                                                    const int bx, const int by, SfcSmem &sm,
+                                                    float (&acc)[4]) {
   const int tid = threadIdx.x, tn = tid & 63, tmg = tid >> 6;
   const int m0 = by * SFC_TM, n0 = bx * SFC_TN;
   // staging coordinates: consecutive threads walk the operand's contiguous direction
   const bool a_k_fast = a.s_k == 1, b_k_fast = b.s_k == 1;
-  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  acc[0] = acc[1] = acc[2] = acc[3] = 0.0f;
   float ra[SFC_NA], rb[SFC_NB];
   auto fetch = [&](int k0) {
 #pragma unroll
@@ -69,8 +72,10 @@ __device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const Str
     }
     __syncthreads();
     if (k0 + SFC_KC < K) fetch(k0 + SFC_KC);
+    // the rows of the panel past K hold zeros: a short product leaves them out, eight at a time
+    const int kend = min(SFC_KC, (K - k0 + 7) & ~7);
 #pragma unroll 8
-    for (int k = 0; k < SFC_KC; ++k) {
+    for (int k = 0; k < kend; ++k) {
       const float4 av = *reinterpret_cast<const float4 *>(&sm.As[k][4 * tmg]);
       const float bv  = sm.Bs[k][tn];
       acc[0] += av.x * bv;
@@ -79,6 +84,17 @@ __device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const Str
       acc[3] += av.w * bv;
     }
   }
+}
+
+// The tile with the epilogue applied.
+template <class Epi>
+__device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const StridedOperand &b,
+                                              const Epi &epi, const int M, const int N, const int K,
+                                              const int bx, const int by, SfcSmem &sm) {
+  const int tn = threadIdx.x & 63, tmg = threadIdx.x >> 6;
+  const int m0 = by * SFC_TM, n0 = bx * SFC_TN;
+  float acc[4];
+  small_fc_accumulate(a, b, M, N, K, bx, by, sm, acc);
   const int n = n0 + tn;
   if (n < N) {
     const typename Epi::Col c = epi.col(n);
@@ -144,6 +160,111 @@ __global__ void __launch_bounds__(SFC_NT) fc_bwd_fused_kernel(const FcBwdFused f
   }
 }
 
+// The last fully-connected layer of a net that ends in softmax and is trained with
+// cross_entropy_multiclass, from its input to the gradient of its input in one launch: every
+// step of that chain stays inside a sample row (only the weight and bias gradients add over
+// the batch; they are another launch, off the chain the next layer waits for). A workgroup
+// takes 16 rows. The product is small_fc_accumulate's, the softmax and the loss gradient are
+// softmax_fwd_xent_kernel's butterflies (a row's outputs sit in the lanes of one wave), the
+// input gradient is the dX product of fc_bwd with the filters still in LDS: same terms, same
+// order, same results as the three launches.
+struct FcTail {
+  StridedOperand a, b;  // X[s][k], W[k][n]
+  const float *bias;    // or null
+  float *out, *soft;    // the layer's output and the softmax layer's
+  const float *t;
+  float *dz;
+  EpiRowMajor xepi;     // dX (with the activation gradient of the layer in front folded in)
+  int M, N, K;          // batch, out, in
+};
+
+__device__ __forceinline__ float sfc_wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float sfc_wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__global__ void __launch_bounds__(SFC_NT) fc_softmax_xent_kernel(const FcTail f) {
+  __shared__ SfcSmem sm;
+  const int tn = threadIdx.x & 63, tmg = threadIdx.x >> 6;
+  const int m0 = blockIdx.x * SFC_TM;
+  // Everything the later phases read from memory is asked for now, with the panels: each of
+  // these loads would otherwise be a trip to memory of its own in a chain that has nothing to
+  // hide it behind. prev[] is the output of the activation in front (for its gradient factor)
+  // at this thread's first 64 dX columns.
+  const bool col   = tn < f.N;
+  const float bias = (col && f.bias) ? f.bias[tn] : 0.0f;
+  const int ag     = f.xepi.ag.kind;
+  float tv[4], prev[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + 4 * tmg + i;
+    tv[i]       = (col && m < f.M) ? f.t[m * f.N + tn] : 0.0f;
+    prev[i]     = (ag != TDH_ACT_NONE && tn < f.K && m < f.M) ? f.xepi.ag.y[m * f.K + tn] : 0.0f;
+  }
+  float acc[4];
+  small_fc_accumulate(f.a, f.b, f.M, f.N, f.K, 0, blockIdx.x, sm, acc);
+  // every lane takes part in the butterflies; the lanes past the row's end hold neutral values
+  float dzv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m     = m0 + 4 * tmg + i;
+    const bool live = col && m < f.M;
+    const int idx   = m * f.N + tn;
+    const float v   = (acc[i] + bias) + 0.0f;
+    const float mx  = sfc_wave_max(col ? fmaxf(-FLT_MAX, v) : -FLT_MAX);
+    const float e   = col ? expf(v - mx) : 0.0f;
+    const float se  = sfc_wave_sum(e);
+    const float st  = sfc_wave_sum(tv[i]);
+    const float y   = e / se;
+    dzv[i]          = live ? fmaf(y, st, -tv[i]) : 0.0f;
+    if (live) {
+      f.out[idx]  = v;
+      f.soft[idx] = y;
+      f.dz[idx]   = dzv[i];
+    }
+  }
+  // dX[m][c] = sum_o dz[m][o] * W[c][o]: the tile of dz takes the place of the panel of X
+  __syncthreads();
+  float *dzs = &sm.As[0][0];  // [SFC_TM][SFC_TN]
+#pragma unroll
+  for (int i = 0; i < 4; ++i) dzs[(4 * tmg + i) * SFC_TN + tn] = dzv[i];
+  __syncthreads();
+  for (int c0 = 0; c0 < f.K; c0 += 64) {
+    const int c = c0 + tn;
+    if (c0 > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + 4 * tmg + i;
+        prev[i]     = (ag != TDH_ACT_NONE && c < f.K && m < f.M) ? f.xepi.ag.y[m * f.K + c] : 0.0f;
+      }
+    }
+    float g[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int o = 0; o < f.N; ++o) {
+      const float bv = sm.Bs[c][o];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) g[i] += dzs[(4 * tmg + i) * SFC_TN + o] * bv;
+    }
+    if (c < f.K) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + 4 * tmg + i;
+        if (m < f.M) {
+          // the steps of EpiRowMajor::store without a bias, not accumulating
+          float v = g[i] + 0.0f;
+          if (ag != TDH_ACT_NONE) v *= act_grad_factor(ag, prev[i]);
+          f.xepi.out[m * f.K + c] = v + 0.0f;
+        }
+      }
+    }
+  }
+}
+
 bool small_fc_applies(int M, int N, int K) {
   return K <= 4 * SFC_KC && static_cast<long>(M) * N <= (1L << 18) &&
          static_cast<long>(M) * N * K <= (1L << 24);
@@ -164,6 +285,29 @@ int launch_small_fc(const StridedOperand &a, const StridedOperand &b, const Epi 
 // dX, dW and db of this layer leave one launch (when all three are asked for)
 bool fc_bwd_fuses(int in, int out, int batch) {
   return small_fc_applies(batch, in, out) && small_fc_applies(in, out, batch);
+}
+
+// forward, softmax, cross-entropy gradient and dX of this layer can leave one launch
+bool fc_softmax_xent_applies(int in, int out, int batch) {
+  return in <= SFC_KC && out <= SFC_TN && small_fc_applies(batch, out, in) && small_fc_applies(batch, in, out);
+}
+
+int fc_softmax_xent(int in, int out, int has_bias, int batch, const float *x, const float *w,
+                    const float *b, float *y, float *soft, const float *t, float *dz, float *dx,
+                    ActGrad dx_act) {
+  if (!fc_softmax_xent_applies(in, out, batch))
+    return set_error(TDH_ERR_INVALID, "fc_softmax_xent: layer too large for the one-launch kernel");
+  FcTail f;
+  f.a    = StridedOperand{x, in, 1, batch};
+  f.b    = StridedOperand{w, 1, out, out};
+  f.bias = has_bias ? b : nullptr;
+  f.out = y; f.soft = soft; f.t = t; f.dz = dz;
+  f.xepi = EpiRowMajor{dx, in, nullptr, dx_act, 0};
+  f.M = batch; f.N = out; f.K = in;
+  ProfScope prof("fc_fwd_softmax_xent_dx", 4.0 * batch * in * out, WORK_FLOP);
+  TDH_LAUNCH(fc_softmax_xent_kernel, dim3(ceil_div(batch, SFC_TM)), dim3(SFC_NT), 0, ctx().stream, f);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
 }
 
 size_t fc_workspace_bytes(int in, int out, int batch) {
@@ -189,23 +333,24 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
 
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act) {
-  if (dx && dw && fc_bwd_fuses(in, out, batch)) {
+  const bool bias_grad = db && has_bias;
+  if (dw && (dx || bias_grad) && fc_bwd_fuses(in, out, batch)) {
     FcBwdFused f;
     f.xa = StridedOperand{dy, out, 1, batch};
     f.xb = StridedOperand{w, out, 1, in};
     f.xepi = EpiRowMajor{dx, in, nullptr, dx_act, 0};
     f.xM = batch; f.xN = in; f.xK = out;
     f.x_tiles_n = ceil_div(in, SFC_TN);
-    f.nx = f.x_tiles_n * ceil_div(batch, SFC_TM);
+    f.nx = dx ? f.x_tiles_n * ceil_div(batch, SFC_TM) : 0;  // no dX: its workgroups are left out
     f.wa = StridedOperand{x, 1, in, in};
     f.wb = StridedOperand{dy, 1, out, out};
     f.wepi = EpiRowMajor{dw, out, nullptr, ActGrad(), accumulate};
     f.wM = in; f.wN = out; f.wK = batch;
     f.w_tiles_n = ceil_div(out, SFC_TN);
     f.nw = f.w_tiles_n * ceil_div(in, SFC_TM);
-    const bool bias = db && has_bias;
+    const bool bias = bias_grad;
     f.dy = dy; f.db = db; f.batch = batch; f.out = out; f.db_accumulate = accumulate;
-    ProfScope prof("fc_bwd_small", 4.0 * batch * in * out, WORK_FLOP);
+    ProfScope prof(dx ? "fc_bwd_small" : "fc_dw_db_small", (dx ? 4.0 : 2.0) * batch * in * out, WORK_FLOP);
     TDH_LAUNCH(fc_bwd_fused_kernel, dim3(f.nx + f.nw + (bias ? ceil_div(out, 32) : 0)),
                        dim3(SFC_NT), 0, ctx().stream, f);
     TDH_LAUNCH_CHECK();

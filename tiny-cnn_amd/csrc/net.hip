@@ -133,11 +133,41 @@ bool layer_forks(const tdh_net::Layer &L) {
   return L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC;
 }
 
+// Where the gradient of a layer's input goes in a train step: the gradient buffer of the
+// layer in front, or, when that layer is an activation whose gradient the producing kernel
+// applies, the buffer in front of the activation.
+struct DxTarget {
+  float *dx;
+  ActGrad fold;
+};
+DxTarget dx_target(tdh_net *net, int i) {
+  DxTarget d;
+  d.dx = i == 0 ? net->dx_in : net->layers[i - 1].dout;
+  if (i >= 1 && net->layers[i - 1].grad_folded) {
+    d.fold.kind = net->layers[i - 1].spec.act;
+    d.fold.y    = net->layers[i - 1].out;
+    d.dx        = i - 1 == 0 ? net->dx_in : net->layers[i - 2].dout;
+  }
+  return d;
+}
+
+// the fully-connected layer in front of the closing softmax, when a train step with
+// cross_entropy_multiclass runs it, the softmax, the loss gradient and its dX as one launch
+bool tail_in_one_launch(const tdh_net *net, int batch) {
+  const int n = static_cast<int>(net->layers.size());
+  if (!(net->flags & TDH_NET_FUSE_ACT_GRAD) || n < 2) return false;
+  const tdh_layer &fc = net->layers[n - 2].spec, &sm = net->layers[n - 1].spec;
+  return sm.kind == TDH_L_ACT && sm.act == TDH_ACT_SOFTMAX && fc.kind == TDH_L_FC &&
+         fc_softmax_xent_applies(fc.fc_in, fc.fc_out, batch);
+}
+
 // packed: the layers' wp_fwd hold the current filters in the stride-1 kernels' layout
 // xent_t / xent_dz: the net ends in softmax and the step's loss is cross_entropy_multiclass: the
 // last layer's kernel also writes the loss gradient with respect to the softmax input
+// tail: the fully-connected layer in front of that softmax runs as fc_softmax_xent and also
+// writes the gradient of its input there
 int forward(tdh_net *net, int batch, const float *x, bool packed = false, const float *xent_t = nullptr,
-            float *xent_dz = nullptr) {
+            float *xent_dz = nullptr, const DxTarget *tail = nullptr) {
   const float *in = x;
   const int n     = static_cast<int>(net->layers.size());
   for (int i = 0; i < n; ++i) {
@@ -182,6 +212,11 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
+        if (tail && i == n - 2) {
+          TDH_TRY(fc_softmax_xent(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out, net->layers[n - 1].out,
+                                  xent_t, xent_dz, tail->dx, tail->fold));
+          ++i;
+        } else
         if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
             is_pointwise_act(net->layers[i + 1].spec.act)) {
           // the activation layer behind the product leaves the same kernel
@@ -485,11 +520,14 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   const bool packed = net->packs_valid;
   tdh_net::Layer &last = net->layers[n - 1];
   int first_bwd        = n - 1;
+  bool tail_done       = false;  // layer n-2 already has the gradient of its input
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
   // the full softmax Jacobian, and that kernel is the softmax layer's forward kernel
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
       last.spec.act == TDH_ACT_SOFTMAX && n >= 2) {
-    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout));
+    tail_done = tail_in_one_launch(net, batch);
+    const DxTarget tail = tail_done ? dx_target(net, n - 2) : DxTarget();
+    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done ? &tail : nullptr));
     first_bwd = n - 2;
   } else {
     TDH_TRY(forward(net, batch, x, packed));
@@ -501,8 +539,26 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     tdh_net::Layer &L  = net->layers[i];
     const tdh_layer &s = L.spec;
     const float *in    = i == 0 ? x : net->layers[i - 1].out;
-    float *dx          = i == 0 ? net->dx_in : net->layers[i - 1].dout;
-    ActGrad fold;
+    const DxTarget target = dx_target(net, i);
+    float *dx             = target.dx;
+    const ActGrad fold    = target.fold;
+    if (tail_done && i == n - 2) {
+      // only the weight and bias gradients are left, and nothing before the optimizer reads
+      // them: one launch, on the side stream when the step branches
+      TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
+      if (forked) {
+        TDH_HIP(hipEventRecord(net->events[i], c.stream));
+        TDH_HIP(hipStreamWaitEvent(c.side[0], net->events[i], 0));
+        side_used[0] = true;
+        StreamSwap on_side(c.side[0]);
+        TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw,
+                       L.b_size ? L.db : nullptr, 1, ActGrad()));
+      } else {
+        TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw,
+                       L.b_size ? L.db : nullptr, 1, ActGrad()));
+      }
+      continue;
+    }
     // a small fully-connected layer computes its three gradients in one launch on the main
     // chain: its weight and bias products are too small to be worth a branch
     const bool fc_one_launch = s.kind == TDH_L_FC && fc_bwd_fuses(s.fc_in, s.fc_out, batch);
@@ -518,12 +574,6 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         TDH_HIP(hipStreamWaitEvent(c.side[1], net->events[i], 0));
         side_used[1] = true;
       }
-    }
-    if (i >= 1 && net->layers[i - 1].grad_folded) {
-      // write straight into the activation's input gradient, scaled by act'(its output)
-      fold.kind = net->layers[i - 1].spec.act;
-      fold.y    = net->layers[i - 1].out;
-      dx        = i - 1 == 0 ? net->dx_in : net->layers[i - 2].dout;
     }
     switch (s.kind) {
       case TDH_L_CONV:
