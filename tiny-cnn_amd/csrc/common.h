@@ -32,6 +32,9 @@ struct Context {
   // a train step collects the split reductions of its weight gradients and the row sums of its
   // bias gradients and launches each kind once (flush_deferred_*)
   bool defer_reduce = false, defer_rowsum = false;
+  // leave_split_sum: the caller of a convolution asks it to leave a split reduction to the
+  // kernel that reads the result next; split_sum_left: one was left (left_split_sum())
+  bool leave_split_sum = false, split_sum_left = false;
   // two more streams (default priority) for work that branches off the main one inside a
   // captured train step; created on first use
   hipStream_t side[2]   = {nullptr, nullptr};
@@ -218,6 +221,25 @@ struct ActGrad {
   const float *y = nullptr; // activation OUTPUT, same indexing as the GEMM result
 };
 
+// A split reduction that the kernel reading the result finishes: value i is
+// part[i] + part[stride + i] + ... (in this order) (+ bias of i's channel plane) (* act'(y[i])),
+// and whoever computes it also writes it to out[i]. The 2x2 max-pool kernels behind a
+// stride-1 convolution take it (a reduction kernel of its own costs a launch on the chain
+// every later layer waits for).
+struct SplitSum {
+  const float *part = nullptr;
+  int splits = 0;
+  size_t stride = 0;  // elements of one partial = elements of the result
+  const float *bias = nullptr;
+  int MC = 1;
+  FastDiv div_plane;
+  ActGrad ag;
+  float *out = nullptr;
+};
+SplitSum &left_split_sum();  // meaningful while ctx().split_sum_left
+int finish_split_sum();      // the reduction as a launch of its own, when nobody took it
+
+
 // conv.hip / fc.hip
 // prepacked: filters already packed by conv_pack_filters for this direction (and only then)
 // A 2x2 / stride-2 max-pool layer (and the pointwise activation behind it) computed by the
@@ -312,6 +334,37 @@ __device__ __forceinline__ float act_grad_factor(int kind, float y) {
     case TDH_ACT_SIGMOID: return y * (1.0f - y);
     default: return 1.0f;
   }
+}
+
+// VEC consecutive values of one channel plane (i a multiple of VEC, VEC in {1, 2, 4})
+template <int VEC>
+__device__ __forceinline__ void split_sum_values(const SplitSum &s, const size_t i, float (&v)[VEC]) {
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) v[e] = 0.0f;
+  for (int z = 0; z < s.splits; ++z) {
+    const float *p = s.part + z * s.stride + i;
+    if (VEC == 4) {
+      const float4 f = *reinterpret_cast<const float4 *>(p);
+      v[0] += f.x; v[1 % VEC] += f.y; v[2 % VEC] += f.z; v[3 % VEC] += f.w;
+    } else if (VEC == 2) {
+      const float2 f = *reinterpret_cast<const float2 *>(p);
+      v[0] += f.x; v[1 % VEC] += f.y;
+    } else {
+      v[0] += p[0];
+    }
+  }
+  const float b = s.bias ? s.bias[s.div_plane.div(static_cast<uint32_t>(i)) % s.MC] : 0.0f;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    v[e] += b;
+    if (s.ag.kind != TDH_ACT_NONE) v[e] *= act_grad_factor(s.ag.kind, s.ag.y[i + e]);
+  }
+  if (VEC == 4)
+    *reinterpret_cast<float4 *>(s.out + i) = make_float4(v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]);
+  else if (VEC == 2)
+    *reinterpret_cast<float2 *>(s.out + i) = make_float2(v[0], v[1 % VEC]);
+  else
+    s.out[i] = v[0];
 }
 
 }  // namespace tdh

@@ -10,38 +10,29 @@ namespace {
 // thread when a channel plane is a multiple of four
 template <int VEC>
 __global__ void __launch_bounds__(256)
-s1_split_reduce_kernel(const float *__restrict__ part, const int splits, const size_t stride,
-                       float *__restrict__ out, const float *__restrict__ bias, const ActGrad ag,
-                       const int MC, const FastDiv div_plane, const size_t total,
-                       float *__restrict__ act_out, const int act_kind) {
+s1_split_reduce_kernel(const SplitSum sum, float *__restrict__ act_out, const int act_kind) {
   const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
-  if (i >= total) return;
+  if (i >= sum.stride) return;
   float v[VEC];
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) v[e] = 0.0f;
-  for (int z = 0; z < splits; ++z) {
-    if (VEC == 4) {
-      const float4 f = *reinterpret_cast<const float4 *>(part + z * stride + i);
-      v[0] += f.x; v[1] += f.y; v[2] += f.z; v[VEC - 1] += f.w;
-    } else {
-      v[0] += part[z * stride + i];
-    }
-  }
-  const int m = div_plane.div(static_cast<uint32_t>(i)) % MC;  // the plane of all VEC elements
-  const float b = bias ? bias[m] : 0.0f;
-#pragma unroll
-  for (int e = 0; e < VEC; ++e) {
-    v[e] += b;
-    if (ag.kind != TDH_ACT_NONE) v[e] *= act_grad_factor(ag.kind, ag.y[i + e]);
-  }
-  if (VEC == 4)
-    *reinterpret_cast<float4 *>(out + i) = make_float4(v[0], v[1], v[2], v[VEC - 1]);
-  else
-    out[i] = v[0];
+  split_sum_values<VEC>(sum, i, v);
   if (act_out) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) act_out[i + e] = act_apply(act_kind, v[e]);
   }
+}
+
+int launch_split_reduce(const SplitSum &sum, int plane, float *act_out, int act_kind) {
+  const size_t total = sum.stride;
+  ProfScope prof("conv_s1_split_reduce", 4.0 * total * (sum.splits + 1 + (sum.ag.kind != TDH_ACT_NONE)),
+                 WORK_BYTE);
+  if (plane % 4 == 0)
+    TDH_LAUNCH((s1_split_reduce_kernel<4>), dim3(static_cast<unsigned>(ceil_div_sz(total / 4, 256))), dim3(256), 0,
+               ctx().stream, sum, act_out, act_kind);
+  else
+    TDH_LAUNCH((s1_split_reduce_kernel<1>), dim3(static_cast<unsigned>(ceil_div_sz(total, 256))), dim3(256), 0,
+               ctx().stream, sum, act_out, act_kind);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
 }
 
 // wp[t][kc][m]: forward (flip = 0): kc = ci, m = co, t as is; dX (flip = 1): kc = co, m = ci,
@@ -213,21 +204,30 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
     else TDH_TRY(R == 3 ? s1_launch_3x3_scalar(p) : s1_launch_5x5_scalar(p));
   }
   if (p.splits > 1) {
-    const size_t total = p.args.part_stride;
-    const int plane    = OH * OW;
-    ProfScope prof("conv_s1_split_reduce", 4.0 * total * (p.splits + 1 + (ag.kind != TDH_ACT_NONE)),
-                   WORK_BYTE);
-    if (plane % 4 == 0)
-      TDH_LAUNCH((s1_split_reduce_kernel<4>), dim3(static_cast<unsigned>(ceil_div_sz(total / 4, 256))), dim3(256), 0,
-                         ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
-                         FastDiv(plane), total, act_out, act_kind);
-    else
-      TDH_LAUNCH((s1_split_reduce_kernel<1>), dim3(static_cast<unsigned>(ceil_div_sz(total, 256))), dim3(256), 0,
-                         ctx().stream, p.args.part, p.splits, total, out, bias, ag, MC,
-                         FastDiv(plane), total, act_out, act_kind);
-    TDH_LAUNCH_CHECK();
+    SplitSum sum;
+    sum.part = p.args.part; sum.splits = p.splits; sum.stride = p.args.part_stride;
+    sum.bias = bias; sum.MC = MC; sum.div_plane = FastDiv(OH * OW); sum.ag = ag; sum.out = out;
+    if (ctx().leave_split_sum && !act_out) {
+      // the kernel that reads `out` next adds the partials up (and writes `out`)
+      left_split_sum()     = sum;
+      ctx().split_sum_left = true;
+      return TDH_OK;
+    }
+    TDH_TRY(launch_split_reduce(sum, OH * OW, act_out, act_kind));
   }
   return TDH_OK;
+}
+
+SplitSum &left_split_sum() {
+  static SplitSum sum;
+  return sum;
+}
+
+int finish_split_sum() {
+  if (!ctx().split_sum_left) return TDH_OK;
+  ctx().split_sum_left = false;
+  const SplitSum &sum = left_split_sum();
+  return launch_split_reduce(sum, static_cast<int>(sum.div_plane.d), nullptr, TDH_ACT_NONE);
 }
 
 }  // namespace tdh

@@ -133,6 +133,14 @@ bool layer_forks(const tdh_net::Layer &L) {
   return L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC;
 }
 
+// Asks the convolution called inside the scope to leave a split reduction to the max-pool
+// kernel that reads its result next (maxpool_fwd / maxpool_bwd take it or finish it).
+struct LeaveSplitSum {
+  Context &c;
+  LeaveSplitSum(Context &cc, bool on) : c(cc) { c.leave_split_sum = on; }
+  ~LeaveSplitSum() { c.leave_split_sum = false; }
+};
+
 // Where the gradient of a layer's input goes in a train step: the gradient buffer of the
 // layer in front, or, when that layer is an activation whose gradient the producing kernel
 // applies, the buffer in front of the activation.
@@ -205,8 +213,13 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
             pf.act_kind = net->layers[last].spec.act;
           }
         }
-        TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp, act_out, act_kind,
-                           pf.out ? &pf : nullptr));
+        {
+          // nothing behind the convolution left its kernel and a max-pool reads the result
+          LeaveSplitSum leave(ctx(), fuse && last == i && i + 1 < n &&
+                                         net->layers[i + 1].spec.kind == TDH_L_MAXPOOL);
+          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp, act_out, act_kind,
+                             pf.out ? &pf : nullptr));
+        }
         i = last;
       }
         break;
@@ -248,7 +261,7 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
     }
     in = net->layers[i].out;  // of the activation layer when one was fused
   }
-  return TDH_OK;
+  return finish_split_sum();  // (a max-pool has taken or finished it; this is for the error paths)
 }
 
 }  // namespace
@@ -508,6 +521,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     explicit Deferred(Context &cc) : c(cc) {}
     ~Deferred() {
       c.defer_reduce = c.defer_rowsum = false;
+      c.leave_split_sum = c.split_sum_left = false;
       flush_deferred_reduces(false);
       flush_deferred_rowsums(false);
     }
@@ -580,13 +594,22 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         TDH_TRY(ws_begin((forked ? 3 : 1) * conv2d_workspace_bytes(&s.conv, batch)));
       {
         const float *wp = packed && L.wp_dx && conv_uses_packed(&s.conv, batch, 1) ? L.wp_dx : nullptr;
+        // the layer that reads this dX next (behind a folded activation) is a max-pool: its
+        // backward kernel can add up a split reduction of dX
+        const int reader = i - 1 - ((i >= 1 && net->layers[i - 1].grad_folded) ? 1 : 0);
+        const bool pool_reads = (net->flags & TDH_NET_FUSE_ACT_GRAD) && reader >= 0 &&
+                                net->layers[reader].spec.kind == TDH_L_MAXPOOL;
         if (forked) {
           if (!fork) {
+            LeaveSplitSum leave(c, pool_reads);
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1, fold,
                                L.tbl_dev, wp));
             break;
           }
-          TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+          {
+            LeaveSplitSum leave(c, pool_reads);
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+          }
           const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
           {
             StreamSwap on_side(c.side[0]);
@@ -602,6 +625,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             c.defer_rowsum = false;
           }
         } else {
+          LeaveSplitSum leave(c, pool_reads);
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
                              fold, L.tbl_dev, wp));
         }
@@ -642,6 +666,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         break;
     }
   }
+  TDH_TRY(finish_split_sum());  // (a max-pool has taken or finished it)
   if (side_used[0]) {
     StreamSwap on_side(c.side[0]);
     TDH_TRY(flush_deferred_reduces());

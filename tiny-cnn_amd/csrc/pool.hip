@@ -64,19 +64,31 @@ maxpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
 // height, 16-byte aligned tensors. A thread owns two neighbouring outputs, i.e. two input rows
 // of four floats, read as 16-byte words; the window scan order (row by row, left to right) and
 // the strict '>' are those of the general kernel.
+// SUM: the input is a split reduction left to this kernel (sum.out is x): the thread adds up
+// the eight values it reads, and writes them to x as the reduction kernel would have.
+template <bool SUM>
 __global__ void __launch_bounds__(PT)
 maxpool2x2_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
                       int32_t *__restrict__ argmax, const int pairs, const int W, const int OW2,
                       const FastDiv div_ow2, const int rows_per_sample, float *__restrict__ act_out,
-                      const int act_kind) {
+                      const int act_kind, const SplitSum sum) {
   const int t = blockIdx.x * PT + threadIdx.x;  // pair index: (plane*OH + oy)*OW2 + ox2
   if (t >= pairs) return;
   uint32_t row, ox2;
   div_ow2.divmod(t, row, ox2);                   // row = plane*OH + oy
   // input rows 2*row and 2*row+1 of the [planes*H][W] image, columns 4*ox2 .. 4*ox2+3
-  const float *p   = x + (static_cast<size_t>(2 * row) * W + 4 * ox2);
-  const float4 r0  = *reinterpret_cast<const float4 *>(p);
-  const float4 r1  = *reinterpret_cast<const float4 *>(p + W);
+  const size_t at = static_cast<size_t>(2 * row) * W + 4 * ox2;
+  float4 r0, r1;
+  if (SUM) {
+    float a[4], b[4];
+    split_sum_values<4>(sum, at, a);
+    split_sum_values<4>(sum, at + W, b);
+    r0 = make_float4(a[0], a[1], a[2], a[3]);
+    r1 = make_float4(b[0], b[1], b[2], b[3]);
+  } else {
+    r0 = *reinterpret_cast<const float4 *>(x + at);
+    r1 = *reinterpret_cast<const float4 *>(x + at + W);
+  }
   const float v[2][4] = {{r0.x, r0.y, r1.x, r1.y}, {r0.z, r0.w, r1.z, r1.w}};
   float best[2];
   int idx[2];
@@ -108,16 +120,26 @@ maxpool2x2_fwd_kernel(const float *__restrict__ x, float *__restrict__ y,
 }
 
 // dx rows 2*row, 2*row+1, columns 4*ox2..4*ox2+3 from two outputs and their argmax records
+// SUM: dy is a split reduction left to this kernel (sum.out is dy), as in the forward kernel
+template <bool SUM>
 __global__ void __launch_bounds__(PT)
 maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ argmax,
                       float *__restrict__ dx, const int pairs, const int W, const int OW2,
-                      const FastDiv div_ow2, const int rows_per_sample, const ActGrad ag) {
+                      const FastDiv div_ow2, const int rows_per_sample, const ActGrad ag,
+                      const SplitSum sum) {
   const int t = blockIdx.x * PT + threadIdx.x;
   if (t >= pairs) return;
   uint32_t row, ox2;
   div_ow2.divmod(t, row, ox2);
   const size_t o  = static_cast<size_t>(row) * (2 * OW2) + 2 * ox2;
-  const float2 g  = *reinterpret_cast<const float2 *>(dy + o);
+  float2 g;
+  if (SUM) {
+    float v[2];
+    split_sum_values<2>(sum, o, v);
+    g = make_float2(v[0], v[1]);
+  } else {
+    g = *reinterpret_cast<const float2 *>(dy + o);
+  }
   const int2 a    = *reinterpret_cast<const int2 *>(argmax + o);
   const int base  = (static_cast<int>(2 * row) % rows_per_sample) * W + 4 * static_cast<int>(ox2);
   float4 r0, r1;
@@ -287,14 +309,32 @@ int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int
                 float *act_out, int act_kind) {
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.OH * g.OW;
+  const bool fast  = is_2x2_tiling(g) && aligned16(x) && aligned8(y) && aligned8(argmax) && aligned8(act_out) &&
+                    total / 2 < (1L << 31);
+  // a split reduction left for the reader of x: taken by the 2x2 kernel, else finished first
+  const size_t in_total = static_cast<size_t>(batch) * g.C * g.H * g.W;
+  const bool take = ctx().split_sum_left && fast && total > 0 && left_split_sum().out == x &&
+                    left_split_sum().stride == in_total;
+  if (!take) TDH_TRY(finish_split_sum());
   if (total <= 0) return TDH_OK;
+  if (take) {
+    const SplitSum sum   = left_split_sum();
+    ctx().split_sum_left = false;
+    ProfScope prof(act_out ? "maxpool_fwd_act_sum" : "maxpool_fwd_sum",
+                   4.0 * in_total * (sum.splits + 1) + (act_out ? 12.0 : 8.0) * total, WORK_BYTE);
+    const int pairs = static_cast<int>(total / 2);
+    TDH_LAUNCH(maxpool2x2_fwd_kernel<true>, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, x, y, argmax,
+               pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, act_out, act_kind, sum);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   ProfScope prof(act_out ? "maxpool_fwd_act" : "maxpool_fwd",
                  4.0 * batch * g.C * g.H * g.W + (act_out ? 12.0 : 8.0) * total, WORK_BYTE);
-  if (is_2x2_tiling(g) && aligned16(x) && aligned8(y) && aligned8(argmax) && aligned8(act_out) &&
-      total / 2 < (1L << 31)) {
+  if (fast) {
     const int pairs = static_cast<int>(total / 2);
-    TDH_LAUNCH(maxpool2x2_fwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, x,
-                       y, argmax, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, act_out, act_kind);
+    TDH_LAUNCH(maxpool2x2_fwd_kernel<false>, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, x,
+                       y, argmax, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, act_out, act_kind,
+                       SplitSum());
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
@@ -308,14 +348,32 @@ int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_
                 float *dx, ActGrad ag) {
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.H * g.W;
+  const bool fast  = is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) &&
+                    total / 8 < (1L << 31) && (ag.kind == TDH_ACT_NONE || aligned16(ag.y));
+  // a split reduction left for the reader of dy: taken by the 2x2 kernel, else finished first
+  const size_t out_total = static_cast<size_t>(batch) * g.C * g.OH * g.OW;
+  const bool take = ctx().split_sum_left && fast && total > 0 && g.OH > 0 && g.OW > 0 &&
+                    left_split_sum().out == dy && left_split_sum().stride == out_total;
+  if (!take) TDH_TRY(finish_split_sum());
   TDH_CHECK_ARG(g.OH > 0 && g.OW > 0, "maxpool backward: empty output");
+  if (take) {
+    const SplitSum sum   = left_split_sum();
+    ctx().split_sum_left = false;
+    ProfScope prof(ag.kind != TDH_ACT_NONE ? "maxpool_bwd_act_sum" : "maxpool_bwd_sum",
+                   4.0 * out_total * (sum.splits + 2 + (sum.ag.kind != TDH_ACT_NONE)) +
+                     (ag.kind != TDH_ACT_NONE ? 8.0 : 4.0) * total, WORK_BYTE);
+    const int pairs = static_cast<int>(total / 8);
+    TDH_LAUNCH(maxpool2x2_bwd_kernel<true>, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy, argmax, dx,
+               pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag, sum);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   ProfScope prof(ag.kind != TDH_ACT_NONE ? "maxpool_bwd_act" : "maxpool_bwd",
                  8.0 * batch * g.C * g.OH * g.OW + (ag.kind != TDH_ACT_NONE ? 8.0 : 4.0) * total, WORK_BYTE);
-  if (is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) && total / 8 < (1L << 31) &&
-      (ag.kind == TDH_ACT_NONE || aligned16(ag.y))) {
+  if (fast) {
     const int pairs = static_cast<int>(total / 8);
-    TDH_LAUNCH(maxpool2x2_bwd_kernel, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
-                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag);
+    TDH_LAUNCH(maxpool2x2_bwd_kernel<false>, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
+                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag, SplitSum());
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
