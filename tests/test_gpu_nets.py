@@ -218,7 +218,32 @@ def test_first_conv_with_pool_in_its_kernel_matches_oracle(T, O, W, spec):
     """The first convolution of a fusing net also computes the 2x2 max-pool (and the activations)
     behind it: every layer output, the argmax records (bit-exact) and all gradients against the
     oracle, and the same net without fusion gives the same outputs."""
-    batch = 5
+    check_fusing_and_plain_net(T, O, W, spec, 5)
+
+
+@pytest.mark.parametrize("spec", [
+    # 2x2 pools behind and in front of the second convolution: they add up its split reductions
+    [("conv", 16, 16, 3, 5, 32, True), ("maxpool", 16, 16, 32, 2), ("act", "relu"),
+     ("conv", 8, 8, 32, 5, 64, True), ("maxpool", 8, 8, 64, 2), ("act", "relu"), ("fc", 1024, 10)],
+    # the same without activations: the pool in front reads dX directly
+    [("conv", 16, 16, 3, 5, 32, True), ("maxpool", 16, 16, 32, 2),
+     ("conv", 8, 8, 32, 5, 64, True), ("maxpool", 8, 8, 64, 2), ("fc", 1024, 10)],
+    # 4x4 pools: not the kernel that can take the sums, the reductions run on their own
+    [("conv", 32, 32, 3, 5, 32, True), ("maxpool", 32, 32, 32, 4), ("act", "tanh"),
+     ("conv", 8, 8, 32, 5, 64, True), ("maxpool", 8, 8, 64, 4), ("act", "relu"), ("fc", 256, 10)],
+    # an activation between convolution and pool: the reduction applies it, nothing is left
+    [("conv", 16, 16, 3, 5, 32, True), ("maxpool", 16, 16, 32, 2), ("act", "relu"),
+     ("conv", 8, 8, 32, 5, 64, True), ("act", "sigmoid"), ("maxpool", 8, 8, 64, 2), ("fc", 1024, 10)],
+])
+def test_split_convolution_sums_taken_by_the_pools_match_oracle(T, O, W, spec):
+    """A stride-1 convolution too small to fill the chip splits its reduction; in a fusing net the
+    2x2 max-pool kernel that reads the result (forward: behind it; backward: in front of it) adds
+    the partial sums up instead of a reduction launch. Same checks as above, at a batch where the
+    second convolution runs on the stride-1 kernel and splits four ways."""
+    check_fusing_and_plain_net(T, O, W, spec, 64)
+
+
+def check_fusing_and_plain_net(T, O, W, spec, batch):
     rng = np.random.default_rng(len(spec) * 131 + spec[0][1])
     nets = [T.Net(W.build_layers(T, spec), batch, f) for f in (0, T.NET_FUSE_ACT_GRAD)]
     ref = O.OracleNet(W.build_layers(O, spec), batch)
