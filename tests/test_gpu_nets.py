@@ -266,6 +266,10 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
             assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
             if l[0] == "maxpool":
                 assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64), ref.layer_argmax(i, batch))
+                if i >= 1 and spec[i - 1][0] == "conv":
+                    # the gradient routed through the pool (by the pool's kernel, or by the dX
+                    # epilogue of the fully-connected layer behind it)
+                    assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), REL_TOL, f"layer {i} dX")
             if net.param_size(i, 0):
                 assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
                 assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")

@@ -272,8 +272,21 @@ int conv_pack_filters(const tdh_conv_desc *d, int flip, const float *w, const ui
                       float *wp);
 int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *b, float *y, float *act_out = nullptr, int act_kind = 0);
+// The backward pass of a 2x2 / stride-2 max-pool layer in front of a fully-connected layer,
+// done by that layer's dX epilogue: the gradient of pooled element n of sample m goes to the
+// input position the argmax record names, zeros to the other three of its window.
+struct PoolScatter {
+  const int32_t *argmax = nullptr;  // [batch][C*OH*OW], flat CHW input index inside the sample
+  float *dx = nullptr;              // [batch][C*H*W]
+  int W = 0, OW = 0, OH = 0;        // input width, pooled width and height (H = 2*OH, W = 2*OW)
+};
+// (pool.hip) the layer is such a pool; fills the geometry
+bool maxpool_scatters_from_fc(const tdh_pool_desc *d, PoolScatter *geom);
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
-           const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act);
+           const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
+           const PoolScatter *pool = nullptr);
+// the one-launch backward kernel of this layer can also scatter dX through a max-pool
+bool fc_bwd_scatters_pool(int in, int out, int batch);
 // conv_s1.hip: stride-1 forward / dX with LDS halo tiles (3x3 and 5x5 windows)
 bool conv_s1_applicable(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
                         int ph, int pw);

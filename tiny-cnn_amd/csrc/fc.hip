@@ -120,13 +120,55 @@ small_fc_gemm_kernel(const StridedOperand a, const StridedOperand b, const Epi e
   small_fc_tile(a, b, epi, M, N, K, blockIdx.x, blockIdx.y, sm);
 }
 
+// dX of a fully-connected layer whose input is the output of a 2x2 / stride-2 max-pool (behind
+// an activation whose gradient `row.ag` folds in): the value is stored as EpiRowMajor stores
+// it, and also routed through the pool: to the input position its argmax record names, zeros
+// to the other three positions of the window (maxpool_grad_op_internal,
+// maxpool_op_internal.h:42-57, for windows that tile the input).
+struct EpiRowMajorPool {
+  EpiRowMajor row;
+  PoolScatter pool;  // argmax == nullptr: no pool, plain EpiRowMajor
+  FastDiv div_ow, div_oh;
+  int sample_in;     // C*H*W
+  struct Col {
+    EpiRowMajor::Col c;
+    int base;  // flat input index of the window's top-left corner
+  };
+  __device__ __forceinline__ Col col(int n) const {
+    Col r{row.col(n), 0};
+    if (pool.argmax) {
+      uint32_t rest, ox, plane, oy;
+      div_ow.divmod(static_cast<uint32_t>(n), rest, ox);
+      div_oh.divmod(rest, plane, oy);
+      r.base = static_cast<int>((plane * 2 * pool.OH + 2 * oy) * pool.W + 2 * ox);
+    }
+    return r;
+  }
+  __device__ __forceinline__ float prior(int m, const Col &c) const { return row.prior(m, c.c); }
+  __device__ __forceinline__ void store(int m, const Col &c, float v, float before) const {
+    const int idx = m * row.ld + c.c.n;
+    row.store(m, c.c, v, before);
+    if (!pool.argmax) return;
+    // the value as stored (the same steps as EpiRowMajor::store)
+    v += c.c.bias;
+    if (row.ag.kind != TDH_ACT_NONE) v *= act_grad_factor(row.ag.kind, row.ag.y[idx]);
+    v += before;
+    const int a = pool.argmax[idx];
+    float *p    = pool.dx + static_cast<size_t>(m) * sample_in + c.base;
+    *reinterpret_cast<float2 *>(p) = make_float2(a == c.base ? v : 0.0f, a == c.base + 1 ? v : 0.0f);
+    *reinterpret_cast<float2 *>(p + pool.W) =
+      make_float2(a == c.base + pool.W ? v : 0.0f, a == c.base + pool.W + 1 ? v : 0.0f);
+  }
+};
+
 // The whole backward pass of a small fully-connected layer in one launch: the first nx
 // workgroups take the tiles of dX, the next nw those of dW, the rest 32 columns each of the bias
 // gradient (rows g, g+8, ... per 32-lane group, group sums added in order, as the stand-alone
 // column sum does). The three products only share their inputs, and none of them fills the chip.
 struct FcBwdFused {
   StridedOperand xa, xb, wa, wb;
-  EpiRowMajor xepi, wepi;
+  EpiRowMajorPool xepi;
+  EpiRowMajor wepi;
   int xM, xN, xK, x_tiles_n, nx;
   int wM, wN, wK, w_tiles_n, nw;
   const float *dy;
@@ -286,6 +328,7 @@ int launch_small_fc(const StridedOperand &a, const StridedOperand &b, const Epi 
 bool fc_bwd_fuses(int in, int out, int batch) {
   return small_fc_applies(batch, in, out) && small_fc_applies(in, out, batch);
 }
+bool fc_bwd_scatters_pool(int in, int out, int batch) { return fc_bwd_fuses(in, out, batch); }
 
 // forward, softmax, cross-entropy gradient and dX of this layer can leave one launch
 bool fc_softmax_xent_applies(int in, int out, int batch) {
@@ -332,13 +375,22 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
 }
 
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
-           const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act) {
+           const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
+           const PoolScatter *pool) {
   const bool bias_grad = db && has_bias;
+  if (pool && !(dx && dw && fc_bwd_fuses(in, out, batch) && pool->OH * pool->OW > 0 && in % (pool->OH * pool->OW) == 0))
+    return set_error(TDH_ERR_INVALID, "fc_bwd: the pool scatter needs the one-launch kernel");
   if (dw && (dx || bias_grad) && fc_bwd_fuses(in, out, batch)) {
     FcBwdFused f;
     f.xa = StridedOperand{dy, out, 1, batch};
     f.xb = StridedOperand{w, out, 1, in};
-    f.xepi = EpiRowMajor{dx, in, nullptr, dx_act, 0};
+    f.xepi.row = EpiRowMajor{dx, in, nullptr, dx_act, 0};
+    if (pool) {
+      f.xepi.pool      = *pool;
+      f.xepi.div_ow    = FastDiv(pool->OW);
+      f.xepi.div_oh    = FastDiv(pool->OH);
+      f.xepi.sample_in = 4 * in;
+    }
     f.xM = batch; f.xN = in; f.xK = out;
     f.x_tiles_n = ceil_div(in, SFC_TN);
     f.nx = dx ? f.x_tiles_n * ceil_div(batch, SFC_TM) : 0;  // no dX: its workgroups are left out
@@ -350,7 +402,7 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     f.nw = f.w_tiles_n * ceil_div(in, SFC_TM);
     const bool bias = bias_grad;
     f.dy = dy; f.db = db; f.batch = batch; f.out = out; f.db_accumulate = accumulate;
-    ProfScope prof(dx ? "fc_bwd_small" : "fc_dw_db_small", (dx ? 4.0 : 2.0) * batch * in * out, WORK_FLOP);
+    ProfScope prof(pool ? "fc_bwd_small_pool" : dx ? "fc_bwd_small" : "fc_dw_db_small", (dx ? 4.0 : 2.0) * batch * in * out, WORK_FLOP);
     TDH_LAUNCH(fc_bwd_fused_kernel, dim3(f.nx + f.nw + (bias ? ceil_div(out, 32) : 0)),
                        dim3(SFC_NT), 0, ctx().stream, f);
     TDH_LAUNCH_CHECK();

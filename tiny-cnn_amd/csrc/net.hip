@@ -535,6 +535,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   tdh_net::Layer &last = net->layers[n - 1];
   int first_bwd        = n - 1;
   bool tail_done       = false;  // layer n-2 already has the gradient of its input
+  int pool_done        = -1;     // a max-pool layer whose backward pass the layer behind it did
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
   // the full softmax Jacobian, and that kernel is the softmax layer's forward kernel
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
@@ -651,11 +652,32 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           if (L.b_size)
             TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad()));
         } else {
+          // a 2x2 max-pool in front (behind a folded activation, nothing folded into the pool
+          // itself): the one-launch kernel's dX epilogue also routes the gradient through it
+          PoolScatter through;
+          int reader = -1;
+          if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && fc_one_launch &&
+              fc_bwd_scatters_pool(s.fc_in, s.fc_out, batch)) {
+            const int r = i - 1 - ((i >= 1 && net->layers[i - 1].grad_folded) ? 1 : 0);
+            if (r >= 0 && net->layers[r].spec.kind == TDH_L_MAXPOOL &&
+                maxpool_scatters_from_fc(&net->layers[r].spec.pool, &through)) {
+              const DxTarget behind = dx_target(net, r);
+              if (behind.fold.kind == TDH_ACT_NONE) {
+                through.argmax = net->layers[r].argmax;
+                through.dx     = behind.dx;
+                reader         = r;
+              }
+            }
+          }
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
-                         L.b_size ? L.db : nullptr, 1, fold));
+                         L.b_size ? L.db : nullptr, 1, fold, reader >= 0 ? &through : nullptr));
+          if (reader >= 0) pool_done = reader;
         }
         break;
-      case TDH_L_MAXPOOL: TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold)); break;
+      case TDH_L_MAXPOOL:
+        if (i == pool_done) break;  // the layer behind has written this layer's dX
+        TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold));
+        break;
       case TDH_L_AVEPOOL:
         TDH_TRY(ws_begin(avepool_workspace_bytes(&s.pool, batch)));
         TDH_TRY(avepool_bwd(&s.pool, batch, in, L.w, L.dout, dx, L.dw, L.db, 1, fold));

@@ -305,6 +305,13 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 }  // namespace
 
+bool maxpool_scatters_from_fc(const tdh_pool_desc *d, PoolScatter *geom) {
+  const PoolGeom g = make_geom(d);
+  if (!is_2x2_tiling(g)) return false;
+  geom->W = g.W; geom->OW = g.OW; geom->OH = g.OH;
+  return true;
+}
+
 int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax,
                 float *act_out, int act_kind) {
   const PoolGeom g = make_geom(d);
