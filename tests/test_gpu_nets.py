@@ -291,11 +291,16 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
     ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("fc", 64, 10), ("act", "softmax")], 9),
     # too wide for the one-launch kernel: the three separate launches
     ([("fc", 20, 200), ("act", "relu"), ("fc", 200, 10), ("act", "softmax")], 8),
+    # nets that end in the fully-connected layer, trained with mse: the same kernel without softmax
+    ([("fc", 50, 70), ("act", "tanh"), ("fc", 70, 3)], 16),
+    ([("fc", 30, 10)], 5),
+    ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("act", "sigmoid"), ("fc", 64, 64)], 19),
 ])
 @pytest.mark.parametrize("targets", ["one_hot", "soft"])
 def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch, targets):
-    """A fusing net trained with cross_entropy_multiclass runs its last fully-connected layer,
-    the softmax, the loss gradient and that layer's dX as one kernel: outputs and gradients
+    """A fusing net trained with cross_entropy_multiclass (or, ending in a fully-connected layer,
+    with mse) runs its last fully-connected layer, the softmax, the loss gradient and that
+    layer's dX as one kernel: outputs and gradients
     against the oracle, and bit for bit against the same net without fusion (same terms, same
     order), for one-hot and for soft targets."""
     rng = np.random.default_rng(len(spec) * 17 + batch)
@@ -309,7 +314,10 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
             for net in nets:
                 net.set_param(i, 0, w); net.set_param(i, 1, b)
             ref.weight(i)[:] = w; ref.bias(i)[:] = b
-    first, classes = spec[0], spec[-2][2]
+    softmax = spec[-1] == ("act", "softmax")
+    loss = "ce_multiclass" if softmax else "mse"
+    last_fc = len(spec) - (2 if softmax else 1)
+    first, classes = spec[0], spec[last_fc][2]
     n_in = first[1] if first[0] == "fc" else first[1] * first[2] * first[3]
     x = rng.standard_normal((batch, n_in)).astype(np.float32)
     one_hot = np.eye(classes, dtype=np.float32)[rng.integers(0, classes, batch)]
@@ -317,9 +325,9 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
     xd = T.to_device(x)
     for t in ((one_hot,) if targets == "one_hot" else (soft,)):
         td = T.to_device(t)
-        ref.train_step(O.opt_desc("sgd"), "ce_multiclass", x, t, do_update=False)
+        ref.train_step(O.opt_desc("sgd"), loss, x, t, do_update=False)
         for net in nets:
-            net.train_step(None, "ce_multiclass", batch, xd, td, do_update=False)
+            net.train_step(None, loss, batch, xd, td, do_update=False)
             for i, l in enumerate(spec):
                 assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
                 if net.param_size(i, 0):
@@ -330,7 +338,6 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
             assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
         # (a folded activation gradient rounds differently from the activation layer's own kernel,
         # so the layers in front agree to rounding only)
-        last_fc = len(spec) - 2
         for which in (0, 1):
             assert np.array_equal(nets[0].layer_grad(last_fc, which), nets[1].layer_grad(last_fc, which)), \
                 f"last layer's gradient {which} fused vs not"

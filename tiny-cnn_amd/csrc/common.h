@@ -311,7 +311,8 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch);
 size_t fc_workspace_bytes(int in, int out, int batch);
 bool fc_bwd_fuses(int in, int out, int batch);
 // The last fully-connected layer in front of softmax + cross_entropy_multiclass in one launch:
-// y = x*W + b, soft = softmax(y), dz = dL/dy, dx = dz*W^T (times dx_act's factor)
+// y = x*W + b, soft = softmax(y), dz = dL/dy, dx = dz*W^T (times dx_act's factor); with
+// soft == nullptr the loss is mse on y itself
 bool fc_softmax_xent_applies(int in, int out, int batch);
 int fc_softmax_xent(int in, int out, int has_bias, int batch, const float *x, const float *w,
                     const float *b, float *y, float *soft, const float *t, float *dz, float *dx,

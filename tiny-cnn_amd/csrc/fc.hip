@@ -203,7 +203,9 @@ __global__ void __launch_bounds__(SFC_NT) fc_bwd_fused_kernel(const FcBwdFused f
 }
 
 // The last fully-connected layer of a net that ends in softmax and is trained with
-// cross_entropy_multiclass, from its input to the gradient of its input in one launch: every
+// cross_entropy_multiclass (or ends in this layer and is trained with mse: then dz is
+// 2/outputs * (y - t) and there is no softmax), from its input to the gradient of its input in
+// one launch: every
 // step of that chain stays inside a sample row (only the weight and bias gradients add over
 // the batch; they are another launch, off the chain the next layer waits for). A workgroup
 // takes 16 rows. The product is small_fc_accumulate's, the softmax and the loss gradient are
@@ -213,9 +215,10 @@ __global__ void __launch_bounds__(SFC_NT) fc_bwd_fused_kernel(const FcBwdFused f
 struct FcTail {
   StridedOperand a, b;  // X[s][k], W[k][n]
   const float *bias;    // or null
-  float *out, *soft;    // the layer's output and the softmax layer's
+  float *out, *soft;    // the layer's output and the softmax layer's (null: the loss is mse)
   const float *t;
   float *dz;
+  float mse_factor;     // 2 / outputs (mse::df, loss_function.h:28-36)
   EpiRowMajor xepi;     // dX (with the activation gradient of the layer in front folded in)
   int M, N, K;          // batch, out, in
 };
@@ -259,6 +262,14 @@ __global__ void __launch_bounds__(SFC_NT) fc_softmax_xent_kernel(const FcTail f)
     const bool live = col && m < f.M;
     const int idx   = m * f.N + tn;
     const float v   = (acc[i] + bias) + 0.0f;
+    if (!f.soft) {  // mse on the layer's own output (the same for every lane)
+      dzv[i] = live ? f.mse_factor * (v - tv[i]) : 0.0f;
+      if (live) {
+        f.out[idx] = v;
+        f.dz[idx]  = dzv[i];
+      }
+      continue;
+    }
     const float mx  = sfc_wave_max(col ? fmaxf(-FLT_MAX, v) : -FLT_MAX);
     const float e   = col ? expf(v - mx) : 0.0f;
     const float se  = sfc_wave_sum(e);
@@ -335,6 +346,7 @@ bool fc_softmax_xent_applies(int in, int out, int batch) {
   return in <= SFC_KC && out <= SFC_TN && small_fc_applies(batch, out, in) && small_fc_applies(batch, in, out);
 }
 
+// soft == nullptr: the net ends in this layer and the loss is mse
 int fc_softmax_xent(int in, int out, int has_bias, int batch, const float *x, const float *w,
                     const float *b, float *y, float *soft, const float *t, float *dz, float *dx,
                     ActGrad dx_act) {
@@ -345,9 +357,10 @@ int fc_softmax_xent(int in, int out, int has_bias, int batch, const float *x, co
   f.b    = StridedOperand{w, 1, out, out};
   f.bias = has_bias ? b : nullptr;
   f.out = y; f.soft = soft; f.t = t; f.dz = dz;
+  f.mse_factor = 2.0f / static_cast<float>(out);
   f.xepi = EpiRowMajor{dx, in, nullptr, dx_act, 0};
   f.M = batch; f.N = out; f.K = in;
-  ProfScope prof("fc_fwd_softmax_xent_dx", 4.0 * batch * in * out, WORK_FLOP);
+  ProfScope prof(soft ? "fc_fwd_softmax_xent_dx" : "fc_fwd_mse_dx", 4.0 * batch * in * out, WORK_FLOP);
   TDH_LAUNCH(fc_softmax_xent_kernel, dim3(ceil_div(batch, SFC_TM)), dim3(SFC_NT), 0, ctx().stream, f);
   TDH_LAUNCH_CHECK();
   return TDH_OK;

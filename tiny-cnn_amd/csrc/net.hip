@@ -159,23 +159,30 @@ DxTarget dx_target(tdh_net *net, int i) {
   return d;
 }
 
-// the fully-connected layer in front of the closing softmax, when a train step with
-// cross_entropy_multiclass runs it, the softmax, the loss gradient and its dX as one launch
-bool tail_in_one_launch(const tdh_net *net, int batch) {
+// The layer that a train step runs together with the loss gradient and its own dX as one
+// launch, or -1: the fully-connected layer in front of the closing softmax under
+// cross_entropy_multiclass, or a closing fully-connected layer under mse.
+int tail_layer_in_one_launch(const tdh_net *net, int loss_kind, int batch) {
   const int n = static_cast<int>(net->layers.size());
-  if (!(net->flags & TDH_NET_FUSE_ACT_GRAD) || n < 2) return false;
-  const tdh_layer &fc = net->layers[n - 2].spec, &sm = net->layers[n - 1].spec;
-  return sm.kind == TDH_L_ACT && sm.act == TDH_ACT_SOFTMAX && fc.kind == TDH_L_FC &&
-         fc_softmax_xent_applies(fc.fc_in, fc.fc_out, batch);
+  if (!(net->flags & TDH_NET_FUSE_ACT_GRAD)) return -1;
+  int at = -1;
+  if (loss_kind == TDH_LOSS_CE_MULTICLASS && n >= 2 && net->layers[n - 1].spec.kind == TDH_L_ACT &&
+      net->layers[n - 1].spec.act == TDH_ACT_SOFTMAX)
+    at = n - 2;
+  else if (loss_kind == TDH_LOSS_MSE)
+    at = n - 1;
+  if (at < 0) return -1;
+  const tdh_layer &fc = net->layers[at].spec;
+  return fc.kind == TDH_L_FC && fc_softmax_xent_applies(fc.fc_in, fc.fc_out, batch) ? at : -1;
 }
 
 // packed: the layers' wp_fwd hold the current filters in the stride-1 kernels' layout
 // xent_t / xent_dz: the net ends in softmax and the step's loss is cross_entropy_multiclass: the
 // last layer's kernel also writes the loss gradient with respect to the softmax input
-// tail: the fully-connected layer in front of that softmax runs as fc_softmax_xent and also
-// writes the gradient of its input there
+// tail (with tail_layer): that fully-connected layer runs as fc_softmax_xent, which also writes
+// the loss gradient (to xent_dz, from the targets xent_t) and the gradient of its input
 int forward(tdh_net *net, int batch, const float *x, bool packed = false, const float *xent_t = nullptr,
-            float *xent_dz = nullptr, const DxTarget *tail = nullptr) {
+            float *xent_dz = nullptr, const DxTarget *tail = nullptr, int tail_layer = -1) {
   const float *in = x;
   const int n     = static_cast<int>(net->layers.size());
   for (int i = 0; i < n; ++i) {
@@ -225,10 +232,12 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
-        if (tail && i == n - 2) {
-          TDH_TRY(fc_softmax_xent(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out, net->layers[n - 1].out,
-                                  xent_t, xent_dz, tail->dx, tail->fold));
-          ++i;
+        if (tail && i == tail_layer) {
+          const bool softmax_behind = i == n - 2;
+          TDH_TRY(fc_softmax_xent(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out,
+                                  softmax_behind ? net->layers[n - 1].out : nullptr, xent_t, xent_dz, tail->dx,
+                                  tail->fold));
+          if (softmax_behind) ++i;
         } else
         if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
             is_pointwise_act(net->layers[i + 1].spec.act)) {
@@ -253,7 +262,7 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
         break;
       case TDH_L_AVEPOOL: TDH_TRY(avepool_fwd(&s.pool, batch, in, L.w, L.b, L.out)); break;
       case TDH_L_ACT:
-        if (xent_t && i == n - 1 && s.act == TDH_ACT_SOFTMAX)
+        if (xent_t && tail_layer != n - 1 && i == n - 1 && s.act == TDH_ACT_SOFTMAX)
           TDH_TRY(launch_softmax_fwd_xent(batch, static_cast<int>(L.out_size), in, xent_t, L.out, xent_dz));
         else
           TDH_TRY(launch_act_fwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out));
@@ -534,16 +543,21 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   const bool packed = net->packs_valid;
   tdh_net::Layer &last = net->layers[n - 1];
   int first_bwd        = n - 1;
-  bool tail_done       = false;  // layer n-2 already has the gradient of its input
+  int tail_done        = -1;     // this layer already has the gradient of its input
   int pool_done        = -1;     // a max-pool layer whose backward pass the layer behind it did
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
   // the full softmax Jacobian, and that kernel is the softmax layer's forward kernel
+  tail_done = tail_layer_in_one_launch(net, loss_kind, batch);
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
       last.spec.act == TDH_ACT_SOFTMAX && n >= 2) {
-    tail_done = tail_in_one_launch(net, batch);
-    const DxTarget tail = tail_done ? dx_target(net, n - 2) : DxTarget();
-    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done ? &tail : nullptr));
+    const DxTarget tail = tail_done >= 0 ? dx_target(net, n - 2) : DxTarget();
+    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done >= 0 ? &tail : nullptr,
+                    tail_done));
     first_bwd = n - 2;
+  } else if (tail_done >= 0) {
+    // mse on a closing fully-connected layer: its kernel writes the loss gradient too
+    const DxTarget tail = dx_target(net, n - 1);
+    TDH_TRY(forward(net, batch, x, packed, t, last.dout, &tail, tail_done));
   } else {
     TDH_TRY(forward(net, batch, x, packed));
     TDH_TRY(launch_loss_grad(loss_kind, batch, static_cast<int>(last.out_size), last.out, t,
@@ -557,7 +571,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     const DxTarget target = dx_target(net, i);
     float *dx             = target.dx;
     const ActGrad fold    = target.fold;
-    if (tail_done && i == n - 2) {
+    if (i == tail_done) {
       // only the weight and bias gradients are left, and nothing before the optimizer reads
       // them: one launch, on the side stream when the step branches
       TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
