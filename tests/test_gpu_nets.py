@@ -347,6 +347,37 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
         net.close()
 
 
+def test_layers_without_bias_through_the_one_launch_kernels(T, O):
+    """No layer has a bias: the last layer's one-launch kernel, the fully-connected backward that
+    routes dX through the pool in front, and the convolution kernels against the oracle."""
+    def layers(api):
+        return [api.L_conv(8, 8, 2, 3, 4, pad_same=True, has_bias=False), api.L_maxpool(8, 8, 4, 2),
+                api.L_act("relu"), api.L_fc(64, 24, has_bias=False), api.L_act("tanh"),
+                api.L_fc(24, 10, has_bias=False), api.L_act("softmax")]
+    batch = 9
+    rng = np.random.default_rng(77)
+    nets = [T.Net(layers(T), batch, f) for f in (0, T.NET_FUSE_ACT_GRAD)]
+    ref = O.OracleNet(layers(O), batch)
+    for i, (nw, fan_in) in {0: (72, 18), 3: (64 * 24, 64), 5: (240, 24)}.items():
+        w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+        for net in nets:
+            assert net.param_size(i, 1) == 0
+            net.set_param(i, 0, w)
+        ref.weight(i)[:] = w
+    x = rng.standard_normal((batch, 128)).astype(np.float32)
+    t = np.eye(10, dtype=np.float32)[rng.integers(0, 10, batch)]
+    ref.train_step(O.opt_desc("sgd"), "ce_multiclass", x, t, do_update=False)
+    for net in nets:
+        net.train_step(None, "ce_multiclass", batch, T.to_device(x), T.to_device(t), do_update=False)
+        for i in range(7):
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+        for i in (0, 3, 5):
+            assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
+        assert_close(net.layer_dx(1, batch), ref.layer_dx(1, batch), REL_TOL, "gradient routed through the pool")
+        assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, "input gradient")
+        net.close()
+
+
 def test_feeder_double_buffered_batches_match_oracle(T, O, W):
     """tdh_feeder_*: different host batches every step, a short last batch, graph replay from
     the two alternating device slots; updated weights against the oracle after every step."""
