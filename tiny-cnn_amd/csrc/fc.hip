@@ -93,17 +93,20 @@ __device__ __forceinline__ void small_fc_tile(const StridedOperand &a, const Str
                                               const int bx, const int by, SfcSmem &sm) {
   const int tn = threadIdx.x & 63, tmg = threadIdx.x >> 6;
   const int m0 = by * SFC_TM, n0 = bx * SFC_TN;
+  // what the epilogue reads from memory (the column's bias, the values a store adds to) is
+  // asked for together with the panels: behind the product each would be a trip to memory
+  // with nothing to hide it
+  const int n = n0 + tn;
+  typename Epi::Col c = epi.col(n < N ? n : 0);
+  float before[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + 4 * tmg + i;
+    before[i]   = (n < N && m < M) ? epi.prior(m, c) : 0.0f;
+  }
   float acc[4];
   small_fc_accumulate(a, b, M, N, K, bx, by, sm, acc);
-  const int n = n0 + tn;
   if (n < N) {
-    const typename Epi::Col c = epi.col(n);
-    float before[4];  // all loads before the first store: a load behind a store waits for it
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = m0 + 4 * tmg + i;
-      before[i]   = m < M ? epi.prior(m, c) : 0.0f;
-    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = m0 + 4 * tmg + i;
