@@ -1,13 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the tiny-dnn training hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--others]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others]
 
 Prints ONE JSON line. The default workload is the CIFAR-10-shape CNN train step at batch
 128 (fwd + bwd + update, Adam), the configuration the samples/s target is quoted on; inputs
 are synthetic and resident in HBM before the timed region. Other workloads:
 vgg_stack_b64, lenet5_b16 (train steps), conv2d_bwd_b64 and fc_bwd_adam_b256 (single-op
-backward passes). ``--others`` appends their results under "others".
+backward passes). Their results are appended under "others" in compact form (ms/step,
+samples/s, step TFLOP/s, the slowest kernels with their roofline fraction, a bounded CPU
+baseline), so that one run times all five configurations; ``--no-others`` leaves them out.
 
 "roofline" describes the kernel with the largest total time in the workload: its average
 launch duration is measured with HIP events on the library's stream in a second, separately
@@ -188,18 +190,20 @@ def copy_yardstick(T, mib=256, reps=5):
             "GB/s": round(2 * n / (us * 1e-6) / 1e9, 1)}
 
 
-def measured_traffic(tag):
+def measured_traffic(tag, workload=None):
     """HBM bytes per launch of kernel `tag` from hardware counters, when a counter run of this
     workload has been recorded in profiles/hbm_traffic.json (null otherwise)."""
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            rec = json.load(f)["kernels"].get(tag)
+            js = json.load(f)
+        rec = js.get("workloads", {}).get(workload, {}).get(tag) if workload else None
+        rec = rec or js["kernels"].get(tag)
         return rec and rec["hbm_bytes_per_launch"]
     except (OSError, ValueError, KeyError):
         return None
 
 
-def cpu_baseline(W, name, budget_s=20.0):
+def cpu_baseline(W, name, budget_s=20.0, max_steps=20):
     """Reference CPU figure on a bounded sample of the same workload."""
     from oracle import oracle as O
     try:
@@ -222,7 +226,7 @@ def cpu_baseline(W, name, budget_s=20.0):
                 net.set_param(i, which, a)
             net.fit(opt, loss, x, t, 1)  # warm-up step (allocates the per-sample buffers)
             steps, spent, per = 0, 0.0, []
-            while spent < budget_s and steps < 20:
+            while spent < budget_s and steps < max_steps:
                 sec = net.fit(opt, loss, x, t, 1)
                 per.append(sec); spent += sec; steps += 1
         else:
@@ -230,7 +234,7 @@ def cpu_baseline(W, name, budget_s=20.0):
             for (i, which, a) in params:
                 (net.weight(i) if which == 0 else net.bias(i))[:] = a
             steps, spent, per = 0, 0.0, []
-            while spent < budget_s and steps < 20:
+            while spent < budget_s and steps < max_steps:
                 t0 = time.perf_counter(); net.train_step(opt, loss, x, t)
                 sec = time.perf_counter() - t0
                 per.append(sec); spent += sec; steps += 1
@@ -269,7 +273,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cifar10_cnn_b128")
-    ap.add_argument("--others", action="store_true", help="also run the other workloads")
+    ap.add_argument("--others", action="store_true", help="(default) also run the other workloads")
+    ap.add_argument("--no-others", action="store_true", help="only the named workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -299,7 +304,7 @@ def main():
         "kernels": res["kernels"],
     }
     if out["roofline"]:
-        out["roofline"]["traffic"] = measured_traffic(out["roofline"]["kernel"])
+        out["roofline"]["traffic"] = measured_traffic(out["roofline"]["kernel"], args.workload)
     out["copy_yardstick"] = copy_yardstick(T)
     if hasattr(wl, "step_from_host"):  # never `value`: reported for callers that own host buffers
         for _ in range(8):  # both device slots get their captured step
@@ -323,7 +328,9 @@ def main():
                 out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1)
         except Exception as e:  # the baseline is reported, never required
             out["cpu_baseline"] = {"error": repr(e)}
-    if args.others:
+    if not args.no_others:
+        # the other four configurations, compact: short timed runs, the six slowest kernels, and
+        # a CPU baseline capped at a few seconds each so that the whole run stays within minutes
         others = {}
         for name in ("conv2d_bwd_b64", "fc_bwd_adam_b256", "vgg_stack_b64", "lenet5_b16",
                      "cifar10_cnn_b128"):
@@ -331,12 +338,31 @@ def main():
                 continue
             w2 = make_workload(T, W, name)
             r = run_workload(T, w2, max(5, args.steps // 2), max(2, args.warmup // 2), 5)
-            others[name] = {"samples_per_s": round(r["samples_per_s"], 2),
-                            "ms_per_step": round(r["ms_per_step"], 4), "config": w2.config,
-                            "step_tflops": round(w2.config["flop_per_step"] /
-                                                 (r["ms_per_step"] * 1e-3) / 1e12, 3),
-                            "kernels": r["kernels"][:6]}
+            ks = r["kernels"]
+            flop_k = [k for k in ks if k["bound"] == "mfma"]
+            rec = {"samples_per_s": round(r["samples_per_s"], 2),
+                   "ms_per_step": round(r["ms_per_step"], 4), "config": w2.config,
+                   "step_tflops": round(w2.config["flop_per_step"] / (r["ms_per_step"] * 1e-3) / 1e12, 3),
+                   "roofline": {k: ks[0][k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac",
+                                                      "avg_launch_us")} if ks else None,
+                   "kernels": [{k: e[k] for k in ("kernel", "achieved", "unit", "frac", "avg_launch_us",
+                                                  "launches", "ms_per_step")} for e in ks[:6]]}
+            if rec["roofline"]:
+                rec["roofline"]["traffic"] = measured_traffic(rec["roofline"]["kernel"], name)
+            if flop_k:   # all MFMA-bound kernels of the step together
+                tot_flop = sum(k["algorithmic_work_per_launch"] * k["launches"] for k in flop_k)
+                tot_s = sum(k["avg_launch_us"] * k["launches"] for k in flop_k) * 1e-6
+                rec["mfma_kernels_together"] = {"TFLOP/s": round(tot_flop / tot_s / 1e12, 2),
+                                                "frac": round(tot_flop / tot_s / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
             del w2
+            if not args.no_cpu_baseline:
+                try:
+                    rec["cpu_baseline"] = cpu_baseline(W, name, budget_s=4.0, max_steps=3)
+                    if rec["cpu_baseline"]:
+                        rec["gpu_over_cpu"] = round(rec["samples_per_s"] / rec["cpu_baseline"]["value"], 1)
+                except Exception as e:
+                    rec["cpu_baseline"] = {"error": repr(e)}
+            others[name] = rec
         out["others"] = others
     print(json.dumps(out))
 

@@ -131,11 +131,6 @@ int tdh_profile_end(int32_t *n_entries);
 int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launches,
                       double *total_ms, double *work_per_launch, int32_t *work_unit);
 
-/* Tuning aid: force tile configuration `tile_cfg` (0..9, see gemm_mfma.h) and `splits` K
- * slices for every GEMM launched afterwards; tile_cfg < 0 restores the built-in,
- * shape-only plan. Results stay correct for any setting. */
-int tdh_tune_gemm_plan(int32_t tile_cfg, int32_t splits);
-
 /* shape helpers: conv_out_length / pool_out_length (tiny_dnn/util/util.h:329-363) */
 int tdh_conv_out_w(const tdh_conv_desc *d);
 int tdh_conv_out_h(const tdh_conv_desc *d);

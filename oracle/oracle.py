@@ -371,8 +371,9 @@ def update_weight(o, weight_edge_samples, merged, w, s0=None, s1=None):
 def L_conv(in_w, in_h, in_c, k, out_c, pad_same=False, has_bias=True, stride=1, tbl=None):
     l = LayerDesc()
     l.kind = L_CONV
-    l.conv = conv_desc(in_w, in_h, in_c, k, k, out_c, pad_same, has_bias, stride, stride, tbl=tbl)
-    l._keep = getattr(l.conv, "_keep", None)
+    d = conv_desc(in_w, in_h, in_c, k, k, out_c, pad_same, has_bias, stride, stride, tbl=tbl)
+    l.conv = d                           # copies the struct: the table's array must outlive it
+    l._keep = getattr(d, "_keep", None)
     return l
 
 

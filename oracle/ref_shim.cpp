@@ -522,6 +522,11 @@ double tdr_net_fit(tdr_net *h, const opt_desc *o, int loss, int batch, const flo
       case 0: { gradient_descent p; p.alpha = o->alpha; p.lambda = o->lambda; TDR_FIT(p) } break;
       case 1: { momentum p; p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; TDR_FIT(p) } break;
       case 2: { adam p; p.alpha = o->alpha; p.b1 = o->b1; p.b2 = o->b2; p.b1_t = o->b1_t; p.b2_t = o->b2_t; TDR_FIT(p) } break;
+      /* eps is private in these three; the callers keep the constructor's value */
+      case 3: { adagrad p; p.alpha = o->alpha; TDR_FIT(p) } break;
+      case 4: { RMSprop p; p.alpha = o->alpha; p.mu = o->mu; TDR_FIT(p) } break;
+      case 5: { adamax p; p.alpha = o->alpha; p.b1 = o->b1; p.b2 = o->b2; p.b1_t = o->b1_t; TDR_FIT(p) } break;
+      case 6: { nesterov_momentum p; p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; TDR_FIT(p) } break;
       default: return -2.0;
     }
 #undef TDR_FIT

@@ -33,9 +33,25 @@ def rel_err(got, want):
     return float(np.max(np.abs(got - want) / scale))
 
 
+# The plain element-wise figure, reported beside the gate: |got - want| / max(|want|, floor)
+# with the absolute floor ELEMENTWISE_FLOOR * rms(want) (without a floor an element that is
+# exactly zero in the reference makes the figure infinite).
+ELEMENTWISE_FLOOR = 1e-3
+
+
+def elementwise_rel_err(got, want, floor=ELEMENTWISE_FLOOR):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    if got.size == 0:
+        return 0.0
+    scale = np.maximum(np.abs(want), floor * np.sqrt(np.mean(want * want)) + 1e-300)
+    return float(np.max(np.abs(got - want) / scale))
+
+
 def assert_close(got, want, tol=REL_TOL, what=""):
     e = rel_err(got, want)
-    assert e <= tol, f"{what}: relative error {e:.3e} > {tol:g}"
+    assert e <= tol, (f"{what}: relative error {e:.3e} > {tol:g} (plain element-wise, floor "
+                      f"{ELEMENTWISE_FLOOR:g}*rms: {elementwise_rel_err(got, want):.3e})")
 
 
 @pytest.fixture(scope="session")

@@ -141,10 +141,12 @@ def test_avepool_matches_reference_outputs(O, layer_grads, name):
     assert np.array_equal(db, g[f"{name}.db"])
 
 
-@pytest.mark.parametrize("name", ["lenet5_b16", "cifar10_cnn_b128"])
-def test_net_steps_match_reference_fit(O, W, net_steps, name):
+@pytest.mark.parametrize("key", ["lenet5_b16", "cifar10_cnn_b128", "cifar10_cnn_b128@128", "lenet5_mnist_b16"])
+def test_net_steps_match_reference_fit(O, W, net_steps, key):
     """Parameters after network<sequential>::fit steps of the compiled reference."""
     g = net_steps
+    name, key_full = key.split("@")[0], key
+    g = {k.replace(key_full + ".", name + ".", 1): g[k] for k in g.files if k.startswith(key_full + ".")}
     batch, steps, stride = int(g[f"{name}.batch"]), int(g[f"{name}.steps"]), int(g[f"{name}.stride"])
     spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch)
     assert input_checksum(x, t, params) == float(g[f"{name}.input_checksum"]), \

@@ -150,3 +150,25 @@ def test_dropout_bit_exact(ref, seed, rate):
     assert np.array_equal(mask, rmask)
     assert np.array_equal(O.dropout_fwd(mask, x, rate), ry)
     assert np.array_equal(O.dropout_bwd(mask, dy), rdx)
+
+
+@pytest.mark.parametrize("name,batch,steps", [("lenet5_mnist_b16", 16, 2), ("cifar10_cnn_b128", 128, 2)])
+def test_example_nets_fit_bit_exact(ref, W, name, batch, steps):
+    """The MNIST example's LeNet-5 (C3 with its connection table, adagrad) and the CIFAR-10 net
+    at the batch it is benchmarked at: the oracle's steps equal network<sequential>::fit bit
+    for bit."""
+    O = ref
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch)
+    net = O.OracleNet(W.build_layers(O, spec), batch)
+    rn = O.RefNet(W.build_layers(O, spec), "scalar", 0)
+    for (i, which, a) in params:
+        (net.weight(i) if which == 0 else net.bias(i))[:] = a
+        rn.set_param(i, which, a)
+    o, o2 = O.opt_desc(opt_kind, **opt_kw), O.opt_desc(opt_kind, **opt_kw)
+    for _ in range(steps):
+        net.train_step(o, loss, x, t)
+    rn.fit(o2, loss, x, t, steps)
+    for (i, which, a) in params:
+        got = net.weight(i) if which == 0 else net.bias(i)
+        assert not np.array_equal(got, a) or which == 1
+        assert np.array_equal(got, rn.get_param(i, which)[:a.size]), (i, which)

@@ -67,9 +67,21 @@ int ws_take(size_t bytes, void **out) {
   return TDH_OK;
 }
 
-// tdh_tune_gemm_plan forces one tile configuration and split count for every GEMM (tuning
-// sweeps only; in normal use the plan is a function of the shape alone).
+// Tuning sweeps only: the environment variable TDH_GEMM_PLAN="cfg,splits", read once by
+// tdh_init, forces one tile configuration (0..9, see gemm_mfma.h) and split count for every
+// GEMM of the process; unset, the plan is a function of the shape alone. Not part of the ABI.
 static int g_force_cfg = -1, g_force_splits = 1;
+
+static void read_gemm_plan_override() {
+  g_force_cfg    = -1;
+  g_force_splits = 1;
+  const char *e = std::getenv("TDH_GEMM_PLAN");
+  int cfg = -1, splits = 1;
+  if (e && std::sscanf(e, "%d,%d", &cfg, &splits) == 2 && cfg >= 0 && cfg < 10 && splits >= 1) {
+    g_force_cfg    = cfg;
+    g_force_splits = splits;
+  }
+}
 
 bool gemm_plan_override(int *cfg, int *splits) {
   *cfg    = g_force_cfg;
@@ -231,6 +243,7 @@ int tdh_init(int device) {
   TDH_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
   c.device = device;
   c.ready  = true;
+  read_gemm_plan_override();
   return TDH_OK;
 }
 
@@ -343,14 +356,6 @@ int tdh_event_elapsed_ms(void *start, void *stop, float *ms) {
   TDH_CHECK_ARG(start && stop && ms, "tdh_event_elapsed_ms: null argument");
   TDH_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
   TDH_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
-  return TDH_OK;
-}
-
-int tdh_tune_gemm_plan(int32_t tile_cfg, int32_t splits) {
-  TDH_CHECK_ARG(tile_cfg < 10 && splits >= 1, "tdh_tune_gemm_plan: cfg %d splits %d", tile_cfg,
-                splits);
-  g_force_cfg    = tile_cfg;
-  g_force_splits = splits;
   return TDH_OK;
 }
 

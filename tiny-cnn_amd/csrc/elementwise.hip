@@ -503,8 +503,11 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
     __syncthreads();
     if (threadIdx.x == 0) {
       unsigned int *ticket = reinterpret_cast<unsigned int *>(dev_powers + 2);
+      // acquire + release on the ticket: every workgroup's reads of the powers (made before
+      // its barrier above) happen before its own increment, and the last drawer's increment
+      // sees them all, so its writes below cannot overtake another workgroup's reads
       const unsigned int drawn =
-          __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
       if (drawn == gridDim.x - 1) {
         float q1 = b1_t, q2 = b2_t;
         for (int i = 0; i < n_tensors; ++i) {
@@ -513,7 +516,8 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
         }
         dev_powers[0] = q1;
         dev_powers[1] = q2;
-        __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the reset follows the new powers (release); the next launch starts after this one ends
+        __hip_atomic_store(ticket, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   }

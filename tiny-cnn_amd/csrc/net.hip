@@ -725,9 +725,11 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
 }
 
 static bool same_key(const tdh_net::GraphKey &a, const tdh_net::GraphKey &b) {
+  // field by field: a caller's tdh_opt may carry padding or unused fields it never wrote
+  const tdh_opt &p = a.hyper, &q = b.hyper;
   return a.batch == b.batch && a.loss == b.loss && a.do_update == b.do_update && a.x == b.x &&
-         a.t == b.t && a.scratch == b.scratch &&
-         std::memcmp(&a.hyper, &b.hyper, sizeof(tdh_opt)) == 0;
+         a.t == b.t && a.scratch == b.scratch && p.kind == q.kind && p.alpha == q.alpha &&
+         p.lambda == q.lambda && p.mu == q.mu && p.b1 == q.b1 && p.b2 == q.b2 && p.eps == q.eps;
 }
 
 int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,

@@ -24,6 +24,22 @@ def lenet5():
             ("conv", 5, 5, 16, 5, 120, False), ("act", "tanh"), ("fc", 120, 10)]
 
 
+# connection table of LeNet-5's C3 layer [LeCun 1998, table 1], [in_c = 6][out_c = 16]
+# (examples/mnist/train.cpp:17-24)
+LENET_C3_TABLE = [[c == "O" for c in row] for row in (
+    "OXXXOOOXXOOOOXOO", "OOXXXOOOXXOOOOXO", "OOOXXXOOOXXOXOOO",
+    "XOOOXXOOOOXXOXOO", "XXOOOXXOOOOXOOXO", "XXXOOOXXOOOOXOOO")]
+
+
+def lenet5_mnist():
+    """The LeNet-5 of examples/mnist/train.cpp:44-62: C3 with its connection table, a tanh
+    behind every layer (also behind the pools and the last fully-connected layer)."""
+    return [("conv", 32, 32, 1, 5, 6, False), ("act", "tanh"), ("avepool", 28, 28, 6, 2), ("act", "tanh"),
+            ("conv", 14, 14, 6, 5, 16, False, LENET_C3_TABLE), ("act", "tanh"),
+            ("avepool", 10, 10, 16, 2), ("act", "tanh"),
+            ("conv", 5, 5, 16, 5, 120, False), ("act", "tanh"), ("fc", 120, 10), ("act", "tanh")]
+
+
 def cifar10_cnn():
     """CIFAR-10-shape CNN of examples/cifar10/train.cpp:26-42 (configs[3])."""
     return [("conv", 32, 32, 3, 5, 32, True), ("maxpool", 32, 32, 32, 2), ("act", "relu"),
@@ -46,6 +62,8 @@ def vgg_stack(size=128):
 WORKLOADS = {
     # name: (spec builder, batch, loss, optimizer kind, optimizer kwargs, init, input dist, seed)
     "lenet5_b16": (lenet5, 16, "mse", "sgd", {"alpha": 0.01}, "xavier", "uniform", 1234),
+    # not one of the five benchmark configurations: the reference's own MNIST example net
+    "lenet5_mnist_b16": (lenet5_mnist, 16, "mse", "adagrad", {}, "xavier", "uniform", 1239),
     "cifar10_cnn_b128": (cifar10_cnn, 128, "ce_multiclass", "adam", {}, "xavier", "normal", 1237),
     "vgg_stack_b64": (vgg_stack, 64, "ce_multiclass", "momentum", {"alpha": 0.01, "mu": 0.9},
                       "he", "normal", 1238),
@@ -57,8 +75,8 @@ def build_layers(api, spec):
     for l in spec:
         kind = l[0]
         if kind == "conv":
-            _, w, h, c, k, oc, same = l
-            out.append(api.L_conv(w, h, c, k, oc, pad_same=same))
+            _, w, h, c, k, oc, same = l[:7]
+            out.append(api.L_conv(w, h, c, k, oc, pad_same=same, tbl=l[7] if len(l) > 7 else None))
         elif kind == "fc":
             out.append(api.L_fc(l[1], l[2]))
         elif kind == "maxpool":
@@ -76,7 +94,7 @@ def layer_fans(l):
     """(weight count, bias count, fan_in, fan_out) of a layer tuple."""
     kind = l[0]
     if kind == "conv":
-        _, w, h, c, k, oc, same = l
+        _, w, h, c, k, oc, same = l[:7]
         return k * k * c * oc, oc, k * k * c, k * k * oc
     if kind == "fc":
         return l[1] * l[2], l[2], l[1], l[2]
@@ -111,7 +129,7 @@ def spec_sizes(spec):
     cur = in_size
     for l in spec:
         if l[0] == "conv":
-            _, w, h, c, k, oc, same = l
+            _, w, h, c, k, oc, same = l[:7]
             ow, oh = (w, h) if same else (w - k + 1, h - k + 1)
             cur = ow * oh * oc
         elif l[0] == "fc":
@@ -174,7 +192,7 @@ def flops_per_sample(spec):
     total = 0
     for l in spec:
         if l[0] == "conv":
-            _, w, h, c, k, oc, same = l
+            _, w, h, c, k, oc, same = l[:7]
             ow, oh = (w, h) if same else (w - k + 1, h - k + 1)
             total += 2 * ow * oh * oc * c * k * k
         elif l[0] == "fc":
