@@ -149,6 +149,17 @@ int tdh_conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const floa
 int tdh_conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w,
                    const float *dy, float *dx, float *dw, float *db, int accumulate);
 
+/* tdh_conv2d_bwd for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same
+ * arguments, kernels and results as tdh_conv2d_bwd, but the kernels' scratch (split partial
+ * sums, repacked filters) lies in a static 64 MiB device array that the library holds on every
+ * device it is initialised on, and the call allocates and frees nothing. A shape whose scratch
+ * need exceeds the array is refused with TDH_ERR_INVALID (the message states both sizes); use
+ * tdh_conv2d_bwd for it. All calls on one GPU share that GPU's array: calls are ordered by the
+ * library stream, two processes' or threads' calls that overlap on one GPU would race. */
+int tdh_conv2d_bwd_static(const tdh_conv_desc *d, int batch, const float *x, const float *w,
+                          const float *dy, float *dx, float *dw, float *db, int accumulate);
+
 /* --------------------------------------------------------- fully connected */
 /* FullyConnectedOp::compute (tiny_dnn/core/kernels/fully_connected_op.h:25-63,
  * fully_connected_op_internal.h:15-36) */

@@ -321,6 +321,12 @@ def conv2d_bwd(d, batch, x, w, dy, dx, dw, db, accumulate=False):
                                int(accumulate)), "tdh_conv2d_bwd")
 
 
+def conv2d_bwd_static(d, batch, x, w, dy, dx, dw, db, accumulate=False):
+    """tdh_conv2d_bwd with its scratch in the library's static device array (allocates nothing)."""
+    check(lib().tdh_conv2d_bwd_static(C.byref(d), batch, _p(x), _p(w), _p(dy), _p(dx), _p(dw), _p(db),
+                                      int(accumulate)), "tdh_conv2d_bwd_static")
+
+
 def fc_fwd(n_in, n_out, has_bias, batch, x, w, b, y):
     check(lib().tdh_fc_fwd(n_in, n_out, int(has_bias), batch, _p(x), _p(w), _p(b), _p(y)),
           "tdh_fc_fwd")

@@ -67,6 +67,53 @@ int ws_take(size_t bytes, void **out) {
   return TDH_OK;
 }
 
+// ----------------------------------------------------- scratch that is never allocated
+// tdh_conv2d_bwd_static runs the kernels of tdh_conv2d_bwd with their scratch (split partial
+// sums, repacked filters, staged bias sums) in this file-scope device array instead of the
+// grow-only buffer that ws_begin allocates, for callers that cannot allocate. Every device the
+// library is initialised on holds its own copy of the array, at its own address, until the
+// process ends. In host code the array's NAME is only a handle for hipGetSymbolAddress: the
+// device address is looked up once per device in tdh_init and only that pointer is ever passed
+// to kernels.
+constexpr size_t kStaticScratchBytes = 64u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static char *g_static_scratch[kMaxDevices] = {};
+
+static int lookup_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices)
+    return set_error(TDH_ERR_INVALID, "tdh_init: device %d beyond the %d this library keeps state for",
+                     device, kMaxDevices);
+  if (g_static_scratch[device]) return TDH_OK;
+  void *p = nullptr;
+  TDH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));  // the current device's copy
+  if (!p) return set_error(TDH_ERR_HIP, "tdh_init: the static scratch array has no device address");
+  g_static_scratch[device] = static_cast<char *>(p);
+  return TDH_OK;
+}
+
+// Points the context's scratch at the static array for one call; nothing can allocate meanwhile.
+struct StaticScratchScope {
+  Context &c;
+  char *saved_ws;
+  size_t saved_size, saved_off;
+  bool saved_locked;
+  StaticScratchScope(Context &cc, char *ptr)
+      : c(cc), saved_ws(cc.workspace), saved_size(cc.workspace_size), saved_off(cc.workspace_off),
+        saved_locked(cc.ws_locked) {
+    c.workspace      = ptr;
+    c.workspace_size = kStaticScratchBytes;
+    c.workspace_off  = 0;
+    c.ws_locked      = true;
+  }
+  ~StaticScratchScope() {
+    c.workspace      = saved_ws;
+    c.workspace_size = saved_size;
+    c.workspace_off  = saved_off;
+    c.ws_locked      = saved_locked;
+  }
+};
+
 // Tuning sweeps only: the environment variable TDH_GEMM_PLAN="cfg,splits", read once by
 // tdh_init, forces one tile configuration (0..9, see gemm_mfma.h) and split count for every
 // GEMM of the process; unset, the plan is a function of the shape alone. Not part of the ABI.
@@ -235,6 +282,7 @@ int tdh_init(int device) {
   TDH_HIP(hipGetDeviceCount(&count));
   TDH_CHECK_ARG(device >= 0 && device < count, "tdh_init: device %d of %d", device, count);
   TDH_HIP(hipSetDevice(device));
+  TDH_TRY(lookup_static_scratch(device));
   hipDeviceProp_t prop;
   TDH_HIP(hipGetDeviceProperties(&prop, device));
   std::snprintf(c.name, sizeof(c.name), "%s (%s)", prop.name, prop.gcnArchName);
@@ -453,6 +501,30 @@ int tdh_conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const floa
   if (batch == 0) return TDH_OK;
   TDH_CHECK_ARG(x && w && dy, "tdh_conv2d_bwd: null tensor");
   TDH_TRY(ws_begin(conv2d_workspace_bytes(d, batch)));
+  return conv2d_bwd(d, batch, x, w, dy, dx, dw, d->has_bias ? db : nullptr, accumulate, ActGrad());
+}
+
+int tdh_conv2d_bwd_static(const tdh_conv_desc *d, int batch, const float *x, const float *w,
+                          const float *dy, float *dx, float *dw, float *db, int accumulate) {
+  TDH_REQUIRE_INIT();
+  TDH_TRY(check_conv_desc(d, batch, true));
+  if (batch == 0) return TDH_OK;
+  TDH_CHECK_ARG(x && w && dy, "tdh_conv2d_bwd_static: null tensor");
+  Context &c = ctx();
+  TDH_CHECK_ARG(!c.ws_keep && !c.ws_locked, "tdh_conv2d_bwd_static: called inside a network step");
+  const size_t need = conv2d_workspace_bytes(d, batch);
+  if (need > kStaticScratchBytes)
+    return set_error(TDH_ERR_INVALID,
+                     "tdh_conv2d_bwd_static: this shape needs %zu bytes of scratch, the static buffer "
+                     "holds %zu; use tdh_conv2d_bwd",
+                     need, kStaticScratchBytes);
+  char *ptr = c.device >= 0 && c.device < kMaxDevices ? g_static_scratch[c.device] : nullptr;
+  if (!ptr) return set_error(TDH_ERR_NOT_INIT, "tdh_conv2d_bwd_static: no static scratch on device %d", c.device);
+  // Nothing in the array has to start at zero: every partial-sum slice, packed filter and
+  // staged sum that a reduction reads is written in full by the launch in front of it, so the
+  // previous call's contents are simply overwritten.
+  StaticScratchScope scope(c, ptr);
+  TDH_TRY(ws_begin(need));  // within the array by the test above; a locked scratch never allocates
   return conv2d_bwd(d, batch, x, w, dy, dx, dw, d->has_bias ? db : nullptr, accumulate, ActGrad());
 }
 
