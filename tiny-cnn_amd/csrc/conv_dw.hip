@@ -381,7 +381,10 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
   if (C < 16 || Kc < 16 || OW < 8 || OH < 2 || pw > 4) return p;
   p.tc = OW >= 48 ? 64 : OW >= 24 ? 32 : OW >= 12 ? 16 : 8;
   p.wfy = 1;
-  p.wco = (Kc > 32 && !five) ? 2 : 1;
+  // more than 32 output channels: two channel blocks share a workgroup's staged X patch (half
+  // the row groups each), which also keeps the 5x5 kernel's LDS footprint small enough for a
+  // convolution workgroup of the main chain to share the compute unit
+  p.wco = Kc > 32 ? 2 : 1;
   p.wk  = 4 / p.wco;
   p.nt = 64 * p.wco * p.wk * p.wfy;
   p.rows_block = five ? 1 : R;
@@ -446,7 +449,8 @@ int launch_dw_inst(const DwHaloPlan &p) {
 
 template <int TC, bool VEC>
 int launch_dw_tc(const DwHaloPlan &p) {
-  if (p.rows_block == 1) return launch_dw_inst<1, 5, TC, 1, 4, 1, 5, VEC>(p);
+  if (p.rows_block == 1)
+    return p.wco == 2 ? launch_dw_inst<1, 5, TC, 2, 2, 1, 5, VEC>(p) : launch_dw_inst<1, 5, TC, 1, 4, 1, 5, VEC>(p);
   if (p.wco == 2) return launch_dw_inst<3, 3, TC, 2, 2, 1, 3, VEC>(p);
   // 8 columns x 4 row groups would stage 17 words a thread; the plan leaves that tile out
   if (TC == 8) return set_error(TDH_ERR_INVALID, "conv_dw_halo_run: tile not built");
