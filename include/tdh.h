@@ -271,6 +271,13 @@ int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst);
 /* optimizer::reset() as network::fit calls it before training (tiny_dnn/network.h:856,
  * tiny_dnn/optimizers/optimizer.h:36-38): clears the per-weight state vectors */
 int tdh_net_reset_optimizer(tdh_net *net);
+/* nodes::update_weights (tiny_dnn/nodes.h:103-107): layer::update_weight of every layer, front
+ * to back, weight before bias, on the gradients accumulated since the last update, which are
+ * then cleared (tiny_dnn/layers/layer.h:663-682). What tdh_net_train_step does with
+ * do_update != 0, as a call of its own (network::update_weights, tiny_dnn/network.h:209-213). */
+int tdh_net_update_weights(tdh_net *net, tdh_opt *opt);
+/* nodes::clear_grads (tiny_dnn/nodes.h:118-122): zeroes every weight and bias gradient */
+int tdh_net_clear_grads(tdh_net *net);
 /* device views valid until the net is destroyed */
 float *tdh_net_param(tdh_net *net, int layer, int which);
 const float *tdh_net_layer_out(const tdh_net *net, int layer);

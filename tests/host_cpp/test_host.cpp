@@ -479,6 +479,271 @@ static void net_fit_vs_oracle(const char *name, int opt_kind) {
   tdo_net_destroy(ref);
 }
 
+// ---------------------------------------------------------------- device mirror
+// A conv -> relu -> max-pool -> fc stack driven layer by layer through forward_propagation /
+// back_propagation / optimizer::update on tensors that play the role of the reference's edges
+// (tiny_dnn/node.h:130-135), in resident mode: after the first step nothing but the net's
+// output (read by the host for the loss, as loss_function.h:191-218 does) and its gradient
+// (written by the host) crosses the bus, and the weights after three steps are the oracle's.
+static void resident_stack_through_the_mirror() {
+  std::puts("device mirror: conv -> relu -> max-pool -> fc, three SGD steps, layer by layer");
+  const size_t n = 6;
+  convolutional_layer conv(8, 8, 3, 2, 4, padding::same);
+  relu_layer relu;
+  max_pooling_layer pool(8, 8, 4, 2);
+  fully_connected_layer fc(64, 10);
+  tensor_t x = random_tensor(n, 128, 900);
+  tensor_t w1{random_vec(72, 901, -0.4f, 0.4f)}, b1{random_vec(4, 902, -0.1f, 0.1f)};
+  tensor_t w2{random_vec(640, 903, -0.3f, 0.3f)}, b2{random_vec(10, 904, -0.1f, 0.1f)};
+  tensor_t y1(n), a1(n), p1(n), out(n);
+  tensor_t dout(n, vec_t(10)), dp1(n), da1(n), dy1(n), dx(n);
+  tensor_t dw1(n, vec_t(72, 0.f)), db1(n, vec_t(4, 0.f)), dw2(n, vec_t(640, 0.f)), db2(n, vec_t(10, 0.f));
+  tensor_t target = random_tensor(n, 10, 905);
+  const vec_t w1_0 = w1[0], b1_0 = b1[0], w2_0 = w2[0], b2_0 = b2[0];
+
+  set_device_resident(true);
+  gradient_descent opt;
+  opt.alpha = 0.05f;
+  size_t bytes_after_first = 0, calls_after_first = 0;
+  for (int step = 0; step < 3; ++step) {
+    if (step == 1) reset_transfer_stats();
+    std::vector<tensor_t *> in1{&x, &w1, &b1}, o1{&y1}, in2{&y1}, o2{&a1}, in3{&a1}, o3{&p1}, in4{&p1, &w2, &b2}, o4{&out};
+    conv.forward_propagation(in1, o1);
+    relu.forward_propagation(in2, o2);
+    pool.forward_propagation(in3, o3);
+    fc.forward_propagation(in4, o4);
+    to_host(out);  // the host computes the loss gradient: mse::df = 2/n (y - t)
+    for (size_t s = 0; s < n; ++s)
+      for (size_t i = 0; i < 10; ++i) dout[s][i] = 2.f / 10.f * (out[s][i] - target[s][i]);
+    host_modified(dout);
+    std::vector<tensor_t *> g4{&dout}, ig4{&dp1, &dw2, &db2}, g3{&dp1}, ig3{&da1}, g2{&da1}, ig2{&dy1}, g1{&dy1},
+      ig1{&dx, &dw1, &db1};
+    fc.back_propagation(in4, o4, g4, ig4);
+    pool.back_propagation(in3, o3, g3, ig3);
+    relu.back_propagation(in2, o2, g2, ig2);
+    conv.back_propagation(in1, o1, g1, ig1);
+    // layer::update_weight (layer.h:663-682): the merged gradient is slot 0, then clear_grads
+    opt.update(dw1[0], w1[0], true); opt.update(db1[0], b1[0], true);
+    opt.update(dw2[0], w2[0], true); opt.update(db2[0], b2[0], true);
+    clear_grads(dw1); clear_grads(db1); clear_grads(dw2); clear_grads(db2);
+  }
+  const detail::transfer_counters c = transfer_stats();
+  bytes_after_first = c.h2d_bytes + c.d2h_bytes;
+  calls_after_first = c.h2d_calls + c.d2h_calls;
+  std::printf("  steps 2 and 3: %zu transfers, %zu bytes (net output down, its gradient up)\n",
+              calls_after_first, bytes_after_first);
+  EXPECT(c.d2h_calls == 2 && c.d2h_bytes == 2 * n * 10 * sizeof(float));
+  EXPECT(c.h2d_calls == 2 && c.h2d_bytes == 2 * n * 10 * sizeof(float));
+  to_host(w1); to_host(b1); to_host(w2); to_host(b2); to_host(dx); to_host(y1);
+  set_device_resident(false);
+
+  tdo_layer L[4] = {};
+  L[0].kind = TDO_L_CONV; L[0].conv = tdo_conv_desc{8, 8, 2, 3, 3, 4, 1, 1, 1, 1, 1, 1, nullptr};
+  L[1].kind = TDO_L_ACT;  L[1].act = TDO_ACT_RELU;
+  L[2].kind = TDO_L_MAXPOOL; L[2].pool = tdo_pool_desc{8, 8, 4, 2, 2, 2, 2, 0, 0};
+  L[3].kind = TDO_L_FC; L[3].fc_in = 64; L[3].fc_out = 10; L[3].fc_bias = 1;
+  tdo_net *ref = tdo_net_create(L, 4, static_cast<int>(n));
+  EXPECT(ref != nullptr);
+  std::copy(w1_0.begin(), w1_0.end(), tdo_net_weight(ref, 0)); std::copy(b1_0.begin(), b1_0.end(), tdo_net_bias(ref, 0));
+  std::copy(w2_0.begin(), w2_0.end(), tdo_net_weight(ref, 3)); std::copy(b2_0.begin(), b2_0.end(), tdo_net_bias(ref, 3));
+  tdo_opt o;
+  tdo_opt_default(&o, TDO_OPT_SGD);
+  o.alpha = 0.05f;
+  for (int step = 0; step < 3; ++step)
+    EXPECT(tdo_net_train_step(ref, &o, TDO_LOSS_MSE, static_cast<int>(n), flat(x).data(), flat(target).data(), 1) == 0);
+  expect_near(w1[0].data(), tdo_net_weight(ref, 0), 72, 1e-4f, "conv weights after three resident steps");
+  expect_near(b1[0].data(), tdo_net_bias(ref, 0), 4, 1e-4f, "conv bias");
+  expect_near(w2[0].data(), tdo_net_weight(ref, 3), 640, 1e-4f, "fc weights");
+  expect_near(b2[0].data(), tdo_net_bias(ref, 3), 10, 1e-4f, "fc bias");
+  expect_near(flat(dx).data(), tdo_net_layer_dx(ref, 0), n * 128, 1e-4f, "input gradient of the last step");
+  expect_near(flat(y1).data(), tdo_net_layer_out(ref, 0), n * 256, 1e-4f, "conv output of the last step");
+  // the argmax records were never downloaded; on request they are the oracle's
+  const std::vector<std::vector<size_t>> &am = pool.out2inmax();
+  bool same = am.size() == n;
+  for (size_t s = 0; same && s < n; ++s)
+    for (size_t i = 0; i < 64; ++i) same = same && am[s][i] == static_cast<size_t>(tdo_net_layer_argmax(ref, 2)[s * 64 + i]);
+  EXPECT(same);
+  tdo_net_destroy(ref);
+
+  // write-through (the default): the same calls leave every result in the host vectors at once
+  tensor_t yy(n), xx = random_tensor(n, 128, 906);
+  std::vector<tensor_t *> in1{&xx, &w1, &b1}, o1{&yy};
+  conv.forward_propagation(in1, o1);
+  xx[0][5] += 1.0f;  // no notice needed: inputs are sent again
+  tensor_t yy2(n);
+  std::vector<tensor_t *> o1b{&yy2};
+  conv.forward_propagation(in1, o1b);
+  EXPECT(yy[0] != yy2[0] && yy[1] == yy2[1]);
+  core::OpKernelContext ctx;                 // setLayer / Layer and the const accessors
+  ctx.set_in_out(in1, o1);
+  ctx.setLayer(&conv);
+  const core::OpKernelContext &cctx = ctx;
+  EXPECT(cctx.Layer() == &conv && &cctx.input(0) == &xx && &cctx.output(0) == &yy);
+}
+
+// ---------------------------------------------------------------- weight_init and network API
+static void stats_of(const vec_t &v, double &mean, double &var, float &lo, float &hi) {
+  mean = 0; lo = hi = v.empty() ? 0.f : v[0];
+  for (float x : v) { mean += x; lo = std::min(lo, x); hi = std::max(hi, x); }
+  mean /= v.size();
+  var = 0;
+  for (float x : v) var += (x - mean) * (x - mean);
+  var /= v.size();
+}
+
+static void weight_init_and_network_api() {
+  std::puts("weight_init (tiny_dnn/util/weight_init.h) and network fprop / bprop / update_weights / train_once");
+  auto make = [](network<sequential> &nn) {
+    nn << convolutional_layer(12, 12, 3, 2, 16, padding::same) << relu_layer() << max_pooling_layer(12, 12, 16, 2)
+       << fully_connected_layer(576, 32) << tanh_layer() << fully_connected_layer(32, 10) << softmax_layer();
+  };
+  {
+    network<sequential> nn;
+    make(nn);
+    set_random_seed(1);
+    nn.init_weight();
+    double mean, var; float lo, hi;
+    // conv: xavier, fan_in 3*3*2 = 18, fan_out 3*3*16 = 144 (convolutional_layer.h:269-277)
+    const float bc = std::sqrt(6.f / (18 + 144));
+    stats_of(nn.weights(0, 0), mean, var, lo, hi);
+    EXPECT(lo >= -bc && hi <= bc && hi > 0.9f * bc && lo < -0.9f * bc);
+    EXPECT(std::fabs(mean) < 0.1 * bc && std::fabs(var / (bc * bc / 3) - 1) < 0.25);
+    // fc 576 -> 32: bound sqrt(6 / 608); 18432 draws
+    const float bf = std::sqrt(6.f / (576 + 32));
+    stats_of(nn.weights(3, 0), mean, var, lo, hi);
+    EXPECT(lo >= -bf && hi <= bf && hi > 0.99f * bf && lo < -0.99f * bf);
+    EXPECT(std::fabs(mean) < 0.03 * bf && std::fabs(var / (bf * bf / 3) - 1) < 0.05);
+    for (int i : {0, 3, 5})
+      for (float b : nn.weights(i, 1)) EXPECT(b == 0.f);   // bias_init: constant(0)
+    // the draws are the reference's: one uniform_real_distribution<float> per value from
+    // std::mt19937(1), layers front to back
+    std::mt19937 gen(1);
+    vec_t first = nn.weights(0, 0);
+    bool same = true;
+    for (size_t i = 0; i < first.size(); ++i) {
+      std::uniform_real_distribution<float> dst(-bc, bc);
+      same = same && first[i] == dst(gen);
+    }
+    EXPECT(same);
+  }
+  {
+    network<sequential> nn;
+    convolutional_layer c(12, 12, 3, 2, 16, padding::same);
+    c.weight_init(weight_init::he()).bias_init(weight_init::constant(0.5f));
+    fully_connected_layer f(2304, 10);
+    f.weight_init(weight_init::lecun());
+    fully_connected_layer g(10, 4);
+    g.weight_init(weight_init::gaussian(0.3f));
+    nn << c << f << g;
+    nn.init_weight();
+    double mean, var; float lo, hi;
+    stats_of(nn.weights(0, 0), mean, var, lo, hi);   // he: N(0, sqrt(2 / 18)), 288 draws
+    EXPECT(std::fabs(var / (2.0 / 18) - 1) < 0.3 && std::fabs(mean) < 0.08);
+    for (float b : nn.weights(0, 1)) EXPECT(b == 0.5f);
+    stats_of(nn.weights(1, 0), mean, var, lo, hi);   // lecun: U(+-1/sqrt(2304)), 23040 draws
+    EXPECT(lo >= -1.f / 48 && hi <= 1.f / 48 && std::fabs(var / (1.0 / 2304 / 3) - 1) < 0.05);
+    stats_of(nn.weights(2, 0), mean, var, lo, hi);   // gaussian(0.3), 40 draws
+    EXPECT(var > 0.03 && var < 0.2);
+  }
+  // a fresh network trains without set_weights: fit draws the initial weights (network.h:853)
+  std::vector<vec_t> inputs = random_tensor(8, 288, 31);
+  std::vector<label_t> labels{0, 1, 2, 3, 4, 5, 6, 7};
+  std::vector<vec_t> targets(8, vec_t(10, 0.f));
+  for (size_t i = 0; i < 8; ++i) targets[i][labels[i]] = 1.f;
+  network<sequential> a, b, c;
+  make(a); make(b); make(c);
+  adam oa, ob, oc;
+  set_random_seed(7);
+  EXPECT((a.train<cross_entropy_multiclass>(oa, inputs, labels, 8, 1)));
+  // train_once is the same step
+  set_random_seed(7);
+  b.init_weight();
+  b.train_once<cross_entropy_multiclass>(ob, inputs.data(), targets.data(), 8);
+  // and so are fprop + bprop + update_weights
+  set_random_seed(7);
+  c.init_weight();
+  const std::vector<vec_t> y = c.fprop(inputs);
+  EXPECT(y.size() == 8 && y[0].size() == 10);
+  float sum = 0;
+  for (float v : y[3]) sum += v;
+  EXPECT(std::fabs(sum - 1.f) < 1e-5f);   // softmax output
+  c.bprop<cross_entropy_multiclass>(y, targets);
+  const vec_t g = c.weights_grads(5, 1);  // db of the last layer: sum over samples of y - t
+  vec_t want(10, 0.f);
+  for (size_t s = 0; s < 8; ++s)
+    for (size_t i = 0; i < 10; ++i) want[i] += y[s][i] - targets[s][i];
+  expect_near(g, want, 1e-4f, "db of the last layer after bprop");
+  c.update_weights(&oc);
+  for (float v : c.weights_grads(5, 1)) EXPECT(v == 0.f);   // cleared by the update
+  for (int i : {0, 3, 5})
+    for (int which = 0; which < 2; ++which) {
+      const vec_t wa = a.weights(i, which), wb = b.weights(i, which), wc = c.weights(i, which);
+      EXPECT(wa == wb);
+      EXPECT(wa == wc);
+    }
+  EXPECT(oa.b1_t == ob.b1_t && oa.b1_t == oc.b1_t && oa.b1_t != adam().b1_t);
+  // train() builds its targets from the last layer's out_value_range (tanh: -0.8 / 0.8)
+  network<sequential> t1, t2;
+  t1 << fully_connected_layer(288, 10) << tanh_layer();
+  t2 << fully_connected_layer(288, 10) << tanh_layer();
+  set_random_seed(3); t1.init_weight();
+  set_random_seed(3); t2.init_weight();
+  gradient_descent g1, g2;
+  std::vector<vec_t> scaled(8, vec_t(10, -0.8f));
+  for (size_t i = 0; i < 8; ++i) scaled[i][labels[i]] = 0.8f;
+  EXPECT((t1.train<mse>(g1, inputs, labels, 8, 1)));
+  EXPECT((t2.fit<mse>(g2, inputs, scaled, 8, 1)));
+  EXPECT(t1.weights(0, 0) == t2.weights(0, 0));
+}
+
+// the reference's whole-net numerical gradient checks (test/test_network.h:448-531) with its
+// data generator (test/testhelper.h:227-253) and tolerance (epsilon<float>() = 1e-2,
+// testhelper.h:198-201): an oracle-independent check of the backward pass on the GPU
+template <typename Loss, typename A1, typename A2, typename A3, typename A4>
+static void gradient_check_case(const char *name, float eps, bool last_act = true) {
+  network<sequential> nn;
+  nn << fully_connected_layer(10, 14 * 14 * 3) << A1() << convolutional_layer(14, 14, 5, 3, 6) << A2()
+     << average_pooling_layer(10, 10, 6, 2) << A3() << fully_connected_layer(5 * 5 * 6, 3);
+  if (last_act) nn << A4();
+  std::vector<tensor_t> a(5, tensor_t(1, vec_t(nn.in_data_size(), 0.0f)));
+  std::vector<std::vector<label_t>> t(5, std::vector<label_t>(1));
+  for (size_t sample = 0; sample < 5; ++sample) {
+    for (float &v : a[sample][0]) {
+      std::uniform_real_distribution<float> dst(-1, 1);
+      v = dst(random_generator::get_instance()());
+    }
+    t[sample][0] = sample % 2;
+  }
+  nn.init_weight();
+  const bool ok = nn.gradient_check<Loss>(a, t, eps, GRAD_CHECK_RANDOM);
+  ++g_checks;
+  if (!ok) {
+    ++g_failed;
+    std::printf("  FAILED gradient_check %s: numeric %g, bprop %g\n", name, nn.last_numeric_gradient(),
+                nn.last_bprop_gradient());
+  }
+}
+static void gradient_checks() {
+  std::puts("network.gradient_check 1-5 (test/test_network.h:448-531)");
+  gradient_check_case<cross_entropy, sigmoid_layer, sigmoid_layer, sigmoid_layer, sigmoid_layer>("sigmoid / cross-entropy", 1e-2f);
+  gradient_check_case<mse, tanh_layer, tanh_layer, tanh_layer, tanh_layer>("tanh / mse", 1e-2f);
+  gradient_check_case<mse, tanh_layer, sigmoid_layer, relu_layer, relu_layer>("mixture / mse", 1e-2f, false);
+  gradient_check_case<cross_entropy, softmax_layer, softmax_layer, softmax_layer, softmax_layer>("softmax / cross-entropy", 1e-1f);
+  // not in the reference's list: the closing softmax under cross_entropy_multiclass, which the
+  // device step computes in closed form (smooth activations: a central difference across a
+  // relu kink is off by that unit's whole share of the gradient)
+  gradient_check_case<cross_entropy_multiclass, tanh_layer, sigmoid_layer, tanh_layer, softmax_layer>("softmax / cross-entropy-multiclass", 1e-2f);
+  // GRAD_CHECK_ALL on a small net
+  network<sequential> nn;
+  nn << convolutional_layer(6, 6, 3, 1, 2) << tanh_layer() << max_pooling_layer(4, 4, 2, 2) << fully_connected_layer(8, 2)
+     << sigmoid_layer();
+  std::vector<tensor_t> a(3, tensor_t(1, random_vec(36, 77)));
+  a[1][0] = random_vec(36, 78); a[2][0] = random_vec(36, 79);
+  std::vector<std::vector<label_t>> t{{0}, {1}, {0}};
+  nn.init_weight();
+  EXPECT((nn.gradient_check<mse>(a, t, 1e-2f, GRAD_CHECK_ALL)));
+}
+
 // a crash of the host process names its call chain instead of dying silently
 static void on_fatal_signal(int sig) {
   void *frames[64];
@@ -553,6 +818,9 @@ int main() {
     weight_files();
     net_fit_vs_oracle<gradient_descent>("gradient_descent", TDO_OPT_SGD);
     net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM);
+    resident_stack_through_the_mirror();
+    weight_init_and_network_api();
+    gradient_checks();
   } catch (const std::exception &e) {
     std::printf("EXCEPTION: %s\n", e.what());
     return 2;

@@ -477,6 +477,22 @@ int tdh_net_reset_optimizer(tdh_net *net) {
   }
   return TDH_OK;
 }
+int tdh_net_update_weights(tdh_net *net, tdh_opt *opt) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && opt, "tdh_net_update_weights: null argument");
+  // the optimizer kernel keeps the packed filter copies of a graph net current, as in a step
+  return launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
+                                 net->opt_params, 1.0f, 1, nullptr);
+}
+int tdh_net_clear_grads(tdh_net *net) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net != nullptr, "tdh_net_clear_grads: null net");
+  for (tdh_net::Layer &L : net->layers) {
+    if (L.dw && L.w_size) TDH_TRY(launch_fill_zero(L.dw, L.w_size * sizeof(float)));
+    if (L.db && L.b_size) TDH_TRY(launch_fill_zero(L.db, L.b_size * sizeof(float)));
+  }
+  return TDH_OK;
+}
 int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst) {
   TDH_REQUIRE_INIT();
   const float *src = net_param_ptr(net, layer, which);

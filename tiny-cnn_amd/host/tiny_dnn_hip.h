@@ -154,7 +154,208 @@ class device_tensor {
   std::vector<float> stage_;
 };
 
+// ---- device mirror of host tensors ------------------------------------------------------
+// tiny-dnn's tensors are owned by edges (tiny_dnn/node.h:130-135) and only borrowed by
+// OpKernel::compute (tiny_dnn/core/framework/op_kernel.h:74-96). The operators below keep a
+// device image of every tensor they are handed, in a table keyed by the identity of the host
+// tensor_t (edge tensors have stable addresses), with one valid bit per side:
+//
+//   write-through (the default): compute() uploads its inputs and downloads its outputs, so a
+//     caller sees exactly what the reference's CPU kernels leave in the host vectors;
+//   resident (set_device_resident(true)): an input is uploaded only when the host side is the
+//     newer one, outputs stay on the device, and the host copy is brought up to date only when
+//     the host asks for it with to_host(t). Host code that writes a tensor says so with
+//     host_modified(t). Weights, activations and gradients then stay on the device across
+//     forward_propagation, back_propagation and optimizer::update.
+struct transfer_counters {
+  size_t h2d_calls = 0, h2d_bytes = 0, d2h_calls = 0, d2h_bytes = 0;
+};
+inline transfer_counters &transfers() {
+  static transfer_counters c;
+  return c;
+}
+
+class mirror {
+ public:
+  static mirror &get() {
+    static mirror m;
+    return m;
+  }
+  bool resident = false;
+
+  // device image of rows [0, rows) x len of t, for reading
+  const float *read(const tensor_t &t, size_t rows, size_t len) {
+    entry &e = find(t, rows, len);
+    if (!e.dev_valid || !resident) upload(e, t, rows, len);
+    return e.dev;
+  }
+  // ... for overwriting: nothing is uploaded; the host copy is stale until to_host / commit
+  float *write(tensor_t &t, size_t rows, size_t len) {
+    entry &e = find(t, rows, len);
+    reserve(e, rows * len);
+    e.rows = rows; e.len = len;
+    e.dev_valid = true; e.host_valid = false;
+    return e.dev;
+  }
+  // ... for adding to (weight and bias gradients: the reference's +=)
+  float *update(tensor_t &t, size_t rows, size_t len) {
+    entry &e = find(t, rows, len);
+    if (!e.dev_valid || !resident) upload(e, t, rows, len);
+    e.host_valid = false;
+    return e.dev;
+  }
+  // after a compute(): write-through brings the host copy up to date now
+  void commit(tensor_t &t) {
+    if (!resident) to_host(t);
+  }
+  void to_host(tensor_t &t) {
+    auto it = table_.find(&t);
+    if (it == table_.end() || it->second.host_valid || !it->second.dev_valid) return;
+    entry &e = it->second;
+    const size_t rows = e.rows, len = e.len;
+    e.stage.resize(rows * len);
+    if (rows * len > 0) {
+      check(tdh_memcpy_d2h(e.stage.data(), e.dev, rows * len * sizeof(float)));
+      transfers().d2h_calls++; transfers().d2h_bytes += rows * len * sizeof(float);
+    }
+    if (t.size() < rows) t.resize(rows);
+    for (size_t s = 0; s < rows; ++s) {
+      if (t[s].size() < len) t[s].resize(len);
+      std::memcpy(t[s].data(), e.stage.data() + s * len, len * sizeof(float));
+    }
+    e.host_valid = true;
+    remember(e, t);
+  }
+  void host_modified(const tensor_t &t) {
+    auto it = table_.find(&t);
+    if (it != table_.end()) { it->second.dev_valid = false; it->second.host_valid = true; }
+  }
+  // zero on both sides without a transfer (edge::clear_grads, tiny_dnn/node.h:105-111)
+  void clear(tensor_t &t) {
+    for (auto &row : t) std::fill(row.begin(), row.end(), float_t(0));
+    auto it = table_.find(&t);
+    if (it == table_.end()) return;
+    entry &e = it->second;
+    if (e.dev && e.rows * e.len > 0) check(tdh_fill_zero(e.dev, e.rows * e.len * sizeof(float)));
+    e.dev_valid = e.dev != nullptr; e.host_valid = true;
+  }
+  void release(const tensor_t &t) {
+    auto it = table_.find(&t);
+    if (it == table_.end()) return;
+    if (it->second.dev) tdh_free(it->second.dev);
+    rows_.erase(it->second.row0_vec);
+    table_.erase(it);
+  }
+  // floats per sample of t: of the device image where that is the newer side (the host rows
+  // of a resident tensor may never have been filled), else of the host rows
+  size_t row_length(const tensor_t &t) const {
+    auto it = table_.find(&t);
+    if (it != table_.end() && !it->second.host_valid && it->second.dev_valid) return it->second.len;
+    return t.empty() ? 0 : t[0].size();
+  }
+  // the tensor whose only mirrored row is this vector (optimizer::update is handed rows)
+  tensor_t *owner_of(const vec_t &row) {
+    auto it = rows_.find(&row);
+    return it == rows_.end() ? nullptr : const_cast<tensor_t *>(it->second);
+  }
+  ~mirror() {
+    for (auto &kv : table_)
+      if (kv.second.dev) tdh_free(kv.second.dev);
+  }
+
+ private:
+  struct entry {
+    float *dev = nullptr;
+    size_t cap = 0, rows = 0, len = 0;
+    const float *row0 = nullptr;     // data() of row 0 when the host side was last seen
+    const vec_t *row0_vec = nullptr;
+    bool host_valid = true, dev_valid = false;
+    std::vector<float> stage;
+  };
+  void reserve(entry &e, size_t floats) {
+    if (floats <= e.cap && e.dev) return;
+    if (e.dev) check(tdh_free(e.dev));
+    e.dev = nullptr;
+    void *p = nullptr;
+    check(tdh_malloc(&p, std::max<size_t>(floats, 1) * sizeof(float)));
+    e.dev = static_cast<float *>(p);
+    e.cap = std::max<size_t>(floats, 1);
+  }
+  void remember(entry &e, const tensor_t &t) {
+    if (e.row0_vec) rows_.erase(e.row0_vec);
+    e.row0     = t.empty() ? nullptr : t[0].data();
+    e.row0_vec = t.empty() ? nullptr : &t[0];
+    if (e.row0_vec) rows_[e.row0_vec] = &t;
+  }
+  entry &find(const tensor_t &t, size_t rows, size_t len) {
+    entry &e = table_[&t];
+    // another image than the one held (a resized or re-created host tensor): whatever the
+    // device holds is of no use unless it is the only valid copy
+    const bool same = e.rows == rows && e.len == len && !t.empty() && t[0].data() == e.row0;
+    if (!same && e.host_valid) e.dev_valid = false;
+    if (!same && !e.host_valid && (e.rows < rows || e.len != len)) {
+      // the device holds the newer values of a smaller image: save them before it is replaced
+      to_host(const_cast<tensor_t &>(t));
+      e.dev_valid = false;
+    }
+    if (e.row0_vec == nullptr || (!t.empty() && &t[0] != e.row0_vec)) remember(e, t);
+    return e;
+  }
+  void upload(entry &e, const tensor_t &t, size_t rows, size_t len) {
+    if (!e.host_valid) {  // resident and the device is newer: nothing to send
+      if (e.rows >= rows && e.len == len) return;
+      throw nn_error("device mirror: a tensor was resized while its newest values were on the device");
+    }
+    if (t.size() < rows) throw nn_error("tensor has fewer samples than the call needs");
+    reserve(e, rows * len);
+    e.stage.resize(rows * len);
+    for (size_t s = 0; s < rows; ++s) {
+      if (t[s].size() < len) throw nn_error("tensor row shorter than the layer shape");
+      std::memcpy(e.stage.data() + s * len, t[s].data(), len * sizeof(float));
+    }
+    if (rows * len > 0) {
+      check(tdh_memcpy_h2d(e.dev, e.stage.data(), rows * len * sizeof(float)));
+      transfers().h2d_calls++; transfers().h2d_bytes += rows * len * sizeof(float);
+    }
+    e.rows = rows; e.len = len; e.dev_valid = true;
+    remember(e, t);
+  }
+  std::map<const tensor_t *, entry> table_;
+  std::map<const vec_t *, const tensor_t *> rows_;
+};
+
+// device argmax records of a max-pool layer, shared by its forward and backward operators
+// (the reference keeps them in maxpool_params::out2inmax)
+struct argmax_store {
+  device_tensor idx;
+  size_t samples = 0;
+  bool host_valid = true;
+};
+inline argmax_store &argmax_of(const void *params) {
+  static std::map<const void *, std::shared_ptr<argmax_store>> table;
+  std::shared_ptr<argmax_store> &p = table[params];
+  if (!p) p.reset(new argmax_store());
+  return *p;
+}
+
 }  // namespace detail
+
+// ---- the host's side of the mirror protocol (see detail::mirror) ----
+inline void set_device_resident(bool on) { detail::mirror::get().resident = on; }
+inline bool device_resident() { return detail::mirror::get().resident; }
+// brings the host copy of t up to date (a download only if the device holds newer values)
+inline void to_host(tensor_t &t) { detail::mirror::get().to_host(t); }
+// the host has written t: the device copy is stale
+inline void host_modified(const tensor_t &t) { detail::mirror::get().host_modified(t); }
+// edge::clear_grads (tiny_dnn/node.h:105-111) on both sides, without a transfer
+inline void clear_grads(tensor_t &t) { detail::mirror::get().clear(t); }
+// frees the device image of a tensor that is about to be destroyed
+inline void release_device_copy(const tensor_t &t) { detail::mirror::get().release(t); }
+// host<->device copies made by the mirror since the last reset (for tests of residency)
+inline detail::transfer_counters transfer_stats() { return detail::transfers(); }
+inline void reset_transfer_stats() { detail::transfers() = detail::transfer_counters(); }
+
+class layer;
 
 namespace core {
 
@@ -258,9 +459,15 @@ class OpKernelContext {
     in_grad_  = &in_grad;
   }
   tensor_t &input(const int idx) { return *(*in_data_)[idx]; }
+  const tensor_t &input(const int idx) const { return *(*in_data_)[idx]; }
   tensor_t &output(const int idx) { return *(*out_data_)[idx]; }
+  const tensor_t &output(const int idx) const { return *(*out_data_)[idx]; }
   tensor_t &input_grad(const int idx) { return *(*in_grad_)[idx]; }
+  const tensor_t &input_grad(const int idx) const { return *(*in_grad_)[idx]; }
   tensor_t &output_grad(const int idx) { return *(*out_grad_)[idx]; }
+  const tensor_t &output_grad(const int idx) const { return *(*out_grad_)[idx]; }
+  void setLayer(layer *l) { layer_ = l; }   // op_kernel.h:112-114
+  layer *Layer() const { return layer_; }
   void setParams(Params *params) { params_ = params; }
   Params *params() const { return params_; }
   void setParallelize(const bool parallelize) { parallelize_ = parallelize; }
@@ -275,6 +482,7 @@ class OpKernelContext {
                           *in_grad_ = nullptr;
   Params *params_   = nullptr;
   Device *device_   = nullptr;
+  layer *layer_     = nullptr;
   bool parallelize_ = false;
   backend_t engine_ = default_engine();
 };
@@ -337,6 +545,10 @@ inline tdh_pool_desc pool_desc(const P &p) {
 
 // ---- operators: same class names and compute() contract as tiny_dnn/core/kernels/*_op.h ----
 
+// Every compute() takes its tensors through the device mirror (detail::mirror): inputs are
+// uploaded only when the device does not hold their newest values, outputs stay on the device in
+// resident mode and are written through to the host vectors otherwise.
+
 // tiny_dnn/core/kernels/conv2d_op.h:18-52
 class Conv2dOp : public core::OpKernel {
  public:
@@ -346,19 +558,17 @@ class Conv2dOp : public core::OpKernel {
     detail::ensure_init();
     auto &params = OpKernel::params_->conv();
     detail::conv_desc_holder h(params);
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &in = context.input(0);
-    const tensor_t &W  = context.input(1);
     tensor_t &out      = context.output(0);
     const size_t n = in.size();
-    float *bias = params.has_bias ? b_.upload(context.input(2)[0], params.out.depth_) : nullptr;
-    y_.resize(n * params.out.size());
-    detail::check(tdh_conv2d_fwd(&h.d, static_cast<int>(n), x_.upload(in, n, params.in.size()),
-                                 w_.upload(W[0], params.weight.size()), bias, y_.get()));
-    y_.download(out, n, params.out.size());
+    const float *bias = params.has_bias ? m.read(context.input(2), 1, params.out.depth_) : nullptr;
+    const float *x = m.read(in, n, params.in.size());
+    const float *w = m.read(context.input(1), 1, params.weight.size());
+    if (out.size() < n) out.resize(n);
+    detail::check(tdh_conv2d_fwd(&h.d, static_cast<int>(n), x, w, bias, m.write(out, n, params.out.size())));
+    m.commit(out);
   }
-
- private:
-  detail::device_tensor x_, w_, b_, y_;
 };
 
 // tiny_dnn/core/kernels/conv2d_grad_op.h:17-51
@@ -370,27 +580,25 @@ class Conv2dGradOp : public core::OpKernel {
     detail::ensure_init();
     auto &params = OpKernel::params_->conv();
     detail::conv_desc_holder h(params);
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &prev_out = context.input(0);
-    const tensor_t &W        = context.input(1);
     tensor_t &dW             = context.input_grad(1);
     tensor_t &prev_delta     = context.input_grad(0);
-    tensor_t &curr_delta     = context.output_grad(0);
     const size_t n = prev_out.size();
-    dx_.resize(n * params.in.size());
-    dw_.resize(params.weight.size());
-    db_.resize(params.out.depth_);
-    detail::check(tdh_conv2d_bwd(&h.d, static_cast<int>(n),
-                                 x_.upload(prev_out, n, params.in.size()),
-                                 w_.upload(W[0], params.weight.size()),
-                                 dy_.upload(curr_delta, n, params.out.size()), dx_.get(), dw_.get(),
-                                 params.has_bias ? db_.get() : nullptr, /*accumulate=*/0));
-    dx_.download(prev_delta, n, params.in.size());   // dX is overwritten (conv2d_grad_op.h:34)
-    dw_.download_add(dW[0], params.weight.size());   // dW, db accumulate
-    if (params.has_bias) db_.download_add(context.input_grad(2)[0], params.out.depth_);
+    const float *x  = m.read(prev_out, n, params.in.size());
+    const float *w  = m.read(context.input(1), 1, params.weight.size());
+    const float *dy = m.read(context.output_grad(0), n, params.out.size());
+    if (prev_delta.size() < n) prev_delta.resize(n);
+    // dX is overwritten (conv2d_grad_op.h:34); dW and db are added to, reduced over the batch,
+    // in sample slot 0 of the gradient tensors
+    float *dx = m.write(prev_delta, n, params.in.size());
+    float *dw = m.update(dW, 1, params.weight.size());
+    float *db = params.has_bias ? m.update(context.input_grad(2), 1, params.out.depth_) : nullptr;
+    detail::check(tdh_conv2d_bwd(&h.d, static_cast<int>(n), x, w, dy, dx, dw, db, /*accumulate=*/1));
+    m.commit(prev_delta);
+    m.commit(dW);
+    if (params.has_bias) m.commit(context.input_grad(2));
   }
-
- private:
-  detail::device_tensor x_, w_, dy_, dx_, dw_, db_;
 };
 
 // tiny_dnn/core/kernels/fully_connected_op.h:20-65
@@ -401,20 +609,19 @@ class FullyConnectedOp : public core::OpKernel {
     detail::require_hip(context.engine());
     detail::ensure_init();
     auto &params = OpKernel::params_->fully();
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &in = context.input(0);
+    tensor_t &out      = context.output(0);
     const size_t n = in.size();
-    float *bias = params.has_bias_ ? b_.upload(context.input(2)[0], params.out_size_) : nullptr;
-    y_.resize(n * params.out_size_);
+    const float *bias = params.has_bias_ ? m.read(context.input(2), 1, params.out_size_) : nullptr;
+    const float *x = m.read(in, n, params.in_size_);
+    const float *w = m.read(context.input(1), 1, params.in_size_ * params.out_size_);
+    if (out.size() < n) out.resize(n);
     detail::check(tdh_fc_fwd(static_cast<int>(params.in_size_), static_cast<int>(params.out_size_),
-                             params.has_bias_, static_cast<int>(n),
-                             x_.upload(in, n, params.in_size_),
-                             w_.upload(context.input(1)[0], params.in_size_ * params.out_size_), bias,
-                             y_.get()));
-    y_.download(context.output(0), n, params.out_size_);
+                             params.has_bias_, static_cast<int>(n), x, w, bias,
+                             m.write(out, n, params.out_size_)));
+    m.commit(out);
   }
-
- private:
-  detail::device_tensor x_, w_, b_, y_;
 };
 
 // tiny_dnn/core/kernels/fully_connected_grad_op.h:17-53
@@ -425,26 +632,45 @@ class FullyConnectedGradOp : public core::OpKernel {
     detail::require_hip(context.engine());
     detail::ensure_init();
     auto &params = OpKernel::params_->fully();
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &prev_out = context.input(0);
+    tensor_t &prev_delta     = context.input_grad(0);
     const size_t n = prev_out.size(), in = params.in_size_, out = params.out_size_;
-    dx_.resize(n * in);
-    dw_.resize(in * out);
-    db_.resize(out);
+    const float *x  = m.read(prev_out, n, in);
+    const float *w  = m.read(context.input(1), 1, in * out);
+    const float *dy = m.read(context.output_grad(0), n, out);
+    if (prev_delta.size() < n) prev_delta.resize(n);
+    float *dx = m.write(prev_delta, n, in);
+    float *dw = m.update(context.input_grad(1), 1, in * out);
+    float *db = params.has_bias_ ? m.update(context.input_grad(2), 1, out) : nullptr;
     detail::check(tdh_fc_bwd(static_cast<int>(in), static_cast<int>(out), params.has_bias_,
-                             static_cast<int>(n), x_.upload(prev_out, n, in),
-                             w_.upload(context.input(1)[0], in * out),
-                             dy_.upload(context.output_grad(0), n, out), dx_.get(), dw_.get(),
-                             params.has_bias_ ? db_.get() : nullptr, 0));
-    dx_.download(context.input_grad(0), n, in);
-    dw_.download_add(context.input_grad(1)[0], in * out);
-    if (params.has_bias_) db_.download_add(context.input_grad(2)[0], out);
+                             static_cast<int>(n), x, w, dy, dx, dw, db, 1));
+    m.commit(prev_delta);
+    m.commit(context.input_grad(1));
+    if (params.has_bias_) m.commit(context.input_grad(2));
   }
-
- private:
-  detail::device_tensor x_, w_, dy_, dx_, dw_, db_;
 };
 
-// tiny_dnn/core/kernels/maxpool_op.h:18-63; params.out2inmax receives the argmax indices
+namespace detail {
+// maxpool_params::out2inmax from the device records (a download; resident callers ask for it
+// through max_pooling_layer::out2inmax())
+inline void argmax_to_host(core::maxpool_params &params) {
+  argmax_store &a = argmax_of(&params);
+  if (a.host_valid) return;
+  const size_t n = a.samples, osz = params.out.size();
+  std::vector<int32_t> host(n * osz);
+  if (n * osz > 0) {
+    check(tdh_memcpy_d2h(host.data(), a.idx.get(), host.size() * sizeof(int32_t)));
+    transfers().d2h_calls++; transfers().d2h_bytes += host.size() * sizeof(int32_t);
+  }
+  params.out2inmax.resize(n);
+  for (size_t s = 0; s < n; ++s) params.out2inmax[s].assign(host.begin() + s * osz, host.begin() + (s + 1) * osz);
+  a.host_valid = true;
+}
+}  // namespace detail
+
+// tiny_dnn/core/kernels/maxpool_op.h:18-63; the argmax records stay on the device for the
+// backward operator and reach params.out2inmax in write-through mode or on request
 class MaxPoolOp : public core::OpKernel {
  public:
   explicit MaxPoolOp(const core::OpKernelConstruction &context) : core::OpKernel(context) {}
@@ -453,21 +679,21 @@ class MaxPoolOp : public core::OpKernel {
     detail::ensure_init();
     auto &params = OpKernel::params_->maxpool();
     const tdh_pool_desc d = detail::pool_desc(params);
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &in = context.input(0);
+    tensor_t &out      = context.output(0);
     const size_t n = in.size(), osz = params.out.size();
-    y_.resize(n * osz);
-    idx_.resize(n * osz);
-    detail::check(tdh_maxpool_fwd(&d, static_cast<int>(n), x_.upload(in, n, params.in.size()),
-                                  y_.get(), reinterpret_cast<int32_t *>(idx_.get())));
-    y_.download(context.output(0), n, osz);
-    std::vector<int32_t> host(n * osz);
-    if (n * osz > 0) detail::check(tdh_memcpy_d2h(host.data(), idx_.get(), host.size() * sizeof(int32_t)));
-    params.out2inmax.resize(n);
-    for (size_t s = 0; s < n; ++s) params.out2inmax[s].assign(host.begin() + s * osz, host.begin() + (s + 1) * osz);
+    detail::argmax_store &a = detail::argmax_of(&params);
+    a.idx.resize(n * osz);
+    const float *x = m.read(in, n, params.in.size());
+    if (out.size() < n) out.resize(n);
+    detail::check(tdh_maxpool_fwd(&d, static_cast<int>(n), x, m.write(out, n, osz),
+                                  reinterpret_cast<int32_t *>(a.idx.get())));
+    a.samples = n;
+    a.host_valid = false;
+    m.commit(out);
+    if (!m.resident) detail::argmax_to_host(params);
   }
-
- private:
-  detail::device_tensor x_, y_, idx_;
 };
 
 // tiny_dnn/core/kernels/maxpool_grad_op.h:17-47
@@ -479,23 +705,33 @@ class MaxPoolGradOp : public core::OpKernel {
     detail::ensure_init();
     auto &params = OpKernel::params_->maxpool();
     const tdh_pool_desc d = detail::pool_desc(params);
+    detail::mirror &m = detail::mirror::get();
     tensor_t &prev_delta = context.input_grad(0);
     const tensor_t &curr_delta = context.output_grad(0);
     const size_t n = curr_delta.size(), osz = params.out.size();
-    if (params.out2inmax.size() < n) throw nn_error("max-pool backward without a recorded forward pass");
-    std::vector<int32_t> host(n * osz);
-    for (size_t s = 0; s < n; ++s)
-      for (size_t i = 0; i < osz; ++i) host[s * osz + i] = static_cast<int32_t>(params.out2inmax[s][i]);
-    idx_.resize(n * osz);
-    if (n * osz > 0) detail::check(tdh_memcpy_h2d(idx_.get(), host.data(), host.size() * sizeof(int32_t)));
-    dx_.resize(n * params.in.size());
-    detail::check(tdh_maxpool_bwd(&d, static_cast<int>(n), dy_.upload(curr_delta, n, osz),
-                                  reinterpret_cast<const int32_t *>(idx_.get()), dx_.get()));
-    dx_.download(prev_delta, n, params.in.size());
+    detail::argmax_store &a = detail::argmax_of(&params);
+    if (a.host_valid) {
+      // the host's records are the current ones (a caller wrote out2inmax, or no forward pass
+      // has run on the device yet)
+      if (params.out2inmax.size() < n) throw nn_error("max-pool backward without a recorded forward pass");
+      std::vector<int32_t> host(n * osz);
+      for (size_t s = 0; s < n; ++s)
+        for (size_t i = 0; i < osz; ++i) host[s * osz + i] = static_cast<int32_t>(params.out2inmax[s][i]);
+      a.idx.resize(n * osz);
+      if (n * osz > 0) {
+        detail::check(tdh_memcpy_h2d(a.idx.get(), host.data(), host.size() * sizeof(int32_t)));
+        detail::transfers().h2d_calls++; detail::transfers().h2d_bytes += host.size() * sizeof(int32_t);
+      }
+      a.samples = n;
+    } else if (a.samples < n) {
+      throw nn_error("max-pool backward over more samples than the forward pass");
+    }
+    const float *dy = m.read(curr_delta, n, osz);
+    if (prev_delta.size() < n) prev_delta.resize(n);
+    detail::check(tdh_maxpool_bwd(&d, static_cast<int>(n), dy, reinterpret_cast<const int32_t *>(a.idx.get()),
+                                  m.write(prev_delta, n, params.in.size())));
+    m.commit(prev_delta);
   }
-
- private:
-  detail::device_tensor dy_, dx_, idx_;
 };
 
 // new operators with MaxPool's contract for tiny_average_pooling_kernel / _back_kernel
@@ -508,17 +744,17 @@ class AvePoolOp : public core::OpKernel {
     detail::ensure_init();
     auto &params = OpKernel::params_->avepool();
     const tdh_pool_desc d = detail::pool_desc(params);
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &in = context.input(0);
+    tensor_t &out      = context.output(0);
     const size_t n = in.size(), c = params.in.depth_;
-    y_.resize(n * params.out.size());
-    detail::check(tdh_avepool_fwd(&d, static_cast<int>(n), x_.upload(in, n, params.in.size()),
-                                  w_.upload(context.input(1)[0], c), b_.upload(context.input(2)[0], c),
-                                  y_.get()));
-    y_.download(context.output(0), n, params.out.size());
+    const float *x = m.read(in, n, params.in.size());
+    const float *w = m.read(context.input(1), 1, c);
+    const float *b = m.read(context.input(2), 1, c);
+    if (out.size() < n) out.resize(n);
+    detail::check(tdh_avepool_fwd(&d, static_cast<int>(n), x, w, b, m.write(out, n, params.out.size())));
+    m.commit(out);
   }
-
- private:
-  detail::device_tensor x_, w_, b_, y_;
 };
 
 class AvePoolGradOp : public core::OpKernel {
@@ -529,28 +765,52 @@ class AvePoolGradOp : public core::OpKernel {
     detail::ensure_init();
     auto &params = OpKernel::params_->avepool();
     const tdh_pool_desc d = detail::pool_desc(params);
+    detail::mirror &m = detail::mirror::get();
     const tensor_t &prev_out = context.input(0);
+    tensor_t &prev_delta     = context.input_grad(0);
     const size_t n = prev_out.size(), c = params.in.depth_;
-    dx_.resize(n * params.in.size());
-    dw_.resize(c);
-    db_.resize(c);
-    detail::check(tdh_avepool_bwd(&d, static_cast<int>(n), x_.upload(prev_out, n, params.in.size()),
-                                  w_.upload(context.input(1)[0], c),
-                                  dy_.upload(context.output_grad(0), n, params.out.size()), dx_.get(),
-                                  dw_.get(), db_.get(), 0));
-    dx_.download(context.input_grad(0), n, params.in.size());
-    dw_.download_add(context.input_grad(1)[0], c);
-    db_.download_add(context.input_grad(2)[0], c);
+    const float *x  = m.read(prev_out, n, params.in.size());
+    const float *w  = m.read(context.input(1), 1, c);
+    const float *dy = m.read(context.output_grad(0), n, params.out.size());
+    if (prev_delta.size() < n) prev_delta.resize(n);
+    float *dx = m.write(prev_delta, n, params.in.size());
+    float *dw = m.update(context.input_grad(1), 1, c);
+    float *db = m.update(context.input_grad(2), 1, c);
+    detail::check(tdh_avepool_bwd(&d, static_cast<int>(n), x, w, dy, dx, dw, db, 1));
+    m.commit(prev_delta);
+    m.commit(context.input_grad(1));
+    m.commit(context.input_grad(2));
   }
-
- private:
-  detail::device_tensor x_, w_, dy_, dx_, dw_, db_;
 };
 
 // ---- loss functions (type tags; tiny_dnn/lossfunctions/loss_function.h) ----
-struct mse { static const int kind = TDH_LOSS_MSE; };
-struct cross_entropy { static const int kind = TDH_LOSS_CE; };
-struct cross_entropy_multiclass { static const int kind = TDH_LOSS_CE_MULTICLASS; };
+// f() is the loss value of one sample, evaluated on the host as the reference does (it is only
+// ever read by get_loss / gradient_check); the gradients df() run on the device (tdh_loss_grad)
+struct mse {  // loss_function.h:18-36
+  static const int kind = TDH_LOSS_MSE;
+  static float_t f(const vec_t &y, const vec_t &t) {
+    float_t d{0.0};
+    for (size_t i = 0; i < y.size(); ++i) d += (y[i] - t[i]) * (y[i] - t[i]);
+    return d / static_cast<float_t>(y.size());
+  }
+};
+struct cross_entropy {  // loss_function.h:108-128
+  static const int kind = TDH_LOSS_CE;
+  static float_t f(const vec_t &y, const vec_t &t) {
+    float_t d{0};
+    for (size_t i = 0; i < y.size(); ++i)
+      d += -t[i] * std::log(y[i]) - (float_t(1) - t[i]) * std::log(float_t(1) - y[i]);
+    return d;
+  }
+};
+struct cross_entropy_multiclass {  // loss_function.h:131-150
+  static const int kind = TDH_LOSS_CE_MULTICLASS;
+  static float_t f(const vec_t &y, const vec_t &t) {
+    float_t d{0.0};
+    for (size_t i = 0; i < y.size(); ++i) d += -t[i] * std::log(y[i]);
+    return d;
+  }
+};
 
 // ---- optimizers: the reference's members and update(dW, W, parallelize) signature
 // (tiny_dnn/optimizers/optimizer.h). State vectors live on the device, keyed by &W like the
@@ -574,9 +834,15 @@ struct device_optimizer : public optimizer {
       st.s0.resize(n); st.s1.resize(n); st.n = n;
       if (n) { check(tdh_fill_zero(st.s0.get(), n * sizeof(float))); check(tdh_fill_zero(st.s1.get(), n * sizeof(float))); }
     }
-    float *g = g_.upload(dW, n), *w = w_.upload(W, n);
+    // a weight vector (and its gradient) that the operators have mirrored is updated where it
+    // lies: resident callers never see it cross the bus
+    mirror &m = mirror::get();
+    tensor_t *Wt = m.owner_of(W), *Gt = m.owner_of(dW);
+    const float *g = Gt ? m.read(*Gt, 1, n) : g_.upload(dW, n);
+    float *w = Wt ? m.update(*Wt, 1, n) : w_.upload(W, n);
     check(tdh_opt_update(&o, n, g, 1.0f, w, st.s0.get(), st.s1.get()));
-    if (n) check(tdh_memcpy_d2h(W.data(), w, n * sizeof(float)));
+    if (Wt) m.commit(*Wt);
+    else if (n) check(tdh_memcpy_d2h(W.data(), w, n * sizeof(float)));
     absorb(o);
   }
   void reset() override { states_.clear(); }
@@ -653,6 +919,98 @@ struct nesterov_momentum : public detail::device_optimizer {
   float_t alpha, lambda, mu;
 };
 
+// ---- the reference's random source (tiny_dnn/util/random.h:19-69): one std::mt19937 for the
+// whole process, seeded with 1 until set_random_seed is called; bernoulli(p) is one draw of
+// uniform_real_distribution<float_t>(0, 1) compared with p ----
+class random_generator {
+ public:
+  static random_generator &get_instance() {
+    static random_generator g;
+    return g;
+  }
+  std::mt19937 &operator()() { return engine_; }
+  void set_seed(unsigned int seed) { engine_.seed(seed); }
+
+ private:
+  random_generator() : engine_(1) {}
+  std::mt19937 engine_;
+};
+inline void set_random_seed(unsigned int seed) { random_generator::get_instance().set_seed(seed); }
+inline bool bernoulli(float_t p) {
+  std::uniform_real_distribution<float_t> unit(float_t(0), float_t(1));
+  return unit(random_generator::get_instance()()) <= p;
+}
+
+namespace weight_init {
+// tiny_dnn/util/weight_init.h:15-108: the same classes, formulas and draw order (one fresh
+// std::uniform_real_distribution / std::normal_distribution per value from the process-wide
+// std::mt19937, tiny_dnn/util/random.h:44-79), so a program built against the same C++ library
+// starts from the reference's own initial weights
+class function {
+ public:
+  virtual ~function() {}
+  virtual void fill(vec_t *weight, size_t fan_in, size_t fan_out) = 0;
+};
+class scalable : public function {
+ public:
+  explicit scalable(float_t value) : scale_(value) {}
+  void scale(float_t value) { scale_ = value; }
+
+ protected:
+  float_t scale_;
+};
+inline void uniform_rand(vec_t *w, float_t lo, float_t hi) {
+  for (float_t &v : *w) {
+    std::uniform_real_distribution<float_t> dst(lo, hi);
+    v = dst(random_generator::get_instance()());
+  }
+}
+inline void gaussian_rand(vec_t *w, float_t mean, float_t sigma) {
+  for (float_t &v : *w) {
+    std::normal_distribution<float_t> dst(mean, sigma);
+    v = dst(random_generator::get_instance()());
+  }
+}
+class xavier : public scalable {  // U(+-sqrt(scale / (fan_in + fan_out))), scale 6
+ public:
+  xavier() : scalable(float_t(6)) {}
+  explicit xavier(float_t value) : scalable(value) {}
+  void fill(vec_t *weight, size_t fan_in, size_t fan_out) override {
+    const float_t weight_base = std::sqrt(scale_ / (fan_in + fan_out));
+    uniform_rand(weight, -weight_base, weight_base);
+  }
+};
+class lecun : public scalable {   // U(+-scale / sqrt(fan_in)), scale 1
+ public:
+  lecun() : scalable(float_t{1}) {}
+  explicit lecun(float_t value) : scalable(value) {}
+  void fill(vec_t *weight, size_t fan_in, size_t) override {
+    const float_t weight_base = scale_ / std::sqrt(float_t(fan_in));
+    uniform_rand(weight, -weight_base, weight_base);
+  }
+};
+class gaussian : public scalable {  // N(0, sigma)
+ public:
+  gaussian() : scalable(float_t{1}) {}
+  explicit gaussian(float_t sigma) : scalable(sigma) {}
+  void fill(vec_t *weight, size_t, size_t) override { gaussian_rand(weight, float_t{0}, scale_); }
+};
+class constant : public scalable {
+ public:
+  constant() : scalable(float_t{0}) {}
+  explicit constant(float_t value) : scalable(value) {}
+  void fill(vec_t *weight, size_t, size_t) override { std::fill(weight->begin(), weight->end(), scale_); }
+};
+class he : public scalable {      // N(0, sqrt(scale / fan_in)), scale 2
+ public:
+  he() : scalable(float_t{2}) {}
+  explicit he(float_t value) : scalable(value) {}
+  void fill(vec_t *weight, size_t fan_in, size_t) override {
+    gaussian_rand(weight, float_t{0}, std::sqrt(scale_ / fan_in));
+  }
+};
+}  // namespace weight_init
+
 // ---- layers: constructor arguments as in tiny_dnn/layers/*.h; they only describe the layer,
 // network<sequential> turns the descriptions into one device-resident tdh_net ----
 struct layer_desc {
@@ -662,9 +1020,33 @@ struct layer_desc {
 
 class layer {
  public:
+  layer() : weight_init_(std::make_shared<weight_init::xavier>()),
+            bias_init_(std::make_shared<weight_init::constant>()) {}  // layer.h:72-73
   virtual ~layer() {}
   virtual layer_desc describe(const shape3d &prev_out) const = 0;
   virtual std::string layer_type() const = 0;
+  // number of incoming connections of an output unit / outgoing ones of an input unit, which
+  // the initialisers scale by (layer.h:298-306)
+  virtual size_t fan_in_size() const { return 0; }
+  virtual size_t fan_out_size() const { return 0; }
+  // the (off, on) values label2vec turns class labels into when this is the last layer
+  // (layer.h:276-278; activation layers give their scale(), activation_layer.h:121)
+  virtual std::pair<float_t, float_t> out_value_range() const { return {float_t{0.0}, float_t{1.0}}; }
+  // entries of the weight vector as the reference declares it, where that is more than this
+  // library keeps (average pooling): init_weight draws that many values
+  virtual size_t declared_weight_size(size_t kept) const { return kept; }
+  // layer::weight_init / bias_init (layer.h:338-360)
+  template <typename WeightInit>
+  layer &weight_init(const WeightInit &f) {
+    weight_init_ = std::make_shared<WeightInit>(f);
+    return *this;
+  }
+  template <typename BiasInit>
+  layer &bias_init(const BiasInit &f) {
+    bias_init_ = std::make_shared<BiasInit>(f);
+    return *this;
+  }
+  std::shared_ptr<weight_init::function> weight_init_, bias_init_;
 };
 
 // tiny_dnn/layers/convolutional_layer.h:64-100
@@ -699,6 +1081,12 @@ class convolutional_layer : public layer {
     kernel_back_.reset(new Conv2dGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "conv"; }
+  // convolutional_layer.h:269-277
+  size_t fan_in_size() const override { return params_.weight.width_ * params_.weight.height_ * params_.in.depth_; }
+  size_t fan_out_size() const override {
+    return (params_.weight.width_ / params_.w_stride) * (params_.weight.height_ / params_.h_stride) *
+           params_.out.depth_;
+  }
   std::vector<shape3d> in_shape() const {
     return {params_.in, shape3d(params_.weight.width_, params_.weight.height_, params_.weight.depth_),
             shape3d(1, 1, params_.out.depth_)};
@@ -752,6 +1140,8 @@ class fully_connected_layer : public layer {
     kernel_back_.reset(new FullyConnectedGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "fully-connected"; }
+  size_t fan_in_size() const override { return params_.in_size_; }     // fully_connected_layer.h:51-53
+  size_t fan_out_size() const override { return params_.out_size_; }
   void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data);
@@ -812,6 +1202,12 @@ class max_pooling_layer : public layer {
   }
   std::string layer_type() const override { return "max-pool"; }
   std::vector<shape3d> out_shape() const { return {params_.out}; }
+  // maxpool_params::out2inmax of the last forward pass (downloads the device records if they
+  // are the newer ones)
+  const std::vector<std::vector<size_t>> &out2inmax() {
+    detail::argmax_to_host(params_);
+    return params_.out2inmax;
+  }
   void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data);
@@ -858,6 +1254,13 @@ class average_pooling_layer : public layer {
     kernel_back_.reset(new AvePoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "ave-pool"; }
+  // partial_connected_layer.h:46-48 with the connections of average_pooling_layer.h:270-304:
+  // every output reads pool_x*pool_y inputs, every input feeds one output (windows that tile)
+  size_t fan_in_size() const override { return params_.pool_size_x * params_.pool_size_y; }
+  size_t fan_out_size() const override { return 1; }
+  size_t declared_weight_size(size_t kept) const override {  // average_pooling_layer.h:222-226
+    return kept * params_.pool_size_x * params_.pool_size_y;
+  }
   std::vector<shape3d> out_shape() const { return {params_.out}; }
   void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
     core::OpKernelContext ctx;
@@ -891,6 +1294,13 @@ class average_pooling_layer : public layer {
 class activation_layer : public layer {
  public:
   std::string layer_type() const override { return type_; }
+  // *_layer::scale() of the reference's activations: tanh and asinh (-0.8, 0.8), softmax (0, 1),
+  // all others (0.1, 0.9)
+  std::pair<float_t, float_t> out_value_range() const override {
+    if (kind_ == TDH_ACT_TANH || kind_ == TDH_ACT_ASINH) return {float_t(-0.8), float_t(0.8)};
+    if (kind_ == TDH_ACT_SOFTMAX) return {float_t(0), float_t(1)};
+    return {float_t(0.1), float_t(0.9)};
+  }
   layer_desc describe(const shape3d &) const override {
     layer_desc r;
     std::memset(&r.l, 0, sizeof(r.l));
@@ -899,6 +1309,32 @@ class activation_layer : public layer {
     r.l.act_p[0] = p_[0];
     r.l.act_p[1] = p_[1];
     return r;
+  }
+  // activation_layer::forward_propagation / back_propagation (activation_layer.h:74-91) over
+  // whole batches, through the device mirror like the operators
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+    detail::ensure_init();
+    detail::mirror &m = detail::mirror::get();
+    const tensor_t &x = *in_data[0];
+    tensor_t &y       = *out_data[0];
+    const size_t n = x.size(), len = m.row_length(x);
+    if (y.size() < n) y.resize(n);
+    const float *xd = m.read(x, n, len);
+    detail::check(tdh_act_fwd_p(kind_, p_, static_cast<int>(n), static_cast<int>(len), xd, m.write(y, n, len)));
+    m.commit(y);
+  }
+  void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+    detail::ensure_init();
+    detail::mirror &m = detail::mirror::get();
+    const tensor_t &y = *out_data[0];
+    tensor_t &dx      = *in_grad[0];
+    const size_t n = y.size(), len = m.row_length(y);
+    if (dx.size() < n) dx.resize(n);
+    const float *xd = m.read(*in_data[0], n, len), *yd = m.read(y, n, len), *dyd = m.read(*out_grad[0], n, len);
+    detail::check(tdh_act_bwd_p(kind_, p_, static_cast<int>(n), static_cast<int>(len), xd, yd, dyd,
+                                m.write(dx, n, len)));
+    m.commit(dx);
   }
   void forward_activation(const vec_t &x, vec_t &y) {
     detail::ensure_init();
@@ -964,28 +1400,6 @@ struct softplus_layer : activation_layer {
 struct softsign_layer : activation_layer { softsign_layer() : activation_layer(TDH_ACT_SOFTSIGN, "softsign-activation") {} };
 struct asinh_layer : activation_layer { asinh_layer() : activation_layer(TDH_ACT_ASINH, "asinh-activation") {} };
 struct tanh_p1m2_layer : activation_layer { tanh_p1m2_layer() : activation_layer(TDH_ACT_TANH_P1M2, "tanh-scaled-activation") {} };
-
-// ---- the reference's random source (tiny_dnn/util/random.h:19-69): one std::mt19937 for the
-// whole process, seeded with 1 until set_random_seed is called; bernoulli(p) is one draw of
-// uniform_real_distribution<float_t>(0, 1) compared with p ----
-class random_generator {
- public:
-  static random_generator &get_instance() {
-    static random_generator g;
-    return g;
-  }
-  std::mt19937 &operator()() { return engine_; }
-  void set_seed(unsigned int seed) { engine_.seed(seed); }
-
- private:
-  random_generator() : engine_(1) {}
-  std::mt19937 engine_;
-};
-inline void set_random_seed(unsigned int seed) { random_generator::get_instance().set_seed(seed); }
-inline bool bernoulli(float_t p) {
-  std::uniform_real_distribution<float_t> unit(float_t(0), float_t(1));
-  return unit(random_generator::get_instance()()) <= p;
-}
 
 enum class net_phase { train, test };  // tiny_dnn/util/util.h:71
 
@@ -1234,6 +1648,7 @@ class feeder {
 }  // namespace detail
 
 struct sequential {};
+enum grad_check_mode { GRAD_CHECK_ALL, GRAD_CHECK_RANDOM };  // tiny_dnn/util/util.h:68-69
 
 // network<sequential> (tiny_dnn/network.h:148-1105): operator<<, fit, train, predict. Weights
 // live on the device; weights()/set_weights() copy one parameter tensor at a time.
@@ -1288,9 +1703,19 @@ class network<sequential> {
   template <typename Error, typename Optimizer, typename OnBatch, typename OnEpoch>
   bool fit(Optimizer &opt, const std::vector<vec_t> &inputs, const std::vector<vec_t> &desired_outputs,
            size_t batch_size, int epoch, OnBatch on_batch_enumerate, OnEpoch on_epoch_enumerate) {
+    return fit<Error>(opt, inputs, desired_outputs, batch_size, epoch, on_batch_enumerate,
+                      on_epoch_enumerate, /*reset_weights=*/false);
+  }
+  // reset_weights: network::fit's argument of that name (tiny_dnn/network.h:368-386); weights
+  // that have never been set or initialised are drawn by init_weight either way (:852-853,
+  // layer::setup, tiny_dnn/layers/layer.h:584-614)
+  template <typename Error, typename Optimizer, typename OnBatch, typename OnEpoch>
+  bool fit(Optimizer &opt, const std::vector<vec_t> &inputs, const std::vector<vec_t> &desired_outputs,
+           size_t batch_size, int epoch, OnBatch on_batch_enumerate, OnEpoch on_epoch_enumerate,
+           bool reset_weights) {
     if (inputs.size() != desired_outputs.size() || inputs.empty() || batch_size == 0) return false;
     build(batch_size);
-    if (!initialized_) throw nn_error("fit: weights have not been set (set_weights)");
+    if (reset_weights || !initialized_) init_weight();
     const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
     opt.reset();  // network.h:856; the device copy of the state vectors is cleared with it
     detail::check(tdh_net_reset_optimizer(net_));
@@ -1319,18 +1744,19 @@ class network<sequential> {
     return true;
   }
 
-  // network::train (tiny_dnn/network.h:284-308): labels become one-hot targets {0,1}
-  // (nodes::label2vec with the default out_value_range, tiny_dnn/nodes.h:180-189)
+  // network::train (tiny_dnn/network.h:284-308): labels become one-hot targets whose off / on
+  // values are the last layer's out_value_range (nodes::label2vec, tiny_dnn/nodes.h:180-189)
   template <typename Error, typename Optimizer>
   bool train(Optimizer &opt, const std::vector<vec_t> &inputs, const std::vector<label_t> &class_labels,
              size_t batch_size, int epoch) {
     if (inputs.size() != class_labels.size() || inputs.size() < batch_size) return false;
     build(batch_size);
     const size_t out_len = tdh_net_out_size(net_);
-    std::vector<vec_t> t(class_labels.size(), vec_t(out_len, float_t(0)));
+    const std::pair<float_t, float_t> range = layers_.back()->out_value_range();
+    std::vector<vec_t> t(class_labels.size(), vec_t(out_len, range.first));
     for (size_t i = 0; i < class_labels.size(); ++i) {
       if (class_labels[i] >= out_len) throw nn_error("label out of range");
-      t[i][class_labels[i]] = float_t(1);
+      t[i][class_labels[i]] = range.second;
     }
     return fit<Error>(opt, inputs, t, batch_size, epoch);
   }
@@ -1384,6 +1810,164 @@ class network<sequential> {
     initialized_ = true;
   }
 
+  // network::init_weight (tiny_dnn/network.h:165) -> layer::init_weight
+  // (tiny_dnn/layers/layer.h:625-655): layers front to back, weight before bias, each filled
+  // by the layer's weight_init / bias_init function with the layer's fan sizes
+  void init_weight() {
+    build(max_batch_ ? max_batch_ : 1);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+      layer &l = *layers_[i];
+      for (int which = 0; which < 2; ++which) {
+        const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which);
+        if (!n) continue;
+        vec_t v(which == 0 ? l.declared_weight_size(n) : n);
+        (which == 0 ? l.weight_init_ : l.bias_init_)->fill(&v, l.fan_in_size(), l.fan_out_size());
+        v.resize(n);
+        detail::check(tdh_net_set_param(net_, static_cast<int>(i), which, v.data()));
+      }
+    }
+    initialized_ = true;
+  }
+
+  // network::fprop (tiny_dnn/network.h:184-204): a forward pass of the given samples; the batch
+  // stays on the device as the one bprop works on
+  vec_t fprop(const vec_t &in) { return fprop(std::vector<vec_t>{in})[0]; }
+  std::vector<vec_t> fprop(const std::vector<vec_t> &in) {
+    if (in.empty()) return {};
+    build(std::max(in.size(), max_batch_ ? max_batch_ : 1));
+    if (!initialized_) init_weight();
+    const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
+    for (const vec_t &v : in)
+      if (v.size() != in_len) throw nn_error("input dimension mismatch");
+    last_batch_ = in.size();
+    detail::check(tdh_net_forward(net_, static_cast<int>(in.size()), x_.upload(in, in.size(), in_len)));
+    std::vector<float> flat(in.size() * out_len);
+    detail::check(tdh_memcpy_d2h(flat.data(), tdh_net_layer_out(net_, static_cast<int>(layers_.size()) - 1),
+                                 flat.size() * sizeof(float)));
+    std::vector<vec_t> out(in.size());
+    for (size_t s = 0; s < in.size(); ++s) out[s].assign(flat.begin() + s * out_len, flat.begin() + (s + 1) * out_len);
+    return out;
+  }
+  std::vector<tensor_t> fprop(const std::vector<tensor_t> &in) {  // one channel, as calc_delta asserts
+    std::vector<vec_t> flat_in;
+    for (const tensor_t &t : in) flat_in.push_back(t.at(0));
+    const std::vector<vec_t> y = fprop(flat_in);
+    std::vector<tensor_t> out(y.size());
+    for (size_t s = 0; s < y.size(); ++s) out[s] = tensor_t{y[s]};
+    return out;
+  }
+
+  // network::bprop (tiny_dnn/network.h:169-182): the loss gradient for targets t and the
+  // backward pass through every layer, on the batch of the last fprop; weight and bias
+  // gradients are ADDED to what is there (cleared by update_weights / clear_grads). `out` is
+  // what fprop returned: the device still holds it, so it is not sent back.
+  template <typename E>
+  void bprop(const std::vector<vec_t> &out, const std::vector<vec_t> &t) {
+    if (!net_ || !last_batch_ || out.size() != last_batch_ || t.size() != last_batch_)
+      throw nn_error("bprop: call fprop on the same batch first");
+    const size_t out_len = tdh_net_out_size(net_);
+    detail::check(tdh_net_train_step(net_, nullptr, E::kind, static_cast<int>(last_batch_), x_.get(),
+                                     t_.upload(t, t.size(), out_len), /*do_update=*/0));
+  }
+  template <typename E>
+  void bprop(const std::vector<tensor_t> &out, const std::vector<tensor_t> &t, const std::vector<tensor_t> &) {
+    std::vector<vec_t> o, tt;
+    for (const tensor_t &v : out) o.push_back(v.at(0));
+    for (const tensor_t &v : t) tt.push_back(v.at(0));
+    bprop<E>(o, tt);
+  }
+
+  // network::update_weights (tiny_dnn/network.h:209-213): every layer's update_weight, then
+  // the gradients are clear
+  template <typename Optimizer>
+  void update_weights(Optimizer *opt) {
+    build(max_batch_ ? max_batch_ : 1);
+    tdh_opt o = opt->descriptor();
+    detail::check(tdh_net_update_weights(net_, &o));
+    opt->absorb(o);
+  }
+  void clear_grads() {
+    if (net_) detail::check(tdh_net_clear_grads(net_));
+  }
+  // batch-reduced gradient of layer `index` (which = 0 weight, 1 bias) since the last update
+  vec_t weights_grads(size_t index, int which) {
+    build(max_batch_ ? max_batch_ : 1);
+    vec_t v(tdh_net_param_size(net_, static_cast<int>(index), which));
+    if (!v.empty())
+      detail::check(tdh_memcpy_d2h(v.data(), tdh_net_layer_grad(net_, static_cast<int>(index), which),
+                                   v.size() * sizeof(float)));
+    return v;
+  }
+
+  // network::train_once / train_onebatch (tiny_dnn/network.h:887-926): fprop, bprop and
+  // update_weights of `size` samples as one mini-batch
+  template <typename E, typename Optimizer>
+  void train_once(Optimizer &opt, const vec_t *in, const vec_t *t, size_t size) {
+    build(std::max(size, max_batch_ ? max_batch_ : 1));
+    if (!initialized_) init_weight();
+    const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
+    const std::vector<vec_t> xs(in, in + size), ts(t, t + size);
+    tdh_opt o = opt.descriptor();
+    last_batch_ = size;
+    detail::check(tdh_net_train_step(net_, &o, E::kind, static_cast<int>(size), x_.upload(xs, size, in_len),
+                                     t_.upload(ts, size, out_len), 1));
+    opt.absorb(o);
+  }
+
+  // network::get_loss (tiny_dnn/network.h:486-497): sum of E::f over the samples
+  template <typename E>
+  float_t get_loss(const std::vector<vec_t> &in, const std::vector<vec_t> &t) {
+    float_t sum_loss = float_t(0);
+    const std::vector<vec_t> y = fprop(in);
+    for (size_t i = 0; i < in.size(); ++i) sum_loss += E::f(y[i], t[i]);
+    return sum_loss;
+  }
+
+  // network::gradient_check (tiny_dnn/network.h:541-590, calc_delta :939-989): for every
+  // trainable vector, the loss's central difference in single weights (step sqrt(float
+  // epsilon)) against the gradient the backward pass gives, all (GRAD_CHECK_ALL) or ten random
+  // entries of each vector (GRAD_CHECK_RANDOM, drawn like the reference's uniform_idx).
+  // Samples are one-channel tensors, labels become targets through label2vec.
+  template <typename E>
+  bool gradient_check(const std::vector<tensor_t> &in, const std::vector<std::vector<label_t>> &t,
+                      float_t eps, grad_check_mode mode) {
+    if (in.size() != t.size() || in.empty()) throw nn_error("gradient_check: bad sample set");
+    std::vector<vec_t> x, v;
+    build(std::max(in.size(), max_batch_ ? max_batch_ : 1));
+    if (!initialized_) init_weight();
+    const size_t out_len = tdh_net_out_size(net_);
+    for (size_t s = 0; s < in.size(); ++s) {
+      x.push_back(in[s].at(0));
+      const std::pair<float_t, float_t> range = layers_.back()->out_value_range();
+      vec_t target(out_len, range.first);
+      if (t[s].at(0) >= out_len) throw nn_error("label out of range");
+      target[t[s][0]] = range.second;
+      v.push_back(target);
+    }
+    for (size_t i = 0; i < layers_.size(); ++i) {
+      for (int which = 0; which < 2; ++which) {
+        const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which);
+        if (!n) continue;
+        if (mode == GRAD_CHECK_ALL) {
+          for (size_t j = 0; j < n; ++j)
+            if (!calc_delta<E>(x, v, i, which, j, eps)) return false;
+        } else if (mode == GRAD_CHECK_RANDOM) {
+          for (size_t k = 0; k < 10; ++k) {
+            std::uniform_int_distribution<int> dst(0, static_cast<int>(n) - 1);
+            if (!calc_delta<E>(x, v, i, which, static_cast<size_t>(dst(random_generator::get_instance()())), eps))
+              return false;
+          }
+        } else {
+          throw nn_error("unknown grad-check type");
+        }
+      }
+    }
+    return true;
+  }
+  // the two figures of the last calc_delta (for reports)
+  float_t last_numeric_gradient() const { return last_numeric_; }
+  float_t last_bprop_gradient() const { return last_bprop_; }
+
   // network::predict (tiny_dnn/network.h:226-230)
   vec_t predict(const vec_t &in) {
     build(max_batch_ ? max_batch_ : 1);
@@ -1397,6 +1981,31 @@ class network<sequential> {
   }
 
  private:
+  template <typename E>
+  bool calc_delta(const std::vector<vec_t> &x, const std::vector<vec_t> &v, size_t layer_index, int which,
+                  size_t check_index, double eps) {
+    static const float_t delta = std::sqrt(std::numeric_limits<float_t>::epsilon());
+    clear_grads();
+    vec_t w = weights(layer_index, which);
+    const float_t prev_w = w[check_index];
+    w[check_index] = prev_w + delta;
+    set_weights(layer_index, which, w);
+    float_t f_p = float_t(0);
+    for (size_t i = 0; i < x.size(); ++i) f_p += get_loss<E>({x[i]}, {v[i]});
+    w[check_index] = prev_w - delta;
+    set_weights(layer_index, which, w);
+    float_t f_m = float_t(0);
+    for (size_t i = 0; i < x.size(); ++i) f_m += get_loss<E>({x[i]}, {v[i]});
+    const float_t delta_by_numerical = (f_p - f_m) / (float_t(2) * delta);
+    w[check_index] = prev_w;
+    set_weights(layer_index, which, w);
+    bprop<E>(fprop(x), v);
+    const float_t delta_by_bprop = weights_grads(layer_index, which)[check_index];
+    clear_grads();
+    last_numeric_ = delta_by_numerical;
+    last_bprop_   = delta_by_bprop;
+    return std::abs(delta_by_bprop - delta_by_numerical) <= eps;
+  }
   // entries of trainable vector `which` of layer i in a weight file
   size_t file_length(size_t i, int which) {
     const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which);
@@ -1443,6 +2052,8 @@ class network<sequential> {
   tdh_net *net_     = nullptr;
   size_t max_batch_ = 0;
   bool initialized_ = false;
+  size_t last_batch_ = 0;                // samples of the last fprop / train_once, held in x_
+  float_t last_numeric_ = 0, last_bprop_ = 0;
   detail::device_tensor x_, t_;
 };
 
