@@ -55,7 +55,8 @@ enum { TDH_LOSS_MSE = 0, TDH_LOSS_CE_MULTICLASS = 1, TDH_LOSS_CE = 2 };
 enum { TDH_OPT_SGD = 0, TDH_OPT_MOMENTUM = 1, TDH_OPT_ADAM = 2, TDH_OPT_ADAGRAD = 3,
        TDH_OPT_RMSPROP = 4, TDH_OPT_ADAMAX = 5, TDH_OPT_NESTEROV = 6 };
 /* layer kinds of a sequential network */
-enum { TDH_L_CONV = 0, TDH_L_FC = 1, TDH_L_MAXPOOL = 2, TDH_L_AVEPOOL = 3, TDH_L_ACT = 4 };
+enum { TDH_L_CONV = 0, TDH_L_FC = 1, TDH_L_MAXPOOL = 2, TDH_L_AVEPOOL = 3, TDH_L_ACT = 4,
+       TDH_L_BATCHNORM = 5, TDH_L_DROPOUT = 6 };
 
 /* core::conv_params (tiny_dnn/core/params/conv_params.h:63-90) */
 typedef struct tdh_conv_desc {
@@ -94,6 +95,13 @@ typedef struct tdh_layer {
   tdh_pool_desc pool;
   int32_t fc_in, fc_out, fc_bias;
   float act_p[2]; /* TDH_L_ACT: constructor parameters of the kinds that have them (see tdh_act_fwd_p) */
+  /* TDH_L_BATCHNORM: batch_normalization_layer(in_spatial_size, in_channels, epsilon, momentum)
+   * (tiny_dnn/layers/batch_normalization_layer.h:54-72); tensors are [batch][channels][spatial] */
+  int32_t bn_channels, bn_spatial;
+  float bn_eps, bn_momentum;
+  /* TDH_L_DROPOUT: dropout_layer(in_dim, dropout_rate) (tiny_dnn/layers/dropout_layer.h:32-39);
+   * in_dim is the size of the layer in front */
+  float dropout_rate;
 } tdh_layer;
 
 /* ------------------------------------------------------------ library state */
@@ -264,13 +272,25 @@ int tdh_net_destroy(tdh_net *net);
 size_t tdh_net_in_size(const tdh_net *net);
 size_t tdh_net_out_size(const tdh_net *net);
 size_t tdh_net_layer_out_size(const tdh_net *net, int layer);
-/* which: 0 = weight, 1 = bias; sizes in floats */
+/* which: 0 = weight, 1 = bias; of a batch-norm layer (which has neither) 2 = moving mean,
+ * 3 = moving variance (batch_normalization_layer.h:171-202, one value per channel, not touched
+ * by the optimizer); sizes in floats */
 size_t tdh_net_param_size(const tdh_net *net, int layer, int which);
 int tdh_net_set_param(tdh_net *net, int layer, int which, const float *host_src);
 int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst);
 /* optimizer::reset() as network::fit calls it before training (tiny_dnn/network.h:856,
  * tiny_dnn/optimizers/optimizer.h:36-38): clears the per-weight state vectors */
 int tdh_net_reset_optimizer(tdh_net *net);
+/* network::set_netphase (tiny_dnn/network.h:438-442): train != 0 is net_phase::train, the
+ * state of a new net. In the train phase a batch-norm layer normalises by the moments of the
+ * batch and every update moves its running averages (post_update), a dropout layer applies
+ * its mask; in the test phase batch-norm uses the running averages and dropout is the identity. */
+int tdh_net_set_phase(tdh_net *net, int train);
+/* The mask that the following passes of dropout layer `layer` apply: host bytes [batch][len] of
+ * 0/1, drawn by the caller as the reference draws them (bernoulli(dropout_rate) per element,
+ * sample after sample, tiny_dnn/layers/dropout_layer.h:99-102), once per train step. The copy
+ * is queued on the library stream, behind the kernels of the step before. */
+int tdh_net_set_dropout_mask(tdh_net *net, int layer, int batch, const uint8_t *host_mask);
 /* nodes::update_weights (tiny_dnn/nodes.h:103-107): layer::update_weight of every layer, front
  * to back, weight before bias, on the gradients accumulated since the last update, which are
  * then cleared (tiny_dnn/layers/layer.h:663-682). What tdh_net_train_step does with

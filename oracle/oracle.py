@@ -29,7 +29,7 @@ def act_params(kind, params=None):
     return (C.c_float * 2)(*p)
 LOSS = {"mse": 0, "ce_multiclass": 1, "ce": 2}
 OPT = {"sgd": 0, "momentum": 1, "adam": 2, "adagrad": 3, "rmsprop": 4, "adamax": 5, "nesterov": 6}
-L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT = range(5)
+L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT, L_BATCHNORM, L_DROPOUT = range(7)
 
 f32p = C.POINTER(C.c_float)
 i64p = C.POINTER(C.c_int64)
@@ -54,7 +54,8 @@ class OptDesc(C.Structure):
 class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("act", C.c_int32), ("conv", ConvDesc), ("pool", PoolDesc),
                 ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32),
-                ("act_p", C.c_float * 2)]
+                ("act_p", C.c_float * 2), ("bn_channels", C.c_int32), ("bn_spatial", C.c_int32),
+                ("bn_eps", C.c_float), ("bn_momentum", C.c_float), ("dropout_rate", C.c_float)]
 
 
 def conv_desc(in_w, in_h, in_c, k_w, k_h, out_c, pad_same=False, has_bias=True, w_stride=1,
@@ -302,6 +303,12 @@ def batchnorm_update_moving(momentum, mean_cur, var_cur, mean, variance):
     return mean, variance
 
 
+def mt_seed(state, seed):
+    """Seeds a 625-word generator state (np.uint32) like set_random_seed(seed)."""
+    oracle_lib().tdo_mt_seed(state.ctypes.data_as(C.POINTER(C.c_uint32)), C.c_uint32(seed))
+    return state
+
+
 def dropout_mask(seed, rate, batch, length, state=None):
     """The mask dropout_layer draws after set_random_seed(seed) (one worker thread)."""
     lib = oracle_lib()
@@ -397,6 +404,20 @@ def L_avepool(in_w, in_h, in_c, pool, stride=None):
     return l
 
 
+def L_batchnorm(channels, spatial, eps=1e-5, momentum=0.999):
+    """batch_normalization_layer(in_spatial_size, in_channels, epsilon, momentum)"""
+    l = LayerDesc()
+    l.kind, l.bn_channels, l.bn_spatial, l.bn_eps, l.bn_momentum = L_BATCHNORM, channels, spatial, eps, momentum
+    return l
+
+
+def L_dropout(rate):
+    """dropout_layer(in_dim, dropout_rate); the shape is the previous layer's"""
+    l = LayerDesc()
+    l.kind, l.dropout_rate = L_DROPOUT, rate
+    return l
+
+
 def L_act(kind, params=None):
     l = LayerDesc()
     l.kind, l.act = L_ACT, ACT[kind]
@@ -476,6 +497,22 @@ class OracleNet:
         p = self.lib.tdo_net_layer_argmax(self.h, i)
         return np.ctypeslib.as_array(p, shape=(n * batch,)).reshape(batch, n).copy()
 
+    def set_phase(self, train):
+        self.lib.tdo_net_set_phase(self.h, int(bool(train)))
+
+    def set_dropout_mask(self, i, mask):
+        """mask: uint8 [batch][len] that the next passes of dropout layer i apply"""
+        mask = np.ascontiguousarray(mask, np.uint8)
+        self.lib.tdo_net_dropout_mask.restype = C.POINTER(C.c_uint8)
+        dst = np.ctypeslib.as_array(self.lib.tdo_net_dropout_mask(self.h, i), shape=(mask.size,))
+        dst[:] = mask.ravel()
+
+    def bn_stat(self, i, which):
+        """moving mean (0) / variance (1) of batch-norm layer i (a view)"""
+        self.lib.tdo_net_bn_stat.restype = f32p
+        return np.ctypeslib.as_array(self.lib.tdo_net_bn_stat(self.h, i, which),
+                                     shape=(self.layers[i].bn_channels,))
+
     def forward(self, x):
         x, xp = _f(x)
         _chk(self.lib.tdo_net_forward(self.h, x.shape[0], xp), "net_forward")
@@ -527,6 +564,15 @@ class RefNet:
 
     def load_weights(self, path):
         _chk(self.lib.tdr_net_load_weights(self.h, str(path).encode()), "load_weights")
+
+    def set_random_seed(self, seed):
+        """set_random_seed of the reference: its dropout layers draw from this generator"""
+        self.lib.tdr_set_random_seed(C.c_uint(seed))
+
+    def bn_stat(self, layer, which, channels):
+        a = np.empty(channels, np.float32)
+        _chk(self.lib.tdr_net_get_bn_stat(self.h, layer, which, a.ctypes.data_as(f32p), channels), "bn_stat")
+        return a
 
     def fit(self, opt, loss, x, t, steps=1):
         x, xp = _f(x); t, tp = _f(t)

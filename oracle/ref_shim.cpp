@@ -56,6 +56,9 @@ struct layer_desc {
   pool_desc pool;
   int32_t fc_in, fc_out, fc_bias;
   float act_p[2];
+  int32_t bn_channels, bn_spatial;
+  float bn_eps, bn_momentum;
+  float dropout_rate;
 };
 
 core::backend_t engine_of(int engine) {
@@ -468,6 +471,13 @@ tdr_net *tdr_net_create(const layer_desc *layers, int n_layers, int engine) {
             default: return nullptr;
           }
           break;
+        case 5:
+          h->net << batch_normalization_layer(s.bn_spatial, s.bn_channels, s.bn_eps, s.bn_momentum);
+          break;
+        case 6:
+          if (i == 0) return nullptr;
+          h->net << dropout_layer(h->net[i - 1]->out_data_size(), s.dropout_rate);
+          break;
         default: return nullptr;
       }
     }
@@ -497,6 +507,24 @@ int tdr_net_get_param(tdr_net *h, int layer, int which, float *dst) {
   return 0;
 }
 
+/* set_random_seed (util/random.h:58-60): dropout layers draw their masks from this generator */
+void tdr_set_random_seed(unsigned seed) { set_random_seed(seed); }
+
+/* moving mean (which = 0) / variance (1) of batch-norm layer `layer`, read back through the
+ * layer's own save() (batch_normalization_layer.h:179-189; printed with 8 significant digits) */
+int tdr_net_get_bn_stat(tdr_net *h, int layer, int which, float *dst, int channels) {
+  try {
+    std::stringstream ss;
+    h->net[layer]->save(ss);
+    std::vector<float> v;
+    float f;
+    while (ss >> f) v.push_back(f);
+    if (v.size() != size_t(2 * channels)) return -2;
+    std::copy(v.begin() + which * channels, v.begin() + (which + 1) * channels, dst);
+    return 0;
+  } catch (const std::exception &) { return -1; }
+}
+
 /* `steps` mini-batch steps on the same batch (fit over `steps` epochs of one batch) with one
  * optimizer object; returns seconds per step (negative on error). loss: 0 mse,
  * 1 cross_entropy_multiclass, 2 cross_entropy. */
@@ -509,6 +537,15 @@ double tdr_net_fit(tdr_net *h, const opt_desc *o, int loss, int batch, const flo
       T[s].assign(t + out_len * s, t + out_len * (s + 1));
     }
     auto nop = []() {};
+    /* the samples of a dropout layer share one generator: any thread count but one races */
+    bool has_dropout = false;
+    for (const layer_desc &s : h->spec) has_dropout = has_dropout || s.kind == 6;
+    struct OneThread {
+      int saved;
+      bool on;
+      explicit OneThread(bool o) : saved(omp_get_max_threads()), on(o) { if (on) omp_set_num_threads(1); }
+      ~OneThread() { if (on) omp_set_num_threads(saved); }
+    } one_thread(has_dropout);
     auto t0  = std::chrono::steady_clock::now();
     bool ok  = false;
 #define TDR_FIT(OPT)                                                                   \

@@ -1022,12 +1022,16 @@ typedef struct {
   float *dout; /* gradient wrt out */
   float *dx;   /* gradient wrt in */
   int64_t *argmax;
+  /* batch-norm: moving mean / variance, this batch's moments, stddev; dropout: mask */
+  float *bn_mean, *bn_var, *bn_mean_cur, *bn_var_cur, *bn_stddev;
+  unsigned char *mask;
 } net_layer;
 
 struct tdo_net {
   int n_layers, max_batch;
   net_layer *l;
   float *x; /* copy of the current input batch */
+  int test_phase; /* 0: net_phase::train */
 };
 
 static int layer_sizes(net_layer *L) {
@@ -1053,6 +1057,11 @@ static int layer_sizes(net_layer *L) {
       L->b_size   = L->w_size;
       break;
     case TDO_L_ACT: /* size inherited from the previous layer, filled by the caller */
+    case TDO_L_DROPOUT:
+      L->w_size = L->b_size = 0;
+      break;
+    case TDO_L_BATCHNORM:
+      L->in_size = L->out_size = (size_t)s->bn_channels * s->bn_spatial;
       L->w_size = L->b_size = 0;
       break;
     default: return -2;
@@ -1071,7 +1080,7 @@ tdo_net *tdo_net_create(const tdo_layer *layers, int n_layers, int max_batch) {
   for (int i = 0; i < n_layers; i++) {
     net_layer *L = &net->l[i];
     L->spec      = layers[i];
-    if (layers[i].kind == TDO_L_ACT) {
+    if (layers[i].kind == TDO_L_ACT || layers[i].kind == TDO_L_DROPOUT) {
       if (i == 0) {
         tdo_net_destroy(net);
         return NULL;
@@ -1091,6 +1100,13 @@ tdo_net *tdo_net_create(const tdo_layer *layers, int n_layers, int max_batch) {
     L->dx   = fzalloc(L->in_size * (size_t)max_batch);
     if (layers[i].kind == TDO_L_MAXPOOL)
       L->argmax = (int64_t *)calloc(L->out_size * (size_t)max_batch, sizeof(int64_t));
+    if (layers[i].kind == TDO_L_BATCHNORM) {
+      const size_t c = (size_t)layers[i].bn_channels;
+      L->bn_mean = fzalloc(c); L->bn_var = fzalloc(c); L->bn_mean_cur = fzalloc(c);
+      L->bn_var_cur = fzalloc(c); L->bn_stddev = fzalloc(c);
+    }
+    if (layers[i].kind == TDO_L_DROPOUT)
+      L->mask = (unsigned char *)calloc(L->out_size * (size_t)max_batch + 1, 1);
   }
   net->x = fzalloc(net->l[0].in_size * (size_t)max_batch);
   return net;
@@ -1103,12 +1119,17 @@ void tdo_net_destroy(tdo_net *net) {
     free(L->w); free(L->b); free(L->dw); free(L->db);
     free(L->s0w); free(L->s1w); free(L->s0b); free(L->s1b);
     free(L->out); free(L->dout); free(L->dx); free(L->argmax);
+    free(L->bn_mean); free(L->bn_var); free(L->bn_mean_cur); free(L->bn_var_cur); free(L->bn_stddev);
+    free(L->mask);
   }
   free(net->l);
   free(net->x);
   free(net);
 }
 
+void tdo_net_set_phase(tdo_net *net, int train) { net->test_phase = !train; }
+unsigned char *tdo_net_dropout_mask(tdo_net *net, int i) { return net->l[i].mask; }
+float *tdo_net_bn_stat(tdo_net *net, int i, int which) { return which ? net->l[i].bn_var : net->l[i].bn_mean; }
 int tdo_net_num_layers(const tdo_net *net) { return net->n_layers; }
 size_t tdo_net_in_size(const tdo_net *net) { return net->l[0].in_size; }
 size_t tdo_net_out_size(const tdo_net *net) { return net->l[net->n_layers - 1].out_size; }
@@ -1140,6 +1161,16 @@ int tdo_net_forward(tdo_net *net, int batch, const float *x) {
       case TDO_L_AVEPOOL: rc = tdo_avepool_fwd(&L->spec.pool, batch, in, L->w, L->b, L->out); break;
       case TDO_L_ACT:
         rc = tdo_act_fwd_p(L->spec.act, L->spec.act_p, batch, (int)L->out_size, in, L->out);
+        break;
+      case TDO_L_BATCHNORM: { /* batch_normalization_layer.h:127-169 */
+        const int train = !net->test_phase;
+        rc = tdo_batchnorm_fwd(L->spec.bn_channels, L->spec.bn_spatial, batch, L->spec.bn_eps, train, in,
+                               train ? L->bn_mean_cur : L->bn_mean, train ? L->bn_var_cur : L->bn_var,
+                               L->bn_stddev, L->out);
+      } break;
+      case TDO_L_DROPOUT: /* dropout_layer.h:84-117 */
+        rc = tdo_dropout_fwd(batch, (int)L->out_size, !net->test_phase,
+                             1.0f / (1.0f - L->spec.dropout_rate), L->mask, in, L->out);
         break;
     }
     if (rc) return rc;
@@ -1178,6 +1209,13 @@ int tdo_net_train_step(tdo_net *net, tdo_opt *opt, int loss_kind, int batch, con
         rc = tdo_act_bwd_p(L->spec.act, L->spec.act_p, batch, (int)L->out_size, in, L->out, L->dout,
                            L->dx);
         break;
+      case TDO_L_BATCHNORM: /* batch_normalization_layer.h:87-125 */
+        rc = tdo_batchnorm_bwd(L->spec.bn_channels, L->spec.bn_spatial, batch, L->out, L->dout, L->bn_stddev,
+                               L->dx);
+        break;
+      case TDO_L_DROPOUT: /* dropout_layer.h:62-82 */
+        rc = tdo_dropout_bwd(batch, (int)L->out_size, L->mask, L->dout, L->dx);
+        break;
     }
     if (rc) return rc;
     if (i > 0) memcpy(net->l[i - 1].dout, L->dx, sizeof(float) * L->in_size * (size_t)batch);
@@ -1193,6 +1231,10 @@ int tdo_net_train_step(tdo_net *net, tdo_opt *opt, int loss_kind, int batch, con
       rc = tdo_update_weight(opt, L->b_size, 1, L->db, L->b, L->s0b, L->s1b);
       if (rc) return rc;
     }
+    /* layer::update_weight ends in post_update (layer.h:681): batch_normalization_layer.h:171-177 */
+    if (L->spec.kind == TDO_L_BATCHNORM)
+      tdo_batchnorm_update_moving(L->spec.bn_channels, L->spec.bn_momentum, L->bn_mean_cur, L->bn_var_cur,
+                                  L->bn_mean, L->bn_var);
   }
   return 0;
 }

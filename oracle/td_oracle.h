@@ -138,7 +138,8 @@ int tdo_update_weight(tdo_opt *o, size_t n, int weight_edge_samples, const float
                       float *w, float *s0, float *s1);
 
 /* ---- sequential network (one train step = fprop, loss grad, bprop, update) ---- */
-enum { TDO_L_CONV = 0, TDO_L_FC = 1, TDO_L_MAXPOOL = 2, TDO_L_AVEPOOL = 3, TDO_L_ACT = 4 };
+enum { TDO_L_CONV = 0, TDO_L_FC = 1, TDO_L_MAXPOOL = 2, TDO_L_AVEPOOL = 3, TDO_L_ACT = 4,
+       TDO_L_BATCHNORM = 5, TDO_L_DROPOUT = 6 };
 
 typedef struct tdo_layer {
   int32_t kind;
@@ -147,11 +148,21 @@ typedef struct tdo_layer {
   tdo_pool_desc pool;
   int32_t fc_in, fc_out, fc_bias;
   float act_p[2]; /* TDO_L_ACT: parameters of the kinds that have them */
+  int32_t bn_channels, bn_spatial; /* TDO_L_BATCHNORM: [batch][channels][spatial] */
+  float bn_eps, bn_momentum;
+  float dropout_rate;              /* TDO_L_DROPOUT (shape inherited from the layer in front) */
 } tdo_layer;
 
 typedef struct tdo_net tdo_net;
 
 tdo_net *tdo_net_create(const tdo_layer *layers, int n_layers, int max_batch);
+/* network::set_netphase (tiny_dnn/network.h:438-442): train != 0 is net_phase::train (the
+ * state of a new net, and what fit sets); batch-norm and dropout layers behave by it */
+void tdo_net_set_phase(tdo_net *net, int train);
+/* the mask [max_batch][len] the next forward pass of dropout layer i applies (the caller draws
+ * it, tdo_dropout_mask); which = 0 / 1: moving mean / variance of batch-norm layer i */
+unsigned char *tdo_net_dropout_mask(tdo_net *net, int i);
+float *tdo_net_bn_stat(tdo_net *net, int i, int which);
 void tdo_net_destroy(tdo_net *net);
 int tdo_net_num_layers(const tdo_net *net);
 size_t tdo_net_in_size(const tdo_net *net);

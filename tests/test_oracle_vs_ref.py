@@ -172,3 +172,31 @@ def test_example_nets_fit_bit_exact(ref, W, name, batch, steps):
         got = net.weight(i) if which == 0 else net.bias(i)
         assert not np.array_equal(got, a) or which == 1
         assert np.array_equal(got, rn.get_param(i, which)[:a.size]), (i, which)
+
+
+def test_net_with_batchnorm_and_dropout_fit_bit_exact(ref, W):
+    """conv -> batch-norm -> relu -> pool -> fc -> tanh -> dropout -> fc -> softmax: three Adam
+    steps of network<sequential>::fit after set_random_seed (the dropout masks are drawn from
+    the reference's generator in forward order) against the oracle's net, which is handed the
+    masks drawn by the restated generator; weights and the batch-norm running averages."""
+    O = ref
+    params, x, t = W.bn_dropout_case()
+    batch, steps, seed = x.shape[0], 3, 5
+    net = O.OracleNet(W.build_layers(O, W.BN_DROPOUT_NET), batch)
+    rn = O.RefNet(W.build_layers(O, W.BN_DROPOUT_NET), "scalar", 0)
+    for (i, which, a) in params:
+        (net.weight(i) if which == 0 else net.bias(i))[:] = a
+        rn.set_param(i, which, a)
+    o, o2 = O.opt_desc("adam"), O.opt_desc("adam")
+    state = np.zeros(625, np.uint32)
+    O.mt_seed(state, seed)
+    for _ in range(steps):
+        net.set_dropout_mask(6, O.dropout_mask(seed, 0.4, batch, 20, state))
+        net.train_step(o, "ce_multiclass", x, t)
+    rn.set_random_seed(seed)
+    rn.fit(o2, "ce_multiclass", x, t, steps)
+    for (i, which, a) in params:
+        got = net.weight(i) if which == 0 else net.bias(i)
+        assert np.array_equal(got, rn.get_param(i, which)[:a.size]), (i, which)
+    for which in (0, 1):   # read back through the reference's text format: 8 significant digits
+        np.testing.assert_allclose(net.bn_stat(1, which), rn.bn_stat(1, which, 6), rtol=2e-7, atol=1e-9)

@@ -24,7 +24,7 @@ ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3, "leaky_relu": 4, "elu":
        "softplus": 7, "softsign": 8, "asinh": 9, "tanh_p1m2": 10}
 LOSS = {"mse": 0, "ce_multiclass": 1, "ce": 2}
 OPT = {"sgd": 0, "momentum": 1, "adam": 2, "adagrad": 3, "rmsprop": 4, "adamax": 5, "nesterov": 6}
-L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT = range(5)
+L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT, L_BATCHNORM, L_DROPOUT = range(7)
 NET_FUSE_ACT_GRAD, NET_GRAPH = 1, 2
 
 f32p = C.POINTER(C.c_float)
@@ -54,7 +54,8 @@ class OptDesc(C.Structure):
 class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("act", C.c_int32), ("conv", ConvDesc), ("pool", PoolDesc),
                 ("fc_in", C.c_int32), ("fc_out", C.c_int32), ("fc_bias", C.c_int32),
-                ("act_p", C.c_float * 2)]
+                ("act_p", C.c_float * 2), ("bn_channels", C.c_int32), ("bn_spatial", C.c_int32),
+                ("bn_eps", C.c_float), ("bn_momentum", C.c_float), ("dropout_rate", C.c_float)]
 
 
 def build(verbose=False):
@@ -471,6 +472,20 @@ def L_avepool(in_w, in_h, in_c, pool, stride=None):
     return l
 
 
+def L_batchnorm(channels, spatial, eps=1e-5, momentum=0.999):
+    """batch_normalization_layer(in_spatial_size, in_channels, epsilon, momentum)"""
+    l = LayerDesc()
+    l.kind, l.bn_channels, l.bn_spatial, l.bn_eps, l.bn_momentum = L_BATCHNORM, channels, spatial, eps, momentum
+    return l
+
+
+def L_dropout(rate):
+    """dropout_layer(in_dim, dropout_rate); the shape is the previous layer's"""
+    l = LayerDesc()
+    l.kind, l.dropout_rate = L_DROPOUT, rate
+    return l
+
+
 def L_act(kind, params=None):
     l = LayerDesc()
     l.kind, l.act = L_ACT, ACT[kind]
@@ -549,6 +564,22 @@ class Net:
     def layer_argmax(self, i, batch):
         n = self.layer_out_size(i)
         return DevBuf.view(lib().tdh_net_layer_argmax(self.h, i), (batch, n), np.int32).numpy()
+
+    def set_phase(self, train):
+        """network::set_netphase: train (default) or test; batch-norm and dropout follow it"""
+        check(lib().tdh_net_set_phase(self.h, int(bool(train))), "tdh_net_set_phase")
+
+    def set_dropout_mask(self, i, mask):
+        """mask: uint8 [batch][len] drawn by the caller (dropout_mask) for dropout layer i"""
+        mask = np.ascontiguousarray(mask, np.uint8)
+        check(lib().tdh_net_set_dropout_mask(self.h, i, mask.shape[0], mask.ctypes.data_as(C.c_void_p)),
+              "tdh_net_set_dropout_mask")
+
+    def update_weights(self, opt):
+        check(lib().tdh_net_update_weights(self.h, C.byref(opt)), "tdh_net_update_weights")
+
+    def clear_grads(self):
+        check(lib().tdh_net_clear_grads(self.h), "tdh_net_clear_grads")
 
     def forward(self, batch, x):
         check(lib().tdh_net_forward(self.h, batch, _p(x)), "tdh_net_forward")

@@ -22,10 +22,15 @@ struct tdh_net {
     // filters in the LDS-halo kernels' layout for forward / dX, packed on a side stream at the
     // start of a captured step (stride-1 conv layers of a TDH_NET_GRAPH net)
     float *wp_fwd = nullptr, *wp_dx = nullptr;  // kept current by the optimizer kernel
+    // batch-norm: running averages, this batch's moments, sqrt(variance + eps); dropout: mask
+    float *bn_mean = nullptr, *bn_var = nullptr, *bn_mean_cur = nullptr, *bn_var_cur = nullptr,
+          *bn_stddev = nullptr;
+    uint8_t *mask = nullptr;  // [max_batch][out_size]
   };
   std::vector<Layer> layers;
   int max_batch  = 0;
   int flags      = 0;
+  bool test_phase = false;  // net_phase::test
   float *dx_in   = nullptr;  // gradient w.r.t. the network input
   tdh::OptTensor *opt_table = nullptr;  // device table of trainable tensors, update order
   bool packs_valid = false;  // wp_fwd / wp_dx of every layer match its weights
@@ -34,7 +39,7 @@ struct tdh_net {
   // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
   float *dev_powers = nullptr;          // {b1_t, b2_t, ticket} as the captured optimizer kernel uses them
   struct GraphKey {
-    int batch = 0, loss = 0, do_update = 0;
+    int batch = 0, loss = 0, do_update = 0, test_phase = 0;
     const float *x = nullptr, *t = nullptr;
     const void *scratch = nullptr;      // the library scratch buffer the captured kernels use
     tdh_opt hyper = {};                 // hyper-parameters only (powers zeroed)
@@ -89,7 +94,14 @@ int layer_sizes(tdh_net::Layer &L) {
       L.w_size   = s.kind == TDH_L_AVEPOOL ? s.pool.in_c : 0;
       L.b_size   = L.w_size;
     } break;
-    case TDH_L_ACT: L.w_size = L.b_size = 0; break;
+    case TDH_L_ACT:
+    case TDH_L_DROPOUT: L.w_size = L.b_size = 0; break;
+    case TDH_L_BATCHNORM:
+      if (s.bn_channels <= 0 || s.bn_spatial <= 0)
+        return set_error(TDH_ERR_INVALID, "batch-norm layer: %d channels x %d", s.bn_channels, s.bn_spatial);
+      L.in_size = L.out_size = static_cast<size_t>(s.bn_channels) * s.bn_spatial;
+      L.w_size = L.b_size = 0;
+      break;
     default: return set_error(TDH_ERR_INVALID, "unknown layer kind %d", s.kind);
   }
   return TDH_OK;
@@ -261,6 +273,17 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
         }
         break;
       case TDH_L_AVEPOOL: TDH_TRY(avepool_fwd(&s.pool, batch, in, L.w, L.b, L.out)); break;
+      case TDH_L_BATCHNORM: {  // batch_normalization_layer.h:127-169
+        const int train = !net->test_phase;
+        TDH_TRY(ws_begin(batchnorm_workspace_bytes(s.bn_channels, batch)));
+        TDH_TRY(batchnorm_fwd(s.bn_channels, s.bn_spatial, batch, s.bn_eps, train, in,
+                              train ? L.bn_mean_cur : L.bn_mean, train ? L.bn_var_cur : L.bn_var, L.bn_stddev,
+                              L.out));
+      } break;
+      case TDH_L_DROPOUT:      // dropout_layer.h:84-117
+        TDH_TRY(dropout_fwd(L.out_size * static_cast<size_t>(batch), !net->test_phase,
+                            1.0f / (1.0f - s.dropout_rate), L.mask, in, L.out));
+        break;
       case TDH_L_ACT:
         if (xent_t && tail_layer != n - 1 && i == n - 1 && s.act == TDH_ACT_SOFTMAX)
           TDH_TRY(launch_softmax_fwd_xent(batch, static_cast<int>(L.out_size), in, xent_t, L.out, xent_dz));
@@ -299,9 +322,13 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
                    L.spec.conv.tbl + static_cast<size_t>(L.spec.conv.in_c) * L.spec.conv.out_c);
       L.spec.conv.tbl = L.tbl.data();
     }
-    if (L.spec.kind == TDH_L_ACT) {
+    if (L.spec.kind == TDH_L_ACT || L.spec.kind == TDH_L_DROPOUT) {
       if (i == 0) {
-        rc = set_error(TDH_ERR_INVALID, "tdh_net_create: an activation cannot be the first layer");
+        rc = set_error(TDH_ERR_INVALID, "tdh_net_create: an activation or dropout layer cannot be the first layer");
+        break;
+      }
+      if (L.spec.kind == TDH_L_DROPOUT && !(L.spec.dropout_rate >= 0.0f && L.spec.dropout_rate < 1.0f)) {
+        rc = set_error(TDH_ERR_INVALID, "tdh_net_create: dropout rate %g", L.spec.dropout_rate);
         break;
       }
       L.in_size = L.out_size = net->layers[i - 1].out_size;
@@ -331,6 +358,19 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       if ((rc = net_alloc(net, act, &p, true))) break;
       L.argmax = reinterpret_cast<int32_t *>(p);
     }
+    if (L.spec.kind == TDH_L_BATCHNORM) {
+      const size_t c = static_cast<size_t>(L.spec.bn_channels);
+      if ((rc = net_alloc(net, c, &L.bn_mean, true))) break;
+      if ((rc = net_alloc(net, c, &L.bn_var, true))) break;
+      if ((rc = net_alloc(net, c, &L.bn_mean_cur, true))) break;
+      if ((rc = net_alloc(net, c, &L.bn_var_cur, true))) break;
+      if ((rc = net_alloc(net, c, &L.bn_stddev, true))) break;
+    }
+    if (L.spec.kind == TDH_L_DROPOUT) {
+      float *p = nullptr;
+      if ((rc = net_alloc(net, ceil_div_sz(act, sizeof(float)), &p, true))) break;
+      L.mask = reinterpret_cast<uint8_t *>(p);
+    }
     if ((flags & TDH_NET_GRAPH) && L.spec.kind == TDH_L_CONV && L.spec.conv.w_stride == 1 &&
         L.spec.conv.h_stride == 1) {
       if ((rc = net_alloc(net, L.w_size, &L.wp_fwd, false))) break;
@@ -346,6 +386,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
     if (L.spec.kind == TDH_L_CONV) need = conv2d_workspace_bytes(&L.spec.conv, max_batch);
     if (L.spec.kind == TDH_L_FC) need = fc_workspace_bytes(L.spec.fc_in, L.spec.fc_out, max_batch);
     if (L.spec.kind == TDH_L_AVEPOOL) need = avepool_workspace_bytes(&L.spec.pool, max_batch);
+    if (L.spec.kind == TDH_L_BATCHNORM) need = batchnorm_workspace_bytes(L.spec.bn_channels, max_batch);
     if (flags & TDH_NET_GRAPH)  // three times: dX, dW and db are separate calls of the operator there
       net->scratch += 3 * ws_align(need);
     else if (need > net->scratch)
@@ -449,11 +490,16 @@ size_t tdh_net_layer_out_size(const tdh_net *net, int layer) {
 }
 size_t tdh_net_param_size(const tdh_net *net, int layer, int which) {
   if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return 0;
-  return which == 0 ? net->layers[layer].w_size : (which == 1 ? net->layers[layer].b_size : 0);
+  const tdh_net::Layer &L = net->layers[layer];
+  if ((which == 2 || which == 3) && L.spec.kind == TDH_L_BATCHNORM) return static_cast<size_t>(L.spec.bn_channels);
+  return which == 0 ? L.w_size : (which == 1 ? L.b_size : 0);
 }
 static float *net_param_ptr(tdh_net *net, int layer, int which) {
   if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
-  return which == 0 ? net->layers[layer].w : (which == 1 ? net->layers[layer].b : nullptr);
+  tdh_net::Layer &L = net->layers[layer];
+  if (which == 2) return L.bn_mean;
+  if (which == 3) return L.bn_var;
+  return which == 0 ? L.w : (which == 1 ? L.b : nullptr);
 }
 float *tdh_net_param(tdh_net *net, int layer, int which) {
   if (net) net->packs_valid = false;  // the caller may write through the pointer
@@ -477,12 +523,37 @@ int tdh_net_reset_optimizer(tdh_net *net) {
   }
   return TDH_OK;
 }
+// layer::update_weight ends in post_update (layer.h:681): a batch-norm layer moves its running
+// averages towards the moments of the batch (batch_normalization_layer.h:171-177)
+static int post_update(tdh_net *net) {
+  for (tdh_net::Layer &L : net->layers)
+    if (L.spec.kind == TDH_L_BATCHNORM)
+      TDH_TRY(batchnorm_update_moving(L.spec.bn_channels, L.spec.bn_momentum, L.bn_mean_cur, L.bn_var_cur,
+                                      L.bn_mean, L.bn_var));
+  return TDH_OK;
+}
+
 int tdh_net_update_weights(tdh_net *net, tdh_opt *opt) {
   TDH_REQUIRE_INIT();
   TDH_CHECK_ARG(net && opt, "tdh_net_update_weights: null argument");
   // the optimizer kernel keeps the packed filter copies of a graph net current, as in a step
-  return launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
-                                 net->opt_params, 1.0f, 1, nullptr);
+  TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
+                                  net->opt_params, 1.0f, 1, nullptr));
+  return post_update(net);
+}
+int tdh_net_set_phase(tdh_net *net, int train) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net != nullptr, "tdh_net_set_phase: null net");
+  net->test_phase = !train;
+  return TDH_OK;
+}
+int tdh_net_set_dropout_mask(tdh_net *net, int layer, int batch, const uint8_t *host_mask) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && host_mask && layer >= 0 && layer < static_cast<int>(net->layers.size()) &&
+                  net->layers[layer].spec.kind == TDH_L_DROPOUT && batch > 0 && batch <= net->max_batch,
+                "tdh_net_set_dropout_mask: bad argument");
+  tdh_net::Layer &L = net->layers[layer];
+  return tdh_memcpy_h2d(L.mask, host_mask, L.out_size * static_cast<size_t>(batch));
 }
 int tdh_net_clear_grads(tdh_net *net) {
   TDH_REQUIRE_INIT();
@@ -716,6 +787,15 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         if (!L.grad_folded)
           TDH_TRY(launch_act_bwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out, L.dout, dx));
         break;
+      case TDH_L_BATCHNORM:  // batch_normalization_layer.h:87-125
+        TDH_TRY(ws_begin(batchnorm_workspace_bytes(s.bn_channels, batch)));
+        TDH_TRY(batchnorm_bwd(s.bn_channels, s.bn_spatial, batch, L.out, L.dout, L.bn_stddev, dx));
+        if (fold.kind != TDH_ACT_NONE) return set_error(TDH_ERR_INVALID, "batch-norm behind a folded activation");
+        break;
+      case TDH_L_DROPOUT:    // dropout_layer.h:62-82
+        TDH_TRY(dropout_bwd(L.out_size * static_cast<size_t>(batch), L.mask, L.dout, dx));
+        if (fold.kind != TDH_ACT_NONE) return set_error(TDH_ERR_INVALID, "dropout behind a folded activation");
+        break;
     }
   }
   TDH_TRY(finish_split_sum());  // (a max-pool has taken or finished it)
@@ -736,14 +816,16 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   // nodes::update_weights visits layers front to back, weight before bias; the gradient
   // reaches the optimizer unscaled (rcp_batch_size is 1, see tdh_opt_update) and is then
   // cleared (layer.h:680)
-  return launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
-                                 net->opt_params, 1.0f, 1, dev_powers);
+  TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
+                                  net->opt_params, 1.0f, 1, dev_powers));
+  return post_update(net);
 }
 
 static bool same_key(const tdh_net::GraphKey &a, const tdh_net::GraphKey &b) {
   // field by field: a caller's tdh_opt may carry padding or unused fields it never wrote
   const tdh_opt &p = a.hyper, &q = b.hyper;
-  return a.batch == b.batch && a.loss == b.loss && a.do_update == b.do_update && a.x == b.x &&
+  return a.batch == b.batch && a.loss == b.loss && a.do_update == b.do_update && a.test_phase == b.test_phase &&
+         a.x == b.x &&
          a.t == b.t && a.scratch == b.scratch && p.kind == q.kind && p.alpha == q.alpha &&
          p.lambda == q.lambda && p.mu == q.mu && p.b1 == q.b1 && p.b2 == q.b2 && p.eps == q.eps;
 }
@@ -771,6 +853,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
 
   tdh_net::GraphKey key;
   key.batch = batch; key.loss = loss_kind; key.do_update = do_update; key.x = x; key.t = t;
+  key.test_phase = net->test_phase;
   if (opt) {
     key.hyper      = *opt;
     key.hyper.b1_t = key.hyper.b2_t = 0.0f;

@@ -1403,10 +1403,11 @@ struct tanh_p1m2_layer : activation_layer { tanh_p1m2_layer() : activation_layer
 
 enum class net_phase { train, test };  // tiny_dnn/util/util.h:71
 
-// The two layers below run on the device through their own operators. The device-resident
-// train step of network<sequential> does not include them (describe() says so); they are used
-// the way the reference's tests use a single layer: forward_propagation / back_propagation on
-// host tensors.
+// The two layers below run on the device through their own operators when used the way the
+// reference's tests use a single layer (forward_propagation / back_propagation on host
+// tensors), and are layer kinds of the device-resident step of network<sequential>: there the
+// running averages of batch normalization live on the device (weights(i, 2) / weights(i, 3))
+// and fit draws every step's dropout masks on the host with the reference's generator.
 namespace detail {
 struct norm_buffers {
   device_tensor x, y, dy, dx, mean, var, stddev, mean_cur, var_cur;
@@ -1444,7 +1445,14 @@ class batch_normalization_layer : public layer {
 
   std::string layer_type() const override { return "batch-norm"; }
   layer_desc describe(const shape3d &) const override {
-    throw nn_error("batch_normalization_layer is not part of the device-resident train step");
+    layer_desc r;
+    std::memset(&r.l, 0, sizeof(r.l));
+    r.l.kind        = TDH_L_BATCHNORM;
+    r.l.bn_channels = static_cast<int32_t>(channels_);
+    r.l.bn_spatial  = static_cast<int32_t>(spatial_);
+    r.l.bn_eps      = eps_;
+    r.l.bn_momentum = momentum_;
+    return r;
   }
   std::vector<shape3d> in_shape() const { return {shape3d(spatial_, 1, channels_)}; }
   std::vector<shape3d> out_shape() const { return {shape3d(spatial_, 1, channels_)}; }
@@ -1545,7 +1553,11 @@ class dropout_layer : public layer {
 
   std::string layer_type() const override { return "dropout"; }
   layer_desc describe(const shape3d &) const override {
-    throw nn_error("dropout_layer is not part of the device-resident train step");
+    layer_desc r;
+    std::memset(&r.l, 0, sizeof(r.l));
+    r.l.kind         = TDH_L_DROPOUT;
+    r.l.dropout_rate = dropout_rate_;
+    return r;
   }
   std::vector<shape3d> in_shape() const { return {shape3d(in_size_, 1, 1)}; }
   std::vector<shape3d> out_shape() const { return {shape3d(in_size_, 1, 1)}; }
@@ -1717,6 +1729,7 @@ class network<sequential> {
     build(batch_size);
     if (reset_weights || !initialized_) init_weight();
     const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
+    set_netphase(net_phase::train);  // network.h:852
     opt.reset();  // network.h:856; the device copy of the state vectors is cleared with it
     detail::check(tdh_net_reset_optimizer(net_));
     tdh_opt o = opt.descriptor();
@@ -1736,12 +1749,21 @@ class network<sequential> {
       int n = 0;
       detail::check(tdh_feeder_acquire(feed.get(), &xd, &td, &n));
       if (k + 1 < total) stage(k + 1);  // the feeder's thread copies while this one launches
+      draw_dropout_masks(static_cast<size_t>(n));
       detail::check(tdh_net_train_step(net_, &o, Error::kind, n, xd, td, 1));
       on_batch_enumerate();
       if ((k + 1) % per_epoch == 0) on_epoch_enumerate();
     }
     opt.absorb(o);
+    set_netphase(net_phase::test);  // network.h:877
     return true;
+  }
+
+  // network::set_netphase (tiny_dnn/network.h:438-442)
+  void set_netphase(net_phase phase) {
+    build(max_batch_ ? max_batch_ : 1);
+    phase_ = phase;
+    detail::check(tdh_net_set_phase(net_, phase == net_phase::train));
   }
 
   // network::train (tiny_dnn/network.h:284-308): labels become one-hot targets whose off / on
@@ -1771,8 +1793,8 @@ class network<sequential> {
     build(max_batch_ ? max_batch_ : 1);
     os << std::setprecision(std::numeric_limits<float_t>::digits10 + 2);
     for (size_t i = 0; i < layers_.size(); ++i)
-      for (int which = 0; which < 2; ++which) {
-        const vec_t v = weights(i, which);
+      for (int which = 0; which < 4; ++which) {  // 2, 3: a batch-norm layer's running averages
+        const vec_t v = weights(i, which);       // (batch_normalization_layer.h:179-189)
         for (float_t w : v) os << w << " ";
         for (size_t k = v.size(); k < file_length(i, which); ++k) os << float_t(0) << " ";
       }
@@ -1780,7 +1802,7 @@ class network<sequential> {
   void load(std::istream &is) {
     build(max_batch_ ? max_batch_ : 1);
     for (size_t i = 0; i < layers_.size(); ++i)
-      for (int which = 0; which < 2; ++which) {
+      for (int which = 0; which < 4; ++which) {
         vec_t v(tdh_net_param_size(net_, static_cast<int>(i), which));
         for (float_t &w : v) is >> w;
         float_t skipped;
@@ -1801,7 +1823,7 @@ class network<sequential> {
     build(max_batch_ ? max_batch_ : 1);
     size_t idx = 0;
     for (size_t i = 0; i < layers_.size(); ++i)
-      for (int which = 0; which < 2; ++which) {
+      for (int which = 0; which < 4; ++which) {
         const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which), len = file_length(i, which);
         if (idx + len > data.size()) throw nn_error("fast_load: the file holds fewer weights than the network");
         if (n) set_weights(i, which, vec_t(data.begin() + idx, data.begin() + idx + n));
@@ -1909,6 +1931,7 @@ class network<sequential> {
     const std::vector<vec_t> xs(in, in + size), ts(t, t + size);
     tdh_opt o = opt.descriptor();
     last_batch_ = size;
+    draw_dropout_masks(size);
     detail::check(tdh_net_train_step(net_, &o, E::kind, static_cast<int>(size), x_.upload(xs, size, in_len),
                                      t_.upload(ts, size, out_len), 1));
     opt.absorb(o);
@@ -1981,6 +2004,20 @@ class network<sequential> {
   }
 
  private:
+  // dropout_layer::forward_propagation in the train phase (dropout_layer.h:99-102): every
+  // element of every sample of every dropout layer, front to back, draws its own
+  // bernoulli(rate) from the process-wide generator; the masks are handed to the device net
+  void draw_dropout_masks(size_t n) {
+    if (phase_ != net_phase::train) return;
+    for (size_t i = 0; i < layers_.size(); ++i) {
+      const dropout_layer *d = dynamic_cast<const dropout_layer *>(layers_[i].get());
+      if (!d) continue;
+      const size_t len = tdh_net_layer_out_size(net_, static_cast<int>(i));
+      mask_.resize(n * len);
+      for (size_t e = 0; e < n * len; ++e) mask_[e] = bernoulli(d->dropout_rate());
+      detail::check(tdh_net_set_dropout_mask(net_, static_cast<int>(i), static_cast<int>(n), mask_.data()));
+    }
+  }
   template <typename E>
   bool calc_delta(const std::vector<vec_t> &x, const std::vector<vec_t> &v, size_t layer_index, int which,
                   size_t check_index, double eps) {
@@ -2036,7 +2073,7 @@ class network<sequential> {
                                  TDH_NET_FUSE_ACT_GRAD | TDH_NET_GRAPH, &fresh));
     if (net_) {
       for (size_t i = 0; i < layers_.size(); ++i)
-        for (int which = 0; which < 2; ++which) {
+        for (int which = 0; which < 4; ++which) {
           vec_t v(tdh_net_param_size(net_, static_cast<int>(i), which));
           if (v.empty()) continue;
           detail::check(tdh_net_get_param(net_, static_cast<int>(i), which, v.data()));
@@ -2044,6 +2081,7 @@ class network<sequential> {
         }
       tdh_net_destroy(net_);
     }
+    detail::check(tdh_net_set_phase(fresh, phase_ == net_phase::train));
     net_       = fresh;
     max_batch_ = batch;
   }
@@ -2052,6 +2090,8 @@ class network<sequential> {
   tdh_net *net_     = nullptr;
   size_t max_batch_ = 0;
   bool initialized_ = false;
+  net_phase phase_ = net_phase::train;   // a new net is in the train phase (layer constructors' default)
+  std::vector<uint8_t> mask_;
   size_t last_batch_ = 0;                // samples of the last fprop / train_once, held in x_
   float_t last_numeric_ = 0, last_bprop_ = 0;
   detail::device_tensor x_, t_;

@@ -107,7 +107,7 @@ def _file_length(layer, which, n):
 def save_weights(net, path):
     vectors = []
     for i in range(net.n):
-        for which in (0, 1):
+        for which in (0, 1, 2, 3):   # 2, 3: the running averages a batch-norm layer writes
             n = net.param_size(i, which)
             if not n:
                 continue
@@ -122,7 +122,7 @@ def load_weights(net, path):
         data = text_to_floats(f.read())
     at = 0
     for i in range(net.n):
-        for which in (0, 1):
+        for which in (0, 1, 2, 3):   # 2, 3: the running averages a batch-norm layer writes
             n = net.param_size(i, which)
             if not n:
                 continue

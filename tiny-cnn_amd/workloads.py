@@ -85,6 +85,10 @@ def build_layers(api, spec):
             out.append(api.L_avepool(l[1], l[2], l[3], l[4]))
         elif kind == "act":
             out.append(api.L_act(l[1], l[2] if len(l) > 2 else None))
+        elif kind == "batchnorm":   # (channels, spatial[, eps, momentum])
+            out.append(api.L_batchnorm(*l[1:]))
+        elif kind == "dropout":     # (rate,)
+            out.append(api.L_dropout(l[1]))
         else:
             raise ValueError(kind)
     return out
@@ -198,3 +202,24 @@ def flops_per_sample(spec):
         elif l[0] == "fc":
             total += 2 * l[1] * l[2]
     return total
+
+
+# not a benchmark configuration: a small net with the two layers whose backward pass needs more
+# than the layer's own output gradient, for parity tests of the device-resident step
+BN_DROPOUT_NET = [("conv", 10, 10, 2, 3, 6, True), ("batchnorm", 6, 100), ("act", "relu"),
+                  ("maxpool", 10, 10, 6, 2), ("fc", 150, 20), ("act", "tanh"), ("dropout", 0.4),
+                  ("fc", 20, 10), ("act", "softmax")]
+
+
+def bn_dropout_case(batch=7, seed=21):
+    """Seeded (params, x, one-hot t) for BN_DROPOUT_NET."""
+    rng = np.random.default_rng(seed)
+    params = []
+    for i, l in enumerate(BN_DROPOUT_NET):
+        nw, nb, fan_in, _ = layer_fans(l)
+        if nw:
+            params += [(i, 0, rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(math.sqrt(3.0 / fan_in))),
+                       (i, 1, rng.uniform(-.2, .2, nb).astype(np.float32))]
+    x = rng.standard_normal((batch, 200)).astype(np.float32)
+    t = np.eye(10, dtype=np.float32)[rng.integers(0, 10, batch)]
+    return params, x, t
