@@ -505,6 +505,82 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
         net.close()
 
 
+@pytest.mark.parametrize("spec,batch", [
+    # the benchmarked net's classifier: eight 128-deep slices, a pool in front, ragged batch
+    ([("conv", 16, 16, 3, 5, 16, True), ("maxpool", 16, 16, 16, 2), ("act", "relu"), ("fc", 1024, 64),
+      ("act", "relu"), ("fc", 64, 10), ("act", "softmax")], 37),
+    # the pool in front reads an activation: its own kernel routes the gradient
+    ([("conv", 16, 16, 3, 5, 16, True), ("act", "relu"), ("maxpool", 16, 16, 16, 2), ("fc", 1024, 64),
+      ("act", "relu"), ("fc", 64, 10), ("act", "softmax")], 37),
+    # the first layer of the net (its dX is the input gradient); 300 inputs: a short last slice;
+    # 40 hidden units
+    ([("fc", 300, 40), ("act", "tanh"), ("fc", 40, 10), ("act", "softmax")], 16),
+    # mse on the second layer, both at the 64-unit limit
+    ([("fc", 200, 64), ("act", "sigmoid"), ("fc", 64, 64)], 5),
+    # an activation in front whose gradient the dX epilogue applies; 132 inputs: one full slice and
+    # four more; 130 inputs: not a multiple of four, the separate launches
+    ([("fc", 50, 132), ("act", "tanh"), ("fc", 132, 24), ("act", "relu"), ("fc", 24, 3), ("act", "softmax")], 20),
+    ([("fc", 50, 130), ("act", "tanh"), ("fc", 130, 24), ("act", "relu"), ("fc", 24, 3), ("act", "softmax")], 20),
+    # pool and a folded activation in front
+    ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("act", "sigmoid"), ("fc", 64, 12), ("act", "relu"),
+      ("fc", 12, 10), ("act", "softmax")], 19),
+    # 36 hidden units are fine, 35 are not (rows of the first layer's filters are read four at a time)
+    ([("fc", 260, 36), ("act", "relu"), ("fc", 36, 10), ("act", "softmax")], 33),
+    ([("fc", 260, 35), ("act", "relu"), ("fc", 35, 10), ("act", "softmax")], 33),
+])
+@pytest.mark.parametrize("flags", [1, 3])
+def test_two_closing_fc_layers_in_one_launch_match_oracle(T, O, W, spec, batch, flags):
+    """A fusing net whose classifier is fc -> pointwise activation -> fc [-> softmax] runs both
+    layers' forward passes, the loss gradient and the second layer's input gradient as one kernel
+    (the first layer's product split over workgroups, the last to finish carries on), and the
+    second layer's weight and bias gradients beside the first layer's in its backward launch.
+    Three SGD steps: every layer output, every gradient and every updated weight against the
+    oracle, and the outputs against the same net without fusion. Replayed steps (flags 3) also
+    show that the kernel leaves its tickets ready for the next launch."""
+    rng = np.random.default_rng(len(spec) * 29 + batch)
+    net, plain = T.Net(W.build_layers(T, spec), batch, flags), T.Net(W.build_layers(T, spec), batch, 0)
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for i, l in enumerate(spec):
+        nw, nb, fan_in, _ = W.layer_fans(l)
+        if nw:
+            w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+            b = rng.uniform(-0.5, 0.5, nb).astype(np.float32)
+            for n in (net, plain):
+                n.set_param(i, 0, w); n.set_param(i, 1, b)
+            ref.weight(i)[:] = w; ref.bias(i)[:] = b
+    softmax = spec[-1] == ("act", "softmax")
+    loss = "ce_multiclass" if softmax else "mse"
+    first, classes = spec[0], spec[-2 if softmax else -1][2]
+    n_in = first[1] if first[0] == "fc" else first[1] * first[2] * first[3]
+    x = rng.standard_normal((batch, n_in)).astype(np.float32)
+    t = np.eye(classes, dtype=np.float32)[rng.integers(0, classes, batch)]
+    xd, td = T.to_device(x), T.to_device(t)
+    opt, ropt = T.opt_desc("sgd"), O.opt_desc("sgd")
+    # gradients first (an update clears them), then three steps with updates
+    ref.train_step(ropt, loss, x, t, do_update=False)
+    for n in (net, plain):
+        n.train_step(None, loss, batch, xd, td, do_update=False)
+    for i, l in enumerate(spec):
+        assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+        assert_close(net.layer_out(i, batch), plain.layer_out(i, batch), REL_TOL, f"layer {i} output, fused vs not")
+        if l[0] == "maxpool" and spec[i - 1][0] == "conv":
+            assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), REL_TOL, f"layer {i} dX (through the pool)")
+        if net.param_size(i, 0):
+            assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
+            assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")
+    assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, "input gradient")
+    net.train_step(T.opt_desc("sgd", alpha=0.0), loss, batch, xd, td)   # clears the gradients
+    for step in range(3):
+        net.train_step(opt, loss, batch, xd, td)
+        ref.train_step(ropt, loss, x, t)
+        for i, l in enumerate(spec):
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"step {step} layer {i} output")
+            if net.param_size(i, 0):
+                assert_close(net.get_param(i, 0), ref.weight(i), REL_TOL, f"step {step} layer {i} weights")
+                assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} layer {i} bias")
+    net.close(); plain.close()
+
+
 def test_layers_without_bias_through_the_one_launch_kernels(T, O):
     """No layer has a bias: the last layer's one-launch kernel, the fully-connected backward that
     routes dX through the pool in front, and the convolution kernels against the oracle."""

@@ -282,9 +282,26 @@ struct PoolScatter {
 };
 // (pool.hip) the layer is such a pool; fills the geometry
 bool maxpool_scatters_from_fc(const tdh_pool_desc *d, PoolScatter *geom);
+// the weight and bias gradients (db null: no bias) of another small fully-connected layer of
+// the same batch that fc_bwd's one-launch kernel computes beside its own (both layers within
+// fc_bwd_fuses)
+struct FcGrads {
+  int in, out;
+  const float *x, *dy;
+  float *dw, *db;
+};
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
-           const PoolScatter *pool = nullptr);
+           const PoolScatter *pool = nullptr, const FcGrads *also = nullptr);
+// (fc.hip) the closing classifier, two fully-connected layers deep, in one launch up to the
+// gradient of the first layer's output
+bool fc_two_layer_tail_applies(int in, int hidden, int out, int batch);
+int fc_two_layer_tail(int in, int hidden, int out, int has_bias1, int has_bias2, int batch, const float *x,
+                      const float *w1, const float *b1, float *y1, float *a1, int act_kind, const float *w2,
+                      const float *b2, float *y2, float *soft, const float *t, float *dz, float *dh,
+                      float *partials, unsigned int *tickets);
+size_t fc_two_layer_tail_partials(int in, int batch);
+size_t fc_two_layer_tail_tickets(int batch);
 // the one-launch backward kernel of this layer can also scatter dX through a max-pool
 bool fc_bwd_scatters_pool(int in, int out, int batch);
 // conv_s1.hip: stride-1 forward / dX with LDS halo tiles (3x3 and 5x5 windows)

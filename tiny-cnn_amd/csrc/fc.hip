@@ -6,6 +6,7 @@
 // dW is reduced over the batch inside the GEMM (K spans the samples) instead of being stored
 // per sample and merged afterwards (fully_connected_op_internal.h:54-60, node.h:89-103).
 #include <cfloat>
+#include <type_traits>
 
 #include "gemm_mfma.h"
 
@@ -176,33 +177,59 @@ struct FcBwdFused {
   int wM, wN, wK, w_tiles_n, nw;
   const float *dy;
   float *db;
-  int batch, out, db_accumulate;
+  int batch, out, db_accumulate, ndb;
+  // the weight and bias gradients of another small layer of the same batch, whose workgroups
+  // follow (n2 == 0: none)
+  StridedOperand w2a, w2b;
+  EpiRowMajor w2epi;
+  int w2M, w2N, w2K, w2_tiles_n, nw2;
+  const float *dy2;
+  float *db2;
+  int out2;
 };
+
+// 32 columns (block cb) of the column sums of dy[batch][out]
+__device__ __forceinline__ void fc_bias_grad_block(const float *dy, float *db, int batch, int out, int accumulate,
+                                                   int cb, SfcSmem &sm) {
+  float(*part)[32] = reinterpret_cast<float(*)[32]>(&sm.Bs[0][0]);
+  const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
+  const int c  = cb * 32 + cl;
+  float s = 0.0f;
+  if (c < out)
+    for (int r = g; r < batch; r += 8) s += dy[static_cast<size_t>(r) * out + c];
+  part[g][cl] = s;
+  __syncthreads();
+  if (g == 0 && c < out) {
+    float t = part[0][cl];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) t += part[i][cl];
+    db[c] = accumulate ? db[c] + t : t;
+  }
+}
 
 __global__ void __launch_bounds__(SFC_NT) fc_bwd_fused_kernel(const FcBwdFused f) {
   __shared__ SfcSmem sm;
-  const int b = blockIdx.x;
+  int b = blockIdx.x;
   if (b < f.nx) {
     small_fc_tile(f.xa, f.xb, f.xepi, f.xM, f.xN, f.xK, b % f.x_tiles_n, b / f.x_tiles_n, sm);
-  } else if (b < f.nx + f.nw) {
-    const int t = b - f.nx;
-    small_fc_tile(f.wa, f.wb, f.wepi, f.wM, f.wN, f.wK, t % f.w_tiles_n, t / f.w_tiles_n, sm);
-  } else {
-    float(*part)[32] = reinterpret_cast<float(*)[32]>(&sm.Bs[0][0]);
-    const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
-    const int c  = (b - f.nx - f.nw) * 32 + cl;
-    float s = 0.0f;
-    if (c < f.out)
-      for (int r = g; r < f.batch; r += 8) s += f.dy[static_cast<size_t>(r) * f.out + c];
-    part[g][cl] = s;
-    __syncthreads();
-    if (g == 0 && c < f.out) {
-      float t = part[0][cl];
-#pragma unroll
-      for (int i = 1; i < 8; ++i) t += part[i][cl];
-      f.db[c] = f.db_accumulate ? f.db[c] + t : t;
-    }
+    return;
   }
+  b -= f.nx;
+  if (b < f.nw) {
+    small_fc_tile(f.wa, f.wb, f.wepi, f.wM, f.wN, f.wK, b % f.w_tiles_n, b / f.w_tiles_n, sm);
+    return;
+  }
+  b -= f.nw;
+  if (b < f.ndb) {
+    fc_bias_grad_block(f.dy, f.db, f.batch, f.out, f.db_accumulate, b, sm);
+    return;
+  }
+  b -= f.ndb;
+  if (b < f.nw2) {
+    small_fc_tile(f.w2a, f.w2b, f.w2epi, f.w2M, f.w2N, f.w2K, b % f.w2_tiles_n, b / f.w2_tiles_n, sm);
+    return;
+  }
+  fc_bias_grad_block(f.dy2, f.db2, f.batch, f.out2, f.db_accumulate, b - f.nw2, sm);
 }
 
 // The last fully-connected layer of a net that ends in softmax and is trained with
@@ -321,6 +348,309 @@ __global__ void __launch_bounds__(SFC_NT) fc_softmax_xent_kernel(const FcTail f)
   }
 }
 
+// The closing classifier of a net, two fully-connected layers deep, in one launch:
+//
+//   fc A (K1 -> H) -> pointwise activation -> fc B (H -> O) [-> softmax] -> loss gradient
+//     -> dX of fc B with the activation's gradient applied (= the gradient of fc A's output)
+//
+// Everything on that way stays inside a sample row. As separate kernels the chain is three
+// launches of 4-10 us each with well under a microsecond of arithmetic in each: what they take is
+// launch gaps, start-up, trips to memory one after the other, and instruction fetch: these
+// kernels run once a step on a few compute units whose instruction caches hold other kernels'
+// code by then, and cold straight-line code was measured to run at about a microsecond a
+// kilobyte. So the kernel is written for few instructions and few taken branches: guards are
+// clamped addresses and selects, per-kind arithmetic is folded into coefficients.
+// (The gradients that add over the batch, and dX of fc A with its 2 K1 H flop a row, stay
+// launches of their own: dX in this kernel had a 16-row block's share run on one compute
+// unit, 11 us, as long as fc_bwd's launch that also computes dW and db beside it.)
+//
+// All products run on v_mfma_f32_16x16x4_f32 with both operands read in the fragment layout
+// straight from memory (or from a 16-row tile in LDS), four consecutive floats a lane:
+// lane (r = lane % 16, q = lane / 16) holds, of a 16-deep slice of the reduction, the four
+// indices 4 q .. 4 q + 3, and the instruction that consumes component `comp` adds the terms
+// k = 4 q + comp over q. Where the operand's four floats run along the output columns instead
+// (fc A's filters, [k][h]), component cc feeds a product of its own, whose 16 column slots stand
+// for columns 4 r + cc.
+//
+// Workgroup (split s, row block b), eight waves: wave w multiplies 16 rows by the 16-deep
+// slice 128 s + 16 w of fc A, the eight partial tiles are added through LDS, stored, and the
+// workgroup draws a ticket of row block b. The workgroup that draws the last one goes on alone,
+// the others are done (nobody waits for anybody): it adds the splits in order, applies bias and
+// activation, multiplies by fc B, applies softmax and loss gradient as fc_softmax_xent_kernel
+// does, and takes the gradient back through fc B and the activation.
+struct FcTail2 {
+  const float *x, *w1, *bias1;      // X[s][k], W_A[k][h]
+  const float *w2, *bias2;          // W_B[h][o]
+  float *out1, *act1;               // fc A's output and the activation layer's
+  int act1_kind;
+  float *out2, *soft;               // fc B's output and the softmax layer's (null: the loss is mse)
+  const float *t;
+  float *dz;                        // loss gradient with respect to fc B's output
+  float *dh;                        // gradient with respect to fc A's output (activation gradient applied)
+  float mse_factor;
+  float *partials;                  // [row block][split][16][64]
+  unsigned int *tickets;            // [row block], zero between launches
+  int M, K1, H, O, splits;
+};
+
+typedef float tail_f4 __attribute__((ext_vector_type(4)));
+constexpr int TL_NT = 512, TL_WAVES = TL_NT / 64, TL_TM = 16, TL_KC = 16 * TL_WAVES, TL_LD = 68;
+
+struct TailSmem {
+  __attribute__((aligned(16))) float part[TL_WAVES][TL_TM][TL_LD];  // fc A: a partial tile a wave
+  __attribute__((aligned(16))) float hs[TL_TM][TL_LD];              // act(fc A)
+  __attribute__((aligned(16))) float zs[TL_TM][TL_LD];              // fc B
+  __attribute__((aligned(16))) float dzs[TL_TM][TL_LD];             // loss gradient
+  __attribute__((aligned(16))) float w2[64][TL_LD];                 // fc B's filters, zeros past H x O
+};
+
+// These kernels run once a step on a few compute units with cold instruction caches: what they
+// cost is the instructions a wave executes and the branches it takes. Guards are therefore
+// clamped addresses and selects, not branches around loads.
+__device__ __forceinline__ float4 tail_ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 tail_keep(const float4 &v, bool ok) {
+  return make_float4(ok ? v.x : 0.0f, ok ? v.y : 0.0f, ok ? v.z : 0.0f, ok ? v.w : 0.0f);
+}
+// act_grad_factor for the pointwise activations (and none) as arithmetic on coefficients that
+// are computed once: a select on the kind, which is uniform, becomes a branch tree per value.
+// factor = yp * (yp * c2 + c1) + c0 + (y > 0 ? c3 : 0), yp = min(y, cap): the same operations and
+// roundings as 1 - y * y (tanh), y * (1 - y) (sigmoid), y > 0 ? 1 : 0 (relu, cap = 0 keeps the
+// polynomial at zero), 1 (none).
+struct TailGrad {
+  float c2, c1, c0, c3, cap;
+};
+__device__ __forceinline__ TailGrad tail_grad_coef(int kind) {
+  TailGrad g{0.0f, 0.0f, 1.0f, 0.0f, FLT_MAX};
+  if (kind == TDH_ACT_TANH) g = TailGrad{-1.0f, 0.0f, 1.0f, 0.0f, FLT_MAX};
+  if (kind == TDH_ACT_SIGMOID) g = TailGrad{-1.0f, 1.0f, 0.0f, 0.0f, FLT_MAX};
+  if (kind == TDH_ACT_RELU) g = TailGrad{0.0f, 0.0f, 0.0f, 1.0f, 0.0f};
+  return g;
+}
+__device__ __forceinline__ float tail_grad_factor(const TailGrad &g, float y) {
+  const float yp = fminf(y, g.cap);
+  return fmaf(yp, fmaf(yp, g.c2, g.c1), g.c0) + (y > 0.0f ? g.c3 : 0.0f);
+}
+// all-reduce over each group of 16 lanes on the data-parallel-primitive path (no LDS round trips):
+// neighbours, pairs, mirrored halves of 8, mirrored 16
+template <bool MAX, int CTRL>
+__device__ __forceinline__ float tail_dpp_step(float v) {
+  const float o = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, true));
+  return MAX ? fmaxf(v, o) : v + o;
+}
+template <bool MAX>
+__device__ __forceinline__ float tail_reduce16(float v) {
+  v = tail_dpp_step<MAX, 0xb1>(v);   // quad_perm [1, 0, 3, 2]
+  v = tail_dpp_step<MAX, 0x4e>(v);   // quad_perm [2, 3, 0, 1]
+  v = tail_dpp_step<MAX, 0x141>(v);  // row_half_mirror
+  v = tail_dpp_step<MAX, 0x140>(v);  // row_mirror
+  return v;
+}
+// ... and over the wave when the row is wider than 16 columns
+template <bool MAX>
+__device__ __forceinline__ float tail_reduce(float v, bool wide) {
+  v = tail_reduce16<MAX>(v);
+  if (wide) {
+    float o = __shfl_xor(v, 16, 64);
+    v = MAX ? fmaxf(v, o) : v + o;
+    o = __shfl_xor(v, 32, 64);
+    v = MAX ? fmaxf(v, o) : v + o;
+  }
+  return v;
+}
+
+__global__ void __launch_bounds__(TL_NT) fc_two_layer_tail_kernel(const FcTail2 f) {
+  __shared__ TailSmem sm;
+  __shared__ unsigned int drawn;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int sp = blockIdx.x, rb = blockIdx.y;
+  const int m0 = rb * TL_TM;
+  // ---- this wave's slice of fc A: rows m0 .. m0 + 15, k = kb .. kb + 3 a lane, all columns.
+  //      Rows past the batch and columns past H hold finite values nobody uses.
+  {
+    const int kb = sp * TL_KC + 16 * w + 4 * q;
+    const int mr = min(m0 + r, f.M - 1), kc = min(kb, f.K1 - 4), hc = 4 * r < f.H ? 4 * r : 0;
+    const float4 a = tail_keep(tail_ld4(f.x + static_cast<size_t>(mr) * f.K1 + kc), kb < f.K1);
+    const float *wrow = f.w1 + static_cast<size_t>(kc) * f.H + hc;
+    float4 b[4];
+#pragma unroll
+    for (int comp = 0; comp < 4; ++comp) b[comp] = tail_ld4(wrow + comp * f.H);
+    tail_f4 acc[4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    const float av[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int comp = 0; comp < 4; ++comp) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[comp], b[comp].x, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[comp], b[comp].y, acc[1], 0, 0, 0);
+      acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[comp], b[comp].z, acc[2], 0, 0, 0);
+      acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[comp], b[comp].w, acc[3], 0, 0, 0);
+    }
+    // acc[cc][i]: row 4 q + i, column 4 r + cc
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<float4 *>(&sm.part[w][4 * q + i][4 * r]) = make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
+  }
+  __syncthreads();
+  // every thread owns two consecutive columns of a row from here to the activation
+  const int orow = tid >> 5, ocol = 2 * (tid & 31);
+  float2 sum = make_float2(0.0f, 0.0f);
+#pragma unroll
+  for (int v = 0; v < TL_WAVES; ++v) {
+    const float2 p = *reinterpret_cast<const float2 *>(&sm.part[v][orow][ocol]);
+    sum.x += p.x; sum.y += p.y;
+  }
+  if (f.splits > 1) {
+    float2 *mine = reinterpret_cast<float2 *>(f.partials + (static_cast<size_t>(rb) * f.splits + sp) * (TL_TM * 64));
+    mine[tid] = sum;
+    // Every wave waits until its stores have reached the L2 cache (the vector L1 writes through);
+    // behind the barrier one thread draws the ticket. Its release writes this L2's dirty lines
+    // back for the whole workgroup, its acquire drops what this L2 and this compute unit's L1
+    // hold of other L2s' lines: one device-wide fence a workgroup, not one a wave.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) drawn = __hip_atomic_fetch_add(&f.tickets[rb], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (drawn != static_cast<unsigned int>(f.splits - 1)) return;
+    if (tid == 0) __hip_atomic_store(&f.tickets[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // ---- asked for now, used later: everything the rest reads from memory that does not depend
+  //      on what is computed here, so that the trips to memory overlap
+  float w2r[8];  // fc B's filters, on their way to LDS
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = tid + TL_NT * i, k = e >> 6, n = e & 63;
+    const bool ok = k < f.H && n < f.O;
+    const float v = f.w2[ok ? k * f.O + n : 0];
+    w2r[i]        = ok ? v : 0.0f;
+  }
+  float tv[2];  // targets: wave w owns rows 2 w, 2 w + 1 in the softmax, a column a lane
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m   = m0 + 2 * w + i;
+    const bool ok = lane < f.O && m < f.M;
+    const float v = f.t[ok ? m * f.O + lane : 0];
+    tv[i]         = ok ? v : 0.0f;
+  }
+  float bias2 = 0.0f;
+  if (f.bias2) bias2 = f.bias2[lane < f.O ? lane : 0];
+  // ---- the splits in order, bias, activation
+  {
+    const bool on = ocol < f.H && m0 + orow < f.M;
+    float2 bias = make_float2(0.0f, 0.0f);
+    if (f.bias1) bias = *reinterpret_cast<const float2 *>(f.bias1 + (ocol < f.H ? ocol : 0));
+    if (f.splits > 1) {
+      const float2 *all = reinterpret_cast<const float2 *>(f.partials + static_cast<size_t>(rb) * f.splits * (TL_TM * 64));
+      sum = make_float2(0.0f, 0.0f);
+#pragma unroll 8
+      for (int s = 0; s < f.splits; ++s) {
+        const float2 p = all[s * TL_NT + tid];
+        sum.x += p.x; sum.y += p.y;
+      }
+    }
+    const float2 v = make_float2(sum.x + bias.x, sum.y + bias.y);
+    float2 h;
+    switch (f.act1_kind) {  // act_apply, one branch for the two
+      case TDH_ACT_TANH: h = make_float2(tanhf(v.x), tanhf(v.y)); break;
+      case TDH_ACT_RELU: h = make_float2(v.x > 0.0f ? v.x : 0.0f, v.y > 0.0f ? v.y : 0.0f); break;
+      case TDH_ACT_SIGMOID: h = make_float2(1.0f / (1.0f + expf(-v.x)), 1.0f / (1.0f + expf(-v.y))); break;
+      default: h = v; break;
+    }
+    if (on) {
+      *reinterpret_cast<float2 *>(f.out1 + static_cast<size_t>(m0 + orow) * f.H + ocol) = v;
+      *reinterpret_cast<float2 *>(f.act1 + static_cast<size_t>(m0 + orow) * f.H + ocol) = h;
+    }
+    *reinterpret_cast<float2 *>(&sm.hs[orow][ocol]) = make_float2(on ? h.x : 0.0f, on ? h.y : 0.0f);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = tid + TL_NT * i;
+    sm.w2[e >> 6][e & 63] = w2r[i];
+  }
+  __syncthreads();
+  // ---- fc B: wave w the output columns 16 w .. 16 w + 15
+  const int nob = (f.O + 15) >> 4;
+  if (w < nob) {
+    tail_f4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const float4 a   = *reinterpret_cast<const float4 *>(&sm.hs[r][16 * kk + 4 * q]);
+      const float *wk  = &sm.w2[16 * kk + 4 * q][16 * w + r];
+      z = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, wk[0], z, 0, 0, 0);
+      z = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, wk[TL_LD], z, 0, 0, 0);
+      z = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, wk[2 * TL_LD], z, 0, 0, 0);
+      z = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, wk[3 * TL_LD], z, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sm.zs[4 * q + i][16 * w + r] = z[i];
+  }
+  __syncthreads();
+  // ---- softmax and the loss gradient (fc_softmax_xent_kernel's steps): a row a wave at a time
+  {
+    const bool col = lane < f.O, wide = f.O > 16;
+    float v[2], dzv[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) v[i] = col ? (sm.zs[2 * w + i][lane] + bias2) + 0.0f : 0.0f;
+    if (f.soft) {
+      float y[2], st[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const float mx = tail_reduce<true>(col ? fmaxf(-FLT_MAX, v[i]) : -FLT_MAX, wide);
+        const float e  = col ? expf(v[i] - mx) : 0.0f;
+        const float se = tail_reduce<false>(e, wide);
+        st[i]          = tail_reduce<false>(tv[i], wide);
+        y[i]           = e / se;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int m     = m0 + 2 * w + i;
+        const bool live = col && m < f.M;
+        dzv[i]          = live ? fmaf(y[i], st[i], -tv[i]) : 0.0f;
+        if (live) {
+          f.out2[m * f.O + lane] = v[i];
+          f.soft[m * f.O + lane] = y[i];
+          f.dz[m * f.O + lane]   = dzv[i];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int m     = m0 + 2 * w + i;
+        const bool live = col && m < f.M;
+        dzv[i]          = live ? f.mse_factor * (v[i] - tv[i]) : 0.0f;
+        if (live) {
+          f.out2[m * f.O + lane] = v[i];
+          f.dz[m * f.O + lane]   = dzv[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) sm.dzs[2 * w + i][lane] = dzv[i];
+  }
+  __syncthreads();
+  // ---- dX of fc B: dh[m][c] = (sum_o dz[m][o] * W_B[c][o]) * act'(h[m][c]); wave w the columns
+  //      16 w .. 16 w + 15 of fc A's output (zeros past H: the filters in LDS are zero there)
+  if (w < 4) {
+    const TailGrad g1 = tail_grad_coef(f.act1_kind);
+    tail_f4 g = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int kk = 0; kk < nob; ++kk) {
+      const float4 a = *reinterpret_cast<const float4 *>(&sm.dzs[r][16 * kk + 4 * q]);
+      const float4 b = *reinterpret_cast<const float4 *>(&sm.w2[16 * w + r][16 * kk + 4 * q]);
+      g = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, g, 0, 0, 0);
+      g = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, g, 0, 0, 0);
+      g = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, g, 0, 0, 0);
+      g = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, g, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * q + i, m = m0 + row, c = 16 * w + r;
+      const bool on = c < f.H && m < f.M;
+      float v       = g[i] + 0.0f;
+      v *= tail_grad_factor(g1, sm.hs[row][c]);
+      v = on ? v + 0.0f : 0.0f;
+      if (on) f.dh[m * f.H + c] = v;
+    }
+  }
+}
+
 bool small_fc_applies(int M, int N, int K) {
   return K <= 4 * SFC_KC && static_cast<long>(M) * N <= (1L << 18) &&
          static_cast<long>(M) * N * K <= (1L << 24);
@@ -369,6 +699,45 @@ int fc_softmax_xent(int in, int out, int has_bias, int batch, const float *x, co
   return TDH_OK;
 }
 
+// the two closing fully-connected layers (in -> hidden -> out, a pointwise activation between
+// them) can leave one launch with the loss gradient and both input gradients
+bool fc_two_layer_tail_applies(int in, int hidden, int out, int batch) {
+  return hidden <= 64 && hidden % 4 == 0 && out <= 64 && in >= 4 && in % 4 == 0 && in <= 64 * TL_KC && batch >= 1 &&
+         static_cast<long>(batch) * in < (1L << 24);
+}
+// floats of partial sums and number of tickets the launch needs (the caller owns both; the
+// tickets are zero before the first launch and the kernel leaves them zero)
+size_t fc_two_layer_tail_partials(int in, int batch) {
+  const int splits = ceil_div(in, TL_KC);
+  return splits > 1 ? static_cast<size_t>(ceil_div(batch, TL_TM)) * splits * TL_TM * 64 : 0;
+}
+size_t fc_two_layer_tail_tickets(int batch) { return static_cast<size_t>(ceil_div(batch, TL_TM)); }
+
+// soft == nullptr: the net ends in the second layer and the loss is mse.
+int fc_two_layer_tail(int in, int hidden, int out, int has_bias1, int has_bias2, int batch, const float *x,
+                      const float *w1, const float *b1, float *y1, float *a1, int act_kind, const float *w2,
+                      const float *b2, float *y2, float *soft, const float *t, float *dz, float *dh,
+                      float *partials, unsigned int *tickets) {
+  if (!fc_two_layer_tail_applies(in, hidden, out, batch))
+    return set_error(TDH_ERR_INVALID, "fc_two_layer_tail: layers too large for the one-launch kernel");
+  FcTail2 f;
+  f.x = x; f.w1 = w1; f.bias1 = has_bias1 ? b1 : nullptr;
+  f.w2 = w2; f.bias2 = has_bias2 ? b2 : nullptr;
+  f.out1 = y1; f.act1 = a1; f.act1_kind = act_kind;
+  f.out2 = y2; f.soft = soft; f.t = t; f.dz = dz; f.dh = dh;
+  f.mse_factor = 2.0f / static_cast<float>(out);
+  f.partials = partials; f.tickets = tickets;
+  f.M = batch; f.K1 = in; f.H = hidden; f.O = out;
+  f.splits = ceil_div(in, TL_KC);
+  if (f.splits > 1 && !(partials && tickets))
+    return set_error(TDH_ERR_INVALID, "fc_two_layer_tail: no room for the partial sums");
+  ProfScope prof("fc_two_layer_tail",
+                 2.0 * batch * (static_cast<double>(in) * hidden + 2.0 * hidden * out), WORK_FLOP);
+  TDH_LAUNCH(fc_two_layer_tail_kernel, dim3(f.splits, ceil_div(batch, TL_TM)), dim3(TL_NT), 0, ctx().stream, f);
+  TDH_LAUNCH_CHECK();
+  return TDH_OK;
+}
+
 size_t fc_workspace_bytes(int in, int out, int batch) {
   return gemm_workspace_bytes(batch, out, in, true) + gemm_workspace_bytes(batch, in, out, true) +
          gemm_workspace_bytes(in, out, batch, true);
@@ -392,8 +761,10 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
 
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
-           const PoolScatter *pool) {
+           const PoolScatter *pool, const FcGrads *also) {
   const bool bias_grad = db && has_bias;
+  if (also && !(dw && (dx || bias_grad) && fc_bwd_fuses(in, out, batch) && fc_bwd_fuses(also->in, also->out, batch)))
+    return set_error(TDH_ERR_INVALID, "fc_bwd: another layer's gradients need the one-launch kernel");
   if (pool && !(dx && dw && fc_bwd_fuses(in, out, batch) && pool->OH * pool->OW > 0 && in % (pool->OH * pool->OW) == 0))
     return set_error(TDH_ERR_INVALID, "fc_bwd: the pool scatter needs the one-launch kernel");
   if (dw && (dx || bias_grad) && fc_bwd_fuses(in, out, batch)) {
@@ -416,11 +787,25 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     f.wM = in; f.wN = out; f.wK = batch;
     f.w_tiles_n = ceil_div(out, SFC_TN);
     f.nw = f.w_tiles_n * ceil_div(in, SFC_TM);
-    const bool bias = bias_grad;
     f.dy = dy; f.db = db; f.batch = batch; f.out = out; f.db_accumulate = accumulate;
-    ProfScope prof(pool ? "fc_bwd_small_pool" : dx ? "fc_bwd_small" : "fc_dw_db_small", (dx ? 4.0 : 2.0) * batch * in * out, WORK_FLOP);
-    TDH_LAUNCH(fc_bwd_fused_kernel, dim3(f.nx + f.nw + (bias ? ceil_div(out, 32) : 0)),
-                       dim3(SFC_NT), 0, ctx().stream, f);
+    f.ndb = bias_grad ? ceil_div(out, 32) : 0;
+    f.nw2 = 0;
+    int ndb2 = 0;
+    double flop = (dx ? 4.0 : 2.0) * batch * in * out;
+    if (also) {
+      f.w2a = StridedOperand{also->x, 1, also->in, also->in};
+      f.w2b = StridedOperand{also->dy, 1, also->out, also->out};
+      f.w2epi = EpiRowMajor{also->dw, also->out, nullptr, ActGrad(), accumulate};
+      f.w2M = also->in; f.w2N = also->out; f.w2K = batch;
+      f.w2_tiles_n = ceil_div(also->out, SFC_TN);
+      f.nw2 = f.w2_tiles_n * ceil_div(also->in, SFC_TM);
+      f.dy2 = also->dy; f.db2 = also->db; f.out2 = also->out;
+      ndb2 = also->db ? ceil_div(also->out, 32) : 0;
+      flop += 2.0 * batch * also->in * also->out;
+    }
+    ProfScope prof(also ? (pool ? "fc_bwd_small_pool_two" : "fc_bwd_small_two")
+                        : pool ? "fc_bwd_small_pool" : dx ? "fc_bwd_small" : "fc_dw_db_small", flop, WORK_FLOP);
+    TDH_LAUNCH(fc_bwd_fused_kernel, dim3(f.nx + f.nw + f.ndb + f.nw2 + ndb2), dim3(SFC_NT), 0, ctx().stream, f);
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }

@@ -38,6 +38,8 @@ struct tdh_net {
   double opt_params = 0.0;
   // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
   float *dev_powers = nullptr;          // {b1_t, b2_t, ticket} as the captured optimizer kernel uses them
+  // partial sums and tickets of the one-launch kernel of two closing fully-connected layers
+  float *tail_partials = nullptr, *tail_tickets = nullptr;
   struct GraphKey {
     int batch = 0, loss = 0, do_update = 0, test_phase = 0;
     const float *x = nullptr, *t = nullptr;
@@ -171,30 +173,64 @@ DxTarget dx_target(tdh_net *net, int i) {
   return d;
 }
 
-// The layer that a train step runs together with the loss gradient and its own dX as one
-// launch, or -1: the fully-connected layer in front of the closing softmax under
-// cross_entropy_multiclass, or a closing fully-connected layer under mse.
-int tail_layer_in_one_launch(const tdh_net *net, int loss_kind, int batch) {
-  const int n = static_cast<int>(net->layers.size());
+// The 2x2 max-pool in front of layer i (behind a folded activation, nothing folded into the pool
+// itself) that the dX epilogue of layer i can route its gradient through: its index, or -1.
+int pool_in_front(tdh_net *net, int i, PoolScatter *through) {
   if (!(net->flags & TDH_NET_FUSE_ACT_GRAD)) return -1;
+  const int r = i - 1 - ((i >= 1 && net->layers[i - 1].grad_folded) ? 1 : 0);
+  if (r < 0 || net->layers[r].spec.kind != TDH_L_MAXPOOL ||
+      !maxpool_scatters_from_fc(&net->layers[r].spec.pool, through))
+    return -1;
+  const DxTarget behind = dx_target(net, r);
+  if (behind.fold.kind != TDH_ACT_NONE) return -1;
+  through->argmax = net->layers[r].argmax;
+  through->dx     = behind.dx;
+  return r;
+}
+
+// What a train step runs together with the loss gradient as one launch.
+// layer: the fully-connected layer in front of the closing softmax under
+// cross_entropy_multiclass, or a closing fully-connected layer under mse (forward, loss
+// gradient and its own dX), or -1.
+// first: the fully-connected layer two in front of it (a pointwise activation between them)
+// when the same launch also covers that one's forward pass and leaves the gradient of its
+// output, or -1.
+struct TailPlan {
+  int layer = -1, first = -1;
+  DxTarget target;  // where the dX of `layer` goes (first < 0)
+};
+TailPlan plan_tail(tdh_net *net, int loss_kind, int batch) {
+  TailPlan plan;
+  const int n = static_cast<int>(net->layers.size());
+  if (!(net->flags & TDH_NET_FUSE_ACT_GRAD)) return plan;
   int at = -1;
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && n >= 2 && net->layers[n - 1].spec.kind == TDH_L_ACT &&
       net->layers[n - 1].spec.act == TDH_ACT_SOFTMAX)
     at = n - 2;
   else if (loss_kind == TDH_LOSS_MSE)
     at = n - 1;
-  if (at < 0) return -1;
+  if (at < 0) return plan;
   const tdh_layer &fc = net->layers[at].spec;
-  return fc.kind == TDH_L_FC && fc_softmax_xent_applies(fc.fc_in, fc.fc_out, batch) ? at : -1;
+  if (!(fc.kind == TDH_L_FC && fc_softmax_xent_applies(fc.fc_in, fc.fc_out, batch))) return plan;
+  plan.layer  = at;
+  plan.target = dx_target(net, at);
+  if (at >= 2 && net->layers[at - 1].grad_folded && net->layers[at - 2].spec.kind == TDH_L_FC && net->tail_tickets) {
+    const tdh_layer &a = net->layers[at - 2].spec;
+    if (a.fc_out == fc.fc_in && fc_two_layer_tail_applies(a.fc_in, a.fc_out, fc.fc_out, batch)) {
+      plan.first = at - 2;
+    }
+  }
+  return plan;
 }
 
 // packed: the layers' wp_fwd hold the current filters in the stride-1 kernels' layout
 // xent_t / xent_dz: the net ends in softmax and the step's loss is cross_entropy_multiclass: the
 // last layer's kernel also writes the loss gradient with respect to the softmax input
-// tail (with tail_layer): that fully-connected layer runs as fc_softmax_xent, which also writes
-// the loss gradient (to xent_dz, from the targets xent_t) and the gradient of its input
+// tail: its layer runs as fc_softmax_xent, which also writes the loss gradient (to xent_dz, from
+// the targets xent_t) and the gradient of its input; with tail->first that layer, the activation
+// behind it and tail->layer run as fc_two_layer_tail
 int forward(tdh_net *net, int batch, const float *x, bool packed = false, const float *xent_t = nullptr,
-            float *xent_dz = nullptr, const DxTarget *tail = nullptr, int tail_layer = -1) {
+            float *xent_dz = nullptr, const TailPlan *tail = nullptr) {
   const float *in = x;
   const int n     = static_cast<int>(net->layers.size());
   for (int i = 0; i < n; ++i) {
@@ -244,11 +280,21 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
         break;
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
-        if (tail && i == tail_layer) {
+        if (tail && i == tail->first) {
+          tdh_net::Layer &B = net->layers[i + 2];
+          const bool softmax_behind = i + 2 == n - 2;
+          TDH_TRY(fc_two_layer_tail(s.fc_in, s.fc_out, B.spec.fc_out, s.fc_bias, B.spec.fc_bias, batch, in, L.w,
+                                    L.b, L.out, net->layers[i + 1].out, net->layers[i + 1].spec.act, B.w, B.b,
+                                    B.out, softmax_behind ? net->layers[n - 1].out : nullptr, xent_t, xent_dz,
+                                    L.dout, net->tail_partials,
+                                    reinterpret_cast<unsigned int *>(net->tail_tickets)));
+          i = n - 1;
+        } else
+        if (tail && i == tail->layer) {
           const bool softmax_behind = i == n - 2;
           TDH_TRY(fc_softmax_xent(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.b, L.out,
-                                  softmax_behind ? net->layers[n - 1].out : nullptr, xent_t, xent_dz, tail->dx,
-                                  tail->fold));
+                                  softmax_behind ? net->layers[n - 1].out : nullptr, xent_t, xent_dz,
+                                  tail->target.dx, tail->target.fold));
           if (softmax_behind) ++i;
         } else
         if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && i + 1 < n && net->layers[i + 1].spec.kind == TDH_L_ACT &&
@@ -285,7 +331,7 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
                             1.0f / (1.0f - s.dropout_rate), L.mask, in, L.out));
         break;
       case TDH_L_ACT:
-        if (xent_t && tail_layer != n - 1 && i == n - 1 && s.act == TDH_ACT_SOFTMAX)
+        if (xent_t && !(tail && tail->layer == n - 1) && i == n - 1 && s.act == TDH_ACT_SOFTMAX)
           TDH_TRY(launch_softmax_fwd_xent(batch, static_cast<int>(L.out_size), in, xent_t, L.out, xent_dz));
         else
           TDH_TRY(launch_act_fwd(s.act, s.act_p, batch, static_cast<int>(L.out_size), in, L.out));
@@ -444,6 +490,17 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
     }
   }
   if (rc == TDH_OK) rc = net_alloc(net, 4, &net->dev_powers, true);  // powers, ticket (zero)
+  if (rc == TDH_OK && (flags & TDH_NET_FUSE_ACT_GRAD)) {
+    // [fc, pointwise activation, fc] closes the net, or stands in front of a closing softmax
+    int b = n_layers - 1;
+    if (layers[b].kind == TDH_L_ACT && layers[b].act == TDH_ACT_SOFTMAX) --b;
+    if (b >= 2 && layers[b].kind == TDH_L_FC && layers[b - 2].kind == TDH_L_FC && net->layers[b - 1].grad_folded &&
+        fc_two_layer_tail_applies(layers[b - 2].fc_in, layers[b - 2].fc_out, layers[b].fc_out, max_batch)) {
+      rc = net_alloc(net, fc_two_layer_tail_tickets(max_batch), &net->tail_tickets, true);
+      if (rc == TDH_OK)
+        rc = net_alloc(net, fc_two_layer_tail_partials(layers[b - 2].fc_in, max_batch), &net->tail_partials, false);
+    }
+  }
   if (rc == TDH_OK && (flags & TDH_NET_GRAPH)) {
     Context &c = ctx();
     for (hipStream_t &s : c.side)
@@ -632,19 +689,19 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   int first_bwd        = n - 1;
   int tail_done        = -1;     // this layer already has the gradient of its input
   int pool_done        = -1;     // a max-pool layer whose backward pass the layer behind it did
+  FcGrads also         = {};     // the closing layer's weight and bias gradients, left to ...
+  int also_for         = -1;     // ... this layer's backward launch
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
   // the full softmax Jacobian, and that kernel is the softmax layer's forward kernel
-  tail_done = tail_layer_in_one_launch(net, loss_kind, batch);
+  const TailPlan plan = plan_tail(net, loss_kind, batch);
+  tail_done           = plan.layer;
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
       last.spec.act == TDH_ACT_SOFTMAX && n >= 2) {
-    const DxTarget tail = tail_done >= 0 ? dx_target(net, n - 2) : DxTarget();
-    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done >= 0 ? &tail : nullptr,
-                    tail_done));
+    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done >= 0 ? &plan : nullptr));
     first_bwd = n - 2;
   } else if (tail_done >= 0) {
     // mse on a closing fully-connected layer: its kernel writes the loss gradient too
-    const DxTarget tail = dx_target(net, n - 1);
-    TDH_TRY(forward(net, batch, x, packed, t, last.dout, &tail, tail_done));
+    TDH_TRY(forward(net, batch, x, packed, t, last.dout, &plan));
   } else {
     TDH_TRY(forward(net, batch, x, packed));
     TDH_TRY(launch_loss_grad(loss_kind, batch, static_cast<int>(last.out_size), last.out, t,
@@ -660,7 +717,15 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     const ActGrad fold    = target.fold;
     if (i == tail_done) {
       // only the weight and bias gradients are left, and nothing before the optimizer reads
-      // them: one launch, on the side stream when the step branches
+      // them: they leave with the backward launch of the fully-connected layer two in front
+      // when that is the one-launch kernel, else as one launch, on the side stream when the
+      // step branches
+      if (plan.first >= 0 && fc_bwd_fuses(s.fc_in, s.fc_out, batch) &&
+          fc_bwd_fuses(net->layers[plan.first].spec.fc_in, net->layers[plan.first].spec.fc_out, batch)) {
+        also = FcGrads{s.fc_in, s.fc_out, in, L.dout, L.dw, L.b_size ? L.db : nullptr};
+        also_for = plan.first;
+        continue;
+      }
       TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
       if (forked) {
         TDH_HIP(hipEventRecord(net->events[i], c.stream));
@@ -756,22 +821,11 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           // a 2x2 max-pool in front (behind a folded activation, nothing folded into the pool
           // itself): the one-launch kernel's dX epilogue also routes the gradient through it
           PoolScatter through;
-          int reader = -1;
-          if ((net->flags & TDH_NET_FUSE_ACT_GRAD) && fc_one_launch &&
-              fc_bwd_scatters_pool(s.fc_in, s.fc_out, batch)) {
-            const int r = i - 1 - ((i >= 1 && net->layers[i - 1].grad_folded) ? 1 : 0);
-            if (r >= 0 && net->layers[r].spec.kind == TDH_L_MAXPOOL &&
-                maxpool_scatters_from_fc(&net->layers[r].spec.pool, &through)) {
-              const DxTarget behind = dx_target(net, r);
-              if (behind.fold.kind == TDH_ACT_NONE) {
-                through.argmax = net->layers[r].argmax;
-                through.dx     = behind.dx;
-                reader         = r;
-              }
-            }
-          }
+          const int reader = fc_one_launch && fc_bwd_scatters_pool(s.fc_in, s.fc_out, batch)
+                               ? pool_in_front(net, i, &through) : -1;
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
-                         L.b_size ? L.db : nullptr, 1, fold, reader >= 0 ? &through : nullptr));
+                         L.b_size ? L.db : nullptr, 1, fold, reader >= 0 ? &through : nullptr,
+                         i == also_for ? &also : nullptr));
           if (reader >= 0) pool_done = reader;
         }
         break;
