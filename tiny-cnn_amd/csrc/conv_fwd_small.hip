@@ -66,19 +66,13 @@ __device__ __forceinline__ void act_apply16(const int kind, float (&v)[16]) {
   }
 }
 
+// Stages the input patch under the band (zero-filled where the window leaves the image), the
+// filter slice, the bias and the patch offset of every k into LDS: all loads of a thread are
+// issued before its first store.
 template <int NS>
-__global__ void __launch_bounds__(256, 2) conv_fwd_small_kernel(const FwdSmallArgs a) {
-  extern __shared__ __align__(16) float lds[];
-  float *xs = lds;
-  float *ws = lds + a.x_floats;  // [32][crs], rows past Cout are zero
-  float *bs = ws + 32 * a.crs;   // [32] bias, zero past Cout or without bias
-  int *offs = reinterpret_cast<int *>(bs + 32);  // [2*NS] patch offset of k (0 past K)
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bandi = blockIdx.x, img = blockIdx.y, co0 = blockIdx.z * 32;
-  const int oy0 = bandi * a.band;
-  const int nthr = blockDim.x;  // one wave per tile of the band, two to four waves
-
-  // ---- staging: all loads of a thread are issued before its first store
+__device__ __forceinline__ void fwd_small_stage(const FwdSmallArgs &a, float *xs, float *ws, float *bs, int *offs,
+                                                const int img, const int co0, const int oy0, const int tid,
+                                                const int nthr) {
   {
     const int iy0     = oy0 * a.sh - a.ph;
     const int x_total = a.C * a.rows_in * a.pitch;
@@ -135,6 +129,21 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_kernel(const FwdSmallAr
       offs[tid] = max(o, 0);
     }
   }
+}
+
+template <int NS>
+__global__ void __launch_bounds__(256, 2) conv_fwd_small_kernel(const FwdSmallArgs a) {
+  extern __shared__ __align__(16) float lds[];
+  float *xs = lds;
+  float *ws = lds + a.x_floats;  // [32][crs], rows past Cout are zero
+  float *bs = ws + 32 * a.crs;   // [32] bias, zero past Cout or without bias
+  int *offs = reinterpret_cast<int *>(bs + 32);  // [2*NS] patch offset of k (0 past K)
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bandi = blockIdx.x, img = blockIdx.y, co0 = blockIdx.z * 32;
+  const int oy0 = bandi * a.band;
+  const int nthr = blockDim.x;  // one wave per tile of the band, two to four waves
+
+  fwd_small_stage<NS>(a, xs, ws, bs, offs, img, co0, oy0, tid, nthr);
   __syncthreads();
 
   // ---- per-lane constants: the lane's column of the filter matrix
@@ -250,6 +259,111 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_kernel(const FwdSmallAr
   }
 }
 
+// The same tiles for a layer where nothing needs a guard or a choice per value: every band has
+// whole row pairs, the width is a multiple of 32 columns, the channels a multiple of 32, there is
+// no activation between convolution and pool, and the activation behind the pool is relu or
+// none. These tiles are bound by the vector instructions around the MFMAs (about 25 per MFMA
+// in the kernel above, guards, 64-bit addresses and saved exec masks most of them), so here
+// everything that depends on the tile is kept in scalar registers (the wave index is read from
+// the first lane for that), a lane adds one offset of its own that is computed once, and no
+// store has a condition.
+template <int NS>
+__global__ void __launch_bounds__(256, 2) conv_fwd_small_full_kernel(const FwdSmallArgs a) {
+  extern __shared__ __align__(16) float lds[];
+  float *xs = lds;
+  float *ws = lds + a.x_floats;
+  float *bs = ws + 32 * a.crs;
+  int *offs = reinterpret_cast<int *>(bs + 32);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int bandi = blockIdx.x, img = blockIdx.y, co0 = blockIdx.z * 32;
+  const int oy0 = bandi * a.band;
+  const int nthr = blockDim.x;
+  fwd_small_stage<NS>(a, xs, ws, bs, offs, img, co0, oy0, tid, nthr);
+  __syncthreads();
+
+  const int nl = lane & 31, half = lane >> 5;
+  float areg[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int k = 2 * s + half;
+    areg[s]     = k < a.crs ? ws[nl * a.crs + k] : 0.0f;
+  }
+  const int *offh = offs + half;
+  float bias_r[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) bias_r[i] = bs[(i >> 2) * 8 + half * 4 + (i & 3)];
+
+  const uint32_t ohw = a.OH * a.OW, OW = a.OW, POW = a.OW >> 1, pohw = (a.OH >> 1) * POW;
+  const uint32_t tiles = (a.band >> 1) * a.col_tiles;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = __builtin_amdgcn_readfirstlane(nthr >> 6);
+  // the lane's own part of every address: its channel group and its column
+  const uint32_t lane_out = half * 4 * ohw + nl, lane_pool = half * 4 * pohw + (nl >> 1);
+  const bool even  = !(nl & 1);
+  const bool pool  = a.pool_out != nullptr;
+  const float floor_v = a.pool_act_kind == TDH_ACT_RELU ? 0.0f : -INFINITY;  // relu as a max
+  float *out_img        = a.out + (static_cast<size_t>(img) * a.Kc + co0) * ohw;
+  float *pool_img       = a.pool_out + (static_cast<size_t>(img) * a.Kc + co0) * pohw;
+  float *pool_act_img   = a.pool_act_out + (static_cast<size_t>(img) * a.Kc + co0) * pohw;
+  int32_t *argmax_img   = a.pool_argmax + (static_cast<size_t>(img) * a.Kc + co0) * pohw;
+#pragma unroll 1
+  for (uint32_t tile = wave; tile < tiles; tile += nwaves) {
+    const uint32_t rp = a.div_col_tiles.div(tile), ct = tile - rp * a.col_tiles;
+    const uint32_t r = 2 * rp, c0 = 32 * ct;
+    const float *xb0 = xs + r * a.sh * a.pitch + (c0 + nl) * a.sw;
+    const float *xb1 = xb0 + a.sh * a.pitch;
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc0[i] = acc1[i] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int o = offh[2 * s];
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], xb0[o], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], xb1[o], acc1, 0, 0, 0);
+    }
+    // reg i of lane l holds channel 8*(i/4) + 4*(l/32) + i%4 at column l%32
+    const uint32_t oy = oy0 + r;
+    const uint32_t first = oy * OW + c0;  // of the tile inside a channel plane
+    float v0[16], v1[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      v0[i] = acc0[i] + bias_r[i];
+      v1[i] = acc1[i] + bias_r[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float *o = out_img + (((i >> 2) * 8 + (i & 3)) * ohw + first);  // scalar
+      o[lane_out]        = v0[i];
+      (o + OW)[lane_out] = v1[i];
+    }
+    if (pool) {
+      // as above: the window of an even lane in scan order, strict '>', start value lowest();
+      // where: the winner's distance from the window's first element (0, 1, OW, OW + 1), -1 when
+      // no value beat the start value
+      const uint32_t pfirst = (oy >> 1) * POW + (c0 >> 1);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float w4[4] = {v0[i], lane_xor1(v0[i]), v1[i], lane_xor1(v1[i])};
+        const int at[4]   = {0, 1, static_cast<int>(OW), static_cast<int>(OW) + 1};
+        float best = -FLT_MAX;
+        int where  = -1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (w4[j] > best) {
+            best  = w4[j];
+            where = at[j];
+          }
+        const uint32_t ch     = (i >> 2) * 8 + (i & 3);
+        const uint32_t chfirst = (co0 + ch) * ohw + first;  // scalar: flat CHW index of the tile's first element
+        if (even) {
+          (pool_img + (ch * pohw + pfirst))[lane_pool]   = best;
+          (argmax_img + (ch * pohw + pfirst))[lane_pool] = where < 0 ? 0 : static_cast<int>(chfirst + lane_out) + where;
+          if (a.pool_act_out) (pool_act_img + (ch * pohw + pfirst))[lane_pool] = best > floor_v ? best : floor_v;
+        }
+      }
+    }
+  }
+}
+
 struct FwdSmallPlan {
   FwdSmallArgs a;
   int ns;  // k-steps, rounded up to the next instantiated count
@@ -312,6 +426,16 @@ FwdSmallPlan make_fwd_small_plan(int batch, int C, int Kc, int H, int W, int OH,
 template <int NS>
 int launch_fwd_small(const FwdSmallPlan &p) {
   const int tiles = (p.a.band / 2) * p.a.col_tiles;
+  const FwdSmallArgs &a = p.a;
+  const bool full = a.OH % a.band == 0 && a.band % 2 == 0 && a.OW % 32 == 0 && a.Kc % 32 == 0 && !a.act_out &&
+                    (a.pool_act_kind == TDH_ACT_RELU || a.pool_act_kind == TDH_ACT_NONE || !a.pool_act_out) &&
+                    static_cast<long long>(a.Kc) * a.OH * a.OW < (1LL << 30);
+  if (full) {
+    TDH_LAUNCH((conv_fwd_small_full_kernel<NS>), p.grid, dim3(64 * std::min(4, std::max(2, tiles))), p.lds_bytes,
+               ctx().stream, p.a);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   TDH_LAUNCH((conv_fwd_small_kernel<NS>), p.grid, dim3(64 * std::min(4, std::max(2, tiles))), p.lds_bytes,
              ctx().stream, p.a);
   TDH_LAUNCH_CHECK();
