@@ -168,6 +168,7 @@ int launch_opt_update(tdh_opt *o, size_t n, const float *g, float grad_scale, fl
 struct OptTensor {
   float *g, *w, *s0, *s1;
   uint32_t n, first_block;
+  uint32_t block_elems;  // elements a workgroup updates: OPT_MULTI_ELEMS_PER_BLOCK or OPT_SUM_ELEMS_PER_BLOCK
   // A convolution's OIHW weight tensor whose filters the stride-1 kernels read in their own
   // layout: the update also writes the new value into those copies (wp_fwd[t][ci][co],
   // wp_dx[rs-1-t][co][ci]; unconnected pairs of the connection table as zero). NULL: none.
@@ -176,11 +177,33 @@ struct OptTensor {
   uint32_t C, Kc, rs;
 };
 constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 1024;  // one 16-byte access per thread: a pass of a small net is latency, not bandwidth
-// dev_powers: NULL, or device floats {b1_t, b2_t, ticket (zero), unused} that the kernel reads instead of the
-// host values and that a follow-up kernel advances n_tensors times (graph replay).
+// powers_in / powers_out: both NULL, or two device floats each: {b1_t, b2_t} that the kernel reads
+// instead of the host values, and where it leaves them advanced n_tensors times for the next
+// update (graph replay: a captured launch's arguments are frozen, so two captures whose
+// buffers are swapped take turns). They must not overlap.
+// Sums of K-split partial slices ([splits][mn] floats each) that the multi-tensor update adds to
+// a gradient tensor before it uses it, in the order of the split reduction kernel (eight
+// interleaved groups of slices, the group sums in order): the gradient tensors of a train step
+// whose weight-gradient kernels left their reductions to the optimizer. Such a tensor's table
+// entry has block_elems == OPT_SUM_ELEMS_PER_BLOCK.
+constexpr int OPT_SUM_ELEMS_PER_BLOCK = 128;
+constexpr int OPT_PENDING_MAX         = 8;
+struct OptPendingSum {
+  const float *partial;
+  const float *g;  // the gradient tensor (an OptTensor::g) the sum belongs to
+  uint32_t splits, mn;
+};
+struct OptPending {
+  OptPendingSum sum[OPT_PENDING_MAX];
+  int n;
+};
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
-                            int zero_grad, float *dev_powers);
+                            int zero_grad, const float *powers_in, float *powers_out,
+                            const OptPending *pending = nullptr);
+// conv.hip: the recorded split reductions in the optimizer's form (false: they do not all fit its
+// form or number). They stay recorded: flush_deferred_reduces launches or forgets them.
+bool peek_deferred_reduces(OptPending *out);
 bool profiling_active();
 // api.hip: the argument checks of the convolution entry points (backward: also what only the
 // backward pass refuses)

@@ -531,6 +531,18 @@ int flush_deferred_reduces(bool launch) {
   return TDH_OK;
 }
 
+bool peek_deferred_reduces(OptPending *out) {
+  const std::vector<ReduceJob> &all = deferred_reduces();
+  out->n = 0;
+  if (all.empty() || all.size() > static_cast<size_t>(OPT_PENDING_MAX)) return false;
+  for (const ReduceJob &r : all)  // plain accumulating sums into a dense tensor only
+    if (!(r.epi.accumulate && r.epi.ld == r.N && !r.epi.bias_n && r.epi.ag.kind == TDH_ACT_NONE)) return false;
+  for (const ReduceJob &r : all)
+    out->sum[out->n++] = OptPendingSum{r.partial, r.epi.out, static_cast<uint32_t>(r.splits),
+                                       static_cast<uint32_t>(r.M) * static_cast<uint32_t>(r.N)};
+  return true;
+}
+
 bool defer_reduce(const float *partial, int splits, int M, int N, const EpiRowMajor &epi) {
   if (!ctx().defer_reduce) return false;
   deferred_reduces().push_back(ReduceJob{partial, splits, M, N, epi});

@@ -442,11 +442,23 @@ __device__ __forceinline__ void opt_pack_store(const OptTensor &t, const uint32_
 template <int KIND, int NSTATE>
 __global__ void __launch_bounds__(EW_THREADS)
 opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptScalars p,
-                 float b1_t, float b2_t, float *dev_powers, const int advance,
-                 const int zero_grad) {
-  if (dev_powers) {
-    b1_t = dev_powers[0];
-    b2_t = dev_powers[1];
+                 float b1_t, float b2_t, const float *powers_in, float *powers_out, const int advance,
+                 const int zero_grad, const OptPending pend) {
+  if (powers_in) {
+    b1_t = powers_in[0];
+    b2_t = powers_in[1];
+    // The device copy of the powers advances as n_tensors update() calls would
+    // (optimizer.h:125-126), into the other of two buffers: nobody reads that one during this
+    // launch, so no workgroup has to wait for another. advance: 1 = b1_t only (adamax), 2 = both.
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      float q1 = b1_t, q2 = b2_t;
+      for (int i = 0; i < n_tensors; ++i) {
+        if (advance >= 1) q1 *= p.b1;
+        if (advance == 2) q2 *= p.b2;
+      }
+      powers_out[0] = q1;
+      powers_out[1] = q2;
+    }
   }
   int j = 0;
   while (j + 1 < n_tensors && table[j + 1].first_block <= blockIdx.x) ++j;
@@ -460,12 +472,70 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
   p.omb1t     = 1.0f - p1;
   p.omb2t     = 1.0f - p2;
   p.adamax_lr = static_cast<double>(p.alpha) / (1.0 - static_cast<double>(p1));
-  const uint32_t beg = (blockIdx.x - t.first_block) * OPT_MULTI_ELEMS_PER_BLOCK;
-  const uint32_t end = min(t.n, beg + OPT_MULTI_ELEMS_PER_BLOCK);
+  const uint32_t beg = (blockIdx.x - t.first_block) * t.block_elems;
+  const uint32_t end = min(t.n, beg + t.block_elems);
   // tensors come from separate allocations (256-byte aligned): 16-byte accesses are safe
   const uint32_t end4 = beg + ((end - beg) & ~3u);
+  // K-split partial slices of this gradient that nobody has added up yet: the summation tree of
+  // splitk_reduce_block (eight 32-lane groups each add every eighth slice in order, the group
+  // sums are added in group order), four consecutive elements a lane
+  __shared__ float pending_sum[8][OPT_SUM_ELEMS_PER_BLOCK];
+  int pj = -1;
+  for (int k = 0; k < pend.n; ++k)
+    if (pend.sum[k].g == t.g) pj = k;
+  if (pj >= 0) {
+    const OptPendingSum ps = pend.sum[pj];
+    constexpr uint32_t VEC = OPT_SUM_ELEMS_PER_BLOCK / 32;  // consecutive elements a lane adds up
+    const uint32_t o = threadIdx.x & 31, grp = threadIdx.x >> 5, i0 = beg + VEC * o;
+    float s4[VEC];
+#pragma unroll
+    for (uint32_t c = 0; c < VEC; ++c) s4[c] = 0.0f;
+    if (VEC == 4 && i0 + 4 <= end && (ps.mn & 3u) == 0) {
+      uint32_t z = grp;
+      for (; z + 56 < ps.splits; z += 64) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          v[u] = *reinterpret_cast<const float4 *>(ps.partial + static_cast<size_t>(z + 8 * u) * ps.mn + i0);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          s4[0] += v[u].x; s4[1 % VEC] += v[u].y; s4[2 % VEC] += v[u].z; s4[3 % VEC] += v[u].w;
+        }
+      }
+      for (; z < ps.splits; z += 8) {
+        const float4 v = *reinterpret_cast<const float4 *>(ps.partial + static_cast<size_t>(z) * ps.mn + i0);
+        s4[0] += v.x; s4[1 % VEC] += v.y; s4[2 % VEC] += v.z; s4[3 % VEC] += v.w;
+      }
+    } else {
+#pragma unroll
+      for (uint32_t c = 0; c < VEC; ++c) {
+        if (i0 + c >= end) break;
+        const float *col = ps.partial + i0 + c;
+        uint32_t z = grp;
+        for (; z + 56 < ps.splits; z += 64) {  // eight slices per trip: the loads are issued together
+          float v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = col[static_cast<size_t>(z + 8 * u) * ps.mn];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) s4[c] += v[u];
+        }
+        for (; z < ps.splits; z += 8) s4[c] += col[static_cast<size_t>(z) * ps.mn];
+      }
+    }
+#pragma unroll
+    for (uint32_t c = 0; c < VEC; ++c) pending_sum[grp][VEC * o + c] = s4[c];
+    __syncthreads();
+  }
+  auto grad = [&](const uint32_t i, const float g) {
+    if (pj < 0) return g;
+    float tt = pending_sum[0][i - beg];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) tt += pending_sum[k][i - beg];
+    return tt + g;
+  };
   for (uint32_t i = beg + threadIdx.x * 4; i < end4; i += EW_THREADS * 4) {
-    const float4 vg = *reinterpret_cast<const float4 *>(t.g + i);
+    float4 vg = *reinterpret_cast<const float4 *>(t.g + i);
+    vg = make_float4(grad(i, vg.x), grad(i + 1, vg.y), grad(i + 2, vg.z), grad(i + 3, vg.w));
     float4 vw       = *reinterpret_cast<float4 *>(t.w + i);
     float4 v0       = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
     if (NSTATE >= 1) v0 = *reinterpret_cast<float4 *>(t.s0 + i);
@@ -489,37 +559,12 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
     float ww = t.w[i], a = 0.0f, b = 0.0f;
     if (NSTATE >= 1) a = t.s0[i];
     if (NSTATE >= 2) b = t.s1[i];
-    opt_one<KIND>(t.g[i], ww, a, b, p);
+    opt_one<KIND>(grad(i, t.g[i]), ww, a, b, p);
     t.w[i] = ww;
     if (t.wp_fwd) opt_pack_store(t, i, ww);
     if (NSTATE >= 1) t.s0[i] = a;
     if (NSTATE >= 2) t.s1[i] = b;
     if (zero_grad) t.g[i] = 0.0f;
-  }
-  // The device copy of the powers advances as n_tensors update() calls would. The workgroup
-  // that draws the last ticket does it: by then every workgroup has read the old values.
-  // advance: 0 = leave them, 1 = b1_t only (adamax), 2 = both (adam).
-  if (advance) {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      unsigned int *ticket = reinterpret_cast<unsigned int *>(dev_powers + 2);
-      // acquire + release on the ticket: every workgroup's reads of the powers (made before
-      // its barrier above) happen before its own increment, and the last drawer's increment
-      // sees them all, so its writes below cannot overtake another workgroup's reads
-      const unsigned int drawn =
-          __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      if (drawn == gridDim.x - 1) {
-        float q1 = b1_t, q2 = b2_t;
-        for (int i = 0; i < n_tensors; ++i) {
-          q1 *= p.b1;
-          if (advance == 2) q2 *= p.b2;
-        }
-        dev_powers[0] = q1;
-        dev_powers[1] = q2;
-        // the reset follows the new powers (release); the next launch starts after this one ends
-        __hip_atomic_store(ticket, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
   }
 }
 
@@ -783,8 +828,16 @@ size_t rowsum_workspace_bytes(int outer, int rows, int cols) {
 
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
-                            int zero_grad, float *dev_powers) {
+                            int zero_grad, const float *powers_in, float *powers_out,
+                            const OptPending *pending) {
   if (n_tensors <= 0) return TDH_OK;
+  OptPending pend;
+  pend.n = 0;
+  double pending_bytes = 0.0;
+  if (pending) {
+    pend = *pending;
+    for (int k = 0; k < pend.n; ++k) pending_bytes += 4.0 * pend.sum[k].splits * pend.sum[k].mn;
+  }
   OptScalars p;
   p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; p.b1 = o->b1; p.b2 = o->b2;
   p.eps = o->eps;
@@ -797,16 +850,16 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
                                      "opt_nesterov_multi"};
   TDH_CHECK_ARG(o->kind >= 0 && o->kind <= TDH_OPT_NESTEROV, "optimizer kind %d is not supported",
                 o->kind);
+  const int advance = o->kind == TDH_OPT_ADAM ? 2 : o->kind == TDH_OPT_ADAMAX ? 1 : 0;
   const int nstate = (o->kind == TDH_OPT_SGD) ? 0
                      : (o->kind == TDH_OPT_ADAM || o->kind == TDH_OPT_ADAMAX) ? 2 : 1;
   // gradient read (+ cleared), weight read+write, states read+write
-  ProfScope prof(tags[o->kind], (12.0 + 8.0 * nstate + (zero_grad ? 4.0 : 0.0)) * total_params,
+  ProfScope prof(tags[o->kind], (12.0 + 8.0 * nstate + (zero_grad ? 4.0 : 0.0)) * total_params + pending_bytes,
                  WORK_BYTE);
-  const int advance = !dev_powers ? 0 : o->kind == TDH_OPT_ADAM ? 2 : o->kind == TDH_OPT_ADAMAX ? 1 : 0;
 #define TDH_LAUNCH_MULTI(KIND, NS)                                                            \
   TDH_LAUNCH((opt_multi_kernel<KIND, NS>), dim3(total_blocks), dim3(EW_THREADS), 0,   \
                      ctx().stream, dev_table, n_tensors, p, o->b1_t, o->b2_t,                  \
-                     dev_powers, advance, zero_grad)
+                     powers_in, powers_out, advance, zero_grad, pend)
   switch (o->kind) {
     case TDH_OPT_SGD: TDH_LAUNCH_MULTI(TDH_OPT_SGD, 0); break;
     case TDH_OPT_MOMENTUM: TDH_LAUNCH_MULTI(TDH_OPT_MOMENTUM, 1); break;

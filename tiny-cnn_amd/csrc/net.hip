@@ -37,18 +37,22 @@ struct tdh_net {
   int opt_tensors = 0, opt_blocks = 0;
   double opt_params = 0.0;
   // graph replay (TDH_NET_GRAPH): one captured train step, re-captured when its key changes
-  float *dev_powers = nullptr;          // {b1_t, b2_t, ticket} as the captured optimizer kernel uses them
+  // the powers as the captured optimizer kernels use them: two buffers of {b1_t, b2_t} (at 0 and
+  // at 4); a step reads buffer powers_at and leaves the advanced powers in the other one
+  float *dev_powers = nullptr;
+  int powers_at = 0;
   // partial sums and tickets of the one-launch kernel of two closing fully-connected layers
   float *tail_partials = nullptr, *tail_tickets = nullptr;
   struct GraphKey {
     int batch = 0, loss = 0, do_update = 0, test_phase = 0;
+    int powers_at = 0;                  // which buffer of the powers the captured optimizer reads
     const float *x = nullptr, *t = nullptr;
     const void *scratch = nullptr;      // the library scratch buffer the captured kernels use
     tdh_opt hyper = {};                 // hyper-parameters only (powers zeroed)
   };
   // a few captured steps are kept, so that alternating input buffers (double-buffered
   // uploads) or batch sizes (the short last batch of an epoch) do not re-capture every step
-  static constexpr int kGraphSlots = 4;
+  static constexpr int kGraphSlots = 8;
   struct GraphSlot {
     hipGraphExec_t exec = nullptr;
     GraphKey key;
@@ -473,7 +477,12 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
         t.s1 = which ? L.s1b : L.s1w;
         t.n  = static_cast<uint32_t>(n);
         t.first_block = block;
-        block += static_cast<uint32_t>(ceil_div_sz(n, OPT_MULTI_ELEMS_PER_BLOCK));
+        // weight gradients whose kernels may leave split sums to the optimizer: small blocks,
+        // eight groups of lanes add the slices of OPT_SUM_ELEMS_PER_BLOCK elements
+        t.block_elems = (L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC) && (flags & TDH_NET_GRAPH)
+                          ? OPT_SUM_ELEMS_PER_BLOCK : OPT_MULTI_ELEMS_PER_BLOCK;
+        if (n > (1u << 22)) t.block_elems = OPT_MULTI_ELEMS_PER_BLOCK;  // (bandwidth matters there)
+        block += static_cast<uint32_t>(ceil_div_sz(n, t.block_elems));
         net->opt_params += static_cast<double>(n);
         table.push_back(t);
       }
@@ -489,7 +498,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       }
     }
   }
-  if (rc == TDH_OK) rc = net_alloc(net, 4, &net->dev_powers, true);  // powers, ticket (zero)
+  if (rc == TDH_OK) rc = net_alloc(net, 8, &net->dev_powers, true);
   if (rc == TDH_OK && (flags & TDH_NET_FUSE_ACT_GRAD)) {
     // [fc, pointwise activation, fc] closes the net, or stands in front of a closing softmax
     int b = n_layers - 1;
@@ -506,8 +515,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
     for (hipStream_t &s : c.side)
       if (!s && hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess)
         rc = set_error(TDH_ERR_HIP, "tdh_net_create: cannot create a side stream");
-    // events: [0,n) gradient forks, [n,2n) packed forward filters, 2n and 2n+1 joins,
-    // 2n+2 start of the step, 2n+3 packed dX filters
+    // events: [0,n) gradient forks, 2n and 2n+1 joins, 2n+2 start of the step
     for (int i = 0; rc == TDH_OK && i < 2 * n_layers + 4; ++i) {
       hipEvent_t e = nullptr;
       if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess)
@@ -595,7 +603,7 @@ int tdh_net_update_weights(tdh_net *net, tdh_opt *opt) {
   TDH_CHECK_ARG(net && opt, "tdh_net_update_weights: null argument");
   // the optimizer kernel keeps the packed filter copies of a graph net current, as in a step
   TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
-                                  net->opt_params, 1.0f, 1, nullptr));
+                                  net->opt_params, 1.0f, 1, nullptr, nullptr));
   return post_update(net);
 }
 int tdh_net_set_phase(tdh_net *net, int train) {
@@ -655,7 +663,8 @@ int tdh_net_forward(tdh_net *net, int batch, const float *x) {
 // the chain forward -> loss -> dX ... -> dX, and the two join in front of the optimizer. The
 // kernels and their arguments are the same either way, so are the results.
 static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
-                        const float *t, int do_update, float *dev_powers, bool forked = false) {
+                        const float *t, int do_update, const float *powers_in, float *powers_out,
+                        bool forked = false) {
   Context &c = ctx();
   struct KeepScratch {  // hands out disjoint scratch pieces for the whole backward pass
     Context &c;
@@ -853,7 +862,24 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     }
   }
   TDH_TRY(finish_split_sum());  // (a max-pool has taken or finished it)
-  if (side_used[0]) {
+  // the split sums of the weight gradients: added up by the optimizer kernel when it runs next
+  // and every tensor concerned has the small blocks for that, else by a launch of their own
+  OptPending pending;
+  pending.n = 0;
+  bool to_optimizer = false;
+  if (side_used[0] && do_update && peek_deferred_reduces(&pending)) {
+    to_optimizer = true;
+    for (int k = 0; k < pending.n; ++k) {
+      bool small_blocks = false;
+      for (const tdh_net::Layer &L : net->layers)
+        if ((L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC) &&
+            ((pending.sum[k].g == L.dw && L.w_size <= (1u << 22)) || (pending.sum[k].g == L.db && L.b_size)))
+          small_blocks = true;
+      to_optimizer = to_optimizer && small_blocks;
+    }
+    if (to_optimizer) TDH_TRY(flush_deferred_reduces(false));  // (forgets them: the optimizer has them)
+  }
+  if (side_used[0] && !to_optimizer) {
     StreamSwap on_side(c.side[0]);
     TDH_TRY(flush_deferred_reduces());
   }
@@ -871,7 +897,8 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   // reaches the optimizer unscaled (rcp_batch_size is 1, see tdh_opt_update) and is then
   // cleared (layer.h:680)
   TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
-                                  net->opt_params, 1.0f, 1, dev_powers));
+                                  net->opt_params, 1.0f, 1, powers_in, powers_out,
+                                  to_optimizer ? &pending : nullptr));
   return post_update(net);
 }
 
@@ -879,6 +906,7 @@ static bool same_key(const tdh_net::GraphKey &a, const tdh_net::GraphKey &b) {
   // field by field: a caller's tdh_opt may carry padding or unused fields it never wrote
   const tdh_opt &p = a.hyper, &q = b.hyper;
   return a.batch == b.batch && a.loss == b.loss && a.do_update == b.do_update && a.test_phase == b.test_phase &&
+         a.powers_at == b.powers_at &&
          a.x == b.x &&
          a.t == b.t && a.scratch == b.scratch && p.kind == q.kind && p.alpha == q.alpha &&
          p.lambda == q.lambda && p.mu == q.mu && p.b1 == q.b1 && p.b2 == q.b2 && p.eps == q.eps;
@@ -903,11 +931,14 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   }
   // per-kernel timing needs the launches themselves, not a replay
   if (!(net->flags & TDH_NET_GRAPH) || profiling_active())
-    return enqueue_step(net, opt, loss_kind, batch, x, t, do_update, nullptr);
+    return enqueue_step(net, opt, loss_kind, batch, x, t, do_update, nullptr, nullptr);
 
   tdh_net::GraphKey key;
   key.batch = batch; key.loss = loss_kind; key.do_update = do_update; key.x = x; key.t = t;
   key.test_phase = net->test_phase;
+  // (only steps that advance the powers take turns between the two buffers)
+  const bool powers_move = opt && do_update && (opt->kind == TDH_OPT_ADAM || opt->kind == TDH_OPT_ADAMAX);
+  key.powers_at = powers_move ? net->powers_at : 0;
   if (opt) {
     key.hyper      = *opt;
     key.hyper.b1_t = key.hyper.b2_t = 0.0f;
@@ -941,7 +972,8 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
       tdh_opt capture_opt;
       if (opt) capture_opt = *opt;
       rc = enqueue_step(net, opt ? &capture_opt : nullptr, loss_kind, batch, x, t, do_update,
-                        net->dev_powers, /*forked=*/net_forks(net, batch));
+                        net->dev_powers + 4 * key.powers_at, net->dev_powers + 4 * (1 - key.powers_at),
+                        /*forked=*/net_forks(net, batch));
       e = hipStreamEndCapture(c.stream, &graph);
     }
     c.ws_locked = false;
@@ -966,7 +998,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   // line with the caller's optimizer object whenever the two have drifted apart
   if (opt && do_update && (opt->b1_t != net->mirror_b1_t || opt->b2_t != net->mirror_b2_t)) {
     const float h[2] = {opt->b1_t, opt->b2_t};
-    TDH_TRY(tdh_memcpy_h2d(net->dev_powers, h, sizeof(h)));
+    TDH_TRY(tdh_memcpy_h2d(net->dev_powers + 4 * key.powers_at, h, sizeof(h)));
   }
   slot->last_use = ++net->graph_clock;
   TDH_HIP(hipGraphLaunch(slot->exec, ctx().stream));
@@ -982,6 +1014,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
     }
     net->mirror_b1_t = opt->b1_t;
     net->mirror_b2_t = opt->b2_t;
+    if (powers_move) net->powers_at = 1 - net->powers_at;  // where this step left them
   }
   return TDH_OK;
 }
