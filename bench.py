@@ -139,7 +139,14 @@ def roofline_of(entry):
             "algorithmic_work_per_launch": entry["work"]}
 
 
-def run_workload(T, wl, steps, warmup, profile_steps):
+def mark(T, marker):
+    """Three launches of the fill kernel on one small buffer: a pattern that a trace of this run
+    (which knows kernels by symbol only) can find, in front of every step of the per-kernel pass."""
+    for _ in range(3):
+        T.fill_zero(marker)
+
+
+def run_workload(T, wl, steps, warmup, profile_steps, sequence=None):
     for _ in range(warmup):
         wl.step()
     T.sync()
@@ -160,10 +167,22 @@ def run_workload(T, wl, steps, warmup, profile_steps):
     T.profile_begin()
     wl.step()
     T.profile_end()
+    marker = T.DevBuf((4400,), zero=True)
     T.profile_begin()
     for _ in range(profile_steps):
+        mark(T, marker)
         wl.step()
+    mark(T, marker)
     prof = T.profile_end()
+    # the marks are not part of the workload
+    prof = [e for e in prof if not (e["tag"] == "fill_zero" and e["launches"] == 3 * (profile_steps + 1))]
+    if sequence is not None:  # the tags of one step's launches, in dispatch order
+        tags = T.profile_launches()
+        per = (len(tags) - 3) // profile_steps
+        chunks = [tags[i * per:(i + 1) * per] for i in range(profile_steps)]
+        assert per * profile_steps + 3 == len(tags) and all(c == chunks[0] for c in chunks) \
+            and chunks[0][:3] == ["fill_zero"] * 3, "the steps of the per-kernel pass differ"
+        sequence.extend(chunks[0][3:])
     kernels = [roofline_of(e) for e in prof]
     for k, e in zip(kernels, prof):
         k["ms_per_step"] = round(e["total_ms"] / profile_steps, 4)
@@ -276,6 +295,9 @@ def main():
     ap.add_argument("--others", action="store_true", help="(default) also run the other workloads")
     ap.add_argument("--no-others", action="store_true", help="only the named workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sequence-out", default=None,
+                    help="write the kernel tags of one step in dispatch order to this JSON file "
+                         "(tiny-cnn_amd.profsum reads a rocprofv3 trace of the same run tag by tag with it)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); "
@@ -288,7 +310,11 @@ def main():
 
     wl = make_workload(T, W, args.workload)
     prof_steps = max(1, min(args.steps, 10))
-    res = run_workload(T, wl, args.steps, args.warmup, prof_steps)
+    sequence = [] if args.sequence_out else None
+    res = run_workload(T, wl, args.steps, args.warmup, prof_steps, sequence)
+    if args.sequence_out:
+        with open(args.sequence_out, "w") as f:
+            json.dump({"workload": args.workload, "sequence": sequence}, f, indent=1)
     out = {
         "metric": "train samples/sec (fwd+bwd+update)",
         "value": round(res["samples_per_s"], 2),

@@ -138,6 +138,10 @@ int tdh_profile_begin(void);
 int tdh_profile_end(int32_t *n_entries);
 int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launches,
                       double *total_ms, double *work_per_launch, int32_t *work_unit);
+/* The tag of the index-th kernel launch of the profiled region, in dispatch order ("-" for a
+ * launch outside any tag); TDH_ERR_INVALID (no error text) past the last one. It lets a trace
+ * of the same run, which knows kernels only by symbol, be read tag by tag. */
+int tdh_profile_launch(int32_t index, char *tag, size_t tag_len);
 
 /* shape helpers: conv_out_length / pool_out_length (tiny_dnn/util/util.h:329-363) */
 int tdh_conv_out_w(const tdh_conv_desc *d);

@@ -269,6 +269,19 @@ def profile_end():
     return out
 
 
+def profile_launches():
+    """Tags of the kernel launches between the last profile_begin / profile_end, in dispatch order."""
+    out, tag, i = [], C.create_string_buffer(160), 0
+    while lib().tdh_profile_launch(i, tag, 160) == 0:
+        out.append(tag.value.decode())
+        i += 1
+    return out
+
+
+def fill_zero(buf):
+    check(lib().tdh_fill_zero(buf.ptr, C.c_size_t(buf.nbytes)), "tdh_fill_zero")
+
+
 # ------------------------------------------------------------------ descriptors
 
 def conv_desc(in_w, in_h, in_c, k_w, k_h, out_c, pad_same=False, has_bias=True, w_stride=1,

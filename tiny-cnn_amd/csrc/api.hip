@@ -157,6 +157,10 @@ std::vector<ProfRecord> g_records;
 // hipExtLaunchKernelGGL whether it stands for the begin or the end of the dispatch.
 std::vector<hipEvent_t> g_event_pool[2];  // [0] start events, [1] stop events
 std::vector<ProfEntry> g_entries;
+// the kernel launches of the profiled region in dispatch order, as indices into g_records
+// (-1: outside any scope), and after tdh_profile_end their tags
+std::vector<int> g_launch_order;
+std::vector<std::string> g_launch_tags;
 
 hipEvent_t take_event(int role) {
   if (!g_event_pool[role].empty()) {
@@ -197,6 +201,7 @@ ProfScope::~ProfScope() {
 
 void prof_launch_events(hipEvent_t *start, hipEvent_t *stop) {
   *start = *stop = nullptr;
+  if (g_profiling) g_launch_order.push_back(g_open_scope);
   if (!g_profiling || g_open_scope < 0) return;
   hipEvent_t b = take_event(0), e = take_event(1);
   if (!b || !e) return;
@@ -417,6 +422,8 @@ int tdh_profile_begin(void) {
     }
   g_records.clear();
   g_entries.clear();
+  g_launch_order.clear();
+  g_launch_tags.clear();
   g_open_scope = -1;
   g_profiling  = true;
   return TDH_OK;
@@ -428,6 +435,10 @@ int tdh_profile_end(int32_t *n_entries) {
   TDH_HIP(hipStreamSynchronize(ctx().stream));
   std::map<std::string, ProfEntry> by_tag;
   g_open_scope = -1;
+  g_launch_tags.clear();
+  for (const int slot : g_launch_order)
+    g_launch_tags.push_back(slot >= 0 && slot < static_cast<int>(g_records.size()) ? g_records[slot].tag : "-");
+  g_launch_order.clear();
   for (auto &r : g_records) {
     if (r.launches.empty()) continue;  // a scope that launched nothing (its work was deferred)
     double ms_sum = 0.0;
@@ -465,6 +476,13 @@ int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launche
   if (total_ms) *total_ms = e.total_ms;
   if (work_per_launch) *work_per_launch = e.launches ? e.work / e.launches : 0.0;
   if (work_unit) *work_unit = e.unit;
+  return TDH_OK;
+}
+
+int tdh_profile_launch(int32_t index, char *tag, size_t tag_len) {
+  TDH_REQUIRE_INIT();
+  if (index < 0 || index >= static_cast<int32_t>(g_launch_tags.size())) return TDH_ERR_INVALID;
+  if (tag && tag_len) std::snprintf(tag, tag_len, "%s", g_launch_tags[index].c_str());
   return TDH_OK;
 }
 

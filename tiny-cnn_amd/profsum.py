@@ -3,6 +3,16 @@
 
     python -m tiny-cnn_amd.profsum kernels  <dir>            # --kernel-trace --stats run
     python -m tiny-cnn_amd.profsum counters <dir> [<dir>..]  # --pmc runs (one counter set per dir)
+    python -m tiny-cnn_amd.profsum tags <dir> [<dir>..] --sequence seq.json [--merge profiles/hbm_traffic.json]
+
+`tags` reads the same traces kernel tag by kernel tag. bench.py's per-kernel pass runs the
+workload's steps eagerly with a mark in front of each (three launches of the fill kernel on one
+small buffer) and, with --sequence-out, writes the tags of one step's launches in dispatch order.
+Here the marks are found in the trace, the dispatches between two marks are matched one to one
+with that sequence, and durations (kernel-trace directories) and counters (--pmc directories)
+are averaged per tag: two tags that share a kernel symbol and grid (forward and dX of a
+stride-1 convolution) get rows of their own. --merge writes the scaled FETCH_SIZE / WRITE_SIZE
+bytes per launch into that JSON file under "workloads" / <workload> / <tag>.
 
 `kernels` prints, per kernel symbol and grid size, launches and average/min/max duration from
 `*_kernel_trace.csv` (kernel templates are launched at several problem shapes; the grid size
@@ -113,14 +123,126 @@ def counters(dirs, top, copy_mib):
         print("| " + " | ".join(cells) + " |")
 
 
+def read_dispatches(dirname):
+    """[(order key, symbol, grid, duration ns, {counter: value})] of a trace directory, in dispatch order."""
+    by_id = {}
+    try:
+        for path in find(dirname, "_counter_collection.csv"):
+            with open(path, newline="") as f:
+                for r in csv.DictReader(f):
+                    key = (int(r["Dispatch_Id"]) if r.get("Dispatch_Id") else int(r["Start_Timestamp"]),)
+                    d = by_id.setdefault(key, [short_name(r["Kernel_Name"]), int(r["Grid_Size"]),
+                                               int(r["End_Timestamp"]) - int(r["Start_Timestamp"]), {}])
+                    d[3][r["Counter_Name"]] = d[3].get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+    except SystemExit:
+        pass
+    if not by_id:
+        for path in find(dirname, "_kernel_trace.csv"):
+            with open(path, newline="") as f:
+                for r in csv.DictReader(f):
+                    grid = int(r["Grid_Size"]) if "Grid_Size" in r else \
+                        int(r["Grid_Size_X"]) * int(r["Grid_Size_Y"]) * int(r["Grid_Size_Z"])
+                    by_id[(int(r["Start_Timestamp"]),)] = [short_name(r["Kernel_Name"]), grid,
+                                                          int(r["End_Timestamp"]) - int(r["Start_Timestamp"]), {}]
+    return [(k, *v) for k, v in sorted(by_id.items())]
+
+
+def marked_steps(disp, length):
+    """The runs of `length` dispatches that stand between two marks (three fill kernel launches of
+    one grid size in a row)."""
+    is_fill = [d[1].startswith("fill_zero_kernel") for d in disp]
+    marks = []  # index of the first dispatch behind a mark
+    i = 0
+    while i < len(disp):
+        if is_fill[i]:
+            j = i
+            while j < len(disp) and is_fill[j] and disp[j][2] == disp[i][2]:
+                j += 1
+            if j - i == 3:
+                marks.append((i, j))
+            i = j
+        else:
+            i += 1
+    return [disp[b:a2] for (_, b), (a2, _) in zip(marks, marks[1:]) if a2 - b == length]
+
+
+def tags(dirs, sequence_file, merge, copy_mib):
+    import json
+    with open(sequence_file) as f:
+        seq = json.load(f)
+    workload, sequence = seq["workload"], seq["sequence"]
+    per_tag = collections.OrderedDict((t, {"kernel": None, "grid": None, "ns": [], "counters": collections.defaultdict(list)})
+                                      for t in sequence)
+    scale = {}
+    for dirname in dirs:
+        disp = read_dispatches(dirname)
+        steps = marked_steps(disp, len(sequence))
+        if not steps:
+            raise SystemExit(f"{dirname}: no marked step of {len(sequence)} dispatches found")
+        for step in steps:
+            for tag, (_, sym, grid, ns, ctr) in zip(sequence, step):
+                rec = per_tag[tag]
+                if rec["kernel"] not in (None, sym):
+                    raise SystemExit(f"tag {tag}: kernels {rec['kernel']} and {sym}: the trace is not of this run")
+                rec["kernel"], rec["grid"] = sym, grid
+                if not ctr:
+                    rec["ns"].append(ns)
+                for c, v in ctr.items():
+                    rec["counters"][c].append(v)
+        copies = [d for d in disp if d[1].startswith("copy_kernel")]
+        if copies:  # the yardstick is the largest copy of the run
+            big = max(d[2] for d in copies)
+            for c in ("FETCH_SIZE", "WRITE_SIZE"):
+                v = [d[4][c] for d in copies if d[2] == big and c in d[4]]
+                if v:
+                    scale[c] = copy_mib * (1 << 20) / (sum(v) / len(v) * 1024.0)
+    mean = lambda xs: sum(xs) / len(xs) if xs else float("nan")
+    names = sorted({c for r in per_tag.values() for c in r["counters"]})
+    if scale:
+        print("counter scale from copy_kernel (%d MiB read, %d MiB written; counters in KiB): "
+              % (copy_mib, copy_mib) + ", ".join(f"{c} x{s:.4f}" for c, s in sorted(scale.items())) + "\n")
+    head = ["tag", "kernel", "grid", "launches per step", "avg us"] + names + [c + " bytes (scaled)" for c in sorted(scale)]
+    print("| " + " | ".join(head) + " |")
+    print("|---|---|" + "---:|" * (len(head) - 2))
+    out = {}
+    for tag, r in per_tag.items():
+        cells = [f"`{tag}`", f"`{r['kernel']}`", str(r["grid"]), str(sequence.count(tag)),
+                 f"{mean(r['ns']) / 1e3:.2f}" if r["ns"] else "-"]
+        cells += [f"{mean(r['counters'].get(c, [])):.4g}" for c in names]
+        cells += [f"{mean(r['counters'].get(c, [])) * 1024.0 * scale[c]:.4g}" for c in sorted(scale)]
+        print("| " + " | ".join(cells) + " |")
+        if "FETCH_SIZE" in scale and "WRITE_SIZE" in scale:
+            fb = mean(r["counters"]["FETCH_SIZE"]) * 1024.0 * scale["FETCH_SIZE"]
+            wb = mean(r["counters"]["WRITE_SIZE"]) * 1024.0 * scale["WRITE_SIZE"]
+            out[tag] = {"kernel": r["kernel"], "grid": r["grid"], "fetch_bytes": round(fb), "write_bytes": round(wb),
+                        "hbm_bytes_per_launch": round(fb + wb)}
+    if merge and out:
+        try:
+            with open(merge) as f:
+                js = json.load(f)
+        except OSError:
+            js = {}
+        js.setdefault("workloads", {})[workload] = out
+        js["scale"] = {c: round(v, 4) for c, v in scale.items()}
+        with open(merge, "w") as f:
+            json.dump(js, f, indent=1)
+        print(f"\n{len(out)} tags of {workload} written to {merge}")
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("mode", choices=("kernels", "counters"))
+    ap.add_argument("mode", choices=("kernels", "counters", "tags"))
+    ap.add_argument("--sequence", help="tags: the file bench.py --sequence-out wrote in the traced run")
+    ap.add_argument("--merge", help="tags: JSON file that takes the scaled bytes per launch")
     ap.add_argument("dirs", nargs="+")
     ap.add_argument("--top", type=int, default=40)
     ap.add_argument("--copy-mib", type=int, default=256)
     a = ap.parse_args()
-    if a.mode == "kernels":
+    if a.mode == "tags":
+        if not a.sequence:
+            raise SystemExit("tags needs --sequence")
+        tags(a.dirs, a.sequence, a.merge, a.copy_mib)
+    elif a.mode == "kernels":
         kernels(a.dirs[0], a.top)
     else:
         counters(a.dirs, a.top, a.copy_mib)
