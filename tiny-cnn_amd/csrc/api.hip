@@ -117,23 +117,25 @@ struct StaticScratchScope {
 // Tuning sweeps only: the environment variable TDH_GEMM_PLAN="cfg,splits", read once by
 // tdh_init, forces one tile configuration (0..9, see gemm_mfma.h) and split count for every
 // GEMM of the process; unset, the plan is a function of the shape alone. Not part of the ABI.
-static int g_force_cfg = -1, g_force_splits = 1;
+static int g_force_cfg = -1, g_force_splits = 1, g_force_only_m = -1;
 
 static void read_gemm_plan_override() {
   g_force_cfg    = -1;
   g_force_splits = 1;
   const char *e = std::getenv("TDH_GEMM_PLAN");
-  int cfg = -1, splits = 1;
-  if (e && std::sscanf(e, "%d,%d", &cfg, &splits) == 2 && cfg >= 0 && cfg < 10 && splits >= 1) {
+  int cfg = -1, splits = 1, only_m = -1;
+  g_force_only_m = -1;
+  if (e && std::sscanf(e, "%d,%d,%d", &cfg, &splits, &only_m) >= 2 && cfg >= 0 && cfg < 10 && splits >= 1) {
     g_force_cfg    = cfg;
     g_force_splits = splits;
+    g_force_only_m = only_m;  // "cfg,splits,M": only products with M rows
   }
 }
 
-bool gemm_plan_override(int *cfg, int *splits) {
+bool gemm_plan_override(int *cfg, int *splits, int M) {
   *cfg    = g_force_cfg;
   *splits = g_force_splits;
-  return g_force_cfg >= 0;
+  return g_force_cfg >= 0 && (g_force_only_m < 0 || g_force_only_m == M);
 }
 
 // ----------------------------------------------------------------- profiler

@@ -54,7 +54,7 @@ int set_error(int code, const char *fmt, ...);
 int ws_begin(size_t total);
 // Next 256-byte aligned piece of the reserved scratch.
 int ws_take(size_t bytes, void **out);
-bool gemm_plan_override(int *cfg, int *splits);
+bool gemm_plan_override(int *cfg, int *splits, int M);
 inline size_t ws_align(size_t bytes) { return (bytes + 255) & ~static_cast<size_t>(255); }
 
 #define TDH_REQUIRE_INIT()                                                     \

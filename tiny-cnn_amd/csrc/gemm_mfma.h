@@ -568,8 +568,9 @@ constexpr TileCfg kTiles[] = {
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
-// Optional override "cfg,splits" from the environment (tuning runs only).
-bool gemm_plan_override(int *cfg, int *splits);
+// Optional override "cfg,splits[,M]" from the environment (tuning runs only; with M only
+// products of that many rows).
+bool gemm_plan_override(int *cfg, int *splits, int M);
 
 // Shape-only heuristics (no device queries) so that results are reproducible anywhere.
 inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
@@ -607,7 +608,7 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
     }
   }
   int ocfg, osplits;
-  if (gemm_plan_override(&ocfg, &osplits)) {
+  if (gemm_plan_override(&ocfg, &osplits, M)) {
     best = ocfg;
     best_splits = allow_split ? osplits : 1;
     if (best_splits > K / GEMM_BK && K >= GEMM_BK) best_splits = K / GEMM_BK;
@@ -629,7 +630,7 @@ inline size_t gemm_workspace_bytes(int M, int N, int K, bool allow_split) {
   const GemmPlan p = plan_gemm(M, N, K, allow_split);
   int ocfg, osplits;
   int splits = p.splits;
-  if (gemm_plan_override(&ocfg, &osplits) && osplits > splits) splits = osplits;
+  if (gemm_plan_override(&ocfg, &osplits, M) && osplits > splits) splits = osplits;
   return splits > 1 ? ws_align(static_cast<size_t>(splits) * M * N * sizeof(float)) : 0;
 }
 
