@@ -215,8 +215,7 @@ def measured_traffic(tag, workload=None):
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
             js = json.load(f)
-        rec = js.get("workloads", {}).get(workload, {}).get(tag) if workload else None
-        rec = rec or js["kernels"].get(tag)
+        rec = js.get("workloads", {}).get(workload, {}).get(tag)
         return rec and rec["hbm_bytes_per_launch"]
     except (OSError, ValueError, KeyError):
         return None

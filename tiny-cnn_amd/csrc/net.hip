@@ -672,7 +672,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     KeepScratch(Context &cc, bool o) : c(cc), on(o) {}
     void start() { if (on) { c.workspace_off = 0; c.ws_keep = true; } }
     ~KeepScratch() { c.ws_keep = false; }
-  } keep(c, forked);
+  } keep(c, forked || (!forked && profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch)));
   bool side_used[2] = {false, false};
   // The split reductions behind the weight-gradient kernels and the row sums of the bias
   // gradients of a branching step are collected and launched once each behind the last layer:
@@ -767,7 +767,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     }
     switch (s.kind) {
       case TDH_L_CONV:
-        TDH_TRY(ws_begin((forked ? 3 : 1) * conv2d_workspace_bytes(&s.conv, batch)));
+        TDH_TRY(ws_begin((forked || as_forked ? 3 : 1) * conv2d_workspace_bytes(&s.conv, batch)));
       {
         const float *wp = packed && L.wp_dx && conv_uses_packed(&s.conv, batch, 1) ? L.wp_dx : nullptr;
         // the layer that reads this dX next (behind a folded activation) is a max-pool: its
@@ -800,6 +800,19 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));
             c.defer_rowsum = false;
           }
+        } else if (as_forked) {
+          // the launches of the captured, branching step, one after the other
+          {
+            LeaveSplitSum leave(c, pool_reads);
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+          }
+          const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
+          c.defer_reduce = true;
+          TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, db_with_dw ? L.db : nullptr, 1,
+                             ActGrad(), L.tbl_dev));
+          c.defer_reduce = false;
+          if (L.b_size && !db_with_dw)
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));
         } else {
           LeaveSplitSum leave(c, pool_reads);
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
@@ -823,7 +836,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         } else if (as_forked && !fc_one_launch) {
           // the launches of the captured, branching step, one after the other
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
+          c.defer_reduce = true;
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad()));
+          c.defer_reduce = false;
           if (L.b_size)
             TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad()));
         } else {
@@ -867,7 +882,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   OptPending pending;
   pending.n = 0;
   bool to_optimizer = false;
-  if (side_used[0] && do_update && peek_deferred_reduces(&pending)) {
+  if ((side_used[0] || as_forked) && do_update && peek_deferred_reduces(&pending)) {
     to_optimizer = true;
     for (int k = 0; k < pending.n; ++k) {
       bool small_blocks = false;
@@ -881,6 +896,8 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   }
   if (side_used[0] && !to_optimizer) {
     StreamSwap on_side(c.side[0]);
+    TDH_TRY(flush_deferred_reduces());
+  } else if (as_forked && !to_optimizer) {
     TDH_TRY(flush_deferred_reduces());
   }
   if (side_used[1]) {
@@ -930,8 +947,12 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
     net->packs_valid = true;
   }
   // per-kernel timing needs the launches themselves, not a replay
-  if (!(net->flags & TDH_NET_GRAPH) || profiling_active())
+  if (!(net->flags & TDH_NET_GRAPH) || profiling_active()) {
+    // (the timing pass of a branching step keeps every layer's scratch piece until the optimizer
+    // has read the split sums: the buffer must not grow, and so move, on the way)
+    if (net->flags & TDH_NET_GRAPH) TDH_TRY(ws_begin(net->scratch));
     return enqueue_step(net, opt, loss_kind, batch, x, t, do_update, nullptr, nullptr);
+  }
 
   tdh_net::GraphKey key;
   key.batch = batch; key.loss = loss_kind; key.do_update = do_update; key.x = x; key.t = t;

@@ -180,11 +180,14 @@ def tags(dirs, sequence_file, merge, copy_mib):
         if not steps:
             raise SystemExit(f"{dirname}: no marked step of {len(sequence)} dispatches found")
         for step in steps:
+            if [d[1] for d in step] != [d[1] for d in steps[0]]:
+                raise SystemExit(f"{dirname}: the marked steps launch different kernels: the trace is not of this run")
             for tag, (_, sym, grid, ns, ctr) in zip(sequence, step):
                 rec = per_tag[tag]
-                if rec["kernel"] not in (None, sym):
-                    raise SystemExit(f"tag {tag}: kernels {rec['kernel']} and {sym}: the trace is not of this run")
-                rec["kernel"], rec["grid"] = sym, grid
+                if rec["kernel"] is None:
+                    rec["kernel"], rec["grid"] = sym, grid
+                elif sym not in rec["kernel"].split(" + "):  # a tag may cover launches of several kernels
+                    rec["kernel"] += " + " + sym
                 if not ctr:
                     rec["ns"].append(ns)
                 for c, v in ctr.items():
