@@ -328,6 +328,69 @@ def test_graph_replay_matches_eager_on_every_step(T, W, name, batch):
     eager.close(); graph.close()
 
 
+@pytest.mark.parametrize("opt_kind", ["sgd", "momentum", "nesterov", "adagrad", "rmsprop", "adamax"])
+def test_branching_replay_matches_eager_for_every_optimizer(T, W, opt_kind):
+    """The replayed step of a net that branches leaves the weight gradients' split sums to the
+    optimizer kernel and keeps the bias-correction powers in two device buffers that take turns:
+    four steps of every optimizer kind give bit for bit the weights (and host-side powers) of
+    eager steps, which run the reductions as launches of their own."""
+    spec, params, x, t, _, loss, _, _ = W.make_batch("cifar10_cnn_b128", batch=16)
+    batch = 16
+    eager = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD)
+    graph = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
+    for (i, which, a) in params:
+        eager.set_param(i, which, a)
+        graph.set_param(i, which, a)
+    o1, o2 = T.opt_desc(opt_kind), T.opt_desc(opt_kind)
+    xd, td = T.to_device(x), T.to_device(t)
+    for step in range(4):
+        eager.train_step(o1, loss, batch, xd, td)
+        graph.train_step(o2, loss, batch, xd, td)
+        for (i, which, a) in params:
+            assert np.array_equal(eager.get_param(i, which), graph.get_param(i, which)), (step, i, which)
+        assert o1.b1_t == o2.b1_t and o1.b2_t == o2.b2_t
+    eager.close(); graph.close()
+
+
+def test_branching_replay_with_ragged_gradient_tensors_matches_eager_and_oracle(T, O, W):
+    """Weight tensors whose element counts are no multiples of four (33 x 75, 35 x 297) and odd
+    bias lengths: the optimizer kernel adds their split sums element by element. Three Adam
+    steps of the replayed, branching step against eager steps (bit for bit) and the oracle."""
+    spec = [("conv", 16, 16, 3, 5, 33, True), ("maxpool", 16, 16, 33, 2), ("act", "relu"),
+            ("conv", 8, 8, 33, 3, 35, True), ("act", "tanh"), ("fc", 8 * 8 * 35, 10), ("act", "softmax")]
+    batch = 64
+    rng = np.random.default_rng(321)
+    eager = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD)
+    graph = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    params = []
+    for i, l in enumerate(spec):
+        nw, nb, fan_in, _ = W.layer_fans(l)
+        if nw:
+            w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+            b = rng.uniform(-0.2, 0.2, nb).astype(np.float32)
+            for n in (eager, graph):
+                n.set_param(i, 0, w); n.set_param(i, 1, b)
+            ref.weight(i)[:] = w; ref.bias(i)[:] = b
+            params += [(i, 0), (i, 1)]
+    x = rng.standard_normal((batch, 3 * 16 * 16)).astype(np.float32)
+    t = np.eye(10, dtype=np.float32)[rng.integers(0, 10, batch)]
+    xd, td = T.to_device(x), T.to_device(t)
+    o1, o2, ro = T.opt_desc("adam"), T.opt_desc("adam"), O.opt_desc("adam")
+    for step in range(3):
+        eager.train_step(o1, "ce_multiclass", batch, xd, td)
+        graph.train_step(o2, "ce_multiclass", batch, xd, td)
+        ref.train_step(ro, "ce_multiclass", x, t)
+        for (i, which) in params:
+            assert np.array_equal(eager.get_param(i, which), graph.get_param(i, which)), (step, i, which)
+    # (Adam divides by the gradient's own size: the weights are compared at the looser bound that
+    # the float64 tests justify; the bit-for-bit agreement above is the point here)
+    for (i, which) in params:
+        want = ref.weight(i) if which == 0 else ref.bias(i)
+        assert_close(graph.get_param(i, which), want, 10 * REL_TOL, f"parameter {i}.{which}")
+    eager.close(); graph.close()
+
+
 def test_net_with_every_other_activation_matches_oracle(T, O, W):
     """A small net that chains the parameterised and remaining activation layers: two Adam
     steps, every layer output, gradient and updated weight against the oracle."""
