@@ -330,6 +330,12 @@ def main():
     }
     if out["roofline"]:
         out["roofline"]["traffic"] = measured_traffic(out["roofline"]["kernel"], args.workload)
+    flop_k = [k for k in res["kernels"] if k["unit"] == "TFLOP/s"]
+    if flop_k:  # all MFMA-bound kernels of the step together
+        tot_flop = sum(k["algorithmic_work_per_launch"] * k["launches"] for k in flop_k)
+        tot_s = sum(k["avg_launch_us"] * k["launches"] for k in flop_k) * 1e-6
+        out["mfma_kernels_together"] = {"TFLOP/s": round(tot_flop / tot_s / 1e12, 2),
+                                        "frac": round(tot_flop / tot_s / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
     out["copy_yardstick"] = copy_yardstick(T)
     if hasattr(wl, "step_from_host"):  # never `value`: reported for callers that own host buffers
         for _ in range(8):  # both device slots get their captured step
