@@ -187,7 +187,7 @@ struct EpiImageRowsAct {
 // --------------------------------------------------------------------- kernel
 template <int BM, int BN, int WM, int WN, bool A_LANE_K, bool B_LANE_K, bool A_VEC, bool B_VEC,
           class AOp, class BOp, class Epi>
-__global__ void __launch_bounds__(64 * WM * WN)
+__global__ void __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(3, 8)))
 gemm_mfma_kernel(const AOp aop, const BOp bop, const Epi epi, const int M, const int N,
                  const int K, const int k_per_split, float *__restrict__ partial) {
   constexpr int BK  = GEMM_BK;
