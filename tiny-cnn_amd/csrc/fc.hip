@@ -651,6 +651,209 @@ __global__ void __launch_bounds__(TL_NT) fc_two_layer_tail_kernel(const FcTail2 
   }
 }
 
+// The backward pass of a small fully-connected layer on the matrix cores, one launch: dX, dW, db
+// and, where asked for, dW and db of another small layer of the same batch (the closing layer of
+// a classifier, whose dX left with the loss gradient). Same shape of work as
+// fc_bwd_fused_kernel (a role per workgroup), but every product runs on
+// v_mfma_f32_16x16x4_f32 with its operands read from memory in the fragment layout (see
+// fc_two_layer_tail_kernel), so a wave executes a few dozen instructions instead of a 128-step
+// loop out of LDS: 10.9 -> about 6 us for the CIFAR net's two layers.
+//   dX[m][j]  = sum_c dY[m][c] W[j][c]: a wave a 16 x 16 block, both operands 16 bytes a lane along c
+//   dW[k][o]  = sum_m X[m][k] dY[m][o]: a workgroup a strip of 16 rows k x 64 columns o, its four
+//               waves every fourth 16-deep slice of the batch, added through LDS in wave order;
+//               dY 16 bytes a lane along o (component cc: columns 4 r + cc), X a float a lane
+//   the other layer's dW: 16 x 16 blocks, both operands a float a lane (its width need not be a
+//               multiple of four)
+struct FcBwdMfma {
+  const float *x, *w, *dy;  // X[batch][in], W[in][out], dY[batch][out]; out a multiple of 4
+  EpiRowMajorPool xepi;     // dX (row.out null: not asked for)
+  float *dw, *db;
+  int batch, in, out, accumulate;
+  int nx, xcb;   // dX workgroups (four blocks each), column blocks ceil(in / 16)
+  int nw, wcg;   // dW workgroups, column groups ceil(out / 64)
+  int ndb;       // workgroups of 32 bias columns
+  const float *x2, *dy2;    // the other layer: X2[batch][in2], dY2[batch][out2]
+  float *dw2, *db2;
+  int in2, out2, nw2, w2cb, ndb2;
+};
+
+__global__ void __launch_bounds__(256) fc_bwd_mfma_kernel(const FcBwdMfma f) {
+  __shared__ __attribute__((aligned(16))) float red[4][16][TL_LD];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  int b = blockIdx.x;
+  if (b < f.nx) {
+    // ---- dX: block (rb, jb) of 16 rows and 16 columns
+    const int blk = 4 * b + wave;
+    const int rb = blk / f.xcb, jb = blk - rb * f.xcb;
+    const int m0 = 16 * rb, j0 = 16 * jb;
+    if (m0 >= f.batch) return;
+    const int agk     = f.xepi.row.ag.kind;
+    const bool pooled = f.xepi.pool.argmax != nullptr;
+    // what the epilogue reads, asked for first: rows and columns past the end read the last ones
+    const int j = j0 + r, jc = min(j, f.in - 1);
+    float py[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    int am[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = min(m0 + 4 * q + i, f.batch - 1) * f.in + jc;
+      if (agk != TDH_ACT_NONE) py[i] = f.xepi.row.ag.y[idx];
+      if (pooled) am[i] = f.xepi.pool.argmax[idx];
+    }
+    const float *arow = f.dy + static_cast<size_t>(min(m0 + r, f.batch - 1)) * f.out;
+    const float *brow = f.w + static_cast<size_t>(jc) * f.out;
+    tail_f4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int k0 = 0; k0 < f.out; k0 += 64) {
+      float4 av[4], bv[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const int kc  = k0 + 16 * kk + 4 * q;
+        const bool ok = kc < f.out;
+        av[kk] = tail_keep(tail_ld4(arow + (ok ? kc : 0)), ok);
+        bv[kk] = tail_ld4(brow + (ok ? kc : 0));
+      }
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(av[kk].x, bv[kk].x, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(av[kk].y, bv[kk].y, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(av[kk].z, bv[kk].z, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x4f32(av[kk].w, bv[kk].w, d, 0, 0, 0);
+      }
+    }
+    if (j >= f.in) return;
+    const TailGrad gx = tail_grad_coef(agk);
+    const int cbase   = f.xepi.col(j).base;
+    const int W       = f.xepi.pool.W;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 4 * q + i;
+      if (m >= f.batch) continue;
+      // the steps of EpiRowMajorPool::store without a bias, not accumulating
+      const float v = ((d[i] + 0.0f) * tail_grad_factor(gx, py[i])) + 0.0f;
+      f.xepi.row.out[m * f.in + j] = v;
+      if (pooled) {
+        const int a = am[i] - cbase;
+        float *p    = f.xepi.pool.dx + static_cast<size_t>(m) * f.xepi.sample_in + cbase;
+        *reinterpret_cast<float2 *>(p)     = make_float2(a == 0 ? v : 0.0f, a == 1 ? v : 0.0f);
+        *reinterpret_cast<float2 *>(p + W) = make_float2(a == W ? v : 0.0f, a == W + 1 ? v : 0.0f);
+      }
+    }
+    return;
+  }
+  b -= f.nx;
+  if (b < f.nw) {
+    // ---- dW: rows k0 .. k0 + 15, columns o0 .. o0 + 63
+    const int strip = b / f.wcg, cg = b - strip * f.wcg;
+    const int k0 = 16 * strip, o0 = 64 * cg;
+    const float *xcol = f.x + min(k0 + r, f.in - 1);
+    const float *dcol = f.dy + (o0 + 4 * r < f.out ? o0 + 4 * r : 0);
+    tail_f4 acc[4] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll 2
+    for (int m16 = 16 * wave; m16 < f.batch; m16 += 64) {
+      float a[4];
+      float4 bv[4];
+#pragma unroll
+      for (int comp = 0; comp < 4; ++comp) {
+        const int m   = m16 + 4 * q + comp;
+        const bool ok = m < f.batch;
+        const int mc  = ok ? m : f.batch - 1;
+        const float v = xcol[static_cast<size_t>(mc) * f.in];
+        a[comp]       = ok ? v : 0.0f;
+        bv[comp]      = tail_ld4(dcol + static_cast<size_t>(mc) * f.out);
+      }
+#pragma unroll
+      for (int comp = 0; comp < 4; ++comp) {
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[comp], bv[comp].x, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[comp], bv[comp].y, acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[comp], bv[comp].z, acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[comp], bv[comp].w, acc[3], 0, 0, 0);
+      }
+    }
+    // acc[cc][i]: row 4 q + i, column 4 r + cc
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<float4 *>(&red[wave][4 * q + i][4 * r]) = make_float4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
+    __syncthreads();
+    const int row = tid >> 4, c4 = 4 * (tid & 15);
+    float4 s = *reinterpret_cast<const float4 *>(&red[0][row][c4]);
+#pragma unroll
+    for (int v = 1; v < 4; ++v) {
+      const float4 p = *reinterpret_cast<const float4 *>(&red[v][row][c4]);
+      s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+    }
+    if (k0 + row < f.in && o0 + c4 < f.out) {
+      float4 *dst = reinterpret_cast<float4 *>(f.dw + static_cast<size_t>(k0 + row) * f.out + o0 + c4);
+      if (f.accumulate) {
+        const float4 old = *dst;
+        s.x += old.x; s.y += old.y; s.z += old.z; s.w += old.w;
+      }
+      *dst = s;
+    }
+    return;
+  }
+  b -= f.nw;
+  float(*part)[32] = reinterpret_cast<float(*)[32]>(&red[0][0][0]);
+  auto bias_block = [&](const float *dy, float *db, const int out, const int cb) {
+    // 32 columns of the column sums of dy[batch][out]: rows g, g + 8, ... per 32-lane group, the
+    // group sums in order (as the stand-alone column sum does)
+    const int cl = tid & 31, g = tid >> 5;
+    const int c  = cb * 32 + cl;
+    float s = 0.0f;
+    if (c < out)
+      for (int rr = g; rr < f.batch; rr += 8) s += dy[static_cast<size_t>(rr) * out + c];
+    part[g][cl] = s;
+    __syncthreads();
+    if (g == 0 && c < out) {
+      float t = part[0][cl];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) t += part[i][cl];
+      db[c] = f.accumulate ? db[c] + t : t;
+    }
+  };
+  if (b < f.ndb) {
+    bias_block(f.dy, f.db, f.out, b);
+    return;
+  }
+  b -= f.ndb;
+  if (b < f.nw2) {
+    // ---- the other layer's dW: rows h0 .. h0 + 15, columns o0 .. o0 + 15
+    const int rbk = b / f.w2cb, cbk = b - rbk * f.w2cb;
+    const int h0 = 16 * rbk, o0 = 16 * cbk;
+    const float *xcol = f.x2 + min(h0 + r, f.in2 - 1);
+    const float *dcol = f.dy2 + min(o0 + r, f.out2 - 1);
+    tail_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 2
+    for (int m16 = 16 * wave; m16 < f.batch; m16 += 64) {
+      float a[4], bs[4];
+#pragma unroll
+      for (int comp = 0; comp < 4; ++comp) {
+        const int m   = m16 + 4 * q + comp;
+        const bool ok = m < f.batch;
+        const int mc  = ok ? m : f.batch - 1;
+        const float v = xcol[static_cast<size_t>(mc) * f.in2];
+        a[comp]       = ok ? v : 0.0f;
+        bs[comp]      = dcol[static_cast<size_t>(mc) * f.out2];
+      }
+#pragma unroll
+      for (int comp = 0; comp < 4; ++comp) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[comp], bs[comp], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][4 * q + i][r] = acc[i];
+    __syncthreads();
+    const int row = tid >> 4, col = tid & 15;
+    float s = red[0][row][col];
+#pragma unroll
+    for (int v = 1; v < 4; ++v) s += red[v][row][col];
+    if (h0 + row < f.in2 && o0 + col < f.out2) {
+      float *dst = f.dw2 + static_cast<size_t>(h0 + row) * f.out2 + o0 + col;
+      *dst = f.accumulate ? *dst + s : s;
+    }
+    return;
+  }
+  bias_block(f.dy2, f.db2, f.out2, b - f.nw2);
+}
+
 bool small_fc_applies(int M, int N, int K) {
   return K <= 4 * SFC_KC && static_cast<long>(M) * N <= (1L << 18) &&
          static_cast<long>(M) * N * K <= (1L << 24);
@@ -767,6 +970,42 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     return set_error(TDH_ERR_INVALID, "fc_bwd: another layer's gradients need the one-launch kernel");
   if (pool && !(dx && dw && fc_bwd_fuses(in, out, batch) && pool->OH * pool->OW > 0 && in % (pool->OH * pool->OW) == 0))
     return set_error(TDH_ERR_INVALID, "fc_bwd: the pool scatter needs the one-launch kernel");
+  if (dw && (dx || bias_grad) && fc_bwd_fuses(in, out, batch) && out % 4 == 0 &&
+      !(reinterpret_cast<uintptr_t>(dy) & 15) && !(reinterpret_cast<uintptr_t>(w) & 15) &&
+      !(reinterpret_cast<uintptr_t>(dw) & 15) && static_cast<long>(batch) * in < (1L << 30)) {
+    FcBwdMfma f;
+    f.x = x; f.w = w; f.dy = dy;
+    f.xepi.row = EpiRowMajor{dx, in, nullptr, dx_act, 0};
+    if (pool) {
+      f.xepi.pool      = *pool;
+      f.xepi.div_ow    = FastDiv(pool->OW);
+      f.xepi.div_oh    = FastDiv(pool->OH);
+      f.xepi.sample_in = 4 * in;
+    }
+    f.dw = dw; f.db = bias_grad ? db : nullptr;
+    f.batch = batch; f.in = in; f.out = out; f.accumulate = accumulate;
+    f.xcb = ceil_div(in, 16);
+    f.nx  = dx ? ceil_div(ceil_div(batch, 16) * f.xcb, 4) : 0;
+    f.wcg = ceil_div(out, 64);
+    f.nw  = ceil_div(in, 16) * f.wcg;
+    f.ndb = bias_grad ? ceil_div(out, 32) : 0;
+    f.x2 = f.dy2 = nullptr; f.dw2 = f.db2 = nullptr;
+    f.in2 = f.out2 = 1; f.nw2 = f.w2cb = f.ndb2 = 0;
+    double flop = (dx ? 4.0 : 2.0) * batch * in * out;
+    if (also) {
+      f.x2 = also->x; f.dy2 = also->dy; f.dw2 = also->dw; f.db2 = also->db;
+      f.in2 = also->in; f.out2 = also->out;
+      f.w2cb = ceil_div(also->out, 16);
+      f.nw2  = ceil_div(also->in, 16) * f.w2cb;
+      f.ndb2 = also->db ? ceil_div(also->out, 32) : 0;
+      flop += 2.0 * batch * also->in * also->out;
+    }
+    ProfScope prof(also ? (pool ? "fc_bwd_small_pool_two" : "fc_bwd_small_two")
+                        : pool ? "fc_bwd_small_pool" : dx ? "fc_bwd_small" : "fc_dw_db_small", flop, WORK_FLOP);
+    TDH_LAUNCH(fc_bwd_mfma_kernel, dim3(f.nx + f.nw + f.ndb + f.nw2 + f.ndb2), dim3(256), 0, ctx().stream, f);
+    TDH_LAUNCH_CHECK();
+    return TDH_OK;
+  }
   if (dw && (dx || bias_grad) && fc_bwd_fuses(in, out, batch)) {
     FcBwdFused f;
     f.xa = StridedOperand{dy, out, 1, batch};
