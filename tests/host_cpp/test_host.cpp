@@ -456,7 +456,19 @@ static void net_with_batchnorm_and_dropout_vs_oracle() {
     const vec_t b = nn.weights(0, 1);
     for (size_t k = 0; k < b.size(); ++k) EXPECT(std::fabs(b[k] - tdo_net_bias(ref, 0)[k]) <= 4 * 2 * 0.001f);
   }
-  expect_near(nn.weights(1, 2).data(), tdo_net_bn_stat(ref, 1, 0), 6, 1e-4f, "running mean");
+  {
+    // the running mean carries that free bias with it: (1 - momentum) of the bias's wandering
+    // per step on top of the usual bound
+    const size_t nsteps = 2 * ((samples + batch - 1) / batch);
+    const float allowance = (1.0f - 0.999f) * static_cast<float>(nsteps) * (2.0f * nsteps * 0.001f);
+    const vec_t m = nn.weights(1, 2);
+    const float *want = tdo_net_bn_stat(ref, 1, 0);
+    double sq = 0.0;
+    for (size_t k = 0; k < 6; ++k) sq += static_cast<double>(want[k]) * want[k];
+    const float rms = static_cast<float>(std::sqrt(sq / 6.0));
+    for (size_t k = 0; k < 6; ++k)
+      EXPECT(std::fabs(m[k] - want[k]) <= 1e-4f * std::max(std::fabs(want[k]), rms) + allowance);
+  }
   expect_near(nn.weights(1, 3).data(), tdo_net_bn_stat(ref, 1, 1), 6, 1e-4f, "running variance");
   // fit leaves the net in the test phase (network.h:877): running averages, no mask
   vec_t y = nn.predict(inputs[2]);

@@ -777,6 +777,14 @@ def test_net_with_batchnorm_and_dropout_matches_oracle_and_reference_fit(T, O, W
     for which in (0, 1):
         assert net.param_size(1, 2 + which) == 6
         got = net.get_param(1, 2 + which)
+        if which == 0:
+            # the running mean carries the convolution's free bias with it: (1 - momentum) of that
+            # bias's wandering per step on top of the usual bound
+            slack = (1.0 - 0.999) * steps * (2 * steps * opt.alpha)
+            for want in (ref.bn_stat(1, 0), g["bn_dropout.stat0"]):
+                scale = np.maximum(np.abs(want), np.sqrt(np.mean(np.square(want))))
+                assert np.all(np.abs(got - want) <= REL_TOL * scale + slack), "running mean"
+            continue
         assert_close(got, ref.bn_stat(1, which), what=f"running average {which} vs oracle")
         assert_close(got, g[f"bn_dropout.stat{which}"], what=f"running average {which} vs network::fit")
     # net_phase::test: running averages instead of batch moments, dropout is the identity
