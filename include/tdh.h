@@ -305,6 +305,11 @@ int tdh_net_clear_grads(tdh_net *net);
 /* device views valid until the net is destroyed */
 float *tdh_net_param(tdh_net *net, int layer, int which);
 const float *tdh_net_layer_out(const tdh_net *net, int layer);
+/* the gradient with respect to the layer's input as the last step left it, or NULL where
+ * that step never wrote it to memory: with TDH_NET_FUSE_ACT_GRAD the gradient of a folded
+ * activation's output only exists in registers, and the backward kernels of a first
+ * convolution (few input channels, stride 1) in front of a 2x2 / stride-2 max-pool read the
+ * pooled gradient and the argmax records instead of the pool's input gradient */
 const float *tdh_net_layer_dx(const tdh_net *net, int layer);
 const float *tdh_net_layer_grad(const tdh_net *net, int layer, int which);
 const int32_t *tdh_net_layer_argmax(const tdh_net *net, int layer);

@@ -155,10 +155,16 @@ def check_every_layer(net, ref, spec, batch, name, fused, passes=1, cancelling_d
                 assert np.all(err <= 1e-5 * mag), f"{name} layer {i} db: {err.max():.3e} of {mag.min():.3e}"
             else:
                 assert_close(net.layer_grad(i, 1), passes * ref.layer_db(i), what=f"{name} layer {i} db")
-        # the gradient with respect to a layer's input; a folded activation gradient leaves the
-        # gradient of the activation's OUTPUT unwritten (it only ever exists in registers)
-        if i == 0 or not (fused and spec[i - 1][0] == "act" and spec[i - 1][1] in ("tanh", "relu", "sigmoid")):
+        # the gradient with respect to a layer's input. A fusing net leaves two kinds unwritten:
+        # the gradient of a folded activation's OUTPUT (it only ever exists in registers), and
+        # the input gradient of a max-pool behind a first convolution whose backward kernels read
+        # the pooled gradient and the argmax records themselves
+        if net.dx_written(i):
             assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), what=f"{name} layer {i} dX")
+        else:
+            assert fused and i >= 1 and (
+                (spec[i - 1][0] == "act" and spec[i - 1][1] in ("tanh", "relu", "sigmoid")) or
+                (l[0] == "maxpool" and spec[i - 1][0] == "conv")), f"{name} layer {i} dX is missing"
     return flipped
 
 
@@ -487,9 +493,10 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
             assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
             if l[0] == "maxpool":
                 assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64), ref.layer_argmax(i, batch))
-                if i >= 1 and spec[i - 1][0] == "conv":
+                if i >= 1 and spec[i - 1][0] == "conv" and net.dx_written(i):
                     # the gradient routed through the pool (by the pool's kernel, or by the dX
-                    # epilogue of the fully-connected layer behind it)
+                    # epilogue of the fully-connected layer behind it; not written at all where
+                    # the convolution in front reads the pooled gradient itself)
                     assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), REL_TOL, f"layer {i} dX")
             if net.param_size(i, 0):
                 assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
@@ -501,6 +508,69 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
         net.close()
 
 
+@pytest.mark.parametrize("flags", [1, 3])
+@pytest.mark.parametrize("spec,batch,pool_dx_written", [
+    # the CIFAR net's first layers at a small batch; 5x5 window, a second convolution's dX
+    # (relu folded) produces the pooled gradient
+    ([("conv", 32, 32, 3, 5, 32, True), ("maxpool", 32, 32, 32, 2), ("act", "relu"),
+      ("conv", 16, 16, 32, 5, 8, True), ("act", "tanh"), ("fc", 2048, 10)], 12, False),
+    # one input channel, no padding (24x24 outputs), 6 of 32 output channels in use; a
+    # fully-connected layer's dX (tanh folded) produces the pooled gradient
+    ([("conv", 28, 28, 1, 5, 6, False), ("maxpool", 24, 24, 6, 2), ("act", "tanh"), ("fc", 864, 10)], 7, False),
+    # 40 output channels: a second, partial tile of them in dW and a ragged last chunk in dX;
+    # four input channels, 3x3 window
+    ([("conv", 16, 8, 4, 3, 40, True), ("maxpool", 16, 8, 40, 2), ("act", "sigmoid"), ("fc", 1280, 10)], 5, False),
+    # a window without compile-time loops (4x4, no padding: 13x13 outputs would be odd, so 16+3)
+    ([("conv", 19, 11, 2, 4, 9, False), ("maxpool", 16, 8, 9, 2), ("fc", 288, 10)], 3, False),
+    # output width 18 is not a multiple of four: the kernels read a gradient the pool has written
+    ([("conv", 20, 12, 2, 3, 8, False), ("maxpool", 18, 10, 8, 2), ("act", "relu"), ("fc", 360, 10)], 6, True),
+    # an activation between convolution and pool: the pool's kernel runs and folds its gradient
+    # (so that it is the activation's output gradient that stays in registers)
+    ([("conv", 16, 16, 3, 3, 8, True), ("act", "relu"), ("maxpool", 16, 16, 8, 2), ("fc", 512, 10)], 6, False),
+])
+def test_first_conv_reading_its_gradient_through_the_pool_matches_oracle(T, O, W, spec, batch, pool_dx_written, flags):
+    """The backward kernels of a fusing net's first convolution (few input channels, stride 1)
+    with a 2x2 max-pool directly behind it take the pooled gradient and the argmax records and
+    rebuild their operand on the way to LDS; the pool's backward kernel does not run and its
+    input gradient is reported as not written. Two passes without update (gradients add up),
+    then two SGD steps: gradients, input gradient and weights against the oracle."""
+    rng = np.random.default_rng(len(spec) * 17 + batch)
+    net = T.Net(W.build_layers(T, spec), batch, flags)
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for i, l in enumerate(spec):
+        nw, nb, fan_in, _ = W.layer_fans(l)
+        if nw:
+            w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+            b = rng.uniform(-0.5, 0.5, nb).astype(np.float32)
+            net.set_param(i, 0, w); net.set_param(i, 1, b)
+            ref.weight(i)[:] = w; ref.bias(i)[:] = b
+    first = spec[0]
+    x = rng.standard_normal((batch, first[1] * first[2] * first[3])).astype(np.float32)
+    t = rng.uniform(0.1, 0.9, (batch, 10)).astype(np.float32)
+    xd, td = T.to_device(x), T.to_device(t)
+    pool = [i for i, l in enumerate(spec) if l[0] == "maxpool"][0]
+    ref.train_step(O.opt_desc("sgd"), "mse", x, t, do_update=False)
+    for passes in (1, 2):
+        net.train_step(None, "mse", batch, xd, td, do_update=False)
+        assert net.dx_written(pool) == pool_dx_written
+        assert np.array_equal(net.layer_argmax(pool, batch).astype(np.int64), ref.layer_argmax(pool, batch))
+        for i, l in enumerate(spec):
+            if net.param_size(i, 0):
+                assert_close(net.layer_grad(i, 0), passes * ref.layer_dw(i), REL_TOL, f"pass {passes} layer {i} dW")
+                assert_close(net.layer_grad(i, 1), passes * ref.layer_db(i), REL_TOL, f"pass {passes} layer {i} db")
+        assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, f"pass {passes} input gradient")
+    net.clear_grads()
+    opt, ropt = T.opt_desc("sgd"), O.opt_desc("sgd")
+    for step in range(2):
+        net.train_step(opt, "mse", batch, xd, td, do_update=True)
+        ref.train_step(ropt, "mse", x, t, do_update=True)
+        for i, l in enumerate(spec):
+            if net.param_size(i, 0):
+                assert_close(net.get_param(i, 0), ref.weight(i), REL_TOL, f"step {step} layer {i} weights")
+                assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} layer {i} bias")
+    net.close()
+
+
 @pytest.mark.parametrize("spec,batch", [
     # both limits of the one-launch kernel (128 inputs, 64 outputs), relu folded, ragged batch
     ([("fc", 100, 128), ("act", "relu"), ("fc", 128, 64), ("act", "softmax")], 37),
@@ -508,14 +578,17 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
     ([("fc", 30, 10), ("act", "softmax")], 5),
     # 70 inputs: a second, partial block of dX columns; tanh folded
     ([("fc", 50, 70), ("act", "tanh"), ("fc", 70, 3), ("act", "softmax")], 16),
-    # a pool in front: nothing to fold
+    # a pool in front: nothing to fold (five input channels: the convolution's backward kernels
+    # are not those that read the pooled gradient themselves, so that the dX epilogue scatters)
+    ([("conv", 8, 8, 5, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("fc", 64, 10), ("act", "softmax")], 9),
+    # the same with two: the convolution's kernels read the pooled gradient this layer writes
     ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("fc", 64, 10), ("act", "softmax")], 9),
     # too wide for the one-launch kernel: the three separate launches
     ([("fc", 20, 200), ("act", "relu"), ("fc", 200, 10), ("act", "softmax")], 8),
     # nets that end in the fully-connected layer, trained with mse: the same kernel without softmax
     ([("fc", 50, 70), ("act", "tanh"), ("fc", 70, 3)], 16),
     ([("fc", 30, 10)], 5),
-    ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("act", "sigmoid"), ("fc", 64, 64)], 19),
+    ([("conv", 8, 8, 5, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("act", "sigmoid"), ("fc", 64, 64)], 19),
 ])
 @pytest.mark.parametrize("targets", ["one_hot", "soft"])
 def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch, targets):
@@ -585,7 +658,7 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
     ([("fc", 50, 132), ("act", "tanh"), ("fc", 132, 24), ("act", "relu"), ("fc", 24, 3), ("act", "softmax")], 20),
     ([("fc", 50, 130), ("act", "tanh"), ("fc", 130, 24), ("act", "relu"), ("fc", 24, 3), ("act", "softmax")], 20),
     # pool and a folded activation in front
-    ([("conv", 8, 8, 2, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("act", "sigmoid"), ("fc", 64, 12), ("act", "relu"),
+    ([("conv", 8, 8, 5, 3, 4, True), ("maxpool", 8, 8, 4, 2), ("act", "sigmoid"), ("fc", 64, 12), ("act", "relu"),
       ("fc", 12, 10), ("act", "softmax")], 19),
     # 36 hidden units are fine, 35 are not (rows of the first layer's filters are read four at a time)
     ([("fc", 260, 36), ("act", "relu"), ("fc", 36, 10), ("act", "softmax")], 33),
@@ -627,7 +700,10 @@ def test_two_closing_fc_layers_in_one_launch_match_oracle(T, O, W, spec, batch, 
         assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
         assert_close(net.layer_out(i, batch), plain.layer_out(i, batch), REL_TOL, f"layer {i} output, fused vs not")
         if l[0] == "maxpool" and spec[i - 1][0] == "conv":
-            assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), REL_TOL, f"layer {i} dX (through the pool)")
+            for n_ in (net, plain):
+                if n_.dx_written(i):
+                    assert_close(n_.layer_dx(i, batch), ref.layer_dx(i, batch), REL_TOL, f"layer {i} dX (through the pool)")
+            assert plain.dx_written(i)
         if net.param_size(i, 0):
             assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
             assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")
@@ -648,20 +724,20 @@ def test_layers_without_bias_through_the_one_launch_kernels(T, O):
     """No layer has a bias: the last layer's one-launch kernel, the fully-connected backward that
     routes dX through the pool in front, and the convolution kernels against the oracle."""
     def layers(api):
-        return [api.L_conv(8, 8, 2, 3, 4, pad_same=True, has_bias=False), api.L_maxpool(8, 8, 4, 2),
+        return [api.L_conv(8, 8, 5, 3, 4, pad_same=True, has_bias=False), api.L_maxpool(8, 8, 4, 2),
                 api.L_act("relu"), api.L_fc(64, 24, has_bias=False), api.L_act("tanh"),
                 api.L_fc(24, 10, has_bias=False), api.L_act("softmax")]
     batch = 9
     rng = np.random.default_rng(77)
     nets = [T.Net(layers(T), batch, f) for f in (0, T.NET_FUSE_ACT_GRAD)]
     ref = O.OracleNet(layers(O), batch)
-    for i, (nw, fan_in) in {0: (72, 18), 3: (64 * 24, 64), 5: (240, 24)}.items():
+    for i, (nw, fan_in) in {0: (180, 45), 3: (64 * 24, 64), 5: (240, 24)}.items():
         w = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
         for net in nets:
             assert net.param_size(i, 1) == 0
             net.set_param(i, 0, w)
         ref.weight(i)[:] = w
-    x = rng.standard_normal((batch, 128)).astype(np.float32)
+    x = rng.standard_normal((batch, 320)).astype(np.float32)
     t = np.eye(10, dtype=np.float32)[rng.integers(0, 10, batch)]
     ref.train_step(O.opt_desc("sgd"), "ce_multiclass", x, t, do_update=False)
     for net in nets:

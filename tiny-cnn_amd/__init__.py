@@ -566,9 +566,18 @@ class Net:
         n = self.layer_out_size(i)
         return DevBuf.view(lib().tdh_net_layer_out(self.h, i), (batch, n)).numpy()
 
+    def dx_written(self, i):
+        """False when the last step never wrote the gradient with respect to layer i's input:
+        a fusing net folds an activation gradient into the kernel behind it, and lets a first
+        convolution read its output gradient through the max-pool behind it."""
+        return bool(lib().tdh_net_layer_dx(self.h, i))
+
     def layer_dx(self, i, batch):
         n = self.in_size() if i == 0 else self.layer_out_size(i - 1)
-        return DevBuf.view(lib().tdh_net_layer_dx(self.h, i), (batch, n)).numpy()
+        p = lib().tdh_net_layer_dx(self.h, i)
+        if not p:
+            raise RuntimeError(f"layer {i}: the last step did not write this gradient to memory")
+        return DevBuf.view(p, (batch, n)).numpy()
 
     def layer_grad(self, i, which):
         n = self.param_size(i, which)

@@ -219,9 +219,19 @@ bool conv_dw_small_applicable(int batch, int C, int Kc, int H, int W, int OH, in
                               int sh, int sw, int dh, int dw, int ph, int pw);
 size_t conv_dw_small_workspace_bytes(int batch, int C, int Kc, int H, int W, int OH, int OW, int R,
                                      int S, int sh, int sw, int dh, int dw, int ph, int pw);
+// The output gradient of a convolution whose output feeds a 2x2 / stride-2 max-pool, given as
+// what the pool's backward pass would read instead of as the tensor it would write:
+//   dY[img][co][y][x] = argmax[img][co][y/2][x/2] == (co*OH + y)*OW + x ? g[img][co][y/2][x/2] : 0
+struct PoolGather {
+  const float *g        = nullptr;  // [batch][Cout][OH/2][OW/2] gradient of the pooled output
+  const int32_t *argmax = nullptr;  // same shape: flat CHW index of each window's maximum
+};
+// (dy_pool set: dy is not read; the plan must pass conv_dw_small_reads_pooled)
 int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy, float *dw_out,
                       float *db_out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
-                      int dw, int ph, int pw, int accumulate);
+                      int dw, int ph, int pw, int accumulate, const PoolGather *dy_pool = nullptr);
+bool conv_dw_small_reads_pooled(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
+                                int sh, int sw, int dh, int dw, int ph, int pw);
 // the weight-gradient kernel of this layer also produces the bias gradient when asked for both
 bool conv_dw_gives_db(const tdh_conv_desc *d, int batch);
 // norm.hip
@@ -284,9 +294,15 @@ bool conv_fwd_small_applicable(int batch, int C, int Kc, int H, int W, int OH, i
 int conv_fwd_small_run(int batch, int C, int Kc, const float *x, const float *w, const float *bias,
                        float *out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
                        int dw, int ph, int pw, float *act_out, int act_kind, const PoolFuse *pool);
+// dy_pool: the output gradient is given through the max-pool behind the layer (dy is not read
+// and may be null); only where conv_bwd_reads_pooled says so
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
-               const uint8_t *tbl_resident = nullptr, const float *prepacked_dx = nullptr);
+               const uint8_t *tbl_resident = nullptr, const float *prepacked_dx = nullptr,
+               const PoolGather *dy_pool = nullptr);
+// the backward kernels of this layer (the two of a first layer: few input channels, stride 1)
+// can read their output gradient through this 2x2 / stride-2 max-pool over the layer's output
+bool conv_bwd_reads_pooled(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch);
 // true when forward (flip = 0) / dX (flip = 1) of this layer reads packed filters
 bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip);
 bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked);

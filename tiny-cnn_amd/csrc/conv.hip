@@ -228,19 +228,28 @@ constexpr int DXS_CO_CHUNK = DXS_WAVES * DXS_CPW;
 constexpr int DXS_PX       = 4;                      // adjacent pixels per lane
 constexpr int DXS_NT       = 64 * DXS_WAVES;
 constexpr int DXS_MAX_STAGE = 20;                    // staged tile elements per thread and chunk
+constexpr int DXS_MAX_PSTAGE = 8;                    // POOLED: staged pool windows per thread and chunk
 
 struct DxsPlan {
   int tile_rows, bands, gw, trows, tcols;  // gw: pixel groups per row; tile = [trows][tcols]
   FastDiv div_gw, div_tcols, div_tile;
   size_t lds_bytes;
+  // POOLED: the 2x2 pool windows that can touch a tile, [pnr][pnc] per channel
+  int pnr, pnc;
+  FastDiv div_pnc, div_ptile;
+  bool pooled_ok;
 };
 
-// KR, KS: compile-time window (0 = use the run-time g.R, g.S); CIN: input channels computed
-template <int KR, int KS, int CIN>
+// KR, KS: compile-time window (0 = use the run-time g.R, g.S); CIN: input channels computed.
+// POOLED: dY is not in memory but given through the 2x2 / stride-2 max-pool behind the layer.
+// A thread stages pool windows instead of tile elements: one gradient and one argmax record per
+// window, and writes the window's four elements into the tile (the gradient where the record
+// names the element, else zero; windows outside the image give the zero halo).
+template <int KR, int KS, int CIN, bool POOLED>
 __global__ void __launch_bounds__(DXS_NT)
 conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__ w,
                          float *__restrict__ dx, const ConvGeom g, const DxsPlan p,
-                         const ActGrad ag) {
+                         const ActGrad ag, const PoolGather pooled) {
   extern __shared__ __align__(16) float smem[];
   const int R = KR ? KR : g.R, S = KS ? KS : g.S;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -249,7 +258,10 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
   const int tsz = p.trows * p.tcols, rs = R * S;
   const int oy0 = y0 + g.pad_h - (R - 1), ox0 = g.pad_w - (S - 1);
   const int ohw = g.OH * g.OW;
-  const float *dy_img = dy + static_cast<size_t>(img) * g.Kc * ohw;
+  const int pow_ = g.OW >> 1, pohw = (g.OH >> 1) * pow_;
+  const float *dy_img = POOLED ? pooled.g + static_cast<size_t>(img) * g.Kc * pohw
+                               : dy + static_cast<size_t>(img) * g.Kc * ohw;
+  const int32_t *rec_img = POOLED ? pooled.argmax + static_cast<size_t>(img) * g.Kc * pohw : nullptr;
   float *tile = smem;                                                  // [DXS_CO_CHUNK][tsz]
   float4 *wl  = reinterpret_cast<float4 *>(smem + DXS_CO_CHUNK * tsz);  // [DXS_CO_CHUNK][rs]
 
@@ -267,19 +279,56 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
 
   // staging plan, the same for every chunk: element e = tid + DXS_NT*j of the chunk tile ->
   // channel inside the chunk and offset inside that channel's plane (-1: outside the image)
-  float stage[DXS_MAX_STAGE];
-  int soff[DXS_MAX_STAGE], sch[DXS_MAX_STAGE];
+  constexpr int NS = POOLED ? 1 : DXS_MAX_STAGE, NP = POOLED ? DXS_MAX_PSTAGE : 1;
+  float stage[NS];
+  int soff[NS], sch[NS];
+  if (!POOLED) {
 #pragma unroll
-  for (int j = 0; j < DXS_MAX_STAGE; ++j) {
-    const uint32_t e = tid + DXS_NT * j;
-    uint32_t c, rem, r, q;
-    p.div_tile.divmod(e, c, rem);
-    p.div_tcols.divmod(rem, r, q);
-    const int oy = oy0 + static_cast<int>(r), ox = ox0 + static_cast<int>(q);
-    const bool in = static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
-                    static_cast<unsigned>(ox) < static_cast<unsigned>(g.OW);
-    sch[j]  = static_cast<int>(c);
-    soff[j] = in ? static_cast<int>(c) * ohw + oy * g.OW + ox : -1;
+    for (int j = 0; j < NS; ++j) {
+      const uint32_t e = tid + DXS_NT * j;
+      uint32_t c, rem, r, q;
+      p.div_tile.divmod(e, c, rem);
+      p.div_tcols.divmod(rem, r, q);
+      const int oy = oy0 + static_cast<int>(r), ox = ox0 + static_cast<int>(q);
+      const bool in = static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH) &&
+                      static_cast<unsigned>(ox) < static_cast<unsigned>(g.OW);
+      sch[j]  = static_cast<int>(c);
+      soff[j] = in ? static_cast<int>(c) * ohw + oy * g.OW + ox : -1;
+    }
+  }
+  // POOLED: window e = tid + DXS_NT*j of the chunk -> offset in the pooled planes (-1: outside
+  // the image), flat index of its top left element inside the channel, its channel, and where
+  // its four elements lie in LDS (those outside the tile: a word behind the weights that
+  // nobody reads, so that the stores need no branches)
+  float pgrad[NP];
+  int poff[NP], pflat[NP], pch[NP], prec[NP], pat[NP][4];
+  const int nowhere = DXS_CO_CHUNK * tsz + 4 * DXS_CO_CHUNK * rs;
+  if (POOLED) {
+    const int pr0 = oy0 >> 1, pc0 = ox0 >> 1;  // (floor: the tile may start outside the image)
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      const uint32_t e = tid + DXS_NT * j;
+      uint32_t c, rem, i, k;
+      p.div_ptile.divmod(e, c, rem);
+      p.div_pnc.divmod(rem, i, k);
+      const int pr = pr0 + static_cast<int>(i), pc = pc0 + static_cast<int>(k);
+      const bool live = c < static_cast<uint32_t>(DXS_CO_CHUNK);
+      const bool in = live && static_cast<unsigned>(pr) < static_cast<unsigned>(g.OH >> 1) &&
+                      static_cast<unsigned>(pc) < static_cast<unsigned>(pow_);
+      const int r0 = 2 * pr - oy0, q0 = 2 * pc - ox0;  // tile position of the top left element
+      const bool ra = static_cast<unsigned>(r0) < static_cast<unsigned>(p.trows),
+                 rb = static_cast<unsigned>(r0 + 1) < static_cast<unsigned>(p.trows),
+                 qa = static_cast<unsigned>(q0) < static_cast<unsigned>(p.tcols),
+                 qb = static_cast<unsigned>(q0 + 1) < static_cast<unsigned>(p.tcols);
+      poff[j]  = in ? static_cast<int>(c) * pohw + pr * pow_ + pc : -1;
+      pflat[j] = static_cast<int>(c) * ohw + 2 * pr * g.OW + 2 * pc;
+      pch[j]   = static_cast<int>(c);
+      const int at = static_cast<int>(c) * tsz + r0 * p.tcols + q0;
+      pat[j][0] = live && ra && qa ? at : nowhere;
+      pat[j][1] = live && ra && qb ? at + 1 : nowhere;
+      pat[j][2] = live && rb && qa ? at + p.tcols : nowhere;
+      pat[j][3] = live && rb && qb ? at + p.tcols + 1 : nowhere;
+    }
   }
   // The chunk's weights as [c][tap] -> (w[ci=0..3]), taps flipped so that the inner loops walk
   // the tile forwards. The first two per thread travel with the tile (512 cover 8 channels of
@@ -297,10 +346,20 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
   };
   auto fetch = [&](int co0) {
     const int nco     = min(DXS_CO_CHUNK, g.Kc - co0);
-    const float *base = dy_img + co0 * ohw;
+    const float *base = dy_img + co0 * (POOLED ? pohw : ohw);
+    if (POOLED) {
 #pragma unroll
-    for (int j = 0; j < DXS_MAX_STAGE; ++j)
-      stage[j] = (soff[j] >= 0 && sch[j] < nco) ? base[soff[j]] : 0.0f;
+      for (int j = 0; j < NP; ++j) {
+        const bool live = poff[j] >= 0 && pch[j] < nco;
+        pgrad[j] = live ? base[poff[j]] : 0.0f;
+        // the record minus the flat index of the window's top left element: 0, 1, OW or OW+1
+        prec[j] = live ? rec_img[co0 * pohw + poff[j]] - (co0 * ohw + pflat[j]) : -1;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+        stage[j] = (soff[j] >= 0 && sch[j] < nco) ? base[soff[j]] : 0.0f;
+    }
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const int e = tid + DXS_NT * k;
@@ -312,10 +371,20 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
   for (int co0 = 0; co0 < g.Kc; co0 += DXS_CO_CHUNK) {
     const int nco = min(DXS_CO_CHUNK, g.Kc - co0);
     __syncthreads();  // the previous chunk has been consumed
+    if (POOLED) {
 #pragma unroll
-    for (int j = 0; j < DXS_MAX_STAGE; ++j) {
-      const int e = tid + DXS_NT * j;
-      if (e < DXS_CO_CHUNK * tsz) tile[e] = stage[j];
+      for (int j = 0; j < NP; ++j) {
+        smem[pat[j][0]] = prec[j] == 0 ? pgrad[j] : 0.0f;
+        smem[pat[j][1]] = prec[j] == 1 ? pgrad[j] : 0.0f;
+        smem[pat[j][2]] = prec[j] == g.OW ? pgrad[j] : 0.0f;
+        smem[pat[j][3]] = prec[j] == g.OW + 1 ? pgrad[j] : 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NS; ++j) {
+        const int e = tid + DXS_NT * j;
+        if (e < DXS_CO_CHUNK * tsz) tile[e] = stage[j];
+      }
     }
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -410,22 +479,39 @@ static bool small_cin_dx_plan(const ConvGeom &g, DxsPlan &p) {
   p.div_gw    = FastDiv(p.gw);
   p.div_tcols = FastDiv(p.tcols);
   p.div_tile  = FastDiv(tsz);
-  const size_t stage_floats = static_cast<size_t>(DXS_CO_CHUNK) * tsz + 4 * DXS_CO_CHUNK * g.R * g.S;
+  p.pnr       = p.trows / 2 + 1;
+  p.pnc       = p.tcols / 2 + 1;
+  p.div_pnc   = FastDiv(p.pnc);
+  p.div_ptile = FastDiv(p.pnr * p.pnc);
+  p.pooled_ok = DXS_CO_CHUNK * p.pnr * p.pnc <= DXS_MAX_PSTAGE * DXS_NT;
+  // (one more word: where the POOLED kernels store what falls outside the tile)
+  const size_t stage_floats = static_cast<size_t>(DXS_CO_CHUNK) * tsz + 4 * DXS_CO_CHUNK * g.R * g.S + 1;
   const size_t red_floats   = static_cast<size_t>(DXS_WAVES) * DXS_MAX_CIN * 64 * DXS_PX;
   p.lds_bytes = sizeof(float) * std::max(stage_floats, red_floats);
   return p.lds_bytes <= 64 * 1024;
 }
 
-template <int KR, int KS>
+template <int KR, int KS, bool POOLED>
 static void launch_small_cin_dx(const ConvGeom &g, const DxsPlan &p, int batch, const float *dy,
-                                const float *w, float *dx, ActGrad ag) {
+                                const float *w, float *dx, ActGrad ag, PoolGather pooled) {
   const dim3 grid(batch * p.bands), block(DXS_NT);
   switch (KR ? g.C : DXS_MAX_CIN) {
-    case 1: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 1>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
-    case 2: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 2>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
-    case 3: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 3>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
-    default: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 4>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag); break;
+    case 1: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 1, POOLED>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag, pooled); break;
+    case 2: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 2, POOLED>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag, pooled); break;
+    case 3: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 3, POOLED>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag, pooled); break;
+    default: TDH_LAUNCH((conv_dx_small_cin_kernel<KR, KS, 4, POOLED>), grid, block, p.lds_bytes, ctx().stream, dy, w, dx, g, p, ag, pooled); break;
   }
+}
+
+template <bool POOLED>
+static void launch_small_cin_dx_window(const ConvGeom &g, const DxsPlan &p, int batch, const float *dy,
+                                       const float *w, float *dx, ActGrad ag, PoolGather pooled) {
+  if (g.R == 3 && g.S == 3)
+    launch_small_cin_dx<3, 3, POOLED>(g, p, batch, dy, w, dx, ag, pooled);
+  else if (g.R == 5 && g.S == 5)
+    launch_small_cin_dx<5, 5, POOLED>(g, p, batch, dy, w, dx, ag, pooled);
+  else
+    launch_small_cin_dx<0, 0, POOLED>(g, p, batch, dy, w, dx, ag, pooled);
 }
 
 
@@ -554,6 +640,17 @@ static bool dw_small_applies(const tdh_conv_desc *d, const ConvGeom &g, int batc
                                              g.dh, g.dw, g.pad_h, g.pad_w);
 }
 
+bool conv_bwd_reads_pooled(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch) {
+  const ConvGeom g = make_geom(d);
+  DxsPlan dxs;
+  if (!dw_small_applies(d, g, batch) || !small_cin_dx_plan(g, dxs) || !dxs.pooled_ok) return false;
+  if (pool->pool_w != 2 || pool->pool_h != 2 || pool->stride_w != 2 || pool->stride_h != 2 ||
+      pool->in_w != g.OW || pool->in_h != g.OH || pool->in_c != g.Kc || g.OW % 4 != 0 || g.OH % 2 != 0)
+    return false;
+  return conv_dw_small_reads_pooled(batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw, g.dh,
+                                    g.dw, g.pad_h, g.pad_w);
+}
+
 bool conv_dw_gives_db(const tdh_conv_desc *d, int batch) {
   const ConvGeom g = make_geom(d);
   if (dw_small_applies(d, g, batch)) return true;
@@ -625,9 +722,30 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
 
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
-               const uint8_t *tbl_resident, const float *prepacked_dx) {
+               const uint8_t *tbl_resident, const float *prepacked_dx, const PoolGather *dy_pool) {
   const ConvGeom g = make_geom(d);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
+  if (dy_pool) {
+    // only the two first-layer kernels read the gradient this way, and they leave nothing over
+    tdh_pool_desc over{};
+    over.in_w = g.OW; over.in_h = g.OH; over.in_c = g.Kc;
+    over.pool_w = over.pool_h = over.stride_w = over.stride_h = 2;
+    if (!conv_bwd_reads_pooled(d, &over, batch) || !dy_pool->g || !dy_pool->argmax ||
+        (reinterpret_cast<uintptr_t>(dy_pool->g) & 7) || (reinterpret_cast<uintptr_t>(dy_pool->argmax) & 7) ||
+        (db && !dw))
+      return set_error(TDH_ERR_INVALID, "conv2d_bwd: the pooled gradient cannot be read for this layer");
+    DxsPlan dxs;
+    small_cin_dx_plan(g, dxs);
+    if (dx) {
+      ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
+      launch_small_cin_dx_window<true>(g, dxs, batch, nullptr, w, dx, dx_act, *dy_pool);
+      TDH_LAUNCH_CHECK();
+    }
+    if (dw)
+      TDH_TRY(conv_dw_small_run(batch, g.C, g.Kc, x, nullptr, dw, db, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh,
+                                g.sw, g.dh, g.dw, g.pad_h, g.pad_w, accumulate, dy_pool));
+    return TDH_OK;
+  }
   if (dx && prepacked_dx) {
     TDH_TRY(conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 1, dy, w, nullptr, nullptr, dx, g.OH, g.OW, g.H,
                         g.W, g.R - 1 - g.pad_h, g.S - 1 - g.pad_w, dx_act, "conv_dx_s1", prepacked_dx));
@@ -640,12 +758,7 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   DxsPlan dxs;
   if (dx && small_cin_dx_plan(g, dxs)) {
     ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
-    if (g.R == 3 && g.S == 3)
-      launch_small_cin_dx<3, 3>(g, dxs, batch, dy, w_eff, dx, dx_act);
-    else if (g.R == 5 && g.S == 5)
-      launch_small_cin_dx<5, 5>(g, dxs, batch, dy, w_eff, dx, dx_act);
-    else
-      launch_small_cin_dx<0, 0>(g, dxs, batch, dy, w_eff, dx, dx_act);
+    launch_small_cin_dx_window<false>(g, dxs, batch, dy, w_eff, dx, dx_act, PoolGather());
     TDH_LAUNCH_CHECK();
   } else if (dx && g.sh == 1 && g.sw == 1 &&
              conv_s1_applicable(g.R, g.S, batch, g.Kc, g.C, g.OH, g.OW, g.H, g.W,

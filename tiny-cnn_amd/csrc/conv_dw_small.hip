@@ -41,11 +41,18 @@ struct DwSmallArgs {
   int x_floats;         // LDS floats in front of the two dY buffers
   int dy_floats;        // LDS floats of one dY buffer
   FastDiv div_pitch, div_rows_in, div_quads, div_ow;
+  // dY given through a 2x2 max-pool (POOLED kernels): pooled gradient and argmax records
+  const float *pool_g;
+  const int32_t *pool_argmax;
+  FastDiv div_units, div_ow4;  // units of two pooled elements per channel and chunk; per pooled row
 };
 
 // A workgroup walks its band in chunks of rows. The dY rows of the next chunk are loaded into
 // registers while the MFMAs of the current one run, and go to the other of two LDS buffers.
-template <int NT>
+// POOLED: dY is not in memory; a thread loads two adjacent elements of the pooled gradient with
+// their argmax records (half the bytes of the 2x4 block of dY that they stand for) and routes
+// them into that block on the way to LDS. Bands and chunks hold an even number of rows then.
+template <int NT, bool POOLED>
 __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs a) {
   extern __shared__ __align__(16) float lds[];
   float *xs  = lds;
@@ -88,9 +95,29 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
       if (xo[k] >= 0) xs[xo[k]] = xv[k];
   };
   // chunk c of the band: 32 output channels x quads 16-byte pieces, at most DEPTH per thread
+  const int units = quads / 2;  // POOLED: 2x4 blocks of dY per output channel and chunk
   auto load_dy = [&](int c) {
     const int row0     = c * a.chunk;
     const int quads_ok = min(a.chunk, rows_here - row0) * a.OW / 4;
+    if (POOLED) {
+      const int poh = a.OH >> 1, pow_ = a.OW >> 1;
+#pragma unroll
+      for (int k = 0; k < DEPTH / 2; ++k) {
+        const int u = tid + k * 256;
+        dv[k] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (u < 32 * units) {
+          const int m = a.div_units.div(u), r = u - m * units;
+          if (co0 + m < a.Kc && 2 * r < quads_ok) {
+            const int pr = a.div_ow4.div(r), pc = r - pr * (a.OW >> 2);
+            const size_t o = (static_cast<size_t>(img * a.Kc + co0 + m) * poh + ((oy0 + row0) >> 1) + pr) * pow_ + 2 * pc;
+            const float2 g2 = *reinterpret_cast<const float2 *>(a.pool_g + o);
+            const int2 a2   = *reinterpret_cast<const int2 *>(a.pool_argmax + o);
+            dv[k] = floatx4{g2.x, g2.y, __int_as_float(a2.x), __int_as_float(a2.y)};
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int k = 0; k < DEPTH; ++k) {
       const int q = tid + k * 256;
@@ -103,7 +130,29 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
       }
     }
   };
-  auto store_dy = [&](float *buf) {
+  auto store_dy = [&](float *buf, int c) {
+    if (POOLED) {
+      const int row0 = c * a.chunk;
+#pragma unroll
+      for (int k = 0; k < DEPTH / 2; ++k) {
+        const int u = tid + k * 256;
+        if (u < 32 * units) {
+          const int m = a.div_units.div(u), r = u - m * units;
+          const int pr = a.div_ow4.div(r), pc = r - pr * (a.OW >> 2);
+          // flat index of the block's top left element inside the sample, as the records hold it
+          const int at = ((co0 + m) * a.OH + oy0 + row0 + 2 * pr) * a.OW + 4 * pc;
+          const float gx = dv[k][0], gy = dv[k][1];
+          const int ax = __float_as_int(dv[k][2]) - at, ay = __float_as_int(dv[k][3]) - at;
+          float *dst = buf + m * a.dy_pitch + 2 * pr * a.OW + 4 * pc;
+          *reinterpret_cast<floatx4 *>(dst) =
+            floatx4{ax == 0 ? gx : 0.0f, ax == 1 ? gx : 0.0f, ay == 2 ? gy : 0.0f, ay == 3 ? gy : 0.0f};
+          *reinterpret_cast<floatx4 *>(dst + a.OW) =
+            floatx4{ax == a.OW ? gx : 0.0f, ax == a.OW + 1 ? gx : 0.0f, ay == a.OW + 2 ? gy : 0.0f,
+                    ay == a.OW + 3 ? gy : 0.0f};
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int k = 0; k < DEPTH; ++k) {
       const int q = tid + k * 256;
@@ -115,7 +164,7 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
   };
   load_dy(0);
   load_x(tid);
-  store_dy(dys);
+  store_dy(dys, 0);
   store_x();
   for (int e0 = tid + DEPTH * 256; e0 < x_total; e0 += DEPTH * 256) {
     load_x(e0);
@@ -171,7 +220,7 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
         }
       }
     }
-    if (more) store_dy(dys + ((c + 1) & 1) * a.dy_floats);
+    if (more) store_dy(dys + ((c + 1) & 1) * a.dy_floats, c + 1);
     __syncthreads();  // the next chunk is in place; every wave is done with this one
   }
 
@@ -206,8 +255,9 @@ struct DwSmallPlan {
   bool ok;
 };
 
+// even_rows: bands and chunks of an even number of rows (what the POOLED kernels need)
 DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
-                               int sh, int sw, int dh, int dw, int ph, int pw) {
+                               int sh, int sw, int dh, int dw, int ph, int pw, bool even_rows = false) {
   DwSmallPlan p;
   p.ok = false;
   DwSmallArgs &a = p.a;
@@ -218,6 +268,7 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   a.crs = C * R * S;
   p.nt  = ceil_div(a.crs + 1, 32);
   if (p.nt > 3 || OW % 4 != 0 || OH < 1 || batch < 1 || batch > 65535) return p;
+  if (even_rows && (OH % 2 != 0 || OW > 128)) return p;
   a.pitch = (OW - 1) * sw + (S - 1) * dw + 1;
   a.pitch |= 1;  // odd: the taps of one column fall into different LDS banks
   const int co_tiles = ceil_div(Kc, 32);
@@ -229,6 +280,7 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   auto chunk_of = [&](int band) {
     int c = std::max(1, std::min(band, 256 / OW));
     if (c == band && band > 1) c = (band + 1) / 2;
+    if (even_rows) c = std::max(2, c & ~1);
     return c;
   };
   auto lds_floats = [&](int band) {
@@ -242,6 +294,7 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   // compute unit; a band is not made shorter than 256 positions for that
   int best = 0;
   for (int band = OH; band >= 1; --band) {
+    if (even_rows && band % 2 != 0) continue;
     if (lds_floats(band) * sizeof(float) > 72 * 1024) continue;
     best = band;
     if (static_cast<long long>(batch) * ceil_div(OH, band) * co_tiles >= 2LL * cus || band * OW <= 256)
@@ -260,6 +313,10 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   a.div_rows_in = FastDiv(a.rows_in);
   a.div_quads   = FastDiv(a.chunk * OW / 4);
   a.div_ow      = FastDiv(OW);
+  a.pool_g      = nullptr;
+  a.pool_argmax = nullptr;
+  a.div_units   = FastDiv(std::max(1, a.chunk * OW / 8));
+  a.div_ow4     = FastDiv(OW / 4);
   p.lds_bytes = lds_floats(best) * sizeof(float);
   p.grid      = dim3(a.bands, batch, co_tiles);
   if (static_cast<long long>(batch) * a.bands > (1 << 20)) return p;
@@ -267,15 +324,15 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   return p;
 }
 
-template <int NT>
+template <int NT, bool POOLED>
 int launch_dw_small(const DwSmallPlan &p) {
   static bool raised = false;
   if (!raised) {  // more than the 64 KB a kernel may use without asking
-    TDH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_dw_small_kernel<NT>),
+    TDH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_dw_small_kernel<NT, POOLED>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024));
     raised = true;
   }
-  TDH_LAUNCH((conv_dw_small_kernel<NT>), p.grid, dim3(256), p.lds_bytes, ctx().stream, p.a);
+  TDH_LAUNCH((conv_dw_small_kernel<NT, POOLED>), p.grid, dim3(256), p.lds_bytes, ctx().stream, p.a);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
 }
@@ -289,19 +346,39 @@ bool conv_dw_small_applicable(int batch, int C, int Kc, int H, int W, int OH, in
 
 size_t conv_dw_small_workspace_bytes(int batch, int C, int Kc, int H, int W, int OH, int OW, int R,
                                      int S, int sh, int sw, int dh, int dw, int ph, int pw) {
-  const DwSmallPlan p = make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw);
-  if (!p.ok) return 0;
-  const size_t blocks = static_cast<size_t>(batch) * p.a.bands;
-  return ws_align(blocks * Kc * p.a.crs * sizeof(float)) + ws_align(blocks * Kc * sizeof(float));
+  size_t most = 0;
+  for (int even = 0; even < 2; ++even) {  // (a layer may run either kernel)
+    const DwSmallPlan p = make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw, even != 0);
+    if (!p.ok) continue;
+    const size_t blocks = static_cast<size_t>(batch) * p.a.bands;
+    most = std::max(most, ws_align(blocks * Kc * p.a.crs * sizeof(float)) + ws_align(blocks * Kc * sizeof(float)));
+  }
+  return most;
+}
+
+// the kernel can read dY through a 2x2 / stride-2 max-pool over the layer's output: whole 2x4
+// blocks per band and chunk, records that fit an int
+bool conv_dw_small_reads_pooled(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
+                                int sh, int sw, int dh, int dw, int ph, int pw) {
+  const DwSmallPlan p = make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw, true);
+  return p.ok && p.a.band % 2 == 0 && p.a.chunk % 2 == 0 && static_cast<long long>(Kc) * OH * OW < (1LL << 30);
 }
 
 // dw (required) and db (optional) of one layer; both follow `accumulate`.
 int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy, float *dw_out,
                       float *db_out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
-                      int dw, int ph, int pw, int accumulate) {
-  DwSmallPlan p = make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw);
-  if (!p.ok || (reinterpret_cast<uintptr_t>(dy) & 15))
+                      int dw, int ph, int pw, int accumulate, const PoolGather *dy_pool) {
+  DwSmallPlan p = make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw, dy_pool != nullptr);
+  if (dy_pool) {
+    if (!conv_dw_small_reads_pooled(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw) ||
+        !dy_pool->g || !dy_pool->argmax || (reinterpret_cast<uintptr_t>(dy_pool->g) & 7) ||
+        (reinterpret_cast<uintptr_t>(dy_pool->argmax) & 7))
+      return set_error(TDH_ERR_INVALID, "conv_dw_small_run: the pooled gradient cannot be read for this shape");
+    p.a.pool_g      = dy_pool->g;
+    p.a.pool_argmax = dy_pool->argmax;
+  } else if (!p.ok || (reinterpret_cast<uintptr_t>(dy) & 15)) {
     return set_error(TDH_ERR_INVALID, "conv_dw_small_run: shape or alignment not supported");
+  }
   const int blocks = batch * p.a.bands;
   void *pw_ws = nullptr, *pb_ws = nullptr;
   TDH_TRY(ws_take(static_cast<size_t>(blocks) * Kc * p.a.crs * sizeof(float), &pw_ws));
@@ -312,10 +389,18 @@ int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy,
   p.a.partial_db = static_cast<float *>(pb_ws);
   {
     ProfScope prof("conv_dw_small", Kc, p.a.crs + (db_out ? 1 : 0), batch * OH * OW);
-    switch (p.nt) {
-      case 1: TDH_TRY(launch_dw_small<1>(p)); break;
-      case 2: TDH_TRY(launch_dw_small<2>(p)); break;
-      default: TDH_TRY(launch_dw_small<3>(p)); break;
+    if (dy_pool) {
+      switch (p.nt) {
+        case 1: TDH_TRY((launch_dw_small<1, true>(p))); break;
+        case 2: TDH_TRY((launch_dw_small<2, true>(p))); break;
+        default: TDH_TRY((launch_dw_small<3, true>(p))); break;
+      }
+    } else {
+      switch (p.nt) {
+        case 1: TDH_TRY((launch_dw_small<1, false>(p))); break;
+        case 2: TDH_TRY((launch_dw_small<2, false>(p))); break;
+        default: TDH_TRY((launch_dw_small<3, false>(p))); break;
+      }
     }
   }
   EpiRowMajor epi_w{dw_out, p.a.crs, nullptr, ActGrad(), accumulate};

@@ -57,8 +57,12 @@ struct tdh_net {
     hipGraphExec_t exec = nullptr;
     GraphKey key;
     uint64_t last_use = 0;
+    std::vector<uint8_t> dx_unwritten;  // what the captured step leaves in the net's field of that name
   } graphs[kGraphSlots];
   uint64_t graph_clock = 0;
+  // per layer: the last step kept the gradient with respect to this layer's input in registers
+  // or read it through a pool (tdh_net_layer_dx has nothing to show)
+  std::vector<uint8_t> dx_unwritten;
   float mirror_b1_t = 0.0f, mirror_b2_t = 0.0f;  // what the device copy of the powers holds
   size_t scratch = 0;        // largest per-op scratch need; with TDH_NET_GRAPH the sum over the
                              // layers, because branches of the captured step run side by side
@@ -175,6 +179,16 @@ DxTarget dx_target(tdh_net *net, int i) {
     d.dx        = i - 1 == 0 ? net->dx_in : net->layers[i - 2].dout;
   }
   return d;
+}
+
+// Max-pool layer r of a fusing net sits directly behind a first convolution (few input
+// channels, stride 1) whose backward kernels read the pooled gradient and the argmax records
+// themselves: the pool's backward pass does not run and its input gradient is never written.
+bool pool_read_by_conv(tdh_net *net, int r, int batch) {
+  if (!(net->flags & TDH_NET_FUSE_ACT_GRAD) || r < 1) return false;
+  const tdh_net::Layer &conv = net->layers[r - 1];
+  return conv.spec.kind == TDH_L_CONV && !conv.tbl_dev &&
+         conv_bwd_reads_pooled(&conv.spec.conv, &net->layers[r].spec.pool, batch);
 }
 
 // The 2x2 max-pool in front of layer i (behind a folded activation, nothing folded into the pool
@@ -641,6 +655,7 @@ const float *tdh_net_layer_out(const tdh_net *net, int layer) {
 }
 const float *tdh_net_layer_dx(const tdh_net *net, int layer) {
   if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
+  if (static_cast<size_t>(layer) < net->dx_unwritten.size() && net->dx_unwritten[layer]) return nullptr;
   return layer == 0 ? net->dx_in : net->layers[layer - 1].dout;
 }
 const float *tdh_net_layer_grad(const tdh_net *net, int layer, int which) {
@@ -698,6 +713,8 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   int first_bwd        = n - 1;
   int tail_done        = -1;     // this layer already has the gradient of its input
   int pool_done        = -1;     // a max-pool layer whose backward pass the layer behind it did
+  PoolGather through_pool;       // a max-pool layer whose backward pass the convolution in front
+  int through_pool_for = -1;     // does while it reads its output gradient: that convolution
   FcGrads also         = {};     // the closing layer's weight and bias gradients, left to ...
   int also_for         = -1;     // ... this layer's backward launch
   // softmax + cross_entropy_multiclass: one closed-form kernel instead of -t/y followed by
@@ -717,6 +734,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
                              last.dout));
   }
   keep.start();
+  net->dx_unwritten.assign(n, 0);
+  for (int i = 1; i < n; ++i)  // (a folded activation gradient never leaves the registers)
+    net->dx_unwritten[i] = net->layers[i - 1].grad_folded ? 1 : 0;
   for (int i = first_bwd; i >= 0; --i) {
     tdh_net::Layer &L  = net->layers[i];
     const tdh_layer &s = L.spec;
@@ -769,6 +789,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
       case TDH_L_CONV:
         TDH_TRY(ws_begin((forked || as_forked ? 3 : 1) * conv2d_workspace_bytes(&s.conv, batch)));
       {
+        const PoolGather *gp = i == through_pool_for ? &through_pool : nullptr;
         const float *wp = packed && L.wp_dx && conv_uses_packed(&s.conv, batch, 1) ? L.wp_dx : nullptr;
         // the layer that reads this dX next (behind a folded activation) is a max-pool: its
         // backward kernel can add up a split reduction of dX
@@ -779,44 +800,44 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           if (!fork) {
             LeaveSplitSum leave(c, pool_reads);
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1, fold,
-                               L.tbl_dev, wp));
+                               L.tbl_dev, wp, gp));
             break;
           }
           {
             LeaveSplitSum leave(c, pool_reads);
-            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp, gp));
           }
           const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
           {
             StreamSwap on_side(c.side[0]);
             c.defer_reduce = true;
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, db_with_dw ? L.db : nullptr, 1,
-                               ActGrad(), L.tbl_dev));
+                               ActGrad(), L.tbl_dev, nullptr, gp));
             c.defer_reduce = false;
           }
           if (L.b_size && !db_with_dw) {
             StreamSwap on_side(c.side[1]);
             c.defer_rowsum = true;
-            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev, nullptr, gp));
             c.defer_rowsum = false;
           }
         } else if (as_forked) {
           // the launches of the captured, branching step, one after the other
           {
             LeaveSplitSum leave(c, pool_reads);
-            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp));
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp, gp));
           }
           const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
           c.defer_reduce = true;
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, db_with_dw ? L.db : nullptr, 1,
-                             ActGrad(), L.tbl_dev));
+                             ActGrad(), L.tbl_dev, nullptr, gp));
           c.defer_reduce = false;
           if (L.b_size && !db_with_dw)
-            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev));
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev, nullptr, gp));
         } else {
           LeaveSplitSum leave(c, pool_reads);
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
-                             fold, L.tbl_dev, wp));
+                             fold, L.tbl_dev, wp, gp));
         }
       } break;
       case TDH_L_FC:
@@ -845,8 +866,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           // a 2x2 max-pool in front (behind a folded activation, nothing folded into the pool
           // itself): the one-launch kernel's dX epilogue also routes the gradient through it
           PoolScatter through;
-          const int reader = fc_one_launch && fc_bwd_scatters_pool(s.fc_in, s.fc_out, batch)
-                               ? pool_in_front(net, i, &through) : -1;
+          int reader = fc_one_launch && fc_bwd_scatters_pool(s.fc_in, s.fc_out, batch)
+                         ? pool_in_front(net, i, &through) : -1;
+          if (reader >= 0 && pool_read_by_conv(net, reader, batch)) reader = -1;  // (less to write)
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, L.dw,
                          L.b_size ? L.db : nullptr, 1, fold, reader >= 0 ? &through : nullptr,
                          i == also_for ? &also : nullptr));
@@ -855,6 +877,15 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
         break;
       case TDH_L_MAXPOOL:
         if (i == pool_done) break;  // the layer behind has written this layer's dX
+        // a first convolution directly in front reads the pooled gradient and the argmax
+        // records itself: its output gradient, four times their size, is never written
+        if (pool_read_by_conv(net, i, batch)) {
+          TDH_TRY(finish_split_sum());  // (the kernels read a finished gradient)
+          net->dx_unwritten[i] = 1;
+          through_pool = PoolGather{L.dout, L.argmax};
+          through_pool_for = i - 1;
+          break;
+        }
         TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold));
         break;
       case TDH_L_AVEPOOL:
@@ -1013,6 +1044,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
                        hipGetErrorString(e));
     }
     slot->key = key;
+    slot->dx_unwritten = net->dx_unwritten;
     net->mirror_b1_t = net->mirror_b2_t = -1.0f;  // forces the upload below
   }
   // the captured optimizer kernel reads the powers from device memory; bring that copy in
@@ -1023,6 +1055,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   }
   slot->last_use = ++net->graph_clock;
   TDH_HIP(hipGraphLaunch(slot->exec, ctx().stream));
+  net->dx_unwritten = slot->dx_unwritten;
   if (opt && do_update) {
     // advance the host object exactly as the eager path does
     for (int j = 0; j < net->opt_tensors; ++j) {
