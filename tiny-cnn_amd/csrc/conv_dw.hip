@@ -64,6 +64,7 @@ struct DwHaloArgs {
   int dyp;         // channel stride of the staged dY planes (4 mod 32)
   int pwa;         // staged X column 0 is image column x0 - pwa
   FastDiv div_rowchunks, div_oh;
+  FastDiv div_gy, div_gz, div_tiles_x;  // grid y and z, tiles per row: the workgroup's place
 };
 
 // R: filter rows one workgroup covers, RF: filter rows of the window (RF/R workgroups share a
@@ -109,12 +110,16 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     const int total = gridDim.x * gy * gz, per = total >> 3;
     int id = blockIdx.x + gridDim.x * (blockIdx.y + gy * blockIdx.z);
     if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    bz = id % gz;  // filter row fastest, then input-channel block
-    id /= gz;
-    by = id % gy;
-    bx = id / gy;
+    uint32_t rest, q, m;  // filter row fastest, then input-channel block
+    a.div_gz.divmod(static_cast<uint32_t>(id), rest, m);
+    bz = static_cast<int>(m);
+    a.div_gy.divmod(rest, q, m);
+    by = static_cast<int>(m);
+    bx = static_cast<int>(q);
   }
-  const int tx = bx % a.tiles_x, slice = bx / a.tiles_x;
+  uint32_t slice_u, tx_u;
+  a.div_tiles_x.divmod(static_cast<uint32_t>(bx), slice_u, tx_u);
+  const int tx = static_cast<int>(tx_u), slice = static_cast<int>(slice_u);
   const int x0 = tx * TC, co0 = by * BCO;
   const int ci0 = (bz / FYB) * 32, fy0 = (bz % FYB) * R;
   const int hw = a.H * a.W, ohw = a.OH * a.OW;
@@ -124,33 +129,29 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
   const int xc = tid / TPC, xl = tid % TPC;
   int xrel[NXI];            // offset of word i from the chunk's base, or DWH_NEVER
   unsigned long long xkeep = 0; // scalar loads: 4 bits per word, float k lies inside the row
+  // (written without branches: the plan runs once, cold, in front of the first load)
+  const bool stacked = a.TI > 1;
 #pragma unroll
   for (int i = 0; i < NXI; ++i) {
-    xrel[i] = DWH_NEVER;
     const int pe = xl + TPC * i;
-    if (pe < PRQ && ci0 + xc < a.C) {
-      int r = pe / NQ;
-      const int q = pe - r * NQ;
-      const int ix = x0 - a.pwa + 4 * q;
-      unsigned keep = 0;
+    const int r = pe / NQ, q = pe - r * NQ;
+    const int ix = x0 - a.pwa + 4 * q;
+    unsigned keep = 0;
+    if (VEC) {
+      keep = (ix >= 0 && ix + 3 < a.W) ? 15u : 0u;
+    } else {
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (static_cast<unsigned>(ix + k) < static_cast<unsigned>(a.W)) keep |= 1u << k;
-      bool ok = VEC ? keep == 15u : keep != 0u;
-      int base = 0;
-      if (a.TI > 1) {
-        // stacked whole images: the row inside its image is fixed, the chunk only picks images
-        uint32_t il, rr;
-        a.div_oh.divmod(static_cast<uint32_t>(r), il, rr);
-        r = static_cast<int>(rr) + fy0 - a.ph;
-        ok = ok && static_cast<int>(il) < a.TI && static_cast<unsigned>(r) < static_cast<unsigned>(a.H);
-        base = static_cast<int>(il) * chw;
-      }
-      if (ok) {
-        xrel[i] = base + r * a.W + ix;
-        if (!VEC) xkeep |= static_cast<unsigned long long>(keep) << (4 * i);
-      }
+      for (int k = 0; k < 4; ++k) keep |= (static_cast<unsigned>(ix + k) < static_cast<unsigned>(a.W) ? 1u : 0u) << k;
     }
+    // stacked whole images: the row inside its image is fixed, the chunk only picks images
+    uint32_t il, rr;
+    a.div_oh.divmod(static_cast<uint32_t>(r), il, rr);
+    const int rs   = static_cast<int>(rr) + fy0 - a.ph;
+    const bool in  = !stacked || (static_cast<int>(il) < a.TI && static_cast<unsigned>(rs) < static_cast<unsigned>(a.H));
+    const bool ok  = (pe < PRQ) & (ci0 + xc < a.C) & (VEC ? keep == 15u : keep != 0u) & in;
+    const int base = stacked ? static_cast<int>(il) * chw : 0;
+    xrel[i] = ok ? base + (stacked ? rs : r) * a.W + ix : DWH_NEVER;
+    if (!VEC) xkeep |= static_cast<unsigned long long>(ok ? keep : 0u) << (4 * i);
   }
   const float *x_chan = a.x + static_cast<size_t>(ci0 + xc) * hw;
 
@@ -276,29 +277,41 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
     if (chunk > c_begin) __syncthreads();  // everyone is done reading the previous chunk
     stage();
     __syncthreads();
+    // (behind the last chunk the same loads run against empty limits and fetch the zero word:
+    // a step without branches is one block that the compiler can interleave)
     const bool more = chunk + 1 < c_end;
-    if (more) fetch_begin(chunk + 1);
+    fetch_begin(more ? chunk + 1 : chunk);
+    if (!more) xlimit = dylimit = 0;
+    // The fragments of step s+1 are read from LDS before the products of step s are issued,
+    // and the next chunk's global loads between them: with one wave per SIMD nothing else
+    // would cover their latencies.
+    floatx4 av4[2];
+    float bv[2][RPW][4 + S - 1];
+    auto read_fragments = [&](int s, int to) {
+      const int r = s / NG, g = s % NG;
+      av4[to] = *reinterpret_cast<const floatx4 *>(ap + (r << LOG_TC) + 4 * g);
+#pragma unroll
+      for (int fy = 0; fy < RPW; ++fy)
+#pragma unroll
+        for (int k = 0; k < 4 + S - 1; ++k) bv[to][fy][k] = bp[(r + fy) * PITCH + 4 * g + k];
+    };
+    read_fragments(0, 0);
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
-      {
-        const int r = s / NG, g = s % NG;
-        if (more) fetch_part(s);
-        const floatx4 av4 = *reinterpret_cast<const floatx4 *>(ap + (r << LOG_TC) + 4 * g);
-        const float av[4] = {av4.x, av4.y, av4.z, av4.w};
-        float bv[RPW][4 + S - 1];
+      const int cur = s & 1;
+      if (s + 1 < STEPS) read_fragments(s + 1, cur ^ 1);
+      const float av[4] = {av4[cur].x, av4[cur].y, av4[cur].z, av4[cur].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
 #pragma unroll
         for (int fy = 0; fy < RPW; ++fy)
 #pragma unroll
-          for (int k = 0; k < 4 + S - 1; ++k) bv[fy][k] = bp[(r + fy) * PITCH + 4 * g + k];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int fy = 0; fy < RPW; ++fy)
-#pragma unroll
-            for (int fx = 0; fx < S; ++fx)
-              acc[fy * S + fx] =
-                __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[fy][j + fx], acc[fy * S + fx], 0, 0, 0);
+          for (int fx = 0; fx < S; ++fx)
+            acc[fy * S + fx] =
+              __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[cur][fy][j + fx], acc[fy * S + fx], 0, 0, 0);
+        if (j == 0) fetch_part(s);
       }
+      __builtin_amdgcn_sched_barrier(0);  // (the loads stay in the step they were written for)
     }
   }
 
@@ -425,6 +438,9 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
   if (p.lds_bytes > 150 * 1024) return p;
   if (static_cast<long>(a.tiles_x) * p.slices > 65535L * 16) return p;
   p.grid = dim3(a.tiles_x * p.slices, co_blocks, ci_blocks);
+  a.div_gy      = FastDiv(co_blocks);
+  a.div_gz      = FastDiv(ci_blocks);
+  a.div_tiles_x = FastDiv(a.tiles_x);
   p.ok   = true;
   return p;
 }
