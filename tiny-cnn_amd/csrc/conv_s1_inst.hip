@@ -197,29 +197,33 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
   // arithmetic of a load next to it, where a straight-line version computes the addresses of
   // all loads up front and runs out of registers.
   auto mfma_group = [&](int p0, int next_kc0, auto with_loads) {
-#pragma unroll
-    for (int pp = 0; pp < PU; ++pp) {
+    // the fragments of step u + 1 are read from LDS before the products of step u are issued:
+    // TM + TN registers more, and a wave no longer waits out an LDS read at every step
+    float af[2][TM], bf[2][TN];
+    auto read_fragments = [&](int u, int to) {
+      const int pp = u / RS, t = u % RS;
+      const int fy = t / S, fx = t % S;
       const float *inp = in_l + 2 * (p0 + pp) * plane;
       const float *wlp = w_l + 2 * (p0 + pp) * BM + aoff;
 #pragma unroll
-      for (int t = 0; t < RS; ++t) {
-        const int fy = t / S, fx = t % S;
-        if (decltype(with_loads)::value) fetch_part(next_kc0, pp * RS + t);
-        float af[TM], bf[TN];
+      for (int i = 0; i < TM; ++i) af[to][i] = wlp[t * KCH * BM + i * 32];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) af[i] = wlp[t * KCH * BM + i * 32];
+      for (int j = 0; j < TN; ++j) bf[to][j] = inp[boff[j] + fy * PITCH + fx];
+    };
+    read_fragments(0, 0);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bf[j] = inp[boff[j] + fy * PITCH + fx];
+    for (int u = 0; u < PU * RS; ++u) {
+      const int cur = u & 1;
+      if (u + 1 < PU * RS) read_fragments(u + 1, cur ^ 1);
+      if (decltype(with_loads)::value) fetch_part(next_kc0, u);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
-        // Tiles of several accumulator blocks keep the steps apart: LDS reads moved ahead over
-        // many steps cost more registers than two resident workgroups have. A single-block tile
-        // has the registers, and often the CU to itself, so there the reads may run ahead.
-        if (TM * TN > 1) __builtin_amdgcn_sched_barrier(0);
-      }
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+      // (keeps the steps apart: left alone, the compiler moves the LDS reads ahead over many
+      // steps, which costs more registers than two resident workgroups have)
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 

@@ -575,7 +575,7 @@ bool gemm_plan_override(int *cfg, int *splits, int M);
 // Shape-only heuristics (no device queries) so that results are reproducible anywhere.
 inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
   // relative MFMA efficiency of a tile (operand fetches per MFMA, prologue share)
-  static const double kEff[kNumTiles] = {1.00, 0.88, 0.88, 0.72, 0.62, 0.80, 0.50, 0.50, 0.36, 0.84};
+  static const double kEff[kNumTiles] = {1.00, 0.80, 0.80, 0.72, 0.62, 0.80, 0.50, 0.50, 0.36, 0.84};
   const double kSlots = 512.0;  // workgroups of 256 threads the chip runs at full rate
   int best = 0, best_splits = 1;
   double best_cost = 1e300;
@@ -595,10 +595,11 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool allow_split) {
     const double work  = tiles * t.bm * t.bn * static_cast<double>(K);  // padded MACs
     const double waves = tiles * splits / slots;
     const double fill  = waves >= 1.0 ? waves / static_cast<double>(static_cast<long>(waves + 0.999)) : waves;
-    // a workgroup's prologue and epilogue weigh like bm*bn/80 more steps of K: large tiles
-    // lose on short reductions (4096 x 4096 x 256: 64x64 tiles 92 us, 128x128 tiles 108 us)
+    // a workgroup's prologue and epilogue weigh like bm*bn/160 more steps of K: large tiles
+    // lose on short reductions (4096 x 4096 x 256: 128x128 tiles 88 us, 64x64 tiles 91 us,
+    // 128x64 and 64x128 tiles 101-103 us)
     // (unsplit products only: split ones keep every workgroup resident at once)
-    const double eff = splits > 1 ? kEff[c] : kEff[c] * K / (K + t.bm * t.bn / 80.0);
+    const double eff = splits > 1 ? kEff[c] : kEff[c] * K / (K + t.bm * t.bn / 160.0);
     double cost = work / (eff * (fill > 1.0 ? 1.0 : fill));
     if (splits > 1) cost += 2.0 * tiles * t.bm * t.bn * splits * 64.0;  // partial tile traffic
     if (cost < best_cost) {
