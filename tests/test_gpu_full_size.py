@@ -55,6 +55,33 @@ def test_config2_conv_backward_full_size(T, W):
     assert np.array_equal(db2.numpy(), 2 * dbh)
 
 
+@pytest.mark.parametrize("bs,ni,no", [
+    (37, 4100, 2050),    # no tile of the kernel is whole in either direction; odd batch
+    (8, 4096, 2048),     # exactly 256 workgroups; one group of loads
+    (130, 2052, 4098),   # a tail of two samples behind eight full groups
+])
+def test_large_fc_weight_gradient_from_memory_fragments(T, bs, ni, no):
+    """dW of a fully-connected layer with at least eight million weights runs on a kernel that
+    feeds the matrix cores from memory (no LDS): against float64, stored and accumulated on top
+    of a previous value, with dX and db of the same call."""
+    rng = np.random.default_rng(bs * 7 + ni)
+    x = rng.uniform(-1, 1, (bs, ni)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, ni * no).astype(np.float32)
+    dy = rng.standard_normal((bs, no)).astype(np.float32)
+    before = rng.standard_normal(ni * no).astype(np.float32)
+    xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+    dx, dw, db = T.DevBuf((bs, ni)), T.DevBuf((ni * no,)), T.DevBuf((no,))
+    T.fc_bwd(ni, no, True, bs, xd, wd, dyd, dx, dw, db)
+    want = x.astype(np.float64).T @ dy.astype(np.float64)
+    assert_close(dw.numpy().reshape(ni, no), want, what="dw")
+    assert_close(dx.numpy(), dy.astype(np.float64) @ w.reshape(ni, no).astype(np.float64).T, what="dx")
+    assert_close(db.numpy(), dy.astype(np.float64).sum(0), what="db")
+    dw2, db2 = T.to_device(before), T.DevBuf((no,), zero=True)
+    T.fc_bwd(ni, no, True, bs, xd, wd, dyd, dx, dw2, db2, accumulate=True)
+    # (bit for bit: the same sums, added to the previous value at the end)
+    assert np.array_equal(dw2.numpy(), before + dw.numpy())
+
+
 def test_config3_fc_backward_adam_full_size(T, O, W):
     """configs[2]: batch 256, 4096 -> 4096, tanh, Adam on W and b."""
     x, w, b, dy = W.fc_bwd_case()

@@ -6,6 +6,7 @@
 // dW is reduced over the batch inside the GEMM (K spans the samples) instead of being stored
 // per sample and merged afterwards (fully_connected_op_internal.h:54-60, node.h:89-103).
 #include <cfloat>
+#include <cstdlib>
 #include <type_traits>
 
 #include "gemm_mfma.h"
@@ -962,6 +963,160 @@ int fc_fwd(int in, int out, int has_bias, int batch, const float *x, const float
                                               "fc_fwd_splitk_reduce");
 }
 
+// ---- dW of a large fully-connected layer, operands straight from memory
+//
+//   dW[i][o] (+)= sum_b X[b][i] * dY[b][o]        (fully_connected_op_internal.h:57-64)
+//
+// Both operands have the reduction index (the sample) as their slow one, so the fragment of a
+// v_mfma_f32_32x32x2_f32 (lane = (column l%32, sample l/32)) is a coalesced read of a row: no
+// LDS, no barrier. A lane reads four consecutive inputs and two consecutive outputs of its
+// sample; component c of the first feeds the accumulator blocks whose 32 rows stand for the
+// inputs 4 r + c, component d of the second those whose columns stand for the outputs 2 n + d.
+// A wave so owns 128 inputs x 64 outputs (eight blocks, 128 accumulator registers) with six
+// loaded registers per eight MFMAs; four sample pairs are loaded as a group while the group
+// before is multiplied. The reduction is as short as the batch, so a tile is prologue,
+// products and a 32 KB store, and the chip holds every workgroup of a 4096 x 4096 layer at
+// once (two waves per SIMD).
+constexpr int FDW_WM = 2, FDW_WN = 2;     // waves of a workgroup along the two
+constexpr int FDW_DEPTH = 4;              // sample pairs per group of loads
+
+struct FcDwDirect {
+  const float *x, *dy;
+  float *dw;
+  int batch, in, out, accumulate;
+};
+
+typedef float fdw_x16 __attribute__((ext_vector_type(16)));
+
+// CA, CB: consecutive inputs and outputs a lane reads. Measured on 4096 x 4096 x 256: 4 x 2
+// (two waves per SIMD) 80 us, 4 x 4 (one wave per SIMD) 80 us, 2 x 2 (four waves) 93 us.
+template <int CA, int CB>
+__global__ void __launch_bounds__(64 * FDW_WM * FDW_WN) __attribute__((amdgpu_waves_per_eu(CA * CB > 8 ? 1 : CA * CB > 4 ? 2 : 4, 8)))
+fc_dw_direct_kernel(const FcDwDirect f) {
+  constexpr int FDW_TM = 32 * CA, FDW_TN = 32 * CB;
+  typedef float avec __attribute__((ext_vector_type(CA)));
+  typedef float bvec __attribute__((ext_vector_type(CB)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  // Workgroups go to the eight XCDs (each with its own L2) round-robin in launch order. Each
+  // XCD gets a compact block of the tile grid (a quarter of the rows x half of the columns
+  // where the grid divides so, else a run of consecutive tiles), so that the panels its
+  // workgroups read together fit its L2.
+  int bx, by;
+  {
+    const int gx = gridDim.x, gy = gridDim.y;
+    const int id = blockIdx.x + gx * blockIdx.y, total = gx * gy;
+    const int xcd = id & 7, seq = id >> 3;
+    if (gx % 2 == 0 && gy % 4 == 0) {
+      const int hx = gx >> 1, qy = gy >> 2;
+      bx = (xcd & 1) * hx + seq % hx;
+      by = (xcd >> 1) * qy + seq / hx;
+    } else {
+      const int per = total >> 3;
+      const int at  = id < (per << 3) ? xcd * per + seq : id;
+      bx = at % gx;
+      by = at / gx;
+    }
+  }
+  const int i0 = (by * FDW_WM + (wave % FDW_WM)) * FDW_TM;
+  const int o0 = (bx * FDW_WN + (wave / FDW_WM)) * FDW_TN;
+  // (in is a multiple of four and out of two: a lane's inputs and outputs exist all or not at
+  // all; what does not exist is read from column 0 and never stored)
+  // (offsets in 32 bits on top of the tensors' uniform base pointers)
+  const bool a_ok = i0 + CA * m < f.in, b_ok = o0 + CB * m < f.out;
+  const unsigned acol = a_ok ? i0 + CA * m : 0, bcol = b_ok ? o0 + CB * m : 0;
+
+  fdw_x16 acc[CA][CB];
+#pragma unroll
+  for (int c = 0; c < CA; ++c)
+#pragma unroll
+    for (int d = 0; d < CB; ++d)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[c][d][r] = 0.0f;
+
+  avec ra[2][FDW_DEPTH];
+  bvec rb[2][FDW_DEPTH];
+  auto load = [&](int k0, auto to) {
+    constexpr int T = decltype(to)::value;
+#pragma unroll
+    for (int j = 0; j < FDW_DEPTH; ++j) {
+      const int kk = min(k0 + 2 * j + h, f.batch - 1);
+      ra[T][j] = *reinterpret_cast<const avec *>(f.x + (static_cast<unsigned>(kk) * f.in + acol));
+      rb[T][j] = *reinterpret_cast<const bvec *>(f.dy + (static_cast<unsigned>(kk) * f.out + bcol));
+    }
+  };
+  // (the zeros of samples past the batch go in here, not where the loads are issued: a select
+  // there would wait for the load it follows; a zero on one side is enough)
+  auto products = [&](int k0, auto from) {
+    constexpr int T = decltype(from)::value;
+#pragma unroll
+    for (int j = 0; j < FDW_DEPTH; ++j) {
+      const bool on    = k0 + 2 * j + h < f.batch;
+      float a[CA];
+#pragma unroll
+      for (int c = 0; c < CA; ++c) a[c] = on ? ra[T][j][c] : 0.0f;
+      float b[CB];
+#pragma unroll
+      for (int d = 0; d < CB; ++d) b[d] = rb[T][j][d];
+#pragma unroll
+      for (int c = 0; c < CA; ++c)
+#pragma unroll
+        for (int d = 0; d < CB; ++d)
+          acc[c][d] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c], b[d], acc[c][d], 0, 0, 0);
+    }
+  };
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
+  constexpr int GROUP = 2 * FDW_DEPTH;  // samples per group
+  // (a group past the batch is clamped reads and products with zeros; the scheduling
+  // barriers keep a group's loads in front of the products they run beside: left alone, the
+  // compiler sinks each load to its first use)
+  load(0, Buf0());
+#pragma unroll 1
+  for (int k0 = 0; k0 < f.batch; k0 += 2 * GROUP) {
+    load(k0 + GROUP, Buf1());
+    __builtin_amdgcn_sched_barrier(0);
+    products(k0, Buf0());
+    __builtin_amdgcn_sched_barrier(0);
+    load(k0 + 2 * GROUP, Buf0());
+    __builtin_amdgcn_sched_barrier(0);
+    products(k0 + GROUP, Buf1());
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // reg r of lane l of block (c, d): input i0 + CA*(8*(r/4) + 4*(l/32) + r%4) + c, output
+  // o0 + 2*(l%32) + d; the two blocks d leave as one 8-byte store
+  if (!b_ok) return;
+  float *out = f.dw + o0 + CB * m;
+#pragma unroll
+  for (int c = 0; c < CA; ++c)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = i0 + CA * (8 * (r >> 2) + 4 * h + (r & 3)) + c;
+      if (i >= f.in) continue;
+      bvec *dst = reinterpret_cast<bvec *>(out + static_cast<size_t>(i) * f.out);
+      bvec v;
+#pragma unroll
+      for (int d = 0; d < CB; ++d) v[d] = acc[c][d][r];
+      if (f.accumulate) {
+        const bvec old = *dst;
+#pragma unroll
+        for (int d = 0; d < CB; ++d) v[d] = old[d] + v[d];
+      }
+      *dst = v;
+    }
+}
+
+// the layer is large enough for every compute unit to get a workgroup of that kernel, and its
+// rows allow the 16- and 8-byte reads
+static bool fc_dw_direct_applies(int in, int out, int batch, const float *x, const float *dy, const float *dw) {
+  const long wgs = static_cast<long>(ceil_div(in, 128 * FDW_WM)) * ceil_div(out, 64 * FDW_WN);
+  return in % 4 == 0 && out % 2 == 0 && batch >= 2 && wgs >= 256 && wgs <= 65535L * 16 &&
+         static_cast<long>(batch) * std::max(in, out) < (1L << 30) &&
+         !(reinterpret_cast<uintptr_t>(x) & 15) && !(reinterpret_cast<uintptr_t>(dy) & 7) &&
+         !(reinterpret_cast<uintptr_t>(dw) & 7);
+}
+
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
            const PoolScatter *pool, const FcGrads *also) {
@@ -1062,9 +1217,15 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     StridedOperand A{x, 1, in, in};      // X[k][m], m contiguous
     StridedOperand B{dy, 1, out, out};   // dY[k][n], n contiguous
     EpiRowMajor epi{dw, out, nullptr, ActGrad(), accumulate};
-    if (small_fc_applies(in, out, batch))
+    if (small_fc_applies(in, out, batch)) {
       TDH_TRY(launch_small_fc(A, B, epi, in, out, batch, "fc_dw_small"));
-    else
+    } else if (fc_dw_direct_applies(in, out, batch, x, dy, dw)) {
+      ProfScope prof("fc_dw_direct", in, out, batch);
+      const FcDwDirect f{x, dy, dw, batch, in, out, accumulate};
+      TDH_LAUNCH((fc_dw_direct_kernel<4, 2>), dim3(ceil_div(out, 64 * FDW_WN), ceil_div(in, 128 * FDW_WM)),
+                 dim3(64 * FDW_WM * FDW_WN), 0, ctx().stream, f);
+      TDH_LAUNCH_CHECK();
+    } else
       TDH_TRY((launch_gemm<false, false, true, true>(A, B, epi, in, out, batch, true, "fc_dw_gemm",
                                                    "fc_dw_splitk_reduce")));
   }
