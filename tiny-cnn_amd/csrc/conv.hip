@@ -465,6 +465,249 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
   }
 }
 
+// dX of a first convolution (stride 1, 3x3 or 5x5, Cin*S <= 16, rows of 16, 32 or 64 outputs)
+// on the matrix cores, in two steps. For an input row y,
+//   D[c][(ci,fx)] = sum over (co, fy) of dY[co][y + pad - (R-1) + fy][c] * wflip[co][ci][fy][fx]
+// is a product with the dY columns c as rows (blocks of 16), Cin*S <= 16 columns and the output
+// channels x filter rows as the reduction (v_mfma_f32_16x16x4_f32: the A operand is one LDS
+// read of the staged rows of dY, which need no halo columns, the B operand one LDS read per
+// step and eight channels), and
+//   dX[ci][y][x] = sum over fx of D[x + fx + pad - (S-1)][(ci,fx)]
+// is gathered out of LDS at the end, added in filter-column order. A workgroup owns a band of
+// rows of one image and stages 32 output channels of it at once; its four waves split the rows,
+// so nothing is added across waves. Every thread stages one position (a pool window, or four
+// adjacent elements) of up to 16 channels with all loads in flight together.
+//
+// The geometry is a template argument (NMB blocks of 16 columns in a row, so 16/NMB rows a
+// band): every LDS offset of the product loop is then an immediate of its instruction. With
+// run-time offsets the loop took 7 us instead of 2: forty address additions per eight
+// channels, branches around reads that a condition guarded, and accumulators moved between
+// register files. Nothing that is loaded stands under a condition either: a load under a
+// condition becomes a branch with a wait behind it (sixteen trips to memory one after the
+// other, 6.5 us); what must not be used is read from a valid place and dropped when stored.
+constexpr int DXM_NT    = 256;
+constexpr int DXM_WAVES = 4;
+constexpr int DXM_MCH   = 32;  // output channels staged at a time
+constexpr int DXM_MAXCH = 16;  // channels a thread stages (of DXM_MCH)
+constexpr int DXM_WREG  = 13;  // filter values a thread stages per chunk (32 channels x 4 x 25 / 256)
+
+template <int KR, int NMB, bool POOLED>
+struct DxmGeom {
+  static constexpr int OW        = 16 * NMB;
+  static constexpr int RPW       = 4 / NMB;            // rows of the band a wave owns
+  static constexpr int TILE_ROWS = DXM_WAVES * RPW;
+  static constexpr int TROWS     = TILE_ROWS + KR - 1;
+  // floats per staged channel: the rows, a spare word for stores that fall outside the tile,
+  // padded to 16 (mod 32) so that four channels' rows lie in different banks
+  static constexpr int PLANE   = ((TROWS * OW + 1 + 15) / 32) * 32 + 16;
+  static constexpr int PER_ROW = POOLED ? OW / 2 : OW / 4;  // staging positions per row of them
+  static constexpr int NPOS    = (POOLED ? TROWS / 2 + 1 : TROWS) * PER_ROW;
+  static constexpr int GROUPS  = DXM_NT / NPOS;
+  static constexpr int CPT     = (DXM_MCH + GROUPS - 1) / GROUPS;  // channels per thread
+  static constexpr int WROW    = 4 * KR * KR;          // staged filter floats per output channel
+  static constexpr int WL      = DXM_MCH * WROW;
+  static constexpr int GATHER  = DXM_WAVES * RPW * OW * 17;
+  static constexpr int STAGE   = DXM_MCH * PLANE + WL;
+  static constexpr int LDS_FLOATS = STAGE > GATHER ? STAGE : GATHER;
+  static constexpr bool FITS = GROUPS >= 1 && CPT <= DXM_MAXCH && LDS_FLOATS * 4 <= 64 * 1024;
+};
+
+template <int KR, int KS, int NMB, bool POOLED>
+__global__ void __launch_bounds__(DXM_NT)
+conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict__ w, float *__restrict__ dx,
+                          const ConvGeom g, const ActGrad ag, const PoolGather pooled) {
+  using G = DxmGeom<KR, NMB, POOLED>;
+  extern __shared__ __align__(16) float smem[];
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  constexpr int RS = KR * KS, NJ = 2 * KR;  // step j: filter row j/2, channels 4*(j%2) + (0..3) of eight
+  constexpr int OW = G::OW, PLANE = G::PLANE;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int mr = lane & 15, mq = lane >> 4;
+  const int bands = (g.H + G::TILE_ROWS - 1) / G::TILE_ROWS;
+  const int img = blockIdx.x / bands;
+  const int y0  = (blockIdx.x - img * bands) * G::TILE_ROWS;
+  const int oy0 = y0 + g.pad_h - (KR - 1), ox0 = g.pad_w - (KS - 1);
+  const int ohw = g.OH * OW, pohw = (g.OH >> 1) * (OW / 2);
+  float *wl = smem + DXM_MCH * PLANE;  // the chunk's filters [co][ci (4)][tap]
+
+  // ---- this thread's staging position: the same for every channel it stages
+  const int grp = tid / G::NPOS, pos = tid - grp * G::NPOS;
+  const int pi = pos / G::PER_ROW, pk = pos - pi * G::PER_ROW;
+  const bool stager = grp < G::GROUPS;
+  int src = -1;   // offset inside a channel's plane in memory, or -1
+  int flat = 0;   // POOLED: flat index of the window's top left element
+  int at[4] = {PLANE - 1, PLANE - 1, PLANE - 1, PLANE - 1};  // offsets inside a staged plane
+  if (POOLED) {
+    const int pr = (oy0 >> 1) + pi;  // (floor: the band's tile may start above the image)
+    if (stager && static_cast<unsigned>(pr) < static_cast<unsigned>(g.OH >> 1)) src = pr * (OW / 2) + pk;
+    flat = 2 * pr * OW + 2 * pk;
+    const int r0 = 2 * pr - oy0;
+    if (static_cast<unsigned>(r0) < static_cast<unsigned>(G::TROWS)) {
+      at[0] = r0 * OW + 2 * pk;
+      at[1] = at[0] + 1;
+    }
+    if (static_cast<unsigned>(r0 + 1) < static_cast<unsigned>(G::TROWS)) {
+      at[2] = (r0 + 1) * OW + 2 * pk;
+      at[3] = at[2] + 1;
+    }
+  } else {
+    const int oy = oy0 + pi;
+    if (stager && static_cast<unsigned>(oy) < static_cast<unsigned>(g.OH)) src = oy * OW + 4 * pk;
+    at[0] = pi * OW + 4 * pk;
+  }
+  const float *dy_img = POOLED ? pooled.g + static_cast<size_t>(img) * g.Kc * pohw
+                               : dy + static_cast<size_t>(img) * g.Kc * ohw;
+  const int32_t *rec_img = POOLED ? pooled.argmax + static_cast<size_t>(img) * g.Kc * pohw : nullptr;
+  const int chan = POOLED ? pohw : ohw;  // floats per channel in memory
+
+  // ---- block b of this wave: row wv*RPW + b/NMB of the band, columns 16*(b%NMB)..+15
+  f4 dacc[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) dacc[b] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+  // B column of this lane: (ci, fx) = (mr / S, mr % S); the filter is staged as it lies in
+  // memory and read flipped. A lane whose column stands for no input channel reads something
+  // valid: its column of D is never gathered, and columns do not mix.
+  const int ci_n = min(mr / KS, 3), fx_n = mr % KS;
+  const float *bbase = wl + (mq * 4 + ci_n) * RS + (RS - 1 - fx_n);
+  const float *abase = smem + mq * PLANE + wv * (G::RPW * OW) + mr;
+  const int crs      = g.C * RS;
+
+  for (int co0 = 0; co0 < g.Kc; co0 += DXM_MCH) {
+    // ---- everything this chunk needs from memory, asked for together
+    float sv[POOLED ? DXM_MAXCH : 1];
+    int srec[POOLED ? DXM_MAXCH : 1];
+    f4 sq[POOLED ? 1 : DXM_MAXCH];
+#pragma unroll
+    for (int jj = 0; jj < G::CPT; ++jj) {
+      const int c = grp + G::GROUPS * jj;
+      const bool live = src >= 0 && c < DXM_MCH && co0 + c < g.Kc;
+      const int off = live ? (co0 + c) * chan + src : 0;
+      if (POOLED) {
+        sv[jj]   = dy_img[off];
+        srec[jj] = rec_img[off];
+      } else {
+        sq[jj] = *reinterpret_cast<const f4 *>(dy_img + off);
+      }
+    }
+    float wreg[DXM_WREG];
+    const int nw = min(DXM_MCH, g.Kc - co0) * crs;
+#pragma unroll
+    for (int k = 0; k < DXM_WREG; ++k) wreg[k] = w[static_cast<size_t>(co0) * crs + min(tid + DXM_NT * k, nw - 1)];
+    if (co0 > 0) __syncthreads();  // the previous chunk has been consumed
+    // filters: element e = (co, ci, tap) of memory goes to [co][ci][tap] with four ci slots
+#pragma unroll
+    for (int k = 0; k < DXM_WREG; ++k) {
+      const int e = tid + DXM_NT * k;
+      if (e < DXM_MCH * crs) {
+        const int co = e / crs, rest = e - co * crs;
+        const int ci = rest / RS, tap = rest - ci * RS;
+        wl[(co * 4 + ci) * RS + tap] = e < nw ? wreg[k] : 0.0f;
+      }
+    }
+    if (stager) {
+#pragma unroll
+      for (int jj = 0; jj < G::CPT; ++jj) {
+        const int c = grp + G::GROUPS * jj;
+        if (c >= DXM_MCH) break;
+        float *plane = smem + c * PLANE;
+        const bool live = src >= 0 && co0 + c < g.Kc;
+        if (POOLED) {
+          // the record minus the flat index of the window's top left element: 0, 1, OW or OW+1
+          const int where = live ? srec[jj] - ((co0 + c) * ohw + flat) : -1;
+          plane[at[0]] = where == 0 ? sv[jj] : 0.0f;
+          plane[at[1]] = where == 1 ? sv[jj] : 0.0f;
+          plane[at[2]] = where == OW ? sv[jj] : 0.0f;
+          plane[at[3]] = where == OW + 1 ? sv[jj] : 0.0f;
+        } else {
+          *reinterpret_cast<f4 *>(plane + at[0]) = live ? sq[jj] : f4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+      }
+    }
+    __syncthreads();
+    // ---- products: eight staged channels a round, the four blocks of the wave side by side
+#pragma unroll
+    for (int sub = 0; sub < DXM_MCH / 8; ++sub) {
+      if (co0 + 8 * sub >= g.Kc) break;
+      float breg[NJ];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) breg[j] = bbase[(8 * sub + 4 * (j & 1)) * G::WROW - (j >> 1) * KS];
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          dacc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+            abase[(8 * sub + 4 * (j & 1)) * PLANE + ((b / NMB) + (j >> 1)) * OW + 16 * (b % NMB)], breg[j], dacc[b], 0,
+            0, 0);
+    }
+  }
+
+  // ---- D -> T[row of the wave][dY column][17] (reg i of lane l: column 4*(l/16) + i of the
+  //      block, entry l%16), then an output is S reads of it
+  __syncthreads();
+  float *T = smem + wv * (G::RPW * OW * 17);
+#pragma unroll
+  for (int b = 0; b < 4; ++b)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) T[((b / NMB) * OW + 16 * (b % NMB) + 4 * mq + i) * 17 + mr] = dacc[b][i];
+  __syncthreads();
+  const size_t img_off = static_cast<size_t>(img) * g.C * g.H * g.W;
+#pragma unroll
+  for (int u = 0; u < G::RPW; ++u) {
+    const int y = y0 + wv * G::RPW + u;
+    if (y >= g.H) break;
+    for (int e = lane; e < g.C * g.W; e += 64) {
+      uint32_t ci, x;
+      g.div_w.divmod(e, ci, x);
+      float v = 0.0f;
+#pragma unroll
+      for (int fx = 0; fx < KS; ++fx) {
+        const int d = static_cast<int>(x) + fx + ox0;  // dY column
+        if (static_cast<unsigned>(d) < static_cast<unsigned>(OW)) v += T[(u * OW + d) * 17 + ci * KS + fx];
+      }
+      const size_t idx = img_off + (static_cast<size_t>(ci) * g.H + y) * g.W + x;
+      if (ag.kind != TDH_ACT_NONE) v *= act_grad_factor(ag.kind, ag.y[idx]);
+      dx[idx] = v;
+    }
+  }
+}
+
+// the launch of the instance for this geometry, or false when there is none
+template <int KR, int NMB, bool POOLED>
+static bool launch_first_dx_mfma_inst(const ConvGeom &g, int batch, const float *dy, const float *w, float *dx,
+                                      ActGrad ag, PoolGather pooled, bool only_ask) {
+  using G = DxmGeom<KR, NMB, POOLED>;
+  if constexpr (!G::FITS) {
+    return false;
+  } else {
+    if (g.H < G::TILE_ROWS) return false;
+    if (only_ask) return true;
+    const int bands = ceil_div(g.H, G::TILE_ROWS);
+    TDH_LAUNCH((conv_dx_first_mfma_kernel<KR, KR, NMB, POOLED>), dim3(batch * bands), dim3(DXM_NT),
+               sizeof(float) * G::LDS_FLOATS, ctx().stream, dy, w, dx, g, ag, pooled);
+    return true;
+  }
+}
+
+// Launches the matrix-core kernel where it applies (only_ask: tells whether it would) and
+// returns whether it does.
+template <bool POOLED>
+static bool first_dx_mfma(const ConvGeom &g, int batch, const float *dy, const float *w, float *dx, ActGrad ag,
+                          PoolGather pooled, bool only_ask) {
+  if (g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1 || g.R != g.S || (g.R != 3 && g.R != 5)) return false;
+  if (g.C * g.S > 16 || g.C > 4 || (POOLED && g.OH % 2 != 0)) return false;
+  if (static_cast<long>(g.Kc) * g.OH * g.OW >= (1L << 30) || DXM_MCH * g.C * g.R * g.S > DXM_WREG * DXM_NT) return false;
+  if (!only_ask && !POOLED && (reinterpret_cast<uintptr_t>(dy) & 15)) return false;
+#define TDH_DXM(KR_, NMB_) launch_first_dx_mfma_inst<KR_, NMB_, POOLED>(g, batch, dy, w, dx, ag, pooled, only_ask)
+  switch (g.OW) {
+    case 16: return g.R == 3 ? TDH_DXM(3, 1) : TDH_DXM(5, 1);
+    case 32: return g.R == 3 ? TDH_DXM(3, 2) : TDH_DXM(5, 2);
+    case 64: return g.R == 3 ? TDH_DXM(3, 4) : TDH_DXM(5, 4);
+    default: return false;
+  }
+#undef TDH_DXM
+}
+
 // true when the direct kernel applies; fills the launch geometry
 static bool small_cin_dx_plan(const ConvGeom &g, DxsPlan &p) {
   if (g.C > DXS_MAX_CIN || g.sh != 1 || g.sw != 1) return false;
@@ -643,7 +886,9 @@ static bool dw_small_applies(const tdh_conv_desc *d, const ConvGeom &g, int batc
 bool conv_bwd_reads_pooled(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch) {
   const ConvGeom g = make_geom(d);
   DxsPlan dxs;
-  if (!dw_small_applies(d, g, batch) || !small_cin_dx_plan(g, dxs) || !dxs.pooled_ok) return false;
+  if (!dw_small_applies(d, g, batch) || !small_cin_dx_plan(g, dxs) ||
+      !(dxs.pooled_ok || first_dx_mfma<true>(g, batch, nullptr, nullptr, nullptr, ActGrad(), PoolGather(), true)))
+    return false;
   if (pool->pool_w != 2 || pool->pool_h != 2 || pool->stride_w != 2 || pool->stride_h != 2 ||
       pool->in_w != g.OW || pool->in_h != g.OH || pool->in_c != g.Kc || g.OW % 4 != 0 || g.OH % 2 != 0)
     return false;
@@ -737,8 +982,13 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
     DxsPlan dxs;
     small_cin_dx_plan(g, dxs);
     if (dx) {
-      ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
-      launch_small_cin_dx_window<true>(g, dxs, batch, nullptr, w, dx, dx_act, *dy_pool);
+      if (first_dx_mfma<true>(g, batch, nullptr, w, dx, dx_act, *dy_pool, true)) {
+        ProfScope prof("conv_dx_first_mfma", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
+        first_dx_mfma<true>(g, batch, nullptr, w, dx, dx_act, *dy_pool, false);
+      } else {
+        ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
+        launch_small_cin_dx_window<true>(g, dxs, batch, nullptr, w, dx, dx_act, *dy_pool);
+      }
       TDH_LAUNCH_CHECK();
     }
     if (dw)
@@ -756,7 +1006,12 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
   DxsPlan dxs;
-  if (dx && small_cin_dx_plan(g, dxs)) {
+  if (dx && small_cin_dx_plan(g, dxs) && !(reinterpret_cast<uintptr_t>(dy) & 15) &&
+      first_dx_mfma<false>(g, batch, dy, w_eff, dx, dx_act, PoolGather(), true)) {
+    ProfScope prof("conv_dx_first_mfma", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
+    first_dx_mfma<false>(g, batch, dy, w_eff, dx, dx_act, PoolGather(), false);
+    TDH_LAUNCH_CHECK();
+  } else if (dx && small_cin_dx_plan(g, dxs)) {
     ProfScope prof("conv_dx_small_cin", g.C, batch * g.H * g.W, g.Kc * g.R * g.S);
     launch_small_cin_dx_window<false>(g, dxs, batch, dy, w_eff, dx, dx_act, PoolGather());
     TDH_LAUNCH_CHECK();
