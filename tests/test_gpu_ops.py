@@ -47,6 +47,11 @@ CONV = [
     # several output-channel tiles, one to three column tiles
     (16, 16, 3, 3, 8, True, 2, 4), (19, 14, 2, 5, 33, False, 2, 3), (64, 64, 3, 5, 16, True, 1, 2),
     (32, 37, 3, 3, 70, True, 1, 5), (32, 32, 3, 5, 32, True, 1, 128), (28, 28, 2, 5, 6, True, 1, 40),
+    # first-layer dX on the matrix cores (output rows of 16, 32 or 64): a ragged last band, one
+    # to four input channels, one output channel and two chunks of them, valid padding, and an
+    # image with fewer rows than a band (the vector-ALU kernel takes that one)
+    (16, 19, 4, 3, 40, True, 1, 3), (36, 20, 3, 5, 33, False, 1, 2), (64, 9, 2, 3, 1, True, 1, 2),
+    (18, 7, 1, 3, 70, False, 1, 4), (64, 3, 3, 3, 8, True, 1, 2), (20, 12, 2, 5, 6, False, 1, 5),
 ]
 
 
