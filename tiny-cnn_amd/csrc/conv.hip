@@ -625,7 +625,7 @@ conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict_
       }
     }
     __syncthreads();
-    // ---- products: eight staged channels a round, the four blocks of the wave side by side
+    // ---- products: eight staged channels per pass, the four blocks of the wave side by side
 #pragma unroll
     for (int sub = 0; sub < DXM_MCH / 8; ++sub) {
       if (co0 + 8 * sub >= g.Kc) break;
