@@ -1088,23 +1088,29 @@ fc_dw_direct_kernel(const FcDwDirect f) {
   // o0 + 2*(l%32) + d; the two blocks d leave as one 8-byte store
   if (!b_ok) return;
   float *out = f.dw + o0 + CB * m;
+  // (rows past the layer's inputs are read and written at row i0, with what row i0 holds:
+  // loads and stores without conditions, sixteen loads in flight when the sums are added to
+  // what the gradient held)
 #pragma unroll
-  for (int c = 0; c < CA; ++c)
+  for (int c = 0; c < CA; ++c) {
+    bvec old[16];
+    if (f.accumulate) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = i0 + CA * (8 * (r >> 2) + 4 * h + (r & 3)) + c;
+        old[r] = *reinterpret_cast<const bvec *>(out + static_cast<size_t>(min(i, f.in - 1)) * f.out);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int i = i0 + CA * (8 * (r >> 2) + 4 * h + (r & 3)) + c;
       if (i >= f.in) continue;
-      bvec *dst = reinterpret_cast<bvec *>(out + static_cast<size_t>(i) * f.out);
       bvec v;
 #pragma unroll
-      for (int d = 0; d < CB; ++d) v[d] = acc[c][d][r];
-      if (f.accumulate) {
-        const bvec old = *dst;
-#pragma unroll
-        for (int d = 0; d < CB; ++d) v[d] = old[d] + v[d];
-      }
-      *dst = v;
+      for (int d = 0; d < CB; ++d) v[d] = f.accumulate ? old[r][d] + acc[c][d][r] : acc[c][d][r];
+      *reinterpret_cast<bvec *>(out + static_cast<size_t>(i) * f.out) = v;
     }
+  }
 }
 
 // the layer is large enough for every compute unit to get a workgroup of that kernel, and its
