@@ -1117,7 +1117,8 @@ fc_dw_direct_kernel(const FcDwDirect f) {
 // rows allow the 16- and 8-byte reads
 static bool fc_dw_direct_applies(int in, int out, int batch, const float *x, const float *dy, const float *dw) {
   const long wgs = static_cast<long>(ceil_div(in, 128 * FDW_WM)) * ceil_div(out, 64 * FDW_WN);
-  return in % 4 == 0 && out % 2 == 0 && batch >= 2 && wgs >= 256 && wgs <= 65535L * 16 &&
+  return in % 4 == 0 && out % 2 == 0 && batch >= 2 && wgs >= 256 && ceil_div(in, 128 * FDW_WM) <= 65535 &&
+         ceil_div(out, 64 * FDW_WN) <= 65535 &&
          static_cast<long>(batch) * std::max(in, out) < (1L << 30) &&
          !(reinterpret_cast<uintptr_t>(x) & 15) && !(reinterpret_cast<uintptr_t>(dy) & 7) &&
          !(reinterpret_cast<uintptr_t>(dw) & 7);
