@@ -32,7 +32,8 @@ def test_gradients_of_every_layer_match_oracle(T, O, W, name, batch, size, flags
     net.train_step(None, loss, batch, xd, td, do_update=False)
     ref.train_step(O.opt_desc(opt_kind), loss, x, t, do_update=False)
     for i, l in enumerate(spec):
-        assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{name} layer {i} output")
+        if net.out_written(i):
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{name} layer {i} output")
         if l[0] == "maxpool":
             assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64),
                                   ref.layer_argmax(i, batch)), f"{name} layer {i} argmax"
@@ -135,7 +136,8 @@ def relu_sign_flips(net, ref, spec, batch):
 def check_every_layer(net, ref, spec, batch, name, fused, passes=1, cancelling_db=()):
     flipped = relu_sign_flips(net, ref, spec, batch)
     for i, l in enumerate(spec):
-        assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{name} layer {i} output")
+        if net.out_written(i):
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{name} layer {i} output")
         if l[0] == "maxpool":
             assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64),
                                   ref.layer_argmax(i, batch)), f"{name} layer {i} argmax"
@@ -424,7 +426,8 @@ def test_net_with_every_other_activation_matches_oracle(T, O, W):
             net.train_step(opt, "mse", batch, xd, td)
             ref.train_step(ropt, "mse", x, t)
             for i, l in enumerate(spec):
-                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"step {step} out {i}")
+                if net.out_written(i):
+                    assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"step {step} out {i}")
                 if W.layer_fans(l)[0]:
                     assert_close(net.get_param(i, 0), ref.weight(i), REL_TOL, f"step {step} w {i}")
                     assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} b {i}")
@@ -490,7 +493,8 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
     for net in nets:
         net.train_step(None, "mse", batch, xd, td, do_update=False)
         for i, l in enumerate(spec):
-            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+            if net.out_written(i):
+                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
             if l[0] == "maxpool":
                 assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64), ref.layer_argmax(i, batch))
                 if i >= 1 and spec[i - 1][0] == "conv" and net.dx_written(i):
@@ -502,6 +506,16 @@ def check_fusing_and_plain_net(T, O, W, spec, batch):
                 assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
                 assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")
         assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, "input gradient")
+    for i in range(len(spec)):
+        if nets[0].out_written(i) and nets[1].out_written(i):
+            assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
+    # a train step may keep a convolution's own output in registers when its kernel also computes
+    # the pool behind it; the forward pass of its own writes every layer
+    for net in nets:
+        net.forward(batch, xd)
+        for i in range(len(spec)):
+            assert net.out_written(i)
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"forward pass, layer {i} output")
     for i in range(len(spec)):
         assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
     for net in nets:
@@ -623,13 +637,15 @@ def test_last_fc_softmax_xent_in_one_launch_matches_oracle(T, O, W, spec, batch,
         for net in nets:
             net.train_step(None, loss, batch, xd, td, do_update=False)
             for i, l in enumerate(spec):
-                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+                if net.out_written(i):
+                    assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
                 if net.param_size(i, 0):
                     assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
                     assert_close(net.layer_grad(i, 1), ref.layer_db(i), REL_TOL, f"layer {i} db")
             assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), REL_TOL, "input gradient")
         for i in range(len(spec)):
-            assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
+            if nets[0].out_written(i) and nets[1].out_written(i):
+                assert np.array_equal(nets[0].layer_out(i, batch), nets[1].layer_out(i, batch)), f"layer {i} fused vs not"
         # (a folded activation gradient rounds differently from the activation layer's own kernel,
         # so the layers in front agree to rounding only)
         for which in (0, 1):
@@ -697,8 +713,9 @@ def test_two_closing_fc_layers_in_one_launch_match_oracle(T, O, W, spec, batch, 
     for n in (net, plain):
         n.train_step(None, loss, batch, xd, td, do_update=False)
     for i, l in enumerate(spec):
-        assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
-        assert_close(net.layer_out(i, batch), plain.layer_out(i, batch), REL_TOL, f"layer {i} output, fused vs not")
+        if net.out_written(i):
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+            assert_close(net.layer_out(i, batch), plain.layer_out(i, batch), REL_TOL, f"layer {i} output, fused vs not")
         if l[0] == "maxpool" and spec[i - 1][0] == "conv":
             for n_ in (net, plain):
                 if n_.dx_written(i):
@@ -713,7 +730,8 @@ def test_two_closing_fc_layers_in_one_launch_match_oracle(T, O, W, spec, batch, 
         net.train_step(opt, loss, batch, xd, td)
         ref.train_step(ropt, loss, x, t)
         for i, l in enumerate(spec):
-            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"step {step} layer {i} output")
+            if net.out_written(i):
+                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"step {step} layer {i} output")
             if net.param_size(i, 0):
                 assert_close(net.get_param(i, 0), ref.weight(i), REL_TOL, f"step {step} layer {i} weights")
                 assert_close(net.get_param(i, 1), ref.bias(i), REL_TOL, f"step {step} layer {i} bias")
@@ -743,7 +761,8 @@ def test_layers_without_bias_through_the_one_launch_kernels(T, O):
     for net in nets:
         net.train_step(None, "ce_multiclass", batch, T.to_device(x), T.to_device(t), do_update=False)
         for i in range(7):
-            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
+            if net.out_written(i):
+                assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), REL_TOL, f"layer {i} output")
         for i in (0, 3, 5):
             assert_close(net.layer_grad(i, 0), ref.layer_dw(i), REL_TOL, f"layer {i} dW")
         assert_close(net.layer_dx(1, batch), ref.layer_dx(1, batch), REL_TOL, "gradient routed through the pool")

@@ -562,9 +562,18 @@ class Net:
               "tdh_net_get_param")
         return a
 
+    def out_written(self, i):
+        """False when the last pass never wrote layer i's output: in a train step of a fusing
+        net the kernel of a first convolution that also computes the max-pool directly behind
+        it keeps the convolution's own output in registers."""
+        return bool(lib().tdh_net_layer_out(self.h, i))
+
     def layer_out(self, i, batch):
         n = self.layer_out_size(i)
-        return DevBuf.view(lib().tdh_net_layer_out(self.h, i), (batch, n)).numpy()
+        p = lib().tdh_net_layer_out(self.h, i)
+        if not p:
+            raise RuntimeError(f"layer {i}: the last pass did not write this output to memory")
+        return DevBuf.view(p, (batch, n)).numpy()
 
     def dx_written(self, i):
         """False when the last step never wrote the gradient with respect to layer i's input:

@@ -937,6 +937,9 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
                float *y, const uint8_t *tbl_resident, const float *prepacked, float *act_out,
                int act_kind, const PoolFuse *pool) {
   const ConvGeom g = make_geom(d);
+  // (y null: only the kernel that also computes the pool behind the layer can leave it out)
+  if (!y && !(pool && !prepacked && fwd_small_applies(g, batch)))
+    return set_error(TDH_ERR_INVALID, "conv2d_fwd: no output tensor");
   if (prepacked)
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
                        g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked, act_out,

@@ -192,7 +192,7 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_kernel(const FwdSmallAr
       v0[i] = acc0[i] + bias_r[i];
       v1[i] = acc1[i] + bias_r[i];
     }
-    {
+    if (a.out) {  // (null: the layers behind leave this kernel too and nobody reads the convolution's own output)
       float *o = a.out + pbase;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -329,11 +329,13 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_full_kernel(const FwdSm
       v0[i] = acc0[i] + bias_r[i];
       v1[i] = acc1[i] + bias_r[i];
     }
+    if (a.out) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float *o = out_img + (((i >> 2) * 8 + (i & 3)) * ohw + first);  // scalar
-      o[lane_out]        = v0[i];
-      (o + OW)[lane_out] = v1[i];
+      for (int i = 0; i < 16; ++i) {
+        float *o = out_img + (((i >> 2) * 8 + (i & 3)) * ohw + first);  // scalar
+        o[lane_out]        = v0[i];
+        (o + OW)[lane_out] = v1[i];
+      }
     }
     if (pool) {
       // as above: the window of an even lane in scan order, strict '>', start value lowest();
@@ -456,6 +458,7 @@ int conv_fwd_small_run(int batch, int C, int Kc, const float *x, const float *w,
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: shape not supported");
   if (pool && ((OH | OW) & 1))
     return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: a fused 2x2 pool needs even output sizes");
+  if (!out && !pool) return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: no output");
   p.a.x = x; p.a.w = w; p.a.bias = bias; p.a.out = out;
   p.a.act_out  = act_out;
   p.a.act_kind = act_kind;

@@ -57,12 +57,13 @@ struct tdh_net {
     hipGraphExec_t exec = nullptr;
     GraphKey key;
     uint64_t last_use = 0;
-    std::vector<uint8_t> dx_unwritten;  // what the captured step leaves in the net's field of that name
+    std::vector<uint8_t> dx_unwritten, out_unwritten;  // what the captured step leaves in the net's fields of those names
   } graphs[kGraphSlots];
   uint64_t graph_clock = 0;
   // per layer: the last step kept the gradient with respect to this layer's input in registers
   // or read it through a pool (tdh_net_layer_dx has nothing to show)
   std::vector<uint8_t> dx_unwritten;
+  std::vector<uint8_t> out_unwritten;  // likewise for a layer's output
   float mirror_b1_t = 0.0f, mirror_b2_t = 0.0f;  // what the device copy of the powers holds
   size_t scratch = 0;        // largest per-op scratch need; with TDH_NET_GRAPH the sum over the
                              // layers, because branches of the captured step run side by side
@@ -247,10 +248,14 @@ TailPlan plan_tail(tdh_net *net, int loss_kind, int batch) {
 // tail: its layer runs as fc_softmax_xent, which also writes the loss gradient (to xent_dz, from
 // the targets xent_t) and the gradient of its input; with tail->first that layer, the activation
 // behind it and tail->layer run as fc_two_layer_tail
+// training: the pass is the first half of a train step: an output that only the kernel which
+// computes it would read (a first convolution's, with the max-pool directly behind it in the
+// same kernel) is not written
 int forward(tdh_net *net, int batch, const float *x, bool packed = false, const float *xent_t = nullptr,
-            float *xent_dz = nullptr, const TailPlan *tail = nullptr) {
+            float *xent_dz = nullptr, const TailPlan *tail = nullptr, bool training = false) {
   const float *in = x;
   const int n     = static_cast<int>(net->layers.size());
+  net->out_unwritten.assign(n, 0);
   for (int i = 0; i < n; ++i) {
     tdh_net::Layer &L  = net->layers[i];
     const tdh_layer &s = L.spec;
@@ -290,7 +295,9 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
           // nothing behind the convolution left its kernel and a max-pool reads the result
           LeaveSplitSum leave(ctx(), fuse && last == i && i + 1 < n &&
                                          net->layers[i + 1].spec.kind == TDH_L_MAXPOOL);
-          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, L.out, L.tbl_dev, wp, act_out, act_kind,
+          const bool own_out = !(training && pf.out && !act_out);
+          if (!own_out) net->out_unwritten[i] = 1;
+          TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, own_out ? L.out : nullptr, L.tbl_dev, wp, act_out, act_kind,
                              pf.out ? &pf : nullptr));
         }
         i = last;
@@ -651,7 +658,9 @@ int tdh_net_get_param(tdh_net *net, int layer, int which, float *host_dst) {
   return tdh_memcpy_d2h(host_dst, src, n * sizeof(float));
 }
 const float *tdh_net_layer_out(const tdh_net *net, int layer) {
-  return (layer >= 0 && layer < static_cast<int>(net->layers.size())) ? net->layers[layer].out : nullptr;
+  if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
+  if (static_cast<size_t>(layer) < net->out_unwritten.size() && net->out_unwritten[layer]) return nullptr;
+  return net->layers[layer].out;
 }
 const float *tdh_net_layer_dx(const tdh_net *net, int layer) {
   if (layer < 0 || layer >= static_cast<int>(net->layers.size())) return nullptr;
@@ -724,13 +733,13 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   tail_done           = plan.layer;
   if (loss_kind == TDH_LOSS_CE_MULTICLASS && last.spec.kind == TDH_L_ACT &&
       last.spec.act == TDH_ACT_SOFTMAX && n >= 2) {
-    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done >= 0 ? &plan : nullptr));
+    TDH_TRY(forward(net, batch, x, packed, t, net->layers[n - 2].dout, tail_done >= 0 ? &plan : nullptr, true));
     first_bwd = n - 2;
   } else if (tail_done >= 0) {
     // mse on a closing fully-connected layer: its kernel writes the loss gradient too
-    TDH_TRY(forward(net, batch, x, packed, t, last.dout, &plan));
+    TDH_TRY(forward(net, batch, x, packed, t, last.dout, &plan, true));
   } else {
-    TDH_TRY(forward(net, batch, x, packed));
+    TDH_TRY(forward(net, batch, x, packed, nullptr, nullptr, nullptr, true));
     TDH_TRY(launch_loss_grad(loss_kind, batch, static_cast<int>(last.out_size), last.out, t,
                              last.dout));
   }
@@ -1059,7 +1068,8 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
                        hipGetErrorString(e));
     }
     slot->key = key;
-    slot->dx_unwritten = net->dx_unwritten;
+    slot->dx_unwritten  = net->dx_unwritten;
+    slot->out_unwritten = net->out_unwritten;
     net->mirror_b1_t = net->mirror_b2_t = -1.0f;  // forces the upload below
   }
   // the captured optimizer kernel reads the powers from device memory; bring that copy in
@@ -1070,7 +1080,8 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   }
   slot->last_use = ++net->graph_clock;
   TDH_HIP(hipGraphLaunch(slot->exec, ctx().stream));
-  net->dx_unwritten = slot->dx_unwritten;
+  net->dx_unwritten  = slot->dx_unwritten;
+  net->out_unwritten = slot->out_unwritten;
   if (opt && do_update) {
     // advance the host object exactly as the eager path does
     for (int j = 0; j < net->opt_tensors; ++j) {
