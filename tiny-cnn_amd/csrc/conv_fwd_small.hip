@@ -26,6 +26,8 @@ namespace tdh {
 
 namespace {
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
 struct FwdSmallArgs {
   const float *x, *w, *bias;
   float *out;
@@ -77,6 +79,19 @@ __device__ __forceinline__ void fwd_small_stage(const FwdSmallArgs &a, float *xs
     const int iy0     = oy0 * a.sh - a.ph;
     const int x_total = a.C * a.rows_in * a.pitch;
     constexpr int DEPTH = 8;
+    // the filter slice as 16-byte words, issued in front of the patch and stored behind it: one
+    // trip to memory covers both (a thread's eight words hold 32 rows of up to 128 taps)
+    const int w_total = 32 * a.crs;
+    const int w_valid = min(32, a.Kc - co0) * a.crs;
+    const float *wsrc = a.w + static_cast<size_t>(co0) * a.crs;
+    const bool wvec   = (reinterpret_cast<uintptr_t>(wsrc) & 15u) == 0 && (w_valid & 3) == 0 &&
+                      w_total <= 4 * DEPTH * nthr;
+    floatx4 wq[DEPTH];
+    if (wvec) {
+#pragma unroll
+      for (int k = 0; k < DEPTH; ++k)  // (every load is issued: a word past the slice repeats its last one)
+        wq[k] = *reinterpret_cast<const floatx4 *>(wsrc + min(4 * (tid + k * nthr), w_valid - 4));
+    }
     for (int e0 = tid; e0 < x_total; e0 += DEPTH * nthr) {
       float xv[DEPTH];
       int xo[DEPTH];
@@ -98,10 +113,15 @@ __device__ __forceinline__ void fwd_small_stage(const FwdSmallArgs &a, float *xs
       for (int k = 0; k < DEPTH; ++k)
         if (xo[k] >= 0) xs[xo[k]] = xv[k];
     }
-    const int w_total = 32 * a.crs;
-    const int w_valid = min(32, a.Kc - co0) * a.crs;
-    const float *wsrc = a.w + static_cast<size_t>(co0) * a.crs;
-    for (int e0 = tid; e0 < w_total; e0 += DEPTH * nthr) {
+    if (wvec) {
+#pragma unroll
+      for (int k = 0; k < DEPTH; ++k) {
+        const int e = 4 * (tid + k * nthr);
+        const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (e < w_total) *reinterpret_cast<floatx4 *>(ws + e) = e < w_valid ? wq[k] : zero4;
+      }
+    }
+    for (int e0 = wvec ? w_total : tid; e0 < w_total; e0 += DEPTH * nthr) {
       float wv[DEPTH];
 #pragma unroll
       for (int k = 0; k < DEPTH; ++k) {
@@ -288,7 +308,10 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_full_kernel(const FwdSm
     const int k = 2 * s + half;
     areg[s]     = k < a.crs ? ws[nl * a.crs + k] : 0.0f;
   }
-  const int *offh = offs + half;
+  // the patch offset of every k-step: the same for all tiles of the wave
+  int o[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) o[s] = offs[2 * s + half];
   float bias_r[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) bias_r[i] = bs[(i >> 2) * 8 + half * 4 + (i & 3)];
@@ -314,11 +337,29 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_full_kernel(const FwdSm
     floatx16 acc0, acc1;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc0[i] = acc1[i] = 0.0f;
+    // The patch values of eight k-steps are read while the products of the eight before them
+    // run: read and product one after the other would wait for LDS in every step.
+    constexpr int G = 8;
+    static_assert(NS % G == 0, "k-steps come in groups");
+    float b0[2][G], b1[2][G];
+    auto read_patch = [&](int g, int to) {
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const int o = offh[2 * s];
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], xb0[o], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[s], xb1[o], acc1, 0, 0, 0);
+      for (int j = 0; j < G; ++j) {
+        b0[to][j] = xb0[o[g * G + j]];
+        b1[to][j] = xb1[o[g * G + j]];
+      }
+    };
+    read_patch(0, 0);
+#pragma unroll
+    for (int g = 0; g < NS / G; ++g) {
+      const int cur = g & 1;
+      if (g + 1 < NS / G) read_patch(g + 1, cur ^ 1);
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[g * G + j], b0[cur][j], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(areg[g * G + j], b1[cur][j], acc1, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // (the reads stay in front of the group they were written for)
     }
     // reg i of lane l holds channel 8*(i/4) + 4*(l/32) + i%4 at column l%32
     const uint32_t oy = oy0 + r;
