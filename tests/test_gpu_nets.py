@@ -451,6 +451,30 @@ def test_first_conv_with_pool_in_its_kernel_matches_oracle(T, O, W, spec):
     check_fusing_and_plain_net(T, O, W, spec, 5)
 
 
+@pytest.mark.parametrize("spec,batch", [
+    # rows of 16 pixels, one accumulator block a wave; relu behind the pool leaves the kernel too
+    ([("conv", 16, 16, 16, 3, 32, True), ("maxpool", 16, 16, 32, 2), ("act", "relu"), ("fc", 32 * 64, 10)], 64),
+    # rows of 8 pixels, two images a tile, 5x5 window, an activation between convolution and pool
+    ([("conv", 8, 8, 16, 5, 32, True), ("act", "tanh"), ("maxpool", 8, 8, 32, 2), ("fc", 32 * 16, 10)], 256),
+    # two channel blocks a wave; the sigmoid behind the pool stays a kernel of its own
+    ([("conv", 16, 16, 32, 3, 64, True), ("maxpool", 16, 16, 64, 2), ("act", "sigmoid"), ("fc", 64 * 64, 10)], 128),
+    # two pixel blocks a wave
+    ([("conv", 16, 16, 16, 5, 32, True), ("maxpool", 16, 16, 32, 2), ("fc", 32 * 64, 10)], 256),
+    # ragged tiles: 10 rows in tiles of 8, 12 columns in rows of 16; 40 of 64 channels
+    ([("conv", 12, 10, 16, 3, 40, True), ("maxpool", 12, 10, 40, 2), ("act", "relu"), ("fc", 40 * 30, 10)], 128),
+    # no padding: 18x18 -> 16x16
+    ([("conv", 18, 18, 16, 3, 32, False), ("act", "relu"), ("maxpool", 16, 16, 32, 2), ("act", "relu"),
+      ("fc", 32 * 64, 10)], 64),
+])
+def test_stride1_conv_with_pool_in_its_kernel_matches_oracle(T, O, W, spec, batch):
+    """A stride-1 convolution with many input channels whose 32-pixel accumulator blocks hold
+    whole pool windows also computes the 2x2 max-pool behind it (and a relu behind that): every
+    layer output, the argmax records (bit-exact) and all gradients against the oracle, the same
+    outputs as the net without fusion, and the convolution's own output is left out of a train
+    step only."""
+    check_fusing_and_plain_net(T, O, W, spec, batch)
+
+
 @pytest.mark.parametrize("spec", [
     # 2x2 pools behind and in front of the second convolution: they add up its split reductions
     [("conv", 16, 16, 3, 5, 32, True), ("maxpool", 16, 16, 32, 2), ("act", "relu"),

@@ -288,6 +288,8 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
                float *act_out = nullptr, int act_kind = 0, const PoolFuse *pool = nullptr);
 // the forward kernel of this convolution can also compute the max-pool layer `pool` behind it
 bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked);
+// ... and the pointwise activation of this kind behind that pool
+bool conv_fwd_pool_applies_act(const tdh_conv_desc *d, int batch, bool prepacked, int act_kind);
 // conv_fwd_small.hip
 bool conv_fwd_small_applicable(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
                                int sh, int sw, int dh, int dw, int ph, int pw);
@@ -351,7 +353,12 @@ size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip,
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
                 int OW, int ph, int pw, ActGrad ag, const char *tag,
-                const float *prepacked = nullptr, float *act_out = nullptr, int act_kind = 0);
+                const float *prepacked = nullptr, float *act_out = nullptr, int act_kind = 0,
+                const PoolFuse *pool = nullptr);
+// the forward kernel of this shape can also compute the 2x2 / stride-2 max-pool behind it (and
+// a relu behind that pool); `out` may then be null
+bool conv_s1_fuses_pool(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
+                        int ph, int pw);
 int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const uint8_t *tbl_dev,
                    float *wp);
 // conv_dw.hip: stride-1 weight gradient from LDS-staged tiles (3x3 and 5x5 windows)

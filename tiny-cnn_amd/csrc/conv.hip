@@ -909,11 +909,28 @@ bool conv_fwd_applies_act(const tdh_conv_desc *d, int batch, bool prepacked) {
   return prepacked ? conv_uses_packed(d, batch, 0) : true;
 }
 
+// the stride-1 kernel runs this forward pass (with filters packed by the caller, or by itself)
+static bool fwd_s1_applies(const tdh_conv_desc *d, const ConvGeom &g, int batch, bool prepacked) {
+  if (prepacked) return conv_uses_packed(d, batch, 0);
+  return !fwd_small_applies(g, batch) && g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 &&
+         conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
+}
+
 bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked) {
   const ConvGeom g = make_geom(d);
-  if (prepacked || !fwd_small_applies(g, batch)) return false;
-  return pool->pool_w == 2 && pool->pool_h == 2 && pool->stride_w == 2 && pool->stride_h == 2 &&
-         pool->in_w == g.OW && pool->in_h == g.OH && pool->in_c == g.Kc && g.OW % 2 == 0 && g.OH % 2 == 0;
+  if (!(pool->pool_w == 2 && pool->pool_h == 2 && pool->stride_w == 2 && pool->stride_h == 2 &&
+        pool->in_w == g.OW && pool->in_h == g.OH && pool->in_c == g.Kc && g.OW % 2 == 0 && g.OH % 2 == 0))
+    return false;
+  if (!prepacked && fwd_small_applies(g, batch)) return true;
+  return fwd_s1_applies(d, g, batch, prepacked) &&
+         conv_s1_fuses_pool(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
+}
+
+bool conv_fwd_pool_applies_act(const tdh_conv_desc *d, int batch, bool prepacked, int act_kind) {
+  const ConvGeom g = make_geom(d);
+  // the first-layer kernel applies any pointwise kind, the stride-1 kernel relu
+  if (!prepacked && fwd_small_applies(g, batch)) return true;
+  return act_kind == TDH_ACT_RELU;
 }
 
 bool conv_uses_packed(const tdh_conv_desc *d, int batch, int flip) {
@@ -937,15 +954,20 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
                float *y, const uint8_t *tbl_resident, const float *prepacked, float *act_out,
                int act_kind, const PoolFuse *pool) {
   const ConvGeom g = make_geom(d);
-  // (y null: only the kernel that also computes the pool behind the layer can leave it out)
-  if (!y && !(pool && !prepacked && fwd_small_applies(g, batch)))
-    return set_error(TDH_ERR_INVALID, "conv2d_fwd: no output tensor");
+  if (pool) {
+    tdh_pool_desc behind{};
+    behind.in_w = g.OW; behind.in_h = g.OH; behind.in_c = g.Kc;
+    behind.pool_w = behind.pool_h = behind.stride_w = behind.stride_h = 2;
+    if (!conv_fwd_fuses_pool(d, &behind, batch, prepacked != nullptr) ||
+        (pool->act_out && !conv_fwd_pool_applies_act(d, batch, prepacked != nullptr, pool->act_kind)))
+      return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not compute the pool layer behind it");
+  }
+  // (y null: only a kernel that also computes the pool behind the layer can leave it out)
+  if (!y && !pool) return set_error(TDH_ERR_INVALID, "conv2d_fwd: no output tensor");
   if (prepacked)
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
                        g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked, act_out,
-                       act_kind);
-  if (pool && !fwd_small_applies(g, batch))
-    return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not compute the pool layer behind it");
+                       act_kind, pool);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
   const uint8_t *tbl_dev;
   const float *w_eff;
@@ -957,7 +979,7 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       conv_s1_applicable(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w))
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w_eff, nullptr,
                        d->has_bias ? b : nullptr, y, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w,
-                       ActGrad(), "conv_fwd_s1", nullptr, act_out, act_kind);
+                       ActGrad(), "conv_fwd_s1", nullptr, act_out, act_kind, pool);
   StridedOperand A{w_eff, crs, 1, g.Kc};
   FwdInputOperand B{x, g, batch * ohw};
   if (act_out) {  // the pointwise activation layer that follows leaves the same kernel

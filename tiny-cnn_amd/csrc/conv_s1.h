@@ -28,6 +28,12 @@ struct ConvS1Args {
   ActGrad ag;
   float *act_out;              // forward: act(out) of the pointwise activation layer that follows
   int act_kind;
+  // forward: the 2x2 / stride-2 max-pool layer behind the convolution (or behind act_out) and
+  // the relu behind that pool, all null when the pool runs as a kernel of its own. Only tiles
+  // whose 32-pixel blocks hold whole pool windows (rows of 8 or 16 pixels, no split) take it.
+  float *pool_out;
+  int32_t *pool_argmax;        // flat CHW index inside the sample of the pool's input
+  float *pool_act_out;         // max(pool_out, 0), or null
   int batch, KC, MC, IH, IW, OH, OW, ph, pw;
   int pwa;                     // staged column 0 is image column x0 - pwa
   int TR, TI;                  // tile rows, images per tile (TI*TR*TC = PIX), powers of two

@@ -152,6 +152,16 @@ bool conv_s1_applicable(int R, int S, int batch, int KC, int MC, int IH, int IW,
   return make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw).ok;
 }
 
+// A 32-pixel accumulator block must hold whole 2x2 windows: rows of 8 or 16 pixels (tile rows
+// come in powers of two and start at even image rows), even image sizes, and one pass over the
+// reduction channels (the partial sums of a split have no maximum yet).
+bool conv_s1_fuses_pool(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
+                        int ph, int pw) {
+  const S1Plan p = make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw);
+  return p.ok && p.splits == 1 && p.tc <= 16 && p.args.TR >= 2 && OH % 2 == 0 && OW % 2 == 0 &&
+         static_cast<long>(MC) * OH * OW < (1L << 31);
+}
+
 size_t conv_s1_workspace_bytes(int R, int S, int batch, int C, int Kc, int flip, int IH, int IW,
                                int OH, int OW, int ph, int pw) {
   const int KC = flip ? Kc : C, MC = flip ? C : Kc;
@@ -178,10 +188,15 @@ int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const 
 int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *in, const float *w,
                 const uint8_t *tbl_dev, const float *bias, float *out, int IH, int IW, int OH,
                 int OW, int ph, int pw, ActGrad ag, const char *tag, const float *prepacked,
-                float *act_out, int act_kind) {
+                float *act_out, int act_kind, const PoolFuse *pool) {
   const int KC = flip ? Kc : C, MC = flip ? C : Kc;
   S1Plan p = make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw);
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_s1_run: shape not supported");
+  if (pool && (flip || !pool->out || !pool->argmax ||
+               (pool->act_out && pool->act_kind != TDH_ACT_RELU) ||
+               !conv_s1_fuses_pool(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw)))
+    return set_error(TDH_ERR_INVALID, "conv_s1_run: this shape does not compute the pool layer behind it");
+  if (!out && !pool) return set_error(TDH_ERR_INVALID, "conv_s1_run: no output tensor");
   const void *wp = prepacked;
   if (!prepacked) {
     void *fresh = nullptr;
@@ -192,13 +207,16 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
   p.args.in = in; p.args.wp = static_cast<const float *>(wp); p.args.bias = bias;
   p.args.out = out; p.args.ag = ag;
   p.args.act_out = act_out; p.args.act_kind = act_kind;
+  p.args.pool_out     = pool ? pool->out : nullptr;
+  p.args.pool_argmax  = pool ? pool->argmax : nullptr;
+  p.args.pool_act_out = pool ? pool->act_out : nullptr;
   if (p.splits > 1) {
     void *part = nullptr;
     TDH_TRY(ws_take(sizeof(float) * p.splits * p.args.part_stride, &part));
     p.args.part = static_cast<float *>(part);
   }
   {
-    ProfScope prof(tag, MC, batch * OH * OW, KC * R * S);
+    ProfScope prof(pool ? "conv_fwd_s1_pool" : tag, MC, batch * OH * OW, KC * R * S);
     const bool vec = IW % 4 == 0 && MC % 4 == 0 && aligned16(in) && aligned16(wp);
     if (vec) TDH_TRY(R == 3 ? s1_launch_3x3_vec(p) : s1_launch_5x5_vec(p));
     else TDH_TRY(R == 3 ? s1_launch_3x3_scalar(p) : s1_launch_5x5_scalar(p));

@@ -43,6 +43,16 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // address space, like those of the tensors)
 __device__ __align__(16) float s1_zero_word[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 
+// the value of lane l ^ 1 (a swap inside lane pairs, done by the DPP path of a move)
+__device__ __forceinline__ float s1_lane_xor1(const float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+// the value of lane l ^ X, X = 8 or 16 (a swizzle inside groups of 32 lanes: and 0x1F, or 0, xor X)
+template <int X>
+__device__ __forceinline__ float s1_lane_xor(const float v) {
+  return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (X << 10) | 0x1F));
+}
+
 template <int R, int S, int TC, int TM, int TN, bool VEC>
 __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
   constexpr int KCH   = s1_kch(R * S, TM, TN);
@@ -277,16 +287,51 @@ __global__ void __launch_bounds__(256, 2) conv_s1_kernel(const ConvS1Args a) {
           for (int rr = 0; rr < 16; ++rr) v[rr] *= act_grad_factor(a.ag.kind, yv[rr]);
         }
       }
+      if (dst) {  // (null: the pool behind leaves this kernel too and nobody reads the convolution's own output)
 #pragma unroll
-      for (int rr = 0; rr < 16; ++rr) {
-        const int m = mb + 8 * (rr >> 2) + (rr & 3);
-        if (m < a.MC) dst[pbase + static_cast<size_t>(m) * ohw] = v[rr];
+        for (int rr = 0; rr < 16; ++rr) {
+          const int m = mb + 8 * (rr >> 2) + (rr & 3);
+          if (m < a.MC) dst[pbase + static_cast<size_t>(m) * ohw] = v[rr];
+        }
       }
       if (!a.part && a.act_out) {
 #pragma unroll
         for (int rr = 0; rr < 16; ++rr) {
           const int m = mb + 8 * (rr >> 2) + (rr & 3);
-          if (m < a.MC) a.act_out[pbase + static_cast<size_t>(m) * ohw] = act_apply(a.act_kind, v[rr]);
+          v[rr]       = act_apply(a.act_kind, v[rr]);
+          if (m < a.MC) a.act_out[pbase + static_cast<size_t>(m) * ohw] = v[rr];
+        }
+      }
+      if constexpr (TC <= 16) {
+        if (!a.part && a.pool_out) {
+          // A 32-pixel block is whole rows of TC pixels, the first one even: the window of the
+          // lane with an even row and column is its own value, lane^1's, lane^TC's and
+          // lane^(TC+1)'s, scanned in that order with strict '>' from lowest()
+          // (maxpool_op_internal.h:17-47). Every lane runs the exchange, the anchors store.
+          const bool anchor = !(lane & 1) && !(lane & TC);
+          const int pw2 = a.OW >> 1, pohw = (a.OH >> 1) * pw2;
+          const size_t pobase = static_cast<size_t>(img) * a.MC * pohw + (oy >> 1) * pw2 + (ox >> 1);
+          const int pix = oy * a.OW + ox;
+#pragma unroll
+          for (int rr = 0; rr < 16; ++rr) {
+            const int m = mb + 8 * (rr >> 2) + (rr & 3);
+            const float right = s1_lane_xor1(v[rr]);
+            const float w4[4] = {v[rr], right, s1_lane_xor<TC>(v[rr]), s1_lane_xor<TC>(right)};
+            float best = -3.402823466e+38f;
+            int sel    = -1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              if (w4[k] > best) {
+                best = w4[k];
+                sel  = k;
+              }
+            if (anchor && m < a.MC) {
+              const size_t at = pobase + static_cast<size_t>(m) * pohw;
+              a.pool_out[at]    = best;
+              a.pool_argmax[at] = sel < 0 ? 0 : m * ohw + pix + (sel >> 1) * a.OW + (sel & 1);
+              if (a.pool_act_out) a.pool_act_out[at] = best > 0.0f ? best : 0.0f;
+            }
+          }
         }
       }
     }

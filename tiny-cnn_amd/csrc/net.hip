@@ -285,7 +285,8 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
           ++last;
           pf.out    = net->layers[last].out;
           pf.argmax = net->layers[last].argmax;
-          if (pointwise(last + 1)) {
+          if (pointwise(last + 1) &&
+              conv_fwd_pool_applies_act(&s.conv, batch, wp != nullptr, net->layers[last + 1].spec.act)) {
             ++last;
             pf.act_out  = net->layers[last].out;
             pf.act_kind = net->layers[last].spec.act;
