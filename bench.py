@@ -288,8 +288,8 @@ def cpu_baseline(W, name, budget_s=20.0, max_steps=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cifar10_cnn_b128")
     ap.add_argument("--others", action="store_true", help="(default) also run the other workloads")
     ap.add_argument("--no-others", action="store_true", help="only the named workload")

@@ -664,8 +664,18 @@ colsum_kernel(const float *__restrict__ src, const int rows, const int cols,
   const int cl = threadIdx.x & 31, g = threadIdx.x >> 5;
   const int c  = blockIdx.x * 32 + cl;
   float s = 0.0f;
-  if (c < cols)
-    for (int r = g; r < rows; r += 8) s += src[static_cast<size_t>(r) * cols + c];
+  if (c < cols) {
+    // eight loads in flight, added in row order (one at a time each add waits a trip to memory)
+    int r = g;
+    for (; r + 56 < rows; r += 64) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = src[static_cast<size_t>(r + 8 * k) * cols + c];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) s += v[k];
+    }
+    for (; r < rows; r += 8) s += src[static_cast<size_t>(r) * cols + c];
+  }
   sm[g][cl] = s;
   __syncthreads();
   if (g == 0 && c < cols) {

@@ -520,6 +520,47 @@ splitk_reduce_kernel(const float *__restrict__ partial, const int splits, const 
   splitk_reduce_block(partial, splits, M, N, epi, blockIdx.x, sm);
 }
 
+// The same sums for a large result (N a multiple of four): a thread owns four neighbouring
+// outputs and reads every slice as one 16-byte word, eight slices in flight. Slice z still
+// goes to group z % 8 and the groups are added in order, so the result is the one of the
+// kernel above bit for bit; that kernel gives a workgroup 32 outputs, which for a million
+// outputs and eight slices is 32768 workgroups of one load a thread.
+template <class Epi>
+__global__ void __launch_bounds__(256)
+splitk_reduce_wide_kernel(const float *__restrict__ partial, const int splits, const int M, const int N,
+                          const Epi epi) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const size_t mn = static_cast<size_t>(M) * N;
+  const size_t idx = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (idx >= mn) return;
+  f4 s[REDUCE_GROUPS];
+#pragma unroll
+  for (int g = 0; g < REDUCE_GROUPS; ++g) s[g] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int z0 = 0; z0 < splits; z0 += REDUCE_GROUPS) {
+    f4 v[REDUCE_GROUPS];
+#pragma unroll
+    for (int g = 0; g < REDUCE_GROUPS; ++g)  // (every load is issued: a slice past the last repeats it and is dropped)
+      v[g] = *reinterpret_cast<const f4 *>(partial + static_cast<size_t>(min(z0 + g, splits - 1)) * mn + idx);
+#pragma unroll
+    for (int g = 0; g < REDUCE_GROUPS; ++g)
+      if (z0 + g < splits) s[g] += v[g];
+  }
+  f4 t = s[0];
+#pragma unroll
+  for (int g = 1; g < REDUCE_GROUPS; ++g) t += s[g];
+  const int m = static_cast<int>(idx / N), n = static_cast<int>(idx - static_cast<size_t>(m) * N);
+  typename Epi::Col c[4];
+  float before[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    c[e]      = epi.col(n + e);
+    before[e] = epi.prior(m, c[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) epi.store(m, c[e], t[e], before[e]);
+}
+constexpr long REDUCE_WIDE_MIN = 1L << 18;  // outputs from which the wide kernel is launched
+
 // Several reductions in one launch: the weight gradients of a train step's layers, whose
 // partial tiles are all complete when the last dW kernel ends. Job j owns the workgroups
 // [first_block[j], first_block[j+1]).
@@ -688,8 +729,13 @@ int launch_gemm(const AOp &a, const BOp &b, const Epi &epi, int M, int N, int K,
     // reads every partial tile once and writes the result once
     if (defer_reduce(partial, p.splits, M, N, epi)) return TDH_OK;
     ProfScope prof(reduce_tag, 4.0 * M * N * (p.splits + 1), WORK_BYTE);
-    TDH_LAUNCH((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, REDUCE_OUTPUTS)), dim3(256), 0,
-                       ctx().stream, partial, p.splits, M, N, epi);
+    if (N % 4 == 0 && static_cast<long>(M) * N >= REDUCE_WIDE_MIN &&
+        (reinterpret_cast<uintptr_t>(partial) & 15u) == 0)
+      TDH_LAUNCH((splitk_reduce_wide_kernel<Epi>), dim3(static_cast<unsigned>(ceil_div_sz(static_cast<size_t>(M) * N / 4, 256))),
+                 dim3(256), 0, ctx().stream, partial, p.splits, M, N, epi);
+    else
+      TDH_LAUNCH((splitk_reduce_kernel<Epi>), dim3(ceil_div(M * N, REDUCE_OUTPUTS)), dim3(256), 0,
+                 ctx().stream, partial, p.splits, M, N, epi);
     TDH_LAUNCH_CHECK();
   }
   return TDH_OK;
