@@ -305,9 +305,10 @@ int tdh_net_clear_grads(tdh_net *net);
 /* device views valid until the net is destroyed */
 float *tdh_net_param(tdh_net *net, int layer, int which);
 /* the layer's output as the last pass left it, or NULL where that pass never wrote it to
- * memory: in a train step with TDH_NET_FUSE_ACT_GRAD the kernel of a first convolution that
- * also computes the 2x2 max-pool directly behind it keeps the convolution's own output in
- * registers (nothing in the backward pass reads it); tdh_net_forward always writes it */
+ * memory: in a train step with TDH_NET_FUSE_ACT_GRAD a convolution kernel that also writes the
+ * pointwise activation or computes the 2x2 max-pool behind the convolution keeps the
+ * convolution's own output in registers (nothing in the backward pass reads it: the gradients
+ * of tanh, relu and sigmoid are functions of their outputs); tdh_net_forward always writes it */
 const float *tdh_net_layer_out(const tdh_net *net, int layer);
 /* the gradient with respect to the layer's input as the last step left it, or NULL where
  * that step never wrote it to memory: with TDH_NET_FUSE_ACT_GRAD the gradient of a folded

@@ -123,8 +123,11 @@ def relu_sign_flips(net, ref, spec, batch):
             yg, yr = net.layer_out(i, batch), ref.layer_out(i, batch)
             flips = (yg > 0) != (yr > 0)
             if flips.any():
-                pre_g, pre_r = net.layer_out(i - 1, batch), ref.layer_out(i - 1, batch)
                 if spec[i - 1][0] in ("conv", "fc"):     # the layer in front holds the pre-activation
+                    pre_r = ref.layer_out(i - 1, batch)
+                    # (a train step may have kept the convolution's own output in registers: the
+                    # relu output is the pre-activation wherever it is positive)
+                    pre_g = net.layer_out(i - 1, batch) if net.out_written(i - 1) else yg
                     rms = np.sqrt(np.mean(pre_r.astype(np.float64) ** 2))
                     assert np.all(np.abs(pre_g[flips]) < 1e-5 * rms) and np.all(np.abs(pre_r[flips]) < 1e-5 * rms), \
                         f"layer {i}: relu outputs differ in sign away from zero"

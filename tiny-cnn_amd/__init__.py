@@ -564,8 +564,8 @@ class Net:
 
     def out_written(self, i):
         """False when the last pass never wrote layer i's output: in a train step of a fusing
-        net the kernel of a first convolution that also computes the max-pool directly behind
-        it keeps the convolution's own output in registers."""
+        net a convolution kernel that also writes the activation or computes the max-pool
+        behind the convolution keeps the convolution's own output in registers."""
         return bool(lib().tdh_net_layer_out(self.h, i))
 
     def layer_out(self, i, batch):

@@ -290,6 +290,9 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
 bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked);
 // ... and the pointwise activation of this kind behind that pool
 bool conv_fwd_pool_applies_act(const tdh_conv_desc *d, int batch, bool prepacked, int act_kind);
+// the forward kernel of this layer can leave `y` out (null) when it writes the activation layer
+// or the pool behind the convolution itself
+bool conv_fwd_out_optional(const tdh_conv_desc *d, int batch, bool prepacked);
 // conv_fwd_small.hip
 bool conv_fwd_small_applicable(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
                                int sh, int sw, int dh, int dw, int ph, int pw);
@@ -359,6 +362,9 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
 // a relu behind that pool); `out` may then be null
 bool conv_s1_fuses_pool(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
                         int ph, int pw);
+// one pass over the reduction channels: the kernel's epilogue is the only writer of `out`
+bool conv_s1_single_pass(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
+                         int ph, int pw);
 int conv_s1_repack(int R, int S, int C, int Kc, int flip, const float *w, const uint8_t *tbl_dev,
                    float *wp);
 // conv_dw.hip: stride-1 weight gradient from LDS-staged tiles (3x3 and 5x5 windows)

@@ -926,6 +926,13 @@ bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int 
          conv_s1_fuses_pool(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
 }
 
+bool conv_fwd_out_optional(const tdh_conv_desc *d, int batch, bool prepacked) {
+  const ConvGeom g = make_geom(d);
+  if (!prepacked && fwd_small_applies(g, batch)) return true;
+  return fwd_s1_applies(d, g, batch, prepacked) &&
+         conv_s1_single_pass(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
+}
+
 bool conv_fwd_pool_applies_act(const tdh_conv_desc *d, int batch, bool prepacked, int act_kind) {
   const ConvGeom g = make_geom(d);
   // the first-layer kernel applies any pointwise kind, the stride-1 kernel relu
@@ -962,8 +969,9 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
         (pool->act_out && !conv_fwd_pool_applies_act(d, batch, prepacked != nullptr, pool->act_kind)))
       return set_error(TDH_ERR_INVALID, "conv2d_fwd: this kernel does not compute the pool layer behind it");
   }
-  // (y null: only a kernel that also computes the pool behind the layer can leave it out)
-  if (!y && !pool) return set_error(TDH_ERR_INVALID, "conv2d_fwd: no output tensor");
+  // (y null: only a kernel that also writes the activation or the pool behind the layer can leave it out)
+  if (!y && !pool && !(act_out && conv_fwd_out_optional(d, batch, prepacked != nullptr)))
+    return set_error(TDH_ERR_INVALID, "conv2d_fwd: no output tensor");
   if (prepacked)
     return conv_s1_run(g.R, g.S, batch, g.C, g.Kc, 0, x, w, nullptr, d->has_bias ? b : nullptr, y, g.H,
                        g.W, g.OH, g.OW, g.pad_h, g.pad_w, ActGrad(), "conv_fwd_s1", prepacked, act_out,

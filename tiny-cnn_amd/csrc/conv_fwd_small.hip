@@ -499,7 +499,7 @@ int conv_fwd_small_run(int batch, int C, int Kc, const float *x, const float *w,
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: shape not supported");
   if (pool && ((OH | OW) & 1))
     return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: a fused 2x2 pool needs even output sizes");
-  if (!out && !pool) return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: no output");
+  if (!out && !pool && !act_out) return set_error(TDH_ERR_INVALID, "conv_fwd_small_run: no output");
   p.a.x = x; p.a.w = w; p.a.bias = bias; p.a.out = out;
   p.a.act_out  = act_out;
   p.a.act_kind = act_kind;

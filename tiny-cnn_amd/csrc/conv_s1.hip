@@ -152,6 +152,12 @@ bool conv_s1_applicable(int R, int S, int batch, int KC, int MC, int IH, int IW,
   return make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw).ok;
 }
 
+bool conv_s1_single_pass(int R, int S, int batch, int KC, int MC, int IH, int IW, int OH, int OW,
+                         int ph, int pw) {
+  const S1Plan p = make_plan(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw);
+  return p.ok && p.splits == 1;
+}
+
 // A 32-pixel accumulator block must hold whole 2x2 windows: rows of 8 or 16 pixels (tile rows
 // come in powers of two and start at even image rows), even image sizes, and one pass over the
 // reduction channels (the partial sums of a split have no maximum yet).
@@ -196,7 +202,8 @@ int conv_s1_run(int R, int S, int batch, int C, int Kc, int flip, const float *i
                (pool->act_out && pool->act_kind != TDH_ACT_RELU) ||
                !conv_s1_fuses_pool(R, S, batch, KC, MC, IH, IW, OH, OW, ph, pw)))
     return set_error(TDH_ERR_INVALID, "conv_s1_run: this shape does not compute the pool layer behind it");
-  if (!out && !pool) return set_error(TDH_ERR_INVALID, "conv_s1_run: no output tensor");
+  if (!out && !pool && !(act_out && p.splits == 1))
+    return set_error(TDH_ERR_INVALID, "conv_s1_run: no output tensor");
   const void *wp = prepacked;
   if (!prepacked) {
     void *fresh = nullptr;

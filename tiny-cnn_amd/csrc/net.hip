@@ -296,7 +296,10 @@ int forward(tdh_net *net, int batch, const float *x, bool packed = false, const 
           // nothing behind the convolution left its kernel and a max-pool reads the result
           LeaveSplitSum leave(ctx(), fuse && last == i && i + 1 < n &&
                                          net->layers[i + 1].spec.kind == TDH_L_MAXPOOL);
-          const bool own_out = !(training && pf.out && !act_out);
+          // (the backward pass reads the outputs of the layers that left the kernel, never the
+          // convolution's own: the gradients of the pointwise activations are functions of y)
+          const bool own_out = !(training && ((pf.out && !act_out) ||
+                                              (act_out && conv_fwd_out_optional(&s.conv, batch, wp != nullptr))));
           if (!own_out) net->out_unwritten[i] = 1;
           TDH_TRY(conv2d_fwd(&s.conv, batch, in, L.w, L.b, own_out ? L.out : nullptr, L.tbl_dev, wp, act_out, act_kind,
                              pf.out ? &pf : nullptr));
