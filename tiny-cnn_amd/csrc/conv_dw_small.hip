@@ -301,6 +301,13 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
       break;
   }
   if (best == 0) return p;
+  {
+    // the same number of bands, the rows spread evenly: 32 rows in bands of 10 are 10 + 10 +
+    // 10 + 2, and the workgroups of the last band idle while the others multiply
+    int even = ceil_div(OH, ceil_div(OH, best));
+    if (even_rows && even % 2 != 0) ++even;
+    best = std::min(best, even);
+  }
   a.band    = best;
   a.bands   = ceil_div(OH, best);
   a.chunk   = chunk_of(best);

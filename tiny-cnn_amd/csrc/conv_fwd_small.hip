@@ -452,6 +452,8 @@ FwdSmallPlan make_fwd_small_plan(int batch, int C, int Kc, int H, int W, int OH,
       break;
   }
   if (best == 0) return p;
+  // (the same number of bands, the rows spread evenly over them)
+  best      = std::min(best, (ceil_div(OH2, ceil_div(OH2, best)) + 1) & ~1);
   a.band    = best;
   a.bands   = ceil_div(OH, best);
   a.rows_in = (best - 1) * sh + (R - 1) * dh + 1;
