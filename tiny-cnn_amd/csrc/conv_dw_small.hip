@@ -164,13 +164,7 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
   };
   load_dy(0);
   load_x(tid);
-  store_dy(dys, 0);
-  store_x();
-  for (int e0 = tid + DEPTH * 256; e0 < x_total; e0 += DEPTH * 256) {
-    load_x(e0);
-    store_x();
-  }
-  // ---- per-lane constants of the B gather
+  // ---- per-lane constants of the B gather (worked out while the first loads are on their way)
   const int nl = lane & 31, half = lane >> 5;
   int off[NT];
   bool ones[NT];
@@ -186,6 +180,12 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
       o = ci * a.plane + ky * a.dh * a.pitch + kx * a.dw;
     }
     off[t] = o;
+  }
+  store_dy(dys, 0);
+  store_x();
+  for (int e0 = tid + DEPTH * 256; e0 < x_total; e0 += DEPTH * 256) {
+    load_x(e0);
+    store_x();
   }
   floatx16 acc[NT];
 #pragma unroll
@@ -236,14 +236,23 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
     }
   __syncthreads();
   const int blk = img * a.bands + bandi;
-  for (int e = tid; e < TILE; e += 256) {
+  // (all LDS reads of a thread first: read, add and store one output at a time is twelve trips
+  // to LDS one after the other)
+  float sums[TILE / 256];
+#pragma unroll
+  for (int i = 0; i < TILE / 256; ++i) {
+    const int e = tid + 256 * i;
+    sums[i]     = (dys[e] + dys[TILE + e]) + (dys[2 * TILE + e] + dys[3 * TILE + e]);
+  }
+#pragma unroll
+  for (int i = 0; i < TILE / 256; ++i) {
+    const int e = tid + 256 * i;
     const int m = e / (32 * NT), n = e - m * (32 * NT);
     if (co0 + m >= a.Kc || n > a.crs) continue;
-    const float s = (dys[e] + dys[TILE + e]) + (dys[2 * TILE + e] + dys[3 * TILE + e]);
     if (n < a.crs)
-      a.partial_dw[(static_cast<size_t>(blk) * a.Kc + co0 + m) * a.crs + n] = s;
+      a.partial_dw[(static_cast<size_t>(blk) * a.Kc + co0 + m) * a.crs + n] = sums[i];
     else if (a.partial_db)
-      a.partial_db[static_cast<size_t>(blk) * a.Kc + co0 + m] = s;
+      a.partial_db[static_cast<size_t>(blk) * a.Kc + co0 + m] = sums[i];
   }
 }
 
