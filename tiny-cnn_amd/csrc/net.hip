@@ -141,7 +141,7 @@ bool is_pointwise_act(int act) {
 // synchronisation costs more than it hides, and products that fill the chip for hundreds of
 // microseconds only fight the main chain for its caches (measured: LeNet-style net 5 % slower,
 // VGG-style 1 % slower, CIFAR-10-shape net 12 % faster with branches).
-bool net_forks(const tdh_net *net, int batch) {
+double net_forward_flop(const tdh_net *net, int batch) {
   double macs = 0.0;
   for (const tdh_net::Layer &L : net->layers) {
     if (L.spec.kind == TDH_L_CONV)
@@ -149,8 +149,20 @@ bool net_forks(const tdh_net *net, int batch) {
     else if (L.spec.kind == TDH_L_FC)
       macs += static_cast<double>(L.spec.fc_in) * L.spec.fc_out;
   }
-  const double flop = 2.0 * batch * macs;  // of the forward pass
+  return 2.0 * batch * macs;
+}
+bool net_forks(const tdh_net *net, int batch) {
+  const double flop = net_forward_flop(net, batch);
   return flop >= 1e8 && flop <= 3e10;
+}
+// A step too small to branch (LeNet-5 at batch 16) is a chain of launches of a few
+// microseconds each, and what counts is how many there are: it runs the branching step's
+// launches one after the other, so that the split sums of all weight gradients go to the
+// optimizer kernel and the row sums of all bias gradients leave as one pair of launches.
+// (With the graph flag only: a net created with it reserves every layer's scratch side by side.)
+bool net_defers_serially(const tdh_net *net, int batch) {
+  return (net->flags & TDH_NET_GRAPH) && (net->flags & TDH_NET_FUSE_ACT_GRAD) &&
+         net_forward_flop(net, batch) < 1e8;
 }
 bool layer_forks(const tdh_net::Layer &L) {
   return L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC;
@@ -700,7 +712,8 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     KeepScratch(Context &cc, bool o) : c(cc), on(o) {}
     void start() { if (on) { c.workspace_off = 0; c.ws_keep = true; } }
     ~KeepScratch() { c.ws_keep = false; }
-  } keep(c, forked || (!forked && profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch)));
+  } keep(c, forked || (!forked && ((profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch)) ||
+                                   net_defers_serially(net, batch))));
   bool side_used[2] = {false, false};
   bool last_dw_on_main = false;  // the last split sums were left behind the side stream's work
   // The split reductions behind the weight-gradient kernels and the row sums of the bias
@@ -719,7 +732,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   } deferred(c);
   // the per-kernel timing pass of a net whose captured step branches launches what that step
   // launches (a branching step computes dX, dW and db of a layer separately)
-  const bool as_forked = !forked && profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch);
+  const bool small_defers = !forked && net_defers_serially(net, batch);
+  const bool as_forked = !forked && ((profiling_active() && (net->flags & TDH_NET_GRAPH) && net_forks(net, batch)) ||
+                                     small_defers);
   const int n   = static_cast<int>(net->layers.size());
   // the optimizer kernel keeps the packed filters of the stride-1 kernels current
   const bool packed = net->packs_valid;
@@ -860,8 +875,11 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, db_with_dw ? L.db : nullptr, 1,
                              ActGrad(), L.tbl_dev, nullptr, gp));
           c.defer_reduce = false;
-          if (L.b_size && !db_with_dw)
+          if (L.b_size && !db_with_dw) {
+            c.defer_rowsum = small_defers;
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, nullptr, L.db, 1, ActGrad(), L.tbl_dev, nullptr, gp));
+            c.defer_rowsum = false;
+          }
         } else {
           LeaveSplitSum leave(c, pool_reads);
           TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1,
@@ -961,6 +979,8 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   }
   if (side_used[1]) {
     StreamSwap on_side(c.side[1]);
+    TDH_TRY(flush_deferred_rowsums());
+  } else if (small_defers) {
     TDH_TRY(flush_deferred_rowsums());
   }
   for (int k = 0; k < 2; ++k) {  // the optimizer (and the end of the capture) wait for the branches
