@@ -286,8 +286,9 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   // rows per chunk: at most 256 positions (eight 16-byte loads per thread); two chunks per band
   // where the band allows, so that loading overlaps the products
   const size_t reduce_fl = 4u * 32 * 32 * p.nt;
+  int chunk_cap = std::max(1, 256 / OW);  // rows per chunk at most
   auto chunk_of = [&](int band) {
-    int c = std::max(1, std::min(band, 256 / OW));
+    int c = std::max(1, std::min(band, chunk_cap));
     if (c == band && band > 1) c = (band + 1) / 2;
     if (even_rows) c = std::max(2, c & ~1);
     return c;
@@ -301,15 +302,47 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
   if (OW > 256) return p;
   // the largest band whose LDS fits twice per compute unit and that gives two workgroups per
   // compute unit; a band is not made shorter than 256 positions for that
-  int best = 0;
-  for (int band = OH; band >= 1; --band) {
-    if (even_rows && band % 2 != 0) continue;
-    if (lds_floats(band) * sizeof(float) > 72 * 1024) continue;
-    best = band;
-    if (static_cast<long long>(batch) * ceil_div(OH, band) * co_tiles >= 2LL * cus || band * OW <= 256)
-      break;
+  auto best_band = [&]() {
+    int best = 0;
+    for (int band = OH; band >= 1; --band) {
+      if (even_rows && band % 2 != 0) continue;
+      if (lds_floats(band) * sizeof(float) > 72 * 1024) continue;
+      best = band;
+      if (static_cast<long long>(batch) * ceil_div(OH, band) * co_tiles >= 2LL * cus || band * OW <= 256)
+        break;
+    }
+    return best;
+  };
+  // Wide rows: two chunk buffers of 256 positions leave LDS for a patch of two or three rows,
+  // and every workgroup then pays its prologue, its reduction over the waves and a partial
+  // slice for 256 positions (128-column images at batch 64: 8192 slices, 29 MB). Shorter
+  // chunks buy a longer band: taken where that at least doubles the band.
+  int best = best_band();
+  for (int cap = chunk_cap / 2; cap >= (even_rows ? 2 : 1); cap /= 2) {
+    const int keep = chunk_cap;
+    chunk_cap      = cap;
+    const int b    = best_band();
+    if (b >= 2 * best && b > 0) best = b;
+    else chunk_cap = keep;
   }
   if (best == 0) return p;
+  {
+    // a few bands more where that fills the last round of workgroups (two per compute unit run
+    // at a time): 768 workgroups are two rounds just as 1024 are
+    const long long slots = 2LL * cus;
+    auto fill = [&](int nb) {
+      const long long wgs = static_cast<long long>(batch) * nb * co_tiles;
+      return static_cast<double>(wgs) / static_cast<double>((wgs + slots - 1) / slots * slots);
+    };
+    int nb = ceil_div(OH, best), pick = nb;
+    for (int more = nb + 1; more <= std::min(OH, nb + nb / 2 + 1) && fill(pick) < 0.9; ++more)
+      if (fill(more) > fill(pick) + 0.05) pick = more;
+    if (pick != nb) {
+      int band = ceil_div(OH, pick);
+      if (even_rows && band % 2 != 0) ++band;
+      best = std::min(best, band);
+    }
+  }
   {
     // the same number of bands, the rows spread evenly: 32 rows in bands of 10 are 10 + 10 +
     // 10 + 2, and the workgroups of the last band idle while the others multiply
