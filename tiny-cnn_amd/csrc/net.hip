@@ -840,10 +840,9 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           if (i == 0 && (db_with_dw || !L.b_size)) {
             // The net's first layer: nothing waits for its dX, and its two kernels share nothing
             // and each fills the chip. Side by side they took 53 us on the CIFAR net, one after
-            // the other 33: the weight gradient follows on the main stream, behind the side
-            // stream's work.
-            TDH_HIP(hipEventRecord(net->events[2 * n], c.side[0]));
-            TDH_HIP(hipStreamWaitEvent(c.stream, net->events[2 * n], 0));
+            // the other 33: the weight gradient follows on the main stream. (It does not wait
+            // for the side stream: by then that stream's last kernel is about to end, and a
+            // wait across streams is 5 us of a replayed step whether or not it has to wait.)
             c.defer_reduce = true;
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, nullptr, L.dw, db_with_dw ? L.db : nullptr, 1,
                                ActGrad(), L.tbl_dev, nullptr, gp));
@@ -975,6 +974,10 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     StreamSwap on_side(c.side[0]);
     TDH_TRY(flush_deferred_reduces());
   } else if ((as_forked || last_dw_on_main) && !to_optimizer) {
+    if (last_dw_on_main && side_used[0]) {  // (the side stream's kernels wrote some of the slices)
+      TDH_HIP(hipEventRecord(net->events[2 * n], c.side[0]));
+      TDH_HIP(hipStreamWaitEvent(c.stream, net->events[2 * n], 0));
+    }
     TDH_TRY(flush_deferred_reduces());
   }
   if (side_used[1]) {
