@@ -336,6 +336,22 @@ def test_graph_replay_matches_eager_on_every_step(T, W, name, batch):
     graph.train_step(None, loss, batch, xd, td, do_update=False)
     for (i, which, a) in params:
         assert np.array_equal(eager.layer_grad(i, which), graph.layer_grad(i, which))
+    # what a step keeps out of memory is reported the same way after a replay; a forward pass
+    # writes every output, and the next replay reports its own state again
+    n = len(spec)
+    kept_out = [graph.out_written(i) for i in range(n)]
+    assert kept_out == [eager.out_written(i) for i in range(n)]
+    assert [graph.dx_written(i) for i in range(n)] == [eager.dx_written(i) for i in range(n)]
+    graph.forward(batch, xd)
+    eager.forward(batch, xd)
+    assert all(graph.out_written(i) for i in range(n))
+    for i in range(n):
+        assert np.array_equal(graph.layer_out(i, batch), eager.layer_out(i, batch)), i
+    eager.train_step(o1, loss, batch, xd, td)
+    graph.train_step(o2, loss, batch, xd, td)
+    assert [graph.out_written(i) for i in range(n)] == [eager.out_written(i) for i in range(n)]
+    for (i, which, a) in params:
+        assert np.array_equal(eager.get_param(i, which), graph.get_param(i, which)), (i, which)
     eager.close(); graph.close()
 
 
