@@ -10,6 +10,9 @@ vgg_stack_b64, lenet5_b16 (train steps), conv2d_bwd_b64 and fc_bwd_adam_b256 (si
 backward passes). Their results are appended under "others" in compact form (ms/step,
 samples/s, step TFLOP/s, the slowest kernels with their roofline fraction, a bounded CPU
 baseline), so that one run times all five configurations; ``--no-others`` leaves them out.
+Every timed region (whole steps and the per-kernel pass, of every workload) follows untimed
+steps that keep the device busy for 100 ms, the other workloads run at least 50 timed steps,
+and all CPU legs come after the last GPU measurement.
 
 "roofline" describes the kernel with the largest total time in the workload: its average
 launch duration is measured with HIP events on the library's stream in a second, separately
@@ -139,17 +142,30 @@ def roofline_of(entry):
             "algorithmic_work_per_launch": entry["work"]}
 
 
-def mark(T, marker):
-    """Three launches of the fill kernel on one small buffer: a pattern that a trace of this run
-    (which knows kernels by symbol only) can find, in front of every step of the per-kernel pass."""
-    for _ in range(3):
-        T.fill_zero(marker)
+WARM_MS = 100.0
+
+
+def warm_by_time(T, wl, min_ms=WARM_MS):
+    """Runs untimed steps until the device has been busy for `min_ms`: a GPU that has idled (a
+    CPU leg, a fresh process) clocks down, and a timed region of a few milliseconds would
+    otherwise be measured on the ramp. Returns the number of steps run."""
+    done, spent, chunk = 0, 0.0, 4
+    while spent < min_ms and done < 100000:
+        t0 = time.perf_counter()
+        for _ in range(chunk):
+            wl.step()
+        T.sync()
+        spent += (time.perf_counter() - t0) * 1e3
+        done += chunk
+        chunk = min(chunk * 2, 256)
+    return done
 
 
 def run_workload(T, wl, steps, warmup, profile_steps, sequence=None):
     for _ in range(warmup):
         wl.step()
     T.sync()
+    warm_by_time(T, wl)
     e0, e1 = T.Event(), T.Event()
     t0 = time.perf_counter()
     e0.record()
@@ -167,27 +183,29 @@ def run_workload(T, wl, steps, warmup, profile_steps, sequence=None):
     T.profile_begin()
     wl.step()
     T.profile_end()
+    warm_by_time(T, wl)
     marker = T.DevBuf((4400,), zero=True)
     T.profile_begin()
     for _ in range(profile_steps):
-        mark(T, marker)
+        T.profile_mark(marker)   # three fill launches under a tag of their own
         wl.step()
-    mark(T, marker)
+    T.profile_mark(marker)
     prof = T.profile_end()
     # the marks are not part of the workload
-    prof = [e for e in prof if not (e["tag"] == "fill_zero" and e["launches"] == 3 * (profile_steps + 1))]
+    prof = [e for e in prof if e["tag"] != "profile_mark"]
     if sequence is not None:  # the tags of one step's launches, in dispatch order
         tags = T.profile_launches()
         per = (len(tags) - 3) // profile_steps
         chunks = [tags[i * per:(i + 1) * per] for i in range(profile_steps)]
         assert per * profile_steps + 3 == len(tags) and all(c == chunks[0] for c in chunks) \
-            and chunks[0][:3] == ["fill_zero"] * 3, "the steps of the per-kernel pass differ"
+            and chunks[0][:3] == ["profile_mark"] * 3, "the steps of the per-kernel pass differ"
         sequence.extend(chunks[0][3:])
     kernels = [roofline_of(e) for e in prof]
     for k, e in zip(kernels, prof):
         k["ms_per_step"] = round(e["total_ms"] / profile_steps, 4)
     return {"ms_per_step": ms_per_step, "gpu_ms_per_step": gpu_ms / steps,
-            "samples_per_s": wl.samples / (ms_per_step * 1e-3), "kernels": kernels}
+            "samples_per_s": wl.samples / (ms_per_step * 1e-3), "kernels": kernels,
+            "profile_steps": profile_steps}
 
 
 def copy_yardstick(T, mib=256, reps=5):
@@ -338,41 +356,42 @@ def main():
                                         "frac": round(tot_flop / tot_s / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
     out["copy_yardstick"] = copy_yardstick(T)
     if hasattr(wl, "step_from_host"):  # never `value`: reported for callers that own host buffers
-        for _ in range(8):  # both device slots get their captured step
+        for _ in range(8):  # every device slot gets its captured step
             wl.step_from_host()
         T.sync()
+        host_steps = max(args.steps, 200)
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(host_steps):
             wl.step_from_host()
         T.sync()
-        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        ms = (time.perf_counter() - t0) * 1e3 / host_steps
         out["host_inputs"] = {"ms_per_step": round(ms, 4), "samples_per_s": round(wl.samples / (ms * 1e-3), 2),
+                              "steps": host_steps,
                               "note": "inputs and targets handed over in pageable host memory every step "
-                                      "and uploaded double-buffered (tdh_feeder)"}
+                                      "and uploaded through pinned slots on a copy stream (tdh_feeder)"}
     if wl.config.get("flop_per_step"):
         out["step_tflops"] = round(wl.config["flop_per_step"] / (res["ms_per_step"] * 1e-3) / 1e12, 3)
+    out["timing"] = {"warm_ms_before_each_timed_region": WARM_MS,
+                     "per_kernel_pass_steps": res["profile_steps"],
+                     "order": "all GPU timing first, every CPU baseline afterwards"}
     del wl
-    if not args.no_cpu_baseline:
-        try:
-            out["cpu_baseline"] = cpu_baseline(W, args.workload)
-            if out["cpu_baseline"]:
-                out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1)
-        except Exception as e:  # the baseline is reported, never required
-            out["cpu_baseline"] = {"error": repr(e)}
+    others = {}
     if not args.no_others:
-        # the other four configurations, compact: short timed runs, the six slowest kernels, and
-        # a CPU baseline capped at a few seconds each so that the whole run stays within minutes
-        others = {}
+        # the other four configurations, compact: the six slowest kernels each. Every GPU
+        # measurement of the run comes before the first CPU leg, so no timed region follows
+        # seconds of an idle device.
+        other_steps = max(50, args.steps)
         for name in ("conv2d_bwd_b64", "fc_bwd_adam_b256", "vgg_stack_b64", "lenet5_b16",
                      "cifar10_cnn_b128"):
             if name == args.workload:
                 continue
             w2 = make_workload(T, W, name)
-            r = run_workload(T, w2, max(5, args.steps // 2), max(2, args.warmup // 2), 5)
+            r = run_workload(T, w2, other_steps, max(2, args.warmup), 10)
             ks = r["kernels"]
             flop_k = [k for k in ks if k["bound"] == "mfma"]
             rec = {"samples_per_s": round(r["samples_per_s"], 2),
-                   "ms_per_step": round(r["ms_per_step"], 4), "config": w2.config,
+                   "ms_per_step": round(r["ms_per_step"], 4), "steps": other_steps,
+                   "config": w2.config,
                    "step_tflops": round(w2.config["flop_per_step"] / (r["ms_per_step"] * 1e-3) / 1e12, 3),
                    "roofline": {k: ks[0][k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac",
                                                       "avg_launch_us")} if ks else None,
@@ -386,14 +405,22 @@ def main():
                 rec["mfma_kernels_together"] = {"TFLOP/s": round(tot_flop / tot_s / 1e12, 2),
                                                 "frac": round(tot_flop / tot_s / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
             del w2
-            if not args.no_cpu_baseline:
-                try:
-                    rec["cpu_baseline"] = cpu_baseline(W, name, budget_s=4.0, max_steps=3)
-                    if rec["cpu_baseline"]:
-                        rec["gpu_over_cpu"] = round(rec["samples_per_s"] / rec["cpu_baseline"]["value"], 1)
-                except Exception as e:
-                    rec["cpu_baseline"] = {"error": repr(e)}
             others[name] = rec
+    if not args.no_cpu_baseline:
+        try:
+            out["cpu_baseline"] = cpu_baseline(W, args.workload)
+            if out["cpu_baseline"]:
+                out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1)
+        except Exception as e:  # the baseline is reported, never required
+            out["cpu_baseline"] = {"error": repr(e)}
+        for name, rec in others.items():  # capped at a few seconds each
+            try:
+                rec["cpu_baseline"] = cpu_baseline(W, name, budget_s=4.0, max_steps=3)
+                if rec["cpu_baseline"]:
+                    rec["gpu_over_cpu"] = round(rec["samples_per_s"] / rec["cpu_baseline"]["value"], 1)
+            except Exception as e:
+                rec["cpu_baseline"] = {"error": repr(e)}
+    if others:
         out["others"] = others
     print(json.dumps(out))
 

@@ -142,6 +142,10 @@ int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launche
  * launch outside any tag); TDH_ERR_INVALID (no error text) past the last one. It lets a trace
  * of the same run, which knows kernels only by symbol, be read tag by tag. */
 int tdh_profile_launch(int32_t index, char *tag, size_t tag_len);
+/* A mark in the kernel stream that a trace can find: three launches of the fill kernel on
+ * `dptr` (which they clear), booked under the tag "profile_mark", never under the tag of a
+ * workload's own fills. */
+int tdh_profile_mark(void *dptr, size_t bytes);
 
 /* shape helpers: conv_out_length / pool_out_length (tiny_dnn/util/util.h:329-363) */
 int tdh_conv_out_w(const tdh_conv_desc *d);
@@ -161,8 +165,10 @@ int tdh_conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const floa
 int tdh_conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w,
                    const float *dy, float *dx, float *dw, float *db, int accumulate);
 
-/* tdh_conv2d_bwd for callers that cannot allocate (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. Same
+/* tdh_conv2d_bwd for callers that cannot allocate (tight serving loops, harnesses that forbid
+ * hipMalloc). It has no counterpart in the reference. It is refused (TDH_ERR_INVALID) while a
+ * network step of this library is being captured or holds the scratch buffer, and
+ * (TDH_ERR_UNSUPPORTED) for a descriptor with a connection table. Same
  * arguments, kernels and results as tdh_conv2d_bwd, but the kernels' scratch (split partial
  * sums, repacked filters) lies in a static 64 MiB device array that the library holds on every
  * device it is initialised on, and the call allocates and frees nothing. A shape whose scratch

@@ -48,8 +48,51 @@ def elementwise_rel_err(got, want, floor=ELEMENTWISE_FLOOR):
     return float(np.max(np.abs(got - want) / scale))
 
 
+# Every comparison of a run leaves its figures here; a GPU run writes the maxima per test to
+# gpurun_out/parity_summary.json when the session ends (passing runs included).
+_PARITY_LOG = {}
+_CURRENT_TEST = [""]
+
+
+@pytest.fixture(autouse=True)
+def _name_the_running_test(request):
+    _CURRENT_TEST[0] = request.node.nodeid
+    yield
+    _CURRENT_TEST[0] = ""
+
+
+def pytest_sessionfinish(session, exitstatus):
+    if not _PARITY_LOG:
+        return
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out_dir, exist_ok=True)
+        worst = max(_PARITY_LOG.values(), key=lambda r: r["gate_max"])
+        worst_plain = max(_PARITY_LOG.values(), key=lambda r: r["elementwise_max"])
+        with open(os.path.join(out_dir, "parity_summary.json"), "w") as f:
+            json.dump({"gate": "|got-want| / max(|want|, rms(want))", "tolerance": REL_TOL,
+                       "elementwise": f"|got-want| / max(|want|, {ELEMENTWISE_FLOOR:g}*rms(want))",
+                       "comparisons": sum(r["comparisons"] for r in _PARITY_LOG.values()),
+                       "worst_gate": {"test": worst["test"], "what": worst["gate_what"], "value": worst["gate_max"]},
+                       "worst_elementwise": {"test": worst_plain["test"], "what": worst_plain["elementwise_what"],
+                                             "value": worst_plain["elementwise_max"]},
+                       "tests": sorted(_PARITY_LOG.values(), key=lambda r: -r["elementwise_max"])}, f, indent=1)
+    except OSError:
+        pass
+
+
 def assert_close(got, want, tol=REL_TOL, what=""):
     e = rel_err(got, want)
+    plain = elementwise_rel_err(got, want)
+    rec = _PARITY_LOG.setdefault(_CURRENT_TEST[0], {"test": _CURRENT_TEST[0], "comparisons": 0, "gate_max": 0.0,
+                                                    "gate_what": "", "elementwise_max": 0.0,
+                                                    "elementwise_what": "", "tolerance_max": 0.0})
+    rec["comparisons"] += 1
+    rec["tolerance_max"] = max(rec["tolerance_max"], tol)
+    if e >= rec["gate_max"]:
+        rec["gate_max"], rec["gate_what"] = e, what
+    if plain >= rec["elementwise_max"]:
+        rec["elementwise_max"], rec["elementwise_what"] = plain, what
     assert e <= tol, (f"{what}: relative error {e:.3e} > {tol:g} (plain element-wise, floor "
                       f"{ELEMENTWISE_FLOOR:g}*rms: {elementwise_rel_err(got, want):.3e})")
 

@@ -44,6 +44,56 @@ def test_static_scratch_calls_in_a_row_match_the_allocating_entry_point(T, O):
     run_both(T, O, (9, 7, 2, 3, 5, True, 3), 5, True)          # generic GEMM path, ragged
 
 
+def device_free_bytes():
+    """hipMemGetInfo of the current device, straight from the HIP runtime the library is linked to."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_static_scratch_calls_leave_device_memory_as_it_was(T):
+    """Nothing is allocated or freed by the call: the free memory of the device is the same before
+    and after, also for a first call of a shape (no scratch of the allocating kind has ever been
+    grown for it in this test) and for a smaller one behind it."""
+    shapes = [(16, 16, 32, 5, 48, True, 96), (8, 8, 16, 3, 24, True, 7)]
+    held = []
+    for (iw, ih, ic, k, oc, same, bs) in shapes:
+        d = T.conv_desc(iw, ih, ic, k, k, oc, pad_same=same)
+        ow, oh = T.conv_out_shape(d)
+        rng = np.random.default_rng(bs)
+        x = T.to_device(rng.standard_normal((bs, ic * ih * iw)).astype(np.float32))
+        w = T.to_device(rng.uniform(-0.3, 0.3, oc * ic * k * k).astype(np.float32))
+        dy = T.to_device(rng.standard_normal((bs, oc * oh * ow)).astype(np.float32))
+        held.append((d, bs, x, w, dy, T.DevBuf((bs, ic * ih * iw)), T.DevBuf((oc * ic * k * k,)), T.DevBuf((oc,))))
+    T.sync()
+    before = device_free_bytes()
+    for _ in range(2):
+        for (d, bs, x, w, dy, dx, dw, db) in held:
+            T.conv2d_bwd_static(d, bs, x, w, dy, dx, dw, db)
+    T.sync()
+    assert device_free_bytes() == before, "tdh_conv2d_bwd_static changed the device's free memory"
+    for (d, bs, x, w, dy, dx, dw, db) in held:   # and the results are those of the allocating call
+        want = [T.DevBuf(dx.shape), T.DevBuf(dw.shape), T.DevBuf(db.shape)]
+        T.conv2d_bwd(d, bs, x, w, dy, *want)
+        for g, r in zip((dx, dw, db), want):
+            assert np.array_equal(g.numpy(), r.numpy())
+
+
+def test_static_scratch_refuses_a_connection_table(T):
+    # the table would be staged through a host copy that the call has to wait for
+    tbl = np.ones((4, 6), np.uint8)
+    tbl[1, 2] = 0
+    d = T.conv_desc(8, 8, 4, 3, 3, 6, pad_same=True, tbl=tbl)
+    x, dy = T.DevBuf((2, 4 * 64), zero=True), T.DevBuf((2, 6 * 64), zero=True)
+    w = T.DevBuf((6 * 4 * 9,), zero=True)
+    dx, dw, db = T.DevBuf((2, 4 * 64)), T.DevBuf((6 * 4 * 9,)), T.DevBuf((6,))
+    with pytest.raises(T.TdhError, match="connection table"):
+        T.conv2d_bwd_static(d, 2, x, w, dy, dx, dw, db)
+    T.conv2d_bwd(d, 2, x, w, dy, dx, dw, db)       # the allocating entry point serves it
+
+
 def test_static_scratch_refuses_what_does_not_fit(T):
     # 768 -> 768 channels, 3x3 on 8x8 images, batch 32: 21 MB of filters whose gradient is summed
     # from several partial slices, about 120 MiB of scratch. The tensors have their real sizes,

@@ -278,6 +278,11 @@ def profile_launches():
     return out
 
 
+def profile_mark(buf):
+    """Three launches of the fill kernel on `buf`, booked under the tag "profile_mark"."""
+    check(lib().tdh_profile_mark(buf.ptr, C.c_size_t(buf.nbytes)), "tdh_profile_mark")
+
+
 def fill_zero(buf):
     check(lib().tdh_fill_zero(buf.ptr, C.c_size_t(buf.nbytes)), "tdh_fill_zero")
 

@@ -481,6 +481,14 @@ int tdh_profile_entry(int32_t index, char *tag, size_t tag_len, int64_t *launche
   return TDH_OK;
 }
 
+int tdh_profile_mark(void *dptr, size_t bytes) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(dptr != nullptr && bytes >= 4 && bytes % 4 == 0,
+                "tdh_profile_mark: needs a buffer of a positive multiple of 4 bytes");
+  for (int i = 0; i < 3; ++i) TDH_TRY(launch_fill_zero(dptr, bytes, "profile_mark"));
+  return TDH_OK;
+}
+
 int tdh_profile_launch(int32_t index, char *tag, size_t tag_len) {
   TDH_REQUIRE_INIT();
   if (index < 0 || index >= static_cast<int32_t>(g_launch_tags.size())) return TDH_ERR_INVALID;
@@ -530,6 +538,12 @@ int tdh_conv2d_bwd_static(const tdh_conv_desc *d, int batch, const float *x, con
   TDH_TRY(check_conv_desc(d, batch, true));
   if (batch == 0) return TDH_OK;
   TDH_CHECK_ARG(x && w && dy, "tdh_conv2d_bwd_static: null tensor");
+  // a connection table is uploaded from host memory through a staging copy that the call would
+  // have to wait for: neither fits a caller that may not allocate or synchronize
+  if (d->tbl)
+    return set_error(TDH_ERR_UNSUPPORTED,
+                     "tdh_conv2d_bwd_static: descriptors with a connection table are not served "
+                     "(the table is staged through a host copy); use tdh_conv2d_bwd");
   Context &c = ctx();
   TDH_CHECK_ARG(!c.ws_keep && !c.ws_locked, "tdh_conv2d_bwd_static: called inside a network step");
   const size_t need = conv2d_workspace_bytes(d, batch);

@@ -150,7 +150,7 @@ int pool_out_length(int in_length, int window, int stride, int ceil_mode, int pa
 
 // ------------------------------------------------- internal launchers (device ptrs)
 // elementwise.hip
-int launch_fill_zero(void *p, size_t bytes);
+int launch_fill_zero(void *p, size_t bytes, const char *tag = "fill_zero");
 int launch_copy(void *dst, const void *src, size_t bytes);  // bytes % 4 == 0
 // p: two constructor parameters (never null); x may be null unless the kind's gradient reads it
 int launch_act_fwd(int kind, const float *p, int batch, int len, const float *x, float *y);

@@ -483,6 +483,9 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
   int pj = -1;
   for (int k = 0; k < pend.n; ++k)
     if (pend.sum[k].g == t.g) pj = k;
+  // (the host hands over pending sums only for tensors with the small blocks; a tensor with
+  // large blocks would index pending_sum out of bounds, so it is left alone here)
+  if (t.block_elems != OPT_SUM_ELEMS_PER_BLOCK) pj = -1;
   if (pj >= 0) {
     const OptPendingSum ps = pend.sum[pj];
     constexpr uint32_t VEC = OPT_SUM_ELEMS_PER_BLOCK / 32;  // consecutive elements a lane adds up
@@ -688,8 +691,8 @@ colsum_kernel(const float *__restrict__ src, const int rows, const int cols,
 
 }  // namespace
 
-int launch_fill_zero(void *p, size_t bytes) {
-  ProfScope prof("fill_zero", static_cast<double>(bytes), WORK_BYTE);
+int launch_fill_zero(void *p, size_t bytes, const char *tag) {
+  ProfScope prof(tag, static_cast<double>(bytes), WORK_BYTE);
   const size_t n  = bytes / 4;
   const size_t n4 = aligned16(p) ? n / 4 : 0;
   TDH_LAUNCH(fill_zero_kernel, dim3(ew_blocks(n4 ? n4 + 3 : n)), dim3(EW_THREADS), 0,

@@ -19,6 +19,9 @@ struct tdh_net {
     float *dout = nullptr;  // gradient w.r.t. out; the next layer's backward writes it
     int32_t *argmax = nullptr;
     bool grad_folded = false;  // activation whose backward runs in the next layer's dX epilogue
+    // set where the optimizer table is built: the tensor's entry there has the small blocks
+    // (OPT_SUM_ELEMS_PER_BLOCK) that let the optimizer kernel add up K-split partial slices
+    bool w_sums_in_opt = false, b_sums_in_opt = false;
     // filters in the LDS-halo kernels' layout for forward / dX, packed on a side stream at the
     // start of a captured step (stride-1 conv layers of a TDH_NET_GRAPH net)
     float *wp_fwd = nullptr, *wp_dx = nullptr;  // kept current by the optimizer kernel
@@ -519,6 +522,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
         t.block_elems = (L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC) && (flags & TDH_NET_GRAPH)
                           ? OPT_SUM_ELEMS_PER_BLOCK : OPT_MULTI_ELEMS_PER_BLOCK;
         if (n > (1u << 22)) t.block_elems = OPT_MULTI_ELEMS_PER_BLOCK;  // (bandwidth matters there)
+        (which ? L.b_sums_in_opt : L.w_sums_in_opt) = t.block_elems == OPT_SUM_ELEMS_PER_BLOCK;
         block += static_cast<uint32_t>(ceil_div_sz(n, t.block_elems));
         net->opt_params += static_cast<double>(n);
         table.push_back(t);
@@ -963,8 +967,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     for (int k = 0; k < pending.n; ++k) {
       bool small_blocks = false;
       for (const tdh_net::Layer &L : net->layers)
-        if ((L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC) &&
-            ((pending.sum[k].g == L.dw && L.w_size <= (1u << 22)) || (pending.sum[k].g == L.db && L.b_size)))
+        if ((pending.sum[k].g == L.dw && L.w_sums_in_opt) || (pending.sum[k].g == L.db && L.b_sums_in_opt))
           small_blocks = true;
       to_optimizer = to_optimizer && small_blocks;
     }
