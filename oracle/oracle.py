@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_SO = os.path.join(HERE, "libtd_oracle.so")
 REF_SCALAR_SO = os.path.join(HERE, "_ref", "libtd_ref_scalar.so")
 REF_AVX_SO = os.path.join(HERE, "_ref", "libtd_ref_avx.so")
+REF_SER_SO = os.path.join(HERE, "_ref", "libtd_ref_ser.so")  # scalar build with serialization on
 
 ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3, "leaky_relu": 4, "elu": 5, "selu": 6,
        "softplus": 7, "softsign": 8, "asinh": 9, "tanh_p1m2": 10}
@@ -121,9 +122,10 @@ def oracle_lib():
 
 
 def ref_lib(kind="scalar"):
-    """The compiled reference ('scalar' or 'avx'), or None when it is not built."""
+    """The compiled reference ('scalar', 'avx', or 'ser': the scalar build with the
+    reference's cereal serialization compiled in), or None when it is not built."""
     if kind not in _ref:
-        path = REF_SCALAR_SO if kind == "scalar" else REF_AVX_SO
+        path = {"scalar": REF_SCALAR_SO, "avx": REF_AVX_SO, "ser": REF_SER_SO}[kind]
         if not os.path.exists(path):
             _ref[kind] = None
         else:
@@ -564,6 +566,14 @@ class RefNet:
 
     def load_weights(self, path):
         _chk(self.lib.tdr_net_load_weights(self.h, str(path).encode()), "load_weights")
+
+    # network::save / load with cereal archives (kind "ser" only): what 0 weights, 1 model,
+    # 2 weights_and_model; fmt 0 binary, 1 portable_binary, 2 json
+    def save_archive(self, path, what=0, fmt=0):
+        _chk(self.lib.tdr_net_save_archive(self.h, str(path).encode(), what, fmt), "save_archive")
+
+    def load_archive(self, path, what=0, fmt=0):
+        _chk(self.lib.tdr_net_load_archive(self.h, str(path).encode(), what, fmt), "load_archive")
 
     def set_random_seed(self, seed):
         """set_random_seed of the reference: its dropout layers draw from this generator"""

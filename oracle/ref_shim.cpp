@@ -604,6 +604,33 @@ int tdr_net_load_weights(tdr_net *h, const char *path) {
   } catch (const std::exception &) { return -1; }
 }
 
+/* network::save / load with cereal archives (tiny_dnn/network.h:676-728, to_archive /
+ * from_archive :787-811): what = content_type (0 weights, 1 model, 2 weights_and_model),
+ * format = file_format (0 binary, 1 portable_binary, 2 json). Only in the build without
+ * CNN_NO_SERIALIZATION; -3 elsewhere. */
+int tdr_net_save_archive(tdr_net *h, const char *path, int what, int format) {
+#ifndef CNN_NO_SERIALIZATION
+  try {
+    h->net.save(path, static_cast<content_type>(what), static_cast<file_format>(format));
+    return 0;
+  } catch (const std::exception &) { return -1; }
+#else
+  (void)h; (void)path; (void)what; (void)format;
+  return -3;
+#endif
+}
+int tdr_net_load_archive(tdr_net *h, const char *path, int what, int format) {
+#ifndef CNN_NO_SERIALIZATION
+  try {
+    h->net.load(path, static_cast<content_type>(what), static_cast<file_format>(format));
+    return 0;
+  } catch (const std::exception &) { return -1; }
+#else
+  (void)h; (void)path; (void)what; (void)format;
+  return -3;
+#endif
+}
+
 /* io/mnist_parser.h, io/cifar10_parser.h. out_images: [count][len] floats (may be NULL to
  * query), out_labels: [count] int64. Returns the number of items, -1 on nn_error. */
 long tdr_parse_mnist_images(const char *path, float scale_min, float scale_max, int x_pad, int y_pad,

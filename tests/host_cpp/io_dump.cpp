@@ -3,6 +3,8 @@
 //   io_dump mnist_images <file> <scale_min> <scale_max> <x_pad> <y_pad> <out>
 //   io_dump mnist_labels <file> <out>
 //   io_dump cifar10 <file> <scale_min> <scale_max> <x_pad> <y_pad> <out>
+//   io_dump archive <file> <format: 0 binary, 1 portable_binary> <out> <vectors of layer 0> <of layer 1> ...
+//           (reads a weights archive with the mirror's reader and writes it again with its writer)
 // <out>: int64 count, int64 length, then count*length float32 (images) and count int64 (labels).
 // Exit status 3 and the message on stdout when the reader throws nn_error.
 #include <cstdio>
@@ -33,7 +35,18 @@ int main(int argc, char **argv) {
   try {
     std::vector<vec_t> images;
     std::vector<label_t> labels;
-    if (!std::strcmp(argv[1], "mnist_labels")) {
+    if (argc >= 5 && !std::strcmp(argv[1], "archive")) {
+      const file_format format = std::atoi(argv[3]) ? file_format::portable_binary : file_format::binary;
+      std::vector<size_t> counts;
+      for (int i = 5; i < argc; ++i) counts.push_back(static_cast<size_t>(std::atoi(argv[i])));
+      std::ifstream is(argv[2], std::ios::binary);
+      if (!is.good()) throw nn_error(std::string("failed to open:") + argv[2]);
+      const std::vector<detail::archive_layer> layers = detail::read_weight_archive(is, counts, format);
+      std::ofstream os(argv[4], std::ios::binary);
+      detail::write_weight_archive(os, layers, format);
+      for (const detail::archive_layer &l : layers) std::printf("%s ", l.type.c_str());
+      std::puts("");
+    } else if (!std::strcmp(argv[1], "mnist_labels")) {
       parse_mnist_labels(argv[2], &labels);
       dump(argv[3], images, labels);
     } else if (argc == 8 && !std::strcmp(argv[1], "mnist_images")) {

@@ -880,6 +880,38 @@ static void weight_files() {
     threw = true;
   }
   EXPECT(threw);
+
+  // cereal archives (network.h:676-728): weights in binary and portable_binary, bit for bit
+  std::puts("network save / load with content_type::weights, binary and portable_binary");
+  for (file_format fmt : {file_format::binary, file_format::portable_binary}) {
+    network<sequential> d;
+    make(d);
+    const std::string p1 = "/tmp/tdh_test_weights.bin", p2 = "/tmp/tdh_test_weights2.bin";
+    a.save(p1, content_type::weights, fmt);
+    d.load(p1, content_type::weights, fmt);
+    for (size_t i = 0; i < 4; ++i)
+      for (int which = 0; which < 2; ++which)
+        if (sizes[i][which]) EXPECT(d.weights(i, which) == a.weights(i, which));
+    d.save(p2, content_type::weights, fmt);
+    std::ifstream f1(p1, std::ios::binary), f2(p2, std::ios::binary);
+    const std::string b1((std::istreambuf_iterator<char>(f1)), std::istreambuf_iterator<char>());
+    const std::string b2((std::istreambuf_iterator<char>(f2)), std::istreambuf_iterator<char>());
+    // 4 type names ("conv", "tanh", "avepool", "fully_connected") + 6 vectors of 54,3,12,3,240,5
+    const size_t want = (fmt == file_format::portable_binary ? 1 : 0) + 4 * 8 + 4 + 4 + 7 + 15 + 6 * 8 + 317 * 4;
+    EXPECT(b1 == b2 && b1.size() == want);
+    EXPECT(b1.compare(fmt == file_format::portable_binary ? 9 : 8, 4, "conv") == 0);
+  }
+  int refused = 0;
+  try { a.save("/tmp/tdh_test_weights.bin"); } catch (const nn_error &) { ++refused; }             // model: not built
+  try { a.load("/tmp/tdh_test_weights.bin", content_type::weights, file_format::json); } catch (const nn_error &) { ++refused; }
+  try { a.load("/tmp/tdh_no_such_file", content_type::weights); } catch (const nn_error &) { ++refused; }
+  {
+    network<sequential> other;   // another architecture: the vector lengths do not fit
+    other << fully_connected_layer(48, 5);
+    try { other.load("/tmp/tdh_test_weights.bin", content_type::weights, file_format::portable_binary); }
+    catch (const nn_error &) { ++refused; }
+  }
+  EXPECT(refused == 4);
 }
 
 int main() {

@@ -869,6 +869,34 @@ def test_weight_files_round_trip_with_the_reference(T, tmp_path):
         io.load_weights(T.Net(nets["weights_avepool"], 2), str(tmp_path / "weights_plain.txt"))
 
 
+def test_weight_archives_round_trip_with_the_reference(T, W, tmp_path):
+    """The cereal archives that the reference's network::save(file, content_type::weights, ...)
+    wrote (tests/golden/archives.npz) load into the device network bit for bit, and what the
+    device network writes is byte for byte the reference's file, in both binary formats."""
+    import importlib, os
+    io = importlib.import_module("tiny-cnn_amd.io")
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "archives.npz"))
+    specs = {"avepool": [("conv", 8, 8, 2, 3, 3, True), ("act", "tanh"), ("avepool", 8, 8, 3, 2),
+                         ("act", "leaky_relu", (0.05, 0.0)), ("fc", 48, 5), ("act", "softmax")],
+             "lenet5_mnist": W.lenet5_mnist(), "cifar10_cnn": W.cifar10_cnn(),
+             "bn_dropout": [("fc", 12, 8), ("batchnorm", 8, 1), ("act", "relu"), ("dropout", 0.3), ("fc", 8, 4),
+                            ("act", "tanh_p1m2")]}
+    for name, spec in specs.items():
+        for fmt in ("binary", "portable_binary"):
+            path = str(tmp_path / f"{name}.{fmt}")
+            g[f"{name}.{fmt}"].tofile(path)
+            net = T.Net(W.build_layers(T, spec), 2, T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
+            io.load_weights_archive(net, path, fmt)
+            for k, (i, which, n) in enumerate(net.params()):
+                assert np.array_equal(net.get_param(i, which), g[f"{name}.param{k}"]), (name, fmt, k)
+            out = path + ".out"
+            io.save_weights_archive(net, out, fmt)
+            assert open(out, "rb").read() == open(path, "rb").read(), (name, fmt)
+            net.close()
+    with pytest.raises(ValueError, match="holds|ends inside"):
+        io.load_weights_archive(T.Net(W.build_layers(T, specs["avepool"]), 2), str(tmp_path / "bn_dropout.binary"))
+
+
 @pytest.mark.parametrize("flags", [0, 1, 3])
 def test_net_with_batchnorm_and_dropout_matches_oracle_and_reference_fit(T, O, W, net_steps, flags):
     """batch_normalization_layer and dropout_layer as layer kinds of the device-resident step:

@@ -123,3 +123,132 @@ def test_weight_text_matches_network_save(io, golden):
         # eight significant digits do not always round-trip a float: the reference's own
         # save/load has the same loss; the parsed value is the float nearest to the text
         assert np.allclose(back, want, rtol=1e-7, atol=0) and back.dtype == np.float32
+
+
+# ------------------------------------------------------------------ cereal weight archives
+ARCHIVE_NETS = {
+    "avepool": [("conv", 8, 8, 2, 3, 3, True), ("act", "tanh"), ("avepool", 8, 8, 3, 2),
+                ("act", "leaky_relu", (0.05, 0.0)), ("fc", 48, 5), ("act", "softmax")],
+    "lenet5_mnist": "lenet5_mnist",
+    "bn_dropout": [("fc", 12, 8), ("batchnorm", 8, 1), ("act", "relu"), ("dropout", 0.3), ("fc", 8, 4),
+                   ("act", "tanh_p1m2")],
+    "cifar10_cnn": "cifar10_cnn",
+}
+
+
+@pytest.fixture(scope="module")
+def archives():
+    return np.load(os.path.join(GOLDEN, "archives.npz"))
+
+
+def archive_layout(io, name):
+    """(layer descriptors, type names, per layer: [(parameter index, file length)]) of a fixture net."""
+    T = importlib.import_module("tiny-cnn_amd")
+    W = importlib.import_module("tiny-cnn_amd.workloads")
+    spec = ARCHIVE_NETS[name]
+    spec = getattr(W, spec)() if isinstance(spec, str) else spec
+    layers = W.build_layers(T, spec)
+    names, slots, k = [], [], 0
+    for l, desc in zip(spec, layers):
+        names.append(io.archive_type_name(desc))
+        nw, nb, _, _ = W.layer_fans(l)
+        here = []
+        if nw:
+            here.append((k, nw * (l[4] * l[4] if l[0] == "avepool" else 1)))
+            k += 1
+        if nb:
+            here.append((k, nb))
+            k += 1
+        slots.append(here)
+    return layers, names, slots
+
+
+def test_weight_archives_match_network_save(io, archives):
+    """weights_to_archive is byte for byte what the compiled reference's network::save(file,
+    content_type::weights, binary / portable_binary) wrote for the same weights, and
+    archive_to_weights reads those files back to the same values."""
+    for name in ARCHIVE_NETS:
+        _, names, slots = archive_layout(io, name)
+        vectors = []
+        for here in slots:
+            vs = []
+            for (k, length) in here:
+                a = archives[f"{name}.param{k}"]
+                vs.append(np.concatenate([a, np.zeros(length - a.size, np.float32)]))
+            vectors.append(vs)
+        for fmt in ("binary", "portable_binary"):
+            want = archives[f"{name}.{fmt}"].tobytes()
+            assert io.weights_to_archive(names, vectors, fmt) == want, (name, fmt)
+            back = io.archive_to_weights(want, [len(h) for h in slots], fmt)
+            assert [n for n, _ in back] == names
+            for (_, got), vs in zip(back, vectors):
+                assert len(got) == len(vs) and all(np.array_equal(g, v) for g, v in zip(got, vs))
+        assert archives[f"{name}.portable_binary"].tobytes() == b"\x01" + archives[f"{name}.binary"].tobytes()
+
+
+def test_weight_archive_errors_and_big_endian_files(io, archives):
+    raw = archives["avepool.binary"].tobytes()
+    _, names, slots = archive_layout(io, "avepool")
+    counts = [len(h) for h in slots]
+    with pytest.raises(ValueError, match="ends inside"):
+        io.archive_to_weights(raw[:-3], counts, "binary")
+    with pytest.raises(ValueError, match="binary or portable_binary"):
+        io.archive_to_weights(raw, counts, "json")
+    # a portable archive written on a big-endian host: flag 0, every field byte-swapped
+    layers = io.archive_to_weights(raw, counts, "binary")
+    swapped = [b"\x00"]
+    for name, vectors in layers:
+        swapped.append(np.array(len(name), ">u8").tobytes() + name.encode())
+        for v in vectors:
+            swapped.append(np.array(v.size, ">u8").tobytes() + v.astype(">f4").tobytes())
+    back = io.archive_to_weights(b"".join(swapped), counts, "portable_binary")
+    for (n0, v0), (n1, v1) in zip(layers, back):
+        assert n0 == n1 and all(np.array_equal(a, b) for a, b in zip(v0, v1))
+
+
+def test_cpp_archive_reader_and_writer_round_trip_the_reference_files(io, io_dump, archives, tmp_path):
+    """The mirror's read_weight_archive / write_weight_archive (what network::save / load of
+    tiny_dnn_hip.h sit on) reproduce the reference's files byte for byte."""
+    for name in ARCHIVE_NETS:
+        _, names, slots = archive_layout(io, name)
+        for code, fmt in ((0, "binary"), (1, "portable_binary")):
+            src, dst = str(tmp_path / f"{name}.{fmt}"), str(tmp_path / f"{name}.{fmt}.out")
+            archives[f"{name}.{fmt}"].tofile(src)
+            r = subprocess.run([io_dump, "archive", src, str(code), dst] + [str(len(h)) for h in slots],
+                               capture_output=True, text=True)
+            assert r.returncode == 0, r.stdout
+            assert r.stdout.split() == names
+            assert np.array_equal(np.fromfile(dst, np.uint8), archives[f"{name}.{fmt}"])
+    short = str(tmp_path / "short.bin")
+    archives["avepool.binary"][:100].tofile(short)
+    _, _, slots = archive_layout(io, "avepool")
+    r = subprocess.run([io_dump, "archive", short, "0", str(tmp_path / "x")] + [str(len(h)) for h in slots],
+                       capture_output=True, text=True)
+    assert r.returncode == 3 and "ends inside" in r.stdout
+
+
+def test_compiled_reference_loads_the_archives_written_here(io, archives, tmp_path):
+    """Where oracle/_ref is built with serialization: network::load of the reference itself reads
+    a file written by weights_to_archive and ends up with the weights that went in."""
+    from oracle import oracle as O
+    if O.ref_lib("ser") is None:
+        pytest.skip("oracle/_ref/libtd_ref_ser.so is not built (needs the tiny-dnn tree)")
+    W = importlib.import_module("tiny-cnn_amd.workloads")
+    rng = np.random.default_rng(77)
+    for name in ("avepool", "bn_dropout"):
+        spec = ARCHIVE_NETS[name]
+        _, names, slots = archive_layout(io, name)
+        vectors = [[rng.standard_normal(length).astype(np.float32) for (_, length) in here] for here in slots]
+        for code, fmt in ((0, "binary"), (1, "portable_binary")):
+            path = str(tmp_path / f"{name}.{fmt}")
+            with open(path, "wb") as f:
+                f.write(io.weights_to_archive(names, vectors, fmt))
+            net = O.RefNet(W.build_layers(O, spec), "ser", 0)
+            net.load_archive(path, 0, code)
+            for li, vs in enumerate(vectors):
+                which = 0
+                for v in vs:
+                    while net.param_size(li, which) == 0:
+                        which += 1
+                    assert np.array_equal(net.get_param(li, which), v), (name, fmt, li, which)
+                    which += 1

@@ -1025,6 +1025,9 @@ class layer {
   virtual ~layer() {}
   virtual layer_desc describe(const shape3d &prev_out) const = 0;
   virtual std::string layer_type() const = 0;
+  // the name the reference registers for the class (tiny_dnn/util/serialization_layer_list.h),
+  // which serialize_prolog writes in front of a layer's weights in a cereal archive
+  virtual std::string archive_type_name() const = 0;
   // number of incoming connections of an output unit / outgoing ones of an input unit, which
   // the initialisers scale by (layer.h:298-306)
   virtual size_t fan_in_size() const { return 0; }
@@ -1081,6 +1084,7 @@ class convolutional_layer : public layer {
     kernel_back_.reset(new Conv2dGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "conv"; }
+  std::string archive_type_name() const override { return "conv"; }
   // convolutional_layer.h:269-277
   size_t fan_in_size() const override { return params_.weight.width_ * params_.weight.height_ * params_.in.depth_; }
   size_t fan_out_size() const override {
@@ -1140,6 +1144,7 @@ class fully_connected_layer : public layer {
     kernel_back_.reset(new FullyConnectedGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "fully-connected"; }
+  std::string archive_type_name() const override { return "fully_connected"; }
   size_t fan_in_size() const override { return params_.in_size_; }     // fully_connected_layer.h:51-53
   size_t fan_out_size() const override { return params_.out_size_; }
   void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
@@ -1201,6 +1206,7 @@ class max_pooling_layer : public layer {
     kernel_back_.reset(new MaxPoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "max-pool"; }
+  std::string archive_type_name() const override { return "maxpool"; }
   std::vector<shape3d> out_shape() const { return {params_.out}; }
   // maxpool_params::out2inmax of the last forward pass (downloads the device records if they
   // are the newer ones)
@@ -1254,6 +1260,7 @@ class average_pooling_layer : public layer {
     kernel_back_.reset(new AvePoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
   }
   std::string layer_type() const override { return "ave-pool"; }
+  std::string archive_type_name() const override { return "avepool"; }
   // partial_connected_layer.h:46-48 with the connections of average_pooling_layer.h:270-304:
   // every output reads pool_x*pool_y inputs, every input feeds one output (windows that tile)
   size_t fan_in_size() const override { return params_.pool_size_x * params_.pool_size_y; }
@@ -1294,6 +1301,11 @@ class average_pooling_layer : public layer {
 class activation_layer : public layer {
  public:
   std::string layer_type() const override { return type_; }
+  std::string archive_type_name() const override {
+    static const char *const names[] = {"tanh", "relu", "softmax", "sigmoid", "leaky_relu", "elu", "selu",
+                                        "softplus", "softsign", "asinh", "tanh_scaled"};
+    return names[kind_];
+  }
   // *_layer::scale() of the reference's activations: tanh and asinh (-0.8, 0.8), softmax (0, 1),
   // all others (0.1, 0.9)
   std::pair<float_t, float_t> out_value_range() const override {
@@ -1444,6 +1456,7 @@ class batch_normalization_layer : public layer {
       buf_(new detail::norm_buffers()) {}
 
   std::string layer_type() const override { return "batch-norm"; }
+  std::string archive_type_name() const override { return "batchnorm"; }
   layer_desc describe(const shape3d &) const override {
     layer_desc r;
     std::memset(&r.l, 0, sizeof(r.l));
@@ -1552,6 +1565,7 @@ class dropout_layer : public layer {
       in_size_(in_dim), mask_(1, std::vector<uint8_t>(in_dim)), buf_(new detail::norm_buffers()) {}
 
   std::string layer_type() const override { return "dropout"; }
+  std::string archive_type_name() const override { return "dropout"; }
   layer_desc describe(const shape3d &) const override {
     layer_desc r;
     std::memset(&r.l, 0, sizeof(r.l));
@@ -1657,6 +1671,95 @@ class feeder {
   size_t x_len_, t_len_;
   std::vector<float> x_, t_;
 };
+}  // namespace detail
+
+// tiny_dnn/network.h:32-38
+enum class content_type { weights, model, weights_and_model };
+enum class file_format { binary, portable_binary, json };
+
+namespace detail {
+// Weights-only cereal archives as network::save(filename, content_type::weights, binary /
+// portable_binary) writes them (tiny_dnn/network.h:676-728,787-811, nodes::save_weights
+// tiny_dnn/nodes.h:203-214): per layer the registered type name as a string (u64 length +
+// bytes; serialize_prolog, tiny_dnn/util/serialization_helper.h:118-123), then every trainable
+// vector as u64 element count + float32 values (serialization_functions.h:747-754). A
+// portable_binary archive starts with one byte: 1 when what follows is little-endian, which is
+// what cereal writes on such a host and what is written here.
+struct archive_layer {
+  std::string type;
+  std::vector<vec_t> vectors;
+};
+inline void put_u64(std::ostream &os, uint64_t v) {
+  unsigned char b[8];
+  for (int i = 0; i < 8; ++i) b[i] = static_cast<unsigned char>(v >> (8 * i));
+  os.write(reinterpret_cast<const char *>(b), 8);
+}
+inline void write_weight_archive(std::ostream &os, const std::vector<archive_layer> &layers, file_format format) {
+  if (format != file_format::binary && format != file_format::portable_binary)
+    throw nn_error("invalid serialization format");
+  if (format == file_format::portable_binary) os.put(char(1));
+  for (const archive_layer &l : layers) {
+    put_u64(os, l.type.size());
+    os.write(l.type.data(), static_cast<std::streamsize>(l.type.size()));
+    for (const vec_t &v : l.vectors) {
+      put_u64(os, v.size());
+      for (float_t f : v) {  // little-endian float32, whatever the host
+        uint32_t bits;
+        std::memcpy(&bits, &f, 4);
+        const unsigned char b[4] = {static_cast<unsigned char>(bits), static_cast<unsigned char>(bits >> 8),
+                                    static_cast<unsigned char>(bits >> 16), static_cast<unsigned char>(bits >> 24)};
+        os.write(reinterpret_cast<const char *>(b), 4);
+      }
+    }
+  }
+}
+// vector_counts[i]: trainable vectors of layer i. Throws nn_error when the stream ends early.
+inline std::vector<archive_layer> read_weight_archive(std::istream &is, const std::vector<size_t> &vector_counts,
+                                                      file_format format) {
+  if (format != file_format::binary && format != file_format::portable_binary)
+    throw nn_error("invalid serialization format");
+  bool little = true;
+  if (format == file_format::portable_binary) {
+    const int flag = is.get();
+    if (flag == std::char_traits<char>::eof()) throw nn_error("archive is empty");
+    little = flag != 0;
+  }
+  auto bytes = [&](unsigned char *dst, size_t n) {
+    is.read(reinterpret_cast<char *>(dst), static_cast<std::streamsize>(n));
+    if (static_cast<size_t>(is.gcount()) != n) throw nn_error("archive ends inside a layer record");
+  };
+  auto u64 = [&]() {
+    unsigned char b[8];
+    bytes(b, 8);
+    uint64_t v = 0;
+    for (int i = 0; i < 8; ++i) v |= static_cast<uint64_t>(b[i]) << (8 * (little ? i : 7 - i));
+    return v;
+  };
+  std::vector<archive_layer> out;
+  for (size_t count : vector_counts) {
+    archive_layer l;
+    const uint64_t name_len = u64();
+    if (name_len > 4096) throw nn_error("archive: a layer name of " + std::to_string(name_len) + " bytes");
+    l.type.resize(name_len);
+    if (name_len) bytes(reinterpret_cast<unsigned char *>(&l.type[0]), name_len);
+    for (size_t k = 0; k < count; ++k) {
+      const uint64_t n = u64();
+      if (n > (uint64_t(1) << 32)) throw nn_error("archive: a weight vector of " + std::to_string(n) + " values");
+      vec_t v(n);
+      std::vector<unsigned char> raw(4 * n);
+      if (n) bytes(raw.data(), raw.size());
+      for (uint64_t i = 0; i < n; ++i) {
+        const unsigned char *b = raw.data() + 4 * i;
+        const uint32_t bits = little ? (uint32_t(b[0]) | uint32_t(b[1]) << 8 | uint32_t(b[2]) << 16 | uint32_t(b[3]) << 24)
+                                     : (uint32_t(b[3]) | uint32_t(b[2]) << 8 | uint32_t(b[1]) << 16 | uint32_t(b[0]) << 24);
+        std::memcpy(&v[i], &bits, 4);
+      }
+      l.vectors.push_back(std::move(v));
+    }
+    out.push_back(std::move(l));
+  }
+  return out;
+}
 }  // namespace detail
 
 struct sequential {};
@@ -1812,6 +1915,54 @@ class network<sequential> {
       }
     initialized_ = true;
   }
+  // network::save / load (tiny_dnn/network.h:676-728) with the reference's arguments and
+  // defaults. content_type::weights in binary or portable_binary is read and written, byte for
+  // byte the reference's files; the model description (content_type::model and the default
+  // weights_and_model) and json are not part of this library and raise nn_error.
+  void save(const std::string &filename, content_type what = content_type::weights_and_model,
+            file_format format = file_format::binary) {
+    require_weights_archive(what, format);
+    build(max_batch_ ? max_batch_ : 1);
+    std::vector<detail::archive_layer> layers(layers_.size());
+    for (size_t i = 0; i < layers_.size(); ++i) {
+      layers[i].type = layers_[i]->archive_type_name();
+      for (int which = 0; which < 2; ++which) {
+        vec_t v = weights(i, which);
+        if (v.empty()) continue;
+        v.resize(file_length(i, which), float_t(0));
+        layers[i].vectors.push_back(std::move(v));
+      }
+    }
+    std::ofstream ofs(filename.c_str(), std::ios::binary | std::ios::out);
+    if (ofs.fail() || ofs.bad()) throw nn_error("failed to open:" + filename);
+    detail::write_weight_archive(ofs, layers, format);
+  }
+  void load(const std::string &filename, content_type what = content_type::weights_and_model,
+            file_format format = file_format::binary) {
+    require_weights_archive(what, format);
+    std::ifstream ifs(filename.c_str(), std::ios::binary | std::ios::in);
+    if (ifs.fail() || ifs.bad()) throw nn_error("failed to open:" + filename);
+    build(max_batch_ ? max_batch_ : 1);
+    std::vector<size_t> counts(layers_.size(), 0);
+    for (size_t i = 0; i < layers_.size(); ++i)
+      for (int which = 0; which < 2; ++which)
+        if (tdh_net_param_size(net_, static_cast<int>(i), which)) ++counts[i];
+    const std::vector<detail::archive_layer> layers = detail::read_weight_archive(ifs, counts, format);
+    for (size_t i = 0; i < layers_.size(); ++i) {
+      size_t k = 0;
+      for (int which = 0; which < 2; ++which) {
+        const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which);
+        if (!n) continue;
+        const vec_t &v = layers[i].vectors[k++];
+        if (v.size() != file_length(i, which))
+          throw nn_error("load: layer " + std::to_string(i) + " of the archive holds " + std::to_string(v.size()) +
+                         " values, the network's " + std::to_string(file_length(i, which)));
+        set_weights(i, which, vec_t(v.begin(), v.begin() + n));
+      }
+    }
+    initialized_ = true;
+  }
+
   // network::fast_load (tiny_dnn/network.h:777-785): the same file through fscanf
   void fast_load(const char *filepath) {
     FILE *stream = std::fopen(filepath, "r");
@@ -2042,6 +2193,14 @@ class network<sequential> {
     last_numeric_ = delta_by_numerical;
     last_bprop_   = delta_by_bprop;
     return std::abs(delta_by_bprop - delta_by_numerical) <= eps;
+  }
+  static void require_weights_archive(content_type what, file_format format) {
+    if (what != content_type::weights)
+      throw nn_error("save/load: only content_type::weights is built; the model description is not part of "
+                     "this library");
+    if (format == file_format::json) throw nn_error("save/load: json archives are not built");
+    if (format != file_format::binary && format != file_format::portable_binary)
+      throw nn_error("invalid serialization format");
   }
   // entries of trainable vector `which` of layer i in a weight file
   size_t file_length(size_t i, int which) {

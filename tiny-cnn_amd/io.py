@@ -131,3 +131,101 @@ def load_weights(net, path):
                 raise ValueError("load_weights: the file holds fewer weights than the network")
             net.set_param(i, which, data[at:at + n])
             at += length
+
+
+# ------------------------------------------------------------------ cereal weight archives
+# network::save(filename, content_type::weights, file_format::binary / portable_binary)
+# (tiny_dnn/network.h:676-728, to_archive :787-799, nodes::save_weights tiny_dnn/nodes.h:203-214):
+# for every layer in order, the layer's registered type name (serialize_prolog,
+# tiny_dnn/util/serialization_helper.h:118-123; names in serialization_layer_list.h) as a string
+# = u64 length + bytes, then every trainable vector (serialization_functions.h:747-754) as u64
+# element count + float32 values. A portable_binary archive starts with one byte that says
+# whether what follows is little-endian (cereal writes 1 on such a host). Batch-norm running
+# averages are not trainable vectors and are not in these files.
+ACT_TYPE_NAMES = {0: "tanh", 1: "relu", 2: "softmax", 3: "sigmoid", 4: "leaky_relu", 5: "elu",
+                  6: "selu", 7: "softplus", 8: "softsign", 9: "asinh", 10: "tanh_scaled"}
+LAYER_TYPE_NAMES = {0: "conv", 1: "fully_connected", 2: "maxpool", 3: "avepool", 5: "batchnorm",
+                    6: "dropout"}
+
+
+def archive_type_name(layer):
+    """The name the reference registers for this layer's class."""
+    return ACT_TYPE_NAMES[layer.act] if layer.kind == 4 else LAYER_TYPE_NAMES[layer.kind]
+
+
+def weights_to_archive(type_names, vectors_per_layer, file_format="binary"):
+    """The bytes of a weights-only archive: `type_names[i]` and the trainable vectors
+    `vectors_per_layer[i]` (in file order, at their file length) of every layer."""
+    if file_format not in ("binary", "portable_binary"):
+        raise ValueError("weight archives are written as binary or portable_binary")
+    out = [b"\x01"] if file_format == "portable_binary" else []
+    for name, vectors in zip(type_names, vectors_per_layer):
+        raw = name.encode()
+        out.append(np.uint64(len(raw)).tobytes() + raw)
+        for v in vectors:
+            v = np.ascontiguousarray(v, dtype="<f4").ravel()
+            out.append(np.uint64(v.size).tobytes() + v.tobytes())
+    return b"".join(out)
+
+
+def archive_to_weights(data, vector_counts, file_format="binary"):
+    """[(type name, [float32 vectors])] of a weights-only archive whose i-th layer holds
+    `vector_counts[i]` trainable vectors. Raises ValueError on a truncated file."""
+    data = bytes(data)
+    at, order = 0, "<"
+    if file_format == "portable_binary":
+        if not data:
+            raise ValueError("archive is empty")
+        order, at = ("<" if data[0] else ">"), 1
+    elif file_format != "binary":
+        raise ValueError("weight archives are read as binary or portable_binary")
+
+    def take(n):
+        nonlocal at
+        if at + n > len(data):
+            raise ValueError("archive ends inside a layer record")
+        at += n
+        return data[at - n:at]
+
+    out = []
+    for count in vector_counts:
+        n = int(np.frombuffer(take(8), order + "u8")[0])
+        name = take(n).decode()
+        vectors = []
+        for _ in range(count):
+            m = int(np.frombuffer(take(8), order + "u8")[0])
+            vectors.append(np.frombuffer(take(4 * m), order + "f4").astype(F32))
+        out.append((name, vectors))
+    return out
+
+
+def save_weights_archive(net, path, file_format="binary"):
+    names, vectors = [], []
+    for i in range(net.n):
+        names.append(archive_type_name(net.layers[i]))
+        vs = []
+        for which in (0, 1):
+            n = net.param_size(i, which)
+            if n:
+                v = net.get_param(i, which)
+                vs.append(np.concatenate([v, np.zeros(_file_length(net.layers[i], which, n) - n, F32)]))
+        vectors.append(vs)
+    with open(path, "wb") as f:
+        f.write(weights_to_archive(names, vectors, file_format))
+
+
+def load_weights_archive(net, path, file_format="binary"):
+    counts = [sum(1 for which in (0, 1) if net.param_size(i, which)) for i in range(net.n)]
+    with open(path, "rb") as f:
+        layers = archive_to_weights(f.read(), counts, file_format)
+    for i, (_, vectors) in enumerate(layers):
+        k = 0
+        for which in (0, 1):
+            n = net.param_size(i, which)
+            if not n:
+                continue
+            if vectors[k].size != _file_length(net.layers[i], which, n):
+                raise ValueError(f"load_weights_archive: layer {i} holds {vectors[k].size} values, "
+                                 f"the network's layer {_file_length(net.layers[i], which, n)}")
+            net.set_param(i, which, vectors[k][:n])
+            k += 1
