@@ -490,9 +490,11 @@ static void net_with_batchnorm_and_dropout_vs_oracle() {
 
 // -------------------------------------------------- network<sequential>::fit
 template <typename Opt>
-static void net_fit_vs_oracle(const char *name, int opt_kind) {
-  std::printf("network<sequential>::fit<cross_entropy_multiclass> with %s vs oracle (short last batch)\n", name);
+static void net_fit_vs_oracle(const char *name, int opt_kind, bool layer_by_layer = false) {
+  std::printf("network<sequential>::fit<cross_entropy_multiclass> with %s vs oracle (short last batch)%s\n", name,
+              layer_by_layer ? ", layer by layer through OpKernel::compute" : "");
   network<sequential> nn;
+  if (layer_by_layer) nn.set_execution(network<sequential>::execution::layer_by_layer);
   nn << convolutional_layer(12, 12, 3, 1, 4, padding::same) << tanh_layer()
      << max_pooling_layer(12, 12, 4, 2) << convolutional_layer(6, 6, 3, 4, 6) << leaky_relu_layer(0.1f)
      << average_pooling_layer(4, 4, 6, 2) << fully_connected_layer(24, 10) << softmax_layer();
@@ -660,6 +662,150 @@ static void resident_stack_through_the_mirror() {
   ctx.setLayer(&conv);
   const core::OpKernelContext &cctx = ctx;
   EXPECT(cctx.Layer() == &conv && &cctx.input(0) == &xx && &cctx.output(0) == &yy);
+}
+
+// ---------------------------------------------------------------- the reference's layer chain
+// The CIFAR-10-shape net (examples/cifar10/train.cpp:26-42) as a `sequential` of layers joined
+// by edges, driven the way network::train_once drives it (tiny_dnn/network.h:169-213, 887-926;
+// nodes.h:276-303): forward(), loss gradient on the host, backward(), update_weights(). Nothing
+// in this test says where a tensor lives: after the first step only the batch, the net's output
+// and the loss gradient cross the bus, and the weights after three Adam steps are the oracle's.
+static void layer_chain_keeps_tensors_on_the_device() {
+  std::puts("sequential of layers and edges: CIFAR-10-shape net, batch 8, three Adam steps through layer::forward / backward / update_weight");
+  const size_t n = 8;
+  sequential seq;
+  seq.add(convolutional_layer(32, 32, 5, 3, 32, padding::same));
+  seq.add(max_pooling_layer(32, 32, 32, 2));
+  seq.add(relu_layer());
+  seq.add(convolutional_layer(16, 16, 5, 32, 32, padding::same));
+  seq.add(max_pooling_layer(16, 16, 32, 2));
+  seq.add(relu_layer());
+  seq.add(convolutional_layer(8, 8, 5, 32, 64, padding::same));
+  seq.add(max_pooling_layer(8, 8, 64, 2));
+  seq.add(relu_layer());
+  seq.add(fully_connected_layer(4 * 4 * 64, 64));
+  seq.add(relu_layer());
+  seq.add(fully_connected_layer(64, 10));
+  seq.add(softmax_layer());
+  seq.setup(false);
+  EXPECT(seq.size() == 13 && seq.in_data_size() == 3072 && seq.out_data_size() == 10);
+
+  tdo_layer L[13] = {};
+  const int chans[4] = {3, 32, 32, 64};
+  for (int b = 0; b < 3; ++b) {
+    const int hw = 32 >> b;
+    L[3 * b].kind = TDO_L_CONV; L[3 * b].conv = tdo_conv_desc{hw, hw, chans[b], 5, 5, chans[b + 1], 1, 1, 1, 1, 1, 1, nullptr};
+    L[3 * b + 1].kind = TDO_L_MAXPOOL; L[3 * b + 1].pool = tdo_pool_desc{hw, hw, chans[b + 1], 2, 2, 2, 2, 0, 0};
+    L[3 * b + 2].kind = TDO_L_ACT; L[3 * b + 2].act = TDO_ACT_RELU;
+  }
+  L[9].kind = TDO_L_FC; L[9].fc_in = 1024; L[9].fc_out = 64; L[9].fc_bias = 1;
+  L[10].kind = TDO_L_ACT; L[10].act = TDO_ACT_RELU;
+  L[11].kind = TDO_L_FC; L[11].fc_in = 64; L[11].fc_out = 10; L[11].fc_bias = 1;
+  L[12].kind = TDO_L_ACT; L[12].act = TDO_ACT_SOFTMAX;
+  tdo_net *ref = tdo_net_create(L, 13, static_cast<int>(n));
+  EXPECT(ref != nullptr);
+  for (int i = 0; i < 13; ++i) {
+    const size_t nw = tdo_net_weight_size(ref, i), nb = tdo_net_bias_size(ref, i);
+    if (!nw) continue;
+    const float bound = std::sqrt(6.f / float(i < 9 ? 25 * (chans[i / 3] + chans[i / 3 + 1]) : (i == 9 ? 1088 : 74)));
+    const vec_t w = random_vec(nw, 700 + i, -bound, bound), b = random_vec(nb, 800 + i, -0.05f, 0.05f);
+    std::copy(w.begin(), w.end(), tdo_net_weight(ref, i));
+    std::copy(b.begin(), b.end(), tdo_net_bias(ref, i));
+    std::vector<vec_t *> dst = seq[i]->weights();
+    EXPECT(dst.size() == 2 && dst[0]->size() == nw && dst[1]->size() == nb);
+    *dst[0] = w;
+    *dst[1] = b;
+  }
+  const tensor_t x = random_tensor(n, 3072, 950);
+  tensor_t target(n, vec_t(10, 0.f));
+  for (size_t s = 0; s < n; ++s) target[s][(3 * s + 1) % 10] = 1.f;
+  std::vector<tensor_t> in_batch(n), t_batch(n);
+  for (size_t s = 0; s < n; ++s) { in_batch[s] = tensor_t{x[s]}; t_batch[s] = tensor_t{target[s]}; }
+
+  adam opt;
+  for (int step = 0; step < 3; ++step) {
+    if (step == 1) reset_transfer_stats();
+    const std::vector<tensor_t> out = seq.forward(in_batch);
+    const std::vector<tensor_t> delta = gradient<cross_entropy_multiclass>(out, t_batch, std::vector<tensor_t>());
+    seq.backward(delta);
+    seq.update_weights(&opt);
+  }
+  const detail::transfer_counters c = transfer_stats();
+  std::printf("  steps 2 and 3: %zu uploads of %zu bytes, %zu downloads of %zu bytes\n", c.h2d_calls, c.h2d_bytes,
+              c.d2h_calls, c.d2h_bytes);
+  // per step: the batch and the loss gradient up, the net's output down
+  EXPECT(c.h2d_calls == 4 && c.h2d_bytes == 2 * n * (3072 + 10) * sizeof(float));
+  EXPECT(c.d2h_calls == 2 && c.d2h_bytes == 2 * n * 10 * sizeof(float));
+
+  tdo_opt o;
+  tdo_opt_default(&o, TDO_OPT_ADAM);
+  for (int step = 0; step < 3; ++step)
+    EXPECT(tdo_net_train_step(ref, &o, TDO_LOSS_CE_MULTICLASS, static_cast<int>(n), flat(x).data(), flat(target).data(), 1) == 0);
+  for (int i = 0; i < 13; ++i) {
+    const size_t nw = tdo_net_weight_size(ref, i), nb = tdo_net_bias_size(ref, i);
+    if (!nw) continue;
+    const layer &l = *seq[i];
+    const std::vector<const vec_t *> w = l.weights();   // const access: a download, no write
+    expect_near(w[0]->data(), tdo_net_weight(ref, i), nw, 1e-4f, "weights after three steps of the layer chain");
+    expect_near(w[1]->data(), tdo_net_bias(ref, i), nb, 1e-4f, "biases after three steps of the layer chain");
+  }
+  // host access to an inner edge brings its values down on request: the first pool's output
+  const tensor_t &pooled = *static_cast<const edge &>(*seq[1]->outputs()[0]).get_data();
+  EXPECT(pooled.size() == n);
+  expect_near(flat(pooled).data(), tdo_net_layer_out(ref, 1), n * 32 * 16 * 16, 1e-4f, "first pool's output of the last step");
+  tdo_net_destroy(ref);
+
+  // a host write through the non-const accessors is seen by the next pass without a notice
+  sequential two;
+  two.add(fully_connected_layer(6, 4));
+  two.add(tanh_layer());
+  two.setup(false);
+  *two[0]->weights()[0] = random_vec(24, 31);
+  std::vector<tensor_t> one{tensor_t{random_vec(6, 32)}};
+  const std::vector<tensor_t> y0 = two.forward(one);
+  (*two[0]->weights()[1])[2] += 0.5f;
+  const std::vector<tensor_t> y1 = two.forward(one);
+  EXPECT(y0[0][0][2] != y1[0][0][2] && y0[0][0][1] == y1[0][0][1]);
+}
+
+// A loose tensor that is destroyed while the device holds its newest values, and another one
+// that then lives at the same address: the old image must be neither used nor copied.
+static void mirror_drops_the_image_of_a_tensor_that_is_gone() {
+  std::puts("device mirror: another tensor at the address of one that is gone (resident mode)");
+  set_device_resident(true);
+  fully_connected_layer fc(5, 3, false);
+  tensor_t w{random_vec(15, 41)};
+  alignas(tensor_t) unsigned char room_x[sizeof(tensor_t)], room_y[sizeof(tensor_t)];
+  vec_t first_out, second_out;
+  std::vector<vec_t> parked;  // keeps round 1's rows allocated, so that round 2's lie elsewhere
+  for (int round = 0; round < 2; ++round) {
+    // the same addresses in both rounds, new tensors (and new rows) each time
+    tensor_t *x = new (room_x) tensor_t{random_vec(5, 50 + round)};
+    tensor_t *y = new (room_y) tensor_t(1);
+    std::vector<tensor_t *> in{x, &w}, out{y};
+    fc.forward_propagation(in, out);   // y's newest values are on the device only
+    if (round == 1) {
+      to_host(*y);
+      second_out = (*y)[0];
+    } else {
+      tensor_t keep(1);
+      std::vector<tensor_t *> out2{&keep};
+      fc.forward_propagation(in, out2);
+      to_host(keep);
+      first_out = keep[0];
+      release_device_copy(keep);
+    }
+    parked.push_back(std::move((*x)[0]));
+    x->~tensor_t();   // destroyed without release_device_copy
+    y->~tensor_t();
+  }
+  set_device_resident(false);
+  // round 2 used x of round 2 (not the image of round 1's x), and y of round 2 was not filled
+  // with round 1's result
+  tensor_t x2{random_vec(5, 51)}, y2(1);
+  std::vector<tensor_t *> in{&x2, &w}, out{&y2};
+  fc.forward_propagation(in, out);
+  EXPECT(second_out.size() == 3 && second_out == y2[0] && second_out != first_out);
 }
 
 // ---------------------------------------------------------------- weight_init and network API
@@ -931,6 +1077,10 @@ int main() {
     weight_files();
     net_fit_vs_oracle<gradient_descent>("gradient_descent", TDO_OPT_SGD);
     net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM);
+    net_fit_vs_oracle<adam>("adam", TDO_OPT_ADAM, /*layer_by_layer=*/true);
+    net_fit_vs_oracle<momentum>("momentum", TDO_OPT_MOMENTUM, /*layer_by_layer=*/true);
+    layer_chain_keeps_tensors_on_the_device();
+    mirror_drops_the_image_of_a_tensor_that_is_gone();
     net_with_batchnorm_and_dropout_vs_oracle();
     resident_stack_through_the_mirror();
     weight_init_and_network_api();

@@ -2,8 +2,8 @@
 //
 // A thin, header-only C++14 mirror of the part of tiny-dnn's API that drives the training hot
 // path, with the same names, argument meaning and error behaviour, sitting on the C ABI of
-// libtdh.so (include/tdh.h). It is not a copy of tiny-dnn: no CPU kernels, no serialization,
-// no graph networks — only what a program needs to switch this path to the GPU:
+// libtdh.so (include/tdh.h). It is not a copy of tiny-dnn: no CPU kernels, no model
+// serialization, no graph networks — only what a program needs to switch this path to the GPU:
 //
 //   * vec_t / tensor_t / shape3d / padding / nn_error      (tiny_dnn/util/util.h, nn_error.h)
 //   * core::backend_t with the added value `hip`           (tiny_dnn/core/backend.h:30)
@@ -13,12 +13,17 @@
 //   * Conv2dOp, Conv2dGradOp, FullyConnectedOp, FullyConnectedGradOp, MaxPoolOp, MaxPoolGradOp
 //     and the new AvePoolOp / AvePoolGradOp, whose compute(OpKernelContext&) dispatch to libtdh
 //   * gradient_descent / momentum / adam with the reference's members and update() signature
-//   * network<sequential> with operator<<, fit<Loss>, train<Loss>, predict — the whole step stays
-//     on the device (tdh_net_*)
+//   * node / edge / layer with forward(), backward(), setup(), update_weight(), connect() and the
+//     `sequential` container (tiny_dnn/node.h, layers/layer.h, nodes.h): the reference's call
+//     chain from network::train down to OpKernel::compute, with the edges' tensors resident on
+//     the device between the layers
+//   * network<sequential> with operator<<, fit<Loss>, train<Loss>, predict, save / load — by
+//     default the whole step is one fused, graph-replayed device program (tdh_net_*);
+//     set_execution(layer_by_layer) runs the layer chain instead
 //
-// Per-operator calls take host tensors, as the OpKernelContext contract requires: compute()
-// uploads its inputs, runs the kernels and downloads its outputs. Device residency across
-// forward, backward and update is what network<sequential> provides.
+// compute() takes host tensors, as the OpKernelContext contract requires. Tensors that belong to
+// an edge stay on the device until host code asks for them; tensors a caller built by hand are
+// uploaded and downloaded around every compute() unless set_device_resident(true) is in force.
 //
 // Differences from the reference that a caller can observe (all follow from the C ABI):
 //   * the HIP engine takes UNPADDED convolution tensors (padding::same is applied in the
@@ -157,16 +162,24 @@ class device_tensor {
 // ---- device mirror of host tensors ------------------------------------------------------
 // tiny-dnn's tensors are owned by edges (tiny_dnn/node.h:130-135) and only borrowed by
 // OpKernel::compute (tiny_dnn/core/framework/op_kernel.h:74-96). The operators below keep a
-// device image of every tensor they are handed, in a table keyed by the identity of the host
-// tensor_t (edge tensors have stable addresses), with one valid bit per side:
+// device image of every tensor they are handed, in a table keyed by the address of the host
+// tensor_t, with one valid bit per side:
 //
-//   write-through (the default): compute() uploads its inputs and downloads its outputs, so a
-//     caller sees exactly what the reference's CPU kernels leave in the host vectors;
-//   resident (set_device_resident(true)): an input is uploaded only when the host side is the
-//     newer one, outputs stay on the device, and the host copy is brought up to date only when
-//     the host asks for it with to_host(t). Host code that writes a tensor says so with
-//     host_modified(t). Weights, activations and gradients then stay on the device across
-//     forward_propagation, back_propagation and optimizer::update.
+//   tensors of an edge (class edge below) are ADOPTED by the mirror for the edge's lifetime and
+//     always resident: an input is uploaded only when the host side is the newer one, outputs
+//     stay on the device, and edge::get_data() / get_gradient() bring the host copy up to date
+//     when host code asks for it (the non-const forms also mark the host side as the newer
+//     one). Weights, activations and gradients so stay on the device across layer::forward,
+//     layer::backward and layer::update_weight without the caller doing anything;
+//   loose tensors (handed to compute() by a caller that built the pointer vectors itself) are
+//     write-through by default: compute() uploads its inputs and downloads its outputs, so a
+//     caller sees exactly what the reference's CPU kernels leave in the host vectors. With
+//     set_device_resident(true) they are treated like edge tensors, and the host says
+//     to_host(t) / host_modified(t) itself. A loose tensor is recognised by its address and the
+//     address of its first row's values; when another tensor turns up at a known address, the
+//     image held for the old one is dropped, never used and never copied into the new one.
+//     (A new tensor whose first row also lands at the old row's address cannot be told apart:
+//     release_device_copy(t) before destroying a loose tensor in resident mode, or use edges.)
 struct transfer_counters {
   size_t h2d_calls = 0, h2d_bytes = 0, d2h_calls = 0, d2h_bytes = 0;
 };
@@ -181,12 +194,29 @@ class mirror {
     static mirror m;
     return m;
   }
-  bool resident = false;
+  bool resident = false;  // loose tensors; adopted ones always are
+
+  // an edge's tensor: identity is certain until release(), residency does not depend on the mode
+  void adopt(const tensor_t &t) {
+    entry &e = table_[&t];
+    e.owned = true;
+    e.seen  = true;
+    remember(e, t);
+  }
+  bool is_resident(const tensor_t &t) const {
+    auto it = table_.find(&t);
+    return resident || (it != table_.end() && it->second.owned);
+  }
+  // the device holds values of t that the host copy does not
+  bool device_is_newer(const tensor_t &t) const {
+    auto it = table_.find(&t);
+    return it != table_.end() && it->second.dev_valid && !it->second.host_valid;
+  }
 
   // device image of rows [0, rows) x len of t, for reading
   const float *read(const tensor_t &t, size_t rows, size_t len) {
     entry &e = find(t, rows, len);
-    if (!e.dev_valid || !resident) upload(e, t, rows, len);
+    if (!e.dev_valid || !(resident || e.owned)) upload(e, t, rows, len);
     return e.dev;
   }
   // ... for overwriting: nothing is uploaded; the host copy is stale until to_host / commit
@@ -200,13 +230,13 @@ class mirror {
   // ... for adding to (weight and bias gradients: the reference's +=)
   float *update(tensor_t &t, size_t rows, size_t len) {
     entry &e = find(t, rows, len);
-    if (!e.dev_valid || !resident) upload(e, t, rows, len);
+    if (!e.dev_valid || !(resident || e.owned)) upload(e, t, rows, len);
     e.host_valid = false;
     return e.dev;
   }
   // after a compute(): write-through brings the host copy up to date now
   void commit(tensor_t &t) {
-    if (!resident) to_host(t);
+    if (!is_resident(t)) to_host(t);
   }
   void to_host(tensor_t &t) {
     auto it = table_.find(&t);
@@ -270,6 +300,8 @@ class mirror {
     const float *row0 = nullptr;     // data() of row 0 when the host side was last seen
     const vec_t *row0_vec = nullptr;
     bool host_valid = true, dev_valid = false;
+    bool owned = false;              // adopted by an edge: the address cannot be reused meanwhile
+    bool seen  = false;              // a tensor has been met at this address before
     std::vector<float> stage;
   };
   void reserve(entry &e, size_t floats) {
@@ -289,9 +321,17 @@ class mirror {
   }
   entry &find(const tensor_t &t, size_t rows, size_t len) {
     entry &e = table_[&t];
-    // another image than the one held (a resized or re-created host tensor): whatever the
-    // device holds is of no use unless it is the only valid copy
-    const bool same = e.rows == rows && e.len == len && !t.empty() && t[0].data() == e.row0;
+    const float *r0 = t.empty() ? nullptr : t[0].data();
+    // the tensor this entry was made for? An adopted one always; a loose one when its first
+    // row's values still lie where they were last seen
+    const bool known = e.owned || (e.seen && r0 == e.row0);
+    e.seen = true;
+    if (!known) {
+      // another tensor lives at this address now: the image belonged to one that is gone
+      e.dev_valid  = false;
+      e.host_valid = true;
+    }
+    const bool same = known && e.rows == rows && e.len == len;
     if (!same && e.host_valid) e.dev_valid = false;
     if (!same && !e.host_valid && (e.rows < rows || e.len != len)) {
       // the device holds the newer values of a smaller image: save them before it is replaced
@@ -302,7 +342,7 @@ class mirror {
     return e;
   }
   void upload(entry &e, const tensor_t &t, size_t rows, size_t len) {
-    if (!e.host_valid) {  // resident and the device is newer: nothing to send
+    if (!e.host_valid) {  // the device is newer: nothing to send
       if (e.rows >= rows && e.len == len) return;
       throw nn_error("device mirror: a tensor was resized while its newest values were on the device");
     }
@@ -692,7 +732,7 @@ class MaxPoolOp : public core::OpKernel {
     a.samples = n;
     a.host_valid = false;
     m.commit(out);
-    if (!m.resident) detail::argmax_to_host(params);
+    if (!m.is_resident(out)) detail::argmax_to_host(params);
   }
 };
 
@@ -793,6 +833,12 @@ struct mse {  // loss_function.h:18-36
     for (size_t i = 0; i < y.size(); ++i) d += (y[i] - t[i]) * (y[i] - t[i]);
     return d / static_cast<float_t>(y.size());
   }
+  static vec_t df(const vec_t &y, const vec_t &t) {
+    vec_t d(t.size());
+    const float_t factor = float_t(2) / static_cast<float_t>(t.size());
+    for (size_t i = 0; i < y.size(); ++i) d[i] = factor * (y[i] - t[i]);
+    return d;
+  }
 };
 struct cross_entropy {  // loss_function.h:108-128
   static const int kind = TDH_LOSS_CE;
@@ -800,6 +846,11 @@ struct cross_entropy {  // loss_function.h:108-128
     float_t d{0};
     for (size_t i = 0; i < y.size(); ++i)
       d += -t[i] * std::log(y[i]) - (float_t(1) - t[i]) * std::log(float_t(1) - y[i]);
+    return d;
+  }
+  static vec_t df(const vec_t &y, const vec_t &t) {
+    vec_t d(t.size());
+    for (size_t i = 0; i < y.size(); ++i) d[i] = (y[i] - t[i]) / (y[i] * (float_t(1) - y[i]));
     return d;
   }
 };
@@ -810,7 +861,41 @@ struct cross_entropy_multiclass {  // loss_function.h:131-150
     for (size_t i = 0; i < y.size(); ++i) d += -t[i] * std::log(y[i]);
     return d;
   }
+  static vec_t df(const vec_t &y, const vec_t &t) {
+    vec_t d(t.size());
+    for (size_t i = 0; i < y.size(); ++i) d[i] = -t[i] / y[i];
+    return d;
+  }
 };
+// loss_function.h:158-218: the loss gradient of one sample / of a mini-batch, on the host as in
+// the reference (the layer-by-layer chain below hands it to the last layer's output edge; the
+// device-resident step of network<sequential> computes the same values in its own kernels)
+template <typename E>
+vec_t gradient(const vec_t &y, const vec_t &t) {
+  return E::df(y, t);
+}
+template <typename E>
+std::vector<vec_t> gradient(const std::vector<vec_t> &y, const std::vector<vec_t> &t) {
+  std::vector<vec_t> grads(y.size());
+  for (size_t i = 0; i < y.size(); ++i) grads[i] = gradient<E>(y[i], t[i]);
+  return grads;
+}
+inline void apply_cost_if_defined(std::vector<vec_t> &sample_gradient, const std::vector<vec_t> &sample_cost) {
+  if (sample_gradient.size() != sample_cost.size()) return;
+  for (size_t channel = 0; channel < sample_gradient.size(); ++channel)
+    if (sample_gradient[channel].size() == sample_cost[channel].size())
+      for (size_t e = 0; e < sample_gradient[channel].size(); ++e) sample_gradient[channel][e] *= sample_cost[channel][e];
+}
+template <typename E>
+std::vector<tensor_t> gradient(const std::vector<tensor_t> &y, const std::vector<tensor_t> &t,
+                               const std::vector<tensor_t> &t_cost) {
+  std::vector<tensor_t> gradients(y.size());
+  for (size_t sample = 0; sample < y.size(); ++sample) {
+    gradients[sample] = gradient<E>(y[sample], t[sample]);
+    if (sample < t_cost.size()) apply_cost_if_defined(gradients[sample], t_cost[sample]);
+  }
+  return gradients;
+}
 
 // ---- optimizers: the reference's members and update(dW, W, parallelize) signature
 // (tiny_dnn/optimizers/optimizer.h). State vectors live on the device, keyed by &W like the
@@ -1011,18 +1096,179 @@ class he : public scalable {      // N(0, sqrt(scale / fan_in)), scale 2
 };
 }  // namespace weight_init
 
-// ---- layers: constructor arguments as in tiny_dnn/layers/*.h; they only describe the layer,
-// network<sequential> turns the descriptions into one device-resident tdh_net ----
+// tiny_dnn/util/util.h:273-315
+enum class vector_type : int32_t {
+  data   = 0x0001000,  // input/output data, fed by other layer or input channel
+  weight = 0x0002000,  // trainable parameters, updated for each back propagation
+  bias   = 0x0002001,
+  label  = 0x0004000,
+  aux    = 0x0010000   // layer-specific storage
+};
+inline vector_type operator&(vector_type lhs, vector_type rhs) {
+  return static_cast<vector_type>(static_cast<int32_t>(lhs) & static_cast<int32_t>(rhs));
+}
+inline bool is_trainable_weight(vector_type vtype) { return (vtype & vector_type::weight) == vector_type::weight; }
+inline std::vector<vector_type> std_input_order(bool has_bias) {
+  if (has_bias) return {vector_type::data, vector_type::weight, vector_type::bias};
+  return {vector_type::data, vector_type::weight};
+}
+
+enum class net_phase { train, test };  // tiny_dnn/util/util.h:71
+
+// ---- the computational graph: node, edge (tiny_dnn/node.h:40-136) ----
+class node;
+class layer;
+class edge;
+typedef std::shared_ptr<edge> edgeptr_t;
+
+class node : public std::enable_shared_from_this<node> {
+ public:
+  node(size_t in_size, size_t out_size) : prev_(in_size), next_(out_size) {}
+  virtual ~node() {}
+  const std::vector<edgeptr_t> &prev() const { return prev_; }
+  const std::vector<edgeptr_t> &next() const { return next_; }
+  size_t prev_port(const edge &e) const {
+    auto it = std::find_if(prev_.begin(), prev_.end(), [&](edgeptr_t ep) { return ep.get() == &e; });
+    return static_cast<size_t>(std::distance(prev_.begin(), it));
+  }
+  size_t next_port(const edge &e) const {
+    auto it = std::find_if(next_.begin(), next_.end(), [&](edgeptr_t ep) { return ep.get() == &e; });
+    return static_cast<size_t>(std::distance(next_.begin(), it));
+  }
+  std::vector<node *> prev_nodes() const;
+  std::vector<node *> next_nodes() const;
+
+ protected:
+  node() = delete;
+  friend void connect(layer *head, layer *tail, size_t head_index, size_t tail_index);
+  mutable std::vector<edgeptr_t> prev_;
+  mutable std::vector<edgeptr_t> next_;
+};
+
+// An edge owns the data and the gradient tensor between two layers, as in the reference, and
+// both are adopted by the device mirror for the edge's lifetime: the operators find them on the
+// device, and the accessors below are where host code meets them.
+class edge {
+ public:
+  edge(node *prev, const shape3d &shape, vector_type vtype)
+    : shape_(shape), vtype_(vtype), data_({vec_t(shape.size())}), grad_({vec_t(shape.size())}), prev_(prev) {
+    detail::mirror::get().adopt(data_);
+    detail::mirror::get().adopt(grad_);
+  }
+  edge(const edge &) = delete;
+  edge &operator=(const edge &) = delete;
+  ~edge() {
+    detail::mirror::get().release(data_);
+    detail::mirror::get().release(grad_);
+  }
+
+  // node.h:89-103: dst = sum over the samples' gradients, in sample order
+  void merge_grads(vec_t *dst) {
+    detail::mirror::get().to_host(grad_);
+    const vec_t &grad_head = grad_[0];
+    const size_t sz = grad_head.size();
+    dst->resize(sz);
+    std::copy(grad_head.begin(), grad_head.end(), dst->begin());
+    for (size_t sample = 1; sample < grad_.size(); ++sample)
+      for (size_t i = 0; i < sz; ++i) (*dst)[i] += grad_[sample][i];
+  }
+  // node.h:105-111, on both sides without a transfer
+  void clear_grads() {
+    detail::mirror::get().clear(grad_);
+    host_wrote_grad_ = false;
+  }
+
+  // Host access. The host copy is brought up to date first (a download only when the device
+  // holds newer values); through the non-const forms the host may write, so the device image
+  // counts as stale afterwards.
+  tensor_t *get_data() {
+    detail::mirror::get().to_host(data_);
+    detail::mirror::get().host_modified(data_);
+    return &data_;
+  }
+  const tensor_t *get_data() const {
+    detail::mirror::get().to_host(const_cast<tensor_t &>(data_));
+    return &data_;
+  }
+  tensor_t *get_gradient() {
+    detail::mirror::get().to_host(grad_);
+    detail::mirror::get().host_modified(grad_);
+    host_wrote_grad_ = true;
+    return &grad_;
+  }
+  const tensor_t *get_gradient() const {
+    detail::mirror::get().to_host(const_cast<tensor_t &>(grad_));
+    return &grad_;
+  }
+
+  // What layer::forward / backward / update_weight hand to the operators: the same tensors,
+  // without a transfer and without a change of the valid bits (the operators set those).
+  tensor_t *borrowed_data() { return &data_; }
+  tensor_t *borrowed_gradient() { return &grad_; }
+  // The operators add a weight gradient, already summed over the batch, into sample slot 0 on
+  // the device. While no host code has had write access to the gradient since clear_grads, the
+  // other slots are still zero and slot 0 on the device is what merge_grads would return.
+  bool merged_gradient_on_device() const {
+    return !host_wrote_grad_ && detail::mirror::get().device_is_newer(grad_);
+  }
+
+  const std::vector<node *> &next() const { return next_; }
+  node *prev() { return prev_; }
+  const node *prev() const { return prev_; }
+  const shape3d &shape() const { return shape_; }
+  vector_type vtype() const { return vtype_; }
+  void add_next_node(node *next) { next_.push_back(next); }
+
+ private:
+  shape3d shape_;
+  vector_type vtype_;
+  tensor_t data_;
+  tensor_t grad_;
+  node *prev_;                // previous node, "producer" of this tensor
+  std::vector<node *> next_;  // next nodes, "consumers" of this tensor
+  bool host_wrote_grad_ = false;
+};
+
+inline std::vector<node *> node::prev_nodes() const {
+  std::vector<node *> vecs;
+  for (auto &e : prev_)
+    if (e && e->prev()) vecs.insert(vecs.end(), e->prev());
+  return vecs;
+}
+inline std::vector<node *> node::next_nodes() const {
+  std::vector<node *> vecs;
+  for (auto &e : next_)
+    if (e) {
+      auto n = e->next();
+      vecs.insert(vecs.end(), n.begin(), n.end());
+    }
+  return vecs;
+}
+
+// ---- layers: constructor arguments as in tiny_dnn/layers/*.h. A layer works in two ways:
+//  * layer by layer, as in the reference (tiny_dnn/layers/layer.h): forward() / backward()
+//    marshal the tensors of the layer's edges into forward_propagation / back_propagation,
+//    which run the layer's OpKernel::compute; update_weight hands the merged gradient and the
+//    weights to optimizer::update. Every tensor of an edge stays on the device in between.
+//  * described to network<sequential> (describe()), which turns the descriptions into one
+//    device-resident tdh_net whose whole train step is fused and replayed as a graph.
 struct layer_desc {
   tdh_layer l;
   std::vector<uint8_t> tbl;
 };
 
-class layer {
+class layer : public node {
  public:
-  layer() : weight_init_(std::make_shared<weight_init::xavier>()),
-            bias_init_(std::make_shared<weight_init::constant>()) {}  // layer.h:72-73
+  // layer.h:58-76
+  layer(const std::vector<vector_type> &in_type, const std::vector<vector_type> &out_type)
+    : node(in_type.size(), out_type.size()), initialized_(false), parallelize_(true),
+      in_channels_(in_type.size()), out_channels_(out_type.size()), in_type_(in_type), out_type_(out_type),
+      trainable_(true), weight_init_(std::make_shared<weight_init::xavier>()),
+      bias_init_(std::make_shared<weight_init::constant>()) {}
   virtual ~layer() {}
+  layer(const layer &) = default;
+  layer &operator=(const layer &) = default;
+
   virtual layer_desc describe(const shape3d &prev_out) const = 0;
   virtual std::string layer_type() const = 0;
   // the name the reference registers for the class (tiny_dnn/util/serialization_layer_list.h),
@@ -1032,6 +1278,8 @@ class layer {
   // the initialisers scale by (layer.h:298-306)
   virtual size_t fan_in_size() const { return 0; }
   virtual size_t fan_out_size() const { return 0; }
+  virtual size_t fan_in_size(size_t) const { return fan_in_size(); }
+  virtual size_t fan_out_size(size_t) const { return fan_out_size(); }
   // the (off, on) values label2vec turns class labels into when this is the last layer
   // (layer.h:276-278; activation layers give their scale(), activation_layer.h:121)
   virtual std::pair<float_t, float_t> out_value_range() const { return {float_t{0.0}, float_t{1.0}}; }
@@ -1049,8 +1297,264 @@ class layer {
     bias_init_ = std::make_shared<BiasInit>(f);
     return *this;
   }
+
+  // layer.h:271-295
+  virtual std::vector<shape3d> in_shape() const = 0;
+  virtual std::vector<shape3d> out_shape() const = 0;
+  virtual void set_in_shape(const shape3d &) {
+    throw nn_error("Can't set shape. Shape inferring not applicable for this layer (yet).");
+  }
+  // layer.h:414-433
+  virtual void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) = 0;
+  virtual void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
+                                std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) = 0;
+  virtual void post_update() {}
+  virtual void set_context(net_phase) {}
+
+  void set_parallelize(bool parallelize) { parallelize_ = parallelize; }
+  bool parallelize() const { return parallelize_; }
+  core::backend_t engine() const { return core::backend_t::hip; }
+  size_t in_channels() const { return in_channels_; }
+  size_t out_channels() const { return out_channels_; }
+  size_t in_data_size() const {
+    size_t n = 0;
+    const std::vector<shape3d> sh = in_shape();
+    for (size_t i = 0; i < sh.size(); ++i)
+      if (in_type_[i] == vector_type::data) n += sh[i].size();
+    return n;
+  }
+  size_t out_data_size() const {
+    size_t n = 0;
+    const std::vector<shape3d> sh = out_shape();
+    for (size_t i = 0; i < sh.size(); ++i)
+      if (out_type_[i] == vector_type::data) n += sh[i].size();
+    return n;
+  }
+  size_t in_size() const { return in_data_size(); }
+  size_t out_size() const { return out_data_size(); }
+  std::vector<vector_type> in_types() const { return in_type_; }
+  std::vector<vector_type> out_types() const { return out_type_; }
+  void set_trainable(bool trainable) { trainable_ = trainable; }
+  bool trainable() const { return trainable_; }
+
+  // layer.h:153-211. The vectors handed out are the edges' own: the const forms download what
+  // the device holds newer, the non-const forms also count as a write by the host.
+  std::vector<const vec_t *> weights() const {
+    std::vector<const vec_t *> v;
+    for (size_t i = 0; i < in_channels_; i++)
+      if (is_trainable_weight(in_type_[i])) v.push_back(get_weight_data(i));
+    return v;
+  }
+  std::vector<vec_t *> weights() {
+    std::vector<vec_t *> v;
+    for (size_t i = 0; i < in_channels_; i++)
+      if (is_trainable_weight(in_type_[i])) v.push_back(get_weight_data(i));
+    return v;
+  }
+  std::vector<tensor_t *> weights_grads() {
+    std::vector<tensor_t *> v;
+    for (size_t i = 0; i < in_channels_; i++)
+      if (is_trainable_weight(in_type_[i])) v.push_back(ith_in_node(i)->get_gradient());
+    return v;
+  }
+  std::vector<edgeptr_t> inputs() {
+    std::vector<edgeptr_t> nodes(in_channels_);
+    for (size_t i = 0; i < in_channels_; i++) nodes[i] = ith_in_node(i);
+    return nodes;
+  }
+  std::vector<edgeptr_t> outputs() {
+    std::vector<edgeptr_t> nodes(out_channels_);
+    for (size_t i = 0; i < out_channels_; i++) nodes[i] = ith_out_node(i);
+    return nodes;
+  }
+
+  // layer.h:213-251: the host writes the first layer's input and the last layer's output gradient
+  void set_out_grads(const std::vector<const vec_t *> *grad, size_t cnt) {
+    size_t n = 0;
+    for (size_t i = 0; i < out_channels_; i++) {
+      if (out_type_[i] != vector_type::data) continue;
+      tensor_t &dst_grad = *ith_out_node(i)->get_gradient();
+      if (n >= cnt) throw nn_error("set_out_grads: fewer gradient channels than data outputs");
+      const auto &src_grad = grad[n++];
+      dst_grad.resize(src_grad.size());
+      for (size_t j = 0; j < src_grad.size(); ++j) dst_grad[j] = *src_grad[j];
+    }
+  }
+  void set_in_data(const std::vector<const vec_t *> *data, size_t cnt) {
+    size_t n = 0;
+    for (size_t i = 0; i < in_channels_; i++) {
+      if (in_type_[i] != vector_type::data) continue;
+      tensor_t &dst_data = *ith_in_node(i)->get_data();
+      if (n >= cnt) throw nn_error("set_in_data: fewer data channels than data inputs");
+      const auto &src_data = data[n++];
+      dst_data.resize(src_data.size());
+      for (size_t j = 0; j < src_data.size(); ++j) dst_data[j] = *src_data[j];
+    }
+  }
+  void output(std::vector<const tensor_t *> &out) const {
+    out.clear();
+    for (size_t i = 0; i < out_channels_; i++)
+      if (out_type_[i] == vector_type::data)
+        out.push_back(static_cast<const edge *>(next_[i].get())->get_data());
+  }
+
+  // layer.h:527-575: the tensors of the edges, as they are, go to the layer's operators
+  void forward() {
+    fwd_in_data_.resize(in_channels_);
+    fwd_out_data_.resize(out_channels_);
+    for (size_t i = 0; i < in_channels_; i++) fwd_in_data_[i] = ith_in_node(i)->borrowed_data();
+    set_sample_count(fwd_in_data_[0]->size());
+    for (size_t i = 0; i < out_channels_; i++) {
+      fwd_out_data_[i] = ith_out_node(i)->borrowed_data();
+      ith_out_node(i)->clear_grads();
+    }
+    forward_propagation(fwd_in_data_, fwd_out_data_);
+  }
+  void backward() {
+    bwd_in_data_.resize(in_channels_);
+    bwd_in_grad_.resize(in_channels_);
+    bwd_out_data_.resize(out_channels_);
+    bwd_out_grad_.resize(out_channels_);
+    for (size_t i = 0; i < in_channels_; i++) {
+      const auto &nd  = ith_in_node(i);
+      bwd_in_data_[i] = nd->borrowed_data();
+      bwd_in_grad_[i] = nd->borrowed_gradient();
+    }
+    for (size_t i = 0; i < out_channels_; i++) {
+      const auto &nd   = ith_out_node(i);
+      bwd_out_data_[i] = nd->borrowed_data();
+      bwd_out_grad_[i] = nd->borrowed_gradient();
+    }
+    back_propagation(bwd_in_data_, bwd_out_data_, bwd_out_grad_, bwd_in_grad_);
+  }
+
+  // layer.h:584-655
+  void setup(bool reset_weight) {
+    if (in_shape().size() != in_channels_ || out_shape().size() != out_channels_)
+      throw nn_error("Connection mismatch at setup layer");
+    for (size_t i = 0; i < out_channels_; i++)
+      if (!next_[i]) next_[i] = std::make_shared<edge>(this, out_shape()[i], out_type_[i]);
+    if (reset_weight || !initialized_) init_weight();
+  }
+  void init_weight() {
+    if (!trainable_) {
+      initialized_ = true;
+      return;
+    }
+    for (size_t i = 0; i < in_channels_; i++) {
+      switch (in_type_[i]) {
+        case vector_type::weight: weight_init_->fill(get_weight_data(i), fan_in_size(i), fan_out_size(i)); break;
+        case vector_type::bias: bias_init_->fill(get_weight_data(i), fan_in_size(i), fan_out_size(i)); break;
+        default: break;
+      }
+    }
+    initialized_ = true;
+  }
+  void clear_grads() {
+    for (size_t i = 0; i < in_type_.size(); i++) ith_in_node(i)->clear_grads();
+  }
+  // layer.h:663-682. The operators leave the gradient of a weight tensor summed over the batch
+  // in sample slot 0 on the device; while the host has not written the gradient since the last
+  // clear_grads, that slot IS the merged gradient (the other slots are zero) and it goes to the
+  // optimizer where it lies. Otherwise the reference's merge runs on the host. rcp_batch_size is
+  // 1 / (rows of the weight tensor) = 1, as in the reference.
+  void update_weight(optimizer *o) {
+    vec_t &diff = weights_diff_;
+    for (size_t i = 0; i < in_type_.size(); i++) {
+      if (!(trainable() && is_trainable_weight(in_type_[i]))) continue;
+      edge &e       = *ith_in_node(i);
+      vec_t &target = (*e.borrowed_data())[0];
+      const bool parallelize = target.size() >= 512;
+      if (e.merged_gradient_on_device()) {
+        o->update((*e.borrowed_gradient())[0], target, parallelize);
+      } else {
+        e.merge_grads(&diff);
+        const float_t rcp_batch_size = float_t(1.0) / float_t(e.borrowed_data()->size());
+        for (size_t j = 0; j < diff.size(); ++j) diff[j] *= rcp_batch_size;
+        o->update(diff, target, parallelize);
+      }
+    }
+    clear_grads();
+    post_update();
+  }
+  bool has_same_weights(const layer &rhs, float_t eps) const {
+    auto w1 = weights();
+    auto w2 = rhs.weights();
+    if (w1.size() != w2.size()) return false;
+    for (size_t i = 0; i < w1.size(); i++) {
+      if (w1[i]->size() != w2[i]->size()) return false;
+      for (size_t j = 0; j < w1[i]->size(); j++)
+        if (std::abs(w1[i]->at(j) - w2[i]->at(j)) > eps) return false;
+    }
+    return true;
+  }
+  // layer.h:699-718: room for every sample of the batch; never shrinks. Only the outer vectors
+  // grow: no values cross the bus here.
+  virtual void set_sample_count(size_t sample_count) {
+    auto resize = [sample_count](tensor_t *tensor) { tensor->resize(sample_count, (*tensor)[0]); };
+    for (size_t i = 0; i < in_channels_; i++) {
+      if (!is_trainable_weight(in_type_[i])) resize(ith_in_node(i)->borrowed_data());
+      resize(ith_in_node(i)->borrowed_gradient());
+    }
+    for (size_t i = 0; i < out_channels_; i++) {
+      if (!is_trainable_weight(out_type_[i])) resize(ith_out_node(i)->borrowed_data());
+      resize(ith_out_node(i)->borrowed_gradient());
+    }
+  }
+
+  std::shared_ptr<weight_init::function> weight_init_fn() const { return weight_init_; }
+  std::shared_ptr<weight_init::function> bias_init_fn() const { return bias_init_; }
+
+ protected:
+  bool initialized_;
+  bool parallelize_;
+  size_t in_channels_, out_channels_;
+  std::vector<vector_type> in_type_, out_type_;
+  vec_t weights_diff_;
+
+ private:
+  friend void connect(layer *head, layer *tail, size_t head_index, size_t tail_index);
+  bool trainable_;
   std::shared_ptr<weight_init::function> weight_init_, bias_init_;
+  std::vector<tensor_t *> fwd_in_data_, fwd_out_data_, bwd_in_data_, bwd_in_grad_, bwd_out_data_, bwd_out_grad_;
+
+  // layer.h:790-857
+  edgeptr_t ith_in_node(size_t i) {
+    if (!prev_[i]) prev_[i] = std::make_shared<edge>(nullptr, in_shape()[i], in_type_[i]);
+    return prev()[i];
+  }
+  edgeptr_t ith_out_node(size_t i) {
+    if (!next_[i]) next_[i] = std::make_shared<edge>(this, out_shape()[i], out_type_[i]);
+    return next()[i];
+  }
+  vec_t *get_weight_data(size_t i) { return &(*(ith_in_node(i)->get_data()))[0]; }
+  const vec_t *get_weight_data(size_t i) const {
+    const edge *e = const_cast<layer *>(this)->ith_in_node(i).get();
+    return &(*e->get_data())[0];
+  }
 };
+
+// layer.h:859-884
+inline void connect(layer *head, layer *tail, size_t head_index = 0, size_t tail_index = 0) {
+  const shape3d out_shape = head->out_shape()[head_index];
+  shape3d in_shape        = tail->in_shape()[tail_index];
+  head->setup(false);
+  if (in_shape.size() == 0) {  // shape inferring: activation layers take the shape in front of them
+    tail->set_in_shape(out_shape);
+    in_shape = out_shape;
+  }
+  if (out_shape.size() != in_shape.size())
+    throw nn_error("layer dimension mismatch!\noutput size of Nth layer must be equal to input of (N+1)th layer\n" +
+                   std::to_string(head->out_data_size()) + " != " + std::to_string(tail->in_data_size()) + " (" +
+                   head->layer_type() + " -> " + tail->layer_type() + ")");
+  if (!head->next_[head_index]) throw nn_error("output edge must not be null");
+  tail->prev_[tail_index] = head->next_[head_index];
+  tail->prev_[tail_index]->add_next_node(tail);
+}
+inline layer &operator<<(layer &lhs, layer &rhs) {
+  connect(&lhs, &rhs);
+  return rhs;
+}
 
 // tiny_dnn/layers/convolutional_layer.h:64-100
 class convolutional_layer : public layer {
@@ -1067,7 +1571,8 @@ class convolutional_layer : public layer {
                       const core::connection_table &connection_table,
                       padding pad_type = padding::valid, bool has_bias = true, size_t w_stride = 1,
                       size_t h_stride = 1, size_t w_dilation = 1, size_t h_dilation = 1,
-                      core::backend_t backend_type = core::default_engine()) {
+                      core::backend_t backend_type = core::default_engine())
+    : layer(std_input_order(has_bias), {vector_type::data}) {
     detail::require_hip(backend_type);
     params_.in = shape3d(in_width, in_height, in_channels);
     params_.weight = shape3d(window_width, window_height, in_channels * out_channels);
@@ -1080,8 +1585,16 @@ class convolutional_layer : public layer {
     params_.in_padded = pad_type == padding::same
                           ? shape3d(in_width + window_width - 1, in_height + window_height - 1, in_channels)
                           : params_.in;
-    kernel_fwd_.reset(new Conv2dOp(core::OpKernelConstruction(nullptr, &params_)));
-    kernel_back_.reset(new Conv2dGradOp(core::OpKernelConstruction(nullptr, &params_)));
+    init_backend();
+  }
+  // the operators keep a pointer to this object's params_: a copy gets operators of its own
+  // (the reference rebuilds them in its move constructor, convolutional_layer.h:258-266)
+  convolutional_layer(const convolutional_layer &o) : layer(o), params_(o.params_) { init_backend(); }
+  convolutional_layer &operator=(const convolutional_layer &o) {
+    layer::operator=(o);
+    params_ = o.params_;
+    init_backend();
+    return *this;
   }
   std::string layer_type() const override { return "conv"; }
   std::string archive_type_name() const override { return "conv"; }
@@ -1091,21 +1604,22 @@ class convolutional_layer : public layer {
     return (params_.weight.width_ / params_.w_stride) * (params_.weight.height_ / params_.h_stride) *
            params_.out.depth_;
   }
-  std::vector<shape3d> in_shape() const {
-    return {params_.in, shape3d(params_.weight.width_, params_.weight.height_, params_.weight.depth_),
-            shape3d(1, 1, params_.out.depth_)};
+  // convolutional_layer.h:279-291
+  std::vector<shape3d> in_shape() const override {
+    if (params_.has_bias) return {params_.in, params_.weight, shape3d(1, 1, params_.out.depth_)};
+    return {params_.in, params_.weight};
   }
-  std::vector<shape3d> out_shape() const { return {params_.out}; }
+  std::vector<shape3d> out_shape() const override { return {params_.out}; }
   // layer::forward_propagation / back_propagation (convolutional_layer.h:283-337) on the HIP
   // engine: the unpadded edge tensors go straight to the operators
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data);
     ctx.setEngine(core::backend_t::hip);
     kernel_fwd_->compute(ctx);
   }
   void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data, out_grad, in_grad);
     ctx.setParams(&params_);
@@ -1124,6 +1638,10 @@ class convolutional_layer : public layer {
   const core::conv_params &params() const { return params_; }
 
  private:
+  void init_backend() {  // convolutional_layer.h:508-531
+    kernel_fwd_.reset(new Conv2dOp(core::OpKernelConstruction(nullptr, &params_)));
+    kernel_back_.reset(new Conv2dGradOp(core::OpKernelConstruction(nullptr, &params_)));
+  }
   core::conv_params with_out(size_t out_channels) {
     core::conv_params p = params_;
     p.out = shape3d(0, 0, out_channels);
@@ -1137,24 +1655,39 @@ class convolutional_layer : public layer {
 class fully_connected_layer : public layer {
  public:
   fully_connected_layer(size_t in_dim, size_t out_dim, bool has_bias = true,
-                        core::backend_t backend_type = core::default_engine()) {
+                        core::backend_t backend_type = core::default_engine())
+    : layer(std_input_order(has_bias), {vector_type::data}) {
     detail::require_hip(backend_type);
     params_.in_size_ = in_dim; params_.out_size_ = out_dim; params_.has_bias_ = has_bias;
-    kernel_fwd_.reset(new FullyConnectedOp(core::OpKernelConstruction(nullptr, &params_)));
-    kernel_back_.reset(new FullyConnectedGradOp(core::OpKernelConstruction(nullptr, &params_)));
+    init_backend();
+  }
+  fully_connected_layer(const fully_connected_layer &o) : layer(o), params_(o.params_) { init_backend(); }
+  fully_connected_layer &operator=(const fully_connected_layer &o) {
+    layer::operator=(o);
+    params_ = o.params_;
+    init_backend();
+    return *this;
   }
   std::string layer_type() const override { return "fully-connected"; }
   std::string archive_type_name() const override { return "fully_connected"; }
   size_t fan_in_size() const override { return params_.in_size_; }     // fully_connected_layer.h:51-53
   size_t fan_out_size() const override { return params_.out_size_; }
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  // fully_connected_layer.h:55-68
+  std::vector<shape3d> in_shape() const override {
+    if (params_.has_bias_)
+      return {shape3d(params_.in_size_, 1, 1), shape3d(params_.in_size_, params_.out_size_, 1),
+              shape3d(params_.out_size_, 1, 1)};
+    return {shape3d(params_.in_size_, 1, 1), shape3d(params_.in_size_, params_.out_size_, 1)};
+  }
+  std::vector<shape3d> out_shape() const override { return {shape3d(params_.out_size_, 1, 1)}; }
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data);
     ctx.setEngine(core::backend_t::hip);
     kernel_fwd_->compute(ctx);
   }
   void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data, out_grad, in_grad);
     ctx.setEngine(core::backend_t::hip);
@@ -1171,6 +1704,10 @@ class fully_connected_layer : public layer {
   }
 
  private:
+  void init_backend() {  // fully_connected_layer.h:105-119
+    kernel_fwd_.reset(new FullyConnectedOp(core::OpKernelConstruction(nullptr, &params_)));
+    kernel_back_.reset(new FullyConnectedGradOp(core::OpKernelConstruction(nullptr, &params_)));
+  }
   core::fully_params params_;
   std::shared_ptr<core::OpKernel> kernel_fwd_, kernel_back_;
 };
@@ -1198,30 +1735,38 @@ class max_pooling_layer : public layer {
   max_pooling_layer(size_t in_width, size_t in_height, size_t in_channels, size_t pooling_size_x,
                     size_t pooling_size_y, size_t stride_x, size_t stride_y, bool ceil_mode = false,
                     padding pad_type = padding::valid,
-                    core::backend_t backend_type = core::default_engine()) {
+                    core::backend_t backend_type = core::default_engine())
+    : layer({vector_type::data}, {vector_type::data}) {
     detail::require_hip(backend_type);
     detail::set_pool_params(params_, in_width, in_height, in_channels, pooling_size_x,
                             pooling_size_y, stride_x, stride_y, ceil_mode, pad_type);
-    kernel_fwd_.reset(new MaxPoolOp(core::OpKernelConstruction(nullptr, &params_)));
-    kernel_back_.reset(new MaxPoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
+    init_backend();
+  }
+  max_pooling_layer(const max_pooling_layer &o) : layer(o), params_(o.params_) { init_backend(); }
+  max_pooling_layer &operator=(const max_pooling_layer &o) {
+    layer::operator=(o);
+    params_ = o.params_;
+    init_backend();
+    return *this;
   }
   std::string layer_type() const override { return "max-pool"; }
   std::string archive_type_name() const override { return "maxpool"; }
-  std::vector<shape3d> out_shape() const { return {params_.out}; }
+  std::vector<shape3d> in_shape() const override { return {params_.in}; }
+  std::vector<shape3d> out_shape() const override { return {params_.out}; }
   // maxpool_params::out2inmax of the last forward pass (downloads the device records if they
   // are the newer ones)
   const std::vector<std::vector<size_t>> &out2inmax() {
     detail::argmax_to_host(params_);
     return params_.out2inmax;
   }
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data);
     ctx.setEngine(core::backend_t::hip);
     kernel_fwd_->compute(ctx);
   }
   void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data, out_grad, in_grad);
     ctx.setEngine(core::backend_t::hip);
@@ -1236,6 +1781,10 @@ class max_pooling_layer : public layer {
   }
 
  private:
+  void init_backend() {  // max_pooling_layer.h:237-250
+    kernel_fwd_.reset(new MaxPoolOp(core::OpKernelConstruction(nullptr, &params_)));
+    kernel_back_.reset(new MaxPoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
+  }
   core::maxpool_params params_;
   std::shared_ptr<core::OpKernel> kernel_fwd_, kernel_back_;
 };
@@ -1251,13 +1800,20 @@ class average_pooling_layer : public layer {
                             padding::valid) {}
   average_pooling_layer(size_t in_width, size_t in_height, size_t in_channels, size_t pool_size_x,
                         size_t pool_size_y, size_t stride_x, size_t stride_y, bool ceil_mode = false,
-                        padding pad_type = padding::valid) {
+                        padding pad_type = padding::valid)
+    : layer(std_input_order(true), {vector_type::data}) {
     if ((in_width % pool_size_x) || (in_height % pool_size_y))
       throw nn_error("width/height not multiples of pooling size");
     detail::set_pool_params(params_, in_width, in_height, in_channels, pool_size_x, pool_size_y,
                             stride_x, stride_y, ceil_mode, pad_type);
-    kernel_fwd_.reset(new AvePoolOp(core::OpKernelConstruction(nullptr, &params_)));
-    kernel_back_.reset(new AvePoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
+    init_backend();
+  }
+  average_pooling_layer(const average_pooling_layer &o) : layer(o), params_(o.params_) { init_backend(); }
+  average_pooling_layer &operator=(const average_pooling_layer &o) {
+    layer::operator=(o);
+    params_ = o.params_;
+    init_backend();
+    return *this;
   }
   std::string layer_type() const override { return "ave-pool"; }
   std::string archive_type_name() const override { return "avepool"; }
@@ -1268,15 +1824,21 @@ class average_pooling_layer : public layer {
   size_t declared_weight_size(size_t kept) const override {  // average_pooling_layer.h:222-226
     return kept * params_.pool_size_x * params_.pool_size_y;
   }
-  std::vector<shape3d> out_shape() const { return {params_.out}; }
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  // average_pooling_layer.h:223-227: the weight vector is declared with one entry per window
+  // element and channel (only the first `channels` are ever read)
+  std::vector<shape3d> in_shape() const override {
+    return {params_.in, shape3d(params_.pool_size_x, params_.pool_size_y, params_.in.depth_),
+            shape3d(1, 1, params_.out.depth_)};
+  }
+  std::vector<shape3d> out_shape() const override { return {params_.out}; }
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data);
     ctx.setEngine(core::backend_t::hip);
     kernel_fwd_->compute(ctx);
   }
   void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     core::OpKernelContext ctx;
     ctx.set_in_out(in_data, out_data, out_grad, in_grad);
     ctx.setEngine(core::backend_t::hip);
@@ -1291,6 +1853,10 @@ class average_pooling_layer : public layer {
   }
 
  private:
+  void init_backend() {
+    kernel_fwd_.reset(new AvePoolOp(core::OpKernelConstruction(nullptr, &params_)));
+    kernel_back_.reset(new AvePoolGradOp(core::OpKernelConstruction(nullptr, &params_)));
+  }
   core::avepool_params params_;
   std::shared_ptr<core::OpKernel> kernel_fwd_, kernel_back_;
 };
@@ -1322,9 +1888,13 @@ class activation_layer : public layer {
     r.l.act_p[1] = p_[1];
     return r;
   }
+  // activation_layer.h:66-72: the shape is that of the layer in front (connect() sets it)
+  std::vector<shape3d> in_shape() const override { return {in_shape_}; }
+  std::vector<shape3d> out_shape() const override { return {in_shape_}; }
+  void set_in_shape(const shape3d &in_shape) override { in_shape_ = in_shape; }
   // activation_layer::forward_propagation / back_propagation (activation_layer.h:74-91) over
   // whole batches, through the device mirror like the operators
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     detail::ensure_init();
     detail::mirror &m = detail::mirror::get();
     const tensor_t &x = *in_data[0];
@@ -1336,7 +1906,7 @@ class activation_layer : public layer {
     m.commit(y);
   }
   void back_propagation(const std::vector<tensor_t *> &in_data, const std::vector<tensor_t *> &out_data,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     detail::ensure_init();
     detail::mirror &m = detail::mirror::get();
     const tensor_t &y = *out_data[0];
@@ -1370,13 +1940,14 @@ class activation_layer : public layer {
 
  protected:
   activation_layer(int kind, const char *type, float p0 = 0.f, float p1 = 0.f)
-    : kind_(kind), type_(type) {
+    : layer({vector_type::data}, {vector_type::data}), kind_(kind), type_(type) {
     p_[0] = p0;
     p_[1] = p1;
   }
   int kind_;
   const char *type_;
   float p_[2];
+  shape3d in_shape_;
 
  private:
   struct buffers {
@@ -1413,8 +1984,6 @@ struct softsign_layer : activation_layer { softsign_layer() : activation_layer(T
 struct asinh_layer : activation_layer { asinh_layer() : activation_layer(TDH_ACT_ASINH, "asinh-activation") {} };
 struct tanh_p1m2_layer : activation_layer { tanh_p1m2_layer() : activation_layer(TDH_ACT_TANH_P1M2, "tanh-scaled-activation") {} };
 
-enum class net_phase { train, test };  // tiny_dnn/util/util.h:71
-
 // The two layers below run on the device through their own operators when used the way the
 // reference's tests use a single layer (forward_propagation / back_propagation on host
 // tensors), and are layer kinds of the device-resident step of network<sequential>: there the
@@ -1450,7 +2019,8 @@ class batch_normalization_layer : public layer {
  public:
   batch_normalization_layer(size_t in_spatial_size, size_t in_channels, float_t epsilon = 1e-5,
                             float_t momentum = 0.999, net_phase phase = net_phase::train)
-    : channels_(in_channels), spatial_(in_spatial_size), phase_(phase), momentum_(momentum),
+    : layer({vector_type::data}, {vector_type::data}), channels_(in_channels), spatial_(in_spatial_size),
+      phase_(phase), momentum_(momentum),
       eps_(epsilon), update_immidiately_(false), mean_(in_channels), variance_(in_channels),
       mean_current_(in_channels), variance_current_(in_channels), stddev_(in_channels),
       buf_(new detail::norm_buffers()) {}
@@ -1467,11 +2037,11 @@ class batch_normalization_layer : public layer {
     r.l.bn_momentum = momentum_;
     return r;
   }
-  std::vector<shape3d> in_shape() const { return {shape3d(spatial_, 1, channels_)}; }
-  std::vector<shape3d> out_shape() const { return {shape3d(spatial_, 1, channels_)}; }
+  std::vector<shape3d> in_shape() const override { return {shape3d(spatial_, 1, channels_)}; }
+  std::vector<shape3d> out_shape() const override { return {shape3d(spatial_, 1, channels_)}; }
 
   // batch_normalization_layer.h:127-169
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     detail::ensure_init();
     const tensor_t &in = *in_data[0];
     tensor_t &out      = *out_data[0];
@@ -1499,7 +2069,7 @@ class batch_normalization_layer : public layer {
 
   // batch_normalization_layer.h:87-125
   void back_propagation(const std::vector<tensor_t *> &, const std::vector<tensor_t *> &out_data,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     detail::ensure_init();
     const tensor_t &curr_out = *out_data[0];
     tensor_t &prev_delta     = *in_grad[0];
@@ -1514,9 +2084,9 @@ class batch_normalization_layer : public layer {
     b.dx.download(prev_delta, n, len);
   }
 
-  void set_context(net_phase ctx) { phase_ = ctx; }
+  void set_context(net_phase ctx) override { phase_ = ctx; }
   // batch_normalization_layer.h:171-177
-  void post_update() {
+  void post_update() override {
     detail::ensure_init();
     detail::norm_buffers &b = *buf_;
     detail::check(tdh_batchnorm_update_moving(
@@ -1561,7 +2131,8 @@ class batch_normalization_layer : public layer {
 class dropout_layer : public layer {
  public:
   dropout_layer(size_t in_dim, float_t dropout_rate, net_phase phase = net_phase::train)
-    : phase_(phase), dropout_rate_(dropout_rate), scale_(float_t(1) / (float_t(1) - dropout_rate)),
+    : layer({vector_type::data}, {vector_type::data}), phase_(phase), dropout_rate_(dropout_rate),
+      scale_(float_t(1) / (float_t(1) - dropout_rate)),
       in_size_(in_dim), mask_(1, std::vector<uint8_t>(in_dim)), buf_(new detail::norm_buffers()) {}
 
   std::string layer_type() const override { return "dropout"; }
@@ -1573,8 +2144,8 @@ class dropout_layer : public layer {
     r.l.dropout_rate = dropout_rate_;
     return r;
   }
-  std::vector<shape3d> in_shape() const { return {shape3d(in_size_, 1, 1)}; }
-  std::vector<shape3d> out_shape() const { return {shape3d(in_size_, 1, 1)}; }
+  std::vector<shape3d> in_shape() const override { return {shape3d(in_size_, 1, 1)}; }
+  std::vector<shape3d> out_shape() const override { return {shape3d(in_size_, 1, 1)}; }
   void set_dropout_rate(float_t rate) {
     dropout_rate_ = rate;
     scale_        = float_t(1) / (float_t(1) - dropout_rate_);
@@ -1583,7 +2154,7 @@ class dropout_layer : public layer {
 
   // dropout_layer.h:84-117: in the train phase every element of every sample draws its own
   // bernoulli(rate), sample after sample; the products run on the device
-  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) {
+  void forward_propagation(const std::vector<tensor_t *> &in_data, std::vector<tensor_t *> &out_data) override {
     detail::ensure_init();
     const tensor_t &in = *in_data[0];
     tensor_t &out      = *out_data[0];
@@ -1609,7 +2180,7 @@ class dropout_layer : public layer {
 
   // dropout_layer.h:62-82
   void back_propagation(const std::vector<tensor_t *> &, const std::vector<tensor_t *> &,
-                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) {
+                        std::vector<tensor_t *> &out_grad, std::vector<tensor_t *> &in_grad) override {
     detail::ensure_init();
     const tensor_t &curr_delta = *out_grad[0];
     tensor_t &prev_delta       = *in_grad[0];
@@ -1626,7 +2197,7 @@ class dropout_layer : public layer {
     b.dx.download(prev_delta, n, in_size_);
   }
 
-  void set_context(net_phase ctx) { phase_ = ctx; }
+  void set_context(net_phase ctx) override { phase_ = ctx; }
   const std::vector<uint8_t> &get_mask(size_t sample_index) const { return mask_[sample_index]; }
   void clear_mask() {
     for (auto &sample : mask_) std::fill(sample.begin(), sample.end(), 0);
@@ -1762,7 +2333,124 @@ inline std::vector<archive_layer> read_weight_archive(std::istream &is, const st
 }
 }  // namespace detail
 
-struct sequential {};
+// ---- nodes / sequential (tiny_dnn/nodes.h:60-303): the layer-by-layer chain ----
+// rvalues and shared_ptrs are kept alive by the container, lvalues are referred to, as in the
+// reference. forward() writes the batch into the first layer's input edge, runs every layer's
+// forward() and reads the last layer's output edge; backward() writes the loss gradient into
+// the last layer's output edge and runs every layer's backward() back to front. Everything in
+// between stays on the device (see class edge).
+class nodes {
+ public:
+  typedef std::vector<layer *>::iterator iterator;
+  typedef std::vector<layer *>::const_iterator const_iterator;
+  virtual ~nodes() {}
+  virtual void backward(const std::vector<tensor_t> &first) = 0;
+  virtual std::vector<tensor_t> forward(const std::vector<tensor_t> &first) = 0;
+  virtual void update_weights(optimizer *opt) {
+    for (auto l : nodes_) l->update_weight(opt);
+  }
+  virtual void setup(bool reset_weight) {
+    for (auto l : nodes_) l->setup(reset_weight);
+  }
+  void clear_grads() {
+    for (auto l : nodes_) l->clear_grads();
+  }
+  size_t size() const { return nodes_.size(); }
+  iterator begin() { return nodes_.begin(); }
+  iterator end() { return nodes_.end(); }
+  const_iterator begin() const { return nodes_.begin(); }
+  const_iterator end() const { return nodes_.end(); }
+  layer *operator[](size_t index) { return nodes_[index]; }
+  const layer *operator[](size_t index) const { return nodes_[index]; }
+  size_t in_data_size() const { return nodes_.front()->in_data_size(); }
+  size_t out_data_size() const { return nodes_.back()->out_data_size(); }
+  template <typename T>
+  T &at(size_t index) {
+    T *v = dynamic_cast<T *>(nodes_[index]);
+    if (v) return *v;
+    throw nn_error("failed to cast");
+  }
+  virtual float_t target_value_min(int = 0) const { return nodes_.back()->out_value_range().first; }
+  virtual float_t target_value_max(int = 0) const { return nodes_.back()->out_value_range().second; }
+  void label2vec(const label_t *t, size_t num, std::vector<vec_t> &vec) const {
+    const size_t outdim = out_data_size();
+    vec.reserve(num);
+    for (size_t i = 0; i < num; i++) {
+      if (t[i] >= outdim) throw nn_error("label out of range");
+      vec.emplace_back(outdim, target_value_min());
+      vec.back()[t[i]] = target_value_max();
+    }
+  }
+
+ protected:
+  template <typename T>
+  void push_back(T &&node) {
+    push_back_impl(std::forward<T>(node), typename std::is_rvalue_reference<decltype(node)>::type());
+  }
+  template <typename T>
+  void push_back(std::shared_ptr<T> node) {
+    own_nodes_.push_back(node);
+    nodes_.push_back(own_nodes_.back().get());
+  }
+  // [sample][channel][feature] -> [channel][sample][feature] (nodes.h:228-250)
+  void reorder_for_layerwise_processing(const std::vector<tensor_t> &input,
+                                        std::vector<std::vector<const vec_t *>> &output) {
+    const size_t sample_count = input.size(), channel_count = input[0].size();
+    output.resize(channel_count);
+    for (size_t i = 0; i < channel_count; ++i) output[i].resize(sample_count);
+    for (size_t sample = 0; sample < sample_count; ++sample) {
+      if (input[sample].size() != channel_count) throw nn_error("samples with different channel counts");
+      for (size_t channel = 0; channel < channel_count; ++channel) output[channel][sample] = &input[sample][channel];
+    }
+  }
+  template <typename T>
+  void push_back_impl(T &&node, std::true_type) {
+    own_nodes_.push_back(std::make_shared<typename std::remove_reference<T>::type>(std::forward<T>(node)));
+    nodes_.push_back(own_nodes_.back().get());
+  }
+  template <typename T>
+  void push_back_impl(T &&node, std::false_type) {
+    nodes_.push_back(&node);
+  }
+  std::vector<std::shared_ptr<layer>> own_nodes_;
+  std::vector<layer *> nodes_;
+};
+
+class sequential : public nodes {
+ public:
+  void backward(const std::vector<tensor_t> &first) override {
+    std::vector<std::vector<const vec_t *>> reordered_grad;
+    reorder_for_layerwise_processing(first, reordered_grad);
+    if (reordered_grad.size() != 1) throw nn_error("sequential::backward: one output channel expected");
+    nodes_.back()->set_out_grads(&reordered_grad[0], 1);
+    for (auto l = nodes_.rbegin(); l != nodes_.rend(); l++) (*l)->backward();
+  }
+  std::vector<tensor_t> forward(const std::vector<tensor_t> &first) override {
+    std::vector<std::vector<const vec_t *>> reordered_data;
+    reorder_for_layerwise_processing(first, reordered_data);
+    if (reordered_data.size() != 1) throw nn_error("sequential::forward: one input channel expected");
+    nodes_.front()->set_in_data(&reordered_data[0], 1);
+    for (auto l : nodes_) l->forward();
+    std::vector<const tensor_t *> out;
+    nodes_.back()->output(out);
+    // back to [sample][layer][feature] (nodes.h:346-359)
+    const size_t sample_count = first.size();  // (the edge may hold more rows than this batch)
+    std::vector<tensor_t> normalized_output(sample_count, tensor_t(1));
+    for (size_t sample = 0; sample < sample_count; ++sample) normalized_output[sample][0] = (*out[0])[sample];
+    return normalized_output;
+  }
+  template <typename T>
+  void add(T &&layer) {
+    push_back(std::forward<T>(layer));
+    if (nodes_.size() != 1) connect(nodes_[nodes_.size() - 2], nodes_[nodes_.size() - 1], 0, 0);
+    check_connectivity();
+  }
+  void check_connectivity() {
+    for (size_t i = 0; i + 1 < nodes_.size(); i++)
+      if (nodes_[i]->outputs()[0] != nodes_[i + 1]->inputs()[0]) throw nn_error("");
+  }
+};
+
 enum grad_check_mode { GRAD_CHECK_ALL, GRAD_CHECK_RANDOM };  // tiny_dnn/util/util.h:68-69
 
 // network<sequential> (tiny_dnn/network.h:148-1105): operator<<, fit, train, predict. Weights
@@ -1786,21 +2474,61 @@ class network<sequential> {
     drop();
     return *this;
   }
+
+  // How a step runs. fused (the default): the layers are described to one device-resident
+  // tdh_net whose whole train step is fused and replayed as a HIP graph. layer_by_layer: the
+  // reference's own loop (tiny_dnn/network.h:169-213, 840-926, nodes.h:276-303): every layer's
+  // forward() / backward() marshals its edges' tensors into OpKernel::compute, the loss gradient
+  // is computed on the host from the net's output, and layer::update_weight hands gradients and
+  // weights to optimizer::update; the tensors stay on the device between the layers either way.
+  // Each mode keeps its own copy of the weights: choose before weights are set or drawn.
+  enum class execution { fused, layer_by_layer };
+  void set_execution(execution mode) {
+    if (mode != mode_ && initialized_) throw nn_error("set_execution: choose the mode before weights are set");
+    mode_ = mode;
+  }
+  execution get_execution() const { return mode_; }
+  // the chain of layer_by_layer execution (the layers of this network, connected by edges)
+  sequential &chain() {
+    if (chain_.size() != layers_.size()) {
+      if (chain_.size()) throw nn_error("layers were added after the layer-by-layer chain was built");
+      for (auto &l : layers_) chain_.add(*l);
+    }
+    return chain_;
+  }
   size_t layer_size() const { return layers_.size(); }
   size_t depth() const { return layer_size(); }
   const layer *operator[](size_t index) const { return layers_[index].get(); }
 
-  size_t in_data_size() { return build(1), tdh_net_in_size(net_); }
-  size_t out_data_size() { return build(1), tdh_net_out_size(net_); }
+  size_t in_data_size() {
+    return mode_ == execution::layer_by_layer ? chain().in_data_size() : (build(1), tdh_net_in_size(net_));
+  }
+  size_t out_data_size() {
+    return mode_ == execution::layer_by_layer ? chain().out_data_size() : (build(1), tdh_net_out_size(net_));
+  }
 
   // trainable tensors of layer `index`: which = 0 weight, 1 bias
   vec_t weights(size_t index, int which) {
+    if (mode_ == execution::layer_by_layer) {  // the edge's vector, at its declared length
+      chain().setup(false);
+      const layer &l = *layers_[index];
+      const std::vector<const vec_t *> w = l.weights();
+      return static_cast<size_t>(which) < w.size() ? *w[which] : vec_t();
+    }
     build(max_batch_ ? max_batch_ : 1);
     vec_t v(tdh_net_param_size(net_, static_cast<int>(index), which));
     detail::check(tdh_net_get_param(net_, static_cast<int>(index), which, v.data()));
     return v;
   }
   void set_weights(size_t index, int which, const vec_t &v) {
+    if (mode_ == execution::layer_by_layer) {
+      chain().setup(false);
+      const std::vector<vec_t *> w = layers_[index]->weights();
+      if (static_cast<size_t>(which) >= w.size() || v.size() > w[which]->size()) throw nn_error("set_weights: size mismatch");
+      std::copy(v.begin(), v.end(), w[which]->begin());  // (a used prefix of an average-pooling vector is enough)
+      initialized_ = true;
+      return;
+    }
     build(max_batch_ ? max_batch_ : 1);
     if (v.size() != tdh_net_param_size(net_, static_cast<int>(index), which))
       throw nn_error("set_weights: size mismatch");
@@ -1829,6 +2557,9 @@ class network<sequential> {
            size_t batch_size, int epoch, OnBatch on_batch_enumerate, OnEpoch on_epoch_enumerate,
            bool reset_weights) {
     if (inputs.size() != desired_outputs.size() || inputs.empty() || batch_size == 0) return false;
+    if (mode_ == execution::layer_by_layer)
+      return fit_layer_by_layer<Error>(opt, inputs, desired_outputs, batch_size, epoch, on_batch_enumerate,
+                                       on_epoch_enumerate, reset_weights);
     build(batch_size);
     if (reset_weights || !initialized_) init_weight();
     const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
@@ -1864,6 +2595,11 @@ class network<sequential> {
 
   // network::set_netphase (tiny_dnn/network.h:438-442)
   void set_netphase(net_phase phase) {
+    if (mode_ == execution::layer_by_layer) {
+      phase_ = phase;
+      for (auto &l : layers_) l->set_context(phase);
+      return;
+    }
     build(max_batch_ ? max_batch_ : 1);
     phase_ = phase;
     detail::check(tdh_net_set_phase(net_, phase == net_phase::train));
@@ -1875,8 +2611,8 @@ class network<sequential> {
   bool train(Optimizer &opt, const std::vector<vec_t> &inputs, const std::vector<label_t> &class_labels,
              size_t batch_size, int epoch) {
     if (inputs.size() != class_labels.size() || inputs.size() < batch_size) return false;
-    build(batch_size);
-    const size_t out_len = tdh_net_out_size(net_);
+    if (mode_ != execution::layer_by_layer) build(batch_size);
+    const size_t out_len = out_data_size();
     const std::pair<float_t, float_t> range = layers_.back()->out_value_range();
     std::vector<vec_t> t(class_labels.size(), vec_t(out_len, range.first));
     for (size_t i = 0; i < class_labels.size(); ++i) {
@@ -1987,6 +2723,11 @@ class network<sequential> {
   // (tiny_dnn/layers/layer.h:625-655): layers front to back, weight before bias, each filled
   // by the layer's weight_init / bias_init function with the layer's fan sizes
   void init_weight() {
+    if (mode_ == execution::layer_by_layer) {
+      chain().setup(true);
+      initialized_ = true;
+      return;
+    }
     build(max_batch_ ? max_batch_ : 1);
     for (size_t i = 0; i < layers_.size(); ++i) {
       layer &l = *layers_[i];
@@ -1994,7 +2735,7 @@ class network<sequential> {
         const size_t n = tdh_net_param_size(net_, static_cast<int>(i), which);
         if (!n) continue;
         vec_t v(which == 0 ? l.declared_weight_size(n) : n);
-        (which == 0 ? l.weight_init_ : l.bias_init_)->fill(&v, l.fan_in_size(), l.fan_out_size());
+        (which == 0 ? l.weight_init_fn() : l.bias_init_fn())->fill(&v, l.fan_in_size(), l.fan_out_size());
         v.resize(n);
         detail::check(tdh_net_set_param(net_, static_cast<int>(i), which, v.data()));
       }
@@ -2007,6 +2748,16 @@ class network<sequential> {
   vec_t fprop(const vec_t &in) { return fprop(std::vector<vec_t>{in})[0]; }
   std::vector<vec_t> fprop(const std::vector<vec_t> &in) {
     if (in.empty()) return {};
+    if (mode_ == execution::layer_by_layer) {
+      if (!initialized_) init_weight();
+      std::vector<tensor_t> batch(in.size());
+      for (size_t s = 0; s < in.size(); ++s) batch[s] = tensor_t{in[s]};
+      const std::vector<tensor_t> y = chain().forward(batch);
+      std::vector<vec_t> out(y.size());
+      for (size_t s = 0; s < y.size(); ++s) out[s] = y[s][0];
+      last_batch_ = in.size();
+      return out;
+    }
     build(std::max(in.size(), max_batch_ ? max_batch_ : 1));
     if (!initialized_) init_weight();
     const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
@@ -2036,6 +2787,14 @@ class network<sequential> {
   // what fprop returned: the device still holds it, so it is not sent back.
   template <typename E>
   void bprop(const std::vector<vec_t> &out, const std::vector<vec_t> &t) {
+    if (mode_ == execution::layer_by_layer) {  // network.h:169-182
+      if (!last_batch_ || out.size() != last_batch_ || t.size() != last_batch_)
+        throw nn_error("bprop: call fprop on the same batch first");
+      std::vector<tensor_t> delta(out.size());
+      for (size_t s = 0; s < out.size(); ++s) delta[s] = tensor_t{gradient<E>(out[s], t[s])};
+      chain().backward(delta);
+      return;
+    }
     if (!net_ || !last_batch_ || out.size() != last_batch_ || t.size() != last_batch_)
       throw nn_error("bprop: call fprop on the same batch first");
     const size_t out_len = tdh_net_out_size(net_);
@@ -2054,13 +2813,18 @@ class network<sequential> {
   // the gradients are clear
   template <typename Optimizer>
   void update_weights(Optimizer *opt) {
+    if (mode_ == execution::layer_by_layer) {
+      chain().update_weights(opt);
+      return;
+    }
     build(max_batch_ ? max_batch_ : 1);
     tdh_opt o = opt->descriptor();
     detail::check(tdh_net_update_weights(net_, &o));
     opt->absorb(o);
   }
   void clear_grads() {
-    if (net_) detail::check(tdh_net_clear_grads(net_));
+    if (mode_ == execution::layer_by_layer) chain().clear_grads();
+    else if (net_) detail::check(tdh_net_clear_grads(net_));
   }
   // batch-reduced gradient of layer `index` (which = 0 weight, 1 bias) since the last update
   vec_t weights_grads(size_t index, int which) {
@@ -2076,6 +2840,12 @@ class network<sequential> {
   // update_weights of `size` samples as one mini-batch
   template <typename E, typename Optimizer>
   void train_once(Optimizer &opt, const vec_t *in, const vec_t *t, size_t size) {
+    if (mode_ == execution::layer_by_layer) {  // network.h:887-926
+      const std::vector<vec_t> xs(in, in + size), ts(t, t + size);
+      bprop<E>(fprop(xs), ts);
+      chain().update_weights(&opt);
+      return;
+    }
     build(std::max(size, max_batch_ ? max_batch_ : 1));
     if (!initialized_) init_weight();
     const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
@@ -2144,6 +2914,7 @@ class network<sequential> {
 
   // network::predict (tiny_dnn/network.h:226-230)
   vec_t predict(const vec_t &in) {
+    if (mode_ == execution::layer_by_layer) return fprop(in);
     build(max_batch_ ? max_batch_ : 1);
     tensor_t xb{in};
     const size_t in_len = tdh_net_in_size(net_), out_len = tdh_net_out_size(net_);
@@ -2155,6 +2926,26 @@ class network<sequential> {
   }
 
  private:
+  // network::fit on the layer chain (tiny_dnn/network.h:840-879): setup, train phase, optimizer
+  // reset, epochs over mini-batches of train_once, test phase
+  template <typename Error, typename Optimizer, typename OnBatch, typename OnEpoch>
+  bool fit_layer_by_layer(Optimizer &opt, const std::vector<vec_t> &inputs, const std::vector<vec_t> &desired_outputs,
+                          size_t batch_size, int epoch, OnBatch on_batch_enumerate, OnEpoch on_epoch_enumerate,
+                          bool reset_weights) {
+    if (reset_weights || !initialized_) init_weight();
+    else chain().setup(false);
+    set_netphase(net_phase::train);
+    opt.reset();
+    for (int iter = 0; iter < epoch; iter++) {
+      for (size_t i = 0; i < inputs.size(); i += batch_size) {
+        train_once<Error>(opt, &inputs[i], &desired_outputs[i], std::min(batch_size, inputs.size() - i));
+        on_batch_enumerate();
+      }
+      on_epoch_enumerate();
+    }
+    set_netphase(net_phase::test);
+    return true;
+  }
   // dropout_layer::forward_propagation in the train phase (dropout_layer.h:99-102): every
   // element of every sample of every dropout layer, front to back, draws its own
   // bernoulli(rate) from the process-wide generator; the masks are handed to the device net
@@ -2246,6 +3037,8 @@ class network<sequential> {
   }
 
   std::vector<std::unique_ptr<layer>> layers_;
+  execution mode_ = execution::fused;
+  sequential chain_;
   tdh_net *net_     = nullptr;
   size_t max_batch_ = 0;
   bool initialized_ = false;
