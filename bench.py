@@ -67,12 +67,13 @@ class NetWorkload:
 
     def step_from_host(self):
         """The same step when the caller hands over host buffers: inputs and targets cross PCIe,
-        double-buffered (the upload of the next batch overlaps this step)."""
+        two batches ahead (a batch is copied and uploaded while the step before it runs)."""
         if self.feeder is None:
             self.feeder = self.T.Feeder(self.host_x.shape[1], self.host_t.shape[1], self.batch)
             self.feeder.stage(self.host_x, self.host_t)
+            self.feeder.stage(self.host_x, self.host_t)
         xd, td, n = self.feeder.acquire()
-        self.feeder.stage(self.host_x, self.host_t)  # the worker copies while this thread launches
+        self.feeder.stage(self.host_x, self.host_t)  # the worker copies and uploads while this thread launches
         self.net.train_step(self.opt, self.loss, n, xd, td)
 
 
@@ -356,7 +357,7 @@ def main():
                                         "frac": round(tot_flop / tot_s / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
     out["copy_yardstick"] = copy_yardstick(T)
     if hasattr(wl, "step_from_host"):  # never `value`: reported for callers that own host buffers
-        for _ in range(8):  # every device slot gets its captured step
+        for _ in range(12):  # every device slot gets its captured steps (three slots, two Adam buffers)
             wl.step_from_host()
         T.sync()
         host_steps = max(args.steps, 200)

@@ -333,14 +333,17 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
 /* ------------------------------------------------ batches from host memory */
 /* network::fit hands each mini-batch over as host vectors (tiny_dnn/network.h:866-879;
  * layer::set_in_data copies them into the first layer, tiny_dnn/layers/layer.h:230-251).
- * A feeder uploads them double-buffered: tdh_feeder_stage copies batch k+1 from pageable
- * host memory into a pinned slot and queues its upload on a copy stream while the step on
- * batch k runs; tdh_feeder_acquire makes the library stream wait for that upload and returns
- * the device pointers to hand to tdh_net_train_step / tdh_net_forward. Calls alternate
- * stage, acquire, stage, acquire ...; x: [batch][x_len], t: [batch][t_len] floats. The host
- * copy runs on a worker thread of the feeder: x_host / t_host must stay valid and unchanged
- * until the matching tdh_feeder_acquire returns. The device pointers stay valid until the
- * second-next acquire. */
+ * A feeder takes them ahead of time: tdh_feeder_stage hands a batch in pageable host memory to
+ * a worker thread of the feeder, which copies it into a pinned slot and queues its upload on a
+ * copy stream at once; tdh_feeder_acquire makes the library stream wait for the upload of the
+ * oldest staged batch and returns the device pointers to hand to tdh_net_train_step /
+ * tdh_net_forward. Up to two batches may be staged and not yet acquired (stage, stage, then
+ * acquire, stage, step, acquire, stage, step ...: the upload of a batch then overlaps the step
+ * before it; staging one batch ahead works as well), a third is refused with TDH_ERR_INVALID.
+ * x: [batch][x_len], t: [batch][t_len] floats; x_host / t_host must stay valid and unchanged
+ * until the tdh_feeder_acquire that returns that batch. Queue every piece of work that reads a
+ * batch before acquiring the next one: its device slot is reused by the second stage call
+ * after that. */
 typedef struct tdh_feeder tdh_feeder;
 int tdh_feeder_create(size_t x_len, size_t t_len, int max_batch, tdh_feeder **feeder);
 int tdh_feeder_destroy(tdh_feeder *feeder);

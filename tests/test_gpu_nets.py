@@ -813,9 +813,12 @@ def test_layers_without_bias_through_the_one_launch_kernels(T, O):
         net.close()
 
 
-def test_feeder_double_buffered_batches_match_oracle(T, O, W):
+@pytest.mark.parametrize("ahead", [1, 2])
+def test_feeder_batches_staged_ahead_match_oracle(T, O, W, ahead):
     """tdh_feeder_*: different host batches every step, a short last batch, graph replay from
-    the two alternating device slots; updated weights against the oracle after every step."""
+    the three device slots in turn, staged one and two batches ahead of the step; updated weights
+    against the oracle after every step. A third outstanding batch and an acquire with nothing
+    staged are refused."""
     spec, params, _, _, _, loss, opt_kind, opt_kw = W.make_batch("cifar10_cnn_b128", batch=8)
     batch = 8
     net = T.Net(W.build_layers(T, spec), batch, T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
@@ -829,19 +832,33 @@ def test_feeder_double_buffered_batches_match_oracle(T, O, W):
     ts = [np.eye(10, dtype=np.float32)[rng.integers(0, 10, n)] for n in sizes]
     opt, ropt = T.opt_desc(opt_kind, **opt_kw), O.opt_desc(opt_kind, **opt_kw)
     feed = T.Feeder(3072, 10, batch)
-    feed.stage(xs[0], ts[0])
+    for k in range(ahead):
+        feed.stage(xs[k], ts[k])
     for k in range(len(sizes)):
         xd, td, n = feed.acquire()
         assert n == sizes[k]
+        if k + ahead < len(sizes):
+            feed.stage(xs[k + ahead], ts[k + ahead])
         net.train_step(opt, loss, n, xd, td)
-        if k + 1 < len(sizes):
-            feed.stage(xs[k + 1], ts[k + 1])
-        with pytest.raises(T.TdhError, match="nothing has been staged|has not been acquired"):
-            feed.acquire() if k + 1 == len(sizes) else feed.stage(xs[k], ts[k])
+        if k == 2:    # as many staged as the feeder takes (two), or nothing staged at the end
+            extra = 2 - ahead
+            for _ in range(extra):
+                feed.stage(xs[k], ts[k])
+            with pytest.raises(T.TdhError, match="batches are staged and have not been acquired"):
+                feed.stage(xs[k], ts[k])
+            for _ in range(extra):   # drop what this check staged: acquire it and move on
+                feed.acquire()
+            if extra:                # the order of the real batches is restored
+                feed.close()
+                feed = T.Feeder(3072, 10, batch)
+                for j in range(k + 1, min(k + 1 + ahead, len(sizes))):
+                    feed.stage(xs[j], ts[j])
         ref.train_step(ropt, loss, xs[k], ts[k])
         for (i, which, _) in params:
             want = ref.weight(i) if which == 0 else ref.bias(i)
             assert_close(net.get_param(i, which), want, REL_TOL, f"step {k} layer {i}.{which}")
+    with pytest.raises(T.TdhError, match="nothing has been staged"):
+        feed.acquire()
     feed.close()
 
 
@@ -965,4 +982,120 @@ def test_net_with_batchnorm_and_dropout_matches_oracle_and_reference_fit(T, O, W
     assert not np.array_equal(net.layer_out(6, batch), net.layer_out(5, batch))
     with pytest.raises(T.TdhError):
         net.set_dropout_mask(5, probe)     # not a dropout layer
+    net.close()
+
+
+@pytest.mark.parametrize("flags", [0, 3])
+def test_decisions_that_hang_on_summation_order_are_legitimate_and_the_gradients_follow_them(T, O, flags):
+    """The one class of difference from the oracle that no tolerance covers: a relu whose
+    pre-activation, or a max-pool whose two best candidates, differ by less than fp32 rounding
+    of the sums behind them. Which way such a decision falls depends on the order of the
+    additions, and everything behind it changes by whole gradient values.
+
+    conv 3x3 (1 -> 3 channels, 6x6, pad same) -> relu -> max-pool 2x2 -> fc 27 -> 3 -> softmax,
+    with an input built so that (i) channel 0 at pixel (2,2) is 1 + 3e-8 - 1: exactly 0 when
+    added in tap order (the oracle: relu closed), 3e-8 in another order (relu open); (ii) channel
+    1 has 0.25 at (0,4) and 1 + 0.25 + 3e-8 - 1 at (0,5): a tie that the first candidate wins in
+    tap order, a win of the second candidate in another; (iii) channel 2 has an exact tie 1 / 1
+    at (4,0) / (4,1), which the first candidate must win on both sides. Checked: every decision
+    the GPU took is one that fp32 arithmetic allows (the float64 value lies within rounding of
+    the threshold), the exact tie goes to the first candidate, and all gradients equal the
+    float64 gradients of the net with the GPU's own decisions imposed. Where the oracle took the
+    same decisions, the two are also compared directly."""
+    e = np.float32(3e-8)
+    X = np.zeros((6, 6), np.float32)
+    X[1, 1] = X[2, 2] = X[3, 3] = 1.0; X[4, 4] = 2.0                                  # (i)
+    X[0, 3] = X[0, 4] = X[0, 5] = X[1, 4] = X[1, 5] = X[2, 4] = 1.0; X[2, 5] = 2.0     # (ii)
+    X[4, 0] = X[4, 1] = 2.0                                                           # (iii)
+    w = np.zeros((3, 1, 3, 3), np.float32)
+    w[0, 0, 0, 0], w[0, 0, 1, 1], w[0, 0, 2, 2] = 1.0, e, -1.0
+    w[1, 0, 1, 0], w[1, 0, 1, 1], w[1, 0, 2, 0], w[1, 0, 2, 1] = 1.0, 0.25, e, -1.0
+    w[2, 0, 1, 1] = 0.5
+    x = np.zeros((2, 36), np.float32)
+    x[0] = X.ravel()
+    x[1] = np.linspace(-1.0, 1.0, 36, dtype=np.float32)     # an ordinary second sample
+    b = np.zeros(3, np.float32)
+    wf = np.random.default_rng(12).uniform(-0.5, 0.5, 27 * 3).astype(np.float32)
+    bf = np.zeros(3, np.float32)
+    t = np.zeros((2, 3), np.float32)
+    t[0, 1] = t[1, 2] = 1.0
+    layers = lambda api: [api.L_conv(6, 6, 1, 3, 3, pad_same=True), api.L_act("relu"), api.L_maxpool(6, 6, 3, 2),
+                          api.L_fc(27, 3), api.L_act("softmax")]
+    net, ref = T.Net(layers(T), 2, flags), O.OracleNet(layers(O), 2)
+    for i, which, a in ((0, 0, w.ravel()), (0, 1, b), (3, 0, wf), (3, 1, bf)):
+        net.set_param(i, which, a)
+        (ref.weight(i) if which == 0 else ref.bias(i))[:] = a
+    net.train_step(None, "ce_multiclass", 2, T.to_device(x), T.to_device(t), do_update=False)
+    ref.train_step(O.opt_desc("sgd"), "ce_multiclass", x, t, do_update=False)
+
+    # float64 pre-activations and the magnitude of the sums behind them
+    xp = np.zeros((2, 8, 8)); xp[:, 1:7, 1:7] = x.reshape(2, 6, 6)
+    z = np.zeros((2, 3, 6, 6)); mag = np.zeros_like(z)
+    for ky in range(3):
+        for kx in range(3):
+            for c in range(3):
+                term = np.float64(w[c, 0, ky, kx]) * xp[:, ky:ky + 6, kx:kx + 6]
+                z[:, c] += term; mag[:, c] += np.abs(term)
+    slack = 4 * np.finfo(np.float32).eps * mag       # what fp32 additions in any order can move a sum by
+    # the construction is what the docstring says
+    assert 0 < z[0, 0, 2, 2] < 1e-7 and z[0, 0, 2:4, 2:4].max() == z[0, 0, 2, 2]
+    assert z[0, 1, 0, 4] == 0.25 and 0 < z[0, 1, 0, 5] - 0.25 < 1e-7 and z[0, 1, 1, 4:6].max() < 0
+    assert z[0, 2, 4, 0] == z[0, 2, 4, 1] == 1.0 and z[0, 2, 5, 0:2].max() < 1.0
+
+    def decisions(relu_out, pooled, argmax):
+        arg = argmax.reshape(2, 27).astype(np.int64)
+        if relu_out is not None:
+            mask = relu_out.reshape(2, 3, 6, 6) > 0
+        else:
+            # a fused step keeps the relu's output out of memory: its decision is visible where it
+            # matters, at the winners of the pool windows (no gradient reaches the other elements)
+            mask = (z > 0).reshape(2, -1)
+            np.put_along_axis(mask, arg, pooled.reshape(2, 27) > 0, axis=1)
+            mask = mask.reshape(2, 3, 6, 6)
+        wrong = mask != (z > 0)
+        assert np.all(np.abs(z[wrong]) <= slack[wrong]), "a relu decision that fp32 rounding does not explain"
+        a = np.where(mask, z, 0.0).reshape(2, -1)
+        win = np.take_along_axis(a, arg, axis=1).reshape(2, 3, 3, 3)
+        best = a.reshape(2, 3, 3, 2, 3, 2).max(axis=(3, 5))
+        sl = slack.reshape(2, 3, 3, 2, 3, 2).max(axis=(3, 5))
+        assert np.all(win >= best - sl), "a max-pool winner that fp32 rounding does not explain"
+        return mask, arg
+
+    mask, arg = decisions(net.layer_out(1, 2) if net.out_written(1) else None, net.layer_out(2, 2),
+                          net.layer_argmax(2, 2))
+    omask, oarg = decisions(ref.layer_out(1, 2), ref.layer_out(2, 2), ref.layer_argmax(2, 2))
+    # the oracle adds in tap order: (i) gives exactly 0 (relu closed), (ii) a tie (first wins)
+    assert not omask[0, 0, 2, 2] and oarg[0, 9 + 2] == 36 + 4
+    # (iii) exact tie: the first candidate on both sides, whatever the order
+    assert arg[0, 18 + 6] == oarg[0, 18 + 6] == 72 + 4 * 6
+    same = np.array_equal(mask, omask) and np.array_equal(arg, oarg)
+    print(f"flags {flags}: GPU relu at (i) {'open' if mask[0, 0, 2, 2] else 'closed'}, pool winner at (ii) "
+          f"column {int(arg[0, 11]) - 36}; same decisions as the oracle: {same}", flush=True)
+
+    # float64 gradients with the GPU's decisions imposed
+    a = np.where(mask, z, 0.0).reshape(2, -1)
+    p = np.take_along_axis(a, arg, axis=1)
+    wf64 = wf.astype(np.float64).reshape(27, 3)
+    logits = p @ wf64 + bf
+    y = np.exp(logits - logits.max(1, keepdims=True)); y /= y.sum(1, keepdims=True)
+    dlog = y * t.sum(1, keepdims=True) - t
+    dwf, dbf = p.T @ dlog, dlog.sum(0)
+    dp = dlog @ wf64.T
+    da = np.zeros_like(a); np.put_along_axis(da, arg, dp, axis=1)
+    dz = da.reshape(2, 3, 6, 6) * mask
+    dw = np.zeros((3, 1, 3, 3)); dx = np.zeros((2, 8, 8))
+    for ky in range(3):
+        for kx in range(3):
+            for c in range(3):
+                dw[c, 0, ky, kx] = np.sum(xp[:, ky:ky + 6, kx:kx + 6] * dz[:, c])
+                dx[:, ky:ky + 6, kx:kx + 6] += np.float64(w[c, 0, ky, kx]) * dz[:, c]
+    want = {(0, 0): dw.ravel(), (0, 1): dz.sum(axis=(0, 2, 3)), (3, 0): dwf.ravel(), (3, 1): dbf}
+    for (i, which), v in want.items():
+        assert_close(net.layer_grad(i, which), v, what=f"flags {flags}: gradient {i}.{which} under the GPU's decisions")
+    if net.dx_written(0):
+        assert_close(net.layer_dx(0, 2), dx[:, 1:7, 1:7].reshape(2, 36), what=f"flags {flags}: input gradient")
+    if same:
+        for (i, which) in want:
+            assert_close(net.layer_grad(i, which), ref.layer_dw(i) if which == 0 else ref.layer_db(i),
+                         what=f"flags {flags}: gradient {i}.{which} vs oracle")
     net.close()

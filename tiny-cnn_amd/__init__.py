@@ -179,12 +179,14 @@ def copy_d2d(dst, src, nbytes=None, dst_offset=0, src_offset=0):
 
 
 class Feeder:
-    """Double-buffered upload of host batches (tdh_feeder_*): stage(x, t) copies the next batch
-    while the current step runs, acquire() returns device views of the batch staged last."""
+    """Pipelined upload of host batches (tdh_feeder_*): stage(x, t) hands a batch to the
+    feeder's worker thread (pinned copy + upload while earlier steps run; up to two batches
+    ahead), acquire() returns device views of the oldest staged batch."""
 
     def __init__(self, x_len, t_len, max_batch):
         self.x_len, self.t_len, self.max_batch = int(x_len), int(t_len), int(max_batch)
         self.h = C.c_void_p()
+        self._staged = []  # host arrays the worker thread may still read
         check(lib().tdh_feeder_create(C.c_size_t(self.x_len), C.c_size_t(self.t_len), self.max_batch,
                                       C.byref(self.h)), "tdh_feeder_create")
 
@@ -193,14 +195,15 @@ class Feeder:
         t = np.ascontiguousarray(t, np.float32)
         batch = x.shape[0]
         assert x.size == batch * self.x_len and t.size == batch * self.t_len
-        self._staged = (x, t)  # the worker thread reads them until acquire() returns
         check(lib().tdh_feeder_stage(self.h, batch, x.ctypes.data_as(C.c_void_p),
                                      t.ctypes.data_as(C.c_void_p)), "tdh_feeder_stage")
+        self._staged.append((x, t))  # the worker thread reads them until their acquire() returns
 
     def acquire(self):
         xp, tp, b = C.c_void_p(), C.c_void_p(), C.c_int()
         check(lib().tdh_feeder_acquire(self.h, C.byref(xp), C.byref(tp), C.byref(b)),
               "tdh_feeder_acquire")
+        self._staged.pop(0)
         return (DevBuf.view(xp.value, (b.value, self.x_len)), DevBuf.view(tp.value, (b.value, self.t_len)),
                 b.value)
 

@@ -2218,29 +2218,37 @@ class feeder {
  public:
   feeder(size_t x_len, size_t t_len, size_t max_batch) : x_len_(x_len), t_len_(t_len) {
     check(tdh_feeder_create(x_len, t_len, static_cast<int>(max_batch), &f_));
-    x_.resize(x_len * max_batch);
-    t_.resize(t_len * max_batch);
+    for (int b = 0; b < 2; ++b) {
+      x_[b].resize(x_len * max_batch);
+      t_[b].resize(t_len * max_batch);
+    }
   }
   feeder(const feeder &) = delete;
   feeder &operator=(const feeder &) = delete;
   ~feeder() {
     if (f_) tdh_feeder_destroy(f_);
   }
+  // Two batches may be on their way at once, and the feeder's thread reads a batch until it
+  // is acquired: the flattened copies alternate between two buffers (the one written here
+  // belonged to the batch staged two calls ago, which has been acquired by now).
   void stage(const std::vector<vec_t> &x, const std::vector<vec_t> &t, size_t first, size_t n) {
+    std::vector<float> &xf = x_[turn_], &tf = t_[turn_];
+    turn_ ^= 1;
     for (size_t s = 0; s < n; ++s) {
       if (x[first + s].size() < x_len_ || t[first + s].size() < t_len_)
         throw nn_error("fit: sample shorter than the network's input / output");
-      std::memcpy(x_.data() + s * x_len_, x[first + s].data(), x_len_ * sizeof(float));
-      std::memcpy(t_.data() + s * t_len_, t[first + s].data(), t_len_ * sizeof(float));
+      std::memcpy(xf.data() + s * x_len_, x[first + s].data(), x_len_ * sizeof(float));
+      std::memcpy(tf.data() + s * t_len_, t[first + s].data(), t_len_ * sizeof(float));
     }
-    check(tdh_feeder_stage(f_, static_cast<int>(n), x_.data(), t_.data()));
+    check(tdh_feeder_stage(f_, static_cast<int>(n), xf.data(), tf.data()));
   }
   tdh_feeder *get() const { return f_; }
 
  private:
   tdh_feeder *f_ = nullptr;
   size_t x_len_, t_len_;
-  std::vector<float> x_, t_;
+  std::vector<float> x_[2], t_[2];
+  int turn_ = 0;
 };
 }  // namespace detail
 
@@ -2567,8 +2575,8 @@ class network<sequential> {
     opt.reset();  // network.h:856; the device copy of the state vectors is cleared with it
     detail::check(tdh_net_reset_optimizer(net_));
     tdh_opt o = opt.descriptor();
-    // batches travel double-buffered: while a step runs, the next batch is flattened, copied
-    // to pinned memory and uploaded
+    // batches travel two ahead: while a step runs, the batch after it is being uploaded and the
+    // one after that flattened and copied to pinned memory
     detail::feeder feed(in_len, out_len, batch_size);
     const size_t per_epoch = (inputs.size() + batch_size - 1) / batch_size;
     const size_t total     = per_epoch * static_cast<size_t>(epoch);
@@ -2578,11 +2586,12 @@ class network<sequential> {
       feed.stage(inputs, desired_outputs, i, n);
     };
     if (total) stage(0);
+    if (total > 1) stage(1);
     for (size_t k = 0; k < total; ++k) {
       const float *xd = nullptr, *td = nullptr;
       int n = 0;
       detail::check(tdh_feeder_acquire(feed.get(), &xd, &td, &n));
-      if (k + 1 < total) stage(k + 1);  // the feeder's thread copies while this one launches
+      if (k + 2 < total) stage(k + 2);  // the feeder's thread copies and uploads while this one launches
       draw_dropout_masks(static_cast<size_t>(n));
       detail::check(tdh_net_train_step(net_, &o, Error::kind, n, xd, td, 1));
       on_batch_enumerate();
