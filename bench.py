@@ -48,7 +48,7 @@ class NetWorkload:
         (self.spec, self.params, x, t, self.batch, self.loss, self.opt_kind,
          self.opt_kw) = W.make_batch(name)
         self.net = T.Net(W.build_layers(T, self.spec), self.batch,
-                         T.NET_FUSE_ACT_GRAD | T.NET_GRAPH)
+                         T.NET_FUSE_ACT_GRAD | T.NET_GRAPH | T.NET_SAMPLE_STEP)
         for (i, which, a) in self.params:
             self.net.set_param(i, which, a)
         self.opt = T.opt_desc(self.opt_kind, **self.opt_kw)

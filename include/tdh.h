@@ -273,7 +273,16 @@ typedef struct tdh_net tdh_net;
 
 enum {
   TDH_NET_FUSE_ACT_GRAD = 1, /* fold activation gradients into the next layer's dX epilogue */
-  TDH_NET_GRAPH         = 2  /* replay the step as a captured HIP graph */
+  TDH_NET_GRAPH         = 2, /* replay the step as a captured HIP graph */
+  /* A net whose activations of one sample fit in a workgroup's local memory (LeNet-5) trains in
+   * three launches: one workgroup per sample runs forward, the loss gradient and the input
+   * gradients of every layer; a second launch computes every sample's weight and bias
+   * gradients; the optimizer launch adds those up and updates (a step without an update adds
+   * them to the gradient tensors in sample order instead, edge::merge_grads,
+   * tiny_dnn/node.h:89-103). Every layer output, input gradient and max-pool record is still
+   * written to memory. Nets that do not qualify (size, batch normalization, dropout, a softmax
+   * that is not the closing layer of a cross_entropy_multiclass net) ignore the flag. */
+  TDH_NET_SAMPLE_STEP   = 4
 };
 
 int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int flags,

@@ -134,4 +134,6 @@ def assert_within_propagated_tolerance(gpu, oracle, truth, opt, trace, what, tol
           f"p99 {qo:.3e}; gpu-oracle max {rel_err(gpu, oracle):.3e}; worst element uses "
           f"{eg[worst] / allowed[worst]:.2f} of its allowance ({allowed[worst] / scale[worst]:.2e} relative)")
     assert np.all(eg <= allowed), f"{what}: element {worst} is {eg[worst]:.3e} off, allowed {allowed[worst]:.3e}"
-    assert qg <= 2 * qo + 1e-6, f"{what}: 99th percentile of the error {qg:.3e}, the oracle's {qo:.3e}"
+    # (slack 3e-6: for a tensor of 16 biases the 99th percentile is the largest error, and two
+    # fp32 summation orders differ by a few 1e-6 there whichever is nearer to float64)
+    assert qg <= 2 * qo + 3e-6, f"{what}: 99th percentile of the error {qg:.3e}, the oracle's {qo:.3e}"

@@ -985,7 +985,7 @@ def test_net_with_batchnorm_and_dropout_matches_oracle_and_reference_fit(T, O, W
     net.close()
 
 
-@pytest.mark.parametrize("flags", [0, 3])
+@pytest.mark.parametrize("flags", [0, 3, 7])
 def test_decisions_that_hang_on_summation_order_are_legitimate_and_the_gradients_follow_them(T, O, flags):
     """The one class of difference from the oracle that no tolerance covers: a relu whose
     pre-activation, or a max-pool whose two best candidates, differ by less than fp32 rounding

@@ -1,0 +1,172 @@
+"""TDH_NET_SAMPLE_STEP: a small net trains with one workgroup per sample (forward, loss gradient
+and the input gradients in one launch out of LDS), a launch for every sample's weight and bias
+gradients, and the optimizer launch that adds them up (a step without an update adds them in
+sample order with a launch of its own). Against the oracle (every layer output, input gradient,
+max-pool record, weight and bias gradient; updated weights over several steps), against the
+layer-by-layer step of the same library, against tiny-dnn's own fit (tests/golden/net_steps.npz),
+and replayed from a captured graph bit for bit."""
+import numpy as np
+import pytest
+
+from conftest import assert_close, input_checksum, REL_TOL
+from f64_truth import assert_within_propagated_tolerance, f64_net_steps
+
+pytestmark = pytest.mark.gpu
+
+SAMPLE, FUSE, GRAPH = 4, 1, 2
+
+# nets that the per-sample kernel takes: every layer kind it knows, a connection table, sizes
+# that leave a column outside every pool window, each loss
+NETS = {
+    "lenet5": ("workload", "lenet5_b16"),
+    "lenet5_c3_table": ("workload", "lenet5_mnist_b16"),
+    "maxpool_relu_softmax_xent": ([("conv", 12, 12, 2, 3, 8, True), ("maxpool", 12, 12, 8, 2), ("act", "relu"),
+                                   ("conv", 6, 6, 8, 3, 12, False), ("act", "leaky_relu", (0.1, 0.0)),
+                                   ("fc", 12 * 16, 24), ("act", "sigmoid"), ("fc", 24, 10), ("act", "softmax")],
+                                  "ce_multiclass", "adam"),
+    "odd_sizes_uncovered_column_ce": ([("conv", 15, 11, 3, 5, 6, True), ("act", "tanh"), ("maxpool", 15, 11, 6, 2),
+                                      ("fc", 6 * 5 * 7, 6), ("act", "sigmoid")], "ce", "momentum"),
+    "fc_only_mse": ([("fc", 40, 30), ("act", "tanh"), ("fc", 30, 7)], "mse", "adagrad"),
+}
+
+
+def build(T, O, W, name, batch, flags, seed=3):
+    spec = NETS[name]
+    if spec[0] == "workload":
+        spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(spec[1], batch=batch)
+    else:
+        spec, loss, opt_kind = spec
+        opt_kw = {}
+        rng = np.random.default_rng(seed)
+        params = W.init_params(spec, "xavier", rng)
+        params = [(i, which, a if which == 0 else rng.uniform(-0.1, 0.1, a.size).astype(np.float32))
+                  for (i, which, a) in params]
+        first = spec[0]
+        n_in = first[1] * first[2] * first[3] if first[0] == "conv" else first[1]
+        n_out = [l for l in spec if l[0] == "fc"][-1][2]
+        x = rng.standard_normal((batch, n_in)).astype(np.float32)
+        if loss == "ce":
+            t = rng.uniform(0.05, 0.95, (batch, n_out)).astype(np.float32)
+        elif loss == "ce_multiclass":
+            t = np.eye(n_out, dtype=np.float32)[rng.integers(0, n_out, batch)]
+        else:
+            t = rng.uniform(-0.8, 0.8, (batch, n_out)).astype(np.float32)
+    net = T.Net(W.build_layers(T, spec), batch, flags)
+    ref = O.OracleNet(W.build_layers(O, spec), batch)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+        (ref.weight(i) if which == 0 else ref.bias(i))[:] = a
+    return spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref
+
+
+@pytest.mark.parametrize("name", list(NETS))
+@pytest.mark.parametrize("batch", [16, 5])
+def test_every_tensor_of_a_sample_step_matches_oracle(T, O, W, name, batch):
+    spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref = build(T, O, W, name, batch, SAMPLE | FUSE)
+    xd, td = T.to_device(x), T.to_device(t)
+    net.train_step(None, loss, batch, xd, td, do_update=False)
+    ref.train_step(O.opt_desc(opt_kind), loss, x, t, do_update=False)
+    for i, l in enumerate(spec):
+        assert net.out_written(i)      # the kernel writes every layer's output to memory as well
+        assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{name} layer {i} output")
+        if l[0] == "maxpool":
+            assert np.array_equal(net.layer_argmax(i, batch).astype(np.int64), ref.layer_argmax(i, batch)), f"{name} layer {i} argmax"
+        if net.param_size(i, 0):
+            assert_close(net.layer_grad(i, 0), ref.layer_dw(i), what=f"{name} layer {i} dW")
+            assert_close(net.layer_grad(i, 1), ref.layer_db(i), what=f"{name} layer {i} db")
+        assert net.dx_written(i)
+        assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), what=f"{name} layer {i} dX")
+    # a second backward pass adds to the weight gradients (layer.h:680 clears them at the update)
+    net.train_step(None, loss, batch, xd, td, do_update=False)
+    for (i, which, _) in params:
+        want = 2.0 * (ref.layer_dw(i) if which == 0 else ref.layer_db(i))
+        assert_close(net.layer_grad(i, which), want, what=f"{name} gradient {i}.{which} after two passes")
+    net.close()
+
+
+@pytest.mark.parametrize("name", list(NETS))
+def test_updated_weights_of_sample_steps_match_oracle_and_the_layered_step(T, O, W, name):
+    """Three optimizer steps: against the oracle, and the captured replay (flags 7) bit for bit
+    against eager launches (flags 5); a short last batch goes through the same kernels."""
+    batch, steps = 16, 3
+    spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref = build(T, O, W, name, batch, SAMPLE | FUSE)
+    *_, replay, _ = build(T, O, W, name, batch, SAMPLE | FUSE | GRAPH)
+    *_, layered, _ = build(T, O, W, name, batch, FUSE)
+    opts = [T.opt_desc(opt_kind, **opt_kw) for _ in range(3)]
+    ropt = O.opt_desc(opt_kind, **opt_kw)
+    xd, td = T.to_device(x), T.to_device(t)
+    sizes = [batch, batch, 7] if opt_kind != "adagrad" else [batch] * steps   # (the float64 helper steps whole batches)
+    for n in sizes:
+        for k, m in enumerate((net, replay, layered)):
+            m.train_step(opts[k], loss, n, xd, td)
+        ref.train_step(ropt, loss, x[:n], t[:n])
+    truth = None
+    if opt_kind == "adagrad":      # see test_updated_weights_match_oracle in test_gpu_nets.py
+        o64 = {"kind": "adagrad", "alpha": opts[0].alpha}
+        truth, trace = f64_net_steps(spec, params, x, t, loss, steps, o64, want_trace=True)
+    for (i, which, a) in params:
+        got, want = net.get_param(i, which), (ref.weight(i) if which == 0 else ref.bias(i))
+        assert np.array_equal(got, replay.get_param(i, which)), f"{name} parameter {i}.{which}: replay differs from eager"
+        if truth is not None:
+            assert_within_propagated_tolerance(got, want, truth[(i, which)], o64, trace[(i, which)],
+                                               f"{name} updated parameter {i}.{which}")
+        else:
+            assert_close(got, want, what=f"{name} updated parameter {i}.{which}")
+            assert_close(got, layered.get_param(i, which), what=f"{name} parameter {i}.{which} against the layered step")
+        assert not net.layer_grad(i, which).any()
+    assert opts[0].b1_t == ropt.b1_t == opts[1].b1_t and opts[0].b2_t == ropt.b2_t
+    for m in (net, replay, layered):
+        m.close()
+
+
+@pytest.mark.parametrize("key", ["lenet5_b16", "lenet5_mnist_b16"])
+def test_sample_steps_match_reference_fit(T, W, net_steps, key):
+    """Against what tiny-dnn's network<sequential>::fit itself produced, replayed from a graph."""
+    g = net_steps
+    batch, steps, stride = int(g[f"{key}.batch"]), int(g[f"{key}.steps"]), int(g[f"{key}.stride"])
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(key, batch=batch)
+    assert input_checksum(x, t, params) == float(g[f"{key}.input_checksum"])
+    net = T.Net(W.build_layers(T, spec), batch, SAMPLE | FUSE | GRAPH)
+    for (i, which, a) in params:
+        net.set_param(i, which, a)
+    opt = T.opt_desc(opt_kind, **opt_kw)
+    xd, td = T.to_device(x), T.to_device(t)
+    for _ in range(steps):
+        net.train_step(opt, loss, batch, xd, td)
+    truth = None
+    if opt_kind == "adagrad":
+        o64 = {"kind": "adagrad", "alpha": opt.alpha}
+        truth, trace = f64_net_steps(spec, params, x, t, loss, steps, o64, want_trace=True)
+    for (i, which, a) in params:
+        got = net.get_param(i, which)
+        if truth is not None:
+            assert_within_propagated_tolerance(got, g[f"{key}.p{i}.{which}"], truth[(i, which)], o64,
+                                               trace[(i, which)], f"{key} parameter {i}.{which}")
+        else:
+            assert_close(got[::stride], g[f"{key}.p{i}.{which}"], what=f"{key} parameter {i}.{which}")
+    net.close()
+
+
+def test_nets_that_do_not_qualify_ignore_the_flag(T, O, W):
+    """Batch normalization, or more arithmetic per sample than the kernel is meant for: the flag
+    changes nothing, the layer-by-layer step runs (same bits as without the flag)."""
+    for spec, batch in (([("fc", 12, 8), ("batchnorm", 8, 1), ("act", "relu"), ("fc", 8, 4)], 6),
+                        (W.cifar10_cnn(), 4)):
+        rng = np.random.default_rng(8)
+        params = W.init_params([l for l in spec], "xavier", rng)
+        first = spec[0]
+        n_in = first[1] * first[2] * first[3] if first[0] == "conv" else first[1]
+        n_out = [l for l in spec if l[0] == "fc"][-1][2]
+        x = rng.standard_normal((batch, n_in)).astype(np.float32)
+        t = np.eye(n_out, dtype=np.float32)[rng.integers(0, n_out, batch)]
+        loss = "ce_multiclass" if spec[-1][0] == "act" else "mse"
+        got = []
+        for flags in (FUSE, FUSE | SAMPLE):
+            net = T.Net(W.build_layers(T, spec), batch, flags)
+            for (i, which, a) in params:
+                net.set_param(i, which, a)
+            net.train_step(T.opt_desc("sgd"), loss, batch, T.to_device(x), T.to_device(t))
+            got.append([net.get_param(i, which) for (i, which, _) in params])
+            net.close()
+        for a, b in zip(*got):
+            assert np.array_equal(a, b)

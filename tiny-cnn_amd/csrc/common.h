@@ -187,7 +187,7 @@ constexpr int OPT_MULTI_ELEMS_PER_BLOCK = 1024;  // one 16-byte access per threa
 // whose weight-gradient kernels left their reductions to the optimizer. Such a tensor's table
 // entry has block_elems == OPT_SUM_ELEMS_PER_BLOCK.
 constexpr int OPT_SUM_ELEMS_PER_BLOCK = 128;
-constexpr int OPT_PENDING_MAX         = 8;
+constexpr int OPT_PENDING_MAX         = 32;
 struct OptPendingSum {
   const float *partial;
   const float *g;  // the gradient tensor (an OptTensor::g) the sum belongs to

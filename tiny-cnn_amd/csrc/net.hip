@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "tiny_net.h"
 
 struct tdh_net {
   struct Layer {
@@ -72,6 +73,11 @@ struct tdh_net {
                              // layers, because branches of the captured step run side by side
   std::vector<hipEvent_t> events;  // fork/join points of the captured step
   std::vector<void *> allocs;
+  // the one-workgroup-per-sample step of a small net (tiny_net.hip), when the net qualifies
+  bool tiny_ok = false;
+  tdh::TinyPlan tiny;
+  tdh::TinyPlan *tiny_dev = nullptr;  // the same in device memory
+  tdh::TinyMerge tiny_merge;
 };
 
 namespace tdh {
@@ -167,6 +173,138 @@ bool net_defers_serially(const tdh_net *net, int batch) {
   return (net->flags & TDH_NET_GRAPH) && (net->flags & TDH_NET_FUSE_ACT_GRAD) &&
          net_forward_flop(net, batch) < 1e8;
 }
+
+// The plan of the one-workgroup-per-sample step (tiny_net.hip) for a net that qualifies: at most
+// TINY_MAX_LAYERS layers of the kinds that kernel knows, every layer output of one sample and two
+// gradient buffers within a workgroup's LDS, little arithmetic per sample, and room for the
+// per-sample gradient slices. Leaves net->tiny_ok false otherwise: the layer-by-layer step runs.
+int build_tiny_plan(tdh_net *net) {
+  net->tiny_ok = false;
+  const int n = static_cast<int>(net->layers.size());
+  if (!(net->flags & TDH_NET_SAMPLE_STEP) || n > TINY_MAX_LAYERS || net->max_batch > 512) return TDH_OK;
+  if (net_forward_flop(net, 1) > 4e6) return TDH_OK;
+  TinyPlan &P = net->tiny;
+  std::memset(&P, 0, sizeof(P));
+  P.n       = n;
+  P.in_size = static_cast<int>(net->layers[0].in_size);
+  size_t lds = net->layers[0].in_size, gmax = net->layers[0].in_size, slice_floats = 0;
+  int tensors = 0;
+  for (int i = 0; i < n; ++i) {
+    const tdh_net::Layer &L = net->layers[i];
+    const tdh_layer &sp = L.spec;
+    TinyLayer &T = P.l[i];
+    T.kind = sp.kind;
+    T.in_size = static_cast<int>(L.in_size); T.out_size = static_cast<int>(L.out_size);
+    T.w = L.w; T.b = L.b; T.out = L.out;
+    T.dx = i == 0 ? net->dx_in : net->layers[i - 1].dout;
+    T.nw = static_cast<int>(L.w_size); T.nb = static_cast<int>(L.b_size);
+    T.lds_in  = i == 0 ? 0 : P.l[i - 1].lds_out;
+    T.lds_out = static_cast<int>(lds);
+    lds += L.out_size;
+    gmax = std::max(gmax, L.out_size);
+    switch (sp.kind) {
+      case TDH_L_CONV: {
+        const tdh_conv_desc &d = sp.conv;
+        T.C = d.in_c; T.H = d.in_h; T.W = d.in_w; T.K = d.out_c;
+        T.OW = conv_out_length(d.in_w, d.k_w, d.w_stride, d.w_dilation, d.pad_same);
+        T.OH = conv_out_length(d.in_h, d.k_h, d.h_stride, d.h_dilation, d.pad_same);
+        T.R = d.k_h; T.S = d.k_w; T.sh = d.h_stride; T.sw = d.w_stride;
+        T.ph = d.pad_same ? d.k_h / 2 : 0; T.pw = d.pad_same ? d.k_w / 2 : 0;
+        T.has_bias = d.has_bias;
+        T.tbl = d.tbl ? L.tbl_dev : nullptr;
+        if (d.w_dilation != 1 || d.h_dilation != 1) return TDH_OK;
+        P.flop_per_sample += 6.0 * L.out_size * d.in_c * d.k_w * d.k_h;
+      } break;
+      case TDH_L_FC:
+        T.has_bias = sp.fc_bias;
+        P.flop_per_sample += 6.0 * sp.fc_in * sp.fc_out;
+        break;
+      case TDH_L_MAXPOOL:
+      case TDH_L_AVEPOOL: {
+        const tdh_pool_desc &d = sp.pool;
+        if (d.pad_same) return TDH_OK;
+        if (sp.kind == TDH_L_AVEPOOL && (d.stride_w != d.pool_w || d.stride_h != d.pool_h)) return TDH_OK;
+        T.C = d.in_c; T.H = d.in_h; T.W = d.in_w; T.K = d.in_c;
+        T.OW = pool_out_length(d.in_w, d.pool_w, d.stride_w, d.ceil_mode, d.pad_same);
+        T.OH = pool_out_length(d.in_h, d.pool_h, d.stride_h, d.ceil_mode, d.pad_same);
+        T.R = d.pool_h; T.S = d.pool_w; T.sh = d.stride_h; T.sw = d.stride_w;
+        T.scale = 1.0f / static_cast<float>(d.pool_w * d.pool_h);
+        T.argmax = L.argmax;
+        T.has_bias = sp.kind == TDH_L_AVEPOOL;
+      } break;
+      case TDH_L_ACT:
+        T.act = sp.act; T.p0 = sp.act_p[0];
+        if (sp.act == TDH_ACT_SOFTMAX) {
+          if (i != n - 1) return TDH_OK;   // only as the closing layer (with cross_entropy_multiclass)
+        } else if (sp.act != TDH_ACT_TANH && sp.act != TDH_ACT_RELU && sp.act != TDH_ACT_SIGMOID &&
+                   sp.act != TDH_ACT_LEAKY_RELU) {
+          return TDH_OK;
+        }
+        break;
+      default: return TDH_OK;   // batch normalization, dropout: the layer-by-layer step
+    }
+    tensors += (L.w_size ? 1 : 0) + (L.b_size ? 1 : 0);
+    slice_floats += (ceil_div_sz(L.w_size * static_cast<size_t>(net->max_batch), 4) * 4) +
+                    (ceil_div_sz(L.b_size * static_cast<size_t>(net->max_batch), 4) * 4);   // (16-byte aligned slices)
+  }
+  P.lds_g0 = static_cast<int>(lds);
+  P.lds_g1 = static_cast<int>(lds + gmax);
+  lds += 2 * gmax;
+  lds = (lds + 3) & ~static_cast<size_t>(3);   // (16-byte reads of the staged filters)
+  P.lds_w = static_cast<int>(lds);
+  lds += TINY_SCRATCH_FLOATS;
+  P.lds_floats = static_cast<int>(lds);
+  P.dloss      = net->layers[n - 1].dout;
+  P.mse_factor = 2.0f / static_cast<float>(net->layers[n - 1].out_size);
+  if (tensors > TINY_MAX_TENSORS || slice_floats > (64u << 20)) return TDH_OK;
+  TDH_TRY(tiny_build_jobs(P));   // (adds the framed dY's LDS to the plan's)
+  if (std::max(P.lds_floats, P.lds_job_floats) * sizeof(float) > TINY_LDS_MAX_BYTES) return TDH_OK;
+  float *slices = nullptr;
+  TDH_TRY(net_alloc(net, slice_floats, &slices, false));
+  TinyMerge &M = net->tiny_merge;
+  std::memset(&M, 0, sizeof(M));
+  int blocks = 0;
+  for (int i = 0; i < n; ++i) {
+    tdh_net::Layer &L = net->layers[i];
+    TinyLayer &T = P.l[i];
+    for (int which = 0; which < 2; ++which) {
+      const size_t len = which ? L.b_size : L.w_size;
+      if (!len) continue;
+      (which ? T.gb : T.gw) = slices;
+      M.slices[M.n] = slices;
+      M.g[M.n]      = which ? L.db : L.dw;
+      M.len[M.n]    = static_cast<int>(len);
+      M.first_block[M.n] = blocks;
+      blocks += ceil_div(static_cast<int>(len), 256);
+      ++M.n;
+      slices += ceil_div_sz(len * static_cast<size_t>(net->max_batch), 4) * 4;
+    }
+  }
+  M.first_block[M.n] = blocks;
+  for (int i = 0; i < n; ++i) {
+    TinyLayer &T = P.l[i];
+    const auto fd = [](int v) { return FastDiv(static_cast<uint32_t>(v > 0 ? v : 1)); };
+    T.d_oplane = fd(T.OH * T.OW); T.d_ow = fd(T.OW); T.d_iplane = fd(T.H * T.W); T.d_w = fd(T.W);
+    T.d_taps = fd(T.R * T.S); T.d_s = fd(T.S); T.d_c = fd(T.C); T.d_out = fd(T.out_size);
+    T.d_nk = fd(T.C * T.R * T.S);
+  }
+  float *dev = nullptr;
+  TDH_TRY(net_alloc(net, ceil_div_sz(sizeof(TinyPlan), sizeof(float)), &dev, false));
+  net->tiny_dev = reinterpret_cast<TinyPlan *>(dev);
+  TDH_TRY(tdh_memcpy_h2d(net->tiny_dev, &P, sizeof(TinyPlan)));
+  TDH_TRY(tiny_prepare());
+  net->tiny_ok = true;
+  return TDH_OK;
+}
+
+// whether this step runs as the one-workgroup-per-sample kernel
+bool tiny_step_applies(const tdh_net *net, int loss_kind) {
+  if (!net->tiny_ok || net->test_phase) return false;
+  const tdh_layer &last = net->layers.back().spec;
+  if (last.kind == TDH_L_ACT && last.act == TDH_ACT_SOFTMAX && loss_kind != TDH_LOSS_CE_MULTICLASS) return false;
+  return loss_kind == TDH_LOSS_MSE || loss_kind == TDH_LOSS_CE_MULTICLASS || loss_kind == TDH_LOSS_CE;
+}
+
 bool layer_forks(const tdh_net::Layer &L) {
   return L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC;
 }
@@ -519,7 +657,10 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
         t.first_block = block;
         // weight gradients whose kernels may leave split sums to the optimizer: small blocks,
         // eight groups of lanes add the slices of OPT_SUM_ELEMS_PER_BLOCK elements
-        t.block_elems = (L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC) && (flags & TDH_NET_GRAPH)
+        // (and every tensor of a net that may run the workgroup-per-sample step, whose
+        // per-sample slices take the same way)
+        t.block_elems = (((L.spec.kind == TDH_L_CONV || L.spec.kind == TDH_L_FC) && (flags & TDH_NET_GRAPH)) ||
+                         (flags & TDH_NET_SAMPLE_STEP))
                           ? OPT_SUM_ELEMS_PER_BLOCK : OPT_MULTI_ELEMS_PER_BLOCK;
         if (n > (1u << 22)) t.block_elems = OPT_MULTI_ELEMS_PER_BLOCK;  // (bandwidth matters there)
         (which ? L.b_sums_in_opt : L.w_sums_in_opt) = t.block_elems == OPT_SUM_ELEMS_PER_BLOCK;
@@ -565,6 +706,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
         net->events.push_back(e);
     }
   }
+  if (rc == TDH_OK) rc = build_tiny_plan(net);
   // reserve the scratch every layer may need, so that no op ever has to grow it
   if (rc == TDH_OK) rc = ws_begin(net->scratch);
   if (rc != TDH_OK) {
@@ -709,6 +851,36 @@ int tdh_net_forward(tdh_net *net, int batch, const float *x) {
 static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
                         const float *t, int do_update, const float *powers_in, float *powers_out,
                         bool forked = false) {
+  if (tiny_step_applies(net, loss_kind)) {
+    // a small net: one workgroup per sample runs forward, loss and the input gradients out of
+    // LDS, a second launch computes every sample's weight and bias gradients, a third adds
+    // those slices in sample order, the fourth is the optimizer (tiny_net.hip)
+    const tdh_layer &closing = net->layers.back().spec;
+    const int softmax_xent = closing.kind == TDH_L_ACT && closing.act == TDH_ACT_SOFTMAX;
+    net->dx_unwritten.assign(net->layers.size(), 0);   // everything is written to memory as well
+    net->out_unwritten.assign(net->layers.size(), 0);
+    TDH_TRY(launch_tiny_step(net->tiny, net->tiny_dev, loss_kind, softmax_xent, batch, x, t));
+    TDH_TRY(launch_tiny_params(net->tiny, net->tiny_dev, batch, x));
+    // the samples' slices: added to the gradient tensors in sample order by a launch of their
+    // own when the step stops there; otherwise the optimizer adds them up as it does the split
+    // sums of the layer-by-layer step (it clears the gradient tensors afterwards either way)
+    const TinyMerge &M = net->tiny_merge;
+    bool to_optimizer = do_update && M.n <= OPT_PENDING_MAX;
+    OptPending pending;
+    pending.n = 0;
+    for (int j = 0; j < M.n && to_optimizer; ++j) {
+      bool small_blocks = false;
+      for (const tdh_net::Layer &L : net->layers)
+        if ((M.g[j] == L.dw && L.w_sums_in_opt) || (M.g[j] == L.db && L.b_sums_in_opt)) small_blocks = true;
+      to_optimizer = small_blocks;
+      pending.sum[pending.n++] = {M.slices[j], M.g[j], static_cast<uint32_t>(batch), static_cast<uint32_t>(M.len[j])};
+    }
+    if (!to_optimizer) TDH_TRY(launch_tiny_merge(net->tiny_merge, batch));
+    if (!do_update) return TDH_OK;
+    TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks, net->opt_params, 1.0f,
+                                    1, powers_in, powers_out, to_optimizer ? &pending : nullptr));
+    return post_update(net);
+  }
   Context &c = ctx();
   struct KeepScratch {  // hands out disjoint scratch pieces for the whole backward pass
     Context &c;

@@ -3029,7 +3029,7 @@ class network<sequential> {
     }
     tdh_net *fresh = nullptr;
     detail::check(tdh_net_create(raw.data(), static_cast<int>(raw.size()), static_cast<int>(batch),
-                                 TDH_NET_FUSE_ACT_GRAD | TDH_NET_GRAPH, &fresh));
+                                 TDH_NET_FUSE_ACT_GRAD | TDH_NET_GRAPH | TDH_NET_SAMPLE_STEP, &fresh));
     if (net_) {
       for (size_t i = 0; i < layers_.size(); ++i)
         for (int which = 0; which < 4; ++which) {
