@@ -82,6 +82,31 @@ def test_large_fc_weight_gradient_from_memory_fragments(T, bs, ni, no):
     assert np.array_equal(dw2.numpy(), before + dw.numpy())
 
 
+@pytest.mark.parametrize("bs,ni,no", [
+    (250, 3100, 1000),   # ragged in both directions, halves of the outputs that are no whole group, idle tiles
+    (256, 4096, 264),    # the smallest reduction the kernel takes: one group and a tail per half
+    (200, 4160, 2048),   # whole groups; a last column tile of its own
+])
+def test_large_fc_input_gradient_from_memory_fragments(T, bs, ni, no):
+    """dX of a fully-connected layer with a tile for (nearly) every compute unit runs on a kernel
+    that feeds the matrix cores from memory (no LDS, no split reduction): against float64, twice
+    with equal bits, and linear in dY bit for bit."""
+    rng = np.random.default_rng(bs + ni + no)
+    x = rng.uniform(-1, 1, (bs, ni)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, ni * no).astype(np.float32)
+    dy = rng.standard_normal((bs, no)).astype(np.float32)
+    xd, wd = T.to_device(x), T.to_device(w)
+    dx, dw, db = T.DevBuf((bs, ni)), T.DevBuf((ni * no,)), T.DevBuf((no,))
+    T.fc_bwd(ni, no, True, bs, xd, wd, T.to_device(dy), dx, dw, db)
+    got = dx.numpy().copy()
+    assert_close(got, dy.astype(np.float64) @ w.reshape(ni, no).astype(np.float64).T, what="dx")
+    dx.upload(np.full((bs, ni), np.nan, np.float32))
+    T.fc_bwd(ni, no, True, bs, xd, wd, T.to_device(dy), dx, dw, db)
+    assert np.array_equal(dx.numpy(), got)
+    T.fc_bwd(ni, no, True, bs, xd, wd, T.to_device(dy * 2), dx, dw, db)
+    assert np.array_equal(dx.numpy(), 2 * got)
+
+
 def test_config3_fc_backward_adam_full_size(T, O, W):
     """configs[2]: batch 256, 4096 -> 4096, tanh, Adam on W and b."""
     x, w, b, dy = W.fc_bwd_case()

@@ -1124,6 +1124,145 @@ static bool fc_dw_direct_applies(int in, int out, int batch, const float *x, con
          !(reinterpret_cast<uintptr_t>(dw) & 7);
 }
 
+// ---- dX of a large fully-connected layer
+//
+//   dX[b][i] = sum_o dY[b][o] * W[i][o]        (fully_connected_op_internal.h:42-54)
+//
+// Both operands have the reduction index (the output) as their fast one, so a tile of either is
+// staged with 16-byte reads along its rows and 16-byte LDS writes, untransposed: [row][128
+// outputs], rows padded by four floats. A lane of a v_mfma_f32_32x32x2_f32 stands for (row l%32,
+// reduction element l/32) on both sides, so one 16-byte LDS read, the row's outputs
+// k + 4*(l/32) .. + 3, feeds four MFMAs: component j pairs output k + j (lanes 0-31) with
+// k + 4 + j (lanes 32-63), the same pairing on both sides. No split of the reduction over
+// workgroups and no second launch: a workgroup owns 64 samples x 64 inputs (one workgroup per
+// compute unit for 256 x 4096), eight waves = 2 x 2 blocks of 32 x 32 times the two halves of
+// every staged chunk, so a SIMD holds two waves that fill each other's waits; the halves meet in
+// LDS at the end and add up in a fixed order. (Fragments read straight from memory, a lane's
+// 16-byte word of its own row, touch 32 cache lines per load: 124 us against 96 for the general
+// kernel and its split reduction.)
+constexpr int FDX_BK = 128;            // outputs per staged chunk
+constexpr int FDX_LD = FDX_BK + 4;     // floats of a staged row
+
+struct FcDxTile {
+  const float *dy, *w;
+  float *dx;
+  ActGrad ag;
+  int batch, in, out, tiles_m, tiles_n, n_per_xcd;
+};
+
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+fc_dx_tile_kernel(const FcDxTile f) {
+  __shared__ __attribute__((aligned(16))) float tile[2][128][FDX_LD];   // rows 0-63: dY, 64-127: W
+  // (behind the last chunk the same memory carries the upper half's blocks, [block][register][lane])
+  float (*halves)[16][64] = reinterpret_cast<float (*)[16][64]>(&tile[0][0][0]);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 31, h = lane >> 5;
+  const int wm = wave & 1, wn = (wave >> 1) & 1, kh = wave >> 2;
+  // Workgroups go to the eight XCDs round-robin in launch order. An XCD gets a run of column
+  // tiles with all their row tiles, so that the rows of W it reads are read by nobody else and
+  // its row tiles share them in its L2.
+  const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+  const int tm = seq % f.tiles_m, tn = xcd * f.n_per_xcd + seq / f.tiles_m;
+  if (tn >= f.tiles_n) return;
+  const int b0 = tm * 64, i0 = tn * 64;
+
+  // staging: thread t moves the 16-byte word t % W4 of the rows t / W4 + ROWS*i
+  // (rows past the batch or the layer's inputs are read at the last row and never stored)
+  constexpr int W4 = FDX_BK / 4, ROWS = 512 / W4, PASSES = 128 / ROWS;
+  const int s_row = tid / W4, s_c4 = tid % W4;
+  unsigned s_off[PASSES];
+#pragma unroll
+  for (int i = 0; i < PASSES; ++i) {
+    const int row = s_row + ROWS * i;
+    s_off[i] = i < PASSES / 2 ? static_cast<unsigned>(min(b0 + row, f.batch - 1)) * f.out
+                              : static_cast<unsigned>(min(i0 + row - 64, f.in - 1)) * f.out;
+  }
+  // two chunks are on their way from memory while a third is multiplied: W streams in from
+  // memory, and one chunk's products are shorter than that trip
+  float4 stg[2][PASSES];
+  auto fetch = [&](int k0, auto to) {
+    constexpr int T = decltype(to)::value;
+    const int k = min(k0 + 4 * s_c4, f.out - 4);
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      stg[T][i] = *reinterpret_cast<const float4 *>((i < PASSES / 2 ? f.dy : f.w) + (s_off[i] + static_cast<unsigned>(k)));
+  };
+  // (a word past the layer's outputs was read somewhere valid and is stored as zeros)
+  auto stage = [&](int k0, int buf, auto from) {
+    constexpr int T = decltype(from)::value;
+    const bool on = k0 + 4 * s_c4 < f.out;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      *reinterpret_cast<float4 *>(&tile[buf][s_row + ROWS * i][4 * s_c4]) = on ? stg[T][i] : make_float4(0.f, 0.f, 0.f, 0.f);
+  };
+
+  floatx16 acc0, acc1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc0[r] = acc1[r] = 0.0f;
+  const int a_row = wm * 32 + m, b_row = 64 + wn * 32 + m, k_lane = kh * (FDX_BK / 2) + 4 * h;
+  auto products = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < FDX_BK / 16; ++s) {
+      const float4 a = *reinterpret_cast<const float4 *>(&tile[buf][a_row][k_lane + 8 * s]);
+      const float4 b = *reinterpret_cast<const float4 *>(&tile[buf][b_row][k_lane + 8 * s]);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc1, 0, 0, 0);
+    }
+  };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+
+  // chunk c sits in tile[c % 2]; chunk c + 1 waits in registers (set (c + 1) % 2), chunk c + 2
+  // is asked for (fetches past the end read the last words again and are dropped)
+  fetch(0, Set0());
+  fetch(FDX_BK, Set1());
+  stage(0, 0, Set0());
+  __syncthreads();
+#pragma unroll 1
+  for (int k0 = 0; k0 < f.out; k0 += 2 * FDX_BK) {
+    fetch(k0 + 2 * FDX_BK, Set0());
+    products(0);
+    stage(k0 + FDX_BK, 1, Set1());
+    __syncthreads();
+    if (k0 + FDX_BK >= f.out) break;
+    fetch(k0 + 3 * FDX_BK, Set1());
+    products(1);
+    stage(k0 + 2 * FDX_BK, 0, Set0());
+    __syncthreads();
+  }
+
+  const int blk = wm + 2 * wn;
+  if (kh) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) halves[blk][r][lane] = acc0[r] + acc1[r];
+  }
+  __syncthreads();
+  if (kh) return;
+  // register r of lane l: sample b0 + 32*wm + 8*(r/4) + 4*(l/32) + r%4, input i0 + 32*wn + l%32
+  const int i = i0 + wn * 32 + m;
+  if (i >= f.in) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int b = b0 + wm * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+    if (b >= f.batch) continue;
+    const size_t idx = static_cast<size_t>(b) * f.in + i;
+    float v = (acc0[r] + acc1[r]) + halves[blk][r][lane];
+    if (f.ag.kind != TDH_ACT_NONE) v *= act_grad_factor(f.ag.kind, f.ag.y[idx]);
+    f.dx[idx] = v;
+  }
+}
+
+// the layer is large enough to give (nearly) every compute unit a workgroup of that kernel, and
+// its rows allow the 16-byte reads
+static bool fc_dx_tile_applies(int in, int out, int batch, const float *dy, const float *w) {
+  const long wgs = static_cast<long>(ceil_div(batch, 64)) * ceil_div(in, 64);
+  return out % 4 == 0 && out >= 256 && wgs >= 192 && wgs <= 4096 &&
+         static_cast<long>(std::max(batch, in)) * out < (1L << 30) &&
+         !(reinterpret_cast<uintptr_t>(dy) & 15) && !(reinterpret_cast<uintptr_t>(w) & 15);
+}
+
 int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float *w,
            const float *dy, float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
            const PoolScatter *pool, const FcGrads *also) {
@@ -1214,9 +1353,15 @@ int fc_bwd(int in, int out, int has_bias, int batch, const float *x, const float
     StridedOperand A{dy, out, 1, batch};  // dY[s][k]
     StridedOperand B{w, out, 1, in};      // W[n][k], k contiguous
     EpiRowMajor epi{dx, in, nullptr, dx_act, 0};
-    if (small_fc_applies(batch, in, out))
+    if (small_fc_applies(batch, in, out)) {
       TDH_TRY(launch_small_fc(A, B, epi, batch, in, out, "fc_dx_small"));
-    else
+    } else if (fc_dx_tile_applies(in, out, batch, dy, w)) {
+      ProfScope prof("fc_dx_tile", batch, in, out);
+      FcDxTile f{dy, w, dx, dx_act, batch, in, out, ceil_div(batch, 64), ceil_div(in, 64), 0};
+      f.n_per_xcd = ceil_div(f.tiles_n, 8);
+      TDH_LAUNCH(fc_dx_tile_kernel, dim3(8 * f.n_per_xcd * f.tiles_m), dim3(512), 0, ctx().stream, f);
+      TDH_LAUNCH_CHECK();
+    } else
       TDH_TRY((launch_gemm<true, true, false, false>(A, B, epi, batch, in, out, true, "fc_dx_gemm",
                                                  "fc_dx_splitk_reduce")));
   }
