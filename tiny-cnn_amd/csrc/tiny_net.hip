@@ -479,7 +479,7 @@ __host__ __device__ inline int scalar_block(const int channels) {
   return channels == 1 ? 1 : ((channels % 3 == 0 && (channels & 3) != 0) ? 3 : 4);
 }
 
-template <int R, int S, bool PAD, int NB>
+template <int R, int S, bool PAD, int NB, bool TBL>
 TN_INLINE void conv_fwd_scalar(const TinyLayer *__restrict__ Lp, const float *in, float *out, float *__restrict__ gout,
                                float *scratch) {
   const int C = Lp->C, H = Lp->H, W = Lp->W, K = Lp->K, OH = Lp->OH, OW = Lp->OW;
@@ -536,7 +536,7 @@ TN_INLINE void conv_fwd_scalar(const TinyLayer *__restrict__ Lp, const float *in
       }
 #pragma unroll
       for (int q = 0; q < NB; ++q)
-        if (!tbl || tbl[ci * K + cob[q]]) acc[q] += sum[q];
+        if (!TBL || tbl[ci * K + cob[q]]) acc[q] += sum[q];
     }
     if (parts > 1) {
       if (active && cp > 0) {
@@ -565,14 +565,22 @@ TN_INLINE void conv_fwd_scalar(const TinyLayer *__restrict__ Lp, const float *in
 template <int R, int S, bool PAD>
 TN_INLINE void conv_fwd_scalar_any(const TinyLayer *__restrict__ Lp, const float *in, float *out,
                                    float *__restrict__ gout, float *scratch) {
-  if (scalar_block(Lp->K) == 3) conv_fwd_scalar<R, S, PAD, 3>(Lp, in, out, gout, scratch);
-  else conv_fwd_scalar<R, S, PAD, 4>(Lp, in, out, gout, scratch);
+  // (a connection table makes every channel sum conditional: a version of its own, so that the
+  // loops of a net without one stay free of branches)
+  const bool tbl = Lp->tbl != nullptr;
+  if (scalar_block(Lp->K) == 3) {
+    if (tbl) conv_fwd_scalar<R, S, PAD, 3, true>(Lp, in, out, gout, scratch);
+    else conv_fwd_scalar<R, S, PAD, 3, false>(Lp, in, out, gout, scratch);
+  } else {
+    if (tbl) conv_fwd_scalar<R, S, PAD, 4, true>(Lp, in, out, gout, scratch);
+    else conv_fwd_scalar<R, S, PAD, 4, false>(Lp, in, out, gout, scratch);
+  }
 }
 
 // dX from the zero-framed dY (stage_framed_dy); the waves of a workgroup of NT threads take the
 // items [item0, item1) of items * parts in turn (item = part * items + block * chunks + chunk);
 // dx (LDS) may be NULL
-template <int R, int S, int NB, int NT>
+template <int R, int S, int NB, int NT, bool TBL>
 TN_INLINE void conv_bwd_dx_scalar(const TinyLayer *__restrict__ Lp, const float *framed, float *dx,
                                   float *__restrict__ gdx, float *scratch, const int item0, const int item1,
                                   const int parts) {
@@ -621,7 +629,7 @@ TN_INLINE void conv_bwd_dx_scalar(const TinyLayer *__restrict__ Lp, const float 
       }
 #pragma unroll
       for (int q = 0; q < NB; ++q)
-        if (!tbl || tbl[cib[q] * K + co]) acc[q] += sum[q];
+        if (!TBL || tbl[cib[q] * K + co]) acc[q] += sum[q];
     }
     if (parts > 1) {
       if (active && kp > 0) {
@@ -656,9 +664,15 @@ TN_INLINE void conv_bwd_dx_scalar_any(const TinyLayer *__restrict__ Lp, const fl
                                       float *__restrict__ gdx, float *scratch, const int item0, const int item1,
                                       const int parts) {
   const int nb = scalar_block(Lp->C);
-  if (nb == 1) conv_bwd_dx_scalar<R, S, 1, NT>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
-  else if (nb == 3) conv_bwd_dx_scalar<R, S, 3, NT>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
-  else conv_bwd_dx_scalar<R, S, 4, NT>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+  if (Lp->tbl) {
+    if (nb == 1) conv_bwd_dx_scalar<R, S, 1, NT, true>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+    else if (nb == 3) conv_bwd_dx_scalar<R, S, 3, NT, true>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+    else conv_bwd_dx_scalar<R, S, 4, NT, true>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+  } else {
+    if (nb == 1) conv_bwd_dx_scalar<R, S, 1, NT, false>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+    else if (nb == 3) conv_bwd_dx_scalar<R, S, 3, NT, false>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+    else conv_bwd_dx_scalar<R, S, 4, NT, false>(Lp, framed, dx, gdx, scratch, item0, item1, parts);
+  }
 }
 
 // A convolution whose window is the whole input (one output pixel per channel, no padding) is a
@@ -674,50 +688,45 @@ inline bool conv_dx_shape_is_framed(const TinyLayer &L) {
   return !conv_is_matvec(L) && L.sh == 1 && L.sw == 1 &&
          ((L.R == 5 && L.S == 5) || (L.R == 3 && L.S == 3));
 }
-// the same with 16-byte reads: no connection table, n_k a multiple of four, `in` 16-byte aligned
+// the same with 16-byte reads: no connection table, n_k a multiple of four, `in` 16-byte aligned.
+// A group of lanes per output channel, as many as keep the whole workgroup busy in one round;
+// the lanes of a group read neighbouring 16-byte pieces of the filter row, eight in flight each.
 TN_INLINE void conv_fwd_matvec4(const TinyLayer *__restrict__ Lp, const float *in, float *out, float *__restrict__ gout) {
   const int K = Lp->K, has_bias = Lp->has_bias;
   const float *__restrict__ b = Lp->b;
-  const int n_k4 = (Lp->C * Lp->R * Lp->S) >> 2, lane = threadIdx.x & 63;
+  const int n_k4 = (Lp->C * Lp->R * Lp->S) >> 2;
   const float4 *__restrict__ w4 = reinterpret_cast<const float4 *>(Lp->w);
   const float4 *in4 = reinterpret_cast<const float4 *>(in);
-  constexpr int ROWS = 8, PER = 2;   // filter rows per wave and round, 16-byte pieces of each per lane and trip
-  for (int co0 = wave_index(); co0 < K; co0 += ROWS * TN_WAVES) {
-    float s[ROWS];
+  int g = 64;
+  while (g > 1 && (K * g > TN_THREADS || 4 * g > n_k4)) g >>= 1;
+  const int gs = __ffs(g) - 1, total = K * g;
+  for (int base = 0; base < total; base += TN_THREADS) {
+    const int it = base + threadIdx.x, part = it & (g - 1);
+    const bool on = it < total;
+    const int co = on ? it >> gs : 0;
+    const float4 *wr = w4 + static_cast<size_t>(co) * n_k4;
+    float sum = 0.0f;
+    for (int k0 = 0; k0 < n_k4; k0 += 8 * g) {
+      float4 a[8];
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) s[r] = 0.0f;
-    for (int k0 = 0; k0 < n_k4; k0 += 64 * PER) {
-      float4 a[ROWS][PER];
-#pragma unroll
-      for (int r = 0; r < ROWS; ++r) {
-        const int co = co0 + r * TN_WAVES;
-        const float4 *wr = w4 + static_cast<size_t>(co < K ? co : co0) * n_k4;
-#pragma unroll
-        for (int j = 0; j < PER; ++j) {
-          const int k = k0 + 64 * j + lane;
-          a[r][j] = wr[k < n_k4 ? k : 0];
-        }
+      for (int j = 0; j < 8; ++j) {
+        const int k = k0 + g * j + part;
+        a[j] = wr[k < n_k4 ? k : 0];
       }
 #pragma unroll
-      for (int j = 0; j < PER; ++j) {
-        const int k = k0 + 64 * j + lane;
+      for (int j = 0; j < 8; ++j) {
+        const int k = k0 + g * j + part;
         if (k < n_k4) {
           const float4 xv = in4[k];
-#pragma unroll
-          for (int r = 0; r < ROWS; ++r)
-            s[r] += (a[r][j].x * xv.x + a[r][j].y * xv.y) + (a[r][j].z * xv.z + a[r][j].w * xv.w);
+          sum += (a[j].x * xv.x + a[j].y * xv.y) + (a[j].z * xv.z + a[j].w * xv.w);
         }
       }
     }
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int co = co0 + r * TN_WAVES;
-      const float sum = group_sum(s[r], 64);
-      if (lane == 0 && co < K) {
-        const float v = has_bias ? sum + b[co] : sum;
-        out[co]  = v;
-        gout[co] = v;
-      }
+    sum = group_sum(sum, g);
+    if (on && part == 0) {
+      const float v = has_bias ? sum + b[co] : sum;
+      out[co]  = v;
+      gout[co] = v;
     }
   }
 }
