@@ -313,6 +313,9 @@ def main():
     ap.add_argument("--others", action="store_true", help="(default) also run the other workloads")
     ap.add_argument("--no-others", action="store_true", help="only the named workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-host-inputs", action="store_true",
+                    help="leave out the leg that hands over host batches every step (profiler runs: rocprofv3 "
+                         "7.2 dies in that leg of the VGG workload, in a host copy below hipGraphInstantiate)")
     ap.add_argument("--sequence-out", default=None,
                     help="write the kernel tags of one step in dispatch order to this JSON file "
                          "(tiny-cnn_amd.profsum reads a rocprofv3 trace of the same run tag by tag with it)")
@@ -356,7 +359,7 @@ def main():
         out["mfma_kernels_together"] = {"TFLOP/s": round(tot_flop / tot_s / 1e12, 2),
                                         "frac": round(tot_flop / tot_s / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
     out["copy_yardstick"] = copy_yardstick(T)
-    if hasattr(wl, "step_from_host"):  # never `value`: reported for callers that own host buffers
+    if hasattr(wl, "step_from_host") and not args.no_host_inputs:  # never `value`: reported for callers that own host buffers
         for _ in range(12):  # every device slot gets its captured steps (three slots, two Adam buffers)
             wl.step_from_host()
         T.sync()

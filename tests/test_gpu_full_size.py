@@ -83,14 +83,14 @@ def test_large_fc_weight_gradient_from_memory_fragments(T, bs, ni, no):
 
 
 @pytest.mark.parametrize("bs,ni,no", [
-    (250, 3100, 1000),   # ragged in both directions, halves of the outputs that are no whole group, idle tiles
-    (256, 4096, 264),    # the smallest reduction the kernel takes: one group and a tail per half
-    (200, 4160, 2048),   # whole groups; a last column tile of its own
+    (250, 3100, 1100),   # ragged in both directions, a last chunk of 76 outputs, idle workgroups at the grid's end
+    (256, 4096, 1028),   # nearly the shortest reduction the kernel takes, a last chunk of one 16-byte word
+    (200, 4160, 2048),   # whole chunks; a last column tile of its own
 ])
-def test_large_fc_input_gradient_from_memory_fragments(T, bs, ni, no):
-    """dX of a fully-connected layer with a tile for (nearly) every compute unit runs on a kernel
-    that feeds the matrix cores from memory (no LDS, no split reduction): against float64, twice
-    with equal bits, and linear in dY bit for bit."""
+def test_large_fc_input_gradient_from_untransposed_tiles(T, bs, ni, no):
+    """dX of a fully-connected layer with a 64 x 64 tile for (nearly) every compute unit and a
+    long reduction runs on a kernel of its own (operands staged untransposed, no split reduction):
+    against float64, twice with equal bits, and linear in dY bit for bit."""
     rng = np.random.default_rng(bs + ni + no)
     x = rng.uniform(-1, 1, (bs, ni)).astype(np.float32)
     w = rng.uniform(-0.05, 0.05, ni * no).astype(np.float32)

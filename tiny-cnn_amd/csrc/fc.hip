@@ -1254,11 +1254,13 @@ fc_dx_tile_kernel(const FcDxTile f) {
   }
 }
 
-// the layer is large enough to give (nearly) every compute unit a workgroup of that kernel, and
-// its rows allow the 16-byte reads
+// the layer is large enough to give (nearly) every compute unit a workgroup of that kernel, its
+// reduction long enough for the kernel's two-chunk prologue to be a small part of it (the VGG
+// classifier, 131072 -> 256, has two chunks in all and stays with the general kernel), and its
+// rows allow the 16-byte reads
 static bool fc_dx_tile_applies(int in, int out, int batch, const float *dy, const float *w) {
   const long wgs = static_cast<long>(ceil_div(batch, 64)) * ceil_div(in, 64);
-  return out % 4 == 0 && out >= 256 && wgs >= 192 && wgs <= 4096 &&
+  return out % 4 == 0 && out >= 8 * FDX_BK && wgs >= 192 && wgs <= 4096 &&
          static_cast<long>(std::max(batch, in)) * out < (1L << 30) &&
          !(reinterpret_cast<uintptr_t>(dy) & 15) && !(reinterpret_cast<uintptr_t>(w) & 15);
 }
