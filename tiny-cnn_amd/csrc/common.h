@@ -120,6 +120,15 @@ void prof_launch_events(hipEvent_t *start, hipEvent_t *stop);  // nulls outside 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline size_t ceil_div_sz(size_t a, size_t b) { return (a + b - 1) / b; }
 
+// Workgroups are handed to the eight XCDs (each with its own L2) round-robin in launch order.
+// This renumbers a workgroup's linear id so that ids that are neighbours after the renumbering,
+// which is how the kernels below give neighbouring pieces of one image to their workgroups, run
+// on the same XCD and find each other's overlapping rows in its L2.
+__device__ __forceinline__ int xcd_compact_id(const int id, const int total) {
+  const int per = total >> 3;
+  return id < (per << 3) ? (id & 7) * per + (id >> 3) : id;
+}
+
 // Division by a runtime constant as multiply-high + shift. Exact for 0 <= n < 2^31.
 struct FastDiv {
   uint32_t d = 1, mul = 1, shift = 0;

@@ -253,8 +253,9 @@ conv_dx_small_cin_kernel(const float *__restrict__ dy, const float *__restrict__
   extern __shared__ __align__(16) float smem[];
   const int R = KR ? KR : g.R, S = KS ? KS : g.S;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int img = blockIdx.x / p.bands;
-  const int y0  = (blockIdx.x - img * p.bands) * p.tile_rows;
+  const int wg  = xcd_compact_id(blockIdx.x, gridDim.x);  // (an image's bands share rows: one XCD)
+  const int img = wg / p.bands;
+  const int y0  = (wg - img * p.bands) * p.tile_rows;
   const int tsz = p.trows * p.tcols, rs = R * S;
   const int oy0 = y0 + g.pad_h - (R - 1), ox0 = g.pad_w - (S - 1);
   const int ohw = g.OH * g.OW;
@@ -525,8 +526,9 @@ conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict_
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int mr = lane & 15, mq = lane >> 4;
   const int bands = (g.H + G::TILE_ROWS - 1) / G::TILE_ROWS;
-  const int img = blockIdx.x / bands;
-  const int y0  = (blockIdx.x - img * bands) * G::TILE_ROWS;
+  const int wg  = xcd_compact_id(blockIdx.x, gridDim.x);  // (an image's bands share rows: one XCD)
+  const int img = wg / bands;
+  const int y0  = (wg - img * bands) * G::TILE_ROWS;
   const int oy0 = y0 + g.pad_h - (KR - 1), ox0 = g.pad_w - (KS - 1);
   const int ohw = g.OH * OW, pohw = (g.OH >> 1) * (OW / 2);
   float *wl = smem + DXM_MCH * PLANE;  // the chunk's filters [co][ci (4)][tap]

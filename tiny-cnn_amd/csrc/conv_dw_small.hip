@@ -58,7 +58,10 @@ __global__ void __launch_bounds__(256, 2) conv_dw_small_kernel(const DwSmallArgs
   float *xs  = lds;
   float *dys = lds + a.x_floats;  // two chunk buffers; later the accumulators of the four waves
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bandi = blockIdx.x, img = blockIdx.y, co0 = blockIdx.z * 32;
+  // (an image's bands share rows: they go to one XCD)
+  const int wg = xcd_compact_id(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z),
+                                gridDim.x * gridDim.y * gridDim.z);
+  const int bandi = wg % gridDim.x, img = (wg / gridDim.x) % gridDim.y, co0 = (wg / (gridDim.x * gridDim.y)) * 32;
   const int oy0   = bandi * a.band;
   const int rows_here = min(a.band, a.OH - oy0);
   const int nchunks   = (rows_here + a.chunk - 1) / a.chunk;

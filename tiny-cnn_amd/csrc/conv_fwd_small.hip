@@ -159,7 +159,10 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_kernel(const FwdSmallAr
   float *bs = ws + 32 * a.crs;   // [32] bias, zero past Cout or without bias
   int *offs = reinterpret_cast<int *>(bs + 32);  // [2*NS] patch offset of k (0 past K)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bandi = blockIdx.x, img = blockIdx.y, co0 = blockIdx.z * 32;
+  // (an image's bands share rows: they go to one XCD)
+  const int wg = xcd_compact_id(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z),
+                                gridDim.x * gridDim.y * gridDim.z);
+  const int bandi = wg % gridDim.x, img = (wg / gridDim.x) % gridDim.y, co0 = (wg / (gridDim.x * gridDim.y)) * 32;
   const int oy0 = bandi * a.band;
   const int nthr = blockDim.x;  // one wave per tile of the band, two to four waves
 
@@ -295,7 +298,10 @@ __global__ void __launch_bounds__(256, 2) conv_fwd_small_full_kernel(const FwdSm
   float *bs = ws + 32 * a.crs;
   int *offs = reinterpret_cast<int *>(bs + 32);
   const int tid = threadIdx.x, lane = tid & 63;
-  const int bandi = blockIdx.x, img = blockIdx.y, co0 = blockIdx.z * 32;
+  // (an image's bands share rows: they go to one XCD)
+  const int wg = xcd_compact_id(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z),
+                                gridDim.x * gridDim.y * gridDim.z);
+  const int bandi = wg % gridDim.x, img = (wg / gridDim.x) % gridDim.y, co0 = (wg / (gridDim.x * gridDim.y)) * 32;
   const int oy0 = bandi * a.band;
   const int nthr = blockDim.x;
   fwd_small_stage<NS>(a, xs, ws, bs, offs, img, co0, oy0, tid, nthr);
