@@ -170,3 +170,104 @@ def test_nets_that_do_not_qualify_ignore_the_flag(T, O, W):
             net.close()
         for a, b in zip(*got):
             assert np.array_equal(a, b)
+
+
+def _random_small_net(rng):
+    """A random net that the per-sample kernel takes: one to three convolutions (3x3 or 5x5, with
+    and without padding, 1 to 12 channels), pools that leave rows or columns uncovered, every
+    activation it knows, one or two fully-connected layers, each loss."""
+    def act():
+        a = str(rng.choice(["relu", "tanh", "sigmoid", "leaky_relu"]))
+        return ("act", a, (0.1, 0.0)) if a == "leaky_relu" else ("act", a)
+    w, h, c = int(rng.choice([6, 8, 10, 12, 14, 16])), int(rng.choice([6, 8, 10, 12, 13])), int(rng.choice([1, 2, 3, 6]))
+    spec = []
+    for _ in range(int(rng.integers(1, 4))):
+        k, oc, same = int(rng.choice([3, 5])), int(rng.choice([1, 3, 4, 5, 6, 8, 12])), bool(rng.integers(0, 2))
+        same = same or w < k or h < k
+        spec.append(("conv", w, h, c, k, oc, same))
+        if not same:
+            w, h = w - k + 1, h - k + 1
+        c = oc
+        order = int(rng.integers(0, 4))
+        if order in (1, 3):
+            spec.append(act())
+        if w >= 4 and h >= 4 and rng.random() < 0.7:
+            if rng.random() < 0.5:
+                spec.append(("maxpool", w, h, c, 2))
+                w, h = w // 2, h // 2
+            elif w % 2 == 0 and h % 2 == 0:
+                spec.append(("avepool", w, h, c, 2))
+                w, h = w // 2, h // 2
+            if order in (2, 3):
+                spec.append(act())
+    if rng.random() < 0.6:
+        hid = int(rng.choice([7, 10, 24]))
+        spec += [("fc", c * w * h, hid), act(), ("fc", hid, 10)]
+    else:
+        spec.append(("fc", c * w * h, 10))
+    r = rng.random()
+    if r < 0.4:
+        return spec + [("act", "softmax")], "ce_multiclass"
+    if r < 0.6:
+        return spec + [("act", "sigmoid")], "ce"
+    return spec, "mse"
+
+
+def test_random_small_nets_match_oracle(T, O, W):
+    """A seeded sweep: every layer output, input gradient, weight and bias gradient of one
+    backward pass, then the weights after three steps, eager or replayed."""
+    rng = np.random.default_rng(20)
+    for case in range(40):
+        spec, loss = _random_small_net(rng)
+        batch = int(rng.choice([1, 3, 5, 16, 33]))
+        flags = int(rng.choice([SAMPLE | FUSE, SAMPLE | FUSE | GRAPH]))
+        tag = f"case {case} (batch {batch}, flags {flags}, {loss}, {spec})"
+        params = []
+        for i, l in enumerate(spec):
+            nw, nb, fan_in, _ = W.layer_fans(l)
+            if nw:
+                wv = rng.uniform(-1, 1, nw).astype(np.float32) * np.float32(np.sqrt(3.0 / fan_in))
+                if l[0] == "avepool":
+                    wv = rng.uniform(0.5, 1.5, nw).astype(np.float32)
+                params += [(i, 0, wv), (i, 1, rng.uniform(-0.2, 0.2, nb).astype(np.float32))]
+        first = spec[0]
+        x = rng.standard_normal((batch, first[1] * first[2] * first[3])).astype(np.float32)
+        t = (np.eye(10, dtype=np.float32)[rng.integers(0, 10, batch)] if loss == "ce_multiclass"
+             else rng.uniform(0.1, 0.9, (batch, 10)).astype(np.float32))
+        xd, td = T.to_device(x), T.to_device(t)
+        kind = str(rng.choice(["momentum", "sgd"]))
+
+        def pair():
+            net, ref = T.Net(W.build_layers(T, spec), batch, flags), O.OracleNet(W.build_layers(O, spec), batch)
+            for (i, which, a) in params:
+                net.set_param(i, which, a)
+                (ref.weight(i) if which == 0 else ref.bias(i))[:] = a
+            return net, ref
+        net, ref = pair()
+        net.train_step(None, loss, batch, xd, td, do_update=False)
+        ref.train_step(O.opt_desc(kind), loss, x, t, do_update=False)
+        for i, l in enumerate(spec):
+            assert net.out_written(i) and net.dx_written(i), f"{tag}: the per-sample kernel did not run"
+            assert_close(net.layer_out(i, batch), ref.layer_out(i, batch), what=f"{tag} layer {i} output")
+            assert_close(net.layer_dx(i, batch), ref.layer_dx(i, batch), what=f"{tag} layer {i} dX")
+            if l[0] == "maxpool":
+                got, want = net.layer_argmax(i, batch).astype(np.int64), ref.layer_argmax(i, batch)
+                if not np.array_equal(got, want):   # (another winner only where both hold the same value to rounding)
+                    pin, rows = ref.layer_out(i - 1, batch), np.arange(batch)[:, None]
+                    tol = 1e-5 * np.maximum(np.abs(pin[rows, want]), np.sqrt(np.mean(pin * pin)))
+                    assert np.all(np.abs(pin[rows, got] - pin[rows, want]) <= tol), f"{tag} layer {i} argmax"
+            if W.layer_fans(l)[0]:
+                assert_close(net.layer_grad(i, 0), ref.layer_dw(i), what=f"{tag} layer {i} dW")
+                assert_close(net.layer_grad(i, 1), ref.layer_db(i), what=f"{tag} layer {i} db")
+        net.close()
+        net, ref = pair()
+        # (a rate at which three steps on summed gradients stay finite for every loss)
+        opt, ropt = T.opt_desc(kind, alpha=1e-3), O.opt_desc(kind, alpha=1e-3)
+        for _ in range(3):
+            net.train_step(opt, loss, batch, xd, td)
+            ref.train_step(ropt, loss, x, t)
+        for (i, which, _) in params:
+            want = ref.weight(i) if which == 0 else ref.bias(i)
+            assert np.isfinite(want).all(), f"{tag}: the oracle's step diverged"
+            assert_close(net.get_param(i, which), want, 2e-4, what=f"{tag} parameter {i}.{which} after three steps")
+        net.close()
