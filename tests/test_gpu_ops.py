@@ -38,6 +38,9 @@ CONV = [
     (12, 12, 48, 5, 16, True, 1, 5), (40, 6, 16, 3, 16, False, 1, 1),
     # 5x5 windows split by filter row: stacked small images with a ragged last chunk, row chunks
     (10, 10, 16, 5, 40, True, 1, 7), (36, 36, 16, 5, 16, False, 1, 2), (8, 8, 32, 5, 64, True, 1, 11),
+    # 5x5 windows on 8x8 images, all filter rows in one workgroup (four tap groups, four images a
+    # chunk): a last chunk of two images, several channel blocks either way, several chunks a slice
+    (8, 8, 64, 5, 96, True, 1, 6), (8, 8, 64, 5, 96, True, 1, 130), (8, 8, 32, 5, 32, True, 1, 4),
     # stride-1 MFMA kernel with scalar loads: rows or channel counts that are not multiples of 4,
     # a last chunk of reduction channels that is not full
     (26, 26, 16, 3, 32, True, 1, 32), (14, 14, 16, 5, 32, True, 1, 64), (16, 16, 16, 3, 30, True, 1, 64),
@@ -150,6 +153,40 @@ def test_conv_accumulate_and_skipped_outputs(T, O):
     dwb = T.DevBuf((135,))
     T.conv2d_bwd(d, 3, xd, wd, dyd, None, dwb, None)
     assert_close(dwb.numpy(), rdw)
+
+
+def test_conv_weight_gradient_of_8x8_images_options(T, O):
+    """The 8x8-image dW kernel: added to a previous value, without a bias gradient, without dX,
+    twice with equal bits; tensors that are not 16-byte aligned take the general kernel."""
+    rng = np.random.default_rng(88)
+    bs, ic, oc = 9, 32, 64
+    d, do = T.conv_desc(8, 8, ic, 5, 5, oc, pad_same=True), O.conv_desc(8, 8, ic, 5, 5, oc, pad_same=True)
+    x = rng.standard_normal((bs, ic * 64)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, oc * ic * 25).astype(np.float32)
+    dy = rng.standard_normal((bs, oc * 64)).astype(np.float32)
+    dw0 = rng.standard_normal(w.size).astype(np.float32)
+    rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
+    xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+    dw, db = T.to_device(dw0), T.DevBuf((oc,), zero=True)
+    T.conv2d_bwd(d, bs, xd, wd, dyd, None, dw, db, True)
+    assert_close(dw.numpy(), rdw + dw0, what="dw added to a previous value")
+    assert_close(db.numpy(), rdb, what="db")
+    first = T.DevBuf(w.shape)
+    T.conv2d_bwd(d, bs, xd, wd, dyd, None, first, None)
+    assert_close(first.numpy(), rdw, what="dw alone")
+    again = T.to_device(np.full(w.shape, np.nan, np.float32))
+    T.conv2d_bwd(d, bs, xd, wd, dyd, None, again, None)
+    assert np.array_equal(first.numpy(), again.numpy())
+    # the same tensors one float further on in memory
+    xs, dys = T.DevBuf((x.size + 4,)), T.DevBuf((dy.size + 4,))
+    xs.upload(np.concatenate([np.zeros(1, np.float32), x.ravel(), np.zeros(3, np.float32)]))
+    dys.upload(np.concatenate([np.zeros(1, np.float32), dy.ravel(), np.zeros(3, np.float32)]))
+    xo = T.DevBuf.view(xs.ptr.value + 4, x.shape)
+    dyo = T.DevBuf.view(dys.ptr.value + 4, dy.shape)
+    shifted, dbs = T.DevBuf(w.shape), T.DevBuf((oc,))
+    T.conv2d_bwd(d, bs, xo, wd, dyo, None, shifted, dbs)
+    assert_close(shifted.numpy(), rdw, what="dw of unaligned tensors")
+    assert_close(dbs.numpy(), rdb, what="db of unaligned tensors")
 
 
 def test_conv_errors_and_empty_batch(T):

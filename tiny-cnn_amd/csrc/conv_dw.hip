@@ -370,8 +370,198 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
   }
 }
 
+
+// ---- 5x5 windows (padding 2, stride 1) on 8x8 images: every filter row in one workgroup
+//
+// The kernel above gives such a layer workgroups of (one filter row) x (two chunks of images):
+// 1280 wave-sized pieces of 160 MFMAs for 1024 SIMDs, so some SIMD runs two whatever the split,
+// five workgroups stage the same tiles, and a wave's slice leaves as 80 scattered 4-byte stores.
+// Here a workgroup owns 32 output channels x 32 input channels x one of FOUR GROUPS OF TAPS
+// (7 + 6 + 6 + 6 of the 25, each group lies in two filter rows) for a run of chunks of four
+// images; its four waves take one image each, so a wave's piece is 224 (or 192) MFMAs and a
+// 32 -> 64-channel layer at batch 128 is 256 workgroups of one chunk: every SIMD gets one wave.
+// An image is staged whole with its zero frame (12 x 12 per channel), so the X fragment of
+// output row oy and filter row fy is two 16-byte reads, eight floats, that serve all five taps
+// of the row; a dY fragment (one 16-byte read per output row) serves all taps of the group.
+// The pixel pairing is the one of the kernel above: k = 0 lanes take the left half of a row,
+// k = 1 lanes the right half. The four waves' sums meet in LDS (pairwise, image order), and the
+// whole workgroup stores the slice. The bias gradient comes from the workgroups of tap group 0
+// and input-channel block 0, out of the dY they stage anyway.
+constexpr int I8_NT  = 256;
+constexpr int I8_DYP = 4 * 64 + 4;    // floats per staged dY channel: four images (4 mod 64)
+constexpr int I8_XP  = 4 * 144 + 4;   // floats per staged X channel: four framed images (4 mod 64)
+constexpr int I8_LDS_FLOATS = 32 * I8_DYP + 32 * I8_XP;
+
+struct DwImg8Args {
+  const float *x, *dy;
+  float *partial;      // [slices][Kc][C*25]
+  float *partial_db;   // [slices][Kc], or null
+  int batch, C, Kc;
+  int chunks_total, chunks_per_slice;   // chunks of four images
+  int co_blocks, ci_blocks;
+};
+
+// tap group G: taps T0 .. T0+N-1 of the 25 (tap = 5*fy + fx)
+template <int G> struct I8Taps {
+  static constexpr int T0 = G == 0 ? 0 : G == 1 ? 7 : G == 2 ? 13 : 19;
+  static constexpr int N  = G == 0 ? 7 : 6;
+  static constexpr int FY0 = T0 / 5, FY1 = (T0 + N - 1) / 5;
+};
+
+// the products of one image (the wave's) for tap group G: acc[t - T0] += dY x X shifted by tap t
+template <int G>
+__device__ __forceinline__ void img8_products(const float *ap, const float *bp, floatx16 (&acc)[7]) {
+  using TG = I8Taps<G>;
+#pragma unroll
+  for (int oy = 0; oy < 8; ++oy) {
+    const floatx4 a4 = *reinterpret_cast<const floatx4 *>(ap + oy * 8);
+    const float av[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+    for (int fy = TG::FY0; fy <= TG::FY1; ++fy) {
+      const floatx4 b0 = *reinterpret_cast<const floatx4 *>(bp + (oy + fy) * 12);
+      const floatx4 b1 = *reinterpret_cast<const floatx4 *>(bp + (oy + fy) * 12 + 4);
+      const float bv[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int fx = 0; fx < 5; ++fx) {
+        const int t = 5 * fy + fx - TG::T0;
+        if (t < 0 || t >= TG::N) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[j + fx], acc[t], 0, 0, 0);
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(I8_NT, 1) conv_dw_img8_kernel(const DwImg8Args a) {
+  extern __shared__ __align__(16) float smem[];
+  float *dy_l = smem;                 // [32][I8_DYP]
+  float *x_l  = smem + 32 * I8_DYP;   // [32][I8_XP], frames of zeros around the images
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // workgroups that read the same tiles (the four tap groups and the output-channel blocks of a
+  // slice) are neighbours after the renumbering, and so share an XCD's L2
+  int id = xcd_compact_id(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
+  const int grp = id & 3;
+  id >>= 2;
+  const int cob = id % a.co_blocks;
+  id /= a.co_blocks;
+  const int cib = id % a.ci_blocks, slice = id / a.ci_blocks;
+  const int co0 = cob * 32, ci0 = cib * 32;
+  const int kohw = a.Kc * 64, chw = a.C * 64;
+
+  floatx16 acc[7];
+#pragma unroll
+  for (int t = 0; t < 7; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.0f;
+  const bool sums_dy = a.partial_db != nullptr && grp == 0 && cib == 0;
+  float dbs = 0.0f;   // this thread's share of the bias gradient of channel tid / 8
+
+  // fragment bases: A lane = (output channel l%32, half l/32), B lane = (input channel l%32, half)
+  const float *ap = dy_l + (lane & 31) * I8_DYP + wave * 64 + 4 * (lane >> 5);
+  const float *bp = x_l + (lane & 31) * I8_XP + wave * 144 + 4 * (lane >> 5);
+
+  const int c_begin = slice * a.chunks_per_slice;
+  const int c_end   = min(a.chunks_total, c_begin + a.chunks_per_slice);
+  for (int chunk = c_begin; chunk < c_end; ++chunk) {
+    // ---- stage four images: a thread moves eight 16-byte words of dY and eight of X, all
+    //      loads asked for before the first store (an image past the batch reads image 0 and is
+    //      stored as zeros)
+    floatx4 rdy[8], rx[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = tid + I8_NT * i, im = e >> 9, c = (e >> 4) & 31, q = e & 15;
+      const int img = chunk * 4 + im;
+      const size_t ig = img < a.batch ? img : 0;
+      rdy[i] = *reinterpret_cast<const floatx4 *>(a.dy + ig * kohw + static_cast<size_t>(co0 + c) * 64 + 4 * q);
+      rx[i]  = *reinterpret_cast<const floatx4 *>(a.x + ig * chw + static_cast<size_t>(ci0 + c) * 64 + 4 * q);
+    }
+    if (chunk == c_begin) {   // the frames of zeros, written while the first loads are on their way
+      for (int i = tid; i < 32 * I8_XP / 4; i += I8_NT) reinterpret_cast<floatx4 *>(x_l)[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();   // (the previous chunk's fragments have been read; the first time: the zeros are in place)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = tid + I8_NT * i, im = e >> 9, c = (e >> 4) & 31, q = e & 15;
+      const bool on = chunk * 4 + im < a.batch;
+      const floatx4 z = floatx4{0.f, 0.f, 0.f, 0.f};
+      *reinterpret_cast<floatx4 *>(dy_l + c * I8_DYP + im * 64 + 4 * q) = on ? rdy[i] : z;
+      // X row q/2, half q%2 -> framed row q/2 + 2, columns 2 + 4*(q%2) .. + 3 (8-byte aligned)
+      const floatx4 v = on ? rx[i] : z;
+      float *d = x_l + c * I8_XP + im * 144 + ((q >> 1) + 2) * 12 + 2 + 4 * (q & 1);
+      *reinterpret_cast<float2 *>(d)     = make_float2(v.x, v.y);
+      *reinterpret_cast<float2 *>(d + 2) = make_float2(v.z, v.w);
+    }
+    __syncthreads();
+    if (sums_dy) {   // channel tid/8, floats (tid%8)*32 .. +31 of its four images
+      const floatx4 *row = reinterpret_cast<const floatx4 *>(dy_l + (tid >> 3) * I8_DYP + (tid & 7) * 32);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const floatx4 v = row[k];
+        dbs += (v.x + v.y) + (v.z + v.w);
+      }
+    }
+    switch (grp) {
+      case 0: img8_products<0>(ap, bp, acc); break;
+      case 1: img8_products<1>(ap, bp, acc); break;
+      case 2: img8_products<2>(ap, bp, acc); break;
+      default: img8_products<3>(ap, bp, acc); break;
+    }
+  }
+
+  // ---- the four images' sums, pairwise in image order: (0 + 2) + (1 + 3). Waves 2 and 3 park
+  //      their sums, waves 0 and 1 add them to their own and park the two results transposed,
+  //      [output channel][input channel][tap] (rows of nine floats: no two lanes of a store share
+  //      a bank), and the whole workgroup adds those two and stores: a lane's neighbours then
+  //      write neighbouring taps and input channels, seven cache lines a store instead of 64.
+  float *red = smem;   // [2][7*16][64], then [2][32*32][9]
+  const int ntaps = grp == 0 ? 7 : 6, t0 = grp == 0 ? 0 : 1 + 6 * grp;
+  __syncthreads();
+  if (wave >= 2) {
+    float *dst = red + (wave - 2) * (7 * 16 * 64) + lane;
+#pragma unroll
+    for (int t = 0; t < 7; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst[(t * 16 + r) * 64] = acc[t][r];
+  }
+  __syncthreads();
+  if (wave < 2) {
+    const float *src = red + wave * (7 * 16 * 64) + lane;
+#pragma unroll
+    for (int t = 0; t < 7; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[t][r] += src[(t * 16 + r) * 64];
+  }
+  __syncthreads();
+  if (wave < 2) {
+    // reg r of lane l: output channel 8*(r/4) + 4*(l/32) + r%4, input channel l%32
+    float *dst = red + wave * (32 * 32 * 9) + (4 * (lane >> 5) * 32 + (lane & 31)) * 9;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+#pragma unroll
+      for (int t = 0; t < 7; ++t) dst[(8 * (r >> 2) + (r & 3)) * (32 * 9) + t] = acc[t][r];
+  }
+  __syncthreads();
+  const int crs = a.C * 25;
+  float *out = a.partial + (static_cast<size_t>(slice) * a.Kc + co0) * crs + ci0 * 25 + t0;
+  for (int e = tid; e < 32 * 32 * 8; e += I8_NT) {
+    const int t = e & 7, pair = e >> 3;   // pair = output channel * 32 + input channel
+    if (t < ntaps)
+      out[static_cast<size_t>(pair >> 5) * crs + (pair & 31) * 25 + t] = red[pair * 9 + t] + red[32 * 32 * 9 + pair * 9 + t];
+  }
+  if (sums_dy) {
+    // the eight shares of a channel sit in neighbouring lanes: added with a fixed butterfly
+    dbs += __shfl_xor(dbs, 1, 64);
+    dbs += __shfl_xor(dbs, 2, 64);
+    dbs += __shfl_xor(dbs, 4, 64);
+    if ((tid & 7) == 0) a.partial_db[static_cast<size_t>(slice) * a.Kc + co0 + (tid >> 3)] = dbs;
+  }
+}
+
 struct DwHaloPlan {
   bool ok;
+  bool img8;            // the 8x8-image kernel runs this shape
+  DwImg8Args i8;
   int tc, wco, wk, wfy, nt;
   int rows_block;  // filter rows one workgroup covers
   DwHaloArgs args;
@@ -386,12 +576,31 @@ int pad_to_4_mod_32(int v) {
 }
 
 DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, int OH, int OW, int ph,
-                        int pw) {
+                        int pw, bool allow_img8 = true) {
   DwHaloPlan p;
   p.ok = false;
   const bool five = R == 5 && S == 5;
   if (!(R == 3 && S == 3) && !five) return p;
   if (C < 16 || Kc < 16 || OW < 8 || OH < 2 || pw > 4) return p;
+  p.img8 = false;
+  if (allow_img8 && five && H == 8 && W == 8 && OH == 8 && OW == 8 && ph == 2 && pw == 2 && C % 32 == 0 && Kc % 32 == 0 && batch >= 4 &&
+      static_cast<long>(batch) * std::max(C, Kc) * 64 < (1L << 30)) {
+    DwImg8Args &i = p.i8;
+    i.batch = batch; i.C = C; i.Kc = Kc;
+    i.co_blocks = Kc / 32; i.ci_blocks = C / 32;
+    i.chunks_total = ceil_div(batch, 4);
+    // one workgroup per compute unit where the batch allows it
+    const int base = 4 * i.co_blocks * i.ci_blocks;
+    int slices = std::max(1, 256 / base);
+    slices = std::min(slices, i.chunks_total);
+    i.chunks_per_slice = ceil_div(i.chunks_total, slices);
+    p.slices = ceil_div(i.chunks_total, i.chunks_per_slice);
+    p.grid   = dim3(static_cast<unsigned>(p.slices));   // (grid.x counts the slices, as below; the launch multiplies)
+    p.lds_bytes = sizeof(float) * I8_LDS_FLOATS;
+    p.img8 = true;
+    p.ok   = true;
+    return p;
+  }
   p.tc = OW >= 48 ? 64 : OW >= 24 ? 32 : OW >= 12 ? 16 : 8;
   p.wfy = 1;
   // more than 32 output channels: two channel blocks share a workgroup's staged X patch (half
@@ -496,15 +705,19 @@ size_t conv_dw_halo_workspace_bytes(int R, int S, int batch, int C, int Kc, int 
                                     int OW, int ph, int pw) {
   const DwHaloPlan p = make_dw_plan(R, S, batch, C, Kc, H, W, OH, OW, ph, pw);
   if (!p.ok) return 0;
-  return ws_align(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc * C * R * S) +
-         ws_align(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc);
+  // (tensors that are not 16-byte aligned take the general kernel's plan where the 8x8-image
+  // kernel would run: room for whichever has more slices)
+  const DwHaloPlan q = p.img8 ? make_dw_plan(R, S, batch, C, Kc, H, W, OH, OW, ph, pw, false) : p;
+  const size_t slices = std::max(p.grid.x, q.ok ? q.grid.x : 0u);
+  return ws_align(sizeof(float) * slices * Kc * C * R * S) + ws_align(sizeof(float) * slices * Kc);
 }
 
 // dw (+)= sum over the batch; the caller has checked applicability and reserved the workspace
 int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, const float *dy,
                      float *dw, int H, int W, int OH, int OW, int ph, int pw, int accumulate,
                      float *db) {
-  DwHaloPlan p = make_dw_plan(R, S, batch, C, Kc, H, W, OH, OW, ph, pw);
+  const bool vec = W % 4 == 0 && OW % 4 == 0 && aligned16(x) && aligned16(dy);
+  DwHaloPlan p = make_dw_plan(R, S, batch, C, Kc, H, W, OH, OW, ph, pw, /*allow_img8=*/vec);
   if (!p.ok) return set_error(TDH_ERR_INVALID, "conv_dw_halo_run: shape not supported");
   const int crs = C * R * S;
   void *part = nullptr;
@@ -516,11 +729,24 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
     TDH_TRY(ws_take(sizeof(float) * static_cast<size_t>(p.grid.x) * Kc, &part_db));
     p.args.partial_db = static_cast<float *>(part_db);
   }
-  const bool vec = W % 4 == 0 && OW % 4 == 0 && aligned16(x) && aligned16(dy);
   {
     ProfScope prof(db ? "conv_dw_db_halo" : "conv_dw_halo", Kc, crs, batch * OH * OW);
-    if (vec) TDH_TRY(launch_dw_vec<true>(p));
-    else TDH_TRY(launch_dw_vec<false>(p));
+    if (p.img8) {
+      p.i8.x = x; p.i8.dy = dy; p.i8.partial = p.args.partial; p.i8.partial_db = p.args.partial_db;
+      static bool raised = false;
+      if (!raised) {
+        TDH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_dw_img8_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(p.lds_bytes)));
+        raised = true;
+      }
+      TDH_LAUNCH(conv_dw_img8_kernel, dim3(p.slices * p.i8.ci_blocks * p.i8.co_blocks * 4), dim3(I8_NT), p.lds_bytes,
+                 ctx().stream, p.i8);
+      TDH_LAUNCH_CHECK();
+    } else if (vec) {
+      TDH_TRY(launch_dw_vec<true>(p));
+    } else {
+      TDH_TRY(launch_dw_vec<false>(p));
+    }
   }
   const int slices = static_cast<int>(p.grid.x);
   EpiRowMajor epi{dw, crs, nullptr, ActGrad(), accumulate};
