@@ -282,7 +282,14 @@ enum {
    * tiny_dnn/node.h:89-103). Every layer output, input gradient and max-pool record is still
    * written to memory. Nets that do not qualify (size, batch normalization, dropout, a softmax
    * that is not the closing layer of a cross_entropy_multiclass net) ignore the flag. */
-  TDH_NET_SAMPLE_STEP   = 4
+  TDH_NET_SAMPLE_STEP   = 4,
+  /* Training never reads the gradient with respect to the net's input, which the reference
+   * computes like every other (layer::backward of the first layer fills the gradient of its
+   * data edge, tiny_dnn/layers/layer.h:557-575). With this flag a net whose first layer is a
+   * convolution or a fully-connected layer leaves that product out: tdh_net_layer_dx(net, 0)
+   * returns NULL after a step, everything else is what it is without the flag. Other first
+   * layers ignore the flag. */
+  TDH_NET_NO_INPUT_GRAD = 8
 };
 
 int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int flags,

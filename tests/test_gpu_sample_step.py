@@ -30,8 +30,8 @@ NETS = {
 }
 
 
-def build(T, O, W, name, batch, flags, seed=3):
-    spec = NETS[name]
+def build(T, O, W, name, batch, flags, seed=3, nets=None):
+    spec = (nets or NETS)[name]
     if spec[0] == "workload":
         spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(spec[1], batch=batch)
     else:
@@ -42,7 +42,7 @@ def build(T, O, W, name, batch, flags, seed=3):
         params = [(i, which, a if which == 0 else rng.uniform(-0.1, 0.1, a.size).astype(np.float32))
                   for (i, which, a) in params]
         first = spec[0]
-        n_in = first[1] * first[2] * first[3] if first[0] == "conv" else first[1]
+        n_in = first[1] * first[2] * first[3] if first[0] in ("conv", "maxpool", "avepool") else first[1]
         n_out = [l for l in spec if l[0] == "fc"][-1][2]
         x = rng.standard_normal((batch, n_in)).astype(np.float32)
         if loss == "ce":
@@ -270,4 +270,64 @@ def test_random_small_nets_match_oracle(T, O, W):
             want = ref.weight(i) if which == 0 else ref.bias(i)
             assert np.isfinite(want).all(), f"{tag}: the oracle's step diverged"
             assert_close(net.get_param(i, which), want, 2e-4, what=f"{tag} parameter {i}.{which} after three steps")
+        net.close()
+
+
+NO_INPUT_GRAD = 8
+INPUT_GRAD_NETS = dict(NETS, cifar10=("workload", "cifar10_cnn_b128"),
+                       fc_first_large=([("fc", 300, 200), ("act", "relu"), ("fc", 200, 10), ("act", "softmax")],
+                                       "ce_multiclass", "adam"),
+                       valid_conv_first=([("conv", 13, 13, 2, 3, 5, False), ("act", "tanh"), ("fc", 5 * 121, 4)],
+                                         "mse", "sgd"))
+
+
+@pytest.mark.parametrize("flags", [0, FUSE, FUSE | GRAPH, SAMPLE | FUSE, SAMPLE | FUSE | GRAPH])
+@pytest.mark.parametrize("name", list(INPUT_GRAD_NETS))
+def test_step_without_the_input_gradient_changes_nothing_else(T, O, W, name, flags):
+    """TDH_NET_NO_INPUT_GRAD leaves out the first layer's input gradient (layer.h:557-575 computes
+    it, training never reads it): that gradient is reported as not written, every other tensor
+    of a pass and the weights after three updates are bit for bit those of the net without the flag."""
+    batch = 16
+    spec, params, x, t, batch, loss, opt_kind, opt_kw, full, ref = build(T, O, W, name, batch, flags, nets=INPUT_GRAD_NETS)
+    *_, lean, _ = build(T, O, W, name, batch, flags | NO_INPUT_GRAD, nets=INPUT_GRAD_NETS)
+    xd, td = T.to_device(x), T.to_device(t)
+    for m in (full, lean):
+        m.train_step(None, loss, batch, xd, td, do_update=False)
+    ref.train_step(O.opt_desc(opt_kind), loss, x, t, do_update=False)
+    assert full.dx_written(0) and not lean.dx_written(0)
+    assert_close(full.layer_dx(0, batch), ref.layer_dx(0, batch), what=f"{name} input gradient")
+    for i, l in enumerate(spec):
+        assert full.out_written(i) == lean.out_written(i)
+        if full.out_written(i):
+            assert np.array_equal(full.layer_out(i, batch), lean.layer_out(i, batch)), f"{name} layer {i} output"
+        if i:
+            assert full.dx_written(i) == lean.dx_written(i)
+            if full.dx_written(i):
+                assert np.array_equal(full.layer_dx(i, batch), lean.layer_dx(i, batch)), f"{name} layer {i} dX"
+        for which in (0, 1):
+            if full.param_size(i, which):
+                assert np.array_equal(full.layer_grad(i, which), lean.layer_grad(i, which)), f"{name} gradient {i}.{which}"
+                want = ref.layer_dw(i) if which == 0 else ref.layer_db(i)
+                assert_close(lean.layer_grad(i, which), want, what=f"{name} gradient {i}.{which}")
+    opts = [T.opt_desc(opt_kind, **opt_kw) for _ in range(2)]
+    for m in (full, lean):
+        m.clear_grads()
+    for n in (batch, batch, 7):
+        for m, o in zip((full, lean), opts):
+            m.train_step(o, loss, n, xd, td)
+    for (i, which, _) in params:
+        assert np.array_equal(full.get_param(i, which), lean.get_param(i, which)), f"{name} parameter {i}.{which}"
+    assert not lean.dx_written(0)
+    full.close()
+    lean.close()
+
+
+def test_first_layers_of_other_kinds_ignore_the_input_gradient_flag(T, O, W):
+    nets = {"pool_first": ([("maxpool", 8, 8, 3, 2), ("fc", 48, 5)], "mse", "sgd")}
+    for flags in (0, FUSE | GRAPH, SAMPLE | FUSE):
+        spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref = build(T, O, W, "pool_first", 6, flags | NO_INPUT_GRAD, nets=nets)
+        net.train_step(None, loss, batch, T.to_device(x), T.to_device(t), do_update=False)
+        ref.train_step(O.opt_desc(opt_kind), loss, x, t, do_update=False)
+        assert net.dx_written(0)
+        assert_close(net.layer_dx(0, batch), ref.layer_dx(0, batch), what="input gradient of a net that starts with a pool")
         net.close()

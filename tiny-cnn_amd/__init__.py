@@ -25,7 +25,7 @@ ACT = {"tanh": 0, "relu": 1, "softmax": 2, "sigmoid": 3, "leaky_relu": 4, "elu":
 LOSS = {"mse": 0, "ce_multiclass": 1, "ce": 2}
 OPT = {"sgd": 0, "momentum": 1, "adam": 2, "adagrad": 3, "rmsprop": 4, "adamax": 5, "nesterov": 6}
 L_CONV, L_FC, L_MAXPOOL, L_AVEPOOL, L_ACT, L_BATCHNORM, L_DROPOUT = range(7)
-NET_FUSE_ACT_GRAD, NET_GRAPH, NET_SAMPLE_STEP = 1, 2, 4
+NET_FUSE_ACT_GRAD, NET_GRAPH, NET_SAMPLE_STEP, NET_NO_INPUT_GRAD = 1, 2, 4, 8
 
 f32p = C.POINTER(C.c_float)
 

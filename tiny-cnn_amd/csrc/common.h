@@ -206,10 +206,22 @@ struct OptPending {
   OptPendingSum sum[OPT_PENDING_MAX];
   int n;
 };
+// What a workgroup of the multi-tensor update needs to find its tensor and that tensor's pending
+// sum without walking the device table entry by entry (each step of such a walk is a memory
+// latency, and a step of a small net is little more than a few of those): the first block of
+// every tensor and the index of its pending sum, as kernel arguments. n == 0: no index (more
+// tensors than OPT_INDEX_MAX, or no host copy of the table), the kernel walks and searches.
+constexpr int OPT_INDEX_MAX = 32;
+struct OptIndex {
+  uint32_t first_block[OPT_INDEX_MAX];  // 0xffffffff past the last tensor
+  int8_t pend_of[OPT_INDEX_MAX];        // index into OptPending::sum, or -1
+  int n;
+};
+// host_table: the host copy of dev_table (for the index above), or NULL
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
                             int zero_grad, const float *powers_in, float *powers_out,
-                            const OptPending *pending = nullptr);
+                            const OptPending *pending = nullptr, const OptTensor *host_table = nullptr);
 // conv.hip: the recorded split reductions in the optimizer's form (false: they do not all fit its
 // form or number). They stay recorded: flush_deferred_reduces launches or forgets them.
 bool peek_deferred_reduces(OptPending *out);

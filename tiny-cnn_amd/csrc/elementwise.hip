@@ -443,7 +443,7 @@ template <int KIND, int NSTATE>
 __global__ void __launch_bounds__(EW_THREADS)
 opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptScalars p,
                  float b1_t, float b2_t, const float *powers_in, float *powers_out, const int advance,
-                 const int zero_grad, const OptPending pend) {
+                 const int zero_grad, const OptPending pend, const OptIndex idx) {
   if (powers_in) {
     b1_t = powers_in[0];
     b2_t = powers_in[1];
@@ -460,8 +460,15 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
       powers_out[1] = q2;
     }
   }
-  int j = 0;
-  while (j + 1 < n_tensors && table[j + 1].first_block <= blockIdx.x) ++j;
+  int j = 0, pj = -1;
+  if (idx.n) {
+    // first blocks ascend, and those past the last tensor compare false
+#pragma unroll
+    for (int k = 1; k < OPT_INDEX_MAX; ++k) j += idx.first_block[k] <= blockIdx.x ? 1 : 0;
+    pj = idx.pend_of[j];
+  } else {
+    while (j + 1 < n_tensors && table[j + 1].first_block <= blockIdx.x) ++j;
+  }
   const OptTensor t = table[j];
   // the reference multiplies b1_t by b1 after every update() call (optimizer.h:125-126)
   float p1 = b1_t, p2 = b2_t;
@@ -480,9 +487,9 @@ opt_multi_kernel(const OptTensor *__restrict__ table, const int n_tensors, OptSc
   // splitk_reduce_block (eight 32-lane groups each add every eighth slice in order, the group
   // sums are added in group order), four consecutive elements a lane
   __shared__ float pending_sum[8][OPT_SUM_ELEMS_PER_BLOCK];
-  int pj = -1;
-  for (int k = 0; k < pend.n; ++k)
-    if (pend.sum[k].g == t.g) pj = k;
+  if (!idx.n)
+    for (int k = 0; k < pend.n; ++k)
+      if (pend.sum[k].g == t.g) pj = k;
   // (the host hands over pending sums only for tensors with the small blocks; a tensor with
   // large blocks would index pending_sum out of bounds, so it is left alone here)
   if (t.block_elems != OPT_SUM_ELEMS_PER_BLOCK) pj = -1;
@@ -842,7 +849,7 @@ size_t rowsum_workspace_bytes(int outer, int rows, int cols) {
 int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensors,
                             int total_blocks, double total_params, float grad_scale,
                             int zero_grad, const float *powers_in, float *powers_out,
-                            const OptPending *pending) {
+                            const OptPending *pending, const OptTensor *host_table) {
   if (n_tensors <= 0) return TDH_OK;
   OptPending pend;
   pend.n = 0;
@@ -850,6 +857,17 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
   if (pending) {
     pend = *pending;
     for (int k = 0; k < pend.n; ++k) pending_bytes += 4.0 * pend.sum[k].splits * pend.sum[k].mn;
+  }
+  OptIndex idx;
+  idx.n = 0;
+  if (host_table && n_tensors <= OPT_INDEX_MAX) {
+    idx.n = n_tensors;
+    for (int k = 0; k < OPT_INDEX_MAX; ++k) {
+      idx.first_block[k] = k < n_tensors ? host_table[k].first_block : 0xffffffffu;
+      idx.pend_of[k]     = -1;
+      for (int q = 0; k < n_tensors && q < pend.n; ++q)  // (the last match, as the kernel's search)
+        if (pend.sum[q].g == host_table[k].g) idx.pend_of[k] = static_cast<int8_t>(q);
+    }
   }
   OptScalars p;
   p.alpha = o->alpha; p.lambda = o->lambda; p.mu = o->mu; p.b1 = o->b1; p.b2 = o->b2;
@@ -872,7 +890,7 @@ int launch_opt_update_multi(tdh_opt *o, const OptTensor *dev_table, int n_tensor
 #define TDH_LAUNCH_MULTI(KIND, NS)                                                            \
   TDH_LAUNCH((opt_multi_kernel<KIND, NS>), dim3(total_blocks), dim3(EW_THREADS), 0,   \
                      ctx().stream, dev_table, n_tensors, p, o->b1_t, o->b2_t,                  \
-                     powers_in, powers_out, advance, zero_grad, pend)
+                     powers_in, powers_out, advance, zero_grad, pend, idx)
   switch (o->kind) {
     case TDH_OPT_SGD: TDH_LAUNCH_MULTI(TDH_OPT_SGD, 0); break;
     case TDH_OPT_MOMENTUM: TDH_LAUNCH_MULTI(TDH_OPT_MOMENTUM, 1); break;

@@ -37,6 +37,7 @@ struct tdh_net {
   bool test_phase = false;  // net_phase::test
   float *dx_in   = nullptr;  // gradient w.r.t. the network input
   tdh::OptTensor *opt_table = nullptr;  // device table of trainable tensors, update order
+  std::vector<tdh::OptTensor> opt_table_host;  // (its host copy)
   bool packs_valid = false;  // wp_fwd / wp_dx of every layer match its weights
   int opt_tensors = 0, opt_blocks = 0;
   double opt_params = 0.0;
@@ -160,6 +161,13 @@ double net_forward_flop(const tdh_net *net, int batch) {
   }
   return 2.0 * batch * macs;
 }
+// TDH_NET_NO_INPUT_GRAD on a net whose first layer is one of the kinds that honour it
+bool net_skips_input_grad(const tdh_net *net) {
+  if (!(net->flags & TDH_NET_NO_INPUT_GRAD) || net->layers.empty()) return false;
+  const int kind = net->layers[0].spec.kind;
+  return kind == TDH_L_CONV || kind == TDH_L_FC;
+}
+
 bool net_forks(const tdh_net *net, int batch) {
   const double flop = net_forward_flop(net, batch);
   return flop >= 1e8 && flop <= 3e10;
@@ -197,6 +205,10 @@ int build_tiny_plan(tdh_net *net) {
     T.in_size = static_cast<int>(L.in_size); T.out_size = static_cast<int>(L.out_size);
     T.w = L.w; T.b = L.b; T.out = L.out;
     T.dx = i == 0 ? net->dx_in : net->layers[i - 1].dout;
+    if (i == 0 && net_skips_input_grad(net)) {
+      T.dx = nullptr;
+      P.skip_first_dx = 1;
+    }
     T.nw = static_cast<int>(L.w_size); T.nb = static_cast<int>(L.b_size);
     T.lds_in  = i == 0 ? 0 : P.l[i - 1].lds_out;
     T.lds_out = static_cast<int>(lds);
@@ -677,6 +689,7 @@ int tdh_net_create(const tdh_layer *layers, int n_layers, int max_batch, int fla
       if (rc == TDH_OK) {
         net->opt_table = reinterpret_cast<OptTensor *>(p);
         rc = tdh_memcpy_h2d(net->opt_table, table.data(), table.size() * sizeof(OptTensor));
+        net->opt_table_host = table;
       }
     }
   }
@@ -786,7 +799,7 @@ int tdh_net_update_weights(tdh_net *net, tdh_opt *opt) {
   TDH_CHECK_ARG(net && opt, "tdh_net_update_weights: null argument");
   // the optimizer kernel keeps the packed filter copies of a graph net current, as in a step
   TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
-                                  net->opt_params, 1.0f, 1, nullptr, nullptr));
+                                  net->opt_params, 1.0f, 1, nullptr, nullptr, nullptr, net->opt_table_host.data()));
   return post_update(net);
 }
 int tdh_net_set_phase(tdh_net *net, int train) {
@@ -858,6 +871,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     const tdh_layer &closing = net->layers.back().spec;
     const int softmax_xent = closing.kind == TDH_L_ACT && closing.act == TDH_ACT_SOFTMAX;
     net->dx_unwritten.assign(net->layers.size(), 0);   // everything is written to memory as well
+    if (net_skips_input_grad(net)) net->dx_unwritten[0] = 1;
     net->out_unwritten.assign(net->layers.size(), 0);
     TDH_TRY(launch_tiny_step(net->tiny, net->tiny_dev, loss_kind, softmax_xent, batch, x, t));
     TDH_TRY(launch_tiny_params(net->tiny, net->tiny_dev, batch, x));
@@ -878,7 +892,8 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     if (!to_optimizer) TDH_TRY(launch_tiny_merge(net->tiny_merge, batch));
     if (!do_update) return TDH_OK;
     TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks, net->opt_params, 1.0f,
-                                    1, powers_in, powers_out, to_optimizer ? &pending : nullptr));
+                                    1, powers_in, powers_out, to_optimizer ? &pending : nullptr,
+                                    net->opt_table_host.data()));
     return post_update(net);
   }
   Context &c = ctx();
@@ -949,12 +964,16 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
     const DxTarget target = dx_target(net, i);
     float *dx             = target.dx;
     const ActGrad fold    = target.fold;
+    if (i == 0 && net_skips_input_grad(net)) {
+      dx = nullptr;
+      net->dx_unwritten[0] = 1;
+    }
     if (i == tail_done) {
       // only the weight and bias gradients are left, and nothing before the optimizer reads
       // them: they leave with the backward launch of the fully-connected layer two in front
       // when that is the one-launch kernel, else as one launch, on the side stream when the
       // step branches
-      if (plan.first >= 0 && fc_bwd_fuses(s.fc_in, s.fc_out, batch) &&
+      if (plan.first >= 0 && !(plan.first == 0 && net_skips_input_grad(net)) && fc_bwd_fuses(s.fc_in, s.fc_out, batch) &&
           fc_bwd_fuses(net->layers[plan.first].spec.fc_in, net->layers[plan.first].spec.fc_out, batch)) {
         also = FcGrads{s.fc_in, s.fc_out, in, L.dout, L.dw, L.b_size ? L.db : nullptr};
         also_for = plan.first;
@@ -1009,7 +1028,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             break;
           }
           const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
-          {
+          if (dx) {
             LeaveSplitSum leave(c, pool_reads);
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp, gp));
           }
@@ -1041,7 +1060,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           }
         } else if (as_forked) {
           // the launches of the captured, branching step, one after the other
-          {
+          if (dx) {
             LeaveSplitSum leave(c, pool_reads);
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp, gp));
           }
@@ -1064,7 +1083,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
       case TDH_L_FC:
         TDH_TRY(ws_begin(fc_workspace_bytes(s.fc_in, s.fc_out, batch)));
         if (fork) {
-          TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
+          if (dx) TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
           {
             StreamSwap on_side(c.side[0]);
             c.defer_reduce = true;
@@ -1077,7 +1096,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           }
         } else if (as_forked && !fc_one_launch) {
           // the launches of the captured, branching step, one after the other
-          TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
+          if (dx) TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold));
           c.defer_reduce = true;
           TDH_TRY(fc_bwd(s.fc_in, s.fc_out, s.fc_bias, batch, in, L.w, L.dout, nullptr, L.dw, nullptr, 1, ActGrad()));
           c.defer_reduce = false;
@@ -1172,7 +1191,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
   // cleared (layer.h:680)
   TDH_TRY(launch_opt_update_multi(opt, net->opt_table, net->opt_tensors, net->opt_blocks,
                                   net->opt_params, 1.0f, 1, powers_in, powers_out,
-                                  to_optimizer ? &pending : nullptr));
+                                  to_optimizer ? &pending : nullptr, net->opt_table_host.data()));
   return post_update(net);
 }
 

@@ -53,6 +53,7 @@ struct TinyPlan {
   TinyJob jobs[TINY_MAX_JOBS];
   int n_jobs;
   int first_dx_as_job;         // the first layer's input gradient is among the jobs
+  int skip_first_dx;           // nobody wants the gradient of the net's input: it is not computed
   int lds_job_floats;          // LDS of the parameter-gradient kernel
 };
 

@@ -1043,7 +1043,7 @@ tiny_net_step_kernel(const TinyPlan *__restrict__ plan, const int loss, const in
   }
   __syncthreads();   // (also: the max-pool records written to memory above are read back below)
   // input gradients only: the parameter-gradient kernel reads what this loop leaves in memory
-  const int last_bwd = plan->first_dx_as_job ? 1 : 0;
+  const int last_bwd = (plan->first_dx_as_job || plan->skip_first_dx) ? 1 : 0;
   for (int li = first_bwd; li >= last_bwd; --li) {
     const TinyLayer *__restrict__ L = &plan->l[li];
     const int kind = L->kind, in_sz = L->in_size;
@@ -1083,8 +1083,8 @@ constexpr int TP_THREADS = 256;
 __global__ void __launch_bounds__(TP_THREADS)
 tiny_net_param_kernel(const TinyPlan *__restrict__ plan, const float *__restrict__ x) {
   extern __shared__ float lds[];
-  const TinyJob job = plan->jobs[blockIdx.x];
-  const int s = blockIdx.y, n = plan->n, li = job.layer;
+  const TinyJob job = plan->jobs[blockIdx.y];
+  const int s = blockIdx.x, n = plan->n, li = job.layer;
   const TinyLayer *__restrict__ L = &plan->l[li];
   const int in_sz = L->in_size, out_sz = L->out_size, kind = L->kind;
   const float *gin = (li == 0 ? x : plan->l[li - 1].out) + static_cast<size_t>(s) * in_sz;
@@ -1176,7 +1176,7 @@ int tiny_build_jobs(TinyPlan &P) {
       L.d_pw     = FastDiv(static_cast<uint32_t>(L.W + L.S - 1));
     }
   }
-  P.first_dx_as_job = P.l[0].dx_framed && P.n > 1;
+  P.first_dx_as_job = P.l[0].dx_framed && P.n > 1 && !P.skip_first_dx;
   for (int i = 0; i < P.n; ++i) {
     const TinyLayer &L = P.l[i];
     if (i == 0 && P.first_dx_as_job) {
@@ -1226,7 +1226,9 @@ int launch_tiny_step(const TinyPlan &plan, const TinyPlan *dev_plan, int loss, i
 int launch_tiny_params(const TinyPlan &plan, const TinyPlan *dev_plan, int batch, const float *x) {
   if (plan.n_jobs == 0) return TDH_OK;
   ProfScope prof("tiny_net_param_grads", plan.flop_per_sample * batch * (1.0 / 3.0), WORK_FLOP);
-  TDH_LAUNCH(tiny_net_param_kernel, dim3(plan.n_jobs, batch), dim3(TP_THREADS), plan.lds_job_floats * sizeof(float),
+  // (x counts the samples: consecutive workgroups go to different XCDs, and this way each XCD
+  // gets every job of the samples that fall to it rather than every sample of a few jobs)
+  TDH_LAUNCH(tiny_net_param_kernel, dim3(batch, plan.n_jobs), dim3(TP_THREADS), plan.lds_job_floats * sizeof(float),
              ctx().stream, dev_plan, x);
   TDH_LAUNCH_CHECK();
   return TDH_OK;
