@@ -27,6 +27,13 @@ NETS = {
     "odd_sizes_uncovered_column_ce": ([("conv", 15, 11, 3, 5, 6, True), ("act", "tanh"), ("maxpool", 15, 11, 6, 2),
                                       ("fc", 6 * 5 * 7, 6), ("act", "sigmoid")], "ce", "momentum"),
     "fc_only_mse": ([("fc", 40, 30), ("act", "tanh"), ("fc", 30, 7)], "mse", "adagrad"),
+    # unpadded stride-1 convolutions with eight or more output channels run their forward products
+    # on the matrix cores: as the first layer with more pixel tiles than waves, as the layer whose
+    # filters travel in registers, and with a connection table
+    "valid_convs_on_matrix_cores": ([("conv", 22, 20, 3, 5, 12, False), ("act", "relu"), ("maxpool", 18, 16, 12, 2),
+                                     ("conv", 9, 8, 12, 3, 16, False), ("act", "tanh"),
+                                     ("conv", 7, 6, 16, 3, 8, False, [[(ci + co) % 3 != 0 for co in range(8)] for ci in range(16)]),
+                                     ("act", "sigmoid"), ("fc", 8 * 5 * 4, 10), ("act", "softmax")], "ce_multiclass", "adam"),
 }
 
 

@@ -211,8 +211,15 @@ int build_tiny_plan(tdh_net *net) {
     }
     T.nw = static_cast<int>(L.w_size); T.nb = static_cast<int>(L.b_size);
     T.lds_in  = i == 0 ? 0 : P.l[i - 1].lds_out;
-    T.lds_out = static_cast<int>(lds);
-    lds += L.out_size;
+    // a pointwise activation overwrites its input: of the forward values the backward pass
+    // of the step kernel reads only the outputs of activations (the gradients of tanh, relu,
+    // sigmoid and leaky relu are functions of those), and the weight gradients read the
+    // copies in memory
+    // (unless that input is itself an activation's output)
+    const bool in_place = i > 0 && sp.kind == TDH_L_ACT && sp.act != TDH_ACT_SOFTMAX &&
+                          net->layers[i - 1].spec.kind != TDH_L_ACT;
+    T.lds_out = in_place ? T.lds_in : static_cast<int>(lds);
+    if (!in_place) lds += L.out_size;
     gmax = std::max(gmax, L.out_size);
     switch (sp.kind) {
       case TDH_L_CONV: {

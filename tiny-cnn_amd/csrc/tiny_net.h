@@ -33,6 +33,10 @@ struct TinyLayer {
   // [K][H + R - 1][W + S - 1] floats in LDS; 0 when the layer takes the general loops
   int dx_framed;
   FastDiv d_pplane, d_pw;
+  // A stride-1 convolution's forward product without padding on the matrix cores (conv_mfma in
+  // tiny_net.hip): where in LDS the step kernel keeps the filters as [co][k] (k = (ci, tap), rows
+  // padded with zeros), the input offset of every k and a copy of the bias; -1: the scalar loops
+  int mf_fwd_w, mf_fwd_ko, mf_fwd_b;
 };
 
 // One workgroup's share of the parameter-gradient kernel for one sample: the units
@@ -47,6 +51,8 @@ struct TinyPlan {
   TinyLayer l[TINY_MAX_LAYERS];
   int n, in_size;
   int lds_g0, lds_g1, lds_w, lds_pad, lds_floats;   // lds_pad: the zero-framed dY
+  int n_mfma, mfma_layers[TINY_MAX_LAYERS];   // the layers with operands to stage for the matrix cores
+  int mf_ahead;                // the layer (> 0) whose filters wait in registers until the layer in front of it runs, or -1
   float mse_factor;            // 2 / outputs
   float *dloss;                // memory: gradient w.r.t. the net's output [batch][out_size]
   double flop_per_sample;

@@ -675,6 +675,154 @@ TN_INLINE void conv_bwd_dx_scalar_any(const TinyLayer *__restrict__ Lp, const fl
   }
 }
 
+// ---------------------------------------------------------------- convolutions on the matrix cores
+// out[m][p] = bias[m] + sum_k A[m][k] * in[koff[k] + poff(p)]: the forward pass of a stride-1
+// convolution without padding (every tap of every output pixel lies inside the input) as a
+// product of the filters with the patches of the input. v_mfma_f32_16x16x4_f32: lane
+// (r = lane % 16, q = lane / 16) supplies A[row r][one k] and B[the same k][column r] and holds
+// D[row 4 q + i][column r], i = 0..3; which four k an instruction adds up is free, and here step
+// st of `steps` takes k = q * steps + st, so that a lane's operands of four steps in a row are
+// 16 consecutive bytes of a filter row and of the offset table. A wave takes 16 channels x
+// T tiles of 16 pixels at once (what bounds a tile is the chain of LDS reads in front of its
+// first product, not the products: T tiles share that chain). `a` holds A as [M][pitch] with
+// zeros from n_k on, `koff` the input offset of every k < 4 * steps, `bias` the bias or NULL,
+// all in LDS (stage_mfma_operands); steps is a multiple of four.
+typedef float tn_f4 __attribute__((ext_vector_type(4)));
+__host__ __device__ inline int mfma_steps(const int n_k) { return ((n_k + 15) >> 4) << 2; }
+// (a row pitch of 4 * odd floats: sixteen rows read 16 bytes each from different banks, two rows a bank group)
+__host__ __device__ inline int mfma_pitch(const int n_k) { return (4 * mfma_steps(n_k)) | 4; }
+template <int T>
+TN_INLINE void conv_mfma(const float *src, const float *a, const int *koff, const int M, const int n_k,
+                         const int plane, const FastDiv d_row, const int src_pitch, const float *bias,
+                         float *out, float *__restrict__ gout) {
+  const int lane = threadIdx.x & 63, r = lane & 15, q = lane >> 4;
+  const int steps = mfma_steps(n_k), pitch = mfma_pitch(n_k), groups = steps >> 2;
+  const int m_tiles = (M + 15) >> 4, p_tiles = (plane + 15) >> 4, p_items = (p_tiles + T - 1) / T;
+  const int total = m_tiles * p_items;
+  const int k_left = n_k - q * steps;   // this lane's steps from k_left on are padding
+  for (int it0 = 0; it0 < total; it0 += TN_WAVES) {
+    const int item = it0 + wave_index();
+    if (item >= total) break;     // (no barrier inside)
+    const int mt = item / p_items, pi = item - mt * p_items;
+    const int arow = min(mt * 16 + r, M - 1);
+    const float *sp[T];
+#pragma unroll
+    for (int j = 0; j < T; ++j) {
+      uint32_t py, px;
+      d_row.divmod(min((pi * T + j) * 16 + r, plane - 1), py, px);
+      sp[j] = src + static_cast<int>(py) * src_pitch + static_cast<int>(px);
+    }
+    const float4 *a4 = reinterpret_cast<const float4 *>(a + arow * pitch + q * steps);
+    const int4 *k4 = reinterpret_cast<const int4 *>(koff + q * steps);
+    tn_f4 acc[T];
+#pragma unroll
+    for (int j = 0; j < T; ++j) acc[j] = tn_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float4 av = a4[0];
+    int4 ko   = k4[0];
+    for (int g = 0; g < groups; ++g) {
+      float b[T][4];
+#pragma unroll
+      for (int j = 0; j < T; ++j) {
+        b[j][0] = sp[j][ko.x]; b[j][1] = sp[j][ko.y]; b[j][2] = sp[j][ko.z]; b[j][3] = sp[j][ko.w];
+      }
+      const float4 ac = av;
+      const int gn = min(g + 1, groups - 1);
+      av = a4[gn];
+      ko = k4[gn];
+      // (a zero filter value times an infinity would be a NaN)
+      const int st = 4 * g;
+      const bool on0 = st < k_left, on1 = st + 1 < k_left, on2 = st + 2 < k_left, on3 = st + 3 < k_left;
+#pragma unroll
+      for (int j = 0; j < T; ++j) {
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ac.x, on0 ? b[j][0] : 0.0f, acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ac.y, on1 ? b[j][1] : 0.0f, acc[j], 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < T; ++j) {
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ac.z, on2 ? b[j][2] : 0.0f, acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ac.w, on3 ? b[j][3] : 0.0f, acc[j], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = mt * 16 + 4 * q + i;
+      if (m >= M) continue;
+      const float bv = bias ? bias[m] : 0.0f;
+#pragma unroll
+      for (int j = 0; j < T; ++j) {
+        const int p = (pi * T + j) * 16 + r;
+        if (p < plane) {
+          const float v = bias ? acc[j][i] + bv : acc[j][i];
+          out[m * plane + p]  = v;
+          gout[m * plane + p] = v;
+        }
+      }
+    }
+  }
+}
+// The operands above for a layer that has them, straight from the weight tensor. Every filter
+// value is read once, in the tensor's own order ([co][(ci, tap)], which is A's); pairs of
+// channels that a connection table leaves unconnected get a zero, and so do the ends of the
+// rows. In two halves, so that the reads can be in flight while other layers run: the first
+// asks for up to MFMA_AHEAD values a thread, the second puts them in LDS.
+constexpr int MFMA_AHEAD = 4;
+TN_INLINE void mfma_filters_load(const TinyLayer *__restrict__ L, const int e0, float (&v)[MFMA_AHEAD], float &bias) {
+  const int nw = L->K * L->C * L->R * L->S;
+#pragma unroll
+  for (int j = 0; j < MFMA_AHEAD; ++j) v[j] = L->w[min(e0 + j * TN_THREADS + static_cast<int>(threadIdx.x), nw - 1)];
+  // (the bias goes with the first piece: a value a thread, there are fewer channels than threads)
+  bias = (e0 == 0 && L->has_bias) ? L->b[min(static_cast<int>(threadIdx.x), L->K - 1)] : 0.0f;
+}
+TN_INLINE void mfma_filters_store(const TinyLayer *__restrict__ L, const int e0, const float (&v)[MFMA_AHEAD],
+                                  const float bias, float *lds) {
+  const int K = L->K, taps = L->R * L->S, n_k = L->C * taps, nw = K * n_k, pitch = mfma_pitch(n_k);
+  const uint8_t *__restrict__ tbl = L->tbl;
+  float *fa = lds + L->mf_fwd_w;
+#pragma unroll
+  for (int j = 0; j < MFMA_AHEAD; ++j) {
+    const int e = e0 + j * TN_THREADS + threadIdx.x;
+    if (e >= nw) continue;
+    uint32_t co, k, ci, t;
+    L->d_nk.divmod(e, co, k);
+    L->d_taps.divmod(k, ci, t);
+    fa[co * pitch + k] = (tbl && !tbl[ci * K + co]) ? 0.0f : v[j];
+  }
+  if (e0 == 0 && L->has_bias && static_cast<int>(threadIdx.x) < K) lds[L->mf_fwd_b + threadIdx.x] = bias;
+}
+// everything else: the rows' zero ends and the offset table
+TN_INLINE void mfma_tables(const TinyLayer *__restrict__ L, float *lds) {
+  const int K = L->K, H = L->H, W = L->W, taps = L->R * L->S;
+  const int n_k = L->C * taps, pitch = mfma_pitch(n_k), k4 = 4 * mfma_steps(n_k), pad = pitch - n_k;
+  float *fa = lds + L->mf_fwd_w;
+  int *ko   = reinterpret_cast<int *>(lds + L->mf_fwd_ko);
+  for (int idx = threadIdx.x; idx < K * pad; idx += TN_THREADS) {
+    const int row = idx / pad;
+    fa[row * pitch + n_k + idx - row * pad] = 0.0f;
+  }
+  for (int k = threadIdx.x; k < k4; k += TN_THREADS) {
+    uint32_t ci, t, wy, wx;
+    L->d_taps.divmod(min(k, n_k - 1), ci, t);
+    L->d_s.divmod(t, wy, wx);
+    ko[k] = k < n_k ? static_cast<int>(ci) * H * W + static_cast<int>(wy) * W + static_cast<int>(wx) : 0;
+  }
+}
+// every layer but the one whose filters travel in registers (`ahead`, or -1): when the kernel starts
+TN_INLINE void stage_mfma_operands(const TinyPlan *__restrict__ plan, float *lds, const int ahead) {
+  const int n = plan->n_mfma;
+  for (int q = 0; q < n; ++q) {   // (the plan lists them: walking every layer is a scalar load and a wait each)
+    const int li = plan->mfma_layers[q];
+    if (li == ahead) continue;
+    const TinyLayer *__restrict__ L = &plan->l[li];
+    mfma_tables(L, lds);
+    const int nw = L->K * L->C * L->R * L->S;
+    for (int e0 = 0; e0 < nw; e0 += MFMA_AHEAD * TN_THREADS) {
+      float v[MFMA_AHEAD], bias;
+      mfma_filters_load(L, e0, v, bias);
+      mfma_filters_store(L, e0, v, bias, lds);
+    }
+  }
+}
+
 // A convolution whose window is the whole input (one output pixel per channel, no padding) is a
 // matrix-vector product: out[co] = sum_k W[co][k] in[k], dX[k] = sum_co W[co][k] dY[co]. Lanes
 // run along k, so the filter rows are read in whole cache lines, and a lane asks for all the
@@ -980,10 +1128,20 @@ tiny_net_step_kernel(const TinyPlan *__restrict__ plan, const int loss, const in
   extern __shared__ float lds[];
   const int s = blockIdx.x, n = plan->n, in_size = plan->in_size;
   float *wl = lds + plan->lds_w;   // where partial sums of split layers meet (TINY_SCRATCH_FLOATS)
+  // (one layer's filters for the matrix cores are asked for here, in front of the sample's input,
+  // and put in LDS while the layer in front of that layer runs: no layer waits for them)
+  const int ahead = plan->mf_ahead;
+  float ahead_w[MFMA_AHEAD] = {0.0f, 0.0f, 0.0f, 0.0f}, ahead_b = 0.0f;
+  if (ahead > 0) mfma_filters_load(&plan->l[ahead], 0, ahead_w, ahead_b);
   fill_lds<TN_THREADS>(lds, x + static_cast<size_t>(s) * in_size, in_size);
+  stage_mfma_operands(plan, lds, ahead);
   lds_barrier();
   for (int li = 0; li < n; ++li) {
     const TinyLayer *__restrict__ L = &plan->l[li];
+    if (li + 1 == ahead) {
+      mfma_filters_store(&plan->l[ahead], 0, ahead_w, ahead_b, lds);
+      mfma_tables(&plan->l[ahead], lds);
+    }
     const int kind = L->kind, out_size = L->out_size;
     const float *in = lds + L->lds_in;
     float *out      = lds + L->lds_out;
@@ -993,6 +1151,14 @@ tiny_net_step_kernel(const TinyPlan *__restrict__ plan, const int loss, const in
         if (conv_is_matvec(*L)) {
           if (!L->tbl && ((L->C * L->R * L->S) & 3) == 0 && (L->lds_in & 3) == 0) conv_fwd_matvec4(L, in, out, gout);
           else conv_fwd_matvec(L, in, out, gout);
+        }
+        else if (L->mf_fwd_w >= 0) {
+          const float *fa = lds + L->mf_fwd_w, *fb = L->has_bias ? lds + L->mf_fwd_b : nullptr;
+          const int *fk = reinterpret_cast<const int *>(lds + L->mf_fwd_ko);
+          const int n_k = L->C * L->R * L->S, plane = L->OH * L->OW;
+          // (several pixel tiles a wave when there are more tiles than waves)
+          if (((L->K + 15) >> 4) * ((plane + 15) >> 4) > TN_WAVES) conv_mfma<4>(in, fa, fk, L->K, n_k, plane, L->d_ow, L->W, fb, out, gout);
+          else conv_mfma<1>(in, fa, fk, L->K, n_k, plane, L->d_ow, L->W, fb, out, gout);
         }
         else if (L->R == 5 && L->S == 5 && L->ph == 0 && L->pw == 0) conv_fwd_scalar_any<5, 5, false>(L, in, out, gout, wl);
         else if (L->R == 5 && L->S == 5) conv_fwd_scalar_any<5, 5, true>(L, in, out, gout, wl);
@@ -1193,6 +1359,32 @@ int tiny_build_jobs(TinyPlan &P) {
   }
   P.lds_pad = P.lds_floats;
   P.lds_floats += static_cast<int>(framed);
+  // operands of the products that run on the matrix cores, while LDS has room for them
+  P.n_mfma = 0;
+  P.mf_ahead = -1;
+  for (int i = 0; i < P.n; ++i) {
+    TinyLayer &L = P.l[i];
+    L.mf_fwd_w = L.mf_fwd_ko = L.mf_fwd_b = -1;
+    // (few output channels leave most of a 16-row tile empty, and a short sum is over before
+    // the operands of its first product have arrived: those stay with the scalar loops)
+    if (L.kind != TDH_L_CONV || conv_is_matvec(L) || L.sh != 1 || L.sw != 1 || L.K < 8 ||
+        L.C * L.R * L.S < 48)
+      continue;
+    const size_t room = TINY_LDS_MAX_BYTES / sizeof(float);
+    const int taps = L.R * L.S;
+    // (both areas start on 16 bytes: rows and offset tables are read four values at a time)
+    if (L.ph == 0 && L.pw == 0) {
+      const int n_k = L.C * taps;
+      const size_t need = static_cast<size_t>(mfma_pitch(n_k)) * L.K + 4 * mfma_steps(n_k) + L.K;
+      const int at = (P.lds_floats + 3) & ~3;
+      if (at + need <= room) {
+        L.mf_fwd_w = at; L.mf_fwd_ko = at + mfma_pitch(n_k) * L.K; L.mf_fwd_b = L.mf_fwd_ko + 4 * mfma_steps(n_k);
+        P.lds_floats = at + static_cast<int>(need);
+        P.mfma_layers[P.n_mfma++] = i;
+        if (P.mf_ahead < 0 && i > 0 && L.K * n_k <= MFMA_AHEAD * TN_THREADS) P.mf_ahead = i;
+      }
+    }
+  }
   for (int scale = 1;; scale *= 2) {
     int jobs = 0;
     for (int q = 0; q < n_pieces; ++q) jobs += ceil_div(pieces[q].units, pieces[q].per_job * scale);
