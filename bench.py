@@ -322,8 +322,9 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="only the named workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-host-inputs", action="store_true",
-                    help="leave out the leg that hands over host batches every step (profiler runs: rocprofv3 "
-                         "7.2 dies in that leg of the VGG workload, in a host copy below hipGraphInstantiate)")
+                    help="leave out the legs beside the headline: host batches handed over every step, the step "
+                         "without the input gradient (profiler runs: rocprofv3 7.2 dies in the first of the two "
+                         "for the VGG workload, in a host copy below hipGraphInstantiate)")
     ap.add_argument("--sequence-out", default=None,
                     help="write the kernel tags of one step in dispatch order to this JSON file "
                          "(tiny-cnn_amd.profsum reads a rocprofv3 trace of the same run tag by tag with it)")
@@ -381,7 +382,7 @@ def main():
                               "steps": host_steps,
                               "note": "inputs and targets handed over in pageable host memory every step "
                                       "and uploaded through pinned slots on a copy stream (tdh_feeder)"}
-    if isinstance(wl, NetWorkload):
+    if isinstance(wl, NetWorkload) and not args.no_host_inputs:
         # never `value` either: the same step without the gradient of the net's input, which the
         # reference computes and training never reads (the caller's choice: TDH_NET_NO_INPUT_GRAD)
         w3 = NetWorkload(T, W, args.workload, T.NET_NO_INPUT_GRAD)
