@@ -40,10 +40,11 @@ struct TinyLayer {
 };
 
 // One workgroup's share of the parameter-gradient kernel for one sample: the units
-// [base, base + count) of a layer's weight-gradient work (the bias gradient goes with base 0),
+// [base, base + count) of a layer's weight-gradient work (the bias gradient goes with base 0,
+// except that of a convolution that is not a matrix-vector product, which is a job of its own),
 // or, for the first layer, the wave items [base, base + count) of its input gradient.
 struct TinyJob {
-  int16_t layer, what;         // what: 0 = weight / bias gradient, 1 = input gradient
+  int16_t layer, what;         // what: 0 = weight (/ bias) gradient, 1 = input gradient, 2 = bias gradient
   int base, count;
 };
 

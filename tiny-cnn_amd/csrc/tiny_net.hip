@@ -1036,9 +1036,9 @@ __host__ __device__ inline int conv_param_group(const TinyLayer &L) {
 // Units [base, base + count) of nw * group (weights x lanes); the bias gradient goes with base 0.
 template <int NT>
 TN_INLINE void conv_bwd_param_rows(const TinyLayer *__restrict__ Lp, const float *in, const float *dy,
-                                   float *__restrict__ gw, float *__restrict__ gb, const int base0, const int count) {
+                                   float *__restrict__ gw, const int base0, const int count) {
   const int H = Lp->H, W = Lp->W, K = Lp->K, OH = Lp->OH, OW = Lp->OW;
-  const int sh = Lp->sh, sw = Lp->sw, ph = Lp->ph, pw = Lp->pw, nb = Lp->nb;
+  const int sh = Lp->sh, sw = Lp->sw, ph = Lp->ph, pw = Lp->pw;
   const FastDiv d_taps = Lp->d_taps, d_s = Lp->d_s, d_c = Lp->d_c;
   const uint8_t *__restrict__ tbl = Lp->tbl;
   const int plane = OH * OW;
@@ -1087,7 +1087,14 @@ TN_INLINE void conv_bwd_param_rows(const TinyLayer *__restrict__ Lp, const float
       if (it < end && part == 0) gw[idx] = sum;
     }
   }
-  if (nb && base0 == 0) {
+}
+// the bias gradient of such a convolution, a job of its own (beside the first units of the weight
+// gradient it made that workgroup the last of the launch to finish): every plane of dY, a group
+// of lanes a channel
+template <int NT>
+TN_INLINE void conv_bwd_param_bias(const TinyLayer *__restrict__ Lp, const float *dy, float *__restrict__ gb) {
+  const int nb = Lp->nb, plane = Lp->OH * Lp->OW;
+  {
     int g = 64;
     while (g > 1 && (nb * g > 2 * NT || g > plane)) g >>= 1;
     const int total = nb * g, gs = __ffs(g) - 1;
@@ -1273,12 +1280,17 @@ tiny_net_param_kernel(const TinyPlan *__restrict__ plan, const float *__restrict
     else conv_bwd_dx_scalar_any<3, 3, TP_THREADS>(L, framed, nullptr, gdx, nullptr, job.base, job.base + job.count, 1);
     return;
   }
+  if (job.what == 2) {   // a convolution's bias gradient: dY alone
+    fill_lds<TP_THREADS>(lds, gdy, out_sz);
+    lds_barrier();
+    conv_bwd_param_bias<TP_THREADS>(L, lds, L->gb + static_cast<size_t>(s) * L->nb);
+    return;
+  }
   float *in = lds, *dy = lds + ((in_sz + 3) & ~3);
   fill_lds<TP_THREADS>(in, gin, in_sz);
-  // (a convolution's weight-gradient units name the output channels whose gradient planes they
-  // read; the units from 0 on also add up the bias gradient of every channel)
+  // (a convolution's weight-gradient units name the output channels whose gradient planes they read)
   int dy_lo = 0, dy_n = out_sz;
-  if (kind == TDH_L_CONV && !conv_is_matvec(*L) && job.base != 0) {
+  if (kind == TDH_L_CONV && !conv_is_matvec(*L)) {
     const int gs = __ffs(conv_param_group(*L)) - 1, plane = L->OH * L->OW;
     const int co_lo = static_cast<int>(L->d_nk.div(job.base >> gs));
     const int co_hi = static_cast<int>(L->d_nk.div((job.base + job.count - 1) >> gs));
@@ -1292,7 +1304,7 @@ tiny_net_param_kernel(const TinyPlan *__restrict__ plan, const float *__restrict
   switch (kind) {
     case TDH_L_CONV:
       if (conv_is_matvec(*L)) conv_bwd_param_matvec<TP_THREADS>(L, in, dy, gw, gb, job.base, job.count);
-      else conv_bwd_param_rows<TP_THREADS>(L, in, dy, gw, gb, job.base, job.count);
+      else conv_bwd_param_rows<TP_THREADS>(L, in, dy, gw, job.base, job.count);
       break;
     case TDH_L_FC: fc_bwd_param<TP_THREADS>(L, in, dy, gw, gb, job.base, job.count); break;
     case TDH_L_AVEPOOL: avepool_bwd_param<TP_THREADS>(L, in, dy, gw, gb); break;
@@ -1331,7 +1343,7 @@ int tiny_build_jobs(TinyPlan &P) {
   // units of work per layer and the units one workgroup takes: a lane's item for the grouped
   // sums, sixteen elements per lane for the element-wise products, a wave's item for the dX
   struct Piece { int layer, what, units, per_job; };
-  Piece pieces[TINY_MAX_LAYERS + 1];
+  Piece pieces[2 * TINY_MAX_LAYERS + 1];
   int n_pieces = 0;
   size_t lds = 0, framed = 0;
   for (int i = 0; i < P.n; ++i) {
@@ -1353,7 +1365,10 @@ int tiny_build_jobs(TinyPlan &P) {
     }
     if (!L.nw) continue;
     lds = std::max(lds, static_cast<size_t>(((L.in_size + 3) & ~3) + ((L.out_size + 3) & ~3)));
-    if (L.kind == TDH_L_CONV && !conv_is_matvec(L)) pieces[n_pieces++] = {i, 0, L.nw * conv_param_group(L), TP_THREADS};
+    if (L.kind == TDH_L_CONV && !conv_is_matvec(L)) {
+      pieces[n_pieces++] = {i, 0, L.nw * conv_param_group(L), TP_THREADS};
+      if (L.nb) pieces[n_pieces++] = {i, 2, 1, 1};
+    }
     else if (L.kind == TDH_L_CONV || L.kind == TDH_L_FC) pieces[n_pieces++] = {i, 0, L.nw, 16 * TP_THREADS};
     else pieces[n_pieces++] = {i, 0, 1, 1};
   }
