@@ -35,6 +35,7 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 PER_KERNEL_PASSES = 2
+STEPS_PER_CALL = 8   # train steps a call of the network workloads' timed region
 
 
 def load_pkg():
@@ -57,7 +58,8 @@ class NetWorkload:
         self.samples = self.batch
         self.config = {"workload": name, "batch": self.batch, "loss": self.loss,
                        "optimizer": self.opt_kind, "step": "fwd+bwd+update",
-                       "launch": "captured HIP graph (per-kernel pass runs the same kernels eagerly)",
+                       "launch": f"captured HIP graphs of {STEPS_PER_CALL} steps each (tdh_net_train_steps; the "
+                                 "per-kernel pass runs the same kernels eagerly, step by step)",
                        "flop_per_step": 3 * self.batch * W.flops_per_sample(self.spec)}
 
         self.host_x, self.host_t = x, t
@@ -65,6 +67,16 @@ class NetWorkload:
 
     def step(self):
         self.net.train_step(self.opt, self.loss, self.batch, self.x, self.t)
+
+    def run(self, n):
+        """n steps, STEPS_PER_CALL at a time (tdh_net_train_steps: one captured graph holds them, so
+        a replay starts once for all of them), the rest one by one."""
+        k = STEPS_PER_CALL
+        xs, ts = [self.x] * k, [self.t] * k
+        for _ in range(n // k):
+            self.net.train_steps(self.opt, self.loss, self.batch, xs, ts)
+        for _ in range(n % k):
+            self.step()
 
     def step_from_host(self):
         """The same step when the caller hands over host buffers: inputs and targets cross PCIe,
@@ -147,6 +159,14 @@ def roofline_of(entry):
 WARM_MS = 100.0
 
 
+def run_steps(wl, n):
+    if hasattr(wl, "run"):
+        wl.run(n)
+    else:
+        for _ in range(n):
+            wl.step()
+
+
 def warm_by_time(T, wl, min_ms=WARM_MS):
     """Runs untimed steps until the device has been busy for `min_ms`: a GPU that has idled (a
     CPU leg, a fresh process) clocks down, and a timed region of a few milliseconds would
@@ -154,8 +174,7 @@ def warm_by_time(T, wl, min_ms=WARM_MS):
     done, spent, chunk = 0, 0.0, 4
     while spent < min_ms and done < 100000:
         t0 = time.perf_counter()
-        for _ in range(chunk):
-            wl.step()
+        run_steps(wl, chunk)
         T.sync()
         spent += (time.perf_counter() - t0) * 1e3
         done += chunk
@@ -164,18 +183,23 @@ def warm_by_time(T, wl, min_ms=WARM_MS):
 
 
 def run_workload(T, wl, steps, warmup, profile_steps, sequence=None):
-    for _ in range(warmup):
-        wl.step()
+    run_steps(wl, warmup)
     T.sync()
     warm_by_time(T, wl)
     e0, e1 = T.Event(), T.Event()
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(steps):
-        wl.step()
+    run_steps(wl, steps)
     e1.record()
     T.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
+    single_ms = None
+    if hasattr(wl, "run"):   # the same steps one call each, for comparison
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            wl.step()
+        T.sync()
+        single_ms = (time.perf_counter() - t0) * 1e3 / steps
     gpu_ms = e1.elapsed_ms_since(e0)
     ms_per_step = wall_ms / steps
     # second pass: per-kernel durations, stamped by the dispatches themselves. A network workload
@@ -212,7 +236,7 @@ def run_workload(T, wl, steps, warmup, profile_steps, sequence=None):
     kernels = [roofline_of(e) for e in prof]
     for k, e in zip(kernels, prof):
         k["ms_per_step"] = round(e["total_ms"] / profile_steps, 4)
-    return {"ms_per_step": ms_per_step, "gpu_ms_per_step": gpu_ms / steps,
+    return {"ms_per_step": ms_per_step, "gpu_ms_per_step": gpu_ms / steps, "single_step_calls_ms": single_ms,
             "samples_per_s": wl.samples / (ms_per_step * 1e-3), "kernels": kernels,
             "profile_steps": profile_steps}
 
@@ -356,6 +380,10 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": wl.config,
         "device": {"name": dev_name, "compute_units": cus},
+        "one_step_per_call": None if res["single_step_calls_ms"] is None else
+        {"ms_per_step": round(res["single_step_calls_ms"], 4),
+         "samples_per_s": round(wl.samples / (res["single_step_calls_ms"] * 1e-3), 2),
+         "note": "the same steps through tdh_net_train_step, one captured graph replayed per step"},
         "roofline": dict(res["kernels"][0]) if res["kernels"] else None,
         "kernels": res["kernels"],
     }
@@ -386,13 +414,11 @@ def main():
         # never `value` either: the same step without the gradient of the net's input, which the
         # reference computes and training never reads (the caller's choice: TDH_NET_NO_INPUT_GRAD)
         w3 = NetWorkload(T, W, args.workload, T.NET_NO_INPUT_GRAD)
-        for _ in range(max(2, args.warmup)):
-            w3.step()
+        run_steps(w3, max(2, args.warmup))
         T.sync()
         warm_by_time(T, w3)
         t0 = time.perf_counter()
-        for _ in range(args.steps):
-            w3.step()
+        run_steps(w3, args.steps)
         T.sync()
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
         out["no_input_grad"] = {"ms_per_step": round(ms, 4), "samples_per_s": round(w3.samples / (ms * 1e-3), 2),
@@ -423,6 +449,7 @@ def main():
             flop_k = [k for k in ks if k["bound"] == "mfma"]
             rec = {"samples_per_s": round(r["samples_per_s"], 2),
                    "ms_per_step": round(r["ms_per_step"], 4), "steps": other_steps,
+                   "one_step_per_call_ms": None if r["single_step_calls_ms"] is None else round(r["single_step_calls_ms"], 4),
                    "config": w2.config,
                    "step_tflops": round(w2.config["flop_per_step"] / (r["ms_per_step"] * 1e-3) / 1e12, 3),
                    "roofline": {k: ks[0][k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac",

@@ -345,6 +345,16 @@ int tdh_net_forward(tdh_net *net, int batch, const float *x);
 /* fprop, loss gradient, bprop and (do_update != 0) update_weights + clear_grads */
 int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
                        const float *t, int do_update);
+/* n_steps (1 to 8) consecutive train steps with update, step s on the mini-batch x[s], t[s]
+ * (arrays of device pointers, which may repeat): what the loop over mini-batches of
+ * network::fit does (tiny_dnn/network.h:866-879, one train_once per mini-batch) when the
+ * batches are on the device already. The results are those of n_steps calls of
+ * tdh_net_train_step; with TDH_NET_GRAPH the steps are captured into one graph, so a replay
+ * starts once for all of them (a few microseconds each time, which is a tenth of a LeNet-5
+ * step). A net with a dropout layer in the train phase is refused: its masks change between
+ * the steps (tdh_net_set_dropout_mask). */
+int tdh_net_train_steps(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, int n_steps,
+                        const float *const *x, const float *const *t);
 
 /* ------------------------------------------------ batches from host memory */
 /* network::fit hands each mini-batch over as host vectors (tiny_dnn/network.h:866-879;

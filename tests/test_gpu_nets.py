@@ -283,6 +283,40 @@ def test_smaller_batch_than_max_and_forward_only(T, O, W):
     net.close()
 
 
+@pytest.mark.parametrize("name,batch,flags", [("cifar10_cnn_b128", 16, 3), ("cifar10_cnn_b128", 16, 1),
+                                              ("lenet5_b16", 16, 7), ("lenet5_b16", 16, 3), ("lenet5_mnist_b16", 8, 0)])
+def test_several_steps_in_one_call_equal_single_steps(T, W, name, batch, flags):
+    """tdh_net_train_steps: up to eight steps a call (one captured graph with TDH_NET_GRAPH), on
+    batches that change from step to step, leave bit for bit the weights of as many single steps;
+    adam's powers keep taking turns between their two buffers across calls of odd length."""
+    spec, params, x, t, batch, loss, opt_kind, opt_kw = W.make_batch(name, batch=batch)
+    nets = [T.Net(W.build_layers(T, spec), batch, flags) for _ in range(2)]
+    for net in nets:
+        for (i, which, a) in params:
+            net.set_param(i, which, a)
+    opts = [T.opt_desc(opt_kind, **opt_kw) for _ in range(2)]
+    rng = np.random.default_rng(17)
+    batches = []
+    for k in range(3):   # three mini-batches that take turns
+        p = rng.permutation(batch)
+        batches.append((T.to_device(np.ascontiguousarray(x[p] * np.float32(1.0 - 0.1 * k))), T.to_device(np.ascontiguousarray(t[p]))))
+    at = 0
+    for n in (3, 2, 5, 1, 8, 3):
+        use = [batches[(at + s) % 3] for s in range(n)]
+        at += n
+        nets[0].train_steps(opts[0], loss, batch, [b[0] for b in use], [b[1] for b in use])
+        for (xb, tb) in use:
+            nets[1].train_step(opts[1], loss, batch, xb, tb)
+        for (i, which, _) in params:
+            assert np.array_equal(nets[0].get_param(i, which), nets[1].get_param(i, which)), \
+                f"{name} flags {flags}: parameter {i}.{which} after a call of {n} steps"
+        assert opts[0].b1_t == opts[1].b1_t and opts[0].b2_t == opts[1].b2_t
+    with pytest.raises(T.TdhError, match="steps a call"):
+        nets[0].train_steps(opts[0], loss, batch, [batches[0][0]] * 9, [batches[0][1]] * 9)
+    for net in nets:
+        net.close()
+
+
 def test_net_rejects_inconsistent_layers(T):
     with pytest.raises(T.TdhError, match="expects"):
         T.Net([T.L_fc(10, 5), T.L_fc(6, 2)], 4)

@@ -627,3 +627,11 @@ class Net:
         check(lib().tdh_net_train_step(self.h, C.byref(opt) if opt is not None else None,
                                        LOSS[loss], batch, _p(x), _p(t), int(do_update)),
               "tdh_net_train_step")
+
+    def train_steps(self, opt, loss, batch, xs, ts):
+        """len(xs) consecutive train steps with update, step s on (xs[s], ts[s]); with NET_GRAPH one
+        captured graph holds them all (tdh_net_train_steps)."""
+        n = len(xs)
+        px = (C.c_void_p * n)(*[x.ptr.value for x in xs])
+        pt = (C.c_void_p * n)(*[t.ptr.value for t in ts])
+        check(lib().tdh_net_train_steps(self.h, C.byref(opt), LOSS[loss], batch, n, px, pt), "tdh_net_train_steps")

@@ -2,6 +2,7 @@
 // network<sequential>::train_onebatch (tiny_dnn/network.h:911-926) = fprop
 // (nodes.h:288-303), loss gradient (loss_function.h:191-218), bprop (nodes.h:276-286) and
 // update_weights (nodes.h:103-107, layer.h:663-682), queued on the library stream.
+#include <algorithm>
 #include <cstring>
 #include <vector>
 
@@ -48,10 +49,12 @@ struct tdh_net {
   int powers_at = 0;
   // partial sums and tickets of the one-launch kernel of two closing fully-connected layers
   float *tail_partials = nullptr, *tail_tickets = nullptr;
+  static constexpr int kMaxSteps = 8;   // train steps one captured graph may hold (tdh_net_train_steps)
   struct GraphKey {
     int batch = 0, loss = 0, do_update = 0, test_phase = 0;
-    int powers_at = 0;                  // which buffer of the powers the captured optimizer reads
-    const float *x = nullptr, *t = nullptr;
+    int powers_at = 0;                  // which buffer of the powers the (first) captured optimizer launch reads
+    int n_steps = 1;
+    const float *x[kMaxSteps] = {}, *t[kMaxSteps] = {};
     const void *scratch = nullptr;      // the library scratch buffer the captured kernels use
     tdh_opt hyper = {};                 // hyper-parameters only (powers zeroed)
   };
@@ -1206,18 +1209,16 @@ static bool same_key(const tdh_net::GraphKey &a, const tdh_net::GraphKey &b) {
   // field by field: a caller's tdh_opt may carry padding or unused fields it never wrote
   const tdh_opt &p = a.hyper, &q = b.hyper;
   return a.batch == b.batch && a.loss == b.loss && a.do_update == b.do_update && a.test_phase == b.test_phase &&
-         a.powers_at == b.powers_at &&
-         a.x == b.x &&
-         a.t == b.t && a.scratch == b.scratch && p.kind == q.kind && p.alpha == q.alpha &&
+         a.powers_at == b.powers_at && a.n_steps == b.n_steps &&
+         std::equal(a.x, a.x + a.n_steps, b.x) && std::equal(a.t, a.t + a.n_steps, b.t) && a.scratch == b.scratch && p.kind == q.kind && p.alpha == q.alpha &&
          p.lambda == q.lambda && p.mu == q.mu && p.b1 == q.b1 && p.b2 == q.b2 && p.eps == q.eps;
 }
 
-int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
-                       const float *t, int do_update) {
-  TDH_REQUIRE_INIT();
-  TDH_CHECK_ARG(net && x && t && batch > 0 && batch <= net->max_batch,
-                "tdh_net_train_step: bad argument");
-  TDH_CHECK_ARG(!do_update || opt, "tdh_net_train_step: update requested without an optimizer");
+// n_steps train steps, step s on the batch (xs[s], ts[s]): launched one after the other, or
+// captured into one graph and replayed
+static int train_steps(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, int n_steps, const float *const *xs,
+                       const float *const *ts, int do_update) {
+  const float *x = xs[0], *t = ts[0];
   // The filters in the stride-1 kernels' layout: packed here when the weights came from
   // outside (creation, tdh_net_set_param, a pointer handed out), by the optimizer kernel after
   // that.
@@ -1233,12 +1234,17 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   if (!(net->flags & TDH_NET_GRAPH) || profiling_active()) {
     // (the timing pass of a branching step keeps every layer's scratch piece until the optimizer
     // has read the split sums: the buffer must not grow, and so move, on the way)
-    if (net->flags & TDH_NET_GRAPH) TDH_TRY(ws_begin(net->scratch));
-    return enqueue_step(net, opt, loss_kind, batch, x, t, do_update, nullptr, nullptr);
+    for (int s = 0; s < n_steps; ++s) {
+      if (net->flags & TDH_NET_GRAPH) TDH_TRY(ws_begin(net->scratch));
+      TDH_TRY(enqueue_step(net, opt, loss_kind, batch, xs[s], ts[s], do_update, nullptr, nullptr));
+    }
+    return TDH_OK;
   }
 
   tdh_net::GraphKey key;
-  key.batch = batch; key.loss = loss_kind; key.do_update = do_update; key.x = x; key.t = t;
+  key.batch = batch; key.loss = loss_kind; key.do_update = do_update;
+  key.n_steps = n_steps;
+  for (int s = 0; s < n_steps; ++s) { key.x[s] = xs[s]; key.t[s] = ts[s]; }
   key.test_phase = net->test_phase;
   // (only steps that advance the powers take turns between the two buffers)
   const bool powers_move = opt && do_update && (opt->kind == TDH_OPT_ADAM || opt->kind == TDH_OPT_ADAMAX);
@@ -1275,9 +1281,13 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
     if (e == hipSuccess) {
       tdh_opt capture_opt;
       if (opt) capture_opt = *opt;
-      rc = enqueue_step(net, opt ? &capture_opt : nullptr, loss_kind, batch, x, t, do_update,
-                        net->dev_powers + 4 * key.powers_at, net->dev_powers + 4 * (1 - key.powers_at),
-                        /*forked=*/net_forks(net, batch));
+      for (int s = 0; s < n_steps && rc == TDH_OK; ++s) {
+        // (steps that advance the powers take turns between the two buffers inside the graph as well)
+        const int at = powers_move ? (key.powers_at + s) & 1 : key.powers_at;
+        rc = enqueue_step(net, opt ? &capture_opt : nullptr, loss_kind, batch, xs[s], ts[s], do_update,
+                          net->dev_powers + 4 * at, net->dev_powers + 4 * (1 - at),
+                          /*forked=*/net_forks(net, batch));
+      }
       e = hipStreamEndCapture(c.stream, &graph);
     }
     c.ws_locked = false;
@@ -1312,7 +1322,7 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
   net->out_unwritten = slot->out_unwritten;
   if (opt && do_update) {
     // advance the host object exactly as the eager path does
-    for (int j = 0; j < net->opt_tensors; ++j) {
+    for (int j = 0; j < net->opt_tensors * n_steps; ++j) {
       if (opt->kind == TDH_OPT_ADAM) {
         opt->b1_t *= opt->b1;
         opt->b2_t *= opt->b2;
@@ -1322,9 +1332,32 @@ int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, con
     }
     net->mirror_b1_t = opt->b1_t;
     net->mirror_b2_t = opt->b2_t;
-    if (powers_move) net->powers_at = 1 - net->powers_at;  // where this step left them
+    if (powers_move) net->powers_at = (net->powers_at + n_steps) & 1;  // where the last step left them
   }
   return TDH_OK;
+}
+
+int tdh_net_train_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, const float *x,
+                       const float *t, int do_update) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && x && t && batch > 0 && batch <= net->max_batch,
+                "tdh_net_train_step: bad argument");
+  TDH_CHECK_ARG(!do_update || opt, "tdh_net_train_step: update requested without an optimizer");
+  return train_steps(net, opt, loss_kind, batch, 1, &x, &t, do_update);
+}
+
+int tdh_net_train_steps(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, int n_steps,
+                        const float *const *x, const float *const *t) {
+  TDH_REQUIRE_INIT();
+  TDH_CHECK_ARG(net && opt && x && t && batch > 0 && batch <= net->max_batch && n_steps >= 1 &&
+                n_steps <= tdh_net::kMaxSteps, "tdh_net_train_steps: bad argument (1 to %d steps a call)",
+                tdh_net::kMaxSteps);
+  for (int s = 0; s < n_steps; ++s) TDH_CHECK_ARG(x[s] && t[s], "tdh_net_train_steps: null batch %d", s);
+  // a dropout layer's masks are handed over once per step, between the steps
+  for (const tdh_net::Layer &L : net->layers)
+    TDH_CHECK_ARG(L.spec.kind != TDH_L_DROPOUT || net->test_phase,
+                  "tdh_net_train_steps: a net with a dropout layer trains one step a call");
+  return train_steps(net, opt, loss_kind, batch, n_steps, x, t, 1);
 }
 
 }  // extern "C"
