@@ -284,7 +284,8 @@ def test_smaller_batch_than_max_and_forward_only(T, O, W):
 
 
 @pytest.mark.parametrize("name,batch,flags", [("cifar10_cnn_b128", 16, 3), ("cifar10_cnn_b128", 16, 1),
-                                              ("lenet5_b16", 16, 7), ("lenet5_b16", 16, 3), ("lenet5_mnist_b16", 8, 0)])
+                                              ("lenet5_b16", 16, 7), ("lenet5_b16", 16, 3), ("lenet5_mnist_b16", 8, 0),
+                                              ("cifar10_cnn_b128", 16, 3 | 8), ("lenet5_b16", 5, 7 | 8)])
 def test_several_steps_in_one_call_equal_single_steps(T, W, name, batch, flags):
     """tdh_net_train_steps: up to eight steps a call (one captured graph with TDH_NET_GRAPH), on
     batches that change from step to step, leave bit for bit the weights of as many single steps;
