@@ -37,6 +37,14 @@ struct TinyLayer {
   // tiny_net.hip): where in LDS the step kernel keeps the filters as [co][k] (k = (ci, tap), rows
   // padded with zeros), the input offset of every k and a copy of the bias; -1: the scalar loops
   int mf_fwd_w, mf_fwd_ko, mf_fwd_b;
+  // The input gradient of the layer whose filters wait in registers (TinyPlan::mf_ahead), from the
+  // framed dY, as the same kind of product with the filter columns folded into the rows:
+  //   D[(ci, wx)][iy][px] = sum over (co, wy) of W[co][ci][wy][wx] * framed[co][iy + R-1-wy][px]
+  // (C * S rows, K * R terms a sum, every position of H framed rows a column), then
+  //   dX[ci][iy][ix] = sum over wx of D[(ci, wx)][iy][ix + S-1-wx].
+  // mf_dx_w / mf_dx_ko: the operand [(ci, wx)][(co, wy)] and its offset table, written into the
+  // scratch area in front of the phase; mf_dx_d: D. -1: the scalar loops.
+  int mf_dx_w, mf_dx_ko, mf_dx_d;
 };
 
 // One workgroup's share of the parameter-gradient kernel for one sample: the units

@@ -688,6 +688,7 @@ TN_INLINE void conv_bwd_dx_scalar_any(const TinyLayer *__restrict__ Lp, const fl
 // zeros from n_k on, `koff` the input offset of every k < 4 * steps, `bias` the bias or NULL,
 // all in LDS (stage_mfma_operands); steps is a multiple of four.
 typedef float tn_f4 __attribute__((ext_vector_type(4)));
+constexpr int MFMA_AHEAD = 4;   // filter values a thread holds for the layer whose filters wait in registers
 __host__ __device__ inline int mfma_steps(const int n_k) { return ((n_k + 15) >> 4) << 2; }
 // (a row pitch of 4 * odd floats: sixteen rows read 16 bytes each from different banks, two rows a bank group)
 __host__ __device__ inline int mfma_pitch(const int n_k) { return (4 * mfma_steps(n_k)) | 4; }
@@ -753,11 +754,56 @@ TN_INLINE void conv_mfma(const float *src, const float *a, const int *koff, cons
         const int p = (pi * T + j) * 16 + r;
         if (p < plane) {
           const float v = bias ? acc[j][i] + bv : acc[j][i];
-          out[m * plane + p]  = v;
-          gout[m * plane + p] = v;
+          out[m * plane + p] = v;
+          if (gout) gout[m * plane + p] = v;
         }
       }
     }
+  }
+}
+// The operand and the offset table of the input gradient described at TinyLayer::mf_dx_w, from
+// the filter values the thread still holds (mfma_filters_load: value j is element
+// e0 + j * TN_THREADS + thread of the weight tensor), the rows' ends zeroed.
+TN_INLINE void mfma_dx_operand_store(const TinyLayer *__restrict__ L, const float (&v)[MFMA_AHEAD], float *lds) {
+  const int C = L->C, K = L->K, R = L->R, S = L->S, taps = R * S, nw = K * C * taps;
+  const int n_k = K * R, pitch = mfma_pitch(n_k), k4 = 4 * mfma_steps(n_k), rows = C * S;
+  const int PW = L->W + S - 1, PP = (L->H + R - 1) * PW;
+  const uint8_t *__restrict__ tbl = L->tbl;
+  float *a = lds + L->mf_dx_w;
+  int *ko  = reinterpret_cast<int *>(lds + L->mf_dx_ko);
+#pragma unroll
+  for (int j = 0; j < MFMA_AHEAD; ++j) {
+    const int e = j * TN_THREADS + threadIdx.x;
+    if (e >= nw) continue;
+    uint32_t pair, t, co, ci, wy, wx;
+    L->d_taps.divmod(e, pair, t);
+    L->d_c.divmod(pair, co, ci);
+    L->d_s.divmod(t, wy, wx);
+    a[(ci * S + wx) * pitch + co * R + wy] = (tbl && !tbl[ci * K + co]) ? 0.0f : v[j];
+  }
+  const int pad = pitch - n_k;
+  for (int idx = threadIdx.x; idx < rows * pad; idx += TN_THREADS) {
+    const int row = idx / pad;
+    a[row * pitch + n_k + idx - row * pad] = 0.0f;
+  }
+  for (int k = threadIdx.x; k < k4; k += TN_THREADS) {
+    const int co = k / R, wy = k - co * R;
+    ko[k] = k < n_k ? co * PP + (R - 1 - wy) * PW : 0;
+  }
+}
+// dX from D (TinyLayer::mf_dx_d): the filter columns' shifted sums, in column order
+TN_INLINE void mfma_dx_gather(const TinyLayer *__restrict__ L, const float *d, float *dx, float *__restrict__ gdx) {
+  const int C = L->C, H = L->H, W = L->W, S = L->S, PW = W + S - 1, cols = H * PW;
+  const FastDiv d_iplane = L->d_iplane, d_w = L->d_w;
+  for (int e = threadIdx.x; e < C * H * W; e += TN_THREADS) {
+    uint32_t ci, r, iy, ix;
+    d_iplane.divmod(e, ci, r);
+    d_w.divmod(r, iy, ix);
+    const float *row = d + (ci * S) * cols + iy * PW + ix + S - 1;
+    float sum = 0.0f;
+    for (int wx = 0; wx < S; ++wx) sum += row[wx * cols - wx];
+    dx[e] = sum;
+    if (gdx) gdx[e] = sum;
   }
 }
 // The operands above for a layer that has them, straight from the weight tensor. Every filter
@@ -765,7 +811,6 @@ TN_INLINE void conv_mfma(const float *src, const float *a, const int *koff, cons
 // channels that a connection table leaves unconnected get a zero, and so do the ends of the
 // rows. In two halves, so that the reads can be in flight while other layers run: the first
 // asks for up to MFMA_AHEAD values a thread, the second puts them in LDS.
-constexpr int MFMA_AHEAD = 4;
 TN_INLINE void mfma_filters_load(const TinyLayer *__restrict__ L, const int e0, float (&v)[MFMA_AHEAD], float &bias) {
   const int nw = L->K * L->C * L->R * L->S;
 #pragma unroll
@@ -1220,6 +1265,9 @@ tiny_net_step_kernel(const TinyPlan *__restrict__ plan, const int loss, const in
   for (int li = first_bwd; li >= last_bwd; --li) {
     const TinyLayer *__restrict__ L = &plan->l[li];
     const int kind = L->kind, in_sz = L->in_size;
+    // (the layer in front of this one in memory order is the next to run: its operand goes into
+    // the scratch area now, which this phase does not use when that is so; see tiny_build_jobs)
+    if (li - 1 == ahead && ahead > 0 && plan->l[ahead].mf_dx_w >= 0) mfma_dx_operand_store(&plan->l[ahead], ahead_w, lds);
     float *gdx = L->dx ? L->dx + static_cast<size_t>(s) * in_sz : nullptr;
     switch (kind) {
       case TDH_L_CONV:
@@ -1233,7 +1281,17 @@ tiny_net_step_kernel(const TinyPlan *__restrict__ plan, const int loss, const in
           stage_framed_dy<TN_THREADS>(L, ga, framed);
           lds_barrier();
           const int items = conv_dx_scalar_items(*L), parts = scalar_parts(items, L->K, TN_WAVES);
-          if (L->R == 5) conv_bwd_dx_scalar_any<5, 5, TN_THREADS>(L, framed, gb, gdx, wl, 0, items * parts, parts);
+          if (L->mf_dx_w >= 0) {
+            // (the operand was written into the scratch area while the layer behind ran; D has every
+            // position of H framed rows as a column, so a column's offset is its index)
+            float *dd = lds + L->mf_dx_d;
+            const int PW = L->W + L->S - 1, cols = L->H * PW;
+            conv_mfma<2>(framed, lds + L->mf_dx_w, reinterpret_cast<const int *>(lds + L->mf_dx_ko), L->C * L->S,
+                         L->K * L->R, cols, L->d_pw, PW, nullptr, dd, nullptr);
+            lds_barrier();
+            mfma_dx_gather(L, dd, gb, gdx);
+          }
+          else if (L->R == 5) conv_bwd_dx_scalar_any<5, 5, TN_THREADS>(L, framed, gb, gdx, wl, 0, items * parts, parts);
           else conv_bwd_dx_scalar_any<3, 3, TN_THREADS>(L, framed, gb, gdx, wl, 0, items * parts, parts);
         }
         break;
@@ -1398,6 +1456,27 @@ int tiny_build_jobs(TinyPlan &P) {
         P.mfma_layers[P.n_mfma++] = i;
         if (P.mf_ahead < 0 && i > 0 && L.K * n_k <= MFMA_AHEAD * TN_THREADS) P.mf_ahead = i;
       }
+    }
+  }
+  for (int i = 0; i < P.n; ++i) P.l[i].mf_dx_w = P.l[i].mf_dx_ko = P.l[i].mf_dx_d = -1;
+  if (P.mf_ahead > 0 && P.mf_ahead + 1 < P.n) {
+    // the input gradient of that layer on the matrix cores: its operand goes into the scratch
+    // area while the layer behind it runs its backward phase, which therefore must be one that
+    // leaves that area alone (a pointwise activation or a pool), and D needs room of its own
+    TinyLayer &L = P.l[P.mf_ahead];
+    const TinyLayer &behind = P.l[P.mf_ahead + 1];
+    // (not a closing softmax either: under cross_entropy_multiclass its backward phase is skipped)
+    const bool quiet = (behind.kind == TDH_L_ACT && behind.act != TDH_ACT_SOFTMAX) || behind.kind == TDH_L_MAXPOOL ||
+                       behind.kind == TDH_L_AVEPOOL;
+    const int n_k = L.K * L.R, rows = L.C * L.S, cols = L.H * (L.W + L.S - 1);
+    const size_t operand = static_cast<size_t>(mfma_pitch(n_k)) * rows + 4 * mfma_steps(n_k);
+    const int at = (P.lds_floats + 3) & ~3;
+    if (L.dx_framed && quiet && operand <= TINY_SCRATCH_FLOATS &&
+        at + static_cast<size_t>(rows) * cols <= TINY_LDS_MAX_BYTES / sizeof(float)) {
+      L.mf_dx_w  = P.lds_w;
+      L.mf_dx_ko = P.lds_w + mfma_pitch(n_k) * rows;
+      L.mf_dx_d  = at;
+      P.lds_floats = at + rows * cols;
     }
   }
   for (int scale = 1;; scale *= 2) {
