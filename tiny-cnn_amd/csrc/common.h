@@ -412,8 +412,10 @@ int fc_softmax_xent(int in, int out, int has_bias, int batch, const float *x, co
 // act_out: also writes act(y) there (tanh / relu / sigmoid), the activation layer behind the pool
 int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int32_t *argmax,
                 float *act_out = nullptr, int act_kind = TDH_ACT_NONE);
+// pooled_y: the pool's forward output, or NULL (with an activation gradient folded in, ag, the 2x2
+// kernel reads it instead of the activation output)
 int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
-                float *dx, ActGrad ag = ActGrad());
+                float *dx, ActGrad ag = ActGrad(), const float *pooled_y = nullptr);
 int avepool_fwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *b,
                 float *y);
 int avepool_bwd(const tdh_pool_desc *d, int batch, const float *x, const float *w, const float *dy,

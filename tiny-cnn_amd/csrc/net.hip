@@ -1136,7 +1136,7 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           through_pool_for = i - 1;
           break;
         }
-        TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold));
+        TDH_TRY(maxpool_bwd(&s.pool, batch, L.dout, L.argmax, dx, fold, L.out));
         break;
       case TDH_L_AVEPOOL:
         TDH_TRY(ws_begin(avepool_workspace_bytes(&s.pool, batch)));

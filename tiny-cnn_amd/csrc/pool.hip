@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(PT)
 maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ argmax,
                       float *__restrict__ dx, const int pairs, const int W, const int OW2,
                       const FastDiv div_ow2, const int rows_per_sample, const ActGrad ag,
-                      const SplitSum sum) {
+                      const SplitSum sum, const float *__restrict__ pooled_y) {
   const int t = blockIdx.x * PT + threadIdx.x;
   if (t >= pairs) return;
   uint32_t row, ox2;
@@ -142,6 +142,19 @@ maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ 
   }
   const int2 a    = *reinterpret_cast<const int2 *>(argmax + o);
   const int base  = (static_cast<int>(2 * row) % rows_per_sample) * W + 4 * static_cast<int>(ox2);
+  const size_t at = static_cast<size_t>(2 * row) * W + 4 * ox2;
+  if (pooled_y) {
+    // The activation in front of the pool: dx *= act'(its output), and the only element of a
+    // window that gets a gradient is the one the pool passed on, so the pool's own output is
+    // that activation output: a quarter of the reads. (A window none of whose elements exceeds
+    // lowest() is recorded as element 0 of the sample, maxpool_op_internal.h:28-36: that element
+    // gets the gradient if the window is the sample's first, and its own value decides.)
+    const float2 pv = *reinterpret_cast<const float2 *>(pooled_y + o);
+    float fx = act_grad_factor(ag.kind, pv.x);
+    if (base == 0 && a.x == 0) fx = act_grad_factor(ag.kind, ag.y[at]);
+    g.x *= fx;
+    g.y *= act_grad_factor(ag.kind, pv.y);
+  }
   float4 r0, r1;
   r0.x = a.x == base ? g.x : 0.0f;
   r0.y = a.x == base + 1 ? g.x : 0.0f;
@@ -151,8 +164,7 @@ maxpool2x2_bwd_kernel(const float *__restrict__ dy, const int32_t *__restrict__ 
   r1.y = a.x == base + W + 1 ? g.x : 0.0f;
   r1.z = a.y == base + W + 2 ? g.y : 0.0f;
   r1.w = a.y == base + W + 3 ? g.y : 0.0f;
-  const size_t at = static_cast<size_t>(2 * row) * W + 4 * ox2;
-  if (ag.kind != TDH_ACT_NONE) {  // the activation layer in front of the pool: dx *= act'(its output)
+  if (!pooled_y && ag.kind != TDH_ACT_NONE) {  // the activation layer in front of the pool: dx *= act'(its output)
     const float4 y0 = *reinterpret_cast<const float4 *>(ag.y + at);
     const float4 y1 = *reinterpret_cast<const float4 *>(ag.y + at + W);
     r0.x *= act_grad_factor(ag.kind, y0.x); r0.y *= act_grad_factor(ag.kind, y0.y);
@@ -352,7 +364,7 @@ int maxpool_fwd(const tdh_pool_desc *d, int batch, const float *x, float *y, int
 }
 
 int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_t *argmax,
-                float *dx, ActGrad ag) {
+                float *dx, ActGrad ag, const float *pooled_y) {
   const PoolGeom g = make_geom(d);
   const long total = static_cast<long>(batch) * g.C * g.H * g.W;
   const bool fast  = is_2x2_tiling(g) && aligned16(dx) && aligned8(dy) && aligned8(argmax) &&
@@ -363,24 +375,26 @@ int maxpool_bwd(const tdh_pool_desc *d, int batch, const float *dy, const int32_
                     left_split_sum().out == dy && left_split_sum().stride == out_total;
   if (!take) TDH_TRY(finish_split_sum());
   TDH_CHECK_ARG(g.OH > 0 && g.OW > 0, "maxpool backward: empty output");
+  // (the pool's own output stands in for the activation output where a gradient lands)
+  const float *py = (ag.kind != TDH_ACT_NONE && pooled_y && aligned8(pooled_y)) ? pooled_y : nullptr;
   if (take) {
     const SplitSum sum   = left_split_sum();
     ctx().split_sum_left = false;
     ProfScope prof(ag.kind != TDH_ACT_NONE ? "maxpool_bwd_act_sum" : "maxpool_bwd_sum",
                    4.0 * out_total * (sum.splits + 2 + (sum.ag.kind != TDH_ACT_NONE)) +
-                     (ag.kind != TDH_ACT_NONE ? 8.0 : 4.0) * total, WORK_BYTE);
+                     (ag.kind == TDH_ACT_NONE ? 4.0 : py ? 5.0 : 8.0) * total, WORK_BYTE);
     const int pairs = static_cast<int>(total / 8);
     TDH_LAUNCH(maxpool2x2_bwd_kernel<true>, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy, argmax, dx,
-               pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag, sum);
+               pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag, sum, py);
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
   ProfScope prof(ag.kind != TDH_ACT_NONE ? "maxpool_bwd_act" : "maxpool_bwd",
-                 8.0 * batch * g.C * g.OH * g.OW + (ag.kind != TDH_ACT_NONE ? 8.0 : 4.0) * total, WORK_BYTE);
+                 8.0 * batch * g.C * g.OH * g.OW + (ag.kind == TDH_ACT_NONE ? 4.0 : (fast && py) ? 5.0 : 8.0) * total, WORK_BYTE);
   if (fast) {
     const int pairs = static_cast<int>(total / 8);
     TDH_LAUNCH(maxpool2x2_bwd_kernel<false>, dim3(ceil_div(pairs, PT)), dim3(PT), 0, ctx().stream, dy,
-                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag, SplitSum());
+                       argmax, dx, pairs, g.W, g.OW / 2, FastDiv(g.OW / 2), g.C * g.H, ag, SplitSum(), py);
     TDH_LAUNCH_CHECK();
     return TDH_OK;
   }
