@@ -189,6 +189,42 @@ def test_conv_weight_gradient_of_8x8_images_options(T, O):
     assert_close(dbs.numpy(), rdb, what="db of unaligned tensors")
 
 
+@pytest.mark.parametrize("w_,h_,c_,k_,oc_,same,batch", [
+    (32, 32, 3, 5, 32, True, 128),    # the CIFAR net's first layer
+    (32, 32, 3, 5, 20, True, 80),     # 20 of 32 output channels, a batch that is no multiple of anything
+    (36, 36, 3, 5, 32, False, 64),    # no padding: 32 x 32 outputs under 36 input rows, five bands
+    (32, 20, 3, 3, 16, True, 96),     # 3x3, a last band of four rows
+    (16, 16, 1, 5, 8, True, 256),     # one input channel, rows of 16, one band an image
+])
+def test_first_conv_gradients_from_one_launch(T, O, w_, h_, c_, k_, oc_, same, batch):
+    """dX, dW and db of a first convolution (few input channels, at most 32 output channels, a
+    workgroup for every compute unit) leave one launch when they are asked for together: each
+    against the oracle, the same bits as the three asked for one by one, and dW / db added to a
+    previous value."""
+    rng = np.random.default_rng(w_ * 7 + h_ + c_ + k_ + oc_)
+    d, do = T.conv_desc(w_, h_, c_, k_, k_, oc_, pad_same=same), O.conv_desc(w_, h_, c_, k_, k_, oc_, pad_same=same)
+    ow, oh = (w_, h_) if same else (w_ - k_ + 1, h_ - k_ + 1)
+    x = rng.standard_normal((batch, c_ * w_ * h_)).astype(np.float32)
+    w = rng.uniform(-0.2, 0.2, oc_ * c_ * k_ * k_).astype(np.float32)
+    dy = rng.standard_normal((batch, oc_ * ow * oh)).astype(np.float32)
+    rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
+    xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)
+    dx, dw, db = T.DevBuf(x.shape), T.DevBuf(w.shape), T.DevBuf((oc_,))
+    T.conv2d_bwd(d, batch, xd, wd, dyd, dx, dw, db)
+    assert_close(dx.numpy(), rdx, what="dX"); assert_close(dw.numpy(), rdw, what="dW"); assert_close(db.numpy(), rdb, what="db")
+    dx1, dw1, db1 = T.DevBuf(x.shape), T.DevBuf(w.shape), T.DevBuf((oc_,))
+    T.conv2d_bwd(d, batch, xd, wd, dyd, dx1, None, None)
+    T.conv2d_bwd(d, batch, xd, wd, dyd, None, dw1, db1)
+    assert np.array_equal(dx.numpy(), dx1.numpy()), "dX alone"
+    assert np.array_equal(dw.numpy(), dw1.numpy()), "dW without dX"
+    assert np.array_equal(db.numpy(), db1.numpy()), "db without dX"
+    dw0 = rng.standard_normal(w.size).astype(np.float32)
+    dw2, dx2 = T.to_device(dw0), T.to_device(np.full(x.shape, np.nan, np.float32))
+    T.conv2d_bwd(d, batch, xd, wd, dyd, dx2, dw2, None, True)     # no bias gradient, added to dw0
+    assert_close(dw2.numpy(), rdw + dw0, what="dW added to a previous value")
+    assert np.array_equal(dx2.numpy(), dx.numpy())
+
+
 def test_conv_errors_and_empty_batch(T):
     d = T.conv_desc(8, 8, 2, 3, 3, 4, w_dilation=2, h_dilation=2)
     buf = T.DevBuf((16,))

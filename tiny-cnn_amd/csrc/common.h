@@ -250,7 +250,8 @@ struct PoolGather {
 // (dy_pool set: dy is not read; the plan must pass conv_dw_small_reads_pooled)
 int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy, float *dw_out,
                       float *db_out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
-                      int dw, int ph, int pw, int accumulate, const PoolGather *dy_pool = nullptr);
+                      int dw, int ph, int pw, int accumulate, const PoolGather *dy_pool = nullptr,
+                      int force_band = 0);
 bool conv_dw_small_reads_pooled(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
                                 int sh, int sw, int dh, int dw, int ph, int pw);
 // the weight-gradient kernel of this layer also produces the bias gradient when asked for both
@@ -307,6 +308,9 @@ struct PoolFuse {
 int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *b,
                float *y, const uint8_t *tbl_resident = nullptr, const float *prepacked = nullptr,
                float *act_out = nullptr, int act_kind = 0, const PoolFuse *pool = nullptr);
+// dX, dW and db of this (first) convolution leave conv2d_bwd as one launch when all three are
+// asked for together (pooled: the gradient is read through the max-pool behind the layer)
+bool conv_bwd_one_launch(const tdh_conv_desc *d, int batch, bool pooled);
 // the forward kernel of this convolution can also compute the max-pool layer `pool` behind it
 bool conv_fwd_fuses_pool(const tdh_conv_desc *d, const tdh_pool_desc *pool, int batch, bool prepacked);
 // ... and the pointwise activation of this kind behind that pool

@@ -492,6 +492,23 @@ constexpr int DXM_MCH   = 32;  // output channels staged at a time
 constexpr int DXM_MAXCH = 16;  // channels a thread stages (of DXM_MCH)
 constexpr int DXM_WREG  = 13;  // filter values a thread stages per chunk (32 channels x 4 x 25 / 256)
 
+// The weight (and bias) gradient of the same layer out of the same launch (DWNT > 0: the
+// number of 32-column blocks of its product, Cin*KH*KW + 1 columns, the last one the bias):
+//   dW[co][(ci,ky,kx)] = sum over the band's output positions of dY[co][p] * X[ci][p + (ky,kx)]
+// reads the staged rows of dY a second time, as the A operand of v_mfma_f32_32x32x2_f32 (lane =
+// (output channel, one of two positions)), and the input patch under the band, staged next to
+// them, as B (one LDS read at patch[position] + offset(column), the offset a per-lane
+// constant). The four waves split the band's positions, their sums meet in LDS and the
+// workgroup writes one slice [band][co][column] that a split reduction adds to the others.
+// Reference: conv2d_op_internal.h:127-180.
+struct FirstDwArgs {
+  const float *x;
+  float *partial_dw, *partial_db;  // [bands of the batch][Kc][crs], [..][Kc] (or null)
+  int pitch, plane, rows_in;       // the staged patch: floats per row (odd) and channel, rows
+  int x_total;                     // its elements
+  FastDiv div_pitch, div_rows_in;
+};
+
 template <int KR, int NMB, bool POOLED>
 struct DxmGeom {
   static constexpr int OW        = 16 * NMB;
@@ -513,13 +530,14 @@ struct DxmGeom {
   static constexpr bool FITS = GROUPS >= 1 && CPT <= DXM_MAXCH && LDS_FLOATS * 4 <= 64 * 1024;
 };
 
-template <int KR, int KS, int NMB, bool POOLED>
-__global__ void __launch_bounds__(DXM_NT)
+template <int KR, int KS, int NMB, bool POOLED, int DWNT = 0>
+__global__ void __launch_bounds__(DXM_NT, DWNT > 0 ? 2 : 1)
 conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict__ w, float *__restrict__ dx,
-                          const ConvGeom g, const ActGrad ag, const PoolGather pooled) {
+                          const ConvGeom g, const ActGrad ag, const PoolGather pooled, const FirstDwArgs dwa) {
   using G = DxmGeom<KR, NMB, POOLED>;
   extern __shared__ __align__(16) float smem[];
   typedef float f4 __attribute__((ext_vector_type(4)));
+  typedef float f16 __attribute__((ext_vector_type(16)));
   constexpr int RS = KR * KS, NJ = 2 * KR;  // step j: filter row j/2, channels 4*(j%2) + (0..3) of eight
   constexpr int OW = G::OW, PLANE = G::PLANE;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -575,6 +593,23 @@ conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict_
   const float *abase = smem + mq * PLANE + wv * (G::RPW * OW) + mr;
   const int crs      = g.C * RS;
 
+  // ---- the weight gradient's side: column n of block t belongs to lane n % 32
+  constexpr int NT_ = DWNT > 0 ? DWNT : 1;
+  constexpr int XDEPTH = 8;
+  f16 wacc[NT_];
+  int woff[NT_];
+  bool wone[NT_];
+  float *xs = smem + G::STAGE;  // the input patch [ci][rows_in][pitch]
+  if constexpr (DWNT > 0) {
+#pragma unroll
+    for (int t = 0; t < DWNT; ++t) {
+      const int n  = t * 32 + (lane & 31);
+      const int ci = n / RS, tap = n - ci * RS;
+      wone[t] = n == crs;
+      woff[t] = n < crs ? ci * dwa.plane + (tap / KS) * dwa.pitch + tap % KS : 0;
+    }
+  }
+
   for (int co0 = 0; co0 < g.Kc; co0 += DXM_MCH) {
     // ---- everything this chunk needs from memory, asked for together
     float sv[POOLED ? DXM_MAXCH : 1];
@@ -596,6 +631,32 @@ conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict_
     const int nw = min(DXM_MCH, g.Kc - co0) * crs;
 #pragma unroll
     for (int k = 0; k < DXM_WREG; ++k) wreg[k] = w[static_cast<size_t>(co0) * crs + min(tid + DXM_NT * k, nw - 1)];
+    // the input patch under the band (zero where the window leaves the image): the first
+    // XDEPTH elements of a thread travel with the loads above
+    float xv[XDEPTH];
+    int xo[XDEPTH];
+    auto load_x = [&](int e0) {
+#pragma unroll
+      for (int k = 0; k < XDEPTH; ++k) {
+        const int e = e0 + k * DXM_NT;
+        xv[k] = 0.0f;
+        xo[k] = -1;
+        if (e < dwa.x_total) {
+          const int rr = dwa.div_pitch.div(e), cx = e - rr * dwa.pitch;
+          const int ci = dwa.div_rows_in.div(rr), r = rr - ci * dwa.rows_in;
+          const int iy = y0 - g.pad_h + r, ix = cx - g.pad_w;
+          xo[k] = ci * dwa.plane + r * dwa.pitch + cx;
+          if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W)
+            xv[k] = dwa.x[(static_cast<size_t>(img * g.C + ci) * g.H + iy) * g.W + ix];
+        }
+      }
+    };
+    auto store_x = [&]() {
+#pragma unroll
+      for (int k = 0; k < XDEPTH; ++k)
+        if (xo[k] >= 0) xs[xo[k]] = xv[k];
+    };
+    if constexpr (DWNT > 0) load_x(tid);
     if (co0 > 0) __syncthreads();  // the previous chunk has been consumed
     // filters: element e = (co, ci, tap) of memory goes to [co][ci][tap] with four ci slots
 #pragma unroll
@@ -626,6 +687,13 @@ conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict_
         }
       }
     }
+    if constexpr (DWNT > 0) {
+      store_x();
+      for (int e0 = tid + XDEPTH * DXM_NT; e0 < dwa.x_total; e0 += XDEPTH * DXM_NT) {
+        load_x(e0);
+        store_x();
+      }
+    }
     __syncthreads();
     // ---- products: eight staged channels per pass, the four blocks of the wave side by side
 #pragma unroll
@@ -641,6 +709,65 @@ conv_dx_first_mfma_kernel(const float *__restrict__ dy, const float *__restrict_
           dacc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(
             abase[(8 * sub + 4 * (j & 1)) * PLANE + ((b / NMB) + (j >> 1)) * OW + 16 * (b % NMB)], breg[j], dacc[b], 0,
             0, 0);
+    }
+    if constexpr (DWNT > 0) {
+      // ---- the weight gradient's products: output rows y0 .. of the band, which the staged
+      //      rows hold from row KR-1-pad on; a half wave takes four consecutive positions a trip
+      // (one chunk of output channels: the sums start here, behind everything the staging held)
+#pragma unroll
+      for (int t = 0; t < DWNT; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wacc[t][i] = 0.0f;
+      const int half  = lane >> 5;
+      const int units = max(min(G::TILE_ROWS, g.OH - y0), 0) * (OW / 4);
+      const float *arow = smem + (lane & 31) * PLANE + (KR - 1 - g.pad_h) * OW;
+      for (int it = 0; it < (units + 7) / 8; ++it) {
+        const int u   = it * 8 + wv * 2 + half;
+        const bool ok = u < units;
+        const int pos = ok ? 4 * u : 0;
+        f4 av         = *reinterpret_cast<const f4 *>(arow + pos);
+        if (!ok) av = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        const float *xb = xs + (pos / OW) * dwa.pitch + pos % OW;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int t = 0; t < DWNT; ++t) {
+            float b = xb[j + woff[t]];
+            b       = wone[t] ? 1.0f : b;
+            wacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], b, wacc[t], 0, 0, 0);
+          }
+      }
+    }
+  }
+
+  if constexpr (DWNT > 0) {
+    // ---- the four waves' sums meet in LDS (over the staged rows, which are done with) and
+    //      leave as one slice, added in wave order
+    constexpr int TILE = 32 * 32 * DWNT;
+    __syncthreads();
+    float *red = smem + wv * TILE;
+#pragma unroll
+    for (int t = 0; t < DWNT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        red[((i >> 2) * 8 + (lane >> 5) * 4 + (i & 3)) * (32 * DWNT) + t * 32 + (lane & 31)] = wacc[t][i];
+    __syncthreads();
+    float sums[TILE / DXM_NT];
+#pragma unroll
+    for (int i = 0; i < TILE / DXM_NT; ++i) {
+      const int e = tid + DXM_NT * i;
+      sums[i]     = (smem[e] + smem[TILE + e]) + (smem[2 * TILE + e] + smem[3 * TILE + e]);
+    }
+    // (a slice per band of OUTPUT rows: without padding the last bands of input rows have none)
+    const int wbands = (g.OH + G::TILE_ROWS - 1) / G::TILE_ROWS, band = wg - img * bands;
+    const size_t slice = static_cast<size_t>(img) * wbands + band;
+#pragma unroll
+    for (int i = 0; i < TILE / DXM_NT; ++i) {
+      const int e = tid + DXM_NT * i;
+      const int m = e / (32 * DWNT), n = e - m * (32 * DWNT);
+      if (band >= wbands || m >= g.Kc || n > crs) continue;
+      if (n < crs) dwa.partial_dw[(slice * g.Kc + m) * crs + n] = sums[i];
+      else if (dwa.partial_db) dwa.partial_db[slice * g.Kc + m] = sums[i];
     }
   }
 
@@ -686,7 +813,43 @@ static bool launch_first_dx_mfma_inst(const ConvGeom &g, int batch, const float 
     if (only_ask) return true;
     const int bands = ceil_div(g.H, G::TILE_ROWS);
     TDH_LAUNCH((conv_dx_first_mfma_kernel<KR, KR, NMB, POOLED>), dim3(batch * bands), dim3(DXM_NT),
-               sizeof(float) * G::LDS_FLOATS, ctx().stream, dy, w, dx, g, ag, pooled);
+               sizeof(float) * G::LDS_FLOATS, ctx().stream, dy, w, dx, g, ag, pooled, FirstDwArgs());
+    return true;
+  }
+}
+
+// ... and of the instance that also computes the weight and bias gradient; dwa comes in without
+// its patch geometry, which depends on the instance's band
+template <int KR, int NMB, bool POOLED, int DWNT>
+static bool launch_first_both_inst(const ConvGeom &g, int batch, const float *dy, const float *w, float *dx,
+                                   ActGrad ag, PoolGather pooled, FirstDwArgs dwa, bool only_ask) {
+  using G = DxmGeom<KR, NMB, POOLED>;
+  if constexpr (!G::FITS) {
+    return false;
+  } else {
+    const int bands = ceil_div(g.H, G::TILE_ROWS);
+    // every output row lies in the staged rows of the band that starts at the same row
+    if (g.H < G::TILE_ROWS || g.OH > bands * G::TILE_ROWS || g.pad_h > KR - 1) return false;
+    dwa.pitch   = (g.OW + KR - 1) | 1;  // odd: the taps of one column fall into different LDS banks
+    dwa.rows_in = G::TILE_ROWS + KR - 1;
+    dwa.plane   = dwa.rows_in * dwa.pitch + 1;
+    dwa.x_total = g.C * dwa.rows_in * dwa.pitch;
+    dwa.div_pitch   = FastDiv(dwa.pitch);
+    dwa.div_rows_in = FastDiv(dwa.rows_in);
+    const size_t x_floats = (static_cast<size_t>(g.C) * dwa.plane + 3) & ~static_cast<size_t>(3);
+    const size_t floats   = std::max<size_t>(G::STAGE + x_floats, std::max<size_t>(G::GATHER, 4u * 32 * 32 * DWNT));
+    if (floats * sizeof(float) > 76 * 1024) return false;  // (two workgroups a compute unit)
+    if (only_ask) return true;
+    auto kernel = conv_dx_first_mfma_kernel<KR, KR, NMB, POOLED, DWNT>;
+    static bool raised = false;
+    if (!raised) {  // more than the 64 KB a kernel may use without asking
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              76 * 1024) != hipSuccess)
+        return false;
+      raised = true;
+    }
+    TDH_LAUNCH(kernel, dim3(batch * bands), dim3(DXM_NT), sizeof(float) * floats, ctx().stream, dy, w, dx, g, ag,
+               pooled, dwa);
     return true;
   }
 }
@@ -708,6 +871,33 @@ static bool first_dx_mfma(const ConvGeom &g, int batch, const float *dy, const f
     default: return false;
   }
 #undef TDH_DXM
+}
+
+// dX, dW and db of a first convolution in one launch: where the matrix-core dX kernel applies,
+// the layer has at most 32 output channels (one staged chunk) and an instance exists for its
+// window and channel count, and every compute unit gets a workgroup. Returns whether it applies
+// (only_ask) / has been launched; band_rows: the rows of a band (one slice per band and image).
+template <bool POOLED>
+static bool first_bwd_both(const ConvGeom &g, int batch, const float *dy, const float *w, float *dx, ActGrad ag,
+                           PoolGather pooled, FirstDwArgs dwa, bool only_ask, int *band_rows) {
+  if (g.Kc > DXM_MCH || g.R != g.S || batch > 65535) return false;
+  if (!first_dx_mfma<POOLED>(g, batch, dy, w, dx, ag, pooled, true)) return false;
+  if (!only_ask && !POOLED && (reinterpret_cast<uintptr_t>(dy) & 15)) return false;
+  const int nt = ceil_div(g.C * g.R * g.S + 1, 32);
+  const int nmb = g.OW / 16;
+  const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+#define TDH_BOTH(KR_, NMB_, NT_) \
+  (*band_rows = DxmGeom<KR_, NMB_, POOLED>::TILE_ROWS, \
+   static_cast<long>(batch) * ceil_div(g.H, *band_rows) >= cus && \
+   launch_first_both_inst<KR_, NMB_, POOLED, NT_>(g, batch, dy, w, dx, ag, pooled, dwa, only_ask))
+  if (g.R == 5 && nt == 3 && nmb == 2) return TDH_BOTH(5, 2, 3);
+  if (g.R == 5 && nt == 3 && nmb == 1) return TDH_BOTH(5, 1, 3);
+  if (g.R == 5 && nt == 1 && nmb == 2) return TDH_BOTH(5, 2, 1);
+  if (g.R == 5 && nt == 1 && nmb == 1) return TDH_BOTH(5, 1, 1);
+  if (g.R == 3 && nt == 1 && nmb == 2) return TDH_BOTH(3, 2, 1);
+  if (g.R == 3 && nt == 1 && nmb == 1) return TDH_BOTH(3, 1, 1);
+#undef TDH_BOTH
+  return false;
 }
 
 // true when the direct kernel applies; fills the launch geometry
@@ -767,6 +957,8 @@ static bool fwd_small_applies(const ConvGeom &g, int batch) {
 
 }  // namespace
 
+static size_t first_both_workspace_bytes(const tdh_conv_desc *d, const ConvGeom &g, int batch);
+
 size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   const ConvGeom g = make_geom(d);
   const int ohw = g.OH * g.OW, crs = g.C * g.R * g.S;
@@ -778,6 +970,7 @@ size_t conv2d_workspace_bytes(const tdh_conv_desc *d, int batch) {
   if (d->tbl) total += ws_align(static_cast<size_t>(g.C) * g.Kc) + 2 * ws_align(sizeof(float) * g.Kc * crs);
   total += conv_dw_small_workspace_bytes(batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw,
                                          g.dh, g.dw, g.pad_h, g.pad_w);
+  total += first_both_workspace_bytes(d, g, batch);
   if (g.sh == 1 && g.sw == 1)
     total += conv_dw_halo_workspace_bytes(g.R, g.S, batch, g.C, g.Kc, g.H, g.W, g.OH, g.OW, g.pad_h, g.pad_w);
   if (g.sh == 1 && g.sw == 1) {  // LDS-halo kernel: repacked filters and split partial sums
@@ -1000,6 +1193,69 @@ int conv2d_fwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   return launch_gemm<true, false>(A, B, epi, g.Kc, batch * ohw, crs, true, "conv_fwd_gemm", "conv_fwd_splitk_reduce");
 }
 
+// the rows of a band of the launch that computes dX, dW and db of this layer together, or 0
+static int one_launch_band(const tdh_conv_desc *d, const ConvGeom &g, int batch, bool pooled) {
+  if (d->tbl) return 0;
+  int rows = 0;
+  const bool ok =
+      pooled ? first_bwd_both<true>(g, batch, nullptr, nullptr, nullptr, ActGrad(), PoolGather(), FirstDwArgs(), true, &rows)
+             : first_bwd_both<false>(g, batch, nullptr, nullptr, nullptr, ActGrad(), PoolGather(), FirstDwArgs(), true, &rows);
+  return ok ? rows : 0;
+}
+bool conv_bwd_one_launch(const tdh_conv_desc *d, int batch, bool pooled) {
+  return one_launch_band(d, make_geom(d), batch, pooled) > 0;
+}
+
+// the slices of that launch: one per band and image
+static size_t first_both_workspace_bytes(const tdh_conv_desc *d, const ConvGeom &g, int batch) {
+  size_t most = 0;
+  for (int pooled = 0; pooled < 2; ++pooled) {
+    const int rows = one_launch_band(d, g, batch, pooled != 0);
+    if (!rows) continue;
+    const size_t blocks = static_cast<size_t>(batch) * ceil_div(g.OH, rows);
+    most = std::max(most, ws_align(blocks * g.Kc * g.C * g.R * g.S * sizeof(float)) + ws_align(blocks * g.Kc * sizeof(float)));
+  }
+  return most;
+}
+
+// dX, dW and (optionally) db of a first convolution as one launch plus the split reduction of
+// its slices; the caller has asked conv_bwd_one_launch
+template <bool POOLED>
+static int run_first_both(const ConvGeom &g, int batch, const float *x, const float *dy, const float *w, float *dx,
+                          float *dw, float *db, int accumulate, ActGrad dx_act, PoolGather pooled) {
+  const int crs = g.C * g.R * g.S;
+  int rows = 0;
+  if (!first_bwd_both<POOLED>(g, batch, dy, w, dx, dx_act, pooled, FirstDwArgs(), true, &rows))
+    return set_error(TDH_ERR_INVALID, "conv2d_bwd: the one-launch kernel does not apply");
+  const int blocks = batch * ceil_div(g.OH, rows);
+  void *pw_ws = nullptr, *pb_ws = nullptr;
+  TDH_TRY(ws_take(static_cast<size_t>(blocks) * g.Kc * crs * sizeof(float), &pw_ws));
+  if (db) TDH_TRY(ws_take(static_cast<size_t>(blocks) * g.Kc * sizeof(float), &pb_ws));
+  FirstDwArgs dwa{};
+  dwa.x = x;
+  dwa.partial_dw = static_cast<float *>(pw_ws);
+  dwa.partial_db = static_cast<float *>(pb_ws);
+  {
+    ProfScope prof("conv_bwd_first_both", 2.0 * batch * (static_cast<double>(g.C) * g.H * g.W * g.Kc * g.R * g.S +
+                                                         static_cast<double>(g.Kc) * (crs + (db ? 1 : 0)) * g.OH * g.OW),
+                   WORK_FLOP);
+    if (!first_bwd_both<POOLED>(g, batch, dy, w, dx, dx_act, pooled, dwa, false, &rows))
+      return set_error(TDH_ERR_HIP, "conv2d_bwd: the one-launch kernel could not be launched");
+    TDH_LAUNCH_CHECK();
+  }
+  EpiRowMajor epi_w{dw, crs, nullptr, ActGrad(), accumulate};
+  EpiRowMajor epi_b{db, 1, nullptr, ActGrad(), accumulate};
+  // the two reductions leave as one launch: collected by the train step, or here
+  const bool collect_here = !ctx().defer_reduce;
+  if (collect_here) flush_deferred_reduces(false);  // nothing may be left from a failed call
+  ctx().defer_reduce = true;
+  defer_reduce(dwa.partial_dw, blocks, g.Kc, crs, epi_w);
+  if (db) defer_reduce(dwa.partial_db, blocks, g.Kc, 1, epi_b);
+  if (!collect_here) return TDH_OK;
+  ctx().defer_reduce = false;
+  return flush_deferred_reduces();
+}
+
 int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w, const float *dy,
                float *dx, float *dw, float *db, int accumulate, ActGrad dx_act,
                const uint8_t *tbl_resident, const float *prepacked_dx, const PoolGather *dy_pool) {
@@ -1014,6 +1270,8 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
         (reinterpret_cast<uintptr_t>(dy_pool->g) & 7) || (reinterpret_cast<uintptr_t>(dy_pool->argmax) & 7) ||
         (db && !dw))
       return set_error(TDH_ERR_INVALID, "conv2d_bwd: the pooled gradient cannot be read for this layer");
+    if (dx && dw && conv_bwd_one_launch(d, batch, true))
+      return run_first_both<true>(g, batch, x, nullptr, w, dx, dw, db, accumulate, dx_act, *dy_pool);
     DxsPlan dxs;
     small_cin_dx_plan(g, dxs);
     if (dx) {
@@ -1027,8 +1285,10 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
       TDH_LAUNCH_CHECK();
     }
     if (dw)
+      // (with the bands of the launch that would also compute dX: the same sums either way)
       TDH_TRY(conv_dw_small_run(batch, g.C, g.Kc, x, nullptr, dw, db, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh,
-                                g.sw, g.dh, g.dw, g.pad_h, g.pad_w, accumulate, dy_pool));
+                                g.sw, g.dh, g.dw, g.pad_h, g.pad_w, accumulate, dy_pool,
+                                one_launch_band(d, g, batch, true)));
     return TDH_OK;
   }
   if (dx && prepacked_dx) {
@@ -1037,6 +1297,8 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
     dx = nullptr;
     if (!dw && !db) return TDH_OK;
   }
+  if (dx && dw && !prepacked_dx && !(reinterpret_cast<uintptr_t>(dy) & 15) && conv_bwd_one_launch(d, batch, false))
+    return run_first_both<false>(g, batch, x, dy, w, dx, dw, db, accumulate, dx_act, PoolGather());
   const uint8_t *tbl_dev;
   const float *w_eff;
   TDH_TRY(prepare_table(d, g, w, tbl_resident, &tbl_dev, &w_eff));
@@ -1064,7 +1326,7 @@ int conv2d_bwd(const tdh_conv_desc *d, int batch, const float *x, const float *w
   }
   if (dw && dw_small_applies(d, g, batch) && !(reinterpret_cast<uintptr_t>(dy) & 15)) {
     TDH_TRY(conv_dw_small_run(batch, g.C, g.Kc, x, dy, dw, db, g.H, g.W, g.OH, g.OW, g.R, g.S, g.sh, g.sw,
-                              g.dh, g.dw, g.pad_h, g.pad_w, accumulate));
+                              g.dh, g.dw, g.pad_h, g.pad_w, accumulate, nullptr, one_launch_band(d, g, batch, false)));
     return TDH_OK;
   }
   if (dw) {

@@ -267,9 +267,12 @@ struct DwSmallPlan {
   bool ok;
 };
 
-// even_rows: bands and chunks of an even number of rows (what the POOLED kernels need)
+// even_rows: bands and chunks of an even number of rows (what the POOLED kernels need);
+// force_band > 0: bands of that many rows (the bands of the kernel that computes this gradient
+// together with the layer's dX, so that the same sums come out with and without the dX)
 DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, int OW, int R, int S,
-                               int sh, int sw, int dh, int dw, int ph, int pw, bool even_rows = false) {
+                               int sh, int sw, int dh, int dw, int ph, int pw, bool even_rows = false,
+                               int force_band = 0) {
   DwSmallPlan p;
   p.ok = false;
   DwSmallArgs &a = p.a;
@@ -353,6 +356,11 @@ DwSmallPlan make_dw_small_plan(int batch, int C, int Kc, int H, int W, int OH, i
     if (even_rows && even % 2 != 0) ++even;
     best = std::min(best, even);
   }
+  if (force_band > 0) {
+    chunk_cap = std::max(1, 256 / OW);
+    if ((even_rows && force_band % 2 != 0) || lds_floats(force_band) * sizeof(float) > 72 * 1024) return p;
+    best = force_band;
+  }
   a.band    = best;
   a.bands   = ceil_div(OH, best);
   a.chunk   = chunk_of(best);
@@ -419,10 +427,16 @@ bool conv_dw_small_reads_pooled(int batch, int C, int Kc, int H, int W, int OH, 
 // dw (required) and db (optional) of one layer; both follow `accumulate`.
 int conv_dw_small_run(int batch, int C, int Kc, const float *x, const float *dy, float *dw_out,
                       float *db_out, int H, int W, int OH, int OW, int R, int S, int sh, int sw, int dh,
-                      int dw, int ph, int pw, int accumulate, const PoolGather *dy_pool) {
+                      int dw, int ph, int pw, int accumulate, const PoolGather *dy_pool, int force_band) {
   DwSmallPlan p = make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw, dy_pool != nullptr);
+  if (force_band > 0) {  // (the hint is dropped where the kernel cannot follow it)
+    const DwSmallPlan forced =
+        make_dw_small_plan(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw, dy_pool != nullptr, force_band);
+    if (forced.ok && forced.a.chunk * OW % 32 == 0) p = forced;
+  }
   if (dy_pool) {
-    if (!conv_dw_small_reads_pooled(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw) ||
+    if (!conv_dw_small_reads_pooled(batch, C, Kc, H, W, OH, OW, R, S, sh, sw, dh, dw, ph, pw) || p.a.band % 2 != 0 ||
+        p.a.chunk % 2 != 0 ||
         !dy_pool->g || !dy_pool->argmax || (reinterpret_cast<uintptr_t>(dy_pool->g) & 7) ||
         (reinterpret_cast<uintptr_t>(dy_pool->argmax) & 7))
       return set_error(TDH_ERR_INVALID, "conv_dw_small_run: the pooled gradient cannot be read for this shape");

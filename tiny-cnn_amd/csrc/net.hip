@@ -153,7 +153,13 @@ bool is_pointwise_act(int act) {
 // packing beside the main chain): mid-sized steps only. With tiny kernels the cross-queue
 // synchronisation costs more than it hides, and products that fill the chip for hundreds of
 // microseconds only fight the main chain for its caches (measured: LeNet-style net 5 % slower,
-// VGG-style 1 % slower, CIFAR-10-shape net 12 % faster with branches).
+// VGG-style 1 % slower with branches). In between, a branch point and a join cost a replayed
+// step about 5 us each, and what a branch buys depends on how the kernels fill the chip. The
+// CIFAR-10-shape net, us a step with / without branches: batch 16 138 / 149, 32 143 / 151,
+// 64 140 / 151, 128 181 / 177, 256 288 / 285, 512 517 / 541. Up to batch 64 its kernels leave
+// compute units idle that a branch fills; at 128 and 256 every kernel is about one full round
+// of workgroups, two kernels side by side only take turns, and the step is the sum of its
+// kernels either way; beyond, the rounds of one kernel overlap the tail of another again.
 double net_forward_flop(const tdh_net *net, int batch) {
   double macs = 0.0;
   for (const tdh_net::Layer &L : net->layers) {
@@ -173,16 +179,17 @@ bool net_skips_input_grad(const tdh_net *net) {
 
 bool net_forks(const tdh_net *net, int batch) {
   const double flop = net_forward_flop(net, batch);
-  return flop >= 1e8 && flop <= 3e10;
+  return flop >= 1e8 && flop <= 3e10 && !(flop >= 2.2e9 && flop < 1e10);
 }
 // A step too small to branch (LeNet-5 at batch 16) is a chain of launches of a few
-// microseconds each, and what counts is how many there are: it runs the branching step's
+// microseconds each, and what counts is how many there are (and so it is for a step inside
+// the window above that does not branch): it runs the branching step's
 // launches one after the other, so that the split sums of all weight gradients go to the
 // optimizer kernel and the row sums of all bias gradients leave as one pair of launches.
 // (With the graph flag only: a net created with it reserves every layer's scratch side by side.)
 bool net_defers_serially(const tdh_net *net, int batch) {
   return (net->flags & TDH_NET_GRAPH) && (net->flags & TDH_NET_FUSE_ACT_GRAD) &&
-         net_forward_flop(net, batch) < 1e8;
+         !net_forks(net, batch) && net_forward_flop(net, batch) <= 3e10;
 }
 
 // The plan of the one-workgroup-per-sample step (tiny_net.hip) for a net that qualifies: at most
@@ -1038,6 +1045,16 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
             break;
           }
           const bool db_with_dw = L.b_size && conv_dw_gives_db(&s.conv, batch);
+          if (i == 0 && dx && !wp && conv_bwd_one_launch(&s.conv, batch, gp != nullptr)) {
+            // the net's first layer, all its gradients from one launch (on the main stream,
+            // like the two launches below)
+            c.defer_reduce = true;
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1, fold,
+                               L.tbl_dev, nullptr, gp));
+            c.defer_reduce = false;
+            last_dw_on_main = true;
+            break;
+          }
           if (dx) {
             LeaveSplitSum leave(c, pool_reads);
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp, gp));
@@ -1070,6 +1087,13 @@ static int enqueue_step(tdh_net *net, tdh_opt *opt, int loss_kind, int batch, co
           }
         } else if (as_forked) {
           // the launches of the captured, branching step, one after the other
+          if (i == 0 && dx && !wp && conv_bwd_one_launch(&s.conv, batch, gp != nullptr)) {
+            c.defer_reduce = true;
+            TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, L.dw, L.b_size ? L.db : nullptr, 1, fold,
+                               L.tbl_dev, nullptr, gp));
+            c.defer_reduce = false;
+            break;
+          }
           if (dx) {
             LeaveSplitSum leave(c, pool_reads);
             TDH_TRY(conv2d_bwd(&s.conv, batch, in, L.w, L.dout, dx, nullptr, nullptr, 1, fold, L.tbl_dev, wp, gp));
