@@ -155,15 +155,16 @@ def test_conv_accumulate_and_skipped_outputs(T, O):
     assert_close(dwb.numpy(), rdw)
 
 
-def test_conv_weight_gradient_of_8x8_images_options(T, O):
-    """The 8x8-image dW kernel: added to a previous value, without a bias gradient, without dX,
-    twice with equal bits; tensors that are not 16-byte aligned take the general kernel."""
-    rng = np.random.default_rng(88)
-    bs, ic, oc = 9, 32, 64
-    d, do = T.conv_desc(8, 8, ic, 5, 5, oc, pad_same=True), O.conv_desc(8, 8, ic, 5, 5, oc, pad_same=True)
-    x = rng.standard_normal((bs, ic * 64)).astype(np.float32)
+@pytest.mark.parametrize("hw,bs,ic,oc", [(8, 9, 32, 64), (16, 97, 32, 32), (16, 128, 64, 32)])
+def test_conv_weight_gradient_of_whole_images_options(T, O, hw, bs, ic, oc):
+    """The dW kernel that stages whole 8x8 or 16x16 images (the latter from batch 96 on): added to
+    a previous value, without a bias gradient, without dX, twice with equal bits; tensors that
+    are not 16-byte aligned take the general kernel."""
+    rng = np.random.default_rng(88 + hw + bs)
+    d, do = T.conv_desc(hw, hw, ic, 5, 5, oc, pad_same=True), O.conv_desc(hw, hw, ic, 5, 5, oc, pad_same=True)
+    x = rng.standard_normal((bs, ic * hw * hw)).astype(np.float32)
     w = rng.uniform(-0.1, 0.1, oc * ic * 25).astype(np.float32)
-    dy = rng.standard_normal((bs, oc * 64)).astype(np.float32)
+    dy = rng.standard_normal((bs, oc * hw * hw)).astype(np.float32)
     dw0 = rng.standard_normal(w.size).astype(np.float32)
     rdx, rdw, rdb = O.conv2d_bwd(do, x, w, dy)
     xd, wd, dyd = T.to_device(x), T.to_device(w), T.to_device(dy)

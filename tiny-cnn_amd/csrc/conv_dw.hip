@@ -387,10 +387,20 @@ __global__ void __launch_bounds__(64 * WCO * WK * WFY, 1) conv_dw_halo_kernel(co
 // k = 1 lanes the right half. The four waves' sums meet in LDS (pairwise, image order), and the
 // whole workgroup stores the slice. The bias gradient comes from the workgroups of tap group 0
 // and input-channel block 0, out of the dY they stage anyway.
+//
+// 16x16 images (IS = 16) run the same way with ONE image a chunk: a wave takes four of its rows,
+// 64 pixels again, as eight groups of eight; with more than one chunk a workgroup the next
+// chunk's words travel while the current one is multiplied.
 constexpr int I8_NT  = 256;
-constexpr int I8_DYP = 4 * 64 + 4;    // floats per staged dY channel: four images (4 mod 64)
-constexpr int I8_XP  = 4 * 144 + 4;   // floats per staged X channel: four framed images (4 mod 64)
-constexpr int I8_LDS_FLOATS = 32 * I8_DYP + 32 * I8_XP;
+constexpr int I8_DYP = 4 * 64 + 4;    // floats per staged dY channel: 256 pixels (4 mod 64)
+// geometry of a chunk for images of IS x IS pixels
+template <int IS> struct I8Geom {
+  static constexpr int IPC   = IS == 8 ? 4 : 1;              // images a chunk
+  static constexpr int FP    = IS + 4;                       // framed row
+  static constexpr int XP    = IPC * FP * FP + 4;            // floats per staged X channel (4 mod 32 / 20 mod 32)
+  static constexpr int WAVEX = IS == 8 ? FP * FP : 4 * FP;   // a wave's first framed row: its image / its four rows
+  static constexpr int LDS_FLOATS = 32 * I8_DYP + 32 * XP;
+};
 
 struct DwImg8Args {
   const float *x, *dy;
@@ -408,18 +418,21 @@ template <int G> struct I8Taps {
   static constexpr int FY0 = T0 / 5, FY1 = (T0 + N - 1) / 5;
 };
 
-// the products of one image (the wave's) for tap group G: acc[t - T0] += dY x X shifted by tap t
-template <int G>
+// the products of the wave's 64 pixels (eight groups of eight: an image's rows, or halves of four
+// rows) for tap group G: acc[t - T0] += dY x X shifted by tap t
+template <int G, int IS>
 __device__ __forceinline__ void img8_products(const float *ap, const float *bp, floatx16 (&acc)[7]) {
   using TG = I8Taps<G>;
+  constexpr int FP = I8Geom<IS>::FP;
 #pragma unroll
-  for (int oy = 0; oy < 8; ++oy) {
-    const floatx4 a4 = *reinterpret_cast<const floatx4 *>(ap + oy * 8);
+  for (int u = 0; u < 8; ++u) {
+    const int oy = IS == 8 ? u : u >> 1, ox = IS == 8 ? 0 : 8 * (u & 1);
+    const floatx4 a4 = *reinterpret_cast<const floatx4 *>(ap + u * 8);
     const float av[4] = {a4.x, a4.y, a4.z, a4.w};
 #pragma unroll
     for (int fy = TG::FY0; fy <= TG::FY1; ++fy) {
-      const floatx4 b0 = *reinterpret_cast<const floatx4 *>(bp + (oy + fy) * 12);
-      const floatx4 b1 = *reinterpret_cast<const floatx4 *>(bp + (oy + fy) * 12 + 4);
+      const floatx4 b0 = *reinterpret_cast<const floatx4 *>(bp + (oy + fy) * FP + ox);
+      const floatx4 b1 = *reinterpret_cast<const floatx4 *>(bp + (oy + fy) * FP + ox + 4);
       const float bv[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
       for (int fx = 0; fx < 5; ++fx) {
@@ -433,7 +446,10 @@ __device__ __forceinline__ void img8_products(const float *ap, const float *bp, 
   }
 }
 
+template <int IS>
 __global__ void __launch_bounds__(I8_NT, 1) conv_dw_img8_kernel(const DwImg8Args a) {
+  using GE = I8Geom<IS>;
+  constexpr int I8_XP = GE::XP, IPC = GE::IPC, FP = GE::FP, PIX = IS * IS;
   extern __shared__ __align__(16) float smem[];
   float *dy_l = smem;                 // [32][I8_DYP]
   float *x_l  = smem + 32 * I8_DYP;   // [32][I8_XP], frames of zeros around the images
@@ -447,7 +463,7 @@ __global__ void __launch_bounds__(I8_NT, 1) conv_dw_img8_kernel(const DwImg8Args
   id /= a.co_blocks;
   const int cib = id % a.ci_blocks, slice = id / a.ci_blocks;
   const int co0 = cob * 32, ci0 = cib * 32;
-  const int kohw = a.Kc * 64, chw = a.C * 64;
+  const int kohw = a.Kc * PIX, chw = a.C * PIX;
 
   floatx16 acc[7];
 #pragma unroll
@@ -459,41 +475,49 @@ __global__ void __launch_bounds__(I8_NT, 1) conv_dw_img8_kernel(const DwImg8Args
 
   // fragment bases: A lane = (output channel l%32, half l/32), B lane = (input channel l%32, half)
   const float *ap = dy_l + (lane & 31) * I8_DYP + wave * 64 + 4 * (lane >> 5);
-  const float *bp = x_l + (lane & 31) * I8_XP + wave * 144 + 4 * (lane >> 5);
+  const float *bp = x_l + (lane & 31) * I8_XP + wave * GE::WAVEX + 4 * (lane >> 5);
 
   const int c_begin = slice * a.chunks_per_slice;
   const int c_end   = min(a.chunks_total, c_begin + a.chunks_per_slice);
-  for (int chunk = c_begin; chunk < c_end; ++chunk) {
-    // ---- stage four images: a thread moves eight 16-byte words of dY and eight of X, all
-    //      loads asked for before the first store (an image past the batch reads image 0 and is
-    //      stored as zeros)
-    floatx4 rdy[8], rx[8];
+  // ---- staging: a thread moves eight 16-byte words of dY and eight of X per chunk, all loads
+  //      asked for before the first store (an image past the batch reads image 0 and is stored
+  //      as zeros). Word e: IS = 8: image e / 512 of the chunk's four, channel (e / 16) % 32,
+  //      word e % 16 of its 64 pixels; IS = 16: channel e / 64, word e % 64 of the image.
+  floatx4 rdy[8], rx[8];
+  auto fetch = [&](int chunk) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int e = tid + I8_NT * i, im = e >> 9, c = (e >> 4) & 31, q = e & 15;
-      const int img = chunk * 4 + im;
+      const int e = tid + I8_NT * i;
+      const int im = IS == 8 ? e >> 9 : 0, c = IS == 8 ? (e >> 4) & 31 : e >> 6, q = IS == 8 ? e & 15 : e & 63;
+      const int img = chunk * IPC + im;
       const size_t ig = img < a.batch ? img : 0;
-      rdy[i] = *reinterpret_cast<const floatx4 *>(a.dy + ig * kohw + static_cast<size_t>(co0 + c) * 64 + 4 * q);
-      rx[i]  = *reinterpret_cast<const floatx4 *>(a.x + ig * chw + static_cast<size_t>(ci0 + c) * 64 + 4 * q);
+      rdy[i] = *reinterpret_cast<const floatx4 *>(a.dy + ig * kohw + static_cast<size_t>(co0 + c) * PIX + 4 * q);
+      rx[i]  = *reinterpret_cast<const floatx4 *>(a.x + ig * chw + static_cast<size_t>(ci0 + c) * PIX + 4 * q);
     }
+  };
+  fetch(c_begin);
+  for (int chunk = c_begin; chunk < c_end; ++chunk) {
     if (chunk == c_begin) {   // the frames of zeros, written while the first loads are on their way
       for (int i = tid; i < 32 * I8_XP / 4; i += I8_NT) reinterpret_cast<floatx4 *>(x_l)[i] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
     __syncthreads();   // (the previous chunk's fragments have been read; the first time: the zeros are in place)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int e = tid + I8_NT * i, im = e >> 9, c = (e >> 4) & 31, q = e & 15;
-      const bool on = chunk * 4 + im < a.batch;
+      const int e = tid + I8_NT * i;
+      const int im = IS == 8 ? e >> 9 : 0, c = IS == 8 ? (e >> 4) & 31 : e >> 6, q = IS == 8 ? e & 15 : e & 63;
+      const bool on = chunk * IPC + im < a.batch;
       const floatx4 z = floatx4{0.f, 0.f, 0.f, 0.f};
       *reinterpret_cast<floatx4 *>(dy_l + c * I8_DYP + im * 64 + 4 * q) = on ? rdy[i] : z;
-      // X row q/2, half q%2 -> framed row q/2 + 2, columns 2 + 4*(q%2) .. + 3 (8-byte aligned)
+      // X row, word of the row -> framed row + 2, columns 2 + 4 * word .. + 3 (8-byte aligned)
+      constexpr int WPR = IS / 4;   // words per image row
       const floatx4 v = on ? rx[i] : z;
-      float *d = x_l + c * I8_XP + im * 144 + ((q >> 1) + 2) * 12 + 2 + 4 * (q & 1);
+      float *d = x_l + c * I8_XP + im * (FP * FP) + ((q / WPR) + 2) * FP + 2 + 4 * (q % WPR);
       *reinterpret_cast<float2 *>(d)     = make_float2(v.x, v.y);
       *reinterpret_cast<float2 *>(d + 2) = make_float2(v.z, v.w);
     }
     __syncthreads();
-    if (sums_dy) {   // channel tid/8, floats (tid%8)*32 .. +31 of its four images
+    if (chunk + 1 < c_end) fetch(chunk + 1);   // (travels while this chunk is multiplied)
+    if (sums_dy) {   // channel tid/8, floats (tid%8)*32 .. +31 of its 256 pixels
       const floatx4 *row = reinterpret_cast<const floatx4 *>(dy_l + (tid >> 3) * I8_DYP + (tid & 7) * 32);
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
@@ -502,10 +526,10 @@ __global__ void __launch_bounds__(I8_NT, 1) conv_dw_img8_kernel(const DwImg8Args
       }
     }
     switch (grp) {
-      case 0: img8_products<0>(ap, bp, acc); break;
-      case 1: img8_products<1>(ap, bp, acc); break;
-      case 2: img8_products<2>(ap, bp, acc); break;
-      default: img8_products<3>(ap, bp, acc); break;
+      case 0: img8_products<0, IS>(ap, bp, acc); break;
+      case 1: img8_products<1, IS>(ap, bp, acc); break;
+      case 2: img8_products<2, IS>(ap, bp, acc); break;
+      default: img8_products<3, IS>(ap, bp, acc); break;
     }
   }
 
@@ -560,7 +584,8 @@ __global__ void __launch_bounds__(I8_NT, 1) conv_dw_img8_kernel(const DwImg8Args
 
 struct DwHaloPlan {
   bool ok;
-  bool img8;            // the 8x8-image kernel runs this shape
+  bool img8;            // the image-sized kernel runs this shape
+  int img_size;         // ... on images of 8x8 or 16x16 pixels
   DwImg8Args i8;
   int tc, wco, wk, wfy, nt;
   int rows_block;  // filter rows one workgroup covers
@@ -583,12 +608,17 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
   if (!(R == 3 && S == 3) && !five) return p;
   if (C < 16 || Kc < 16 || OW < 8 || OH < 2 || pw > 4) return p;
   p.img8 = false;
-  if (allow_img8 && five && H == 8 && W == 8 && OH == 8 && OW == 8 && ph == 2 && pw == 2 && C % 32 == 0 && Kc % 32 == 0 && batch >= 4 &&
-      static_cast<long>(batch) * std::max(C, Kc) * 64 < (1L << 30)) {
+  // (16x16 images: from the batch on where the chunks give every compute unit a workgroup; the
+  // kernel below has fewer, longer workgroups, which is what a step that runs it beside its
+  // main chain wants)
+  const int is = H == 8 ? 8 : 16;
+  if (allow_img8 && five && H == is && W == is && OH == is && OW == is && ph == 2 && pw == 2 && C % 32 == 0 &&
+      Kc % 32 == 0 && batch >= (is == 8 ? 4 : 96) && static_cast<long>(batch) * std::max(C, Kc) * is * is < (1L << 30)) {
     DwImg8Args &i = p.i8;
+    p.img_size = is;
     i.batch = batch; i.C = C; i.Kc = Kc;
     i.co_blocks = Kc / 32; i.ci_blocks = C / 32;
-    i.chunks_total = ceil_div(batch, 4);
+    i.chunks_total = is == 8 ? ceil_div(batch, 4) : batch;
     // one workgroup per compute unit where the batch allows it
     const int base = 4 * i.co_blocks * i.ci_blocks;
     int slices = std::max(1, 256 / base);
@@ -596,7 +626,7 @@ DwHaloPlan make_dw_plan(int R, int S, int batch, int C, int Kc, int H, int W, in
     i.chunks_per_slice = ceil_div(i.chunks_total, slices);
     p.slices = ceil_div(i.chunks_total, i.chunks_per_slice);
     p.grid   = dim3(static_cast<unsigned>(p.slices));   // (grid.x counts the slices, as below; the launch multiplies)
-    p.lds_bytes = sizeof(float) * I8_LDS_FLOATS;
+    p.lds_bytes = sizeof(float) * (is == 8 ? I8Geom<8>::LDS_FLOATS : I8Geom<16>::LDS_FLOATS);
     p.img8 = true;
     p.ok   = true;
     return p;
@@ -733,13 +763,15 @@ int conv_dw_halo_run(int R, int S, int batch, int C, int Kc, const float *x, con
     ProfScope prof(db ? "conv_dw_db_halo" : "conv_dw_halo", Kc, crs, batch * OH * OW);
     if (p.img8) {
       p.i8.x = x; p.i8.dy = dy; p.i8.partial = p.args.partial; p.i8.partial_db = p.args.partial_db;
-      static bool raised = false;
-      if (!raised) {
-        TDH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(conv_dw_img8_kernel),
+      static bool raised[2] = {false, false};
+      const int which = p.img_size == 8 ? 0 : 1;
+      void (*kernel)(const DwImg8Args) = which ? conv_dw_img8_kernel<16> : conv_dw_img8_kernel<8>;
+      if (!raised[which]) {
+        TDH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(p.lds_bytes)));
-        raised = true;
+        raised[which] = true;
       }
-      TDH_LAUNCH(conv_dw_img8_kernel, dim3(p.slices * p.i8.ci_blocks * p.i8.co_blocks * 4), dim3(I8_NT), p.lds_bytes,
+      TDH_LAUNCH(kernel, dim3(p.slices * p.i8.ci_blocks * p.i8.co_blocks * 4), dim3(I8_NT), p.lds_bytes,
                  ctx().stream, p.i8);
       TDH_LAUNCH_CHECK();
     } else if (vec) {
