@@ -175,9 +175,9 @@ def check_every_layer(net, ref, spec, batch, name, fused, passes=1, cancelling_d
 
 def test_cifar_net_at_the_benchmarked_batch_and_flags_matches_oracle(T, O, W):
     """configs[3] exactly as bench.py runs it: batch 128, folded activation gradients, the step
-    captured into a graph whose weight-gradient kernels run on side streams with deferred split
-    reductions. Every layer's output, argmax, dW, db and dX, then the parameters after each of
-    two Adam steps."""
+    captured into a graph (at this batch one chain of launches: the first layer's three gradients
+    from one launch, every weight gradient's split sums left to the optimizer kernel). Every
+    layer's output, argmax, dW, db and dX, then the parameters after each of two Adam steps."""
     name = "cifar10_cnn_b128"
     flags = T.NET_FUSE_ACT_GRAD | T.NET_GRAPH
     spec, params, x, t, batch, loss, opt_kind, opt_kw, net, ref = make_pair(T, O, W, name, None, flags)
@@ -330,7 +330,9 @@ def test_net_rejects_inconsistent_layers(T):
         T.Net([dilated, T.L_fc(4 * 4 * 4, 2)], 4)
 
 
-@pytest.mark.parametrize("name,batch", [("cifar10_cnn_b128", 16), ("lenet5_b16", 16)])
+# (the CIFAR net branches at batch 16 and runs as one chain, its first layer's gradients from one
+# launch, at batch 128)
+@pytest.mark.parametrize("name,batch", [("cifar10_cnn_b128", 16), ("cifar10_cnn_b128", 128), ("lenet5_b16", 16)])
 def test_graph_replay_matches_eager_on_every_step(T, W, name, batch):
     """TDH_NET_GRAPH: the captured step is replayed five times with eager work, readbacks and
     synchronisations in between; after every replay all parameters equal the eager net's bit
