@@ -182,14 +182,14 @@ bool net_forks(const tdh_net *net, int batch) {
   return flop >= 1e8 && flop <= 3e10 && !(flop >= 2.2e9 && flop < 1e10);
 }
 // A step too small to branch (LeNet-5 at batch 16) is a chain of launches of a few
-// microseconds each, and what counts is how many there are (and so it is for a step inside
-// the window above that does not branch): it runs the branching step's
+// microseconds each, and what counts is how many there are; a larger step that does not
+// branch gains the reduction launches it does not make (VGG-style stack: 5.40 -> 5.37 ms): it runs the branching step's
 // launches one after the other, so that the split sums of all weight gradients go to the
 // optimizer kernel and the row sums of all bias gradients leave as one pair of launches.
 // (With the graph flag only: a net created with it reserves every layer's scratch side by side.)
 bool net_defers_serially(const tdh_net *net, int batch) {
   return (net->flags & TDH_NET_GRAPH) && (net->flags & TDH_NET_FUSE_ACT_GRAD) &&
-         !net_forks(net, batch) && net_forward_flop(net, batch) <= 3e10;
+         !net_forks(net, batch);
 }
 
 // The plan of the one-workgroup-per-sample step (tiny_net.hip) for a net that qualifies: at most
